@@ -1,0 +1,102 @@
+"""ctypes binding of libmuillm_amd.so (the C ABI declared in include/muillm_amd.h).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
+from typing import Dict, List, Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmuillm_amd.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "muillm_amd.h")
+
+MUI_OK = 0
+MUI_DTYPE_F16 = 0
+MUI_DTYPE_BF16 = 1
+MUI_MAX_TOKENS = 8
+
+
+class MuiDeviceInfo(ctypes.Structure):
+    _fields_ = [
+        ("device", c_int),
+        ("compute_units", c_int),
+        ("wave_size", c_int),
+        ("simd_lanes", c_int),
+        ("lds_bytes_per_block", c_int),
+        ("l2_bytes", c_int),
+        ("clock_khz", c_int),
+        ("is_gfx950", c_int),
+        ("hbm_bytes", ctypes.c_uint64),
+        ("arch", ctypes.c_char * 64),
+    ]
+
+
+class MuiLibraryError(RuntimeError):
+    pass
+
+
+_P = c_void_p
+# name -> (restype, argtypes).  Must list every function include/muillm_amd.h declares.
+_SIGNATURES = {
+    "mui_abi_version": (c_int, []),
+    "mui_status_string": (c_char_p, [c_int]),
+    "mui_device_info": (c_int, [c_int, ctypes.POINTER(MuiDeviceInfo)]),
+    "mui_linear": (c_int, [_P, c_int, _P, c_long, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_int]),
+    "mui_rmsnorm": (c_int, [_P, c_int, _P, _P, c_float, _P, c_int, c_int]),
+    "mui_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def declared_functions(header_path: str = HEADER_PATH) -> List[str]:
+    """Names of the functions the public header declares."""
+    with open(header_path, "r") as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mui_[a-z0-9_]+)\s*\(", text)))
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MuiLibraryError(
+            f"{LIB_PATH} is missing: build it with `make -C muillm_amd/csrc` "
+            "(or __graft_entry__.build()). There is no CPU fallback."
+        )
+    # torch ships its own HIP runtime with the same SONAME; importing it first makes the
+    # kernels and torch's allocator/streams share one runtime instance.
+    import torch  # noqa: F401
+
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def status_string(status: int) -> str:
+    return load().mui_status_string(status).decode()
+
+
+def check(status: int, what: str) -> None:
+    if status != MUI_OK:
+        raise MuiLibraryError(f"{what} failed: {status_string(status)} (status {status})")
+
+
+def device_info(device: int = 0) -> Dict[str, object]:
+    info = MuiDeviceInfo()
+    check(load().mui_device_info(device, ctypes.byref(info)), "mui_device_info")
+    out = {name: getattr(info, name) for name, _ in MuiDeviceInfo._fields_}
+    out["arch"] = info.arch.decode()
+    return out

@@ -1,0 +1,160 @@
+// Shared device helpers for the gfx950 decode kernels: 128-bit streaming loads,
+// 16-bit <-> fp32 conversion, wave64 reductions built from DPP + readlane.
+//
+// Everything here assumes wavefront size 64 (CDNA4) and is compiled for gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/muillm_amd.h"
+
+namespace mui {
+
+constexpr int kWave = 64;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------------------
+// element types: storage is 16 bits, arithmetic is fp32
+// ---------------------------------------------------------------------------------------
+struct F16 {
+  static constexpr int kDtype = MUI_DTYPE_F16;
+  // low / high half of a packed 32-bit word -> fp32
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return (float)__builtin_bit_cast(f16x2, w).x;
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return (float)__builtin_bit_cast(f16x2, w).y;
+  }
+  static __device__ __forceinline__ float one(uint16_t b) {
+    return (float)__builtin_bit_cast(_Float16, b);
+  }
+  // fp32 -> 16 bit storage, round-to-nearest-even (single rounding)
+  static __device__ __forceinline__ uint16_t pack(float v) {
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+  }
+};
+
+struct BF16 {
+  static constexpr int kDtype = MUI_DTYPE_BF16;
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return __builtin_bit_cast(float, w << 16);
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return __builtin_bit_cast(float, w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ float one(uint16_t b) {
+    return __builtin_bit_cast(float, ((uint32_t)b) << 16);
+  }
+  static __device__ __forceinline__ uint16_t pack(float v) {
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+    return (uint16_t)(u >> 16);
+  }
+};
+
+template <typename T>
+__device__ __forceinline__ void unpack8(const u32x4 w, float (&f)[8]) {
+  f[0] = T::lo(w.x); f[1] = T::hi(w.x);
+  f[2] = T::lo(w.y); f[3] = T::hi(w.y);
+  f[4] = T::lo(w.z); f[5] = T::hi(w.z);
+  f[6] = T::lo(w.w); f[7] = T::hi(w.w);
+}
+
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+  u32x4 w;
+  w.x = (uint32_t)T::pack(f[0]) | ((uint32_t)T::pack(f[1]) << 16);
+  w.y = (uint32_t)T::pack(f[2]) | ((uint32_t)T::pack(f[3]) << 16);
+  w.z = (uint32_t)T::pack(f[4]) | ((uint32_t)T::pack(f[5]) << 16);
+  w.w = (uint32_t)T::pack(f[6]) | ((uint32_t)T::pack(f[7]) << 16);
+  return w;
+}
+
+// ---------------------------------------------------------------------------------------
+// loads. Weights are read exactly once per call, so they are streamed with the
+// non-temporal hint; small reused vectors (x, gamma) use ordinary cached loads.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ u32x4 ld16_stream(const void* p) {
+  return __builtin_nontemporal_load((const u32x4*)p);
+}
+__device__ __forceinline__ u32x4 ld16(const void* p) { return *(const u32x4*)p; }
+__device__ __forceinline__ u32x2 ld8_stream(const void* p) {
+  return __builtin_nontemporal_load((const u32x2*)p);
+}
+__device__ __forceinline__ u32x2 ld8(const void* p) { return *(const u32x2*)p; }
+
+template <bool STREAM>
+__device__ __forceinline__ u32x4 ld16_sel(const void* p) {
+  if constexpr (STREAM) return ld16_stream(p); else return ld16(p);
+}
+
+// ---------------------------------------------------------------------------------------
+// wave64 reductions. Within a row of 16 lanes the butterfly runs on DPP (no LDS traffic);
+// the four row totals are then fetched with v_readlane, giving a wave-uniform result.
+// ---------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  int i = __builtin_bit_cast(int, v);
+  i = __builtin_amdgcn_update_dpp(0, i, CTRL, 0xf, 0xf, false);
+  return __builtin_bit_cast(float, i);
+}
+
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i within 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15-i within 16
+
+// every lane of each 16-lane row ends up holding that row's total
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f32<kDppXor1>(v);
+  v += dpp_f32<kDppXor2>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  v += dpp_f32<kDppMirror>(v);
+  return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f32<kDppXor1>(v));
+  v = fmaxf(v, dpp_f32<kDppXor2>(v));
+  v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_f32<kDppMirror>(v));
+  return v;
+}
+
+__device__ __forceinline__ float readlane_f32(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// total over all 64 lanes, uniform across the wave
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  return (readlane_f32(v, 0) + readlane_f32(v, 16)) + (readlane_f32(v, 32) + readlane_f32(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = row16_max(v);
+  return fmaxf(fmaxf(readlane_f32(v, 0), readlane_f32(v, 16)),
+               fmaxf(readlane_f32(v, 32), readlane_f32(v, 48)));
+}
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+
+// host-side helpers ----------------------------------------------------------------------
+static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+#define MUI_CHECK_ARG(cond)                 \
+  do {                                      \
+    if (!(cond)) return MUI_ERR_INVALID_ARG; \
+  } while (0)
+
+static inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? MUI_OK : MUI_ERR_LAUNCH;
+}
+
+}  // namespace mui

@@ -1,0 +1,315 @@
+// Single-token fused GEMV family for gfx950:
+//   linear      y = (W . xn) * mul_bias + add_bias + residual
+//   gate/up     h = silu(G . xn) * (U . xn)
+// with xn = x (plain) or gamma * x * rsqrt(mean(x^2) + eps) (RMSNorm fused in).
+//
+// Counterpart of the reference's single-token kernels (csrc/linear/linear_fp16_kernels.cu:163-626,
+// csrc/ffn/gateup_fp16_kernels.cu:160-604) but laid out for CDNA4:
+//   * a workgroup is 4 wave64s; thread t owns the 16-byte weight chunks t, t+256, ... of
+//     every row, so each wave-level load instruction covers 1 KiB of contiguous weights and
+//     the 4 waves cover 4 KiB -- whole DRAM pages, perfectly coalesced;
+//   * gamma*x lives in fp32 registers for the lifetime of the workgroup (CH chunks of 8),
+//     loaded once; sum(x^2) is reduced once per workgroup while the first weights are in flight;
+//   * R rows are in flight together (R*CH 128-bit loads per thread) and the next row group
+//     is requested before the current one is reduced, so a persistent workgroup never
+//     drains its memory pipeline;
+//   * the k-split is reduced with DPP inside a wave and through LDS across the 4 waves; one
+//     barrier per row group (double-buffered LDS);
+//   * the rsqrt factor is applied to the finished dot product, not to the 4096 inputs.
+#include "common.cuh"
+
+namespace mui {
+
+enum { EPI_LINEAR = 0, EPI_GATEUP = 1 };
+
+struct GemvParams {
+  const uint16_t* w0;  // linear: the matrix; gate/up: gate rows
+  const uint16_t* w1;  // gate/up: up rows
+  long pitch;          // row pitch in elements
+  const uint16_t* x;   // [K]
+  const uint16_t* gamma;
+  const uint16_t* mul_bias;
+  const uint16_t* add_bias;
+  const uint16_t* residual;
+  uint16_t* y;
+  int n;  // outputs (rows of W, or gate/up pairs)
+  int k;
+  float eps;
+};
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+
+template <typename T, int R, int CH, bool NORM, int EPI>
+__global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvParams p) {
+  constexpr int OUT = (EPI == EPI_GATEUP) ? R / 2 : R;  // outputs per row group
+  static_assert(EPI != EPI_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
+
+  __shared__ float red[2][kWaves][R];
+  __shared__ float red_ss[kWaves];
+
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int kc = p.k >> 3;  // 16-byte chunks per row
+  const int n_groups = (p.n + OUT - 1) / OUT;
+
+  // chunk offsets (in elements); chunks past the end of the row are redirected to chunk 0
+  // and meet xs == 0 there, so the hot loop has no predication at all.
+  int coff[CH];
+  bool cvalid[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const int c = t + kThreads * j;
+    cvalid[j] = c < kc;
+    coff[j] = cvalid[j] ? (c << 3) : 0;
+  }
+
+  u32x4 w[R][CH];
+  auto issue = [&](int rg) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int row;
+      const uint16_t* base;
+      if constexpr (EPI == EPI_GATEUP) {
+        row = rg * OUT + (r >> 1);
+        base = (r & 1) ? p.w1 : p.w0;
+      } else {
+        row = rg * R + r;
+        base = p.w0;
+      }
+      row = row < p.n ? row : p.n - 1;  // clamp: result is dropped in the epilogue
+      const uint16_t* rp = base + (long)row * p.pitch;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) w[r][j] = ld16_stream(rp + coff[j]);
+    }
+  };
+
+  int rg = blockIdx.x;
+  if (rg < n_groups) issue(rg);  // weights first: they are the long pole
+
+  // ---- inputs: gamma * x in fp32 registers, sum of squares on the side ----
+  float xs[CH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    if (cvalid[j]) {
+      float xf[8];
+      unpack8<T>(ld16(p.x + coff[j]), xf);
+      if constexpr (NORM) {
+        float gf[8];
+        unpack8<T>(ld16(p.gamma + coff[j]), gf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          ss = fmaf(xf[i], xf[i], ss);
+          xs[j][i] = xf[i] * gf[i];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xs[j][i] = xf[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xs[j][i] = 0.f;
+    }
+  }
+
+  float rs = 1.f;
+  if constexpr (NORM) {
+    ss = wave_sum(ss);
+    if (lane == 0) red_ss[wave] = ss;
+    __syncthreads();
+    const float tot = (red_ss[0] + red_ss[1]) + (red_ss[2] + red_ss[3]);
+    rs = rsqrtf(tot / (float)p.k + p.eps);
+  }
+
+  int buf = 0;
+  for (; rg < n_groups; rg += gridDim.x) {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float a0 = 0.f, a1 = 0.f;  // two chains per row to shorten the dependency
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        float wf[8];
+        unpack8<T>(w[r][j], wf);
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+          a0 = fmaf(wf[i], xs[j][i], a0);
+          a1 = fmaf(wf[i + 1], xs[j][i + 1], a1);
+        }
+      }
+      acc[r] = a0 + a1;
+    }
+
+    const int nxt = rg + gridDim.x;
+    if (nxt < n_groups) issue(nxt);  // keep the memory pipe full during the reduction
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) red[buf][wave][r] = acc[r];
+    }
+    __syncthreads();
+
+    if (t < OUT) {
+      const int n = rg * OUT + t;
+      if (n < p.n) {
+        float v;
+        if constexpr (EPI == EPI_GATEUP) {
+          const int rg_ = 2 * t, ru_ = 2 * t + 1;
+          const float g = ((red[buf][0][rg_] + red[buf][1][rg_]) + (red[buf][2][rg_] + red[buf][3][rg_])) * rs;
+          const float u = ((red[buf][0][ru_] + red[buf][1][ru_]) + (red[buf][2][ru_] + red[buf][3][ru_])) * rs;
+          v = silu_f32(g) * u;
+        } else {
+          v = ((red[buf][0][t] + red[buf][1][t]) + (red[buf][2][t] + red[buf][3][t])) * rs;
+          if (p.mul_bias) v *= T::one(p.mul_bias[n]);
+          if (p.add_bias) v += T::one(p.add_bias[n]);
+          if (p.residual) v += T::one(p.residual[n]);
+        }
+        p.y[n] = T::pack(v);
+      }
+    }
+    buf ^= 1;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+struct Tuning {
+  int rows_linear = 4;      // R for linear (2 or 4)
+  int wgs_per_cu = 8;       // cap on resident workgroups per CU used to size persistent grids
+  int cus = 0;              // filled on first use
+};
+static Tuning g_tune;
+
+static int device_cus() {
+  if (g_tune.cus == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    g_tune.cus = cus;
+  }
+  return g_tune.cus;
+}
+
+template <typename T, int R, int CH, int EPI>
+static int launch_rc(hipStream_t s, const GemvParams& p, int grid) {
+  if (p.gamma)
+    hipLaunchKernelGGL((gemv_kernel<T, R, CH, true, EPI>), dim3(grid), dim3(kThreads), 0, s, p);
+  else
+    hipLaunchKernelGGL((gemv_kernel<T, R, CH, false, EPI>), dim3(grid), dim3(kThreads), 0, s, p);
+  return launch_status();
+}
+
+template <typename T, int R, int EPI>
+static int launch_r(hipStream_t s, const GemvParams& p) {
+  constexpr int OUT = (EPI == EPI_GATEUP) ? R / 2 : R;
+  const int n_groups = ceil_div(p.n, OUT);
+  const int ch = ceil_div(p.k >> 3, kThreads);
+  // resident workgroups per CU are bounded by registers: ~64 VGPRs up to CH=2, more beyond
+  int per_cu = g_tune.wgs_per_cu;
+  if (ch > 2 && per_cu > 4) per_cu = 4;
+  int grid = device_cus() * per_cu;
+  if (grid > n_groups) grid = n_groups;
+  if (ch <= 1) return launch_rc<T, R, 1, EPI>(s, p, grid);
+  if (ch <= 2) return launch_rc<T, R, 2, EPI>(s, p, grid);
+  if (ch <= 4) return launch_rc<T, R, 4, EPI>(s, p, grid);
+  if (ch <= 7) return launch_rc<T, R, 7, EPI>(s, p, grid);
+  if (ch <= 8) return launch_rc<T, R, 8, EPI>(s, p, grid);
+  return MUI_ERR_UNSUPPORTED;
+}
+
+template <int EPI>
+static int launch_gemv(hipStream_t s, int dtype, const GemvParams& p) {
+  if (dtype == MUI_DTYPE_F16) {
+    if (EPI == EPI_GATEUP) return launch_r<F16, 4, EPI>(s, p);
+    return g_tune.rows_linear == 2 ? launch_r<F16, 2, EPI>(s, p) : launch_r<F16, 4, EPI>(s, p);
+  }
+  if (dtype == MUI_DTYPE_BF16) {
+    if (EPI == EPI_GATEUP) return launch_r<BF16, 4, EPI>(s, p);
+    return g_tune.rows_linear == 2 ? launch_r<BF16, 2, EPI>(s, p) : launch_r<BF16, 4, EPI>(s, p);
+  }
+  return MUI_ERR_INVALID_ARG;
+}
+
+}  // namespace mui
+
+using namespace mui;
+
+extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
+  if (rows_linear == 2 || rows_linear == 4) g_tune.rows_linear = rows_linear;
+  if (wgs_per_cu >= 1 && wgs_per_cu <= 16) g_tune.wgs_per_cu = wgs_per_cu;
+  return MUI_OK;
+}
+
+extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, long w_pitch,
+                          const void* x, const void* norm_weights, float epsilon,
+                          const void* mul_bias, const void* add_bias, const void* residual,
+                          void* y, int n_out, int k_in, int tokens) {
+  MUI_CHECK_ARG(weights && x && y);
+  MUI_CHECK_ARG(n_out > 0 && k_in > 0 && tokens > 0);
+  MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
+  if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
+  if (w_pitch < k_in) return MUI_ERR_INVALID_ARG;
+  if ((k_in & 7) || (w_pitch & 7)) return MUI_ERR_UNSUPPORTED;
+  if (k_in > 8 * 8 * kThreads) return MUI_ERR_UNSUPPORTED;
+  if (!aligned16(weights) || !aligned16(x) || (norm_weights && !aligned16(norm_weights)))
+    return MUI_ERR_ALIGNMENT;
+
+  hipStream_t s = (hipStream_t)stream;
+  for (int tkn = 0; tkn < tokens; ++tkn) {
+    GemvParams p;
+    p.w0 = (const uint16_t*)weights;
+    p.w1 = nullptr;
+    p.pitch = w_pitch;
+    p.x = (const uint16_t*)x + (long)tkn * k_in;
+    p.gamma = (const uint16_t*)norm_weights;
+    p.mul_bias = (const uint16_t*)mul_bias;
+    p.add_bias = (const uint16_t*)add_bias;
+    p.residual = residual ? (const uint16_t*)residual + (long)tkn * n_out : nullptr;
+    p.y = (uint16_t*)y + (long)tkn * n_out;
+    p.n = n_out;
+    p.k = k_in;
+    p.eps = epsilon;
+    int st = launch_gemv<EPI_LINEAR>(s, dtype, p);
+    if (st != MUI_OK) return st;
+  }
+  return MUI_OK;
+}
+
+extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate, const void* up,
+                               long gu_pitch, const void* x, const void* norm_weights,
+                               float epsilon, void* h, int n_inter, int k_in, int tokens) {
+  MUI_CHECK_ARG(gate && up && x && h);
+  MUI_CHECK_ARG(n_inter > 0 && k_in > 0 && tokens > 0);
+  MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
+  if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
+  if (gu_pitch < k_in) return MUI_ERR_INVALID_ARG;
+  if ((k_in & 7) || (gu_pitch & 7)) return MUI_ERR_UNSUPPORTED;
+  if (k_in > 8 * 8 * kThreads) return MUI_ERR_UNSUPPORTED;
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(x) ||
+      (norm_weights && !aligned16(norm_weights)))
+    return MUI_ERR_ALIGNMENT;
+
+  hipStream_t s = (hipStream_t)stream;
+  for (int tkn = 0; tkn < tokens; ++tkn) {
+    GemvParams p;
+    p.w0 = (const uint16_t*)gate;
+    p.w1 = (const uint16_t*)up;
+    p.pitch = gu_pitch;
+    p.x = (const uint16_t*)x + (long)tkn * k_in;
+    p.gamma = (const uint16_t*)norm_weights;
+    p.mul_bias = p.add_bias = p.residual = nullptr;
+    p.y = (uint16_t*)h + (long)tkn * n_inter;
+    p.n = n_inter;
+    p.k = k_in;
+    p.eps = epsilon;
+    int st = launch_gemv<EPI_GATEUP>(s, dtype, p);
+    if (st != MUI_OK) return st;
+  }
+  return MUI_OK;
+}

@@ -1,0 +1,381 @@
+"""CPU restatement of the reference's layer semantics (test infrastructure only).
+
+All functions take torch CPU tensors.  Unless `reference_path=True`, inputs are upcast to
+float64 and the float64 result is returned un-rounded: this is the accumulate-in-high-
+precision reference the stated tolerances are measured against.
+
+Citations are into the reference tree (Epliz/muiLLM).
+"""
+
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+
+__all__ = [
+    "rmsnorm",
+    "linear",
+    "multilinear",
+    "gateupdown_mlp",
+    "gateup_silu",
+    "rtn_quantize_group",
+    "rtn_dequantize_group",
+    "rtn_quantize_channel",
+    "rtn_dequantize_channel",
+    "int8_channel_linear",
+    "int8_group_linear",
+    "rope_inv_freq",
+    "rope_tables",
+    "rotate_half",
+    "apply_rope",
+    "static_cache_update",
+    "repeat_kv",
+    "decode_attention",
+    "decoder_layer",
+    "next_pow2",
+    "rel_err",
+]
+
+_HI = torch.float64
+
+
+def _hi(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return None if t is None else t.detach().to("cpu", _HI)
+
+
+def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """max |got - ref| / max |ref|  (the denominator the parity gates use)."""
+    ref = ref.to(_HI)
+    return float((got.to(_HI) - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+# --------------------------------------------------------------------------------------
+# RMSNorm -- muillm/modules/norm/rmsnorm.py:138-146 (HF LlamaRMSNorm form)
+# --------------------------------------------------------------------------------------
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, reference_path: bool = False):
+    """y = weight * x * rsqrt(mean(x^2, -1) + eps).
+
+    reference_path=True reproduces the fallback literally: fp32 upcast, the normalised
+    activations rounded back to the input dtype BEFORE the multiply by weight
+    (rmsnorm.py:140-146)."""
+    if reference_path:
+        input_dtype = x.dtype
+        h = x.to(torch.float32)
+        variance = h.pow(2).mean(-1, keepdim=True)
+        h = h * torch.rsqrt(variance + eps)
+        return weight * h.to(input_dtype)
+    xh, wh = _hi(x), _hi(weight)
+    variance = xh.pow(2).mean(-1, keepdim=True)
+    return wh * (xh * torch.rsqrt(variance + eps))
+
+
+# --------------------------------------------------------------------------------------
+# Linear (+ fused input norm, bias, residual) -- muillm/modules/linear.py:324-333
+# --------------------------------------------------------------------------------------
+def linear(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    norm_weights: Optional[torch.Tensor] = None,
+    eps: float = 0.0,
+    bias: Optional[torch.Tensor] = None,
+    residual: Optional[torch.Tensor] = None,
+    mul_bias: Optional[torch.Tensor] = None,
+    reference_path: bool = False,
+):
+    """y = F.linear(rmsnorm(x) if norm_weights else x, weight, bias) (+ residual).
+
+    `mul_bias` follows the kernel-level form y = (W x) * mul_bias + bias + residual
+    (csrc/linear/linear_fp16_kernels.cu:163-356); the Python layer always passes None."""
+    if reference_path:
+        if norm_weights is not None:
+            x = rmsnorm(x, norm_weights, eps, reference_path=True)
+        out = F.linear(x, weight, None)
+        if mul_bias is not None:
+            out = out * mul_bias
+        if bias is not None:
+            out = out + bias
+        if residual is not None:
+            out = out + residual
+        return out
+    xh = rmsnorm(x, norm_weights, eps) if norm_weights is not None else _hi(x)
+    out = xh @ _hi(weight).T
+    if mul_bias is not None:
+        out = out * _hi(mul_bias)
+    if bias is not None:
+        out = out + _hi(bias)
+    if residual is not None:
+        out = out + _hi(residual)
+    return out
+
+
+def multilinear(
+    x: torch.Tensor,
+    weights: Sequence[torch.Tensor],
+    norm_weights: Optional[torch.Tensor] = None,
+    eps: float = 0.0,
+    biases: Optional[Sequence[torch.Tensor]] = None,
+) -> Tuple[torch.Tensor, ...]:
+    """Fused QKV: one linear over the row-concatenated weights, returned as last-dim slices
+    (muillm/modules/multilinear.py:56-66,186-237)."""
+    w = torch.cat(list(weights), dim=0)
+    b = torch.cat(list(biases), dim=0) if biases is not None else None
+    out = linear(x, w, norm_weights, eps, b)
+    outs, start = [], 0
+    for wi in weights:
+        outs.append(out[..., start : start + wi.shape[0]])
+        start += wi.shape[0]
+    return tuple(outs)
+
+
+# --------------------------------------------------------------------------------------
+# Gate/Up/Down MLP -- muillm/modules/gateupdownmlp.py:343-359
+# --------------------------------------------------------------------------------------
+def gateup_silu(x, gate_w, up_w, norm_weights=None, eps: float = 0.0):
+    """silu(G xn) * (U xn): the intermediate the fused kernel writes
+    (csrc/ffn/gateup_fp16_kernels.cu:596-601)."""
+    xh = rmsnorm(x, norm_weights, eps) if norm_weights is not None else _hi(x)
+    g = xh @ _hi(gate_w).T
+    u = xh @ _hi(up_w).T
+    return F.silu(g) * u
+
+
+def gateupdown_mlp(
+    x, gate_w, up_w, down_w, norm_weights=None, eps: float = 0.0, residual=None,
+    reference_path: bool = False, round_intermediate: Optional[torch.dtype] = None,
+):
+    """out = down(silu(gate(xn)) * up(xn)) + residual  (_forward_unfused, :343-359).
+
+    round_intermediate=torch.float16 rounds the 14336-wide intermediate to 16 bits the way
+    both the reference kernels and this build store it between the two GEMVs."""
+    if reference_path:
+        if norm_weights is not None:
+            x = rmsnorm(x, norm_weights, eps, reference_path=True)
+        g = F.linear(x, gate_w)
+        u = F.linear(x, up_w)
+        out = F.linear(F.silu(g) * u, down_w)
+        if residual is not None:
+            out = out + residual
+        return out
+    h = gateup_silu(x, gate_w, up_w, norm_weights, eps)
+    if round_intermediate is not None:
+        h = h.to(round_intermediate).to(_HI)
+    out = h @ _hi(down_w).T
+    if residual is not None:
+        out = out + _hi(residual)
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# RTN quantisation
+# --------------------------------------------------------------------------------------
+def rtn_quantize_group(w: torch.Tensor, group_size: int = 128, f: float = 1.0):
+    """The reference's asymmetric group-wise uint8 RTN
+    (muillm/quantization/rtnquantizer.py:49-88): returns (uint8 [N,K], (scale,min) [N*G,2])
+    with the pair stored in w's dtype."""
+    if group_size <= 0 or (group_size & (group_size - 1)) != 0:
+        raise ValueError("group size must be a power of two")
+    if w.dim() != 2 or w.shape[-1] % group_size != 0:
+        raise ValueError("group size must divide the last dimension of a 2-D weight")
+    to_quant = w.reshape(-1, group_size).to(torch.float32)
+    max_val = to_quant.amax(dim=1, keepdim=True)
+    min_val = to_quant.amin(dim=1, keepdim=True)
+    val_range = (f * (max_val - min_val)).clamp(min=1e-6)
+    val_center = (min_val + max_val) * 0.5
+    min_val = val_center - val_range * 0.5
+    scales = val_range / 255
+    q = to_quant.sub(min_val).div(scales).clamp(0, 255).round().to(torch.uint8).reshape_as(w)
+    return q, torch.cat([scales, min_val], dim=-1).to(w.dtype)
+
+
+def rtn_dequantize_group(q: torch.Tensor, scales_min_vals: torch.Tensor, group_size: int,
+                         dtype: torch.dtype = torch.float16, kernel_form: bool = True):
+    """kernel_form=True: half(float(q)*float(scale) + float(min)), one rounding
+    (csrc/int8_dequantization_kernel.cu:50-59).  kernel_form=False: the Python fallback,
+    multiply then add in the scale dtype, two roundings (rtnquantizer.py:91-102)."""
+    qg = q.reshape(-1, group_size)
+    scales = scales_min_vals[:, None, 0]
+    mins = scales_min_vals[:, None, 1]
+    if kernel_form:
+        # q*scale+min is exact in float64; rounding it to fp32 reproduces the fp32 fma's
+        # single rounding, the store then rounds fp32 -> 16 bit.
+        dq = torch.addcmul(mins.to(_HI), qg.to(_HI), scales.to(_HI))
+        return dq.to(torch.float32).reshape_as(q).to(dtype)
+    return qg.mul(scales).add(mins).reshape_as(q).to(dtype)
+
+
+def rtn_quantize_channel(w: torch.Tensor):
+    """Symmetric per-output-channel int8 RTN (the on-device format of the int8 decode
+    GEMVs): s[n] = half(max|w[n,:]| / 127), q = clamp(round_half_even(w / s), -127, 127).
+
+    The divide is done in fp32 on the fp16-rounded scale so that quantise and dequantise
+    agree on s.  An all-zero row gets the smallest positive fp16 as scale (q = 0)."""
+    if w.dim() != 2:
+        raise ValueError("only 2-D weights can be quantised")
+    wf = w.to(torch.float32)
+    amax = wf.abs().amax(dim=1)
+    s = (amax / 127.0).to(torch.float16)
+    tiny = torch.tensor(2.0 ** -24, dtype=torch.float16)
+    s = torch.where(s > 0, s, tiny)
+    q = torch.round(wf / s.to(torch.float32)[:, None]).clamp(-127, 127).to(torch.int8)
+    return q, s
+
+
+def rtn_dequantize_channel(q: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+    """w = half(float(q) * float(s)): an 8-bit integer times an 11-bit significand is exact
+    in fp32, so this equals torch's q.half() * s[:, None] bit for bit."""
+    return (q.to(torch.float32) * s.to(torch.float32)[:, None]).to(s.dtype)
+
+
+def int8_channel_linear(x, q, s, norm_weights=None, eps=0.0, bias=None, residual=None):
+    """Dequantise-then-linear (muillm/modules/quantized/int8linear.py:279-293) on the
+    per-channel format, accumulated in float64."""
+    return linear(x, rtn_dequantize_channel(q, s), norm_weights, eps, bias, residual)
+
+
+def int8_group_linear(x, q, scales_min_vals, group_size, norm_weights=None, eps=0.0,
+                      bias=None, residual=None):
+    """Same for the reference's group format; the weights are the exact (un-rounded)
+    q*scale+min values, which is what the reference int8 GEMV accumulates
+    (csrc/int8_linear_kernels.cu:213-236)."""
+    qg = q.reshape(-1, group_size).to(_HI)
+    w = (qg * scales_min_vals[:, None, 0].to(_HI) + scales_min_vals[:, None, 1].to(_HI)).reshape(q.shape)
+    return linear(x, w, norm_weights, eps, bias, residual)
+
+
+# --------------------------------------------------------------------------------------
+# RoPE -- muillm/modules/attention/rotaryembedding.py:23-64,313-351
+# --------------------------------------------------------------------------------------
+def rope_inv_freq(theta: float, dim: int) -> torch.Tensor:
+    """HF 'default' rope init: 1 / theta^(2i/dim), computed in fp32."""
+    return 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.int64).to(torch.float32) / dim))
+
+
+def rope_tables(theta: float, dim: int, max_pos: int, dtype=torch.float32, attention_scaling=1.0):
+    """cos/sin tables [max_pos, dim] with emb = cat(freqs, freqs) (:313-337).  The angle is
+    formed in fp32 like the reference does."""
+    inv_freq = rope_inv_freq(theta, dim)
+    t = torch.arange(max_pos, dtype=torch.int64).type_as(inv_freq)
+    freqs = torch.outer(t, inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return (emb.cos() * attention_scaling).to(dtype), (emb.sin() * attention_scaling).to(dtype)
+
+
+def rotate_half(x: torch.Tensor) -> torch.Tensor:
+    x1 = x[..., : x.shape[-1] // 2]
+    x2 = x[..., x.shape[-1] // 2 :]
+    return torch.cat((-x2, x1), dim=-1)
+
+
+def apply_rope(q, k, cos, sin, position_ids, reference_path: bool = False):
+    """q, k: [B, H, T, D]; cos, sin: tables [max_pos, D]; position_ids [B, T].
+    q' = q*cos + rotate_half(q)*sin (:31-64)."""
+    c = cos[position_ids].unsqueeze(1)  # [B,1,T,D]
+    s = sin[position_ids].unsqueeze(1)
+    if reference_path:
+        c, s = c.to(q.dtype), s.to(q.dtype)
+        return (q * c) + (rotate_half(q) * s), (k * c) + (rotate_half(k) * s)
+    c, s, qh, kh = _hi(c), _hi(s), _hi(q), _hi(k)
+    return (qh * c) + (rotate_half(qh) * s), (kh * c) + (rotate_half(kh) * s)
+
+
+# --------------------------------------------------------------------------------------
+# Static KV cache -- muillm/modules/kvcache/cache_utils.py:185-204,681-712
+# --------------------------------------------------------------------------------------
+def next_pow2(x: int) -> int:
+    if x < 0:
+        raise ValueError("x should be positive")
+    p = 1
+    while p < x:
+        p *= 2
+    return p
+
+
+def static_cache_update(k_cache, v_cache, k_new, v_new, cache_position, seen_tokens: int):
+    """Index-copy the new rows at cache_position along dim 2, then return views narrowed to
+    the tokens seen so far (StaticCache.update + narrow, cache_utils.py:185-204).
+    Caches are [B, Hkv, MAX_T, D] and are modified in place."""
+    k_cache.index_copy_(2, cache_position, k_new.to(k_cache.dtype))
+    v_cache.index_copy_(2, cache_position, v_new.to(v_cache.dtype))
+    seen = seen_tokens + k_new.shape[-2]
+    return k_cache.narrow(2, 0, seen), v_cache.narrow(2, 0, seen), seen
+
+
+# --------------------------------------------------------------------------------------
+# Decode attention -- muillm/modules/attention/baseattention.py:219-253, kvcache.py:3-12
+# --------------------------------------------------------------------------------------
+def repeat_kv(h: torch.Tensor, n_rep: int) -> torch.Tensor:
+    b, hk, s, d = h.shape
+    if n_rep == 1:
+        return h
+    return h[:, :, None, :, :].expand(b, hk, n_rep, s, d).reshape(b, hk * n_rep, s, d)
+
+
+def decode_attention(q, k, v, mask=None, reference_path: bool = False):
+    """q [B,Hq,T,D], k/v [B,Hkv,S,D], additive mask broadcastable to [B,1,T,S] or None.
+    Returns [B, T, Hq*D].  softmax(q k^T / sqrt(D) + mask) v with GQA head h -> kv head
+    h // (Hq/Hkv)."""
+    b, hq, t, d = q.shape
+    n_rep = hq // k.shape[1]
+    if reference_path:
+        kk, vv = repeat_kv(k, n_rep), repeat_kv(v, n_rep)
+        w = torch.matmul(q, kk.transpose(2, 3)) / math.sqrt(d)
+        if mask is not None:
+            w = w + mask
+        w = F.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+        o = torch.matmul(w, vv)
+        return o.transpose(1, 2).contiguous().reshape(b, t, hq * d)
+    qh, kk, vv = _hi(q), repeat_kv(_hi(k), n_rep), repeat_kv(_hi(v), n_rep)
+    w = torch.matmul(qh, kk.transpose(2, 3)) / math.sqrt(d)
+    if mask is not None:
+        w = w + _hi(mask)
+    w = F.softmax(w, dim=-1)
+    o = torch.matmul(w, vv)
+    return o.transpose(1, 2).contiguous().reshape(b, t, hq * d)
+
+
+# --------------------------------------------------------------------------------------
+# Decoder layer -- muillm/modules/decoder/decoder.py:130-165
+# --------------------------------------------------------------------------------------
+def decoder_layer(
+    h: torch.Tensor,            # [B, T, hidden]
+    p: dict,                    # weights: ln1, wq, wk, wv, wo, ln2, wg, wu, wd (+ eps)
+    k_cache: torch.Tensor,      # [B, Hkv, MAX_T, D]  (modified in place)
+    v_cache: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    position_ids: torch.Tensor,  # [B, T]
+    cache_position: torch.Tensor,  # [T]
+    seen_tokens: int,
+    n_heads: int,
+    n_kv_heads: int,
+    store_dtype: torch.dtype = torch.float16,
+):
+    """One decoder layer with the rounding points of the fused path: q/k/v, attention
+    output, post-attention hidden state and MLP intermediate are stored in `store_dtype`
+    between kernels; everything inside a kernel is float64 here.
+    Causal masking is applied for T > 1 (prefill)."""
+    b, t, hid = h.shape
+    d = hid // n_heads
+    eps = p["eps"]
+    rnd = lambda z: z.to(store_dtype)
+    q, k, v = multilinear(h, [p["wq"], p["wk"], p["wv"]], p["ln1"], eps)
+    q = rnd(q).view(b, t, n_heads, d).transpose(1, 2)
+    k = rnd(k).view(b, t, n_kv_heads, d).transpose(1, 2)
+    v = rnd(v).view(b, t, n_kv_heads, d).transpose(1, 2)
+    qr, kr = apply_rope(q, k, cos, sin, position_ids)
+    qr, kr = rnd(qr), rnd(kr)
+    kk, vv, seen = static_cache_update(k_cache, v_cache, kr, v, cache_position, seen_tokens)
+    mask = None
+    if t > 1:
+        s = kk.shape[2]
+        qpos = cache_position.view(t, 1)
+        kpos = torch.arange(s).view(1, s)
+        mask = torch.where(kpos <= qpos, 0.0, float("-inf")).to(_HI).view(1, 1, t, s)
+    attn = rnd(decode_attention(qr, kk, vv, mask))
+    h1 = rnd(linear(attn, p["wo"], residual=h))
+    out = gateupdown_mlp(h1, p["wg"], p["wu"], p["wd"], p["ln2"], eps, residual=h1,
+                         round_intermediate=store_dtype)
+    return rnd(out), seen

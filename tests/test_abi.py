@@ -1,0 +1,58 @@
+"""CPU checks of the drop-in boundary: the C-ABI library loads and exports exactly the
+functions the public header declares (no compute calls here)."""
+import ctypes
+import os
+import re
+
+from muillm_amd import _lib
+
+
+def test_library_is_built():
+    assert os.path.exists(_lib.LIB_PATH), "run `make -C muillm_amd/csrc` first"
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    declared = _lib.declared_functions()
+    assert len(declared) >= 6
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/muillm_amd.h but not exported"
+        assert name in _lib._SIGNATURES, f"{name} has no ctypes signature in muillm_amd/_lib.py"
+    for name in _lib._SIGNATURES:
+        assert name in declared, f"{name} is bound in _lib.py but not declared in the header"
+
+
+def test_signature_arity_matches_header():
+    with open(_lib.HEADER_PATH) as f:
+        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    for name, (_, argtypes) in _lib._SIGNATURES.items():
+        m = re.search(r"\b%s\s*\(([^;]*?)\)\s*;" % name, text, flags=re.S)
+        assert m, name
+        args = m.group(1).strip()
+        n = 0 if args in ("", "void") else len(args.split(","))
+        assert n == len(argtypes), f"{name}: header has {n} parameters, ctypes binding {len(argtypes)}"
+
+
+def test_no_framework_types_in_header():
+    with open(_lib.HEADER_PATH) as f:
+        text = f.read()
+    for banned in ("torch", "at::", "Tensor", "hipStream_t stream", "#include <hip"):
+        assert banned not in re.sub(r"/\*.*?\*/", "", text, flags=re.S), banned
+
+
+def test_status_strings_and_version():
+    lib = _lib.load()
+    assert lib.mui_abi_version() == 1
+    assert _lib.status_string(0) == "ok"
+    for code in (-1, -2, -3, -4, -5):
+        assert _lib.status_string(code) not in ("ok", "unknown status")
+    assert _lib.status_string(-99) == "unknown status"
+
+
+def test_argument_validation_needs_no_gpu():
+    """Null pointers and bad sizes are rejected on the host before any HIP call."""
+    lib = _lib.load()
+    assert lib.mui_linear(None, 0, None, 8, None, None, 0.0, None, None, None, None, 8, 8, 1) == -1
+    assert lib.mui_rmsnorm(None, 0, None, None, 0.0, None, 1, 8) == -1
+    assert lib.mui_gateup_silu(None, 0, None, None, 8, None, None, 0.0, None, 8, 8, 1) == -1
+    assert lib.mui_device_info(0, None) == -1
