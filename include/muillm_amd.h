@@ -106,6 +106,145 @@ int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate, const void
                     long gu_pitch, const void* x, const void* norm_weights, float epsilon,
                     void* h, int n_inter, int k_in, int tokens);
 
+/* ------------------------------------------------------------------------------------
+ * int8 weight-only family
+ * ---------------------------------------------------------------------------------- */
+
+/* muillm_int8_linear_forward (csrc/module.cpp:31-54,181; csrc/int8_linear_kernels.cu:703-785)
+ * on the symmetric per-output-channel format of the decode benchmarks:
+ *   weights_i8 int8 [n_out, k_in] (row pitch w_pitch bytes), scales 16-bit [n_out],
+ *   w[n, k] = q[n, k] * scales[n];   y = W xn + add_bias + residual   (xn as in mui_linear).
+ * The reference passes the residual through add_bias (int8linear.py:53-57); here both exist.
+ * Requirements: k_in % 16 == 0, k_in <= 16384, 16-byte aligned rows. */
+int mui_int8_linear(mui_stream_t stream, int dtype, const void* weights_i8, long w_pitch,
+                    const void* scales, const void* x, const void* norm_weights, float epsilon,
+                    const void* add_bias, const void* residual, void* y, int n_out, int k_in,
+                    int tokens);
+
+/* muillm_int8_gateupsilu_forward (csrc/module.cpp:248; csrc/int8_gateup_kernels.cu:871-940),
+ * per-channel format. gate/up are int8 [n_inter, k_in] sharing the row pitch gu_pitch (bytes):
+ * two dense matrices, or the two halves of a row-interleaved [n_inter, 2, k_in] buffer
+ * (up == gate + k_in, gu_pitch == 2 * k_in). Scale of row n: gate_scales[n * scale_stride],
+ * up_scales[n * scale_stride] (scale_stride 2 for an interleaved [n_inter, 2] scale buffer).
+ *   h[t, n] = silu(sg[n] * Gq[n,:] . xn[t]) * (su[n] * Uq[n,:] . xn[t]) */
+int mui_int8_gateup_silu(mui_stream_t stream, int dtype, const void* gate_i8, const void* up_i8,
+                         long gu_pitch, const void* gate_scales, const void* up_scales,
+                         long scale_stride, const void* x, const void* norm_weights, float epsilon,
+                         void* h, int n_inter, int k_in, int tokens);
+
+/* muillm_int8_linear_forward on the reference's own RTN format
+ * (muillm/quantization/rtnquantizer.py:49-88): weights_u8 uint8 [n_out, k_in],
+ * scales_min_vals 16-bit [n_out * G, 2] = (scale, min) per group of 2^group_size_shift
+ * inputs, w = u8 * scale + min. Requirements as above plus group size >= 16. */
+int mui_int8_group_linear(mui_stream_t stream, int dtype, const void* weights_u8, long w_pitch,
+                          const void* scales_min_vals, int group_size_shift, const void* x,
+                          const void* norm_weights, float epsilon, const void* add_bias,
+                          const void* residual, void* y, int n_out, int k_in, int tokens);
+
+/* muillm_int8_gateupsilu_forward on the reference's RTN format. gate/up rows share gu_pitch
+ * (bytes); the (scale, min) pairs of row n start at gate_smv + n * smv_pitch and
+ * up_smv + n * smv_pitch (16-bit elements; 2 * G when dense, 4 * G when row-interleaved). */
+int mui_int8_group_gateup_silu(mui_stream_t stream, int dtype, const void* gate_u8,
+                               const void* up_u8, long gu_pitch, const void* gate_smv,
+                               const void* up_smv, long smv_pitch, int group_size_shift,
+                               const void* x, const void* norm_weights, float epsilon, void* h,
+                               int n_inter, int k_in, int tokens);
+
+/* Dense dequantisation of the per-channel format (the non-single-token branch of
+ * muillm/modules/quantized/int8linear.py:279-293): out[n, k] = T(float(q[n,k]) * float(s[n])),
+ * bit-identical to torch's q.to(T) * s[:, None]. scale of row n at scales[n * scale_stride]. */
+int mui_int8_dequantize(mui_stream_t stream, int dtype, const void* weights_i8, long w_pitch,
+                        const void* scales, long scale_stride, void* out, long out_pitch, int n,
+                        int k);
+
+/* muillm_int8_dequantize_forward (csrc/module.cpp:180; csrc/int8_dequantization_kernel.cu:50-59,156-193):
+ * out[n, k] = T(fma(float(u8), float(scale_g), float(min_g))). */
+int mui_int8_group_dequantize(mui_stream_t stream, int dtype, const void* weights_u8, long w_pitch,
+                              const void* scales_min_vals, long smv_pitch, int group_size_shift,
+                              void* out, long out_pitch, int n, int k);
+
+/* ------------------------------------------------------------------------------------
+ * RoPE, static KV cache, decode attention (head_dim 128; Hq/Hkv in {1, 2, 4, 8})
+ *
+ * Common conventions: q/k/v inputs and the cache have unit inner stride; all other strides
+ * are in elements. cos/sin tables are fp32 [max_position, rope_row_stride] with
+ * rope_row_stride >= head_dim/2 and column f (f < head_dim/2) holding cos/sin(pos * inv_freq[f])
+ * (the first half of the reference's cos_cached/sin_cached rows,
+ * muillm/modules/attention/rotaryembedding.py:313-337); rotation is the HF rotate-half form
+ * q' = q*cos + rotate_half(q)*sin in fp32, rounded once. position_ids / cache_position are
+ * int64 device arrays like the reference's (csrc/rope/rotary.cu:209-211). The cache is
+ * [batch, n_kv_heads, max_cache_len, head_dim] (muillm/modules/kvcache/cache_utils.py:113-204).
+ * ---------------------------------------------------------------------------------- */
+
+/* muillm_rope_forward_static_cache / muillm_rope_forward_no_cache / muillm_static_kvcache_update
+ * (csrc/module.cpp:266-268,272; csrc/rope/rotary.cu:603-756; csrc/kvcaches/static_kvcache.cpp:35-121)
+ * for `tokens` new tokens per batch row:
+ *   q_out[b, h, t, :]               = rope(q[b, t, h, :], position_ids[b, t])     (dense [B,Hq,T,D])
+ *   k_out[b, h, slot(t), :]         = rope(k[b, t, h, :], position_ids[b, t])
+ *   v_out[b, h, slot(t), :]         = v[b, t, h, :]
+ * slot(t) = cache_position[t] when cache_position != NULL (k_out/v_out are the caches; slots
+ * outside [0, max_cache_len) are skipped), else t (k_out/v_out are dense [B,Hkv,T,D] given by
+ * the out strides). q, k or v may be NULL to skip that part; cos_table == NULL copies without
+ * rotating (plain cache update). position_batch_stride 0 shares one row of positions. */
+int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                      long q_token_stride, long q_head_stride, const void* k, long k_batch_stride,
+                      long k_token_stride, long k_head_stride, const void* v, long v_batch_stride,
+                      long v_token_stride, long v_head_stride, const float* cos_table,
+                      const float* sin_table, int rope_row_stride, const int64_t* position_ids,
+                      long position_batch_stride, const int64_t* cache_position, void* q_out,
+                      void* k_out, void* v_out, long out_batch_stride, long out_head_stride,
+                      long out_token_stride, int batch, int tokens, int n_q_heads, int n_kv_heads,
+                      int head_dim, int max_cache_len);
+
+/* Number of sequence splits to use for a decode over about seq_len_hint cached tokens
+ * (enough workgroups to fill the GPU, at least two passes of work per split), and the
+ * scratch size in bytes that mui_flash_decode / mui_attn_decode_fused need for it (0 when
+ * n_splits == 1). The reference fixes 4 tokens per group (csrc/attention/flash_decoding.cu:15,153-158)
+ * and allocates its partials inside the call. */
+int mui_flash_decode_splits(int batch, int n_kv_heads, int seq_len_hint);
+size_t mui_flash_decode_scratch_bytes(int batch, int n_q_heads, int head_dim, int n_splits);
+
+/* muillm_causal_transformer_decoding_no_mask / _masked (csrc/module.cpp:276-277;
+ * csrc/attention/flash_decoding.cu:99-325) for one query token per batch row:
+ *   out[b, h*D:(h+1)*D] = softmax_s(q[b,h,:] . K[b, h/(Hq/Hkv), s, :] / sqrt(D)) V[b, h/(Hq/Hkv), s, :]
+ * over s < seq_len. q is dense [batch, n_q_heads, head_dim] (already rotated); out is
+ * [batch, n_q_heads * head_dim]. mask (optional, 16-bit, [batch, >= seq_len] rows
+ * mask_batch_stride apart): 0 keeps key s, any other value drops it
+ * (csrc/attention/flash_decoding_fp16_kernels.cu:386-393); a fully masked row yields 0.
+ * scratch: mui_flash_decode_scratch_bytes() bytes, may be NULL when n_splits == 1. */
+int mui_flash_decode(mui_stream_t stream, int dtype, const void* q, const void* k_cache,
+                     const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                     long cache_token_stride, const void* mask, long mask_batch_stride, int seq_len,
+                     void* scratch, int n_splits, void* out, int batch, int n_q_heads,
+                     int n_kv_heads, int head_dim, int max_cache_len);
+
+/* One call for what the reference does in three (muillm_rotary_embedding_module_forward
+ * csrc/module.cpp:381 -> RoPE + cache write kernel, then the two flash-decoding kernels,
+ * muillm/modules/attention/sdpaattention.py:189-209): rotate q and the new k at
+ * position_ids[b], write rotated k and v into cache slot cache_position[0], and attend over
+ * cache rows [0, seq_len) including the new one. seq_len < 0 means cache_position[0] + 1,
+ * read on the device, so the launch is replayable from a HIP graph as the sequence grows.
+ * q, k_new, v_new: [batch, heads, head_dim] with head stride head_dim and the given batch
+ * strides (views into a fused QKV output). q_out (optional): dense rotated queries. */
+int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                          const void* k_new, long k_batch_stride, const void* v_new,
+                          long v_batch_stride, const float* cos_table, const float* sin_table,
+                          int rope_row_stride, const int64_t* position_ids,
+                          long position_batch_stride, const int64_t* cache_position, int seq_len,
+                          void* k_cache, void* v_cache, long cache_batch_stride,
+                          long cache_head_stride, long cache_token_stride, const void* mask,
+                          long mask_batch_stride, void* q_out, void* scratch, int n_splits,
+                          void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                          int max_cache_len);
+
+/* ------------------------------------------------------------------------------------
+ * Launch-shape knobs used by the benchmark sweeps (0 restores the built-in choice). They
+ * have no counterpart in the reference, whose launch shapes are compile-time constants
+ * (csrc/linear/linear_fp16_kernels.cu:646-654).
+ * ---------------------------------------------------------------------------------- */
+int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
+int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
+
 #ifdef __cplusplus
 }
 #endif

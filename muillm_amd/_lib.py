@@ -49,6 +49,24 @@ _SIGNATURES = {
     "mui_linear": (c_int, [_P, c_int, _P, c_long, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_int]),
     "mui_rmsnorm": (c_int, [_P, c_int, _P, _P, c_float, _P, c_int, c_int]),
     "mui_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
+    "mui_int8_linear": (c_int, [_P, c_int, _P, c_long, _P, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int]),
+    "mui_int8_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
+    "mui_int8_group_linear": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int]),
+    "mui_int8_group_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_long, c_int, _P, _P, c_float, _P, c_int, c_int, c_int]),
+    "mui_int8_dequantize": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, c_int, c_int]),
+    "mui_int8_group_dequantize": (c_int, [_P, c_int, _P, c_long, _P, c_long, c_int, _P, c_long, c_int, c_int]),
+    "mui_rope_kv_write": (c_int, [_P, c_int, _P, c_long, c_long, c_long, _P, c_long, c_long, c_long,
+                                  _P, c_long, c_long, c_long, _P, _P, c_int, _P, c_long, _P, _P, _P, _P,
+                                  c_long, c_long, c_long, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "mui_flash_decode_splits": (c_int, [c_int, c_int, c_int]),
+    "mui_flash_decode_scratch_bytes": (ctypes.c_size_t, [c_int, c_int, c_int, c_int]),
+    "mui_flash_decode": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, _P, c_long, c_int, _P,
+                                 c_int, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, _P,
+                                      c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
+                                      _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mui_tune_gemv": (c_int, [c_int, c_int]),
+    "mui_tune_int8": (c_int, [c_int, c_int]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -1,0 +1,559 @@
+// Decode-time attention for gfx950: flash decoding over a static KV cache with the RoPE of
+// the new token and its cache write-out fused in.
+//
+// Reference counterparts: RoPE + static-cache write (csrc/rope/rotary_fp16_kernels.cu:575-765),
+// cache update (csrc/kvcaches/static_kvcache_xx16_kernels.cu:26-123), flash decoding partial
+// pass and final reduce (csrc/attention/flash_decoding_fp16_kernels.cu:199-586, 642-785).
+//
+// Layout of the work (T = 1 new token per batch row, head_dim 128):
+//   grid = (splits of the cached sequence, KV heads, batch); one workgroup = 4 wave64s.
+//   A workgroup serves ALL G = Hq/Hkv query heads that share its KV head, so K and V are
+//   read from HBM exactly once (the reference re-reads them once per query head).
+//   Inside a wave, the 16 lanes of a DPP row own the 16 x 16-byte chunks of ONE token's K/V
+//   row; the 4 rows of a wave take 4 consecutive tokens, so one load instruction covers 1 KiB
+//   of contiguous cache. q.k is a packed-fp16 dot (v_dot2_f32_f16) reduced over the 16 lanes
+//   with DPP; softmax runs online in fp32 with one rescale per block of U tokens; p.v is
+//   accumulated in fp32. Each DPP row therefore is an independent online-softmax worker over
+//   its tokens; the 16 workers of a workgroup are merged through LDS (log-sum-exp combine),
+//   and workgroups are merged by a small second kernel (fp32 partials, unlike the
+//   reference's fp16 max/denominator).
+//   The new token: every workgroup rotates the G query heads it needs on the fly (fp32 math,
+//   rounded once to the 16-bit type); the workgroup whose split contains the new slot rotates
+//   k, writes k/v into the cache and folds them in from LDS, so no workgroup ever reads the
+//   slot that is being written.
+//   The sequence length can come from device memory (cache_position[0] + 1), which keeps
+//   the launch shape fixed under HIP-graph replay.
+#include "common.cuh"
+
+namespace mui {
+
+constexpr int kHeadDim = 128;
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kWorkers = kAttnWaves * 4;  // DPP rows per workgroup
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct AttnParams {
+  const uint16_t* q;      // [B, Hq, D] (strides below), un-rotated when cos != null
+  long q_bs, q_hs;
+  const uint16_t* k_new;  // [B, Hkv, D] or null (no new token: attend over the cache as is)
+  long k_bs, k_hs;
+  const uint16_t* v_new;
+  long v_bs, v_hs;
+  const float* cos;       // [max_pos, rope_stride] fp32 tables, or null (no rotation)
+  const float* sin;
+  int rope_stride;
+  const int64_t* position_ids;  // rotary position of the new token per batch row, or null
+  long pos_bs;
+  const int64_t* cache_position;  // device scalar: cache slot of the new token
+  int seq_len;            // valid cache length incl. the new token; < 0: cache_position[0] + 1
+  uint16_t* k_cache;      // [B, Hkv, max_t, D]
+  uint16_t* v_cache;
+  long c_bs, c_hs, c_ts;
+  const uint16_t* mask;   // [B, >= seq_len]: 0 keeps a key, anything else drops it; or null
+  long mask_bs;
+  uint16_t* q_out;        // optional dense [B, Hq, D] rotated queries
+  float* part_acc;        // [B, Hq, n_splits, D]
+  float* part_ml;         // [B, Hq, n_splits, 2]
+  uint16_t* out;          // [B, Hq * D]
+  int hq, hkv, n_splits, max_t;
+  float scale_log2;       // log2(e) / sqrt(D)
+};
+
+template <typename T>
+__device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c);
+template <>
+__device__ __forceinline__ float dot2_acc<F16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+template <>
+__device__ __forceinline__ float dot2_acc<BF16>(uint32_t a, uint32_t b, float c) {
+  c = fmaf(BF16::lo(a), BF16::lo(b), c);
+  return fmaf(BF16::hi(a), BF16::hi(b), c);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// rotate-half RoPE of element d of a 128-wide head held at `src` (16-bit), fp32 math:
+//   r = x * cos[d mod 64] + (d < 64 ? -x[d+64] : x[d-64]) * sin[d mod 64]
+template <typename T>
+__device__ __forceinline__ float rope_elem(const uint16_t* src, int d, const float* cos_row,
+                                           const float* sin_row) {
+  const float x = T::one(src[d]);
+  if (cos_row == nullptr) return x;
+  constexpr int half = kHeadDim / 2;
+  const float partner = d < half ? -T::one(src[d + half]) : T::one(src[d - half]);
+  const int f = d & (half - 1);
+  return fmaf(partner, sin_row[f], x * cos_row[f]);
+}
+
+// One block of UU tokens per DPP row: scores, online-softmax update, p.v accumulation.
+template <typename T, int G, int UU>
+__device__ __forceinline__ void attend_block(const u32x4 (&kreg)[UU], const u32x4 (&vreg)[UU],
+                                             const bool (&valid)[UU], const float (&mask_add)[UU],
+                                             const uint32_t (&qreg)[G][4], float scale_log2,
+                                             float (&m)[G], float (&l)[G], float (&acc)[G][8]) {
+  float s2[UU][G];
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float s = dot2_acc<T>(kreg[u].x, qreg[g][0], 0.f);
+      s = dot2_acc<T>(kreg[u].y, qreg[g][1], s);
+      s = dot2_acc<T>(kreg[u].z, qreg[g][2], s);
+      s = dot2_acc<T>(kreg[u].w, qreg[g][3], s);
+      s = row16_sum(s);
+      s2[u][g] = valid[u] ? fmaf(s, scale_log2, mask_add[u]) : -INFINITY;
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float m_new = m[g];
+#pragma unroll
+    for (int u = 0; u < UU; ++u) m_new = fmaxf(m_new, s2[u][g]);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = fast_exp2(m[g] - m_use);
+    float p[UU];
+    float psum = 0.f;
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+      p[u] = fast_exp2(s2[u][g] - m_use);
+      psum += p[u];
+    }
+    l[g] = fmaf(l[g], corr, psum);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] *= corr;
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+      float vf[8];
+      unpack8<T>(vreg[u], vf);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p[u], vf[i], acc[g][i]);
+    }
+    m[g] = m_new;
+  }
+}
+
+template <typename T, int G, int U, bool DIRECT>
+__global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnParams p) {
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[G][kHeadDim];
+  __shared__ __attribute__((aligned(16))) uint16_t kn_lds[kHeadDim];
+  __shared__ __attribute__((aligned(16))) uint16_t vn_lds[kHeadDim];
+  __shared__ float lds_m[kWorkers][G];
+  __shared__ float lds_l[kWorkers][G];
+  __shared__ __attribute__((aligned(16))) float tile[kWorkers][G][kHeadDim];
+
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int ts = lane >> 4;  // DPP row = token sub-index
+  const int dc = lane & 15;  // 16-byte chunk of the head
+  const int wk = wave * 4 + ts;
+
+  const bool has_new = p.k_new != nullptr;
+  const int slot = has_new ? (int)p.cache_position[0] : -1;
+  int S = p.seq_len >= 0 ? p.seq_len : slot + 1;
+  S = S < p.max_t ? S : p.max_t;
+  const long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+
+  constexpr int kBlock = kWorkers * U;  // tokens per workgroup iteration
+  int chunk = (S + p.n_splits - 1) / p.n_splits;
+  chunk = ((chunk + kBlock - 1) / kBlock) * kBlock;
+  const int t_begin = split * chunk;
+  const int t_end = (t_begin + chunk) < S ? (t_begin + chunk) : S;
+  const bool owner = has_new && slot >= t_begin && slot < t_begin + chunk && slot < S;
+
+  const float* cos_row = p.cos ? p.cos + pos * p.rope_stride : nullptr;
+  const float* sin_row = p.sin ? p.sin + pos * p.rope_stride : nullptr;
+
+  // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once) ----
+  for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
+    const int g = e / kHeadDim, d = e % kHeadDim;
+    const int head = kvh * G + g;
+    const uint16_t* qp = p.q + (long)b * p.q_bs + (long)head * p.q_hs;
+    const uint16_t r = T::pack(rope_elem<T>(qp, d, cos_row, sin_row));
+    q_lds[g][d] = r;
+    if (p.q_out && split == 0) p.q_out[((long)b * p.hq + head) * kHeadDim + d] = r;
+  }
+  // ---- the owner of the new slot rotates k, writes k/v to the cache and keeps them in LDS ----
+  if (owner) {
+    const long coff = (long)b * p.c_bs + (long)kvh * p.c_hs + (long)slot * p.c_ts;
+    if (t < kHeadDim) {
+      const uint16_t* kp = p.k_new + (long)b * p.k_bs + (long)kvh * p.k_hs;
+      const uint16_t r = T::pack(rope_elem<T>(kp, t, cos_row, sin_row));
+      kn_lds[t] = r;
+      p.k_cache[coff + t] = r;
+    } else {
+      const int d = t - kHeadDim;
+      const uint16_t v = p.v_new[(long)b * p.v_bs + (long)kvh * p.v_hs + d];
+      vn_lds[d] = v;
+      p.v_cache[coff + d] = v;
+    }
+  }
+  __syncthreads();
+
+  uint32_t qreg[G][4];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const u32x4 qv = *(const u32x4*)&q_lds[g][dc * 8];
+    qreg[g][0] = qv.x; qreg[g][1] = qv.y; qreg[g][2] = qv.z; qreg[g][3] = qv.w;
+  }
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+  }
+
+  const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
+  const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
+  const uint16_t* mrow = p.mask ? p.mask + (long)b * p.mask_bs : nullptr;
+
+  for (int base = t_begin; base < t_end; base += kBlock) {
+    u32x4 kreg[U], vreg[U];
+    bool valid[U];
+    float madd[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int tok = base + u * kWorkers + wk;
+      valid[u] = (tok < t_end) && (tok != slot);
+      const int tk = valid[u] ? tok : t_begin;  // t_begin < S: always a readable row
+      kreg[u] = ld16(kc + (long)tk * p.c_ts);
+      vreg[u] = ld16(vc + (long)tk * p.c_ts);
+      madd[u] = 0.f;
+      if (mrow != nullptr && valid[u]) {
+        if (T::one(mrow[tok]) != 0.f) valid[u] = false;
+      }
+    }
+    attend_block<T, G, U>(kreg, vreg, valid, madd, qreg, p.scale_log2, m, l, acc);
+  }
+
+  if (owner && wave == 0) {  // the new token, straight from LDS, on DPP row 0 of wave 0
+    u32x4 kreg[1], vreg[1];
+    bool valid[1];
+    float madd[1] = {0.f};
+    kreg[0] = *(const u32x4*)&kn_lds[dc * 8];
+    vreg[0] = *(const u32x4*)&vn_lds[dc * 8];
+    valid[0] = (ts == 0);
+    if (mrow != nullptr && T::one(mrow[slot]) != 0.f) valid[0] = false;
+    attend_block<T, G, 1>(kreg, vreg, valid, madd, qreg, p.scale_log2, m, l, acc);
+  }
+
+  // ---- merge the 16 workers of the workgroup ----
+  if (dc == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) lds_m[wk][g] = m[g];
+  }
+  __syncthreads();
+  float f[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float mx = lds_m[0][g];
+#pragma unroll
+    for (int w2 = 1; w2 < kWorkers; ++w2) mx = fmaxf(mx, lds_m[w2][g]);
+    const float m_use = (mx == -INFINITY) ? 0.f : mx;
+    f[g] = fast_exp2(m[g] - m_use);
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    if (dc == 0) lds_l[wk][g] = l[g] * f[g];
+    f32x4 a0 = {acc[g][0] * f[g], acc[g][1] * f[g], acc[g][2] * f[g], acc[g][3] * f[g]};
+    f32x4 a1 = {acc[g][4] * f[g], acc[g][5] * f[g], acc[g][6] * f[g], acc[g][7] * f[g]};
+    *(f32x4*)&tile[wk][g][dc * 8] = a0;
+    *(f32x4*)&tile[wk][g][dc * 8 + 4] = a1;
+  }
+  __syncthreads();
+
+  for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
+    const int g = e / kHeadDim, d = e % kHeadDim;
+    const int head = kvh * G + g;
+    float a = 0.f, lsum = 0.f, mx = lds_m[0][g];
+#pragma unroll
+    for (int w2 = 0; w2 < kWorkers; ++w2) {
+      a += tile[w2][g][d];
+      lsum += lds_l[w2][g];
+      mx = fmaxf(mx, lds_m[w2][g]);
+    }
+    if constexpr (DIRECT) {
+      p.out[((long)b * p.hq + head) * kHeadDim + d] = T::pack(lsum > 0.f ? a / lsum : 0.f);
+    } else {
+      const long pi = ((long)b * p.hq + head) * p.n_splits + split;
+      p.part_acc[pi * kHeadDim + d] = a;
+      if (d == 0) {
+        p.part_ml[pi * 2 + 0] = mx;
+        p.part_ml[pi * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// log-sum-exp merge of the per-split partials: one workgroup of 128 threads per (head, batch)
+template <typename T>
+__global__ void __launch_bounds__(kHeadDim) attn_combine_kernel(const float* part_acc,
+                                                                const float* part_ml,
+                                                                uint16_t* out, int hq, int n_splits) {
+  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const long base = ((long)b * hq + head) * n_splits;
+  float mx = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+  const float m_use = (mx == -INFINITY) ? 0.f : mx;
+  float a = 0.f, lsum = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float w = fast_exp2(part_ml[(base + s) * 2] - m_use);
+    lsum = fmaf(w, part_ml[(base + s) * 2 + 1], lsum);
+    a = fmaf(w, part_acc[(base + s) * kHeadDim + d], a);
+  }
+  out[((long)b * hq + head) * kHeadDim + d] = T::pack(lsum > 0.f ? a / lsum : 0.f);
+}
+
+// RoPE of q (-> q_out) and k (-> cache slot or dense k_out), copy of v, for T tokens.
+// grid = (Hq + 2*Hkv, T, B), 128 threads.
+struct RopeParams {
+  const uint16_t* q; long q_bs, q_ts, q_hs;   // [B, T, Hq, D] by strides; may be null
+  const uint16_t* k; long k_bs, k_ts, k_hs;   // may be null
+  const uint16_t* v; long v_bs, v_ts, v_hs;   // may be null
+  const float* cos; const float* sin; int rope_stride;  // null: no rotation (plain cache update)
+  const int64_t* position_ids; long pos_bs;   // [B, T] (pos_bs = 0 broadcasts one row)
+  const int64_t* cache_position;              // [T] slots; null: k_out/v_out are dense [B, Hkv, T, D]
+  uint16_t* q_out;                            // dense [B, Hq, T, D]
+  uint16_t* k_out; uint16_t* v_out; long c_bs, c_hs, c_ts;
+  int hq, hkv, tokens, max_t;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kHeadDim) rope_kv_write_kernel(const RopeParams p) {
+  const int h = blockIdx.x, tkn = blockIdx.y, b = blockIdx.z, d = threadIdx.x;
+  const float* cos_row = nullptr;
+  const float* sin_row = nullptr;
+  if (p.cos) {
+    const long pos = p.position_ids[(long)b * p.pos_bs + tkn];
+    cos_row = p.cos + pos * p.rope_stride;
+    sin_row = p.sin + pos * p.rope_stride;
+  }
+  if (h < p.hq) {
+    if (p.q == nullptr) return;
+    const uint16_t* src = p.q + (long)b * p.q_bs + (long)tkn * p.q_ts + (long)h * p.q_hs;
+    p.q_out[(((long)b * p.hq + h) * p.tokens + tkn) * kHeadDim + d] = T::pack(rope_elem<T>(src, d, cos_row, sin_row));
+    return;
+  }
+  long slot = tkn;
+  if (p.cache_position) {
+    slot = p.cache_position[tkn];
+    if (slot < 0 || slot >= p.max_t) return;  // out-of-range slots are dropped, never written
+  }
+  if (h < p.hq + p.hkv) {
+    if (p.k == nullptr) return;
+    const int kh = h - p.hq;
+    const uint16_t* src = p.k + (long)b * p.k_bs + (long)tkn * p.k_ts + (long)kh * p.k_hs;
+    p.k_out[(long)b * p.c_bs + (long)kh * p.c_hs + slot * p.c_ts + d] = T::pack(rope_elem<T>(src, d, cos_row, sin_row));
+  } else {
+    if (p.v == nullptr) return;
+    const int vh = h - p.hq - p.hkv;
+    const uint16_t* src = p.v + (long)b * p.v_bs + (long)tkn * p.v_ts + (long)vh * p.v_hs;
+    p.v_out[(long)b * p.c_bs + (long)vh * p.c_hs + slot * p.c_ts + d] = src[d];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+constexpr int kU = 4;
+
+template <typename T, int G>
+static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
+  dim3 grid(p.n_splits, p.hkv, batch), block(kAttnThreads);
+  if (p.n_splits == 1)
+    hipLaunchKernelGGL((attn_decode_kernel<T, G, kU, true>), grid, block, 0, s, p);
+  else
+    hipLaunchKernelGGL((attn_decode_kernel<T, G, kU, false>), grid, block, 0, s, p);
+  int st = launch_status();
+  if (st != MUI_OK) return st;
+  if (p.n_splits > 1) {
+    hipLaunchKernelGGL((attn_combine_kernel<T>), dim3(p.hq, batch), dim3(kHeadDim), 0, s,
+                       (const float*)p.part_acc, (const float*)p.part_ml, p.out, p.hq, p.n_splits);
+    st = launch_status();
+  }
+  return st;
+}
+
+template <typename T>
+static int launch_attn_t(hipStream_t s, const AttnParams& p, int batch) {
+  switch (p.hq / p.hkv) {
+    case 1: return launch_attn_g<T, 1>(s, p, batch);
+    case 2: return launch_attn_g<T, 2>(s, p, batch);
+    case 4: return launch_attn_g<T, 4>(s, p, batch);
+    case 8: return launch_attn_g<T, 8>(s, p, batch);
+    default: return MUI_ERR_UNSUPPORTED;
+  }
+}
+
+static int launch_attn(hipStream_t s, int dtype, const AttnParams& p, int batch) {
+  if (dtype == MUI_DTYPE_F16) return launch_attn_t<F16>(s, p, batch);
+  if (dtype == MUI_DTYPE_BF16) return launch_attn_t<BF16>(s, p, batch);
+  return MUI_ERR_INVALID_ARG;
+}
+
+}  // namespace mui
+
+using namespace mui;
+
+extern "C" int mui_flash_decode_splits(int batch, int n_kv_heads, int seq_len_hint) {
+  if (batch <= 0 || n_kv_heads <= 0 || seq_len_hint <= 0) return 1;
+  constexpr int kBlock = kWorkers * kU;               // tokens per workgroup iteration
+  const int max_useful = ceil_div(seq_len_hint, 2 * kBlock);  // >= 2 iterations per split
+  const int want = ceil_div(4 * device_cus(), batch * n_kv_heads);
+  int n = want < max_useful ? want : max_useful;
+  if (n < 1) n = 1;
+  if (n > 256) n = 256;
+  return n;
+}
+
+extern "C" size_t mui_flash_decode_scratch_bytes(int batch, int n_q_heads, int head_dim, int n_splits) {
+  if (batch <= 0 || n_q_heads <= 0 || head_dim <= 0 || n_splits <= 1) return 0;
+  return (size_t)batch * n_q_heads * n_splits * (head_dim + 2) * sizeof(float);
+}
+
+static int check_attn_shape(int dtype, int batch, int hq, int hkv, int head_dim, int n_splits,
+                            int max_t) {
+  if (!(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16)) return MUI_ERR_INVALID_ARG;
+  if (batch <= 0 || hq <= 0 || hkv <= 0 || n_splits <= 0 || max_t <= 0) return MUI_ERR_INVALID_ARG;
+  if (head_dim != kHeadDim) return MUI_ERR_UNSUPPORTED;
+  if (hq % hkv != 0) return MUI_ERR_INVALID_ARG;
+  const int g = hq / hkv;
+  if (!(g == 1 || g == 2 || g == 4 || g == 8)) return MUI_ERR_UNSUPPORTED;
+  if (batch > 65535 || hkv > 65535) return MUI_ERR_UNSUPPORTED;
+  return MUI_OK;
+}
+
+extern "C" int mui_flash_decode(mui_stream_t stream, int dtype, const void* q, const void* k_cache,
+                                const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                long cache_token_stride, const void* mask, long mask_batch_stride,
+                                int seq_len, void* scratch, int n_splits, void* out, int batch,
+                                int n_q_heads, int n_kv_heads, int head_dim, int max_cache_len) {
+  int st = check_attn_shape(dtype, batch, n_q_heads, n_kv_heads, head_dim, n_splits, max_cache_len);
+  if (st != MUI_OK) return st;
+  MUI_CHECK_ARG(q && k_cache && v_cache && out);
+  MUI_CHECK_ARG(seq_len > 0 && seq_len <= max_cache_len);
+  if (n_splits > 1 && !scratch) return MUI_ERR_INVALID_ARG;
+  if ((cache_token_stride & 7) || (cache_head_stride & 7) || (cache_batch_stride & 7)) return MUI_ERR_ALIGNMENT;
+  if (!aligned16(k_cache) || !aligned16(v_cache)) return MUI_ERR_ALIGNMENT;
+  AttnParams p = {};
+  p.q = (const uint16_t*)q;
+  p.q_bs = (long)n_q_heads * head_dim;
+  p.q_hs = head_dim;
+  p.seq_len = seq_len;
+  p.k_cache = (uint16_t*)k_cache;
+  p.v_cache = (uint16_t*)v_cache;
+  p.c_bs = cache_batch_stride;
+  p.c_hs = cache_head_stride;
+  p.c_ts = cache_token_stride;
+  p.mask = (const uint16_t*)mask;
+  p.mask_bs = mask_batch_stride;
+  p.part_acc = (float*)scratch;
+  p.part_ml = scratch ? (float*)scratch + (size_t)batch * n_q_heads * n_splits * head_dim : nullptr;
+  p.out = (uint16_t*)out;
+  p.hq = n_q_heads;
+  p.hkv = n_kv_heads;
+  p.n_splits = n_splits;
+  p.max_t = max_cache_len;
+  p.scale_log2 = kLog2e / sqrtf((float)head_dim);
+  return launch_attn((hipStream_t)stream, dtype, p, batch);
+}
+
+extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                                     const void* k_new, long k_batch_stride, const void* v_new,
+                                     long v_batch_stride, const float* cos_table, const float* sin_table,
+                                     int rope_row_stride, const int64_t* position_ids,
+                                     long position_batch_stride, const int64_t* cache_position,
+                                     int seq_len, void* k_cache, void* v_cache, long cache_batch_stride,
+                                     long cache_head_stride, long cache_token_stride, const void* mask,
+                                     long mask_batch_stride, void* q_out, void* scratch, int n_splits,
+                                     void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                                     int max_cache_len) {
+  int st = check_attn_shape(dtype, batch, n_q_heads, n_kv_heads, head_dim, n_splits, max_cache_len);
+  if (st != MUI_OK) return st;
+  MUI_CHECK_ARG(q && k_new && v_new && k_cache && v_cache && out && cache_position);
+  MUI_CHECK_ARG((cos_table == nullptr) == (sin_table == nullptr));
+  MUI_CHECK_ARG(seq_len <= max_cache_len);
+  if (cos_table && rope_row_stride < head_dim / 2) return MUI_ERR_INVALID_ARG;
+  if (n_splits > 1 && !scratch) return MUI_ERR_INVALID_ARG;
+  if ((cache_token_stride & 7) || (cache_head_stride & 7) || (cache_batch_stride & 7)) return MUI_ERR_ALIGNMENT;
+  if (!aligned16(k_cache) || !aligned16(v_cache)) return MUI_ERR_ALIGNMENT;
+  AttnParams p = {};
+  p.q = (const uint16_t*)q;
+  p.q_bs = q_batch_stride;
+  p.q_hs = head_dim;
+  p.k_new = (const uint16_t*)k_new;
+  p.k_bs = k_batch_stride;
+  p.k_hs = head_dim;
+  p.v_new = (const uint16_t*)v_new;
+  p.v_bs = v_batch_stride;
+  p.v_hs = head_dim;
+  p.cos = cos_table;
+  p.sin = sin_table;
+  p.rope_stride = rope_row_stride;
+  p.position_ids = position_ids;
+  p.pos_bs = position_batch_stride;
+  p.cache_position = cache_position;
+  p.seq_len = seq_len;
+  p.k_cache = (uint16_t*)k_cache;
+  p.v_cache = (uint16_t*)v_cache;
+  p.c_bs = cache_batch_stride;
+  p.c_hs = cache_head_stride;
+  p.c_ts = cache_token_stride;
+  p.mask = (const uint16_t*)mask;
+  p.mask_bs = mask_batch_stride;
+  p.q_out = (uint16_t*)q_out;
+  p.part_acc = (float*)scratch;
+  p.part_ml = scratch ? (float*)scratch + (size_t)batch * n_q_heads * n_splits * head_dim : nullptr;
+  p.out = (uint16_t*)out;
+  p.hq = n_q_heads;
+  p.hkv = n_kv_heads;
+  p.n_splits = n_splits;
+  p.max_t = max_cache_len;
+  p.scale_log2 = kLog2e / sqrtf((float)head_dim);
+  return launch_attn((hipStream_t)stream, dtype, p, batch);
+}
+
+extern "C" int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                                 long q_token_stride, long q_head_stride, const void* k,
+                                 long k_batch_stride, long k_token_stride, long k_head_stride,
+                                 const void* v, long v_batch_stride, long v_token_stride,
+                                 long v_head_stride, const float* cos_table, const float* sin_table,
+                                 int rope_row_stride, const int64_t* position_ids,
+                                 long position_batch_stride, const int64_t* cache_position, void* q_out,
+                                 void* k_out, void* v_out, long out_batch_stride, long out_head_stride,
+                                 long out_token_stride, int batch, int tokens, int n_q_heads,
+                                 int n_kv_heads, int head_dim, int max_cache_len) {
+  MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
+  MUI_CHECK_ARG(batch > 0 && tokens > 0 && n_q_heads >= 0 && n_kv_heads >= 0 && max_cache_len > 0);
+  MUI_CHECK_ARG((cos_table == nullptr) == (sin_table == nullptr));
+  MUI_CHECK_ARG(!cos_table || position_ids);
+  MUI_CHECK_ARG(!q || q_out);
+  MUI_CHECK_ARG(!k || k_out);
+  MUI_CHECK_ARG(!v || v_out);
+  if (head_dim != kHeadDim) return MUI_ERR_UNSUPPORTED;
+  if (cos_table && rope_row_stride < head_dim / 2) return MUI_ERR_INVALID_ARG;
+  if (tokens > 65535 || batch > 65535) return MUI_ERR_UNSUPPORTED;
+  RopeParams p = {};
+  p.q = (const uint16_t*)q; p.q_bs = q_batch_stride; p.q_ts = q_token_stride; p.q_hs = q_head_stride;
+  p.k = (const uint16_t*)k; p.k_bs = k_batch_stride; p.k_ts = k_token_stride; p.k_hs = k_head_stride;
+  p.v = (const uint16_t*)v; p.v_bs = v_batch_stride; p.v_ts = v_token_stride; p.v_hs = v_head_stride;
+  p.cos = cos_table; p.sin = sin_table; p.rope_stride = rope_row_stride;
+  p.position_ids = position_ids; p.pos_bs = position_batch_stride;
+  p.cache_position = cache_position;
+  p.q_out = (uint16_t*)q_out; p.k_out = (uint16_t*)k_out; p.v_out = (uint16_t*)v_out;
+  p.c_bs = out_batch_stride; p.c_hs = out_head_stride; p.c_ts = out_token_stride;
+  p.hq = q ? n_q_heads : 0; p.hkv = n_kv_heads; p.tokens = tokens; p.max_t = max_cache_len;
+  const int heads = p.hq + 2 * n_kv_heads;
+  if (heads == 0) return MUI_OK;
+  dim3 grid(heads, tokens, batch), block(kHeadDim);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MUI_DTYPE_F16) hipLaunchKernelGGL((rope_kv_write_kernel<F16>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((rope_kv_write_kernel<BF16>), grid, block, 0, s, p);
+  return launch_status();
+}

@@ -152,6 +152,28 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
     if (!(cond)) return MUI_ERR_INVALID_ARG; \
   } while (0)
 
+// number of compute units of the current device (cached; this library drives one GPU)
+static inline int device_cus() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached = cus;
+  }
+  return cached;
+}
+
+// Persistent grid: at most `per_cu` workgroups per CU, and every workgroup gets the same
+// number of work items (a ragged last pass would idle most of the chip for one latency).
+static inline int balanced_grid(int n_items, int per_cu) {
+  const int cap = device_cus() * per_cu;
+  if (n_items <= cap) return n_items;
+  const int iters = ceil_div(n_items, cap);
+  return ceil_div(n_items, iters);
+}
+
 static inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? MUI_OK : MUI_ERR_LAUNCH;

@@ -179,22 +179,10 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvParams p) {
 // host side
 // ---------------------------------------------------------------------------------------
 struct Tuning {
-  int rows_linear = 4;      // R for linear (2 or 4)
-  int wgs_per_cu = 8;       // cap on resident workgroups per CU used to size persistent grids
-  int cus = 0;              // filled on first use
+  int rows_linear = 0;  // 0 = pick per shape; 2 or 4 force R for the linear kernel
+  int wgs_per_cu = 0;   // 0 = pick per shape; else cap on workgroups per CU for persistent grids
 };
 static Tuning g_tune;
-
-static int device_cus() {
-  if (g_tune.cus == 0) {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-      cus = 256;
-    g_tune.cus = cus;
-  }
-  return g_tune.cus;
-}
 
 template <typename T, int R, int CH, int EPI>
 static int launch_rc(hipStream_t s, const GemvParams& p, int grid) {
@@ -206,15 +194,13 @@ static int launch_rc(hipStream_t s, const GemvParams& p, int grid) {
 }
 
 template <typename T, int R, int EPI>
-static int launch_r(hipStream_t s, const GemvParams& p) {
+static int launch_r(hipStream_t s, const GemvParams& p, int ch) {
   constexpr int OUT = (EPI == EPI_GATEUP) ? R / 2 : R;
   const int n_groups = ceil_div(p.n, OUT);
-  const int ch = ceil_div(p.k >> 3, kThreads);
-  // resident workgroups per CU are bounded by registers: ~64 VGPRs up to CH=2, more beyond
-  int per_cu = g_tune.wgs_per_cu;
-  if (ch > 2 && per_cu > 4) per_cu = 4;
-  int grid = device_cus() * per_cu;
-  if (grid > n_groups) grid = n_groups;
+  // measured on MI355X: 2-3 resident workgroups per CU with the next row group prefetched
+  // saturate HBM; more only adds tail imbalance.
+  int per_cu = g_tune.wgs_per_cu > 0 ? g_tune.wgs_per_cu : (ch > 2 ? 2 : 3);
+  const int grid = balanced_grid(n_groups, per_cu);
   if (ch <= 1) return launch_rc<T, R, 1, EPI>(s, p, grid);
   if (ch <= 2) return launch_rc<T, R, 2, EPI>(s, p, grid);
   if (ch <= 4) return launch_rc<T, R, 4, EPI>(s, p, grid);
@@ -223,16 +209,22 @@ static int launch_r(hipStream_t s, const GemvParams& p) {
   return MUI_ERR_UNSUPPORTED;
 }
 
+template <typename T, int EPI>
+static int launch_t(hipStream_t s, const GemvParams& p) {
+  const int ch = ceil_div(p.k >> 3, kThreads);
+  if (EPI == EPI_GATEUP) {
+    // 4 rows = 2 gate/up pairs while a row fits 2 chunks per thread, else one pair
+    return ch > 2 ? launch_r<T, 2, EPI>(s, p, ch) : launch_r<T, 4, EPI>(s, p, ch);
+  }
+  int rows = g_tune.rows_linear;
+  if (rows == 0) rows = ch > 2 ? 2 : 4;  // long rows already give 14+ loads in flight at R=2
+  return rows == 2 ? launch_r<T, 2, EPI>(s, p, ch) : launch_r<T, 4, EPI>(s, p, ch);
+}
+
 template <int EPI>
 static int launch_gemv(hipStream_t s, int dtype, const GemvParams& p) {
-  if (dtype == MUI_DTYPE_F16) {
-    if (EPI == EPI_GATEUP) return launch_r<F16, 4, EPI>(s, p);
-    return g_tune.rows_linear == 2 ? launch_r<F16, 2, EPI>(s, p) : launch_r<F16, 4, EPI>(s, p);
-  }
-  if (dtype == MUI_DTYPE_BF16) {
-    if (EPI == EPI_GATEUP) return launch_r<BF16, 4, EPI>(s, p);
-    return g_tune.rows_linear == 2 ? launch_r<BF16, 2, EPI>(s, p) : launch_r<BF16, 4, EPI>(s, p);
-  }
+  if (dtype == MUI_DTYPE_F16) return launch_t<F16, EPI>(s, p);
+  if (dtype == MUI_DTYPE_BF16) return launch_t<BF16, EPI>(s, p);
   return MUI_ERR_INVALID_ARG;
 }
 
@@ -241,8 +233,10 @@ static int launch_gemv(hipStream_t s, int dtype, const GemvParams& p) {
 using namespace mui;
 
 extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
-  if (rows_linear == 2 || rows_linear == 4) g_tune.rows_linear = rows_linear;
-  if (wgs_per_cu >= 1 && wgs_per_cu <= 16) g_tune.wgs_per_cu = wgs_per_cu;
+  if (!(rows_linear == 0 || rows_linear == 2 || rows_linear == 4)) return MUI_ERR_INVALID_ARG;
+  if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
+  g_tune.rows_linear = rows_linear;
+  g_tune.wgs_per_cu = wgs_per_cu;
   return MUI_OK;
 }
 

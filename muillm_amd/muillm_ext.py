@@ -263,3 +263,449 @@ def muillm_gateupsilu_split_forward(engine, norm_weights, epsilon, gate_weights,
     same path."""
     return muillm_gateupsilu_forward(engine, norm_weights, epsilon, gate_weights, up_weights,
                                      down_weights, residual, x)
+
+
+# --------------------------------------------------------------------------------------
+# int8 weight-only  (csrc/module.cpp:180-181,247-248)
+# --------------------------------------------------------------------------------------
+def _byte_pitch(w: torch.Tensor, name: str) -> int:
+    if w.dim() != 2 or w.stride(1) != 1 or w.element_size() != 1:
+        raise RuntimeError(f"{name} must be a 2-D 8-bit tensor with unit inner stride")
+    return w.stride(0) if w.shape[0] > 1 else max(w.stride(0), w.shape[1])
+
+
+def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
+    return x.is_cuda and _is_16bit(x) and 1 <= _num_tokens(x) <= MUI_MAX_TOKENS and x.shape[-1] % 16 == 0 \
+        and x.shape[-1] <= 16384
+
+
+def mui_int8_channel_dequantize_forward(weights_i8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """Per-channel format: out = T(float(q) * float(s[n])), bit-identical to q.to(T) * s[:, None]."""
+    _check_cuda(weights_i8, "weights")
+    n, k = weights_i8.shape
+    if weights_i8.dtype != torch.int8:
+        raise RuntimeError("per-channel weights must be int8")
+    if k % 16 != 0:
+        return weights_i8.to(scales.dtype) * scales.reshape(-1, 1)
+    out = torch.empty((n, k), dtype=scales.dtype, device=weights_i8.device)
+    sstride = scales.stride(0) if scales.dim() >= 1 and scales.numel() > 1 else 1
+    check(
+        _lib.load().mui_int8_dequantize(_stream(weights_i8), _dtype_code(scales), weights_i8.data_ptr(),
+                                        _byte_pitch(weights_i8, "weights"), scales.data_ptr(), sstride,
+                                        out.data_ptr(), k, n, k),
+        "mui_int8_dequantize",
+    )
+    return out
+
+
+def mui_int8_channel_linear_forward(x, weights_i8, scales, norm_weights=None, epsilon=0.0,
+                                    add_bias=None, residual=None) -> torch.Tensor:
+    """y = (q * s) xn + add_bias + residual on the symmetric per-channel format."""
+    n, k = weights_i8.shape
+    if x.shape[-1] != k:
+        raise RuntimeError(f"input has {x.shape[-1]} features but weights expect {k}")
+    if not int8_kernel_dispatchable(x):
+        w = mui_int8_channel_dequantize_forward(weights_i8, scales)
+        return _linear_unfused(x, w, norm_weights, epsilon, None, add_bias, residual)
+    _check_cuda(weights_i8, "weights")
+    _check_contiguous(scales, "scales")
+    if scales.dtype != x.dtype or scales.numel() != n:
+        raise RuntimeError("scales must be one value per output row in the activation dtype")
+    x = x.contiguous()
+    tokens = _num_tokens(x)
+    if residual is not None:
+        residual = residual.contiguous()
+    y = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
+    check(
+        _lib.load().mui_int8_linear(_stream(x), _dtype_code(x), weights_i8.data_ptr(),
+                                    _byte_pitch(weights_i8, "weights"), scales.data_ptr(), x.data_ptr(),
+                                    _ptr(norm_weights), float(epsilon), _ptr(add_bias), _ptr(residual),
+                                    y.data_ptr(), n, k, tokens),
+        "mui_int8_linear",
+    )
+    return y
+
+
+def mui_int8_channel_gateupsilu_forward(norm_weights, epsilon, gate_i8, up_i8, gate_scales, up_scales, x):
+    """h = silu(sg * Gq xn) * (su * Uq xn); gate/up (and their scales) may be views into
+    row-interleaved [N, 2, K] / [N, 2] buffers."""
+    n, k = gate_i8.shape
+    pitch = _byte_pitch(gate_i8, "gate weights")
+    if _byte_pitch(up_i8, "up weights") != pitch or up_i8.shape != gate_i8.shape:
+        raise RuntimeError("gate and up weights must share shape and row pitch")
+    sstride = gate_scales.stride(0) if gate_scales.numel() > 1 else 1
+    if (up_scales.stride(0) if up_scales.numel() > 1 else 1) != sstride:
+        raise RuntimeError("gate and up scales must share one stride")
+    x = x.contiguous()
+    tokens = _num_tokens(x)
+    h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
+    check(
+        _lib.load().mui_int8_gateup_silu(_stream(x), _dtype_code(x), gate_i8.data_ptr(), up_i8.data_ptr(),
+                                         pitch, gate_scales.data_ptr(), up_scales.data_ptr(), sstride,
+                                         x.data_ptr(), _ptr(norm_weights), float(epsilon), h.data_ptr(),
+                                         n, k, tokens),
+        "mui_int8_gateup_silu",
+    )
+    return h
+
+
+def muillm_int8_dequantize_forward(weights: torch.Tensor, scales_min_vals: torch.Tensor,
+                                   group_size_shift: int) -> torch.Tensor:
+    """Reference RTN group format -> dense 16-bit weights (csrc/module.cpp:180)."""
+    _check_cuda(weights, "weights")
+    n, k = weights.shape
+    g = k >> group_size_shift
+    out = torch.empty((n, k), dtype=scales_min_vals.dtype, device=weights.device)
+    smv = scales_min_vals
+    smv_pitch = 2 * g if smv.is_contiguous() and smv.numel() == n * g * 2 else smv.reshape(n, -1).stride(0)
+    check(
+        _lib.load().mui_int8_group_dequantize(_stream(weights), _dtype_code(smv), weights.data_ptr(),
+                                              _byte_pitch(weights, "weights"), smv.data_ptr(), smv_pitch,
+                                              int(group_size_shift), out.data_ptr(), k, n, k),
+        "mui_int8_group_dequantize",
+    )
+    return out
+
+
+def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, norm_weights=None,
+                               epsilon=0.0, mul_bias=None, add_bias=None, residual=None) -> torch.Tensor:
+    """csrc/module.cpp:181 on the reference's uint8 group format. `residual` is an extension:
+    the reference routes it through add_bias (muillm/modules/quantized/int8linear.py:53-57)."""
+    if mul_bias is not None:
+        raise RuntimeError("mul_bias is not supported by the int8 kernels")
+    n, k = weights.shape
+    if not (int8_kernel_dispatchable(x) and group_size_shift >= 4):
+        w = muillm_int8_dequantize_forward(weights, scales_min_vals, group_size_shift)
+        return _linear_unfused(x, w, norm_weights, epsilon, None, add_bias, residual)
+    if weights.dtype != torch.uint8:
+        raise RuntimeError("group-quantised weights must be uint8")
+    _check_contiguous(scales_min_vals, "scales_min_vals")
+    x = x.contiguous()
+    tokens = _num_tokens(x)
+    if add_bias is not None and add_bias.numel() == tokens * n and residual is None and tokens > 1:
+        residual, add_bias = add_bias, None
+    if residual is not None:
+        residual = residual.contiguous()
+    y = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
+    check(
+        _lib.load().mui_int8_group_linear(_stream(x), _dtype_code(x), weights.data_ptr(),
+                                          _byte_pitch(weights, "weights"), scales_min_vals.data_ptr(),
+                                          int(group_size_shift), x.data_ptr(), _ptr(norm_weights),
+                                          float(epsilon), _ptr(add_bias), _ptr(residual), y.data_ptr(),
+                                          n, k, tokens),
+        "mui_int8_group_linear",
+    )
+    return y
+
+
+def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_up_scales_min_vals,
+                                   group_size_shift, x) -> torch.Tensor:
+    """csrc/module.cpp:248. gate_up_weights is the packed uint8 buffer [N, 2, K] (row n of gate,
+    then row n of up) and gate_up_scales_min_vals is [N, 2, G, 2]; the reference packs per
+    element ([N, K, 2], int8gateupdownmlp.py:211-230), this build per row so that each row
+    stays one contiguous 128-bit-loadable stream."""
+    n, two, k = gate_up_weights.shape
+    if two != 2:
+        raise RuntimeError("gate_up_weights must be [N, 2, K]")
+    g = k >> group_size_shift
+    smv = gate_up_scales_min_vals.reshape(n, 2, g, 2)
+    x = x.contiguous()
+    tokens = _num_tokens(x)
+    h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
+    gw, uw = gate_up_weights[:, 0, :], gate_up_weights[:, 1, :]
+    check(
+        _lib.load().mui_int8_group_gateup_silu(_stream(x), _dtype_code(x), gw.data_ptr(), uw.data_ptr(),
+                                               2 * k, smv[:, 0].data_ptr(), smv[:, 1].data_ptr(), 4 * g,
+                                               int(group_size_shift), x.data_ptr(), _ptr(norm_weights),
+                                               float(epsilon), h.data_ptr(), n, k, tokens),
+        "mui_int8_group_gateup_silu",
+    )
+    return h
+
+
+def muillm_int8_gateupsilu_dequantize_forward(gate_up_weights, gate_up_scales_min_vals, group_size_shift):
+    """csrc/module.cpp:247: packed [N, 2, K] uint8 -> (gate, up) dense 16-bit matrices."""
+    n, _, k = gate_up_weights.shape
+    g = k >> group_size_shift
+    smv = gate_up_scales_min_vals.reshape(n, 2, g, 2)
+    outs = []
+    for s in range(2):
+        w = gate_up_weights[:, s, :]
+        out = torch.empty((n, k), dtype=smv.dtype, device=w.device)
+        check(
+            _lib.load().mui_int8_group_dequantize(_stream(w), _dtype_code(smv), w.data_ptr(), 2 * k,
+                                                  smv[:, s].data_ptr(), 4 * g, int(group_size_shift),
+                                                  out.data_ptr(), k, n, k),
+            "mui_int8_group_dequantize",
+        )
+        outs.append(out)
+    return outs[0], outs[1]
+
+
+# --------------------------------------------------------------------------------------
+# RoPE + static KV cache  (csrc/module.cpp:266-272,357-362,379-381)
+# --------------------------------------------------------------------------------------
+def _f32_table(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype != torch.float32:
+        t = t.float()
+    if t.dim() != 2 or t.stride(1) != 1:
+        t = t.reshape(-1, t.shape[-1]).contiguous()
+    return t
+
+
+def _bhtd_strides(t: torch.Tensor, name: str):
+    """Element strides (batch, token, head) of a [B, H, T, D] tensor with unit inner stride."""
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise RuntimeError(f"{name} must be [B, H, T, D] with unit inner stride")
+    return t.stride(0), t.stride(2), t.stride(1)
+
+
+def _positions(position_ids: torch.Tensor, cos: torch.Tensor, b: int, t: int):
+    """Returns (tables, position_ids[B or 1, T] int64, batch stride). cos/sin given already
+    gathered as [B, T, E] are used as a table indexed by b*T + t
+    (csrc/rope/rotary_position_layout.h:4-9)."""
+    if cos.dim() == 3:
+        rows = cos.shape[0] * cos.shape[1]
+        pos = torch.arange(rows, device=cos.device, dtype=torch.int64).reshape(cos.shape[0], cos.shape[1])
+        return pos, (t if cos.shape[0] > 1 else 0)
+    pos = position_ids.to(torch.int64).reshape(-1, t).contiguous()
+    return pos, (t if pos.shape[0] > 1 else 0)
+
+
+def mui_rope_kv_write(q, k, v, cos, sin, position_ids, cache_position, k_out, v_out, max_cache_len):
+    """q/k/v: [B, H, T, D] views; returns q_out [B, Hq, T, D]. k_out/v_out: caches
+    [B, Hkv, MAX_T, D] (cache_position given) or dense outputs."""
+    ref_t = q if q is not None else k
+    b, _, t, d = ref_t.shape
+    hq = q.shape[1] if q is not None else 0
+    hkv = k.shape[1] if k is not None else (v.shape[1] if v is not None else 0)
+    q_out = torch.empty((b, hq, t, d), dtype=q.dtype, device=q.device) if q is not None else None
+    qs = _bhtd_strides(q, "q") if q is not None else (0, 0, 0)
+    ks = _bhtd_strides(k, "k") if k is not None else (0, 0, 0)
+    vs = _bhtd_strides(v, "v") if v is not None else (0, 0, 0)
+    pos, pos_bs = (None, 0)
+    cos32 = sin32 = None
+    if cos is not None:
+        pos, pos_bs = _positions(position_ids, cos, b, t)
+        cos32, sin32 = _f32_table(cos), _f32_table(sin)
+    out_ref = k_out if k_out is not None else v_out
+    if out_ref is not None:
+        if out_ref.dim() != 4 or out_ref.stride(3) != 1:
+            raise RuntimeError("k/v outputs must be [B, H, T, D] with unit inner stride")
+        ob, oh, ot = out_ref.stride(0), out_ref.stride(1), out_ref.stride(2)
+        if k_out is not None and v_out is not None and k_out.stride() != v_out.stride():
+            raise RuntimeError("k and v outputs must share strides")
+    else:
+        ob = oh = ot = 0
+    if cache_position is not None:
+        cache_position = cache_position.to(torch.int64).contiguous()
+    check(
+        _lib.load().mui_rope_kv_write(
+            _stream(ref_t), _dtype_code(ref_t),
+            _ptr(q), qs[0], qs[1], qs[2], _ptr(k), ks[0], ks[1], ks[2], _ptr(v), vs[0], vs[1], vs[2],
+            _ptr(cos32), _ptr(sin32), cos32.stride(0) if cos32 is not None else 0,
+            _ptr(pos), pos_bs, _ptr(cache_position), _ptr(q_out), _ptr(k_out), _ptr(v_out), ob, oh, ot,
+            b, t, hq, hkv, d, int(max_cache_len)),
+        "mui_rope_kv_write",
+    )
+    return q_out
+
+
+def muillm_rope_forward_no_cache(position_ids, cos_cached, sin_cached, q, k) -> Tuple[torch.Tensor, torch.Tensor]:
+    """csrc/module.cpp:266: rotated (q, k) as dense [B, H, T, D]."""
+    b, hk, t, d = k.shape
+    k_out = torch.empty((b, hk, t, d), dtype=k.dtype, device=k.device)
+    q_out = mui_rope_kv_write(q, k, None, cos_cached, sin_cached, position_ids, None, k_out, None, t)
+    return q_out, k_out
+
+
+def muillm_static_kvcache_update(k_cache, v_cache, k, v, cache_position, seen_tokens: int):
+    """csrc/module.cpp:272: scatter new k/v rows at cache_position (no rotation), return the
+    caches narrowed to `seen_tokens`."""
+    mui_rope_kv_write(None, k, v, None, None, None, cache_position, k_cache, v_cache, k_cache.shape[2])
+    return k_cache.narrow(2, 0, seen_tokens), v_cache.narrow(2, 0, seen_tokens)
+
+
+def muillm_rope_forward_static_cache(position_ids, cos_cached, sin_cached, q, k, v, k_cache, v_cache,
+                                     cache_position, seen_tokens: int):
+    """csrc/module.cpp:268: rotate q and k, write rotated k and v into the static cache at
+    cache_position, return (q_rot, k_cache[:, :, :seen], v_cache[:, :, :seen])."""
+    q_out = mui_rope_kv_write(q, k, v, cos_cached, sin_cached, position_ids, cache_position,
+                              k_cache, v_cache, k_cache.shape[2])
+    return q_out, k_cache.narrow(2, 0, seen_tokens), v_cache.narrow(2, 0, seen_tokens)
+
+
+class MuiStaticKVCacheHandle:
+    """Stand-in for the C++ MuillmStaticKVCache (csrc/modules/static_kvcache.cpp:3-49,
+    csrc/modules/kvcache.h:13-48): aliases the per-layer cache tensors, mirrors seen_tokens."""
+
+    def __init__(self, engine, key_cache: List[torch.Tensor], value_cache: List[torch.Tensor], seen_tokens: int):
+        self.engine = engine
+        self.key_cache = key_cache
+        self.value_cache = value_cache
+        self.seen_tokens = int(seen_tokens)
+
+
+def muillm_static_kvcache_module_init(engine, key_cache, value_cache, seen_tokens):
+    return MuiStaticKVCacheHandle(engine, key_cache, value_cache, seen_tokens)
+
+
+def muillm_static_kvcache_module_deinit(module: MuiStaticKVCacheHandle) -> None:
+    module.key_cache = module.value_cache = None
+
+
+def muillm_static_kvcache_module_sync_back(module: MuiStaticKVCacheHandle):
+    return module.key_cache, module.value_cache
+
+
+def muillm_kvcache_module_get_set_seen_tokens(module: MuiStaticKVCacheHandle, seen_tokens: int) -> int:
+    """Keeps the larger of the two counters (csrc/modules/kvcache.h:27-33)."""
+    module.seen_tokens = max(module.seen_tokens, int(seen_tokens))
+    return module.seen_tokens
+
+
+class MuiRotaryModuleHandle:
+    """Stand-in for MuillmRotaryEmbedding (csrc/modules/rotary_module.cpp:25-125)."""
+
+    def __init__(self, engine, layer_idx, cos_cached, sin_cached):
+        self.engine = engine
+        self.layer_idx = layer_idx
+        self.cos_cached = cos_cached
+        self.sin_cached = sin_cached
+        self.cos32 = _f32_table(cos_cached)
+        self.sin32 = _f32_table(sin_cached)
+
+
+def muillm_rotary_embedding_module_init(engine, layer_idx, cos_cached, sin_cached):
+    return MuiRotaryModuleHandle(engine, layer_idx, cos_cached, sin_cached)
+
+
+def muillm_rotary_embedding_module_deinit(module: MuiRotaryModuleHandle) -> None:
+    module.cos_cached = module.sin_cached = module.cos32 = module.sin32 = None
+
+
+def muillm_rotary_embedding_module_forward(module, cache, q, k, v, position_ids, cos_sin, cache_positions):
+    """csrc/module.cpp:381 / rotary_module.cpp:25-94: bump seen_tokens on layer 0, rotate,
+    write the cache, return (q_rot, k_view, v_view). The module's own fp32 tables indexed by
+    position_ids are used (same values as cos_sin, without the 16-bit rounding)."""
+    t = k.shape[2]
+    if module.layer_idx == 0:
+        cache.seen_tokens += t
+    k_cache = cache.key_cache[module.layer_idx]
+    v_cache = cache.value_cache[module.layer_idx]
+    if position_ids is not None:
+        cos, sin = module.cos32, module.sin32
+    else:
+        cos, sin = cos_sin
+    q_out = mui_rope_kv_write(q, k, v, cos, sin, position_ids, cache_positions, k_cache, v_cache,
+                              k_cache.shape[2])
+    seen = cache.seen_tokens
+    return q_out, k_cache.narrow(2, 0, seen), v_cache.narrow(2, 0, seen)
+
+
+# --------------------------------------------------------------------------------------
+# Decode attention  (csrc/module.cpp:276-277)
+# --------------------------------------------------------------------------------------
+def _cache_strides(k: torch.Tensor, v: torch.Tensor):
+    if k.dim() != 4 or k.stride(3) != 1 or v.stride(3) != 1:
+        raise RuntimeError("k innermost stride must be 1")
+    if k.stride() != v.stride():
+        raise RuntimeError("k and v strides must match")
+    return k.stride(0), k.stride(1), k.stride(2)
+
+
+def _scratch(lib, x: torch.Tensor, b: int, hq: int, d: int, n_splits: int) -> Optional[torch.Tensor]:
+    nbytes = lib.mui_flash_decode_scratch_bytes(b, hq, d, n_splits)
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
+
+
+def _decode(q, k, v, m, n_splits=None) -> torch.Tensor:
+    lib = _lib.load()
+    _check_cuda(q, "q")
+    _check_cuda(k, "k")
+    _check_cuda(v, "v")
+    _check_contiguous(q, "q")
+    b, hq, t, d = q.shape
+    if t != 1:
+        raise RuntimeError("T > 1 not supported")
+    hkv, s = k.shape[1], k.shape[2]
+    cb, chs, cts = _cache_strides(k, v)
+    mask_ptr, mask_bs = None, 0
+    if m is not None:
+        _check_cuda(m, "m")
+        m = m.reshape(b, -1)
+        if m.shape[1] < s or m.dtype != q.dtype:
+            raise RuntimeError("mask must be [B, 1, 1, S] in the query dtype")
+        m = m.contiguous()
+        mask_ptr, mask_bs = m.data_ptr(), m.stride(0)
+    if n_splits is None:
+        n_splits = lib.mui_flash_decode_splits(b, hkv, s)
+    scratch = _scratch(lib, q, b, hq, d, n_splits)
+    out = torch.empty((b, 1, hq * d), dtype=q.dtype, device=q.device)
+    # max_cache_len: rows reachable through the view (the view is narrowed to s already)
+    check(
+        lib.mui_flash_decode(_stream(q), _dtype_code(q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                             cb, chs, cts, mask_ptr, mask_bs, s, _ptr(scratch), n_splits, out.data_ptr(),
+                             b, hq, hkv, d, s),
+        "mui_flash_decode",
+    )
+    return out
+
+
+def muillm_causal_transformer_decoding_no_mask(q, k, v, n_splits=None) -> torch.Tensor:
+    """q [B, Hq, 1, D] contiguous (rotated), k/v [B, Hkv, S, D] cache views -> [B, 1, Hq*D]."""
+    return _decode(q, k, v, None, n_splits)
+
+
+def muillm_causal_transformer_decoding_masked(q, k, v, m, n_splits=None) -> torch.Tensor:
+    """As above with a [B, 1, 1, S] mask: 0 keeps a key, anything else drops it."""
+    return _decode(q, k, v, m, n_splits)
+
+
+def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_position, k_cache, v_cache,
+                               seq_len: Optional[int] = None, mask=None, n_splits: Optional[int] = None,
+                               seq_len_hint: Optional[int] = None, want_q_out: bool = False):
+    """RoPE(q, k) + cache write + flash decoding in one call.
+
+    q [B, Hq*D], k/v [B, Hkv*D]: un-rotated rows of the new token (views into the fused QKV
+    output are fine: unit inner stride, any batch stride). cos32/sin32: fp32 tables.
+    position_ids [B] or [B, 1] int64 (device), cache_position [1] int64 (device).
+    seq_len=None reads the length from cache_position on the device (graph-replayable);
+    the split count then comes from seq_len_hint (default: cache capacity)."""
+    lib = _lib.load()
+    b = q.shape[0]
+    q2, k2, v2 = q.reshape(b, -1), k.reshape(b, -1), v.reshape(b, -1)
+    for name, tns in (("q", q2), ("k", k2), ("v", v2)):
+        _check_cuda(tns, name)
+        if tns.stride(1) != 1:
+            raise RuntimeError(f"{name} must have unit inner stride")
+    hkv, max_t, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    hq = q2.shape[1] // d
+    cb, chs, cts = _cache_strides(k_cache, v_cache)
+    pos = position_ids.reshape(-1)
+    if pos.dtype != torch.int64 or cache_position.dtype != torch.int64:
+        raise RuntimeError("position_ids and cache_position must be int64")
+    pos_bs = 1 if pos.numel() > 1 else 0
+    mask_ptr, mask_bs = None, 0
+    if mask is not None:
+        mask = mask.reshape(b, -1).contiguous()
+        mask_ptr, mask_bs = mask.data_ptr(), mask.stride(0)
+    if n_splits is None:
+        hint = seq_len if seq_len is not None else (seq_len_hint if seq_len_hint is not None else max_t)
+        n_splits = lib.mui_flash_decode_splits(b, hkv, int(hint))
+    scratch = _scratch(lib, q2, b, hq, d, n_splits)
+    out = torch.empty((b, 1, hq * d), dtype=q.dtype, device=q.device)
+    q_out = torch.empty((b, hq, 1, d), dtype=q.dtype, device=q.device) if want_q_out else None
+    bs = lambda tns: tns.stride(0) if b > 1 else tns.shape[1]
+    check(
+        lib.mui_attn_decode_fused(
+            _stream(q2), _dtype_code(q2), q2.data_ptr(), bs(q2), k2.data_ptr(), bs(k2), v2.data_ptr(), bs(v2),
+            _ptr(cos32), _ptr(sin32), cos32.stride(0) if cos32 is not None else 0,
+            pos.data_ptr(), pos_bs, cache_position.data_ptr(), -1 if seq_len is None else int(seq_len),
+            k_cache.data_ptr(), v_cache.data_ptr(), cb, chs, cts, mask_ptr, mask_bs, _ptr(q_out),
+            _ptr(scratch), n_splits, out.data_ptr(), b, hq, hkv, d, max_t),
+        "mui_attn_decode_fused",
+    )
+    return (out, q_out) if want_q_out else out

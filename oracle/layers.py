@@ -327,13 +327,22 @@ def decode_attention(q, k, v, mask=None, reference_path: bool = False):
         w = F.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
         o = torch.matmul(w, vv)
         return o.transpose(1, 2).contiguous().reshape(b, t, hq * d)
-    qh, kk, vv = _hi(q), repeat_kv(_hi(k), n_rep), repeat_kv(_hi(v), n_rep)
-    w = torch.matmul(qh, kk.transpose(2, 3)) / math.sqrt(d)
-    if mask is not None:
-        w = w + _hi(mask)
-    w = F.softmax(w, dim=-1)
-    o = torch.matmul(w, vv)
-    return o.transpose(1, 2).contiguous().reshape(b, t, hq * d)
+    # Same arithmetic without materialising the repeated K/V: query heads are grouped per
+    # KV head ([Hkv, n_rep*T, D] x [Hkv, D, S]); one batch row at a time to bound memory.
+    hkv, s = k.shape[1], k.shape[2]
+    outs = []
+    for bi in range(b):
+        qh = _hi(q[bi]).reshape(hkv, n_rep * t, d)
+        kh, vh = _hi(k[bi]), _hi(v[bi])
+        w = torch.matmul(qh, kh.transpose(1, 2)) / math.sqrt(d)  # [Hkv, n_rep*T, S]
+        if mask is not None:
+            mb = _hi(mask[bi] if mask.shape[0] > 1 else mask[0])  # [1 or Hq, T, S]
+            mb = mb.expand(hq, t, s).reshape(hkv, n_rep * t, s)
+            w = w + mb
+        w = F.softmax(w, dim=-1)
+        o = torch.matmul(w, vh).reshape(hq, t, d)
+        outs.append(o.transpose(0, 1).reshape(t, hq * d))
+    return torch.stack(outs, dim=0)
 
 
 # --------------------------------------------------------------------------------------

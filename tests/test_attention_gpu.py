@@ -1,0 +1,300 @@
+"""GPU parity of RoPE + static-cache write + flash decoding (config 4) through the C ABI.
+
+Gates: attention outputs within 2e-3 absolute of the high-precision oracle; the cache slot
+written by the fused kernel is bit-identical to the standalone rotation; every other cache
+slot is untouched.  The reference has no test for these kernels; the recipes here are the
+closed forms of softmax attention plus the prefill-then-decode sequence of the reference's
+static-cache test (tests/test_static_kvcache.py:52-112 there)."""
+
+import math
+
+import pytest
+import torch
+
+import oracle
+from muillm_amd import _lib, muillm_ext
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+D = 128
+ATOL = 2e-3
+
+
+def _gen(seed=0):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def _mk(shape, g, std=1.0, dtype=torch.float16):
+    return (std * torch.randn(shape, generator=g)).to(dtype)
+
+
+def _max_abs(got, ref):
+    return float((got.detach().cpu().double().reshape(-1) - ref.double().reshape(-1)).abs().max())
+
+
+# ------------------------------------------------------------------------------------
+# standalone RoPE / cache write
+# ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("b,t,hq,hkv", [(1, 1, 32, 8), (2, 5, 8, 2), (1, 64, 32, 8), (8, 1, 32, 8)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_rope_no_cache(b, t, hq, hkv, dtype):
+    g = _gen(0)
+    cos, sin = oracle.rope_tables(500000.0, D, 4096)
+    qkv = _mk((b, t, (hq + 2 * hkv) * D), g, dtype=dtype).to(DEV)  # fused-QKV-like buffer
+    q = qkv[..., : hq * D].view(b, t, hq, D).transpose(1, 2)       # strided views
+    k = qkv[..., hq * D : (hq + hkv) * D].view(b, t, hkv, D).transpose(1, 2)
+    pos = torch.randint(0, 4096, (b, t), generator=g)
+    rq, rk = oracle.apply_rope(q.cpu(), k.cpu(), cos, sin, pos)
+    q_out, k_out = muillm_ext.muillm_rope_forward_no_cache(pos.to(DEV), cos.to(DEV), sin.to(DEV), q, k)
+    assert q_out.shape == (b, hq, t, D) and q_out.is_contiguous() and k_out.shape == (b, hkv, t, D)
+    tol = 2.5e-3 if dtype == torch.float16 else 2e-2  # half an ulp at |x| <= 4
+    assert _max_abs(q_out, rq) <= tol * max(1.0, float(rq.abs().max()) / 4)
+    assert _max_abs(k_out, rk) <= tol * max(1.0, float(rk.abs().max()) / 4)
+    # exact rounding: equals the fp64 result rounded once, up to 1 ulp flips
+    ulp_off = (q_out.cpu().view(torch.int16).int() - rq.to(dtype).view(torch.int16).int()).abs().max()
+    assert int(ulp_off) <= 1
+
+
+def test_rope_invariants():
+    g = _gen(1)
+    cos, sin = oracle.rope_tables(500000.0, D, 1024)
+    q = _mk((1, 4, 1, D), g).to(DEV)
+    k = _mk((1, 4, 1, D), g).to(DEV)
+    z = torch.zeros(1, 1, dtype=torch.int64, device=DEV)
+    q0, k0 = muillm_ext.muillm_rope_forward_no_cache(z, cos.to(DEV), sin.to(DEV), q, k)
+    assert torch.equal(q0, q) and torch.equal(k0, k)  # position 0 is the identity
+    # relative-position property: <rope(q, m), rope(k, n)> depends on m - n only
+    def dots(m, n):
+        pm = torch.full((1, 1), m, dtype=torch.int64, device=DEV)
+        pn = torch.full((1, 1), n, dtype=torch.int64, device=DEV)
+        qm, _ = muillm_ext.muillm_rope_forward_no_cache(pm, cos.to(DEV), sin.to(DEV), q, k)
+        _, kn = muillm_ext.muillm_rope_forward_no_cache(pn, cos.to(DEV), sin.to(DEV), q, k)
+        return (qm.float() * kn.float()).sum(-1)
+    assert torch.allclose(dots(10, 3), dots(507, 500), atol=0.15)
+    # norms of the (i, i + D/2) pairs are preserved
+    p = torch.full((1, 1), 777, dtype=torch.int64, device=DEV)
+    qr, _ = muillm_ext.muillm_rope_forward_no_cache(p, cos.to(DEV), sin.to(DEV), q, k)
+    n0 = q.float()[..., :64] ** 2 + q.float()[..., 64:] ** 2
+    n1 = qr.float()[..., :64] ** 2 + qr.float()[..., 64:] ** 2
+    assert torch.allclose(n0, n1, rtol=5e-3, atol=5e-3)
+
+
+def test_static_cache_prefill_then_decode():
+    """Prefill 64 tokens, then 16 single-token updates: the narrowed views equal the
+    concatenation of everything written (reference tests/test_static_kvcache.py:52-112),
+    slots never written stay zero."""
+    g = _gen(2)
+    b, hkv, cap = 2, 8, 128
+    k_cache = torch.zeros(b, hkv, cap, D, dtype=torch.float16, device=DEV)
+    v_cache = torch.zeros_like(k_cache)
+    ks, vs, seen = [], [], 0
+    for step, t in enumerate([64] + [1] * 16):
+        k = _mk((b, hkv, t, D), g).to(DEV)
+        v = _mk((b, hkv, t, D), g).to(DEV)
+        cp = torch.arange(seen, seen + t, device=DEV)
+        seen += t
+        kv, vv = muillm_ext.muillm_static_kvcache_update(k_cache, v_cache, k, v, cp, seen)
+        ks.append(k)
+        vs.append(v)
+        assert kv.shape == (b, hkv, seen, D)
+        assert torch.equal(kv, torch.cat(ks, dim=2)) and torch.equal(vv, torch.cat(vs, dim=2))
+    assert not k_cache[:, :, seen:].any() and not v_cache[:, :, seen:].any()
+    # out-of-range slots are ignored rather than written
+    bad = torch.tensor([cap + 5], device=DEV)
+    before = k_cache.clone()
+    muillm_ext.muillm_static_kvcache_update(k_cache, v_cache, ks[-1], vs[-1], bad, seen)
+    assert torch.equal(before, k_cache)
+
+
+# ------------------------------------------------------------------------------------
+# flash decoding over an existing cache
+# ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("b,hq,hkv,s,cap", [
+    (1, 32, 8, 1, 16), (1, 32, 8, 5, 8), (1, 32, 8, 63, 64), (2, 32, 8, 64, 128), (1, 32, 8, 65, 128),
+    (1, 32, 8, 1024, 1024), (3, 32, 8, 1000, 1024), (8, 32, 8, 1024, 2048),
+    (1, 8, 8, 300, 512), (1, 16, 8, 300, 512), (2, 64, 8, 300, 512),
+])
+@pytest.mark.parametrize("splits", [None, 1, 7])
+def test_flash_decode(b, hq, hkv, s, cap, splits):
+    g = _gen(3)
+    q = _mk((b, hq, 1, D), g)
+    kc = _mk((b, hkv, cap, D), g)
+    vc = _mk((b, hkv, cap, D), g)
+    kc[:, :, s:] = float("nan")  # anything beyond the sequence must never be read
+    vc[:, :, s:] = float("nan")
+    ref = oracle.decode_attention(q, kc[:, :, :s], vc[:, :, :s])
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = muillm_ext.muillm_causal_transformer_decoding_no_mask(q.to(DEV), kd[:, :, :s], vd[:, :, :s], n_splits=splits)
+    assert out.shape == (b, 1, hq * D)
+    assert torch.isfinite(out).all()
+    assert _max_abs(out, ref) <= ATOL
+
+
+@pytest.mark.parametrize("b,s", [(1, 4096), (4, 16384), (1, 32768), (8, 4096)])
+def test_flash_decode_config4_lengths(b, s):
+    g = _gen(4)
+    hq, hkv = 32, 8
+    cap = oracle.next_pow2(s)
+    q = _mk((b, hq, 1, D), g)
+    kc = _mk((b, hkv, cap, D), g)
+    vc = _mk((b, hkv, cap, D), g)
+    ref = oracle.decode_attention(q, kc[:, :, :s], vc[:, :, :s])
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = muillm_ext.muillm_causal_transformer_decoding_no_mask(q.to(DEV), kd[:, :, :s], vd[:, :, :s])
+    assert _max_abs(out, ref) <= ATOL
+    # split-count invariance (size-independent property)
+    out1 = muillm_ext.muillm_causal_transformer_decoding_no_mask(q.to(DEV), kd[:, :, :s], vd[:, :, :s], n_splits=3)
+    assert _max_abs(out1, out.cpu()) <= 1e-3
+
+
+def test_flash_decode_closed_forms():
+    g = _gen(5)
+    hq, hkv, s = 32, 8, 200
+    q = _mk((1, hq, 1, D), g).to(DEV)
+    v = _mk((1, hkv, s, D), g).to(DEV)
+    # S = 1 -> out = v0 exactly
+    out = muillm_ext.muillm_causal_transformer_decoding_no_mask(q, v[:, :, :1].contiguous(), v[:, :, :1].contiguous())
+    assert torch.equal(out.view(hq, D), v[0, :, 0].repeat_interleave(4, dim=0))
+    # identical keys -> uniform weights -> mean of V
+    k_same = _mk((1, hkv, 1, D), g).to(DEV).expand(1, hkv, s, D).contiguous()
+    out = muillm_ext.muillm_causal_transformer_decoding_no_mask(q, k_same, v)
+    mean_v = v.float().mean(2)[0].repeat_interleave(4, dim=0)
+    assert (out.view(hq, D).float() - mean_v).abs().max() <= ATOL
+    # one dominant key -> its value; heads 4j..4j+3 share KV head j
+    k = torch.zeros(1, hkv, s, D, dtype=torch.float16, device=DEV)
+    qq = torch.zeros(1, hq, 1, D, dtype=torch.float16, device=DEV)
+    qq[..., 0] = 30.0
+    for j in range(hkv):
+        k[0, j, 10 + j, 0] = 30.0
+    out = muillm_ext.muillm_causal_transformer_decoding_no_mask(qq, k, v).view(hq, D)
+    for h in range(hq):
+        assert (out[h].float() - v[0, h // 4, 10 + h // 4].float()).abs().max() <= ATOL
+
+
+def test_flash_decode_masked():
+    g = _gen(6)
+    b, hq, hkv, s = 2, 32, 8, 333
+    q, k, v = _mk((b, hq, 1, D), g), _mk((b, hkv, s, D), g), _mk((b, hkv, s, D), g)
+    drop = torch.rand(b, s, generator=g) < 0.3
+    drop[0, :40] = True  # left padding
+    drop[:, -1] = False
+    minv = torch.finfo(torch.float16).min
+    m = torch.zeros(b, 1, 1, s, dtype=torch.float16)
+    m[drop[:, None, None, :]] = minv
+    add = torch.zeros(b, 1, 1, s, dtype=torch.float64)
+    add[drop[:, None, None, :]] = float("-inf")
+    ref = oracle.decode_attention(q, k, v, add)
+    out = muillm_ext.muillm_causal_transformer_decoding_masked(q.to(DEV), k.to(DEV), v.to(DEV), m.to(DEV))
+    assert _max_abs(out, ref) <= ATOL
+    out7 = muillm_ext.muillm_causal_transformer_decoding_masked(q.to(DEV), k.to(DEV), v.to(DEV), m.to(DEV), n_splits=5)
+    assert _max_abs(out7, ref) <= ATOL
+
+
+# ------------------------------------------------------------------------------------
+# fused RoPE + cache write + decode
+# ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("b,s,cap", [(1, 1, 16), (1, 33, 64), (2, 257, 512), (1, 1024, 1024), (4, 4096, 4096), (8, 1000, 1024)])
+@pytest.mark.parametrize("device_len", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_decode(b, s, cap, device_len, dtype):
+    """Config 4 recipe: cache pre-filled for s-1 positions, new token at position s-1."""
+    if dtype == torch.bfloat16 and s > 1024:
+        pytest.skip("bf16 twin covered at the smaller shapes")
+    g = _gen(7)
+    hq, hkv = 32, 8
+    cos, sin = oracle.rope_tables(500000.0, D, cap)
+    qkv = _mk((b, 1, (hq + 2 * hkv) * D), g, dtype=dtype)
+    kc = torch.zeros(b, hkv, cap, D, dtype=dtype)
+    vc = torch.zeros(b, hkv, cap, D, dtype=dtype)
+    kc[:, :, : s - 1] = _mk((b, hkv, s - 1, D), g, dtype=dtype)
+    vc[:, :, : s - 1] = _mk((b, hkv, s - 1, D), g, dtype=dtype)
+    pos = torch.full((b, 1), s - 1, dtype=torch.int64)
+    cpos = torch.tensor([s - 1], dtype=torch.int64)
+
+    q = qkv[..., : hq * D].view(b, 1, hq, D).transpose(1, 2)
+    k = qkv[..., hq * D : (hq + hkv) * D].view(b, 1, hkv, D).transpose(1, 2)
+    v = qkv[..., (hq + hkv) * D :].view(b, 1, hkv, D).transpose(1, 2)
+    rq, rk = oracle.apply_rope(q, k, cos, sin, pos)
+    rq, rk = rq.to(dtype), rk.to(dtype)
+    kref, vref = kc.clone(), vc.clone()
+    kk, vv, _ = oracle.static_cache_update(kref, vref, rk, v, cpos, s - 1)
+    ref = oracle.decode_attention(rq, kk, vv)
+
+    qkv_d, kd, vd = qkv.to(DEV), kc.to(DEV), vc.to(DEV)
+    qd = qkv_d[:, 0, : hq * D]
+    kn = qkv_d[:, 0, hq * D : (hq + hkv) * D]
+    vn = qkv_d[:, 0, (hq + hkv) * D :]
+    out, q_out = muillm_ext.mui_attention_decode_fused(
+        qd, kn, vn, cos.to(DEV), sin.to(DEV), pos.to(DEV), cpos.to(DEV), kd, vd,
+        seq_len=None if device_len else s, seq_len_hint=s, want_q_out=True)
+    tol = ATOL if dtype == torch.float16 else 1.5e-2
+    assert out.shape == (b, 1, hq * D)
+    assert _max_abs(out, ref) <= tol
+
+    # the written slot is bit-identical to the standalone rotation; all other slots untouched
+    q_sa, k_sa = muillm_ext.muillm_rope_forward_no_cache(
+        pos.to(DEV), cos.to(DEV), sin.to(DEV),
+        qkv_d[..., : hq * D].view(b, 1, hq, D).transpose(1, 2),
+        qkv_d[..., hq * D : (hq + hkv) * D].view(b, 1, hkv, D).transpose(1, 2))
+    assert torch.equal(kd[:, :, s - 1], k_sa[:, :, 0])
+    assert torch.equal(q_out, q_sa)
+    assert torch.equal(vd[:, :, s - 1].cpu(), v[:, :, 0])
+    keep = torch.ones(cap, dtype=torch.bool)
+    keep[s - 1] = False
+    assert torch.equal(kd.cpu()[:, :, keep], kc[:, :, keep]) and torch.equal(vd.cpu()[:, :, keep], vc[:, :, keep])
+    # 1-ulp agreement of the slot with the oracle's rotation rounded once
+    off = (kd[:, :, s - 1].cpu().view(torch.int16).int() - rk[:, :, 0].view(torch.int16).int()).abs().max()
+    assert int(off) <= 1
+
+
+def test_fused_decode_sequence_matches_oracle_steps():
+    """Eight consecutive decode steps with the length read from device memory: the cache
+    grows in place and every step matches the oracle run on the same growing cache."""
+    g = _gen(8)
+    b, hq, hkv, cap, start = 2, 32, 8, 128, 37
+    cos, sin = oracle.rope_tables(500000.0, D, cap)
+    kc = torch.zeros(b, hkv, cap, D, dtype=torch.float16)
+    vc = torch.zeros_like(kc)
+    kc[:, :, :start] = _mk((b, hkv, start, D), g)
+    vc[:, :, :start] = _mk((b, hkv, start, D), g)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    cpos_d = torch.tensor([start], dtype=torch.int64, device=DEV)
+    pos_d = torch.full((b,), start, dtype=torch.int64, device=DEV)
+    cosd, sind = cos.to(DEV), sin.to(DEV)
+    seen = start
+    for step in range(8):
+        qkv = _mk((b, (hq + 2 * hkv) * D), g)
+        qkv_d = qkv.to(DEV)
+        out = muillm_ext.mui_attention_decode_fused(
+            qkv_d[:, : hq * D], qkv_d[:, hq * D : (hq + hkv) * D], qkv_d[:, (hq + hkv) * D :],
+            cosd, sind, pos_d, cpos_d, kd, vd, seq_len=None, n_splits=2)
+        pos = torch.full((b, 1), seen, dtype=torch.int64)
+        q = qkv[:, : hq * D].view(b, 1, hq, D).transpose(1, 2)
+        k = qkv[:, hq * D : (hq + hkv) * D].view(b, 1, hkv, D).transpose(1, 2)
+        v = qkv[:, (hq + hkv) * D :].view(b, 1, hkv, D).transpose(1, 2)
+        rq, rk = oracle.apply_rope(q, k, cos, sin, pos)
+        kk, vv, seen = oracle.static_cache_update(kc, vc, rk.half(), v, torch.tensor([seen]), seen)
+        ref = oracle.decode_attention(rq.half(), kk, vv)
+        assert _max_abs(out, ref) <= ATOL, f"step {step}"
+        cpos_d += 1  # device-side counters, as a HIP-graph replay would advance them
+        pos_d += 1
+    assert (kd.cpu()[:, :, :seen].float() - kc[:, :, :seen].float()).abs().max() <= 8e-3
+
+
+def test_attention_abi_errors():
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    q = torch.zeros(1, 32, 128, dtype=torch.float16, device=DEV)
+    kc = torch.zeros(1, 8, 16, 128, dtype=torch.float16, device=DEV)
+    out = torch.zeros(1, 32 * 128, dtype=torch.float16, device=DEV)
+    args = (kc.stride(0), kc.stride(1), kc.stride(2), None, 0)
+    assert lib.mui_flash_decode(s, 0, q.data_ptr(), kc.data_ptr(), kc.data_ptr(), *args, 4, None, 1, out.data_ptr(), 1, 32, 8, 64, 16) == -2
+    assert lib.mui_flash_decode(s, 0, q.data_ptr(), kc.data_ptr(), kc.data_ptr(), *args, 4, None, 1, out.data_ptr(), 1, 32, 5, 128, 16) == -1
+    assert lib.mui_flash_decode(s, 0, q.data_ptr(), kc.data_ptr(), kc.data_ptr(), *args, 40, None, 1, out.data_ptr(), 1, 32, 8, 128, 16) == -1
+    assert lib.mui_flash_decode(s, 0, q.data_ptr(), kc.data_ptr(), kc.data_ptr(), *args, 4, None, 2, out.data_ptr(), 1, 32, 8, 128, 16) == -1
+    assert lib.mui_flash_decode_scratch_bytes(2, 32, 128, 1) == 0
+    assert lib.mui_flash_decode_scratch_bytes(2, 32, 128, 4) == 2 * 32 * 4 * 130 * 4
+    with pytest.raises(RuntimeError):
+        muillm_ext.muillm_causal_transformer_decoding_no_mask(torch.zeros(1, 32, 2, 128, dtype=torch.float16, device=DEV), kc, kc)

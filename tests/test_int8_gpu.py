@@ -1,0 +1,186 @@
+"""GPU parity of the int8 weight-only path (config 3): symmetric per-output-channel int8 with
+fp16 scales on the Llama-3-8B decode GEMV shapes, plus the reference's own asymmetric
+group-wise uint8 RTN format.  Dequantised weights must be bit-exact; GEMV outputs within
+1e-2 relative of the high-precision oracle on the dequantised matrix."""
+
+import pytest
+import torch
+
+import oracle
+from muillm_amd import _lib, muillm_ext
+from tests.util import assert_parity
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _gen(seed=0):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def _mk(shape, g, std=1.0, mean=0.0, dtype=torch.float16):
+    return (mean + std * torch.randn(shape, generator=g)).to(dtype)
+
+
+SHAPES = [
+    (6144, 4096),    # fused QKV
+    (4096, 4096),    # o_proj
+    (4096, 14336),   # down
+    (1000, 2048),
+    (7, 16),
+    (33, 4112),      # K just above one pass of the workgroup
+    (12, 8192),
+]
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+def test_channel_dequant_bit_exact(n, k):
+    g = _gen(0)
+    w = _mk((n, k), g, 0.02)
+    w[0] = 0  # all-zero row
+    if n > 2:
+        w[1] = w[1] * 1e-4  # tiny scale (fp16 subnormal products)
+    q, s = oracle.rtn_quantize_channel(w)
+    ref = oracle.rtn_dequantize_channel(q, s)
+    assert torch.equal(ref, q.to(torch.float16) * s[:, None])  # the oracle's own closed form
+    dq = muillm_ext.mui_int8_channel_dequantize_forward(q.to(DEV), s.to(DEV))
+    assert dq.dtype == torch.float16
+    assert torch.equal(dq.cpu().view(torch.int16), ref.view(torch.int16)), "dequantised weights are not bit-exact"
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+@pytest.mark.parametrize("tokens", [1, 4])
+@pytest.mark.parametrize("norm", [True, False])
+def test_channel_linear(n, k, tokens, norm):
+    g = _gen(1)
+    w = _mk((n, k), g, 0.02)
+    q, s = oracle.rtn_quantize_channel(w)
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0) if norm else None
+    r = _mk((tokens, n), g)
+    ref = oracle.int8_channel_linear(x, q, s, gamma, 1e-5, None, r)
+    y = muillm_ext.mui_int8_channel_linear_forward(
+        x.to(DEV), q.to(DEV), s.to(DEV), None if gamma is None else gamma.to(DEV), 1e-5, None, r.to(DEV))
+    assert y.shape == (tokens, n)
+    assert_parity(y, ref, 1e-2, f"int8 channel {n}x{k} b={tokens}", tight=4e-3)
+    # and it tracks the unquantised fp16 layer to quantisation accuracy
+    full = oracle.linear(x, w, gamma, 1e-5, None, r)
+    assert oracle.rel_err(y.cpu(), full) < 3e-2
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (300, 1024), (5, 16)])
+@pytest.mark.parametrize("tokens", [1, 4])
+@pytest.mark.parametrize("packed", [True, False])
+def test_channel_gateup(n, k, tokens, packed):
+    g = _gen(2)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    qg, sg = oracle.rtn_quantize_channel(wg)
+    qu, su = oracle.rtn_quantize_channel(wu)
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    ref = oracle.gateup_silu(x, oracle.rtn_dequantize_channel(qg, sg), oracle.rtn_dequantize_channel(qu, su), gamma, 1e-5)
+    if packed:
+        qq = torch.stack([qg, qu], dim=1).to(DEV)
+        ss = torch.stack([sg, su], dim=1).to(DEV)
+        a = (qq[:, 0], qq[:, 1], ss[:, 0], ss[:, 1])
+    else:
+        a = (qg.to(DEV), qu.to(DEV), sg.to(DEV), su.to(DEV))
+    h = muillm_ext.mui_int8_channel_gateupsilu_forward(gamma.to(DEV), 1e-5, a[0], a[1], a[2], a[3], x.to(DEV))
+    assert_parity(h, ref, 1e-2, f"int8 gateup {n}x{k}", tight=6e-3)
+
+
+def test_channel_closed_forms():
+    k = 4096
+    g = _gen(3)
+    x = _mk((k,), g)
+    # q = 127 * I, s = 1/127 (exactly representable? no: use s = 2^-7 and q = 64 -> w = 0.5)
+    q = torch.zeros(k, k, dtype=torch.int8)
+    q[torch.arange(k), torch.arange(k)] = 64
+    s = torch.full((k,), 2.0 ** -7, dtype=torch.float16)
+    y = muillm_ext.mui_int8_channel_linear_forward(x.to(DEV), q.to(DEV), s.to(DEV))
+    assert torch.allclose(y.cpu().float(), 0.5 * x.float(), rtol=1e-3, atol=1e-3)
+    # extreme codes: all -127 / +127 rows
+    q2 = torch.full((4, k), -127, dtype=torch.int8)
+    q2[1] = 127
+    q2[2, ::2] = 127
+    s2 = torch.full((4,), 2.0 ** -10, dtype=torch.float16)
+    ref = oracle.int8_channel_linear(x, q2, s2)
+    y = muillm_ext.mui_int8_channel_linear_forward(x.to(DEV), q2.to(DEV), s2.to(DEV))
+    assert torch.allclose(y.cpu().double(), ref, rtol=2e-3, atol=2e-2)
+
+
+# ------------------------------------------------------------------------------------
+# the reference's group-wise uint8 format
+# ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n,k,gs", [(4096, 4096, 128), (4096, 14336, 2048), (6144, 4096, 32), (50, 256, 16), (9, 4096, 4096)])
+def test_group_dequant_bit_exact(n, k, gs):
+    g = _gen(4)
+    w = _mk((n, k), g, 0.02)
+    q, smv = oracle.rtn_quantize_group(w, gs)
+    shift = gs.bit_length() - 1
+    ref = oracle.rtn_dequantize_group(q, smv, gs, torch.float16, kernel_form=True)
+    dq = muillm_ext.muillm_int8_dequantize_forward(q.to(DEV), smv.to(DEV), shift)
+    assert torch.equal(dq.cpu().view(torch.int16), ref.view(torch.int16))
+    # the reference's Python fallback rounds twice; it may differ from the kernel form by an ulp
+    ref_py = oracle.rtn_dequantize_group(q, smv, gs, torch.float16, kernel_form=False)
+    assert (dq.cpu().float() - ref_py.float()).abs().max() <= 2 * smv[:, 0].float().max()
+
+
+@pytest.mark.parametrize("n,k,gs", [(4096, 4096, 128), (4096, 14336, 1024), (6144, 4096, 64), (50, 256, 16)])
+@pytest.mark.parametrize("tokens", [1, 4])
+def test_group_linear(n, k, gs, tokens):
+    g = _gen(5)
+    w = _mk((n, k), g, 0.02)
+    q, smv = oracle.rtn_quantize_group(w, gs)
+    shift = gs.bit_length() - 1
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    r = _mk((tokens, n), g)
+    ref = oracle.int8_group_linear(x, q, smv, gs, gamma, 1e-5, None, r)
+    y = muillm_ext.muillm_int8_linear_forward(x.to(DEV), q.to(DEV), smv.to(DEV), shift, gamma.to(DEV), 1e-5,
+                                              None, None, r.to(DEV))
+    assert_parity(y, ref, 1e-2, f"int8 group {n}x{k} gs={gs}", tight=4e-3)
+    assert oracle.rel_err(y.cpu(), oracle.linear(x, w, gamma, 1e-5, None, r)) < 3e-2
+
+
+@pytest.mark.parametrize("n,k,gs", [(14336, 4096, 128), (100, 512, 32)])
+def test_group_gateup(n, k, gs):
+    g = _gen(6)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    qg, smg = oracle.rtn_quantize_group(wg, gs)
+    qu, smu = oracle.rtn_quantize_group(wu, gs)
+    shift = gs.bit_length() - 1
+    ng = k // gs
+    x = _mk((1, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    wgd = (qg.reshape(-1, gs).double() * smg[:, None, 0].double() + smg[:, None, 1].double()).reshape(n, k)
+    wud = (qu.reshape(-1, gs).double() * smu[:, None, 0].double() + smu[:, None, 1].double()).reshape(n, k)
+    ref = oracle.gateup_silu(x, wgd, wud, gamma, 1e-5)
+    packed_w = torch.stack([qg, qu], dim=1).to(DEV)                                   # [N, 2, K]
+    packed_s = torch.stack([smg.reshape(n, ng, 2), smu.reshape(n, ng, 2)], dim=1).to(DEV)  # [N, 2, G, 2]
+    h = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, packed_w, packed_s, shift, x.to(DEV))
+    assert_parity(h, ref, 1e-2, f"int8 group gateup {n}x{k}", tight=6e-3)
+    dg, du = muillm_ext.muillm_int8_gateupsilu_dequantize_forward(packed_w, packed_s, shift)
+    assert torch.equal(dg.cpu(), oracle.rtn_dequantize_group(qg, smg, gs))
+    assert torch.equal(du.cpu(), oracle.rtn_dequantize_group(qu, smu, gs))
+
+
+def test_int8_abi_errors():
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    w = torch.zeros(8, 32, dtype=torch.int8, device=DEV)
+    sc = torch.ones(8, dtype=torch.float16, device=DEV)
+    x = torch.zeros(32, dtype=torch.float16, device=DEV)
+    y = torch.zeros(8, dtype=torch.float16, device=DEV)
+    assert lib.mui_int8_linear(s, 0, w.data_ptr(), 32, None, x.data_ptr(), None, 0.0, None, None, y.data_ptr(), 8, 32, 1) == -1
+    assert lib.mui_int8_linear(s, 0, w.data_ptr(), 24, sc.data_ptr(), x.data_ptr(), None, 0.0, None, None, y.data_ptr(), 8, 24, 1) == -2
+    assert lib.mui_int8_group_linear(s, 0, w.data_ptr(), 32, sc.data_ptr(), 3, x.data_ptr(), None, 0.0, None, None, y.data_ptr(), 8, 32, 1) == -2
+    # K % 16 != 0 goes through dequantise + matmul and is still right
+    g = _gen(7)
+    wf = _mk((8, 24), g, 0.02)
+    q, s_ = oracle.rtn_quantize_channel(wf)
+    xx = _mk((24,), g)
+    yy = muillm_ext.mui_int8_channel_linear_forward(xx.to(DEV), q.to(DEV), s_.to(DEV))
+    assert_parity(yy, oracle.int8_channel_linear(xx, q, s_), 1e-2, "K=24")
