@@ -237,6 +237,14 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
                           void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
                           int max_cache_len);
 
+/* Greedy token choice: out_index[r] = argmax_v logits[r, v] (lowest index on ties, NaN never
+ * wins) for a 16-bit [rows, vocab] matrix with row pitch row_stride elements. Stands in for
+ * the torch.argmax of the reference's greedy sampling branch
+ * (muillm/sampling/generation.py:330-335) so that a captured decode step contains no
+ * library reduction. */
+int mui_argmax(mui_stream_t stream, int dtype, const void* logits, long row_stride,
+               int64_t* out_index, int rows, int vocab);
+
 /* ------------------------------------------------------------------------------------
  * Launch-shape knobs used by the benchmark sweeps (0 restores the built-in choice). They
  * have no counterpart in the reference, whose launch shapes are compile-time constants

@@ -65,6 +65,7 @@ _SIGNATURES = {
     "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, _P,
                                       c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
                                       _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mui_argmax": (c_int, [_P, c_int, _P, c_long, _P, c_int, c_int]),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
 }

@@ -1,0 +1,139 @@
+"""Greedy decode loop with the decode step captured into a HIP graph.
+
+The reference issues ~227 kernel launches per token from Python through pybind
+(muillm/sampling/generation.py:244-408 drives muillm/modules/models/llama/model.py:699-801)
+and only has a single-call C++ decoder stack under tensor parallelism
+(csrc/modules/parallel_decoder_stack.cpp). Here one decode step -- embedding gather, all
+decoder layers, final norm, lm_head, argmax, and the advance of the position counters -- is
+recorded once on a side stream and replayed; everything the step needs to know about "where
+are we" lives in device memory (input ids, position ids, cache slot, output slot), and the
+attention kernel reads the sequence length from the cache slot, so the graph never changes
+as the sequence grows. No memset nodes are recorded: counters are advanced with elementwise
+kernels and the argmax is a hand-written kernel."""
+from typing import Optional
+
+import torch
+
+from ... import muillm_ext
+from ..kvcache.cache_utils import MuiStaticCache, _next_pow2, create_static_cache
+
+
+class MuiGraphDecoder:
+    def __init__(self, lm, use_graph: bool = True):
+        self.lm = lm
+        self.use_graph = use_graph
+        self.graph = None
+        self.cache: Optional[MuiStaticCache] = None
+        self._batch = None
+
+    # -- static device state shared by every replay --
+    def _alloc_state(self, batch: int, max_new_tokens: int, device):
+        self.ids = torch.zeros((batch, 1), dtype=torch.int64, device=device)
+        self.pos = torch.zeros((batch, 1), dtype=torch.int64, device=device)
+        self.cpos = torch.zeros((1,), dtype=torch.int64, device=device)
+        self.step = torch.zeros((1,), dtype=torch.int64, device=device)
+        self.out_tokens = torch.zeros((batch, max_new_tokens), dtype=torch.int64, device=device)
+        self.next_token = torch.zeros((batch,), dtype=torch.int64, device=device)
+        self.logits = None
+        self._batch = batch
+        self._max_new = max_new_tokens
+
+    def _step(self):
+        """One decode step on the static buffers (this is what gets captured)."""
+        out = self.lm(input_ids=self.ids, position_ids=self.pos, cache_position=self.cpos,
+                      past_key_values=self.cache, use_cache=True, all_ones_mask=True, float_logits=False)
+        logits = out.logits[:, -1, :]
+        muillm_ext.mui_argmax(logits, out=self.next_token)
+        self.out_tokens.scatter_(1, self.step.expand(self._batch, 1), self.next_token.unsqueeze(1))
+        self.ids.copy_(self.next_token.unsqueeze(1))
+        self.pos.add_(1)
+        self.cpos.add_(1)
+        self.step.add_(1)
+        return logits
+
+    def _capture(self):
+        self.cache.device_length_mode = True
+        seen = self.cache._seen_tokens
+        # warm up on a side stream (allocator, lazy module state), then restore the cache counters
+        saved = [t.clone() for t in (self.ids, self.pos, self.cpos, self.step, self.out_tokens)]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self._restore(saved, seen)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = self._step()
+        # capture does not execute: the device state is as restored; the host counter moved once
+        self.cache._seen_tokens = seen
+        if self.cache.cpp_module is not None:
+            self.cache.cpp_module.seen_tokens = seen
+
+    def _restore(self, saved, seen):
+        for dst, src in zip((self.ids, self.pos, self.cpos, self.step, self.out_tokens), saved):
+            dst.copy_(src)
+        self.cache._seen_tokens = seen
+        if self.cache.cpp_module is not None:
+            self.cache.cpp_module.seen_tokens = seen
+
+    @torch.no_grad()
+    def prefill(self, input_ids: torch.LongTensor, max_new_tokens: int, cache: Optional[MuiStaticCache] = None):
+        lm = self.lm
+        device = input_ids.device
+        batch, prompt_len = input_ids.shape
+        total = prompt_len + max_new_tokens
+        if cache is None:
+            cache = create_static_cache(lm.engine_config, lm.config, batch, total, device, lm.model.mdtype)
+        elif cache.max_cache_len < total:
+            cache.grow_cache(total, max(lm.config.max_position_embeddings, _next_pow2(total)))
+        if self.cache is not cache or self._batch != batch:
+            self.graph = None
+        self.cache = cache
+        cache.device_length_mode = False
+        out = lm(input_ids=input_ids, past_key_values=cache, use_cache=True, all_ones_mask=True,
+                 num_logits_to_keep=1, float_logits=False)
+        if self._batch != batch or getattr(self, "_max_new", 0) < max_new_tokens:
+            self._alloc_state(batch, max_new_tokens, device)
+            self.graph = None
+        first = muillm_ext.mui_argmax(out.logits[:, -1, :])
+        self.ids.copy_(first.unsqueeze(1))
+        self.pos.fill_(prompt_len)
+        self.cpos.fill_(prompt_len)
+        self.step.fill_(1)
+        self.out_tokens.zero_()
+        self.out_tokens[:, 0] = first
+        return out.logits[:, -1, :]
+
+    @torch.no_grad()
+    def decode(self, n_steps: int, collect_logits: bool = False):
+        """Run n_steps decode steps from the current device state."""
+        logits_hist = []
+        if self.use_graph:
+            if self.graph is None:
+                self._capture()
+            for _ in range(n_steps):
+                self.graph.replay()
+                if collect_logits:
+                    logits_hist.append(self.logits.clone())
+            self.cache._seen_tokens += n_steps
+            if self.cache.cpp_module is not None:
+                self.cache.cpp_module.seen_tokens = self.cache._seen_tokens
+        else:
+            self.cache.device_length_mode = False
+            for _ in range(n_steps):
+                lg = self._step()
+                if collect_logits:
+                    logits_hist.append(lg.clone())
+        return logits_hist
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.LongTensor, max_new_tokens: int, cache: Optional[MuiStaticCache] = None,
+                 return_logits: bool = False):
+        first_logits = self.prefill(input_ids, max_new_tokens, cache)
+        hist = self.decode(max_new_tokens - 1, collect_logits=return_logits)
+        tokens = torch.cat([input_ids, self.out_tokens[:, :max_new_tokens]], dim=1)
+        if return_logits:
+            return tokens, torch.stack([first_logits] + hist, dim=1)
+        return tokens

@@ -1,0 +1,343 @@
+"""MuiLlamaModel / MuiLlamaForCausalLM -- the decoder harness around the fused layers
+(muillm/modules/models/llama/model.py:75-873 of the reference; the Mistral file there is a
+rename of the Llama one and is aliased here).
+
+Semantics kept from the reference: embed -> N x MuiDecoderLayer -> final MuiRMSNorm ->
+lm_head (MuiLinear) -> fp32 logits; a MuiStaticCache with power-of-two capacity is created
+on first use and grown when needed; the causal mask is dropped when there is no padding
+(all_ones_mask), decode steps then need no mask at all.
+
+The classes are plain torch modules (the reference derives them from HuggingFace's
+PreTrainedModel / GenerationMixin, whose interfaces differ between transformers versions);
+replace() accepts HuggingFace LlamaModel / LlamaForCausalLM (and Mistral) instances, and
+from_config() builds a randomly initialised model straight from a config for benchmarks.
+Greedy generation is provided by generate_greedy(), with the decode step optionally
+captured once into a HIP graph and replayed (see graphdecoder.py)."""
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Tuple, Union
+
+import torch
+import torch.nn as nn
+
+from .... import muillm_ext
+from ...._hf import (LlamaForCausalLM, LlamaModel, MistralForCausalLM, MistralModel, head_dim_of)
+from ....engineconfig import MuiEngineConfig
+from ....memorymanagement.gc import trigger_gc
+from ....replacement.replacementcontext import MuiReplacementContext
+from ...attention.rotaryembedding import MuiRotaryEmbedding
+from ...attention.sdpaattention import MuiSdpaAttention, _ignore_causal_mask_sdpa
+from ...decoder.decoder import MuiDecoderLayer
+from ...gateupdownmlp import MuiGateUpDownMLP
+from ...kvcache.cache_utils import (MuiCache, MuiStaticCache, create_static_cache,
+                                    grow_static_cache_if_needed)
+from ...linear import MuiLinear
+from ...module import MuiModule
+from ...multilinear import MuiMultiLinear
+from ...norm.rmsnorm import MuiRMSNorm
+
+
+@dataclass
+class MuiDecoderConfig:
+    """The fields of a Llama/Mistral config that the decoder reads (duck-typed stand-in for
+    transformers' LlamaConfig / MistralConfig)."""
+    hidden_size: int = 4096
+    intermediate_size: int = 14336
+    num_hidden_layers: int = 32
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    vocab_size: int = 128256
+    rms_norm_eps: float = 1e-5
+    max_position_embeddings: int = 8192
+    rope_theta: float = 500000.0
+    head_dim: Optional[int] = None
+    rope_scaling: Optional[Dict[str, Any]] = None
+    attention_dropout: float = 0.0
+    attention_bias: bool = False
+    mlp_bias: bool = False
+    pad_token_id: Optional[int] = None
+    tie_word_embeddings: bool = False
+
+    @staticmethod
+    def llama3_8b(**overrides) -> "MuiDecoderConfig":
+        return MuiDecoderConfig(**overrides)
+
+    @staticmethod
+    def mistral_7b(**overrides) -> "MuiDecoderConfig":
+        base = dict(vocab_size=32000, rope_theta=10000.0, max_position_embeddings=32768, rms_norm_eps=1e-5)
+        base.update(overrides)
+        return MuiDecoderConfig(**base)
+
+
+@dataclass
+class MuiModelOutput:
+    last_hidden_state: torch.Tensor
+    past_key_values: Optional[MuiCache] = None
+    hidden_states: Optional[Tuple[torch.Tensor, ...]] = None
+    attentions: Optional[Tuple[torch.Tensor, ...]] = None
+
+
+@dataclass
+class MuiCausalLMOutput:
+    logits: torch.Tensor
+    past_key_values: Optional[MuiCache] = None
+    hidden_states: Optional[Tuple[torch.Tensor, ...]] = None
+    attentions: Optional[Tuple[torch.Tensor, ...]] = None
+    loss: Optional[torch.Tensor] = None
+
+
+class MuiLlamaModel(MuiModule):
+    def __init__(self, engine_config: MuiEngineConfig, config, embed_tokens: nn.Embedding, layers,
+                 norm: MuiRMSNorm, rotary_emb: MuiRotaryEmbedding):
+        super().__init__(engine_config=engine_config)
+        self.config = config
+        self.cpp_engine = engine_config.cpp_engine
+        self.mdevice = embed_tokens.weight.device
+        self.mdtype = embed_tokens.weight.dtype
+        self.padding_idx = getattr(config, "pad_token_id", None)
+        self.vocab_size = config.vocab_size
+        self.embed_tokens = embed_tokens
+        self.layers = layers if isinstance(layers, nn.ModuleList) else nn.ModuleList(layers)
+        self.norm = norm
+        self.rotary_emb = rotary_emb
+
+    def finalize_init(self):
+        self.mdevice = self.embed_tokens.weight.device
+        self.mdtype = self.embed_tokens.weight.dtype
+
+    @staticmethod
+    def replace(replacement_context: MuiReplacementContext, prev_model) -> "MuiLlamaModel":
+        if isinstance(prev_model, MuiLlamaModel):
+            return prev_model
+        engine_config = replacement_context.engine_config
+        device = replacement_context.device
+        if device is None:
+            raise ValueError("device was None")
+        config = prev_model.config
+        embed_tokens = prev_model.embed_tokens.to(device)
+        dtype = embed_tokens.weight.dtype
+        layers = []
+        for i in range(len(prev_model.layers)):
+            layers.append(MuiDecoderLayer.replace(replacement_context, prev_model.layers[i]))
+            prev_model.layers[i] = None  # release the source layer as we go
+        norm = MuiRMSNorm.replace(replacement_context, prev_model.norm)
+        rotary_emb = MuiRotaryEmbedding(engine_config, config, layer_idx=0, device=device, dtype=dtype)
+        new_model = MuiLlamaModel(engine_config, config, embed_tokens, layers, norm, rotary_emb)
+        trigger_gc()
+        return new_model
+
+    def get_input_embeddings(self):
+        return self.embed_tokens
+
+    def set_input_embeddings(self, value):
+        self.embed_tokens = value
+
+    def _update_causal_mask(self, attention_mask, inputs_shape, cache_position, past_key_values,
+                            output_attentions, all_ones_mask, past_seen_tokens: int):
+        """Additive 4-D mask [B, 1, T, S_total] (0 keep / finfo.min drop), or None when SDPA's
+        is_causal / the mask-free decode kernel suffice (llama/model.py:437-613 of the reference)."""
+        if (not output_attentions) and _ignore_causal_mask_sdpa(
+                attention_mask, inputs_shape, past_seen_tokens, all_ones_mask=all_ones_mask,
+                is_training=self.training):
+            return None
+        bsz, q_len = inputs_shape[0], inputs_shape[1]
+        target_length = past_seen_tokens + q_len
+        dtype, device = self.mdtype, self.mdevice
+        min_dtype = torch.finfo(dtype).min
+        if attention_mask is not None and attention_mask.dim() == 4:
+            return attention_mask
+        causal = torch.full((q_len, target_length), fill_value=min_dtype, dtype=dtype, device=device)
+        causal = causal * (torch.arange(target_length, device=device) > cache_position.reshape(-1, 1))
+        causal = causal[None, None, :, :].expand(bsz, 1, -1, -1)
+        if attention_mask is not None:
+            causal = causal.clone()
+            mask_length = attention_mask.shape[-1]
+            padding = causal[:, :, :, :mask_length] + attention_mask[:, None, None, :].to(dtype)
+            causal[:, :, :, :mask_length] = causal[:, :, :, :mask_length].masked_fill(padding == 0, min_dtype)
+        return causal
+
+    def forward(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
+                position_ids: Optional[torch.LongTensor] = None, past_key_values=None,
+                inputs_embeds: Optional[torch.Tensor] = None, use_cache: Optional[bool] = None,
+                output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
+                return_dict: Optional[bool] = None, cache_position: Optional[torch.LongTensor] = None,
+                all_ones_mask: Optional[bool] = None):
+        output_attentions = bool(output_attentions)
+        output_hidden_states = bool(output_hidden_states)
+        use_cache = True if use_cache is None else use_cache
+        if (input_ids is None) == (inputs_embeds is None):
+            raise ValueError(
+                "You cannot specify both input_ids and inputs_embeds at the same time, and must specify either one")
+        inputs_shape = input_ids.shape if input_ids is not None else inputs_embeds.shape
+        batch_size, q_len = inputs_shape[0], inputs_shape[1]
+        if past_key_values is not None and not isinstance(past_key_values, MuiCache):
+            past_key_values = None  # foreign cache types are dropped, a static cache is built instead
+        past_seen_tokens = past_key_values.get_seq_length() if past_key_values is not None else 0
+        tot_seq_len = past_seen_tokens + q_len
+
+        if use_cache:
+            if past_key_values is None:
+                past_key_values = create_static_cache(self.engine_config, self.config, batch_size, tot_seq_len,
+                                                      self.mdevice, self.mdtype)
+            elif isinstance(past_key_values, MuiStaticCache):
+                grow_static_cache_if_needed(past_key_values, tot_seq_len, self.config.max_position_embeddings)
+
+        if cache_position is None:
+            cache_position = torch.arange(past_seen_tokens, tot_seq_len, device=self.mdevice)
+        if position_ids is None:
+            position_ids = cache_position.unsqueeze(0)
+
+        if all_ones_mask is None:
+            all_ones_mask = attention_mask is None
+        causal_mask = None
+        if not all_ones_mask or q_len > 1:
+            causal_mask = self._update_causal_mask(attention_mask, inputs_shape, cache_position, past_key_values,
+                                                   output_attentions, all_ones_mask, past_seen_tokens)
+        if all_ones_mask and q_len == 1:
+            causal_mask = None
+        elif causal_mask is not None:
+            causal_mask = causal_mask[:, :, :, :tot_seq_len]
+        position_ids = position_ids.contiguous()
+
+        if inputs_embeds is None:
+            inputs_embeds = self.embed_tokens(input_ids)
+        hidden_states = inputs_embeds
+
+        # shared position embeddings for the layers that take the unfused route
+        position_embeddings = None
+        if not (q_len == 1 and isinstance(past_key_values, MuiStaticCache) and hidden_states.is_cuda):
+            position_embeddings = self.rotary_emb(hidden_states, position_ids)
+
+        all_hidden_states = () if output_hidden_states else None
+        all_self_attns = () if output_attentions else None
+        for decoder_layer in self.layers:
+            if output_hidden_states:
+                all_hidden_states += (hidden_states,)
+            layer_outputs = decoder_layer(
+                hidden_states=hidden_states, attention_mask=causal_mask, position_ids=position_ids,
+                past_key_value=past_key_values if use_cache else None, output_attentions=output_attentions,
+                use_cache=use_cache, cache_position=cache_position, position_embeddings=position_embeddings,
+                all_ones_mask=all_ones_mask)
+            hidden_states = layer_outputs[0]
+            if output_attentions:
+                all_self_attns += (layer_outputs[1],)
+
+        hidden_states = self.norm(hidden_states)
+        if output_hidden_states:
+            all_hidden_states += (hidden_states,)
+        if use_cache and isinstance(past_key_values, MuiCache):
+            past_key_values.sync_back()
+        return MuiModelOutput(last_hidden_state=hidden_states,
+                              past_key_values=past_key_values if use_cache else None,
+                              hidden_states=all_hidden_states, attentions=all_self_attns)
+
+
+class MuiLlamaForCausalLM(MuiModule):
+    def __init__(self, engine_config: MuiEngineConfig, config, model: MuiLlamaModel, lm_head: MuiLinear):
+        super().__init__(engine_config=engine_config)
+        self.config = config
+        self.model = model
+        self.vocab_size = config.vocab_size
+        self.lm_head = lm_head
+        self._graph_decoder = None
+
+    @staticmethod
+    def replace(replacement_context: MuiReplacementContext, prev_model) -> "MuiLlamaForCausalLM":
+        if isinstance(prev_model, MuiLlamaForCausalLM):
+            return prev_model
+        engine_config = replacement_context.engine_config
+        new_lm_head = MuiLinear.replace(replacement_context, prev_model.lm_head)
+        new_model = MuiLlamaModel.replace(replacement_context, prev_model.model)
+        return MuiLlamaForCausalLM(engine_config, prev_model.config, new_model, new_lm_head)
+
+    @staticmethod
+    def from_config(engine_config: MuiEngineConfig, config, dtype=torch.float16, device="cuda", seed: int = 0,
+                    init_std: float = 0.02, finalize: bool = True) -> "MuiLlamaForCausalLM":
+        """Randomly initialised model (weights ~ N(0, init_std), norm weights 1) built layer by
+        layer on `device`; no checkpoint involved."""
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed)
+        hid, inter = config.hidden_size, config.intermediate_size
+        d = head_dim_of(config)
+        hq = config.num_attention_heads
+        hkv = config.num_key_value_heads if getattr(config, "num_key_value_heads", None) else hq
+        eps = config.rms_norm_eps
+
+        def rnd_(p):
+            p.data.normal_(0.0, init_std, generator=gen)
+
+        embed = nn.Embedding(config.vocab_size, hid, device=device, dtype=dtype)
+        rnd_(embed.weight)
+        layers = []
+        for i in range(config.num_hidden_layers):
+            qkv = MuiMultiLinear(engine_config, hid, [hq * d, hkv * d, hkv * d], bias=False,
+                                 variance_epsilon=eps, normalize=True, device=device, dtype=dtype)
+            rnd_(qkv.linear.weight)
+            o_proj = MuiLinear(engine_config, hq * d, hid, bias=False, device=device, dtype=dtype)
+            rnd_(o_proj.weight)
+            rope = MuiRotaryEmbedding(engine_config, config, layer_idx=i, device=device, dtype=dtype)
+            attn = MuiSdpaAttention(engine_config, config, rope, o_proj, layer_idx=i, device=device, dtype=dtype)
+            mlp = MuiGateUpDownMLP(engine_config, hid, inter, nn.SiLU(), variance_epsilon=eps, normalize=True,
+                                   device=device, dtype=dtype)
+            rnd_(mlp.gate_proj.weight)
+            rnd_(mlp.up_proj.weight)
+            rnd_(mlp.down_proj.weight)
+            layers.append(MuiDecoderLayer(engine_config, qkv, attn, mlp))
+        norm = MuiRMSNorm(engine_config, hid, eps=eps, device=device, dtype=dtype)
+        rotary = MuiRotaryEmbedding(engine_config, config, layer_idx=0, device=device, dtype=dtype)
+        model = MuiLlamaModel(engine_config, config, embed, layers, norm, rotary)
+        lm_head = MuiLinear(engine_config, hid, config.vocab_size, bias=False, device=device, dtype=dtype)
+        rnd_(lm_head.weight)
+        lm = MuiLlamaForCausalLM(engine_config, config, model, lm_head)
+        lm.eval()
+        if finalize:
+            from ....engine import _finalize_module
+            _finalize_module(lm)
+        setattr(lm, "muillm_config", engine_config)
+        return lm
+
+    def get_input_embeddings(self):
+        return self.model.embed_tokens
+
+    def get_output_embeddings(self):
+        return self.lm_head
+
+    def forward(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
+                position_ids: Optional[torch.LongTensor] = None, past_key_values=None,
+                inputs_embeds: Optional[torch.Tensor] = None, labels=None, use_cache: Optional[bool] = None,
+                output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
+                return_dict: Optional[bool] = None, cache_position: Optional[torch.LongTensor] = None,
+                all_ones_mask: Optional[bool] = None, num_logits_to_keep: int = 0, float_logits: bool = True):
+        if labels is not None:
+            raise NotImplementedError("inference only: labels/loss are not supported")
+        outputs = self.model(
+            input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids,
+            past_key_values=past_key_values, inputs_embeds=inputs_embeds, use_cache=use_cache,
+            output_attentions=output_attentions, output_hidden_states=output_hidden_states,
+            cache_position=cache_position, all_ones_mask=all_ones_mask)
+        hidden_states = outputs.last_hidden_state
+        if num_logits_to_keep:
+            hidden_states = hidden_states[:, -num_logits_to_keep:, :]
+        logits = self.lm_head(hidden_states)
+        if float_logits:
+            logits = logits.float()
+        return MuiCausalLMOutput(logits=logits, past_key_values=outputs.past_key_values,
+                                 hidden_states=outputs.hidden_states, attentions=outputs.attentions)
+
+    @torch.no_grad()
+    def generate_greedy(self, input_ids: torch.LongTensor, max_new_tokens: int, use_graph: bool = True,
+                        cache: Optional[MuiStaticCache] = None, return_logits: bool = False):
+        """Prefill on the prompt, then max_new_tokens greedy decode steps at the prompt's batch
+        size. Returns int64 [B, prompt + max_new_tokens] (and, optionally, the per-step fp16
+        logits of the decode steps).
+
+        use_graph=True captures one decode step (model forward, argmax, position bookkeeping,
+        all on the device) into a HIP graph and replays it; False runs the same step eagerly."""
+        from ..graphdecoder import MuiGraphDecoder
+
+        dec = MuiGraphDecoder(self, use_graph=use_graph)
+        return dec.generate(input_ids, max_new_tokens, cache=cache, return_logits=return_logits)
+
+
+# Mistral shares the Llama implementation (the reference's mistral/model.py is a renamed copy)
+MuiMistralModel = MuiLlamaModel
+MuiMistralForCausalLM = MuiLlamaForCausalLM

@@ -709,3 +709,24 @@ def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_positi
         "mui_attn_decode_fused",
     )
     return (out, q_out) if want_q_out else out
+
+
+# --------------------------------------------------------------------------------------
+# greedy sampling helper
+# --------------------------------------------------------------------------------------
+def mui_argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """argmax over the last dim of 16-bit CUDA logits [..., V] -> int64 [...]; lowest index on ties."""
+    _check_cuda(logits, "logits")
+    if logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    v = logits.shape[-1]
+    l2 = logits.reshape(-1, v)
+    rows = l2.shape[0]
+    if out is None:
+        out = torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
+    check(
+        _lib.load().mui_argmax(_stream(l2), _dtype_code(l2), l2.data_ptr(), l2.stride(0) if rows > 1 else v,
+                               out.data_ptr(), rows, v),
+        "mui_argmax",
+    )
+    return out

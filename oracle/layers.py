@@ -35,6 +35,7 @@ __all__ = [
     "repeat_kv",
     "decode_attention",
     "decoder_layer",
+    "decoder_model_step",
     "next_pow2",
     "rel_err",
 ]
@@ -388,3 +389,24 @@ def decoder_layer(
     out = gateupdown_mlp(h1, p["wg"], p["wu"], p["wd"], p["ln2"], eps, residual=h1,
                          round_intermediate=store_dtype)
     return rnd(out), seen
+
+
+# --------------------------------------------------------------------------------------
+# Whole decoder -- muillm/modules/models/llama/model.py:298-322,360-406,778-785
+# --------------------------------------------------------------------------------------
+def decoder_model_step(ids, params, k_caches, v_caches, cos, sin, seen_tokens: int, n_heads: int,
+                       n_kv_heads: int, store_dtype: torch.dtype = torch.float16):
+    """Embed -> layers -> final RMSNorm -> lm_head for `ids` [B, T] appended after
+    `seen_tokens` cached tokens. params: {'embed', 'layers': [layer dicts], 'norm', 'lm_head',
+    'eps'}. Returns (logits float64 [B, T, V], new seen_tokens). Hidden states between layers
+    are stored in `store_dtype` like the fused path does."""
+    b, t = ids.shape
+    h = params["embed"][ids].to(store_dtype)
+    pos = torch.arange(seen_tokens, seen_tokens + t).unsqueeze(0).expand(b, t)
+    cpos = torch.arange(seen_tokens, seen_tokens + t)
+    seen = seen_tokens
+    for li, lp in enumerate(params["layers"]):
+        h, seen = decoder_layer(h, lp, k_caches[li], v_caches[li], cos, sin, pos, cpos, seen_tokens,
+                                n_heads, n_kv_heads, store_dtype)
+    hn = rmsnorm(h, params["norm"], params["eps"]).to(store_dtype)
+    return linear(hn, params["lm_head"]), seen

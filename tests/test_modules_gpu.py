@@ -1,0 +1,260 @@
+"""GPU tests of the layer classes, decoder layer, whole-model harness, int8 quantisation and
+the HIP-graph decode loop, against the CPU oracle and (where importable) HuggingFace's own
+layers on the same device."""
+
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+import oracle
+from muillm_amd import _hf
+from muillm_amd.engine import init_engine
+from muillm_amd.engineconfig import MuiEngineConfig
+from muillm_amd.modules.gateupdownmlp import MuiGateUpDownMLP
+from muillm_amd.modules.kvcache.cache_utils import MuiStaticCache, create_static_cache
+from muillm_amd.modules.linear import MuiLinear
+from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
+from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
+from muillm_amd.modules.multilinear import MuiMultiLinear
+from muillm_amd.modules.norm.rmsnorm import MuiRMSNorm
+from muillm_amd.modules.quantized.int8gateupdownmlp import MuiInt8GateUpDownMLP
+from muillm_amd.modules.quantized.int8linear import MuiInt8Linear
+from muillm_amd.quantization.quantizationmethod import Int8WeightOnlyQuantizationMethod
+from muillm_amd.replacement.replacementcontext import MuiReplacementContext
+from tests.util import assert_parity, reference_allclose
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    return MuiReplacementContext(MuiEngineConfig(), model=None, device=DEV)
+
+
+def test_engine_reports_gfx950(ctx):
+    info = ctx.engine_config.cpp_engine.info
+    assert info["is_gfx950"] == 1 and info["wave_size"] == 64 and info["compute_units"] >= 64
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tokens", [1, 4, 32])
+def test_linear_module(ctx, dtype, tokens):
+    """tests/test_linear.py of the reference (batch 4) plus the single-token and prefill cases."""
+    torch.manual_seed(0)
+    lin = nn.Linear(2048, 1024, bias=True).to(dtype)
+    lin.weight.data = (torch.randn(1024, 2048) * 0.05).to(dtype)
+    mui = MuiLinear.replace(ctx, copy.deepcopy(lin))
+    mui.finalize_init()
+    x = torch.rand(tokens, 2048).to(dtype)
+    r = torch.rand(tokens, 1024).to(dtype)
+    y = mui(x.to(DEV), residual=r.to(DEV))
+    ref = oracle.linear(x, lin.weight.data, bias=lin.bias.data, residual=r)
+    assert reference_allclose(y, ref)
+    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 2e-2, f"MuiLinear {dtype} b={tokens}")
+
+
+def test_multilinear_and_mlp_modules(ctx):
+    torch.manual_seed(1)
+    hid, inter = 512, 1536
+    norm_w = (1 + 0.1 * torch.randn(hid)).half()
+
+    class Norm(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = nn.Parameter(norm_w.clone())
+            self.variance_epsilon = 1e-5
+
+    lins = []
+    for n in (512, 128, 128):
+        l = nn.Linear(hid, n, bias=False).half()
+        l.weight.data = (torch.randn(n, hid) * 0.02).half()
+        lins.append(l)
+    qkv = MuiMultiLinear.replace(ctx, [copy.deepcopy(l) for l in lins], prev_layernorm_module=Norm())
+    qkv.finalize_init()
+    x = torch.randn(1, 1, hid).half()
+    q, k, v = qkv(x.to(DEV))
+    refs = oracle.multilinear(x, [l.weight.data for l in lins], norm_w, 1e-5)
+    for got, ref in zip((q, k, v), refs):
+        assert_parity(got, ref, 1e-2, "fused QKV slice", tight=4e-3)
+    assert q.shape == (1, 1, 512) and k.shape == (1, 1, 128) and not k.is_contiguous() or k.shape[-1] == 128
+
+    class MLP(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_proj = nn.Linear(hid, inter, bias=False).half()
+            self.up_proj = nn.Linear(hid, inter, bias=False).half()
+            self.down_proj = nn.Linear(inter, hid, bias=False).half()
+            self.act_fn = nn.SiLU()
+            for l in (self.gate_proj, self.up_proj, self.down_proj):
+                l.weight.data = (torch.randn_like(l.weight.float()) * 0.02).half()
+
+    mlp = MLP()
+    wg, wu, wd = (mlp.gate_proj.weight.data.clone(), mlp.up_proj.weight.data.clone(), mlp.down_proj.weight.data.clone())
+    mui = MuiGateUpDownMLP.replace(ctx, mlp, prev_layernorm_module=Norm())
+    mui.finalize_init()
+    # the repack aliases gate/up onto one interleaved buffer without changing their values
+    assert mui.gate_up_packed.shape == (inter, 2, hid)
+    assert mui.gate_proj.weight.data_ptr() == mui.gate_up_packed.data_ptr()
+    assert mui.up_proj.weight.data_ptr() == mui.gate_up_packed.data_ptr() + hid * 2
+    assert torch.equal(mui.gate_proj.weight.cpu(), wg) and torch.equal(mui.up_proj.weight.cpu(), wu)
+    for tokens in (1, 4, 32):  # fused kernel, small batch, and the unfused prefill route
+        xx = torch.randn(tokens, hid).half()
+        rr = torch.randn(tokens, hid).half()
+        out = mui(xx.to(DEV), residual=rr.to(DEV))
+        assert_parity(out, oracle.gateupdown_mlp(xx, wg, wu, wd, norm_w, 1e-5, rr), 1e-2, f"MuiGateUpDownMLP b={tokens}")
+
+
+def _small_config(layers=2):
+    return MuiDecoderConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=layers,
+                            num_attention_heads=4, num_key_value_heads=2, vocab_size=1024,
+                            max_position_embeddings=256, rope_theta=500000.0, rms_norm_eps=1e-5)
+
+
+def _oracle_params(lm):
+    """Weights of a MuiLlamaForCausalLM as CPU tensors in the oracle's layout."""
+    cfg = lm.config
+    d = cfg.hidden_size // cfg.num_attention_heads
+    hq, hkv = cfg.num_attention_heads, cfg.num_key_value_heads
+    layers = []
+    for layer in lm.model.layers:
+        w = layer.qkv_proj.linear.weight.detach().cpu()
+        layers.append(dict(
+            ln1=layer.qkv_proj.linear.norm_weights.detach().cpu(), wq=w[: hq * d], wk=w[hq * d : (hq + hkv) * d],
+            wv=w[(hq + hkv) * d :], wo=layer.self_attn.o_proj.weight.detach().cpu(),
+            ln2=layer.mlp.norm_weights.detach().cpu(), wg=layer.mlp.gate_proj.weight.detach().cpu(),
+            wu=layer.mlp.up_proj.weight.detach().cpu(), wd=layer.mlp.down_proj.weight.detach().cpu(),
+            eps=cfg.rms_norm_eps))
+    return dict(embed=lm.model.embed_tokens.weight.detach().cpu(), layers=layers,
+                norm=lm.model.norm.weight.detach().cpu(), lm_head=lm.lm_head.weight.detach().cpu(),
+                eps=cfg.rms_norm_eps)
+
+
+def test_model_prefill_and_decode_vs_oracle():
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=0,
+                                         init_std=0.05)
+    params = _oracle_params(lm)
+    d = 128
+    cos, sin = oracle.rope_tables(cfg.rope_theta, d, cfg.max_position_embeddings)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, cfg.vocab_size, (2, 12), generator=g)
+    cap = 64
+    kcs = [torch.zeros(2, 2, cap, d, dtype=torch.float16) for _ in range(2)]
+    vcs = [torch.zeros(2, 2, cap, d, dtype=torch.float16) for _ in range(2)]
+    ref_logits, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, 4, 2)
+    with torch.no_grad():
+        out = lm(input_ids=ids.to(DEV))
+    assert out.logits.dtype == torch.float32 and out.logits.shape == (2, 12, cfg.vocab_size)
+    assert_parity(out.logits, ref_logits, 1e-2, "prefill logits")
+    cache = out.past_key_values
+    assert isinstance(cache, MuiStaticCache) and cache.get_seq_length() == 12 and cache.get_max_length() == 16
+    # greedy decode, one token at a time, against the oracle on its own growing cache
+    nxt = ref_logits[:, -1].argmax(-1)
+    for step in range(6):
+        ref_logits, seen = oracle.decoder_model_step(nxt.unsqueeze(1), params, kcs, vcs, cos, sin, seen, 4, 2)
+        with torch.no_grad():
+            out = lm(input_ids=nxt.unsqueeze(1).to(DEV), past_key_values=cache)
+        assert_parity(out.logits, ref_logits, 1e-2, f"decode step {step}")
+        assert cache.get_seq_length() == seen
+        nxt = ref_logits[:, -1].argmax(-1)
+    assert cache.get_max_length() == 32  # grew by the power-of-two schedule
+
+
+@pytest.mark.parametrize("batch", [1, 2])
+def test_graph_decode_matches_eager(batch):
+    cfg = _small_config(layers=3)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=1,
+                                         init_std=0.05)
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, cfg.vocab_size, (batch, 32), generator=g).to(DEV)
+    n_new = 24
+    eager, eager_logits = lm.generate_greedy(ids, n_new, use_graph=False, return_logits=True)
+    dec = MuiGraphDecoder(lm, use_graph=True)
+    graph, graph_logits = dec.generate(ids, n_new, return_logits=True)
+    assert eager.shape == (batch, 32 + n_new)
+    assert torch.equal(eager, graph), "graph replay and eager decode disagree"
+    assert torch.equal(eager_logits, graph_logits)
+    # a second generation on the same decoder re-uses the captured graph, with eager work and
+    # synchronisations in between, and must reproduce the result exactly
+    torch.cuda.synchronize()
+    _ = lm(input_ids=ids[:, :5])
+    torch.cuda.synchronize()
+    dec.cache.reset()
+    graph2 = dec.generate(ids, n_new, cache=dec.cache)
+    assert torch.equal(graph2, eager)
+    assert dec.cache.get_seq_length() == 32 + n_new - 1
+
+
+def test_argmax_kernel():
+    from muillm_amd import muillm_ext
+    g = torch.Generator().manual_seed(2)
+    for rows, v in ((1, 128256), (3, 1000), (2, 7), (1, 32000)):
+        x = torch.randn(rows, v, generator=g).half().to(DEV)
+        assert torch.equal(muillm_ext.mui_argmax(x).cpu(), x.float().argmax(-1).cpu())
+    x = torch.zeros(2, 4096, dtype=torch.float16, device=DEV)
+    x[0, 77] = x[0, 3000] = 5.0  # ties -> lowest index
+    x[1, :] = float("-inf")
+    out = muillm_ext.mui_argmax(x).cpu()
+    assert out[0] == 77 and out[1] == 0
+    xb = torch.randn(2, 5000, generator=g).bfloat16().to(DEV)[:, :4999]  # strided rows
+    assert torch.equal(muillm_ext.mui_argmax(xb).cpu(), xb.float().argmax(-1).cpu())
+
+
+@pytest.mark.skipif(not _hf.HAVE_TRANSFORMERS, reason="transformers not installed")
+def test_init_engine_on_hf_llama_gpu_fp16():
+    """Drop-in check: a HuggingFace Llama (fp16, GPU) before and after init_engine."""
+    torch.manual_seed(0)
+    cfg = _hf.LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                          num_key_value_heads=2, vocab_size=1024, max_position_embeddings=256, rms_norm_eps=1e-5,
+                          rope_theta=500000.0)
+    hf = _hf.LlamaForCausalLM(cfg).half().eval()
+    ids = torch.randint(0, 1024, (2, 20))
+    with torch.no_grad():
+        ref = hf.float()(input_ids=ids, use_cache=False).logits.double()  # fp32 reference on CPU
+    hf = hf.half()
+    model = init_engine(copy.deepcopy(hf), device=DEV)
+    with torch.no_grad():
+        out = model(input_ids=ids[:, :16].to(DEV))
+        assert_parity(out.logits, ref[:, :16], 2e-2, "HF prefill logits")
+        cache = out.past_key_values
+        for t in range(16, 20):
+            step = model(input_ids=ids[:, t : t + 1].to(DEV), past_key_values=cache)
+            assert_parity(step.logits[:, 0], ref[:, t], 2e-2, f"HF decode step {t}")
+
+
+@pytest.mark.parametrize("group_size", [0, 128])
+def test_int8_quantized_model(group_size):
+    cfg = _small_config()
+    base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=3,
+                                           init_std=0.05, finalize=False)
+    qm = Int8WeightOnlyQuantizationMethod(group_size=group_size, modules=["qkv_proj", "o_proj", "mlp"])
+    qmodel = init_engine(copy.deepcopy(base), device=DEV, engine_config=MuiEngineConfig(qm))
+    fmodel = init_engine(base, device=DEV, engine_config=MuiEngineConfig())
+    kinds = [type(m).__name__ for m in qmodel.modules()]
+    assert kinds.count("MuiInt8GateUpDownMLP") == 2 and kinds.count("MuiInt8Linear") == 2 + 2 + 2  # qkv, o, down
+    assert isinstance(qmodel.lm_head, MuiLinear)  # filtered out by name, stays 16-bit
+    g = torch.Generator().manual_seed(4)
+    ids = torch.randint(0, cfg.vocab_size, (1, 10), generator=g).to(DEV)
+    with torch.no_grad():
+        fo, qo = fmodel(input_ids=ids), qmodel(input_ids=ids)
+        assert oracle.rel_err(qo.logits.cpu(), fo.logits.cpu().double()) < 6e-2
+        fc, qc = fo.past_key_values, qo.past_key_values
+        tok = fo.logits[:, -1].argmax(-1, keepdim=True)
+        f1 = fmodel(input_ids=tok, past_key_values=fc)   # single-token: the int8 GEMV kernels run here
+        q1 = qmodel(input_ids=tok, past_key_values=qc)
+        assert oracle.rel_err(q1.logits.cpu(), f1.logits.cpu().double()) < 6e-2
+    # the quantised single-token layer equals the oracle on its own quantised weights
+    layer = qmodel.model.layers[0]
+    x = torch.randn(1, 1, cfg.hidden_size, generator=g).half()
+    oproj = layer.self_attn.o_proj
+    assert isinstance(oproj, MuiInt8Linear)
+    y = oproj(x.to(DEV))
+    if group_size == 0:
+        ref = oracle.int8_channel_linear(x, oproj.weights_int8.cpu(), oproj.scales.cpu())
+    else:
+        ref = oracle.int8_group_linear(x, oproj.weights_uint8.cpu(), oproj.scales_min_vals.cpu(), group_size)
+    assert_parity(y, ref, 1e-2, "int8 o_proj")
+    assert isinstance(layer.mlp, MuiInt8GateUpDownMLP)
