@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode hot path on one MI355X.
+
+  python bench.py --gpus 1 --steps K --warmup W
+
+A "step" is one greedy decode step (one token for one user) of a randomly initialised
+Llama-3-8B-shaped fp16 decoder: 32 layers, hidden 4096, 32/8 heads x 128, MLP 14336, vocab
+128256, static KV cache, 32-token random prompt, batch 1. The step (embedding gather, 32 x
+[fused norm+QKV GEMV, fused RoPE + cache write + flash decoding, o_proj GEMV + residual,
+fused norm + gate/up + SiLU GEMV, down GEMV + residual], final norm, lm_head GEMV, argmax)
+is replayed from a HIP graph; all inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line with the whole-job throughput (tokens/s/user), a `roofline` object for
+the dominant kernel (the fused gate/up GEMV: half of all bytes streamed per token) timed
+live with HIP events over cold (distinct) weight buffers, a `cpu_baseline` object (the
+reference's PyTorch fallback path in fp16 on this box's host cores, bounded sample), and a
+`kernels` table (GB/s per fused kernel family, informational).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+BASELINE_TOKENS_PER_S = 210.0  # reference README: Llama-3-8B fp16 bs1 on 1x MI300X
+
+
+def _event_time_us(fn, iters, warm):
+    import torch
+
+    for i in range(warm):
+        fn(i)
+    torch.cuda.synchronize()
+    s = torch.cuda.Event(enable_timing=True)
+    e = torch.cuda.Event(enable_timing=True)
+    s.record()
+    for i in range(iters):
+        fn(i)
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) * 1e3 / iters
+
+
+def bench_decode(lm, steps, warmup, prompt_len=32):
+    import torch
+
+    from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
+
+    dev = "cuda"
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, lm.config.vocab_size, (1, prompt_len), generator=g).to(dev)
+    dec = MuiGraphDecoder(lm, use_graph=True)
+    dec.prefill(ids, steps + warmup + 1)
+    dec.decode(warmup)  # captures the graph on first use, then W untimed replays
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.decode(steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return dt, dec
+
+
+def gateup_roofline(lm):
+    """Average launch duration of the fused gate/up+SiLU GEMV over the model's 32 distinct
+    (cold) weight buffers, HIP events on the launch stream."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    layers = lm.model.layers
+    hid, inter = lm.config.hidden_size, lm.config.intermediate_size
+    x = torch.randn(hid, device="cuda", dtype=torch.float16)
+    h = torch.empty(inter, device="cuda", dtype=torch.float16)
+    stream = torch.cuda.current_stream().cuda_stream
+    ptrs = [(l.mlp.gate_proj.weight.data_ptr(), l.mlp.up_proj.weight.data_ptr(), l.mlp.gate_proj.weight.stride(0),
+             l.mlp.norm_weights.data_ptr()) for l in layers]
+
+    def fn(i):
+        gp, up, pitch, nw = ptrs[i % len(ptrs)]
+        lib.mui_gateup_silu(stream, 0, gp, up, pitch, x.data_ptr(), nw, 1e-5, h.data_ptr(), inter, hid, 1)
+
+    us = _event_time_us(fn, iters=20 * len(ptrs), warm=len(ptrs))
+    alg_bytes = 2 * inter * hid * 2 + 2 * (hid + hid + inter)  # G and U once, x, gamma, h
+    achieved = alg_bytes / us / 1e3
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "kernel": "gemv_kernel<F16,R=4,CH=2,NORM,GATEUP> (fused RMSNorm + gate/up + SiLU*mul)",
+            "avg_launch_us": round(us, 2), "algorithmic_bytes_per_launch": alg_bytes}
+
+
+def kernel_table(lm):
+    """GB/s of each fused kernel family at its Llama-3-8B shape, cold weights (rotating over
+    the model's 32 layers), HIP-event timed through the C ABI with pre-allocated outputs.
+    Informational; per-launch times of the ~5 us kernels include the launch-to-launch gap."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    layers = lm.model.layers
+    nl = len(layers)
+    hid, inter, v = lm.config.hidden_size, lm.config.intermediate_size, lm.config.vocab_size
+    stream = torch.cuda.current_stream().cuda_stream
+    f16 = dict(device="cuda", dtype=torch.float16)
+    x, res, gamma = torch.randn(hid, **f16), torch.randn(hid, **f16), torch.ones(hid, **f16)
+    hmid = torch.randn(inter, **f16)
+    y = torch.empty(max(v, inter), **f16)
+    out = {}
+
+    def add(name, fn, nbytes, iters=10):
+        us = _event_time_us(fn, iters=iters * nl, warm=nl)
+        out[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                     "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3)}
+
+    def linear(w, xin, norm, resid, n, k):
+        return lambda i: lib.mui_linear(stream, 0, w[i % len(w)], k, xin.data_ptr(), norm, 1e-5, None, None,
+                                        resid, y.data_ptr(), n, k, 1)
+
+    qkv = [l.qkv_proj.linear.weight.data_ptr() for l in layers]
+    n_qkv = layers[0].qkv_proj.linear.weight.shape[0]
+    add("qkv_norm_gemv_%dx%d" % (n_qkv, hid), linear(qkv, x, gamma.data_ptr(), None, n_qkv, hid),
+        2 * n_qkv * hid + 2 * (2 * hid + n_qkv))
+    op = [l.self_attn.o_proj.weight.data_ptr() for l in layers]
+    add("o_proj_gemv_residual_%dx%d" % (hid, hid), linear(op, x, None, res.data_ptr(), hid, hid),
+        2 * hid * hid + 2 * (3 * hid))
+    dn = [l.mlp.down_proj.weight.data_ptr() for l in layers]
+    add("down_gemv_residual_%dx%d" % (hid, inter), linear(dn, hmid, None, res.data_ptr(), hid, inter),
+        2 * hid * inter + 2 * (inter + 2 * hid))
+    add("lm_head_gemv_%dx%d" % (v, hid), linear([lm.lm_head.weight.data_ptr()], x, None, None, v, hid),
+        2 * v * hid + 2 * (hid + v), iters=2)
+    return out
+
+
+def cpu_baseline(config, layers_sample=4, steps_sample=100, ctx_len=64):
+    """The reference's PyTorch fallback path (fp16 tensors, CPU) for one decode step, on a
+    bounded sample: `layers_sample` decoder layers x `steps_sample` steps + one lm_head call,
+    extrapolated linearly to the full depth. Reported, not a target."""
+    import torch
+
+    import oracle
+
+    torch.manual_seed(0)
+    hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
+    hq, hkv = config.num_attention_heads, config.num_key_value_heads
+    d = hid // hq
+    mk = lambda *s: (torch.randn(*s) * 0.02).half()
+    layers = []
+    for _ in range(layers_sample):
+        layers.append(dict(ln1=torch.ones(hid).half(), wqkv=mk((hq + 2 * hkv) * d, hid), wo=mk(hid, hid),
+                           ln2=torch.ones(hid).half(), wg=mk(inter, hid), wu=mk(inter, hid), wd=mk(hid, inter),
+                           k=torch.randn(1, hkv, ctx_len, d).half(), v=torch.randn(1, hkv, ctx_len, d).half()))
+    lm_head = mk(v, hid)
+    cos, sin = oracle.rope_tables(500000.0, d, ctx_len + steps_sample + 1, dtype=torch.float16)
+    h0 = torch.randn(1, 1, hid).half()
+
+    def layer_step(p, h, pos):
+        qkv = oracle.linear(h, p["wqkv"], p["ln1"], 1e-5, reference_path=True)
+        q = qkv[..., : hq * d].view(1, 1, hq, d).transpose(1, 2)
+        k = qkv[..., hq * d : (hq + hkv) * d].view(1, 1, hkv, d).transpose(1, 2)
+        vv = qkv[..., (hq + hkv) * d :].view(1, 1, hkv, d).transpose(1, 2)
+        q, k = oracle.apply_rope(q, k, cos, sin, torch.tensor([[pos]]), reference_path=True)
+        kk = torch.cat([p["k"], k], dim=2)
+        vv = torch.cat([p["v"], vv], dim=2)
+        a = oracle.decode_attention(q, kk, vv, reference_path=True)
+        h1 = oracle.linear(a, p["wo"], residual=h, reference_path=True)
+        return oracle.gateupdown_mlp(h1, p["wg"], p["wu"], p["wd"], p["ln2"], 1e-5, h1, reference_path=True)
+
+    with torch.no_grad():
+        layer_step(layers[0], h0, ctx_len)  # warm-up
+        t0 = time.perf_counter()
+        for s in range(steps_sample):
+            h = h0
+            for p in layers:
+                h = layer_step(p, h, ctx_len + s)
+        t_layers = (time.perf_counter() - t0) / (steps_sample * layers_sample)
+        oracle.linear(h0, lm_head, torch.ones(hid).half(), 1e-5, reference_path=True)
+        t0 = time.perf_counter()
+        oracle.linear(h0, lm_head, torch.ones(hid).half(), 1e-5, reference_path=True)
+        t_head = time.perf_counter() - t0
+    per_token = t_layers * config.num_hidden_layers + t_head
+    return {"value": round(1.0 / per_token, 4), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{layers_sample} decoder layers x {steps_sample} decode steps (ctx {ctx_len}) + 1 lm_head call of the "
+                      f"reference's PyTorch fallback path in fp16 on CPU, extrapolated to {config.num_hidden_layers} layers",
+            "s_per_layer": round(t_layers, 4), "s_lm_head": round(t_head, 4), "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=32, help="decoder depth (32 = the Llama-3-8B shape; fewer is NOT the benchmark)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-table", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build drives exactly one GPU (no tensor parallelism, no collectives); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from muillm_amd.engineconfig import MuiEngineConfig
+    from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    config = MuiDecoderConfig.llama3_8b(num_hidden_layers=args.layers, max_position_embeddings=8192)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
+    torch.cuda.synchronize()
+
+    dt, dec = bench_decode(lm, args.steps, args.warmup)
+    tokens_per_s = args.steps / dt
+    hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
+    hq, hkv, d = config.num_attention_heads, config.num_key_value_heads, 128
+    weight_bytes = config.num_hidden_layers * 2 * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter) + 2 * v * hid
+
+    result = {
+        "metric": "tokens/s/user, Llama-3-8B-shaped fp16 decode, batch 1",
+        "value": round(tokens_per_s, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": round(tokens_per_s / BASELINE_TOKENS_PER_S, 3) if args.layers == 32 else None,
+        "dtype": "fp16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Llama-3-8B-shaped decoder, random init N(0,0.02): {config.num_hidden_layers} layers, hidden 4096, "
+                        "32/8 heads x128, MLP 14336, vocab 128256, RMSNorm eps 1e-5; 32-token random prompt then greedy "
+                        "decode at batch 1, static KV cache, HIP-graph replay of the decode step",
+            "prompt_len": 32, "batch": 1, "cache_capacity": dec.cache.max_cache_len,
+            "weight_bytes_per_token": weight_bytes,
+            "hbm_floor_ms": round(weight_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4),
+            "end_to_end_frac_of_hbm_floor": round(weight_bytes / (HBM_PEAK_GBPS * 1e9) / (dt / args.steps), 4),
+        },
+    }
+    result["roofline"] = gateup_roofline(lm)
+    if not args.no_kernel_table:
+        result["kernels"] = kernel_table(lm)
+    del dec
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(config)
+        result["cpu_baseline"]["gpu_over_cpu"] = round(tokens_per_s / result["cpu_baseline"]["value"], 1)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

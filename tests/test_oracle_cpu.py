@@ -1,0 +1,260 @@
+"""Pins the CPU oracle itself (no GPU): every oracle function is checked against something
+that does not retype its formula -- golden vectors written by the HuggingFace library
+(tests/golden/hf_llama_small.npz, made by tests/golden/make_fixtures.py), closed forms,
+invariants, and float64 numpy brute force on tiny inputs -- chosen so that a dropped term,
+a wrong sign/index or a transposed operand fails at least one of them."""
+
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hf_llama_small.npz")
+
+
+@pytest.fixture(scope="module")
+def gold():
+    z = np.load(GOLD, allow_pickle=False)
+    return {k: torch.from_numpy(z[k]) for k in z.files if k != "versions"}
+
+
+# ------------------------------------------------------------------------------------
+# golden vectors from the HuggingFace library
+# ------------------------------------------------------------------------------------
+def test_rmsnorm_vs_hf(gold):
+    y = oracle.rmsnorm(gold["norm_x"], gold["norm_w"], 1e-5)
+    assert torch.allclose(y, gold["norm_y"].double(), atol=1e-6)
+    y16 = oracle.rmsnorm(gold["norm_x"], gold["norm_w"], 1e-5, reference_path=True)
+    assert torch.allclose(y16, gold["norm_y"], atol=1e-6)
+
+
+def test_mlp_vs_hf(gold):
+    y = oracle.gateupdown_mlp(gold["mlp_x"], gold["mlp_wg"], gold["mlp_wu"], gold["mlp_wd"])
+    assert torch.allclose(y, gold["mlp_y"].double(), atol=1e-5)
+    # swapping gate and up must change the result (silu is applied to gate only)
+    y_sw = oracle.gateupdown_mlp(gold["mlp_x"], gold["mlp_wu"], gold["mlp_wg"], gold["mlp_wd"])
+    assert not torch.allclose(y_sw, gold["mlp_y"].double(), atol=1e-3)
+
+
+def test_rope_vs_hf(gold):
+    inv = oracle.rope_inv_freq(500000.0, 64)
+    assert torch.equal(inv, gold["rope_inv_freq"])
+    cos, sin = oracle.rope_tables(500000.0, 64, 96)
+    pos = gold["rope_pos"]
+    assert torch.allclose(cos[pos], gold["rope_cos"], atol=1e-6) and torch.allclose(sin[pos], gold["rope_sin"], atol=1e-6)
+    qr, kr = oracle.apply_rope(gold["rope_q"], gold["rope_k"], cos, sin, pos)
+    assert torch.allclose(qr, gold["rope_qr"].double(), atol=1e-5)
+    assert torch.allclose(kr, gold["rope_kr"].double(), atol=1e-5)
+
+
+def test_llama3_rope_scaling_vs_hf(gold):
+    from muillm_amd.modules.attention.rotaryembedding import compute_rope_inv_freq
+
+    inv, scale = compute_rope_inv_freq("llama3", 500000.0, 128, dict(
+        factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192))
+    assert scale == 1.0 and torch.allclose(inv, gold["llama3_inv_freq"], rtol=1e-6, atol=0)
+    inv_d, _ = compute_rope_inv_freq("default", 500000.0, 64)
+    assert torch.equal(inv_d, gold["rope_inv_freq"])
+
+
+def test_attention_vs_hf(gold):
+    out = oracle.decode_attention(gold["attn_q"], gold["attn_k"], gold["attn_v"], gold["attn_mask"])
+    ref = gold["attn_out"].reshape(2, 1, 4 * 64).double()  # HF returns [B, T, H, D]
+    assert torch.allclose(out, ref, atol=1e-5)
+    out16 = oracle.decode_attention(gold["attn_q"], gold["attn_k"], gold["attn_v"], gold["attn_mask"], reference_path=True)
+    assert torch.allclose(out16.double(), ref, atol=1e-5)
+
+
+def test_whole_model_vs_hf(gold):
+    """decoder_layer / decoder_model_step compose to HF's LlamaForCausalLM logits."""
+    sd = {k[3:]: v.float() for k, v in gold.items() if k.startswith("sd.")}
+    layers = []
+    for i in range(2):
+        p = f"model.layers.{i}."
+        layers.append(dict(ln1=sd[p + "input_layernorm.weight"], wq=sd[p + "self_attn.q_proj.weight"],
+                           wk=sd[p + "self_attn.k_proj.weight"], wv=sd[p + "self_attn.v_proj.weight"],
+                           wo=sd[p + "self_attn.o_proj.weight"], ln2=sd[p + "post_attention_layernorm.weight"],
+                           wg=sd[p + "mlp.gate_proj.weight"], wu=sd[p + "mlp.up_proj.weight"],
+                           wd=sd[p + "mlp.down_proj.weight"], eps=1e-5))
+    params = dict(embed=sd["model.embed_tokens.weight"], layers=layers, norm=sd["model.norm.weight"],
+                  lm_head=sd["lm_head.weight"], eps=1e-5)
+    cos, sin = oracle.rope_tables(500000.0, 64, 32)
+    ids = gold["model_ids"]
+    mk = lambda: [torch.zeros(2, 1, 16, 64, dtype=torch.float64) for _ in range(2)]
+    kc, vc = mk(), mk()
+    logits, seen = oracle.decoder_model_step(ids, params, kc, vc, cos, sin, 0, 2, 1, store_dtype=torch.float64)
+    assert seen == 10
+    assert torch.allclose(logits, gold["model_logits"].double(), atol=2e-5)
+    # prefill 7 tokens then three single-token steps give the same logits (static cache path)
+    kc, vc = mk(), mk()
+    lg, seen = oracle.decoder_model_step(ids[:, :7], params, kc, vc, cos, sin, 0, 2, 1, store_dtype=torch.float64)
+    for t in range(7, 10):
+        lg, seen = oracle.decoder_model_step(ids[:, t : t + 1], params, kc, vc, cos, sin, seen, 2, 1, store_dtype=torch.float64)
+        assert torch.allclose(lg[:, 0], gold["model_logits"][:, t].double(), atol=2e-5)
+
+
+# ------------------------------------------------------------------------------------
+# closed forms, invariants, brute force
+# ------------------------------------------------------------------------------------
+def test_linear_brute_force_and_closed_forms():
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal((5, 7))
+    x = rng.standard_normal((2, 7))
+    g = rng.standard_normal(7)
+    b, r, mb = rng.standard_normal(5), rng.standard_normal((2, 5)), rng.standard_normal(5)
+    eps = 1e-3
+    ref = np.zeros((2, 5))
+    for t in range(2):
+        ms = sum(x[t, k] ** 2 for k in range(7)) / 7
+        xn = [g[k] * x[t, k] / math.sqrt(ms + eps) for k in range(7)]
+        for n in range(5):
+            ref[t, n] = sum(w[n, k] * xn[k] for k in range(7)) * mb[n] + b[n] + r[t, n]
+    T = torch.from_numpy
+    got = oracle.linear(T(x), T(w), T(g), eps, T(b), T(r), T(mb))
+    assert np.allclose(got.numpy(), ref, atol=1e-12)
+    xx = torch.randn(3, 16)
+    assert torch.allclose(oracle.linear(xx, torch.eye(16)), xx.double())
+    assert torch.allclose(oracle.linear(xx, torch.ones(2, 16)), xx.double().sum(-1, keepdim=True).expand(3, 2))
+    outs = oracle.multilinear(xx, [torch.eye(16)[:4], torch.eye(16)[4:6]])
+    assert torch.allclose(outs[0], xx[:, :4].double()) and torch.allclose(outs[1], xx[:, 4:6].double())
+
+
+def test_rmsnorm_invariants():
+    x = torch.randn(4, 64)
+    ones = torch.ones(64)
+    y = oracle.rmsnorm(x, ones, 0.0)
+    assert torch.allclose(y.pow(2).mean(-1), torch.ones(4, dtype=torch.float64))
+    assert torch.allclose(oracle.rmsnorm(x * 7, ones, 0.0), y)
+    c = torch.full((1, 64), -2.5)
+    assert torch.allclose(oracle.rmsnorm(c, ones, 0.0), -torch.ones(1, 64, dtype=torch.float64))
+    # eps is added to the mean, not divided by K
+    assert torch.allclose(oracle.rmsnorm(torch.zeros(1, 64) + 1e-4, ones, 1.0), torch.full((1, 64), 1e-4, dtype=torch.float64), rtol=1e-6)
+
+
+def test_mlp_closed_forms():
+    x, r = torch.randn(2, 8), torch.randn(2, 8)
+    w, wd, z = torch.randn(12, 8), torch.randn(8, 12), torch.zeros(12, 8)
+    assert torch.allclose(oracle.gateupdown_mlp(x, z, w, wd, residual=r), r.double())
+    assert torch.allclose(oracle.gateupdown_mlp(x, w, z, wd, residual=r), r.double())
+    g = oracle.gateup_silu(x, w, w)
+    a = x.double() @ w.double().T
+    assert torch.allclose(g, a * a / (1 + torch.exp(-a)))
+
+
+def test_group_rtn_brute_force():
+    rng = np.random.default_rng(1)
+    w = rng.standard_normal((3, 8)).astype(np.float32)
+    q, smv = oracle.rtn_quantize_group(torch.from_numpy(w), group_size=4)
+    for n in range(3):
+        for gi in range(2):
+            grp = w[n, 4 * gi : 4 * gi + 4]
+            lo, hi = float(grp.min()), float(grp.max())
+            scale = (hi - lo) / 255
+            assert abs(float(smv[n * 2 + gi, 0]) - scale) < 1e-6 and abs(float(smv[n * 2 + gi, 1]) - lo) < 1e-6
+            for j in range(4):
+                assert int(q[n, 4 * gi + j]) == int(np.clip(np.round((grp[j] - lo) / scale), 0, 255))
+    dq = oracle.rtn_dequantize_group(q, smv, 4, torch.float32)
+    assert float((dq - torch.from_numpy(w)).abs().max()) <= float(smv[:, 0].max()) * 0.5 + 1e-6
+    # constant group -> range clamp, no division by zero
+    q0, smv0 = oracle.rtn_quantize_group(torch.full((1, 4), 0.25), 4)
+    assert torch.isfinite(smv0).all() and torch.allclose(oracle.rtn_dequantize_group(q0, smv0, 4, torch.float32), torch.full((1, 4), 0.25), atol=1e-5)
+
+
+def test_group_dequant_kernel_form_vs_python_form():
+    w = (torch.randn(8, 64) * 0.02).half()
+    q, smv = oracle.rtn_quantize_group(w, 16)
+    a = oracle.rtn_dequantize_group(q, smv, 16, torch.float16, kernel_form=True)
+    b = oracle.rtn_dequantize_group(q, smv, 16, torch.float16, kernel_form=False)
+    exact = (q.reshape(-1, 16).double() * smv[:, None, 0].double() + smv[:, None, 1].double()).reshape(8, 64)
+    assert float((a.double() - exact).abs().max()) <= float((b.double() - exact).abs().max()) + 1e-9
+    assert torch.equal(a, exact.float().half())  # fp32 fma then one rounding == exact value rounded twice in order
+
+
+def test_channel_rtn_closed_forms():
+    w = torch.tensor([[0.5, -1.0, 0.25, 0.0], [0.0, 0.0, 0.0, 0.0], [2.0, 1.0, -0.5, 0.125]], dtype=torch.float16)
+    q, s = oracle.rtn_quantize_channel(w)
+    assert q.dtype == torch.int8 and s.dtype == torch.float16
+    assert int(q[0, 1]) == -127 and int(q[2, 0]) == 127 and not q[1].any() and float(s[1]) > 0
+    assert abs(float(s[0]) - 1.0 / 127) < 1e-5
+    dq = oracle.rtn_dequantize_channel(q, s)
+    assert torch.equal(dq, q.half() * s[:, None])
+    assert bool(((dq.float() - w.float()).abs() <= s.float()[:, None] * 0.5 + w.float().abs() * 2.0 ** -9).all())
+    # round-half-even: 2.5 steps -> 2, 3.5 -> 4 (scale exactly 1/64 -> max 127/64)
+    w2 = torch.tensor([[127 / 64, 2.5 / 64, 3.5 / 64, -2.5 / 64]], dtype=torch.float16)
+    q2, s2 = oracle.rtn_quantize_channel(w2)
+    assert float(s2[0]) == 1 / 64 and q2.tolist() == [[127, 2, 4, -2]]
+
+
+def test_rope_properties_and_brute_force():
+    d = 8
+    cos, sin = oracle.rope_tables(10000.0, d, 64)
+    q, k = torch.randn(1, 2, 1, d), torch.randn(1, 2, 1, d)
+    q0, k0 = oracle.apply_rope(q, k, cos, sin, torch.tensor([[0]]))
+    assert torch.allclose(q0, q.double()) and torch.allclose(k0, k.double())
+    # complex-rotation brute force: pairs (i, i + d/2) rotate by pos * theta^(-2i/d)
+    pos = 13
+    qr, _ = oracle.apply_rope(q, k, cos, sin, torch.tensor([[pos]]))
+    for h in range(2):
+        for i in range(d // 2):
+            ang = np.float32(pos) * np.float32(1.0 / (10000.0 ** (2 * i / d)))
+            z = complex(float(q[0, h, 0, i]), float(q[0, h, 0, i + d // 2])) * complex(math.cos(ang), math.sin(ang))
+            assert abs(float(qr[0, h, 0, i]) - z.real) < 1e-5 and abs(float(qr[0, h, 0, i + d // 2]) - z.imag) < 1e-5
+    # relative-position property
+    def dot(m, n):
+        a, _ = oracle.apply_rope(q, k, cos, sin, torch.tensor([[m]]))
+        _, b = oracle.apply_rope(q, k, cos, sin, torch.tensor([[n]]))
+        return (a * b).sum(-1)
+    assert torch.allclose(dot(9, 4), dot(45, 40), atol=1e-4)
+    assert not torch.allclose(dot(9, 4), dot(9, 5), atol=1e-3)
+
+
+def test_static_cache_update_semantics():
+    kc, vc = torch.zeros(1, 2, 8, 4), torch.zeros(1, 2, 8, 4)
+    k1, v1 = torch.randn(1, 2, 3, 4), torch.randn(1, 2, 3, 4)
+    kk, vv, seen = oracle.static_cache_update(kc, vc, k1, v1, torch.arange(3), 0)
+    assert seen == 3 and torch.equal(kk, k1) and torch.equal(vv, v1)
+    k2, v2 = torch.randn(1, 2, 1, 4), torch.randn(1, 2, 1, 4)
+    kk, vv, seen = oracle.static_cache_update(kc, vc, k2, v2, torch.tensor([3]), seen)
+    assert seen == 4 and torch.equal(kk, torch.cat([k1, k2], 2)) and not kc[:, :, 4:].any()
+    assert oracle.next_pow2(288) == 512 and oracle.next_pow2(1) == 1
+
+
+def test_attention_closed_forms_and_brute_force():
+    rng = np.random.default_rng(2)
+    b, hq, hkv, s, d = 1, 4, 2, 5, 6
+    q = rng.standard_normal((b, hq, 1, d))
+    k = rng.standard_normal((b, hkv, s, d))
+    v = rng.standard_normal((b, hkv, s, d))
+    ref = np.zeros((b, 1, hq * d))
+    for h in range(hq):
+        kv = h // (hq // hkv)
+        sc = np.array([sum(q[0, h, 0, i] * k[0, kv, t, i] for i in range(d)) / math.sqrt(d) for t in range(s)])
+        p = np.exp(sc - sc.max())
+        p /= p.sum()
+        for i in range(d):
+            ref[0, 0, h * d + i] = sum(p[t] * v[0, kv, t, i] for t in range(s))
+    T = torch.from_numpy
+    got = oracle.decode_attention(T(q), T(k), T(v))
+    assert np.allclose(got.numpy(), ref, atol=1e-12)
+    # the grouped form equals the reference's repeat_kv form
+    rk = oracle.repeat_kv(T(k), 2)
+    assert rk.shape == (1, 4, 5, 6) and torch.equal(rk[:, 1], T(k)[:, 0]) and torch.equal(rk[:, 2], T(k)[:, 1])
+    # S = 1 -> v0 ; identical keys -> mean of V
+    out1 = oracle.decode_attention(T(q), T(k[:, :, :1]), T(v[:, :, :1]))
+    assert np.allclose(out1.numpy().reshape(hq, d), np.repeat(v[0, :, 0], 2, axis=0))
+    same = np.repeat(k[:, :, :1], s, axis=2)
+    outm = oracle.decode_attention(T(q), T(same), T(v))
+    assert np.allclose(outm.numpy().reshape(hq, d), np.repeat(v[0].mean(1), 2, axis=0))
+    # an additive -inf mask removes keys
+    m = torch.zeros(1, 1, 1, s, dtype=torch.float64)
+    m[..., :2] = float("-inf")
+    outk = oracle.decode_attention(T(q), T(k), T(v), m)
+    assert torch.allclose(outk, oracle.decode_attention(T(q), T(k[:, :, 2:]), T(v[:, :, 2:])))
+
+
+def test_rel_err_denominator():
+    assert oracle.rel_err(torch.tensor([1.0, 2.0]), torch.tensor([1.0, 4.0])) == 0.5
