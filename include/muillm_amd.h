@@ -252,6 +252,9 @@ int mui_argmax(mui_stream_t stream, int dtype, const void* logits, long row_stri
  * ---------------------------------------------------------------------------------- */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
+/* token count from which the 16-bit linears switch from one GEMV per token to the MFMA
+ * skinny-GEMM kernel (default 2; MUI_MAX_TOKENS + 1 disables it) */
+int mui_tune_skinny(int min_tokens);
 
 #ifdef __cplusplus
 }

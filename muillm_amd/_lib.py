@@ -68,6 +68,7 @@ _SIGNATURES = {
     "mui_argmax": (c_int, [_P, c_int, _P, c_long, _P, c_int, c_int]),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
+    "mui_tune_skinny": (c_int, [c_int]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -17,6 +17,7 @@
 //     barrier per row group (double-buffered LDS);
 //   * the rsqrt factor is applied to the finished dot product, not to the 4096 inputs.
 #include "common.cuh"
+#include "skinny.cuh"
 
 namespace mui {
 
@@ -232,6 +233,15 @@ static int launch_gemv(hipStream_t s, int dtype, const GemvParams& p) {
 
 using namespace mui;
 
+// token count from which the MFMA skinny-GEMM kernel takes over (below: one GEMV per token)
+static int g_skinny_min_tokens = 2;
+
+extern "C" int mui_tune_skinny(int min_tokens) {
+  if (min_tokens < 1 || min_tokens > MUI_MAX_TOKENS + 1) return MUI_ERR_INVALID_ARG;
+  g_skinny_min_tokens = min_tokens;
+  return MUI_OK;
+}
+
 extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
   if (!(rows_linear == 0 || rows_linear == 2 || rows_linear == 4)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
@@ -255,6 +265,22 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
+  if (tokens >= g_skinny_min_tokens) {
+    SkinnyParams sp = {};
+    sp.w0 = weights;
+    sp.pitch = w_pitch;
+    sp.x = (const uint16_t*)x;
+    sp.gamma = (const uint16_t*)norm_weights;
+    sp.mul_bias = (const uint16_t*)mul_bias;
+    sp.add_bias = (const uint16_t*)add_bias;
+    sp.residual = (const uint16_t*)residual;
+    sp.y = (uint16_t*)y;
+    sp.n = n_out;
+    sp.k = k_in;
+    sp.tokens = tokens;
+    sp.eps = epsilon;
+    return launch_skinny(s, dtype, WF_16BIT, SK_LINEAR, sp);
+  }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     GemvParams p;
     p.w0 = (const uint16_t*)weights;
@@ -290,6 +316,20 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
+  if (tokens >= g_skinny_min_tokens) {
+    SkinnyParams sp = {};
+    sp.w0 = gate;
+    sp.w1 = up;
+    sp.pitch = gu_pitch;
+    sp.x = (const uint16_t*)x;
+    sp.gamma = (const uint16_t*)norm_weights;
+    sp.y = (uint16_t*)h;
+    sp.n = n_inter;
+    sp.k = k_in;
+    sp.tokens = tokens;
+    sp.eps = epsilon;
+    return launch_skinny(s, dtype, WF_16BIT, SK_GATEUP, sp);
+  }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     GemvParams p;
     p.w0 = (const uint16_t*)gate;

@@ -18,6 +18,7 @@
 // sign bit (q + 128), and the 128 * sum(x) correction is folded into the accumulator's
 // initial value, so dequantisation costs one VALU op per weight.
 #include "common.cuh"
+#include "skinny.cuh"
 
 namespace mui {
 
@@ -355,6 +356,14 @@ extern "C" int mui_int8_linear(mui_stream_t stream, int dtype, const void* weigh
   if (st != MUI_OK) return st;
   MUI_CHECK_ARG(scales && y);
   hipStream_t s = (hipStream_t)stream;
+  if (tokens >= 2) {
+    SkinnyParams sp = {};
+    sp.w0 = weights_i8; sp.pitch = w_pitch; sp.s0 = (const uint16_t*)scales; sp.s_pitch = 1;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.add_bias = (const uint16_t*)add_bias; sp.residual = (const uint16_t*)residual;
+    sp.y = (uint16_t*)y; sp.n = n_out; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_skinny(s, dtype, WF_I8_CHANNEL, SK_LINEAR, sp);
+  }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     Int8Params p = {};
     p.w0 = (const uint8_t*)weights_i8;
@@ -385,6 +394,14 @@ extern "C" int mui_int8_gateup_silu(mui_stream_t stream, int dtype, const void* 
   MUI_CHECK_ARG(up_i8 && gate_scales && up_scales && h && scale_stride >= 1);
   if (!aligned16(up_i8)) return MUI_ERR_ALIGNMENT;
   hipStream_t s = (hipStream_t)stream;
+  if (tokens >= 2) {
+    SkinnyParams sp = {};
+    sp.w0 = gate_i8; sp.w1 = up_i8; sp.pitch = gu_pitch;
+    sp.s0 = (const uint16_t*)gate_scales; sp.s1 = (const uint16_t*)up_scales; sp.s_pitch = scale_stride;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.y = (uint16_t*)h; sp.n = n_inter; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_skinny(s, dtype, WF_I8_CHANNEL, SK_GATEUP, sp);
+  }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     Int8Params p = {};
     p.w0 = (const uint8_t*)gate_i8;
@@ -416,6 +433,15 @@ extern "C" int mui_int8_group_linear(mui_stream_t stream, int dtype, const void*
   if (group_size_shift < 4 || group_size_shift > 30) return MUI_ERR_UNSUPPORTED;
   if (k_in & ((1 << group_size_shift) - 1)) return MUI_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
+  if (tokens >= 2) {
+    SkinnyParams sp = {};
+    sp.w0 = weights_u8; sp.pitch = w_pitch; sp.s0 = (const uint16_t*)scales_min_vals;
+    sp.s_pitch = 2L * (k_in >> group_size_shift); sp.group_shift = group_size_shift;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.add_bias = (const uint16_t*)add_bias; sp.residual = (const uint16_t*)residual;
+    sp.y = (uint16_t*)y; sp.n = n_out; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_skinny(s, dtype, WF_U8_GROUP, SK_LINEAR, sp);
+  }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     Int8Params p = {};
     p.w0 = (const uint8_t*)weights_u8;
@@ -450,6 +476,15 @@ extern "C" int mui_int8_group_gateup_silu(mui_stream_t stream, int dtype, const 
   if (k_in & ((1 << group_size_shift) - 1)) return MUI_ERR_UNSUPPORTED;
   if (smv_pitch < 2L * (k_in >> group_size_shift) || (smv_pitch & 1)) return MUI_ERR_INVALID_ARG;
   hipStream_t s = (hipStream_t)stream;
+  if (tokens >= 2) {
+    SkinnyParams sp = {};
+    sp.w0 = gate_u8; sp.w1 = up_u8; sp.pitch = gu_pitch;
+    sp.s0 = (const uint16_t*)gate_smv; sp.s1 = (const uint16_t*)up_smv; sp.s_pitch = smv_pitch;
+    sp.group_shift = group_size_shift;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.y = (uint16_t*)h; sp.n = n_inter; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_skinny(s, dtype, WF_U8_GROUP, SK_GATEUP, sp);
+  }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     Int8Params p = {};
     p.w0 = (const uint8_t*)gate_u8;

@@ -88,7 +88,7 @@ def test_channel_gateup(n, k, tokens, packed):
     else:
         a = (qg.to(DEV), qu.to(DEV), sg.to(DEV), su.to(DEV))
     h = muillm_ext.mui_int8_channel_gateupsilu_forward(gamma.to(DEV), 1e-5, a[0], a[1], a[2], a[3], x.to(DEV))
-    assert_parity(h, ref, 1e-2, f"int8 gateup {n}x{k}", tight=6e-3)
+    assert_parity(h, ref, 1e-2, f"int8 gateup {n}x{k}", tight=6e-3 if tokens == 1 else 9e-3)
 
 
 def test_channel_closed_forms():
