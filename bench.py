@@ -199,6 +199,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="decoder depth (32 = the Llama-3-8B shape; fewer is NOT the benchmark)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
+    ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS",
+                    help="experiment: mui_tune_attention(waves per workgroup, min tokens per split)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (no tensor parallelism, no collectives); "
@@ -211,6 +213,11 @@ def main():
     from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.tune_attention:
+        from muillm_amd import _lib
+
+        w, mt = (int(v) for v in args.tune_attention.split(","))
+        _lib.check(_lib.load().mui_tune_attention(w, mt), "mui_tune_attention")
     config = MuiDecoderConfig.llama3_8b(num_hidden_layers=args.layers, max_position_embeddings=8192)
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
     torch.cuda.synchronize()

@@ -201,7 +201,7 @@ int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, long q_batc
  * scratch size in bytes that mui_flash_decode / mui_attn_decode_fused need for it (0 when
  * n_splits == 1). The reference fixes 4 tokens per group (csrc/attention/flash_decoding.cu:15,153-158)
  * and allocates its partials inside the call. */
-int mui_flash_decode_splits(int batch, int n_kv_heads, int seq_len_hint);
+int mui_flash_decode_splits(int batch, int n_q_heads, int n_kv_heads, int seq_len_hint);
 size_t mui_flash_decode_scratch_bytes(int batch, int n_q_heads, int head_dim, int n_splits);
 
 /* muillm_causal_transformer_decoding_no_mask / _masked (csrc/module.cpp:276-277;
@@ -252,6 +252,9 @@ int mui_argmax(mui_stream_t stream, int dtype, const void* logits, long row_stri
  * ---------------------------------------------------------------------------------- */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
+/* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16) and
+ * the fewest cached tokens that justify one more sequence split (default: two passes) */
+int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split);
 /* token count from which the 16-bit linears switch from one GEMV per token to the MFMA
  * skinny-GEMM kernel (default 2; MUI_MAX_TOKENS + 1 disables it) */
 int mui_tune_skinny(int min_tokens);

@@ -28,9 +28,10 @@
 namespace mui {
 
 constexpr int kHeadDim = 128;
-constexpr int kAttnThreads = 256;
-constexpr int kAttnWaves = kAttnThreads / kWave;
-constexpr int kWorkers = kAttnWaves * 4;  // DPP rows per workgroup
+// A workgroup is NW wave64s (4 or 16). Each wave holds 4 DPP rows = 4 token workers, so a
+// pass of the workgroup covers NW * 4 * U tokens. 16 waves (4 per SIMD) hide the dependent
+// latency of the per-token math far better than 4; they need <= 128 VGPRs per lane, which
+// rules them out for 8 query heads per KV head.
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct AttnParams {
@@ -134,14 +135,17 @@ __device__ __forceinline__ void attend_block(const u32x4 (&kreg)[UU], const u32x
   }
 }
 
-template <typename T, int G, int U, bool DIRECT>
-__global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnParams p) {
+template <typename T, int G, int U, int NW, bool DIRECT>
+__global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParams p) {
+  constexpr int kAttnThreads = NW * kWave;
+  constexpr int kWorkers = NW * 4;      // DPP rows per workgroup
+  constexpr bool kPipe = (NW <= 4);     // few waves: double-buffer K/V in registers instead
   __shared__ __attribute__((aligned(16))) uint16_t q_lds[G][kHeadDim];
   __shared__ __attribute__((aligned(16))) uint16_t kn_lds[kHeadDim];
   __shared__ __attribute__((aligned(16))) uint16_t vn_lds[kHeadDim];
-  __shared__ float lds_m[kWorkers][G];
-  __shared__ float lds_l[kWorkers][G];
-  __shared__ __attribute__((aligned(16))) float tile[kWorkers][G][kHeadDim];
+  __shared__ float lds_m[NW][G];
+  __shared__ float lds_l[NW][G];
+  __shared__ __attribute__((aligned(16))) float tile[NW][G][kHeadDim];
 
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int t = threadIdx.x;
@@ -167,6 +171,30 @@ __global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnPar
   const float* cos_row = p.cos ? p.cos + pos * p.rope_stride : nullptr;
   const float* sin_row = p.sin ? p.sin + pos * p.rope_stride : nullptr;
 
+  // ---- K/V streaming state; the first block is requested before anything else so that the
+  //      query rotation below overlaps with its latency (the new slot is never read) ----
+  const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
+  const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
+  const uint16_t* mrow = p.mask ? p.mask + (long)b * p.mask_bs : nullptr;
+  auto load_block = [&](int base, u32x4 (&kreg)[U], u32x4 (&vreg)[U], bool (&valid)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int tok = base + u * kWorkers + wk;
+      valid[u] = (tok < t_end) && (tok != slot);
+      const int tk = valid[u] ? tok : t_begin;  // t_begin < S: always a readable row
+      kreg[u] = ld16(kc + (long)tk * p.c_ts);
+      vreg[u] = ld16(vc + (long)tk * p.c_ts);
+      if (mrow != nullptr && valid[u]) {
+        if (T::one(mrow[tok]) != 0.f) valid[u] = false;
+      }
+    }
+  };
+  u32x4 ka[U], va[U], kb[U], vb[U];
+  bool valid_a[U], valid_b[U];
+  int base = t_begin;
+  bool have_a = base < t_end;
+  if (have_a) load_block(base, ka, va, valid_a);
+
   // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once) ----
   for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
     const int g = e / kHeadDim, d = e % kHeadDim;
@@ -184,7 +212,7 @@ __global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnPar
       const uint16_t r = T::pack(rope_elem<T>(kp, t, cos_row, sin_row));
       kn_lds[t] = r;
       p.k_cache[coff + t] = r;
-    } else {
+    } else if (t < 2 * kHeadDim) {
       const int d = t - kHeadDim;
       const uint16_t v = p.v_new[(long)b * p.v_bs + (long)kvh * p.v_hs + d];
       vn_lds[d] = v;
@@ -209,27 +237,34 @@ __global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnPar
     for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
   }
 
-  const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
-  const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
-  const uint16_t* mrow = p.mask ? p.mask + (long)b * p.mask_bs : nullptr;
-
-  for (int base = t_begin; base < t_end; base += kBlock) {
-    u32x4 kreg[U], vreg[U];
-    bool valid[U];
+  {
     float madd[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int tok = base + u * kWorkers + wk;
-      valid[u] = (tok < t_end) && (tok != slot);
-      const int tk = valid[u] ? tok : t_begin;  // t_begin < S: always a readable row
-      kreg[u] = ld16(kc + (long)tk * p.c_ts);
-      vreg[u] = ld16(vc + (long)tk * p.c_ts);
-      madd[u] = 0.f;
-      if (mrow != nullptr && valid[u]) {
-        if (T::one(mrow[tok]) != 0.f) valid[u] = false;
+    for (int u = 0; u < U; ++u) madd[u] = 0.f;
+    if constexpr (kPipe) {
+      // two register sets: the next block is in flight while the current one is consumed
+      for (;;) {
+        if (!have_a) break;
+        const int nb = base + kBlock;
+        const bool have_b = nb < t_end;
+        if (have_b) load_block(nb, kb, vb, valid_b);
+        attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
+        if (!have_b) break;
+        base = nb + kBlock;
+        have_a = base < t_end;
+        if (have_a) load_block(base, ka, va, valid_a);
+        attend_block<T, G, U>(kb, vb, valid_b, madd, qreg, p.scale_log2, m, l, acc);
+      }
+    } else {
+      // 4 waves per SIMD overlap each other's loads; one register set keeps the kernel
+      // under 128 VGPRs
+      while (have_a) {
+        attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
+        base += kBlock;
+        have_a = base < t_end;
+        if (have_a) load_block(base, ka, va, valid_a);
       }
     }
-    attend_block<T, G, U>(kreg, vreg, valid, madd, qreg, p.scale_log2, m, l, acc);
   }
 
   if (owner && wave == 0) {  // the new token, straight from LDS, on DPP row 0 of wave 0
@@ -243,10 +278,26 @@ __global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnPar
     attend_block<T, G, 1>(kreg, vreg, valid, madd, qreg, p.scale_log2, m, l, acc);
   }
 
-  // ---- merge the 16 workers of the workgroup ----
-  if (dc == 0) {
+  // ---- stage 1: merge the 4 workers (DPP rows) of each wave with cross-row shuffles; every
+  //      row ends up with the wave's combined (m, l, acc) ----
 #pragma unroll
-    for (int g = 0; g < G; ++g) lds_m[wk][g] = m[g];
+  for (int off = 16; off <= 32; off <<= 1) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float mo = __shfl_xor(m[g], off);
+      const float mn = fmaxf(m[g], mo);
+      const float mu = (mn == -INFINITY) ? 0.f : mn;
+      const float fs = fast_exp2(m[g] - mu), fo = fast_exp2(mo - mu);
+      l[g] = l[g] * fs + __shfl_xor(l[g], off) * fo;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * fs + __shfl_xor(acc[g][i], off) * fo;
+      m[g] = mn;
+    }
+  }
+  // ---- stage 2: merge the NW waves through LDS ----
+  if (lane == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) lds_m[wave][g] = m[g];
   }
   __syncthreads();
   float f[G];
@@ -254,17 +305,19 @@ __global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnPar
   for (int g = 0; g < G; ++g) {
     float mx = lds_m[0][g];
 #pragma unroll
-    for (int w2 = 1; w2 < kWorkers; ++w2) mx = fmaxf(mx, lds_m[w2][g]);
+    for (int w2 = 1; w2 < NW; ++w2) mx = fmaxf(mx, lds_m[w2][g]);
     const float m_use = (mx == -INFINITY) ? 0.f : mx;
     f[g] = fast_exp2(m[g] - m_use);
   }
+  if (ts == 0) {
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    if (dc == 0) lds_l[wk][g] = l[g] * f[g];
-    f32x4 a0 = {acc[g][0] * f[g], acc[g][1] * f[g], acc[g][2] * f[g], acc[g][3] * f[g]};
-    f32x4 a1 = {acc[g][4] * f[g], acc[g][5] * f[g], acc[g][6] * f[g], acc[g][7] * f[g]};
-    *(f32x4*)&tile[wk][g][dc * 8] = a0;
-    *(f32x4*)&tile[wk][g][dc * 8 + 4] = a1;
+    for (int g = 0; g < G; ++g) {
+      if (dc == 0) lds_l[wave][g] = l[g] * f[g];
+      f32x4 a0 = {acc[g][0] * f[g], acc[g][1] * f[g], acc[g][2] * f[g], acc[g][3] * f[g]};
+      f32x4 a1 = {acc[g][4] * f[g], acc[g][5] * f[g], acc[g][6] * f[g], acc[g][7] * f[g]};
+      *(f32x4*)&tile[wave][g][dc * 8] = a0;
+      *(f32x4*)&tile[wave][g][dc * 8 + 4] = a1;
+    }
   }
   __syncthreads();
 
@@ -273,7 +326,7 @@ __global__ void __launch_bounds__(kAttnThreads) attn_decode_kernel(const AttnPar
     const int head = kvh * G + g;
     float a = 0.f, lsum = 0.f, mx = lds_m[0][g];
 #pragma unroll
-    for (int w2 = 0; w2 < kWorkers; ++w2) {
+    for (int w2 = 0; w2 < NW; ++w2) {
       a += tile[w2][g][d];
       lsum += lds_l[w2][g];
       mx = fmaxf(mx, lds_m[w2][g]);
@@ -361,15 +414,37 @@ __global__ void __launch_bounds__(kHeadDim) rope_kv_write_kernel(const RopeParam
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
-constexpr int kU = 4;
+// tokens per worker and pass: 4 with 4 or 8 waves (<= 256 VGPRs available), 2 with 16 waves
+// (128 VGPRs)
+constexpr int unroll_for(int nw) { return nw == 16 ? 2 : 4; }
+
+static int g_attn_waves = 0;  // 0: built-in choice; 4, 8 or 16 forces the workgroup size
+
+// waves per workgroup for a given number of query heads per KV head
+static inline int attn_waves_for(int g) {
+  if (g > 4) return 4;  // 8 heads per group: ~240 VGPRs, one wave per SIMD
+  return g_attn_waves ? g_attn_waves : 8;
+}
+
+template <typename T, int G, int NW>
+static void launch_attn_nw(hipStream_t s, const AttnParams& p, dim3 grid) {
+  if (p.n_splits == 1)
+    hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, true>), grid, dim3(NW * kWave), 0, s, p);
+  else
+    hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, false>), grid, dim3(NW * kWave), 0, s, p);
+}
 
 template <typename T, int G>
 static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
-  dim3 grid(p.n_splits, p.hkv, batch), block(kAttnThreads);
-  if (p.n_splits == 1)
-    hipLaunchKernelGGL((attn_decode_kernel<T, G, kU, true>), grid, block, 0, s, p);
-  else
-    hipLaunchKernelGGL((attn_decode_kernel<T, G, kU, false>), grid, block, 0, s, p);
+  dim3 grid(p.n_splits, p.hkv, batch);
+  const int nw = attn_waves_for(G);
+  if constexpr (G <= 4) {
+    if (nw == 16) launch_attn_nw<T, G, 16>(s, p, grid);
+    else if (nw == 8) launch_attn_nw<T, G, 8>(s, p, grid);
+    else launch_attn_nw<T, G, 4>(s, p, grid);
+  } else {
+    launch_attn_nw<T, G, 4>(s, p, grid);
+  }
   int st = launch_status();
   if (st != MUI_OK) return st;
   if (p.n_splits > 1) {
@@ -401,14 +476,32 @@ static int launch_attn(hipStream_t s, int dtype, const AttnParams& p, int batch)
 
 using namespace mui;
 
-extern "C" int mui_flash_decode_splits(int batch, int n_kv_heads, int seq_len_hint) {
-  if (batch <= 0 || n_kv_heads <= 0 || seq_len_hint <= 0) return 1;
-  constexpr int kBlock = kWorkers * kU;               // tokens per workgroup iteration
-  const int max_useful = ceil_div(seq_len_hint, 2 * kBlock);  // >= 2 iterations per split
-  const int want = ceil_div(4 * device_cus(), batch * n_kv_heads);
+static int g_attn_min_tokens = 0;  // 0: built-in choice; else fewest tokens worth a split
+
+extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split) {
+  if (!(waves_per_workgroup == 0 || waves_per_workgroup == 4 || waves_per_workgroup == 8 || waves_per_workgroup == 16))
+    return MUI_ERR_INVALID_ARG;
+  if (min_tokens_per_split < 0) return MUI_ERR_INVALID_ARG;
+  g_attn_waves = waves_per_workgroup;
+  g_attn_min_tokens = min_tokens_per_split;
+  return MUI_OK;
+}
+
+extern "C" int mui_flash_decode_splits(int batch, int n_q_heads, int n_kv_heads, int seq_len_hint) {
+  if (batch <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || seq_len_hint <= 0) return 1;
+  const int nw = attn_waves_for(n_q_heads / n_kv_heads);
+  const int kBlock = nw * 4 * unroll_for(nw);  // tokens per workgroup pass
+  // Splitting buys parallelism but every split beyond the first costs the combine launch
+  // (~4 us) and partial traffic, so a split must carry a few passes of work. (Merging the
+  // splits inside the kernel with a device-scope fence + counter was measured slower than
+  // the combine launch on MI355X.) The total is capped near 1.5 workgroups per CU: measured
+  // best at 32 splits for batch 1 and 4-8 splits for batch 8 with 8 KV heads.
+  const int min_tokens = g_attn_min_tokens > 0 ? g_attn_min_tokens : 2 * kBlock;
+  const int max_useful = ceil_div(seq_len_hint, min_tokens);
+  int want = ceil_div(3 * device_cus() / 2, batch * n_kv_heads);
+  if (want > 32) want = 32;
   int n = want < max_useful ? want : max_useful;
   if (n < 1) n = 1;
-  if (n > 256) n = 256;
   return n;
 }
 

@@ -86,8 +86,26 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvParams p) {
     }
   };
 
+  // epilogue operands (biases, residual) of a row group are fetched together with its
+  // weights, one group ahead, so no dependent global load sits behind the final barrier
+  float e_mb = 1.f, e_ab = 0.f, e_res = 0.f;
+  auto issue_epi = [&](int rg) {
+    if constexpr (EPI == EPI_LINEAR) {
+      if (t < OUT) {
+        int n = rg * OUT + t;
+        n = n < p.n ? n : p.n - 1;
+        e_mb = p.mul_bias ? T::one(p.mul_bias[n]) : 1.f;
+        e_ab = p.add_bias ? T::one(p.add_bias[n]) : 0.f;
+        e_res = p.residual ? T::one(p.residual[n]) : 0.f;
+      }
+    }
+  };
+
   int rg = blockIdx.x;
-  if (rg < n_groups) issue(rg);  // weights first: they are the long pole
+  if (rg < n_groups) {
+    issue(rg);  // weights first: they are the long pole
+    issue_epi(rg);
+  }
 
   // ---- inputs: gamma * x in fp32 registers, sum of squares on the side ----
   float xs[CH][8];
@@ -143,8 +161,12 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvParams p) {
       acc[r] = a0 + a1;
     }
 
+    const float c_mb = e_mb, c_ab = e_ab, c_res = e_res;
     const int nxt = rg + gridDim.x;
-    if (nxt < n_groups) issue(nxt);  // keep the memory pipe full during the reduction
+    if (nxt < n_groups) {  // keep the memory pipe full during the reduction
+      issue(nxt);
+      issue_epi(nxt);
+    }
 
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
@@ -165,9 +187,7 @@ __global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvParams p) {
           v = silu_f32(g) * u;
         } else {
           v = ((red[buf][0][t] + red[buf][1][t]) + (red[buf][2][t] + red[buf][3][t])) * rs;
-          if (p.mul_bias) v *= T::one(p.mul_bias[n]);
-          if (p.add_bias) v += T::one(p.add_bias[n]);
-          if (p.residual) v += T::one(p.residual[n]);
+          v = fmaf(v, c_mb, c_ab) + c_res;
         }
         p.y[n] = T::pack(v);
       }

@@ -641,7 +641,7 @@ def _decode(q, k, v, m, n_splits=None) -> torch.Tensor:
         m = m.contiguous()
         mask_ptr, mask_bs = m.data_ptr(), m.stride(0)
     if n_splits is None:
-        n_splits = lib.mui_flash_decode_splits(b, hkv, s)
+        n_splits = lib.mui_flash_decode_splits(b, hq, hkv, s)
     scratch = _scratch(lib, q, b, hq, d, n_splits)
     out = torch.empty((b, 1, hq * d), dtype=q.dtype, device=q.device)
     # max_cache_len: rows reachable through the view (the view is narrowed to s already)
@@ -694,7 +694,7 @@ def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_positi
         mask_ptr, mask_bs = mask.data_ptr(), mask.stride(0)
     if n_splits is None:
         hint = seq_len if seq_len is not None else (seq_len_hint if seq_len_hint is not None else max_t)
-        n_splits = lib.mui_flash_decode_splits(b, hkv, int(hint))
+        n_splits = lib.mui_flash_decode_splits(b, hq, hkv, int(hint))
     scratch = _scratch(lib, q2, b, hq, d, n_splits)
     out = torch.empty((b, 1, hq * d), dtype=q.dtype, device=q.device)
     q_out = torch.empty((b, hq, 1, d), dtype=q.dtype, device=q.device) if want_q_out else None
