@@ -28,6 +28,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the gate/up GEMV at the Llama-3-8B shape, from two `rocprofv3 --pmc` runs of
+# `bench.py --pmc-probe` (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
+# counter reads for the probe's elementwise copy of 234,881,024 B: FETCH_SIZE reads 114,706.1 for the copy
+# (x2.0000 to KiB) and 114,783.2 for the GEMV; WRITE_SIZE reads 229,376.0 for the copy (x1.0) and 224.0 for
+# the GEMV. 235,038,826 B fetched + 229,417 B written.
+GATEUP_TRAFFIC_BYTES = 235038826 + 229417
 BASELINE_TOKENS_PER_S = 210.0  # reference README: Llama-3-8B fp16 bs1 on 1x MI300X
 
 
@@ -90,9 +96,39 @@ def gateup_roofline(lm):
     alg_bytes = 2 * inter * hid * 2 + 2 * (hid + hid + inter)  # G and U once, x, gamma, h
     achieved = alg_bytes / us / 1e3
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": GATEUP_TRAFFIC_BYTES if (hid, inter) == (4096, 14336) else None,
             "kernel": "gemv_kernel<F16,R=4,CH=2,NORM,GATEUP> (fused RMSNorm + gate/up + SiLU*mul)",
             "avg_launch_us": round(us, 2), "algorithmic_bytes_per_launch": alg_bytes}
+
+
+def pmc_probe(launches=6):
+    """Counter probe for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: a few launches of the
+    fused gate/up GEMV at the Llama-3-8B shape over distinct weight buffers, then the same number of
+    launches of a plain elementwise copy kernel that reads and writes exactly as many bytes as one
+    gate/up launch reads (the calibration for the counter's unit)."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    hid, inter = 4096, 14336
+    f16 = dict(device="cuda", dtype=torch.float16)
+    ws = [torch.randn(inter, 2, hid, **f16) * 0.02 for _ in range(launches)]
+    x, gamma, h = torch.randn(hid, **f16), torch.ones(hid, **f16), torch.empty(inter, **f16)
+    src = [torch.randn(inter * 2 * hid, **f16) for _ in range(2)]
+    dst = torch.empty(inter * 2 * hid, **f16)
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    for w in ws:
+        _lib.check(lib.mui_gateup_silu(stream, 0, w[:, 0].data_ptr(), w[:, 1].data_ptr(), 2 * hid, x.data_ptr(),
+                                       gamma.data_ptr(), 1e-5, h.data_ptr(), inter, hid, 1), "mui_gateup_silu")
+    torch.cuda.synchronize()
+    for i in range(launches):
+        torch.mul(src[i % 2], 1.0, out=dst)
+    torch.cuda.synchronize()
+    print(json.dumps({"pmc_probe": {"launches": launches, "gateup_algorithmic_bytes": 2 * inter * hid * 2 + 2 * (2 * hid + inter),
+                                    "copy_bytes_read": dst.numel() * 2, "copy_bytes_written": dst.numel() * 2}}))
 
 
 def kernel_table(lm):
@@ -201,6 +237,8 @@ def main():
     ap.add_argument("--no-kernel-table", action="store_true")
     ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS",
                     help="experiment: mui_tune_attention(waves per workgroup, min tokens per split)")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (no tensor parallelism, no collectives); "
@@ -213,6 +251,9 @@ def main():
     from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.pmc_probe:
+        pmc_probe()
+        return
     if args.tune_attention:
         from muillm_amd import _lib
 
