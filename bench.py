@@ -132,9 +132,11 @@ def pmc_probe(launches=6):
 
 
 def kernel_table(lm):
-    """GB/s of each fused kernel family at its Llama-3-8B shape, cold weights (rotating over
-    the model's 32 layers), HIP-event timed through the C ABI with pre-allocated outputs.
-    Informational; per-launch times of the ~5 us kernels include the launch-to-launch gap."""
+    """GB/s of each fused kernel family at the benchmark shapes, HIP-event timed through the C ABI
+    with pre-allocated outputs. Weights rotate over distinct buffers totalling >= 0.9 GB (the model's
+    32 layers, or a ring) so neither L2 nor the 256 MB Infinity Cache can serve them ("cold").
+    Bytes are algorithmic: weights (+ scales) once plus the mandatory vectors. Informational; times
+    of the few-microsecond kernels include the launch-to-launch gap of back-to-back launches."""
     import torch
 
     from muillm_amd import _lib
@@ -145,33 +147,118 @@ def kernel_table(lm):
     hid, inter, v = lm.config.hidden_size, lm.config.intermediate_size, lm.config.vocab_size
     stream = torch.cuda.current_stream().cuda_stream
     f16 = dict(device="cuda", dtype=torch.float16)
-    x, res, gamma = torch.randn(hid, **f16), torch.randn(hid, **f16), torch.ones(hid, **f16)
-    hmid = torch.randn(inter, **f16)
-    y = torch.empty(max(v, inter), **f16)
+    gamma = (1 + 0.1 * torch.randn(hid)).half().cuda()
+    X, RES = torch.randn(8, hid, **f16), torch.randn(8, hid, **f16)
+    HMID = torch.randn(8, inter, **f16)
+    Y = torch.empty(8 * max(v, inter), **f16)
     out = {}
 
-    def add(name, fn, nbytes, iters=10):
-        us = _event_time_us(fn, iters=iters * nl, warm=nl)
+    def add(name, fn, nbytes, ring, iters=10):
+        us = _event_time_us(fn, iters=max(iters * ring, 40), warm=max(ring, 8))
         out[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                      "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3)}
 
-    def linear(w, xin, norm, resid, n, k):
+    def linear(w, xin, norm, resid, n, k, b=1):
         return lambda i: lib.mui_linear(stream, 0, w[i % len(w)], k, xin.data_ptr(), norm, 1e-5, None, None,
-                                        resid, y.data_ptr(), n, k, 1)
+                                        resid, Y.data_ptr(), n, k, b)
 
+    # ---- 16-bit GEMV family at the decoder's shapes (1 token)
     qkv = [l.qkv_proj.linear.weight.data_ptr() for l in layers]
     n_qkv = layers[0].qkv_proj.linear.weight.shape[0]
-    add("qkv_norm_gemv_%dx%d" % (n_qkv, hid), linear(qkv, x, gamma.data_ptr(), None, n_qkv, hid),
-        2 * n_qkv * hid + 2 * (2 * hid + n_qkv))
     op = [l.self_attn.o_proj.weight.data_ptr() for l in layers]
-    add("o_proj_gemv_residual_%dx%d" % (hid, hid), linear(op, x, None, res.data_ptr(), hid, hid),
-        2 * hid * hid + 2 * (3 * hid))
     dn = [l.mlp.down_proj.weight.data_ptr() for l in layers]
-    add("down_gemv_residual_%dx%d" % (hid, inter), linear(dn, hmid, None, res.data_ptr(), hid, inter),
-        2 * hid * inter + 2 * (inter + 2 * hid))
-    add("lm_head_gemv_%dx%d" % (v, hid), linear([lm.lm_head.weight.data_ptr()], x, None, None, v, hid),
-        2 * v * hid + 2 * (hid + v), iters=2)
+    add("C1_norm_linear_residual_%dx%d" % (hid, hid), linear(op, X, gamma.data_ptr(), RES.data_ptr(), hid, hid),
+        2 * hid * hid + 2 * (4 * hid), nl)
+    add("qkv_norm_gemv_%dx%d" % (n_qkv, hid), linear(qkv, X, gamma.data_ptr(), None, n_qkv, hid),
+        2 * n_qkv * hid + 2 * (2 * hid + n_qkv), nl)
+    add("o_proj_gemv_residual_%dx%d" % (hid, hid), linear(op, X, None, RES.data_ptr(), hid, hid),
+        2 * hid * hid + 2 * (3 * hid), nl)
+    add("down_gemv_residual_%dx%d" % (hid, inter), linear(dn, HMID, None, RES.data_ptr(), hid, inter),
+        2 * hid * inter + 2 * (inter + 2 * hid), nl)
+    add("lm_head_gemv_%dx%d" % (v, hid), linear([lm.lm_head.weight.data_ptr()], X, None, None, v, hid),
+        2 * v * hid + 2 * (hid + v), 1, iters=40)
+
+    # ---- C2: the whole MLP (fused norm + gate/up + SiLU, then down + residual), 1..8 tokens
+    gu = [(l.mlp.gate_proj.weight.data_ptr(), l.mlp.up_proj.weight.data_ptr(), l.mlp.gate_proj.weight.stride(0),
+           l.mlp.norm_weights.data_ptr()) for l in layers]
+    hbuf = torch.empty(8, inter, **f16)
+    for b in (1, 2, 4, 8):
+        def mlp(i, b=b):
+            gp, up, pitch, nw = gu[i % nl]
+            lib.mui_gateup_silu(stream, 0, gp, up, pitch, X.data_ptr(), nw, 1e-5, hbuf.data_ptr(), inter, hid, b)
+            lib.mui_linear(stream, 0, dn[i % nl], inter, hbuf.data_ptr(), None, 0.0, None, None, RES.data_ptr(),
+                           Y.data_ptr(), hid, inter, b)
+        add("C2_mlp_%dx%d_tokens%d" % (inter, hid, b), mlp,
+            3 * inter * hid * 2 + 2 * hid + b * (3 * hid * 2 + 2 * inter * 2), nl)
+
+    # ---- C3: int8 per-channel GEMVs (ring of random codes: speed does not depend on the values)
+    def i8_ring(n, k):
+        cnt = max(2, int(0.95e9 // (n * k)) + 1)
+        return [(torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda"),
+                 (torch.rand(n, **f16) * 1e-3 + 1e-4)) for _ in range(cnt)]
+
+    for b in (1, 4):
+        for name, n, k, norm, resid in (("qkv", n_qkv, hid, True, False), ("o_proj", hid, hid, False, True),
+                                        ("down", hid, inter, False, True)):
+            ring = i8_ring(n, k)
+            xin = X if k == hid else HMID
+
+            def f(i, ring=ring, xin=xin, n=n, k=k, norm=norm, resid=resid, b=b):
+                q, sc = ring[i % len(ring)]
+                lib.mui_int8_linear(stream, 0, q.data_ptr(), k, sc.data_ptr(), xin.data_ptr(),
+                                    gamma.data_ptr() if norm else None, 1e-5, None,
+                                    RES.data_ptr() if resid else None, Y.data_ptr(), n, k, b)
+            add("C3_int8_%s_%dx%d_tokens%d" % (name, n, k, b), f,
+                n * k + 2 * n + 2 * hid * norm + b * 2 * (k + n + n * resid), len(ring))
+            del ring
+        ring = [(torch.randint(-127, 128, (inter, 2, hid), dtype=torch.int8, device="cuda"),
+                 torch.rand(inter, 2, **f16) * 1e-3 + 1e-4) for _ in range(9)]
+
+        def g(i, ring=ring, b=b):
+            q, sc = ring[i % len(ring)]
+            lib.mui_int8_gateup_silu(stream, 0, q.data_ptr(), q.data_ptr() + hid, 2 * hid, sc.data_ptr(),
+                                     sc.data_ptr() + 2, 2, X.data_ptr(), gamma.data_ptr(), 1e-5, hbuf.data_ptr(),
+                                     inter, hid, b)
+        add("C3_int8_gateup_silu_%dx%d_tokens%d" % (2 * inter, hid, b), g,
+            2 * inter * hid + 4 * inter + 2 * hid + b * 2 * (hid + inter), len(ring))
+        del ring
+    torch.cuda.empty_cache()
+
+    # ---- C4: fused RoPE + cache write + flash decoding, GQA 32/8 x 128 (bytes = the K/V rows read)
+    hq, hkv, d = 32, 8, 128
+    for S, B in ((1024, 1), (4096, 1), (16384, 1), (32768, 1), (1024, 8), (4096, 8), (32768, 8)):
+        kvbytes = B * 2 * hkv * S * d * 2
+        cnt = max(2, min(64, int(1.0e9 // kvbytes) + 1))
+        caches = [(torch.randn(B, hkv, S, d, **f16), torch.randn(B, hkv, S, d, **f16)) for _ in range(cnt)]
+        qkvx = torch.randn(B, (hq + 2 * hkv) * d, **f16)
+        cos, sin = [t.cuda() for t in _rope_tables_f32(S, d)]
+        pos = torch.full((B, 1), S - 1, dtype=torch.int64, device="cuda")
+        cpos = torch.full((1,), S - 1, dtype=torch.int64, device="cuda")
+        n_splits = lib.mui_flash_decode_splits(B, hq, hkv, S)
+        scratch = torch.empty(max(lib.mui_flash_decode_scratch_bytes(B, hq, d, n_splits), 16), dtype=torch.uint8, device="cuda")
+        o = torch.empty(B, hq * d, **f16)
+
+        qs = (hq + 2 * hkv) * d
+
+        def att(i, caches=caches, B=B, S=S, n_splits=n_splits):
+            kc, vc = caches[i % len(caches)]
+            lib.mui_attn_decode_fused(stream, 0, qkvx.data_ptr(), qs, qkvx.data_ptr() + 2 * hq * d, qs,
+                                      qkvx.data_ptr() + 2 * (hq + hkv) * d, qs, cos.data_ptr(), sin.data_ptr(), d // 2,
+                                      pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
+                                      hkv * S * d, S * d, d, None, 0, None, scratch.data_ptr(), n_splits, o.data_ptr(),
+                                      B, hq, hkv, d, S)
+        add("C4_rope_cachewrite_flashdecode_ctx%d_batch%d_splits%d" % (S, B, n_splits), att, kvbytes + 4 * B * hq * d, cnt)
+        del caches
+        torch.cuda.empty_cache()
     return out
+
+
+def _rope_tables_f32(max_pos, d, theta=500000.0):
+    import torch
+
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
+    ang = torch.outer(torch.arange(max_pos, dtype=torch.float64), inv)
+    return ang.cos().float().contiguous(), ang.sin().float().contiguous()
 
 
 def cpu_baseline(config, layers_sample=4, steps_sample=100, ctx_len=64):
@@ -235,8 +322,9 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="decoder depth (32 = the Llama-3-8B shape; fewer is NOT the benchmark)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
-    ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS",
-                    help="experiment: mui_tune_attention(waves per workgroup, min tokens per split)")
+    ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS,DIRECT",
+                    help="experiment: mui_tune_attention(waves per workgroup, min tokens per split, "
+                         "longest unsplit sequence; -1 disables the head-parallel unsplit mode)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
     args = ap.parse_args()
@@ -257,8 +345,8 @@ def main():
     if args.tune_attention:
         from muillm_amd import _lib
 
-        w, mt = (int(v) for v in args.tune_attention.split(","))
-        _lib.check(_lib.load().mui_tune_attention(w, mt), "mui_tune_attention")
+        w, mt, dt = (int(v) for v in args.tune_attention.split(","))
+        _lib.check(_lib.load().mui_tune_attention(w, mt, dt), "mui_tune_attention")
     config = MuiDecoderConfig.llama3_8b(num_hidden_layers=args.layers, max_position_embeddings=8192)
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
     torch.cuda.synchronize()

@@ -252,9 +252,11 @@ int mui_argmax(mui_stream_t stream, int dtype, const void* logits, long row_stri
  * ---------------------------------------------------------------------------------- */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
-/* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16) and
- * the fewest cached tokens that justify one more sequence split (default: two passes) */
-int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split);
+/* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
+ * fewest cached tokens that justify one more sequence split (default: two passes), and the
+ * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1024;
+ * negative: never use the unsplit one-workgroup-per-query-head mode) */
+int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens);
 /* token count from which the 16-bit linears switch from one GEMV per token to the MFMA
  * skinny-GEMM kernel (default 2; MUI_MAX_TOKENS + 1 disables it) */
 int mui_tune_skinny(int min_tokens);

@@ -6,9 +6,12 @@
 // pass and final reduce (csrc/attention/flash_decoding_fp16_kernels.cu:199-586, 642-785).
 //
 // Layout of the work (T = 1 new token per batch row, head_dim 128):
-//   grid = (splits of the cached sequence, KV heads, batch); one workgroup = 4 wave64s.
-//   A workgroup serves ALL G = Hq/Hkv query heads that share its KV head, so K and V are
-//   read from HBM exactly once (the reference re-reads them once per query head).
+//   grid = (splits of the cached sequence, blocks of G query heads, batch).
+//   Normally G = Hq/Hkv: a workgroup serves ALL query heads that share its KV head, so K and V
+//   are read from HBM exactly once (the reference re-reads them once per query head).
+//   Short sequences at small batch are latency-bound instead: there the launcher uses G = 1
+//   and no sequence split (one workgroup per query head, the few hundred KB of K/V re-read
+//   from cache by the heads of a group), which needs no second kernel to merge splits.
 //   Inside a wave, the 16 lanes of a DPP row own the 16 x 16-byte chunks of ONE token's K/V
 //   row; the 4 rows of a wave take 4 consecutive tokens, so one load instruction covers 1 KiB
 //   of contiguous cache. q.k is a packed-fp16 dot (v_dot2_f32_f16) reduced over the 16 lanes
@@ -147,7 +150,10 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   __shared__ float lds_l[NW][G];
   __shared__ __attribute__((aligned(16))) float tile[NW][G][kHeadDim];
 
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int split = blockIdx.x, b = blockIdx.z;
+  const int head0 = blockIdx.y * G;          // first query head of this workgroup
+  const int group = p.hq / p.hkv;            // query heads per KV head (a multiple of G)
+  const int kvh = head0 / group;
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t >> 6;
@@ -167,6 +173,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   const int t_begin = split * chunk;
   const int t_end = (t_begin + chunk) < S ? (t_begin + chunk) : S;
   const bool owner = has_new && slot >= t_begin && slot < t_begin + chunk && slot < S;
+  const bool writer = owner && (head0 % group == 0);  // one workgroup per KV head stores the slot
 
   const float* cos_row = p.cos ? p.cos + pos * p.rope_stride : nullptr;
   const float* sin_row = p.sin ? p.sin + pos * p.rope_stride : nullptr;
@@ -198,7 +205,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once) ----
   for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
     const int g = e / kHeadDim, d = e % kHeadDim;
-    const int head = kvh * G + g;
+    const int head = head0 + g;
     const uint16_t* qp = p.q + (long)b * p.q_bs + (long)head * p.q_hs;
     const uint16_t r = T::pack(rope_elem<T>(qp, d, cos_row, sin_row));
     q_lds[g][d] = r;
@@ -211,12 +218,12 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
       const uint16_t* kp = p.k_new + (long)b * p.k_bs + (long)kvh * p.k_hs;
       const uint16_t r = T::pack(rope_elem<T>(kp, t, cos_row, sin_row));
       kn_lds[t] = r;
-      p.k_cache[coff + t] = r;
+      if (writer) p.k_cache[coff + t] = r;
     } else if (t < 2 * kHeadDim) {
       const int d = t - kHeadDim;
       const uint16_t v = p.v_new[(long)b * p.v_bs + (long)kvh * p.v_hs + d];
       vn_lds[d] = v;
-      p.v_cache[coff + d] = v;
+      if (writer) p.v_cache[coff + d] = v;
     }
   }
   __syncthreads();
@@ -323,7 +330,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
 
   for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
     const int g = e / kHeadDim, d = e % kHeadDim;
-    const int head = kvh * G + g;
+    const int head = head0 + g;
     float a = 0.f, lsum = 0.f, mx = lds_m[0][g];
 #pragma unroll
     for (int w2 = 0; w2 < NW; ++w2) {
@@ -419,6 +426,8 @@ __global__ void __launch_bounds__(kHeadDim) rope_kv_write_kernel(const RopeParam
 constexpr int unroll_for(int nw) { return nw == 16 ? 2 : 4; }
 
 static int g_attn_waves = 0;  // 0: built-in choice; 4, 8 or 16 forces the workgroup size
+static int g_attn_head_parallel = 1;  // unsplit decodes at small batch: workgroup per query head
+static int g_attn_direct_tokens = 0;  // 0: built-in choice; longest sequence decoded unsplit
 
 // waves per workgroup for a given number of query heads per KV head
 static inline int attn_waves_for(int g) {
@@ -436,7 +445,7 @@ static void launch_attn_nw(hipStream_t s, const AttnParams& p, dim3 grid) {
 
 template <typename T, int G>
 static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
-  dim3 grid(p.n_splits, p.hkv, batch);
+  dim3 grid(p.n_splits, p.hq / G, batch);
   const int nw = attn_waves_for(G);
   if constexpr (G <= 4) {
     if (nw == 16) launch_attn_nw<T, G, 16>(s, p, grid);
@@ -457,6 +466,9 @@ static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
 
 template <typename T>
 static int launch_attn_t(hipStream_t s, const AttnParams& p, int batch) {
+  // unsplit and too few KV heads to occupy the GPU: one workgroup per query head
+  if (p.n_splits == 1 && g_attn_head_parallel && batch * p.hkv * 4 <= device_cus())
+    return launch_attn_g<T, 1>(s, p, batch);
   switch (p.hq / p.hkv) {
     case 1: return launch_attn_g<T, 1>(s, p, batch);
     case 2: return launch_attn_g<T, 2>(s, p, batch);
@@ -478,12 +490,14 @@ using namespace mui;
 
 static int g_attn_min_tokens = 0;  // 0: built-in choice; else fewest tokens worth a split
 
-extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split) {
+extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens) {
   if (!(waves_per_workgroup == 0 || waves_per_workgroup == 4 || waves_per_workgroup == 8 || waves_per_workgroup == 16))
     return MUI_ERR_INVALID_ARG;
   if (min_tokens_per_split < 0) return MUI_ERR_INVALID_ARG;
   g_attn_waves = waves_per_workgroup;
   g_attn_min_tokens = min_tokens_per_split;
+  g_attn_head_parallel = direct_tokens >= 0;
+  g_attn_direct_tokens = direct_tokens > 0 ? direct_tokens : 0;
   return MUI_OK;
 }
 
@@ -496,6 +510,9 @@ extern "C" int mui_flash_decode_splits(int batch, int n_q_heads, int n_kv_heads,
   // splits inside the kernel with a device-scope fence + counter was measured slower than
   // the combine launch on MI355X.) The total is capped near 1.5 workgroups per CU: measured
   // best at 32 splits for batch 1 and 4-8 splits for batch 8 with 8 KV heads.
+  // Short sequences at small batch: one unsplit workgroup per query head beats split + merge.
+  const int direct = g_attn_direct_tokens > 0 ? g_attn_direct_tokens : 1024;
+  if (g_attn_head_parallel && seq_len_hint <= direct && batch * n_kv_heads * 4 <= device_cus()) return 1;
   const int min_tokens = g_attn_min_tokens > 0 ? g_attn_min_tokens : 2 * kBlock;
   const int max_useful = ceil_div(seq_len_hint, min_tokens);
   int want = ceil_div(3 * device_cus() / 2, batch * n_kv_heads);
