@@ -245,6 +245,24 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
 int mui_argmax(mui_stream_t stream, int dtype, const void* logits, long row_stride,
                int64_t* out_index, int rows, int vocab);
 
+/* One launch for the tail of a greedy decode step, per batch row b (all buffers on the device):
+ *   tok = argmax_v logits[b, v]        (as mui_argmax)
+ *   if unfinished != NULL and n_eos > 0 and unfinished[b] == 0: tok = pad_token
+ *   tokens_out[b, step[b]] = tok  (when step[b] < max_steps);  next_ids[b] = tok
+ *   position_ids[b] += 1;  step[b] += 1;  cache_position[0] += 1 (once)
+ *   unfinished[b] &= (tok is none of eos_ids) && (step[b] < max_steps)
+ * It folds the reference's torch.argmax + muillm_add_tokens_check_finished
+ * (csrc/generation/generation.cu:29-113,115-195; muillm/sampling/generation.py:330-404) and
+ * the position bookkeeping of its sampling loop into one kernel that a HIP graph can replay:
+ * the token history is written in place at a device-side column counter instead of being
+ * re-allocated as [B, T+1] every step. position_ids, cache_position and unfinished may be
+ * NULL. */
+int mui_greedy_advance(mui_stream_t stream, int dtype, const void* logits, long row_stride,
+                       int rows, int vocab, int64_t* next_ids, int64_t* position_ids,
+                       int64_t* cache_position, int64_t* step, int64_t* tokens_out,
+                       long tokens_stride, int max_steps, int64_t* unfinished,
+                       const int64_t* eos_ids, int n_eos, long pad_token);
+
 /* ------------------------------------------------------------------------------------
  * Launch-shape knobs used by the benchmark sweeps (0 restores the built-in choice). They
  * have no counterpart in the reference, whose launch shapes are compile-time constants

@@ -14,16 +14,14 @@ __device__ __forceinline__ void take_better(float& v, int& i, float ov, int oi) 
   if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
 }
 
+// argmax of one row by the whole workgroup; the result is valid on thread 0
 template <typename T>
-__global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const uint16_t* logits, long row_stride,
-                                                                    int64_t* out, int vocab) {
+__device__ __forceinline__ int row_argmax(const uint16_t* row, bool vec, int vocab) {
   __shared__ float sv[kArgmaxThreads / kWave];
   __shared__ int si[kArgmaxThreads / kWave];
-  const uint16_t* row = logits + (long)blockIdx.x * row_stride;
   const int t = threadIdx.x;
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  const bool vec = ((row_stride & 7) == 0) && ((((uintptr_t)logits) & 15u) == 0);
   const int nvec = vec ? (vocab >> 3) : 0;
   for (int c = t; c < nvec; c += kArgmaxThreads) {
     float f[8];
@@ -49,7 +47,53 @@ __global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const uint1
   __syncthreads();
   if (t == 0) {
     for (int w = 1; w < kArgmaxThreads / kWave; ++w) take_better(best, best_i, sv[w], si[w]);
-    out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+  }
+  return best_i == 0x7fffffff ? 0 : best_i;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const uint16_t* logits, long row_stride,
+                                                                    int64_t* out, int vocab) {
+  const bool vec = ((row_stride & 7) == 0) && ((((uintptr_t)logits) & 15u) == 0);
+  const int best_i = row_argmax<T>(logits + (long)blockIdx.x * row_stride, vec, vocab);
+  if (threadIdx.x == 0) out[blockIdx.x] = best_i;
+}
+
+// Greedy choice plus everything the decode loop does with it, for batch row blockIdx.x:
+//   tok = argmax(logits[b]); finished rows emit pad_token instead (eos criterion)
+//   tokens_out[b, step[b]] = tok; next_ids[b] = tok; position_ids[b] += 1; step[b] += 1
+//   cache_position[0] += 1 (row 0 only); unfinished[b] &= tok is no eos and steps remain
+// Every row owns its own counters, so the workgroups never read what another one writes.
+struct GreedyParams {
+  const uint16_t* logits; long row_stride; int vocab;
+  int64_t* next_ids;        // [B]
+  int64_t* position_ids;    // [B] or null
+  int64_t* cache_position;  // [1] or null
+  int64_t* step;            // [B]
+  int64_t* tokens_out; long tokens_stride; int max_steps;  // [B, >= max_steps]
+  int64_t* unfinished;      // [B] or null
+  const int64_t* eos_ids; int n_eos; long pad_token;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kArgmaxThreads) greedy_advance_kernel(const GreedyParams p) {
+  const int b = blockIdx.x;
+  const bool vec = ((p.row_stride & 7) == 0) && ((((uintptr_t)p.logits) & 15u) == 0);
+  const int best_i = row_argmax<T>(p.logits + (long)b * p.row_stride, vec, p.vocab);
+  if (threadIdx.x != 0) return;
+  int64_t tok = best_i;
+  const bool was_unfinished = p.unfinished ? (p.unfinished[b] != 0) : true;
+  if (p.unfinished && p.n_eos > 0 && !was_unfinished) tok = p.pad_token;
+  const int64_t st = p.step[b];
+  if (st >= 0 && st < p.max_steps) p.tokens_out[(long)b * p.tokens_stride + st] = tok;
+  p.next_ids[b] = tok;
+  if (p.position_ids) p.position_ids[b] += 1;
+  p.step[b] = st + 1;
+  if (b == 0 && p.cache_position) p.cache_position[0] += 1;
+  if (p.unfinished) {
+    bool unfinished = was_unfinished && (st + 1 < p.max_steps);
+    for (int i = 0; i < p.n_eos; ++i) unfinished = unfinished && (tok != p.eos_ids[i]);
+    p.unfinished[b] = unfinished ? 1 : 0;
   }
 }
 
@@ -67,6 +111,28 @@ extern "C" int mui_argmax(mui_stream_t stream, int dtype, const void* logits, lo
   else if (dtype == MUI_DTYPE_BF16)
     hipLaunchKernelGGL((argmax_rows_kernel<BF16>), dim3(rows), dim3(kArgmaxThreads), 0, s,
                        (const uint16_t*)logits, row_stride, out_index, vocab);
+  else
+    return MUI_ERR_INVALID_ARG;
+  return launch_status();
+}
+
+extern "C" int mui_greedy_advance(mui_stream_t stream, int dtype, const void* logits, long row_stride,
+                                  int rows, int vocab, int64_t* next_ids, int64_t* position_ids,
+                                  int64_t* cache_position, int64_t* step, int64_t* tokens_out,
+                                  long tokens_stride, int max_steps, int64_t* unfinished,
+                                  const int64_t* eos_ids, int n_eos, long pad_token) {
+  MUI_CHECK_ARG(logits && next_ids && step && tokens_out && rows > 0 && vocab > 0 && row_stride >= vocab);
+  MUI_CHECK_ARG(max_steps >= 0 && tokens_stride >= max_steps && n_eos >= 0 && (n_eos == 0 || eos_ids));
+  GreedyParams p = {};
+  p.logits = (const uint16_t*)logits; p.row_stride = row_stride; p.vocab = vocab;
+  p.next_ids = next_ids; p.position_ids = position_ids; p.cache_position = cache_position;
+  p.step = step; p.tokens_out = tokens_out; p.tokens_stride = tokens_stride; p.max_steps = max_steps;
+  p.unfinished = unfinished; p.eos_ids = eos_ids; p.n_eos = n_eos; p.pad_token = pad_token;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MUI_DTYPE_F16)
+    hipLaunchKernelGGL((greedy_advance_kernel<F16>), dim3(rows), dim3(kArgmaxThreads), 0, s, p);
+  else if (dtype == MUI_DTYPE_BF16)
+    hipLaunchKernelGGL((greedy_advance_kernel<BF16>), dim3(rows), dim3(kArgmaxThreads), 0, s, p);
   else
     return MUI_ERR_INVALID_ARG;
   return launch_status();

@@ -8,8 +8,9 @@ decoder layers, final norm, lm_head, argmax, and the advance of the position cou
 recorded once on a side stream and replayed; everything the step needs to know about "where
 are we" lives in device memory (input ids, position ids, cache slot, output slot), and the
 attention kernel reads the sequence length from the cache slot, so the graph never changes
-as the sequence grows. No memset nodes are recorded: counters are advanced with elementwise
-kernels and the argmax is a hand-written kernel."""
+as the sequence grows. No memset nodes are recorded: one hand-written kernel picks the token,
+stores it, applies the eos criterion and advances every counter (the reference's torch.argmax
++ muillm_add_tokens_check_finished, muillm/sampling/generation.py:330-404)."""
 from typing import Optional
 
 import torch
@@ -19,9 +20,11 @@ from ..kvcache.cache_utils import MuiStaticCache, _next_pow2, create_static_cach
 
 
 class MuiGraphDecoder:
-    def __init__(self, lm, use_graph: bool = True):
+    def __init__(self, lm, use_graph: bool = True, eos_token_ids=None, pad_token_id: int = 0):
         self.lm = lm
         self.use_graph = use_graph
+        self.eos_token_ids = list(eos_token_ids) if eos_token_ids is not None else None
+        self.pad_token_id = int(pad_token_id)
         self.graph = None
         self.cache: Optional[MuiStaticCache] = None
         self._batch = None
@@ -31,9 +34,11 @@ class MuiGraphDecoder:
         self.ids = torch.zeros((batch, 1), dtype=torch.int64, device=device)
         self.pos = torch.zeros((batch, 1), dtype=torch.int64, device=device)
         self.cpos = torch.zeros((1,), dtype=torch.int64, device=device)
-        self.step = torch.zeros((1,), dtype=torch.int64, device=device)
+        self.step = torch.zeros((batch,), dtype=torch.int64, device=device)
+        self.unfinished = torch.ones((batch,), dtype=torch.int64, device=device)
+        self.eos = (torch.tensor(self.eos_token_ids, dtype=torch.int64, device=device)
+                    if self.eos_token_ids else None)
         self.out_tokens = torch.zeros((batch, max_new_tokens), dtype=torch.int64, device=device)
-        self.next_token = torch.zeros((batch,), dtype=torch.int64, device=device)
         self.logits = None
         self._batch = batch
         self._max_new = max_new_tokens
@@ -43,19 +48,16 @@ class MuiGraphDecoder:
         out = self.lm(input_ids=self.ids, position_ids=self.pos, cache_position=self.cpos,
                       past_key_values=self.cache, use_cache=True, all_ones_mask=True, float_logits=False)
         logits = out.logits[:, -1, :]
-        muillm_ext.mui_argmax(logits, out=self.next_token)
-        self.out_tokens.scatter_(1, self.step.expand(self._batch, 1), self.next_token.unsqueeze(1))
-        self.ids.copy_(self.next_token.unsqueeze(1))
-        self.pos.add_(1)
-        self.cpos.add_(1)
-        self.step.add_(1)
+        muillm_ext.mui_greedy_advance(logits, self.ids, self.step, self.out_tokens, position_ids=self.pos,
+                                      cache_position=self.cpos, unfinished=self.unfinished,
+                                      eos_token_ids=self.eos, pad_token_id=self.pad_token_id)
         return logits
 
     def _capture(self):
         self.cache.device_length_mode = True
         seen = self.cache._seen_tokens
         # warm up on a side stream (allocator, lazy module state), then restore the cache counters
-        saved = [t.clone() for t in (self.ids, self.pos, self.cpos, self.step, self.out_tokens)]
+        saved = [t.clone() for t in (self.ids, self.pos, self.cpos, self.step, self.out_tokens, self.unfinished)]
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -72,7 +74,7 @@ class MuiGraphDecoder:
             self.cache.cpp_module.seen_tokens = seen
 
     def _restore(self, saved, seen):
-        for dst, src in zip((self.ids, self.pos, self.cpos, self.step, self.out_tokens), saved):
+        for dst, src in zip((self.ids, self.pos, self.cpos, self.step, self.out_tokens, self.unfinished), saved):
             dst.copy_(src)
         self.cache._seen_tokens = seen
         if self.cache.cpp_module is not None:
@@ -104,6 +106,9 @@ class MuiGraphDecoder:
         self.step.fill_(1)
         self.out_tokens.zero_()
         self.out_tokens[:, 0] = first
+        self.unfinished.fill_(1)
+        if self.eos is not None:
+            self.unfinished.copy_((first.unsqueeze(1) != self.eos.unsqueeze(0)).all(dim=1).to(torch.int64))
         return out.logits[:, -1, :]
 
     @torch.no_grad()

@@ -160,7 +160,9 @@ class MuiLlamaModel(MuiModule):
                 inputs_embeds: Optional[torch.Tensor] = None, use_cache: Optional[bool] = None,
                 output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
                 return_dict: Optional[bool] = None, cache_position: Optional[torch.LongTensor] = None,
-                all_ones_mask: Optional[bool] = None):
+                all_ones_mask: Optional[bool] = None, skip_final_norm: bool = False):
+        """skip_final_norm=True returns the un-normalised last hidden state: the causal-LM head
+        then applies the final RMSNorm inside its GEMV kernel (single-token decode)."""
         output_attentions = bool(output_attentions)
         output_hidden_states = bool(output_hidden_states)
         use_cache = True if use_cache is None else use_cache
@@ -221,7 +223,8 @@ class MuiLlamaModel(MuiModule):
             if output_attentions:
                 all_self_attns += (layer_outputs[1],)
 
-        hidden_states = self.norm(hidden_states)
+        if not skip_final_norm:
+            hidden_states = self.norm(hidden_states)
         if output_hidden_states:
             all_hidden_states += (hidden_states,)
         if use_cache and isinstance(past_key_values, MuiCache):
@@ -309,15 +312,26 @@ class MuiLlamaForCausalLM(MuiModule):
                 all_ones_mask: Optional[bool] = None, num_logits_to_keep: int = 0, float_logits: bool = True):
         if labels is not None:
             raise NotImplementedError("inference only: labels/loss are not supported")
+        shape = input_ids.shape if input_ids is not None else inputs_embeds.shape
+        head, norm = self.lm_head, self.model.norm
+        # single-token decode: the final RMSNorm rides inside the lm_head GEMV
+        fuse_norm = (shape[1] == 1 and not output_hidden_states and type(head) is MuiLinear and head.dispatchable
+                     and not head.normalize and norm.dispatchable and head.weight.dtype == norm.weight.dtype)
         outputs = self.model(
             input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids,
             past_key_values=past_key_values, inputs_embeds=inputs_embeds, use_cache=use_cache,
             output_attentions=output_attentions, output_hidden_states=output_hidden_states,
-            cache_position=cache_position, all_ones_mask=all_ones_mask)
+            cache_position=cache_position, all_ones_mask=all_ones_mask, skip_final_norm=fuse_norm)
         hidden_states = outputs.last_hidden_state
         if num_logits_to_keep:
             hidden_states = hidden_states[:, -num_logits_to_keep:, :]
-        logits = self.lm_head(hidden_states)
+        if fuse_norm and hidden_states.is_cuda:
+            logits = muillm_ext.muillm_linear_forward(self.engine_config.cpp_engine, hidden_states, head.weight, norm.weight, norm.variance_epsilon,
+                                                      None, head.bias, None)
+        else:
+            if fuse_norm:
+                hidden_states = norm(hidden_states)
+            logits = self.lm_head(hidden_states)
         if float_logits:
             logits = logits.float()
         return MuiCausalLMOutput(logits=logits, past_key_values=outputs.past_key_values,

@@ -730,3 +730,46 @@ def mui_argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torc
         "mui_argmax",
     )
     return out
+
+
+def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch.Tensor, tokens_out: torch.Tensor,
+                       position_ids: Optional[torch.Tensor] = None, cache_position: Optional[torch.Tensor] = None,
+                       unfinished: Optional[torch.Tensor] = None, eos_token_ids: Optional[torch.Tensor] = None,
+                       pad_token_id: int = 0) -> None:
+    """Tail of a greedy decode step in one launch (everything in place, on the device):
+    argmax of each logits row -> tokens_out[b, step[b]], next_ids[b]; position_ids[b], step[b]
+    and cache_position[0] advance by one; unfinished[b] is cleared on an eos token or when
+    tokens_out is full (finished rows emit pad_token_id, as the reference's
+    muillm_add_tokens_check_finished does).
+
+    logits [B, V] 16-bit; next_ids [B] or [B, 1]; step [B]; tokens_out [B, max_steps];
+    position_ids [B] or [B, 1]; cache_position [1]; unfinished [B]; all integers int64."""
+    _check_cuda(logits, "logits")
+    if logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    v = logits.shape[-1]
+    l2 = logits.reshape(-1, v)
+    rows = l2.shape[0]
+    for name, tns, n in (("next_ids", next_ids, rows), ("step", step, rows), ("position_ids", position_ids, rows),
+                         ("cache_position", cache_position, 1), ("unfinished", unfinished, rows)):
+        if tns is None:
+            continue
+        _check_cuda(tns, name)
+        if tns.dtype != torch.int64 or tns.numel() != n or not tns.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous int64 tensor with {n} element(s)")
+    _check_cuda(tokens_out, "tokens_out")
+    if tokens_out.dtype != torch.int64 or tokens_out.dim() != 2 or tokens_out.shape[0] != rows or tokens_out.stride(1) != 1:
+        raise RuntimeError("tokens_out must be int64 [B, max_steps] with unit inner stride")
+    n_eos = 0
+    if eos_token_ids is not None:
+        _check_cuda(eos_token_ids, "eos_token_ids")
+        if eos_token_ids.dtype != torch.int64 or not eos_token_ids.is_contiguous():
+            raise RuntimeError("eos_token_ids must be a contiguous int64 tensor")
+        n_eos = eos_token_ids.numel()
+    check(
+        _lib.load().mui_greedy_advance(
+            _stream(l2), _dtype_code(l2), l2.data_ptr(), l2.stride(0) if rows > 1 else v, rows, v,
+            next_ids.data_ptr(), _ptr(position_ids), _ptr(cache_position), step.data_ptr(), tokens_out.data_ptr(),
+            tokens_out.stride(0), tokens_out.shape[1], _ptr(unfinished), _ptr(eos_token_ids), n_eos, int(pad_token_id)),
+        "mui_greedy_advance",
+    )

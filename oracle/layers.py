@@ -16,6 +16,7 @@ import torch
 import torch.nn.functional as F
 
 __all__ = [
+    "greedy_advance",
     "rmsnorm",
     "linear",
     "multilinear",
@@ -410,3 +411,39 @@ def decoder_model_step(ids, params, k_caches, v_caches, cos, sin, seen_tokens: i
                                 n_heads, n_kv_heads, store_dtype)
     hn = rmsnorm(h, params["norm"], params["eps"]).to(store_dtype)
     return linear(hn, params["lm_head"]), seen
+
+
+# ---------------------------------------------------------------------------------------
+# generation-loop helper
+# ---------------------------------------------------------------------------------------
+def greedy_advance(logits, unfinished, eos_token_ids, pad_token_id: int, steps_done: int, max_steps: int):
+    """Greedy token choice plus the stop check of the reference's sampling loop:
+    next_tokens = argmax(logits) (muillm/sampling/generation.py:330-335); rows that had already
+    finished emit pad_token_id when an eos criterion exists; a row stays unfinished while its
+    token is none of eos_token_ids and steps remain (muillm_add_tokens_check_finished_kernel,
+    csrc/generation/generation.cu:29-113: `next_token = prev_unfinished ? next_token : pad`,
+    `unfinished &= next_token != eos`, `unfinished &= T <= max_length`).
+    logits [B, V]; unfinished [B] (0/1); steps_done = tokens already emitted per row.
+    Returns (tokens [B] int64, unfinished [B] int64). Plain Python loops: test sizes only."""
+    lg = logits.float()
+    b = lg.shape[0]
+    toks = torch.zeros(b, dtype=torch.int64)
+    unf = torch.zeros(b, dtype=torch.int64)
+    eos = [int(e) for e in eos_token_ids] if eos_token_ids is not None else []
+    for r in range(b):
+        row = lg[r]
+        best, best_i = float("-inf"), None
+        for i in range(row.shape[0]):  # lowest index wins ties; NaN never wins
+            v = float(row[i])
+            if v > best:
+                best, best_i = v, i
+        tok = 0 if best_i is None else best_i
+        was = bool(unfinished[r]) if unfinished is not None else True
+        if eos and not was:
+            tok = int(pad_token_id)
+        still = was and (steps_done + 1 < max_steps)
+        for e in eos:
+            still = still and tok != e
+        toks[r] = tok
+        unf[r] = 1 if still else 0
+    return toks, unf

@@ -203,6 +203,49 @@ def test_argmax_kernel():
     assert torch.equal(muillm_ext.mui_argmax(xb).cpu(), xb.float().argmax(-1).cpu())
 
 
+def test_greedy_advance_kernel():
+    """mui_greedy_advance against the oracle's restatement of argmax + stop check, over several
+    consecutive steps on the same device-side state."""
+    from muillm_amd import muillm_ext
+    g = torch.Generator().manual_seed(3)
+    B, V, max_steps = 5, 1000, 6
+    eos = [17, 400]
+    ids = torch.zeros(B, 1, dtype=torch.int64, device=DEV)
+    pos = torch.full((B, 1), 40, dtype=torch.int64, device=DEV)
+    cpos = torch.full((1,), 40, dtype=torch.int64, device=DEV)
+    step = torch.zeros(B, dtype=torch.int64, device=DEV)
+    toks = torch.full((B, max_steps), -1, dtype=torch.int64, device=DEV)
+    unf = torch.ones(B, dtype=torch.int64, device=DEV)
+    eos_t = torch.tensor(eos, dtype=torch.int64, device=DEV)
+    ref_unf = torch.ones(B, dtype=torch.int64)
+    for s_i in range(max_steps):
+        logits = torch.randn(B, V, generator=g).half()
+        if s_i == 1:
+            logits[2, 17] = 50.0   # row 2 hits an eos token at step 1
+        if s_i == 3:
+            logits[4, 400] = 50.0  # row 4 at step 3
+        muillm_ext.mui_greedy_advance(logits.to(DEV), ids, step, toks, position_ids=pos, cache_position=cpos,
+                                      unfinished=unf, eos_token_ids=eos_t, pad_token_id=9)
+        exp_tok, ref_unf = oracle.greedy_advance(logits, ref_unf, eos, 9, steps_done=s_i, max_steps=max_steps)
+        assert torch.equal(toks[:, s_i].cpu(), exp_tok), s_i
+        assert torch.equal(ids.cpu().view(-1), exp_tok)
+        assert torch.equal(unf.cpu(), ref_unf), s_i
+        assert int(cpos.item()) == 41 + s_i and torch.equal(pos.cpu().view(-1), torch.full((B,), 41 + s_i))
+        assert torch.equal(step.cpu(), torch.full((B,), s_i + 1))
+    assert toks[2, 2:].eq(9).all() and toks[4, 4:].eq(9).all()  # finished rows emit the pad token
+    assert unf.sum().item() == 0                                   # the step budget finished the rest
+    # one more call beyond the budget must not write outside tokens_out
+    before = toks.clone()
+    muillm_ext.mui_greedy_advance(torch.randn(B, V, generator=g).half().to(DEV), ids, step, toks)
+    assert torch.equal(toks, before)
+    # bf16, no optional state
+    lg = torch.randn(2, 333, generator=g).bfloat16().to(DEV)
+    ids2 = torch.zeros(2, dtype=torch.int64, device=DEV); st2 = torch.zeros(2, dtype=torch.int64, device=DEV)
+    out2 = torch.zeros(2, 4, dtype=torch.int64, device=DEV)
+    muillm_ext.mui_greedy_advance(lg, ids2, st2, out2)
+    assert torch.equal(out2[:, 0].cpu(), lg.float().argmax(-1).cpu())
+
+
 @pytest.mark.skipif(not _hf.HAVE_TRANSFORMERS, reason="transformers not installed")
 def test_init_engine_on_hf_llama_gpu_fp16():
     """Drop-in check: a HuggingFace Llama (fp16, GPU) before and after init_engine."""

@@ -258,3 +258,29 @@ def test_attention_closed_forms_and_brute_force():
 
 def test_rel_err_denominator():
     assert oracle.rel_err(torch.tensor([1.0, 2.0]), torch.tensor([1.0, 4.0])) == 0.5
+
+
+def test_greedy_advance_rules():
+    """Stop-check semantics (csrc/generation/generation.cu:29-113) on hand-made cases: the
+    argmax must agree with torch.argmax, an eos token finishes its row, a finished row emits the
+    pad token from then on, and the step budget finishes every row."""
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(4, 50, generator=g)
+    logits[1, 7] = 100.0   # row 1 picks the eos token 7
+    logits[2, 9] = 100.0   # row 2 is already finished: must emit pad, not 9
+    unfinished = torch.tensor([1, 1, 0, 1])
+    toks, unf = oracle.greedy_advance(logits, unfinished, [7, 11], pad_token_id=3, steps_done=0, max_steps=10)
+    expect = logits.argmax(-1)
+    assert toks[0] == expect[0] and toks[3] == expect[3]
+    assert toks[1] == 7 and toks[2] == 3
+    assert unf.tolist() == [1, 0, 0, 1]
+    # last step of the budget finishes everything
+    _, unf2 = oracle.greedy_advance(logits, unfinished, [7, 11], 3, steps_done=9, max_steps=10)
+    assert unf2.tolist() == [0, 0, 0, 0]
+    # without an eos criterion a finished row keeps its argmax
+    toks3, _ = oracle.greedy_advance(logits, unfinished, None, 3, 0, 10)
+    assert torch.equal(toks3, expect)
+    # ties -> lowest index; all -inf -> 0
+    t = torch.zeros(2, 6); t[0, 2] = t[0, 4] = 1.0; t[1, :] = float("-inf")
+    toks4, _ = oracle.greedy_advance(t, None, None, 0, 0, 10)
+    assert toks4.tolist() == [2, 0]
