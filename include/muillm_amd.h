@@ -275,9 +275,10 @@ int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
  * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1024;
  * negative: never use the unsplit one-workgroup-per-query-head mode) */
 int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens);
-/* token count from which the 16-bit linears switch from one GEMV per token to the MFMA
- * skinny-GEMM kernel (default 2; MUI_MAX_TOKENS + 1 disables it) */
-int mui_tune_skinny(int min_tokens);
+/* fewest tokens that take the MFMA skinny-GEMM kernel instead of one GEMV per token (default 2;
+ * MUI_MAX_TOKENS + 1 disables it); stream_b != 0 forces the variant that re-reads the token
+ * operands per weight tile instead of keeping them in registers (K <= 4096 only) */
+int mui_tune_skinny(int min_tokens, int stream_b);
 
 #ifdef __cplusplus
 }

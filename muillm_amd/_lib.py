@@ -71,7 +71,7 @@ _SIGNATURES = {
                                    c_int, c_long]),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
-    "mui_tune_skinny": (c_int, [c_int]),
+    "mui_tune_skinny": (c_int, [c_int, c_int]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -7,10 +7,11 @@
 // columns: the kernel stays HBM-bound, the MFMA pipe is <10 % busy at 8 tokens).
 //
 //   workgroup = 8 wave64s, one tile of 16 weight rows; the K range is split over the waves.
-//   A operand  = weights: lane l loads 16 bytes of row (l % 16) at k-chunk (l / 16) of the
-//                step, straight from HBM (non-temporal). int8 weights are converted to the
-//                16-bit type in registers (per-channel: exact integers, scale applied in the
-//                epilogue; group format: u8*scale+min rounded once to the 16-bit type).
+//   A operand  = weights: lane l loads 16 bytes of row (l % 16) at position (l / 16) of the
+//                step, straight from HBM (non-temporal): one k-chunk of 8 16-bit weights, or
+//                two k-chunks of 8-bit weights (two MFMAs), converted to the 16-bit type in
+//                registers (per-channel: exact integers, scale applied in the epilogue;
+//                group format: u8*scale+min rounded once to the 16-bit type).
 //   B operand  = gamma * x of token (l % 16), same k-chunk, built on the fly from L2-resident
 //                x and gamma (rounded to the 16-bit type like HF's normalised activations);
 //                lanes of tokens >= batch feed zeros. sum(x^2) per token is accumulated by the
@@ -42,22 +43,38 @@ __device__ __forceinline__ f32x4 mfma16x16x32<BF16>(u32x4 a, u32x4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// 8 weights of a chunk -> the 16-bit MFMA operand
+// 8 int8/uint8 weights (two dwords) -> the 16-bit MFMA operand.
+//   per-channel: exact integers (the row scale is applied in the epilogue). For fp16 the bytes
+//   are dropped into the mantissa of 1024.0 (0x6400 | b = 1024 + b) with two byte permutes and
+//   the offset is removed with a packed subtract: 5 VALU ops per dword instead of a convert
+//   and a pack per weight.
+//   group format: u8 * scale + min, rounded once to the 16-bit type.
 template <typename T, int WF>
-__device__ __forceinline__ u32x4 make_a(const void* rp, int chunk, const uint16_t* srow, int group_shift) {
-  if constexpr (WF == WF_16BIT) {
-    return ld16_stream((const uint16_t*)rp + (chunk << 3));
+__device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint16_t* srow, int elem, int group_shift) {
+  const uint32_t v[2] = {w0, w1};
+  if constexpr (WF == WF_I8_CHANNEL && T::kDtype == MUI_DTYPE_F16) {
+    u32x4 out;
+    const f16x2 off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128 (sign bit flipped below)
+    uint32_t o[4];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      const uint32_t u = v[m] ^ 0x80808080u;
+      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+      o[2 * m + 0] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, lo) - off);
+      o[2 * m + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, hi) - off);
+    }
+    out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
+    return out;
   } else {
-    const u32x2 raw = ld8_stream((const uint8_t*)rp + (chunk << 3));
     float f[8];
-    const uint32_t v[2] = {raw.x, raw.y};
     if constexpr (WF == WF_I8_CHANNEL) {
 #pragma unroll
       for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int b = 0; b < 4; ++b) f[4 * m + b] = (float)(int)(int8_t)((v[m] >> (8 * b)) & 0xffu);
     } else {
-      const uint32_t pr = *(const uint32_t*)(srow + 2 * ((chunk << 3) >> group_shift));
+      const uint32_t pr = *(const uint32_t*)(srow + 2 * (elem >> group_shift));
       const float sc = T::lo(pr), mn = T::hi(pr);
 #pragma unroll
       for (int m = 0; m < 2; ++m)
@@ -65,6 +82,38 @@ __device__ __forceinline__ u32x4 make_a(const void* rp, int chunk, const uint16_
         for (int b = 0; b < 4; ++b) f[4 * m + b] = fmaf((float)((v[m] >> (8 * b)) & 0xffu), sc, mn);
     }
     return pack8<T>(f);
+  }
+}
+
+// B operand of one k-chunk: gamma * x rounded to the 16-bit type, sum of squares on the side.
+// fp16: packed multiply (one rounding, same result as the fp32 product rounded once) and a
+// packed dot for the squares.
+template <typename T, bool NORM>
+__device__ __forceinline__ u32x4 make_b(const u32x4 xv, const u32x4 gv, float& ss) {
+  if constexpr (!NORM) {
+    return xv;
+  } else if constexpr (T::kDtype == MUI_DTYPE_F16) {
+    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f16x2 xx = __builtin_bit_cast(f16x2, xw[i]);
+      ss = __builtin_amdgcn_fdot2(xx, xx, ss, false);
+      o[i] = __builtin_bit_cast(uint32_t, xx * __builtin_bit_cast(f16x2, gw[i]));
+    }
+    u32x4 b = {o[0], o[1], o[2], o[3]};
+    return b;
+  } else {
+    float xf[8], gf[8], o[8];
+    unpack8<T>(xv, xf);
+    unpack8<T>(gv, gf);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      ss = fmaf(xf[i], xf[i], ss);
+      o[i] = xf[i] * gf[i];
+    }
+    return pack8<T>(o);
   }
 }
 
@@ -98,8 +147,12 @@ __global__ void __launch_bounds__(kSkThreads) gemm_skinny_kernel(const SkinnyPar
   const void* rp = (const char*)wbase + (long)row_c * p.pitch * kWBytes;
   const uint16_t* srow = (WF == WF_U8_GROUP) ? sbase + (long)row_c * p.s_pitch : nullptr;
 
-  const int kc = p.k >> 3;                       // 8-element chunks per row
-  const int steps = (kc + 3) >> 2;               // MFMA steps over the whole K
+  // A lane reads 16 bytes of its weight row per step: one 8-element k-chunk of 16-bit weights
+  // or two of 8-bit weights (two MFMAs). A and B label k identically, so any k order works.
+  constexpr int CPL = (WF == WF_16BIT) ? 1 : 2;  // k-chunks per lane and step
+  constexpr int UNR = (WF == WF_16BIT) ? kSkUnroll : kSkUnroll / 2;
+  const int kcl = p.k / (8 * CPL);               // lane-chunks per row
+  const int steps = (kcl + 3) >> 2;
   const int per_wave = (steps + kSkWaves - 1) / kSkWaves;
   const int s_begin = wave * per_wave;
   const int s_end = (s_begin + per_wave) < steps ? (s_begin + per_wave) : steps;
@@ -110,40 +163,68 @@ __global__ void __launch_bounds__(kSkThreads) gemm_skinny_kernel(const SkinnyPar
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   float ss = 0.f;
 
-  for (int s0 = s_begin; s0 < s_end; s0 += kSkUnroll) {
-    u32x4 a[kSkUnroll];
-    u32x4 xv[kSkUnroll];
-    u32x4 gv[kSkUnroll];
-    bool ok[kSkUnroll];
+  // batches of UNR steps; without gamma two register sets: the next batch is in flight while
+  // this one is used
+  struct Batch {
+    u32x4 a[UNR];
+    u32x4 xv[UNR][CPL];
+    u32x4 gv[UNR][CPL];
+    bool ok[UNR];
+    int cidx[UNR];
+  };
+  auto load_batch = [&](int s0, Batch& q) {
 #pragma unroll
-    for (int u = 0; u < kSkUnroll; ++u) {
+    for (int u = 0; u < UNR; ++u) {
       const int chunk = ((s0 + u) << 2) + g;
-      ok[u] = (s0 + u) < s_end && chunk < kc;
-      const int cc = ok[u] ? chunk : 0;
-      a[u] = make_a<T, WF>(rp, cc, srow, p.group_shift);
-      xv[u] = ld16(xrow + (cc << 3));
-      if constexpr (NORM) gv[u] = ld16(p.gamma + (cc << 3));
-    }
+      q.ok[u] = (s0 + u) < s_end && chunk < kcl;
+      const int cc = q.ok[u] ? chunk : 0;
+      q.cidx[u] = cc;
+      q.a[u] = ld16_stream((const char*)rp + ((long)cc << 4));
 #pragma unroll
-    for (int u = 0; u < kSkUnroll; ++u) {
-      u32x4 b = {0u, 0u, 0u, 0u};
-      if (ok[u] && tok_ok) {
-        if constexpr (NORM) {
-          float xf[8], gf[8], o[8];
-          unpack8<T>(xv[u], xf);
-          unpack8<T>(gv[u], gf);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            ss = fmaf(xf[i], xf[i], ss);
-            o[i] = xf[i] * gf[i];
-          }
-          b = pack8<T>(o);
-        } else {
-          b = xv[u];
-        }
+      for (int c = 0; c < CPL; ++c) {
+        q.xv[u][c] = ld16(xrow + ((cc * CPL + c) << 3));
+        if constexpr (NORM) q.gv[u][c] = ld16(p.gamma + ((cc * CPL + c) << 3));
       }
-      if (!ok[u]) a[u] = b;  // a clamped chunk must not contribute: b is zero there
-      acc = mfma16x16x32<T>(a[u], b, acc);
+    }
+  };
+  auto use_batch = [&](const Batch& q) {
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        u32x4 b = {0u, 0u, 0u, 0u};
+        if (q.ok[u] && tok_ok) b = make_b<T, NORM>(q.xv[u][c], q.gv[u][c], ss);
+        u32x4 av;
+        if constexpr (WF == WF_16BIT) {
+          av = q.a[u];
+        } else {
+          av = convert_a<T, WF>(c == 0 ? q.a[u].x : q.a[u].z, c == 0 ? q.a[u].y : q.a[u].w, srow,
+                                (q.cidx[u] * CPL + c) << 3, p.group_shift);
+        }
+        if (!q.ok[u]) av = b;  // a clamped chunk must not contribute: b is zero there
+        acc = mfma16x16x32<T>(av, b, acc);
+      }
+    }
+  };
+  if constexpr (NORM) {
+    // gamma doubles the registers of a batch: one set (measured faster than two here)
+    Batch qa;
+    for (int s0 = s_begin; s0 < s_end; s0 += UNR) {
+      load_batch(s0, qa);
+      use_batch(qa);
+    }
+  } else {
+    Batch qa, qb;
+    int s0 = s_begin;
+    if (s0 < s_end) load_batch(s0, qa);
+    while (s0 < s_end) {
+      const int s1 = s0 + UNR;
+      if (s1 < s_end) load_batch(s1, qb);
+      use_batch(qa);
+      if (s1 >= s_end) break;
+      s0 = s1 + UNR;
+      if (s0 < s_end) load_batch(s0, qa);
+      use_batch(qb);
     }
   }
 
@@ -193,16 +274,190 @@ __global__ void __launch_bounds__(kSkThreads) gemm_skinny_kernel(const SkinnyPar
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// B-stationary variant for K <= 4096: persistent workgroups, one per CU. Wave w always owns
+// the same K range, so its B operands (gamma * x of the 16 token columns) are built ONCE and
+// stay in registers while the workgroup walks over its weight tiles; the inner loop is weight
+// loads + MFMAs only, and the next tile's weights are requested before the current tile is
+// reduced (two register sets), so the HBM stream never drains between tiles. (Parking B in LDS
+// to afford a third weight register set was measured slower: 54 vs 46 us on the gate/up shape.)
+// ---------------------------------------------------------------------------------------
+constexpr int kBsSteps = 16;  // MFMA steps (32 k-values each) per wave: K <= 8 * 16 * 32
+
+template <typename T, int WF, bool NORM, int EPI, bool FULL>
+__global__ void __launch_bounds__(kSkThreads) gemm_skinny_bstat_kernel(const SkinnyParams p, int n_tiles) {
+  constexpr int CPL = (WF == WF_16BIT) ? 1 : 2;   // k-chunks (8 values) per 16-byte weight load
+  constexpr int LCH = kBsSteps / CPL;             // 16-byte weight loads per lane and tile
+  constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
+  constexpr int kWBytes = (WF == WF_16BIT) ? 2 : 1;
+  __shared__ float tile[2][kSkWaves][16][17];
+  __shared__ float ss_part[kSkWaves][kWave];
+
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int r16 = lane & 15;
+  const int g = lane >> 4;
+
+  // K is a multiple of 32 lane-chunks (launcher): every wave owns jmax consecutive steps, and
+  // 16-byte lane-chunk j of this lane is chunk lc0 + 4 * j of the row (a contiguous run per wave)
+  // FULL: K is exactly 8 waves x 16 steps (4096), no step is ever skipped
+  const int jmax = FULL ? LCH : ((p.k / (8 * CPL)) >> 5);
+  const int lc0 = ((wave * jmax) << 2) + g;
+
+  // ---- B operands, once ----
+  const bool tok_ok = r16 < p.tokens;
+  const uint16_t* xrow = p.x + (long)(tok_ok ? r16 : 0) * p.k;
+  u32x4 bq[LCH][CPL];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < LCH; ++j) {
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      u32x4 b = {0u, 0u, 0u, 0u};
+      if ((FULL || j < jmax) && tok_ok) {
+        const int e = ((lc0 + 4 * j) * CPL + c) << 3;
+        const u32x4 xv = ld16(xrow + e);
+        u32x4 gv = xv;
+        if constexpr (NORM) gv = ld16(p.gamma + e);
+        b = make_b<T, NORM>(xv, gv, ss);
+      }
+      bq[j][c] = b;
+    }
+  }
+  if constexpr (NORM) ss_part[wave][lane] = ss;
+
+  auto row_ptr = [&](int tile_idx, const uint16_t*& srow) -> const char* {
+    int out_row;
+    const void* wbase;
+    const uint16_t* sbase;
+    if constexpr (EPI == SK_GATEUP) {
+      out_row = tile_idx * 8 + (r16 >> 1);
+      wbase = (r16 & 1) ? p.w1 : p.w0;
+      sbase = (r16 & 1) ? p.s1 : p.s0;
+    } else {
+      out_row = tile_idx * 16 + r16;
+      wbase = p.w0;
+      sbase = p.s0;
+    }
+    const int row_c = out_row < p.n ? out_row : p.n - 1;
+    srow = (WF == WF_U8_GROUP) ? sbase + (long)row_c * p.s_pitch : nullptr;
+    return (const char*)wbase + (long)row_c * p.pitch * kWBytes;
+  };
+  auto issue = [&](int tile_idx, u32x4 (&a)[LCH], const uint16_t*& srow) {
+    const char* rp = row_ptr(tile_idx, srow) + (lc0 << 4);
+#pragma unroll
+    for (int j = 0; j < LCH; ++j)
+      if (FULL || j < jmax) a[j] = ld16_stream(rp + (j << 6));
+  };
+  auto consume = [&](int tile_idx, const u32x4 (&a)[LCH], const uint16_t* srow, int buf) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < LCH; ++j) {
+      if (FULL || j < jmax) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+          u32x4 av;
+          if constexpr (WF == WF_16BIT) {
+            av = a[j];
+          } else {
+            av = convert_a<T, WF>(c == 0 ? a[j].x : a[j].z, c == 0 ? a[j].y : a[j].w, srow,
+                                  ((lc0 + 4 * j) * CPL + c) << 3, p.group_shift);
+          }
+          acc = mfma16x16x32<T>(av, bq[j][c], acc);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) tile[buf][wave][4 * g + r][r16] = acc[r];
+  };
+  auto epilogue = [&](int tile_idx, int buf) {
+    if (t < OUT * 16) {
+      const int i = t >> 4;
+      const int j = t & 15;
+      const int n = tile_idx * OUT + i;
+      if (j < p.tokens && n < p.n) {
+        float rs = 1.f;
+        if constexpr (NORM) {
+          float tot = 0.f;
+#pragma unroll
+          for (int w = 0; w < kSkWaves; ++w)
+            tot += (ss_part[w][j] + ss_part[w][j + 16]) + (ss_part[w][j + 32] + ss_part[w][j + 48]);
+          rs = rsqrtf(tot / (float)p.k + p.eps);
+        }
+        auto total = [&](int row) {
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < kSkWaves; ++w) v += tile[buf][w][row][j];
+          return v;
+        };
+        float v;
+        if constexpr (EPI == SK_GATEUP) {
+          float gt = total(2 * i) * rs, up = total(2 * i + 1) * rs;
+          if constexpr (WF == WF_I8_CHANNEL) {
+            gt *= T::one(p.s0[(long)n * p.s_pitch]);
+            up *= T::one(p.s1[(long)n * p.s_pitch]);
+          }
+          v = silu_f32(gt) * up;
+        } else {
+          v = total(i) * rs;
+          if constexpr (WF == WF_I8_CHANNEL) v *= T::one(p.s0[(long)n * p.s_pitch]);
+          if (p.mul_bias) v *= T::one(p.mul_bias[n]);
+          if (p.add_bias) v += T::one(p.add_bias[n]);
+          if (p.residual) v += T::one(p.residual[(long)j * p.n + n]);
+        }
+        p.y[(long)j * p.n + n] = T::pack(v);
+      }
+    }
+  };
+
+  // ---- tiles blockIdx.x, blockIdx.x + gridDim.x, ...; two register sets ----
+  u32x4 a0[LCH], a1[LCH];
+  const uint16_t* sr0 = nullptr;
+  const uint16_t* sr1 = nullptr;
+  int tl = blockIdx.x;
+  if (tl < n_tiles) issue(tl, a0, sr0);
+  while (tl < n_tiles) {
+    const int t1 = tl + gridDim.x;
+    if (t1 < n_tiles) issue(t1, a1, sr1);
+    consume(tl, a0, sr0, 0);
+    __syncthreads();
+    epilogue(tl, 0);
+    if (t1 >= n_tiles) break;
+    const int t2 = t1 + gridDim.x;
+    if (t2 < n_tiles) issue(t2, a0, sr0);
+    consume(t1, a1, sr1, 1);
+    __syncthreads();
+    epilogue(t1, 1);
+    tl = t2;
+  }
+}
+
+static int g_skinny_bstat = 1;  // 0: always stream B (experiments)
+
 template <typename T, int WF, int EPI>
 static int launch_skinny_t(hipStream_t s, const SkinnyParams& p) {
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
-  const int grid = ceil_div(p.n, OUT);
+  const int n_tiles = ceil_div(p.n, OUT);
+  constexpr int kGran = 256 * ((WF == WF_16BIT) ? 1 : 2);  // K covered by one lane-chunk index
+  if (g_skinny_bstat && p.k <= kSkWaves * kBsSteps * 32 && p.k % kGran == 0) {
+    const int grid = balanced_grid(n_tiles, 1);
+    const bool full = p.k == kSkWaves * kBsSteps * 32;
+#define MUI_BSTAT(NORMV, FULLV) \
+  hipLaunchKernelGGL((gemm_skinny_bstat_kernel<T, WF, NORMV, EPI, FULLV>), dim3(grid), dim3(kSkThreads), 0, s, p, n_tiles)
+    if (p.gamma) { if (full) MUI_BSTAT(true, true); else MUI_BSTAT(true, false); }
+    else { if (full) MUI_BSTAT(false, true); else MUI_BSTAT(false, false); }
+#undef MUI_BSTAT
+    return launch_status();
+  }
   if (p.gamma)
-    hipLaunchKernelGGL((gemm_skinny_kernel<T, WF, true, EPI>), dim3(grid), dim3(kSkThreads), 0, s, p);
+    hipLaunchKernelGGL((gemm_skinny_kernel<T, WF, true, EPI>), dim3(n_tiles), dim3(kSkThreads), 0, s, p);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<T, WF, false, EPI>), dim3(grid), dim3(kSkThreads), 0, s, p);
+    hipLaunchKernelGGL((gemm_skinny_kernel<T, WF, false, EPI>), dim3(n_tiles), dim3(kSkThreads), 0, s, p);
   return launch_status();
 }
+
+void skinny_set_bstat(int on) { g_skinny_bstat = on; }
 
 // entry used by gemv.hip / int8.hip for tokens >= 2
 int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams& p) {

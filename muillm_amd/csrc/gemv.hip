@@ -256,9 +256,10 @@ using namespace mui;
 // token count from which the MFMA skinny-GEMM kernel takes over (below: one GEMV per token)
 static int g_skinny_min_tokens = 2;
 
-extern "C" int mui_tune_skinny(int min_tokens) {
+extern "C" int mui_tune_skinny(int min_tokens, int stream_b) {
   if (min_tokens < 1 || min_tokens > MUI_MAX_TOKENS + 1) return MUI_ERR_INVALID_ARG;
   g_skinny_min_tokens = min_tokens;
+  skinny_set_bstat(stream_b == 0);
   return MUI_OK;
 }
 

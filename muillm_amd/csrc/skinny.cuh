@@ -30,5 +30,7 @@ struct SkinnyParams {
 
 // launches gemm_skinny_kernel<dtype, weight format, epilogue>; returns a MUI_* status
 int launch_skinny(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
+// experiments: 0 disables the B-stationary persistent variant
+void skinny_set_bstat(int on);
 
 }  // namespace mui
