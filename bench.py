@@ -53,7 +53,7 @@ def _event_time_us(fn, iters, warm):
     return s.elapsed_time(e) * 1e3 / iters
 
 
-def bench_decode(lm, steps, warmup, prompt_len=32):
+def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=True):
     import torch
 
     from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
@@ -61,7 +61,7 @@ def bench_decode(lm, steps, warmup, prompt_len=32):
     dev = "cuda"
     g = torch.Generator().manual_seed(0)
     ids = torch.randint(0, lm.config.vocab_size, (1, prompt_len), generator=g).to(dev)
-    dec = MuiGraphDecoder(lm, use_graph=True)
+    dec = MuiGraphDecoder(lm, use_graph=use_graph)
     dec.prefill(ids, steps + warmup + 1)
     dec.decode(warmup)  # captures the graph on first use, then W untimed replays
     torch.cuda.synchronize()
@@ -70,6 +70,32 @@ def bench_decode(lm, steps, warmup, prompt_len=32):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     return dt, dec
+
+
+def bench_int8_variant(config, steps, warmup):
+    """The same decode benchmark with the decoder layers quantised to int8 (symmetric per output
+    channel; lm_head stays 16-bit, as the reference's module-name filter would leave it)."""
+    import torch
+
+    from muillm_amd.engine import init_engine
+    from muillm_amd.engineconfig import MuiEngineConfig
+    from muillm_amd.modules.models.llama.model import MuiLlamaForCausalLM
+    from muillm_amd.quantization.quantizationmethod import Int8WeightOnlyQuantizationMethod
+
+    qm = Int8WeightOnlyQuantizationMethod(group_size=0, modules=["qkv_proj", "o_proj", "mlp"])
+    base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0,
+                                           finalize=False)
+    lm8 = init_engine(base, device="cuda", engine_config=MuiEngineConfig(qm))
+    torch.cuda.synchronize()
+    dt, dec = bench_decode(lm8, steps, warmup)
+    hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
+    hq, hkv, d = config.num_attention_heads, config.num_key_value_heads, hid // config.num_attention_heads
+    wbytes = config.num_hidden_layers * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter) + 2 * v * hid
+    del dec, lm8, base
+    torch.cuda.empty_cache()
+    return {"tokens_per_s": round(steps / dt, 2), "ms_per_step": round(dt / steps * 1e3, 4),
+            "weight_bytes_per_token": wbytes, "hbm_floor_ms": round(wbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4),
+            "format": "int8 per output channel + fp16 scale; lm_head fp16"}
 
 
 def gateup_roofline(lm):
@@ -322,6 +348,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="decoder depth (32 = the Llama-3-8B shape; fewer is NOT the benchmark)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
+    ap.add_argument("--no-variants", action="store_true", help="skip the eager (no HIP graph) and int8 decode runs")
     ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS,DIRECT",
                     help="experiment: mui_tune_attention(waves per workgroup, min tokens per split, "
                          "longest unsplit sequence; -1 disables the head-parallel unsplit mode)")
@@ -384,6 +411,13 @@ def main():
     if not args.no_kernel_table:
         result["kernels"] = kernel_table(lm)
     del dec
+    if not args.no_variants:
+        dt_e, dec_e = bench_decode(lm, min(args.steps, 64), min(args.warmup, 8), use_graph=False)
+        result["variants"] = {"fp16_eager_no_graph_tokens_per_s": round(min(args.steps, 64) / dt_e, 2)}
+        del dec_e
+        del lm
+        torch.cuda.empty_cache()
+        result["variants"]["int8"] = bench_int8_variant(config, args.steps, args.warmup)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(config)
         result["cpu_baseline"]["gpu_over_cpu"] = round(tokens_per_s / result["cpu_baseline"]["value"], 1)
