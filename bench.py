@@ -349,9 +349,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
     ap.add_argument("--no-variants", action="store_true", help="skip the eager (no HIP graph) and int8 decode runs")
-    ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS,DIRECT",
+    ap.add_argument("--tune-attention", default=None, metavar="WAVES,MIN_TOKENS,DIRECT,MFMA",
                     help="experiment: mui_tune_attention(waves per workgroup, min tokens per split, "
-                         "longest unsplit sequence; -1 disables the head-parallel unsplit mode)")
+                         "longest unsplit sequence (-1 disables the head-parallel unsplit mode), shortest sequence for "
+                         "the matrix-core kernel (-1 disables it))")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
     args = ap.parse_args()
@@ -372,8 +373,8 @@ def main():
     if args.tune_attention:
         from muillm_amd import _lib
 
-        w, mt, dt = (int(v) for v in args.tune_attention.split(","))
-        _lib.check(_lib.load().mui_tune_attention(w, mt, dt), "mui_tune_attention")
+        w, mt, dt, mf = (int(v) for v in args.tune_attention.split(","))
+        _lib.check(_lib.load().mui_tune_attention(w, mt, dt, mf), "mui_tune_attention")
     config = MuiDecoderConfig.llama3_8b(num_hidden_layers=args.layers, max_position_embeddings=8192)
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
     torch.cuda.synchronize()

@@ -211,7 +211,8 @@ size_t mui_flash_decode_scratch_bytes(int batch, int n_q_heads, int head_dim, in
  * [batch, n_q_heads * head_dim]. mask (optional, 16-bit, [batch, >= seq_len] rows
  * mask_batch_stride apart): 0 keeps key s, any other value drops it
  * (csrc/attention/flash_decoding_fp16_kernels.cu:386-393); a fully masked row yields 0.
- * scratch: mui_flash_decode_scratch_bytes() bytes, may be NULL when n_splits == 1. */
+ * scratch: mui_flash_decode_scratch_bytes() bytes, may be NULL when n_splits == 1.
+ * n_splits <= 256. */
 int mui_flash_decode(mui_stream_t stream, int dtype, const void* q, const void* k_cache,
                      const void* v_cache, long cache_batch_stride, long cache_head_stride,
                      long cache_token_stride, const void* mask, long mask_batch_stride, int seq_len,
@@ -273,8 +274,11 @@ int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the
  * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1024;
- * negative: never use the unsplit one-workgroup-per-query-head mode) */
-int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens);
+ * negative: never use the unsplit one-workgroup-per-query-head mode), and the shortest
+ * sequence (or cache capacity, when the length is read on the device) that takes the
+ * matrix-core kernel (default 0 = never: the vector kernel measured faster on MI355X) */
+int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
+                       int mfma_tokens);
 /* fewest tokens that take the MFMA skinny-GEMM kernel instead of one GEMV per token (default 2;
  * MUI_MAX_TOKENS + 1 disables it); stream_b != 0 forces the variant that re-reads the token
  * operands per weight tile instead of keeping them in registers (K <= 4096 only) */

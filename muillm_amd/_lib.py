@@ -59,7 +59,7 @@ _SIGNATURES = {
                                   _P, c_long, c_long, c_long, _P, _P, c_int, _P, c_long, _P, _P, _P, _P,
                                   c_long, c_long, c_long, c_int, c_int, c_int, c_int, c_int, c_int]),
     "mui_flash_decode_splits": (c_int, [c_int, c_int, c_int, c_int]),
-    "mui_tune_attention": (c_int, [c_int, c_int, c_int]),
+    "mui_tune_attention": (c_int, [c_int, c_int, c_int, c_int]),
     "mui_flash_decode_scratch_bytes": (ctypes.c_size_t, [c_int, c_int, c_int, c_int]),
     "mui_flash_decode": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, _P, c_long, c_int, _P,
                                  c_int, _P, c_int, c_int, c_int, c_int, c_int]),

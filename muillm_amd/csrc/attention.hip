@@ -142,7 +142,7 @@ template <typename T, int G, int U, int NW, bool DIRECT>
 __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParams p) {
   constexpr int kAttnThreads = NW * kWave;
   constexpr int kWorkers = NW * 4;      // DPP rows per workgroup
-  constexpr bool kPipe = (NW <= 4);     // few waves: double-buffer K/V in registers instead
+  constexpr bool kPipe = (NW <= 8);     // <= 2 waves per SIMD: double-buffer K/V in registers
   __shared__ __attribute__((aligned(16))) uint16_t q_lds[G][kHeadDim];
   __shared__ __attribute__((aligned(16))) uint16_t kn_lds[kHeadDim];
   __shared__ __attribute__((aligned(16))) uint16_t vn_lds[kHeadDim];
@@ -189,8 +189,8 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
       const int tok = base + u * kWorkers + wk;
       valid[u] = (tok < t_end) && (tok != slot);
       const int tk = valid[u] ? tok : t_begin;  // t_begin < S: always a readable row
-      kreg[u] = ld16(kc + (long)tk * p.c_ts);
-      vreg[u] = ld16(vc + (long)tk * p.c_ts);
+      kreg[u] = ld16_stream(kc + (long)tk * p.c_ts);
+      vreg[u] = ld16_stream(vc + (long)tk * p.c_ts);
       if (mrow != nullptr && valid[u]) {
         if (T::one(mrow[tok]) != 0.f) valid[u] = false;
       }
@@ -198,9 +198,20 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   };
   u32x4 ka[U], va[U], kb[U], vb[U];
   bool valid_a[U], valid_b[U];
-  int base = t_begin;
-  bool have_a = base < t_end;
-  if (have_a) load_block(base, ka, va, valid_a);
+  // The workgroups of a launch start at addresses that are large powers of two apart and
+  // advance at the same speed, so they would all hit the same memory channels at the same
+  // time; softmax does not care about order, so each workgroup starts at its own block and
+  // wraps around.
+  const int n_blocks = t_end > t_begin ? (t_end - t_begin + kBlock - 1) / kBlock : 0;
+  const int rot = n_blocks > 0 ? (int)((blockIdx.x * 7u + blockIdx.y * 13u + blockIdx.z * 29u) % (unsigned)n_blocks) : 0;
+  auto block_base = [&](int bi) {
+    int blk = bi + rot;
+    blk = blk >= n_blocks ? blk - n_blocks : blk;
+    return t_begin + blk * kBlock;
+  };
+  int bi = 0;
+  bool have_a = n_blocks > 0;
+  if (have_a) load_block(block_base(0), ka, va, valid_a);
 
   // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once) ----
   for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
@@ -252,14 +263,13 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
       // two register sets: the next block is in flight while the current one is consumed
       for (;;) {
         if (!have_a) break;
-        const int nb = base + kBlock;
-        const bool have_b = nb < t_end;
-        if (have_b) load_block(nb, kb, vb, valid_b);
+        const bool have_b = bi + 1 < n_blocks;
+        if (have_b) load_block(block_base(bi + 1), kb, vb, valid_b);
         attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
         if (!have_b) break;
-        base = nb + kBlock;
-        have_a = base < t_end;
-        if (have_a) load_block(base, ka, va, valid_a);
+        bi += 2;
+        have_a = bi < n_blocks;
+        if (have_a) load_block(block_base(bi), ka, va, valid_a);
         attend_block<T, G, U>(kb, vb, valid_b, madd, qreg, p.scale_log2, m, l, acc);
       }
     } else {
@@ -267,9 +277,9 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
       // under 128 VGPRs
       while (have_a) {
         attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
-        base += kBlock;
-        have_a = base < t_end;
-        if (have_a) load_block(base, ka, va, valid_a);
+        ++bi;
+        have_a = bi < n_blocks;
+        if (have_a) load_block(block_base(bi), ka, va, valid_a);
       }
     }
   }
@@ -351,22 +361,320 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   }
 }
 
-// log-sum-exp merge of the per-split partials: one workgroup of 128 threads per (head, batch)
+// ---------------------------------------------------------------------------------------
+// Matrix-core formulation for long sequences. Same grid and merge as above with G = Hq/Hkv,
+// but a wave now owns blocks of 32 consecutive tokens:
+//   scores   S^T[token, head] = K[token, :] . q[head, :]   two v_mfma_f32_16x16x32 chains over
+//            D = 128 (A = K rows loaded straight from the cache in operand layout: lane
+//            (g = lane / 16, i = lane % 16) holds 16-byte chunk g + 4j of token i; B = rotated
+//            q of head i from LDS, zero for i >= G). C puts head i's scores of tokens 4g + r
+//            (r < 4) in lane (g, i): softmax needs one running max per lane column, shared by
+//            the four lane groups with two shuffles.
+//   output   O^T[d, head] += V^T[d, token] . P[token, head]   8 MFMAs (16 values of d each),
+//            contraction over the block's 32 tokens. P comes straight from the score
+//            registers (k-slots of lane group g = tokens 4g + r and 16 + 4g + r). V is loaded
+//            with the natural coalesced mapping, parked in a wave-private LDS tile and read
+//            back TRANSPOSED with ds_read_b64_tr_b16: within a 16-lane group, lane i receives
+//            element i % 4 of the 8-byte rows addressed by lanes i/4, i/4 + 4, i/4 + 8,
+//            i/4 + 12, i.e. four tokens of one d when those lanes point at token rows
+//            4g .. 4g + 3 at column 16 * block + 4 * (lane % 4).
+// About 100 instructions per 16 KiB of K/V per wave instead of about 600 on the vector ALUs.
+// ---------------------------------------------------------------------------------------
+typedef _Float16 af16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 abf16x8 __attribute__((ext_vector_type(8)));
+typedef short ai16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+__device__ __forceinline__ f32x4 attn_mfma(u32x4 a, u32x4 b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 attn_mfma<F16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(af16x8, a), __builtin_bit_cast(af16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 attn_mfma<BF16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(abf16x8, a), __builtin_bit_cast(abf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_ptr) {
+  typedef ai16x4 __attribute__((address_space(3))) * lds_v4;
+  const ai16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4)lds_ptr);
+  return __builtin_bit_cast(u32x2, r);
+}
+
+constexpr int kMfTok = 32;        // tokens per wave block
+constexpr int kMfVStride = 144;   // 16-bit elements per V tile row: 288 bytes keep the transposed reads spread over the banks
+
+template <typename T, int G, int NW, bool DIRECT>
+__global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const AttnParams p) {
+  constexpr int kAttnThreads = NW * kWave;
+  constexpr int kBlock = NW * kMfTok;  // tokens per workgroup pass
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[16][kHeadDim];
+  __shared__ __attribute__((aligned(16))) uint16_t kn_lds[kHeadDim];
+  __shared__ __attribute__((aligned(16))) uint16_t vn_lds[kHeadDim];
+  __shared__ float lds_m[NW][G];
+  __shared__ float lds_l[NW][G];
+  // the V tiles during the sweep, the cross-wave merge buffer afterwards
+  constexpr int kVBytes = NW * kMfTok * kMfVStride * 2;
+  constexpr int kMergeBytes = NW * G * kHeadDim * 4;
+  __shared__ __attribute__((aligned(16))) char big_lds[kVBytes > kMergeBytes ? kVBytes : kMergeBytes];
+  uint16_t (*v_lds)[kMfVStride] = (uint16_t (*)[kMfVStride])(big_lds + (size_t)(threadIdx.x >> 6) * kMfTok * kMfVStride * 2);
+  float (*tile)[G][kHeadDim] = (float (*)[G][kHeadDim])big_lds;
+
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int head0 = kvh * G;
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int g = lane >> 4;
+  const int i = lane & 15;
+
+  const bool has_new = p.k_new != nullptr;
+  const int slot = has_new ? (int)p.cache_position[0] : -1;
+  int S = p.seq_len >= 0 ? p.seq_len : slot + 1;
+  S = S < p.max_t ? S : p.max_t;
+  const long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+
+  int chunk = (S + p.n_splits - 1) / p.n_splits;
+  chunk = ((chunk + kBlock - 1) / kBlock) * kBlock;
+  const int t_begin = split * chunk;
+  const int t_end = (t_begin + chunk) < S ? (t_begin + chunk) : S;
+  const bool owner = has_new && slot >= t_begin && slot < t_begin + chunk && slot < S;
+
+  const float* cos_row = p.cos ? p.cos + pos * p.rope_stride : nullptr;
+  const float* sin_row = p.sin ? p.sin + pos * p.rope_stride : nullptr;
+
+  const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
+  const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
+  const uint16_t* mrow = p.mask ? p.mask + (long)b * p.mask_bs : nullptr;
+  const int safe_row = t_begin < S ? t_begin : 0;  // a readable row for out-of-range lanes
+
+  struct Block {
+    u32x4 k[2][4];  // [token half][d step]: token base + 16 * half + i, chunk g + 4 * step
+    u32x4 v[8];     // token base + 4 * u + g, chunk i
+  };
+  auto load_block = [&](int base, Block& q) {
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int tok = base + 16 * h2 + i;
+      const uint16_t* rp = kc + (long)(tok < t_end ? tok : safe_row) * p.c_ts + g * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q.k[h2][j] = ld16(rp + j * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int tok = base + 4 * u + g;
+      q.v[u] = ld16(vc + (long)(tok < t_end ? tok : safe_row) * p.c_ts + i * 8);
+    }
+  };
+
+  Block ba, bb;
+  int base = t_begin + wave * kMfTok;
+  bool have_a = base < t_end;
+  if (have_a) load_block(base, ba);
+
+  // ---- rotate the G query heads into LDS (rows >= G stay zero: the padded MFMA columns) ----
+  for (int e = t; e < 16 * kHeadDim; e += kAttnThreads) {
+    const int hh = e / kHeadDim, d = e % kHeadDim;
+    uint16_t r = 0;
+    if (hh < G) {
+      const int head = head0 + hh;
+      const uint16_t* qp = p.q + (long)b * p.q_bs + (long)head * p.q_hs;
+      r = T::pack(rope_elem<T>(qp, d, cos_row, sin_row));
+      if (p.q_out && split == 0) p.q_out[((long)b * p.hq + head) * kHeadDim + d] = r;
+    }
+    q_lds[hh][d] = r;
+  }
+  if (owner) {
+    const long coff = (long)b * p.c_bs + (long)kvh * p.c_hs + (long)slot * p.c_ts;
+    if (t < kHeadDim) {
+      const uint16_t* kp = p.k_new + (long)b * p.k_bs + (long)kvh * p.k_hs;
+      const uint16_t r = T::pack(rope_elem<T>(kp, t, cos_row, sin_row));
+      kn_lds[t] = r;
+      p.k_cache[coff + t] = r;
+    } else if (t < 2 * kHeadDim) {
+      const int d = t - kHeadDim;
+      const uint16_t v = p.v_new[(long)b * p.v_bs + (long)kvh * p.v_hs + d];
+      vn_lds[d] = v;
+      p.v_cache[coff + d] = v;
+    }
+  }
+  __syncthreads();
+
+  u32x4 qreg[4];  // B operand of the score MFMAs: head i, chunk g + 4j
+#pragma unroll
+  for (int j = 0; j < 4; ++j) qreg[j] = *(const u32x4*)&q_lds[i][(g + 4 * j) * 8];
+
+  float m = -INFINITY, l = 0.f;  // of head i (replicated over the lane groups; l is a partial sum)
+  f32x4 acc[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto attend = [&](int base, Block& q) {
+    // the new token's row comes from LDS, never from the cache slot written above
+    if (owner && slot >= base && slot < base + kMfTok) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2)
+        if (base + 16 * h2 + i == slot) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) q.k[h2][j] = *(const u32x4*)&kn_lds[(g + 4 * j) * 8];
+        }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (base + 4 * u + g == slot) q.v[u] = *(const u32x4*)&vn_lds[i * 8];
+    }
+    // park V (natural layout) in this wave's tile
+#pragma unroll
+    for (int u = 0; u < 8; ++u) *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
+
+    f32x4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      s1 = attn_mfma<T>(q.k[0][j], qreg[j], s1);
+      s2 = attn_mfma<T>(q.k[1][j], qreg[j], s2);
+    }
+    float sc[8];
+    float m_loc = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
+      bool ok = tok < t_end;
+      if (mrow != nullptr && ok) ok = T::one(mrow[tok]) == 0.f;
+      const float raw = r < 4 ? s1[r] : s2[r - 4];
+      sc[r] = ok ? raw * p.scale_log2 : -INFINITY;
+      m_loc = fmaxf(m_loc, sc[r]);
+    }
+    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
+    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+    const float m_new = fmaxf(m, m_loc);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = fast_exp2(m - m_use);
+    float pr[8];
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      pr[r] = fast_exp2(sc[r] - m_use);
+      psum += pr[r];
+    }
+    l = fmaf(l, corr, psum);
+    m = m_new;
+    u32x4 pb;  // B operand: k-slots 8g .. 8g+7 = tokens 4g+r, 16+4g+r
+    pb.x = (uint32_t)T::pack(pr[0]) | ((uint32_t)T::pack(pr[1]) << 16);
+    pb.y = (uint32_t)T::pack(pr[2]) | ((uint32_t)T::pack(pr[3]) << 16);
+    pb.z = (uint32_t)T::pack(pr[4]) | ((uint32_t)T::pack(pr[5]) << 16);
+    pb.w = (uint32_t)T::pack(pr[6]) | ((uint32_t)T::pack(pr[7]) << 16);
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const u32x2 lo = lds_read_tr16(&v_lds[4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x2 hi = lds_read_tr16(&v_lds[16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+      f32x4 a = acc[db];
+      a.x *= corr; a.y *= corr; a.z *= corr; a.w *= corr;
+      acc[db] = attn_mfma<T>(va, pb, a);
+    }
+  };
+
+  for (;;) {
+    if (!have_a) break;
+    const int nb = base + kBlock;
+    const bool have_b = nb < t_end;
+    if (have_b) load_block(nb, bb);
+    attend(base, ba);
+    if (!have_b) break;
+    base = nb + kBlock;
+    have_a = base < t_end;
+    if (have_a) load_block(base, ba);
+    attend(nb, bb);
+  }
+
+  // ---- the wave's totals: l summed over the four lane groups (m is already shared) ----
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+
+  // ---- merge the NW waves through LDS (the V tiles are dead: every wave has finished) ----
+  __syncthreads();
+  if (g == 0 && i < G) lds_m[wave][i] = m;
+  __syncthreads();
+  float mx = -INFINITY;
+  if (i < G) {
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) mx = fmaxf(mx, lds_m[w2][i]);
+  }
+  const float f = fast_exp2(m - ((mx == -INFINITY) ? 0.f : mx));
+  if (i < G) {
+    if (g == 0) lds_l[wave][i] = l * f;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      // C layout: lane (g, i) holds O^T[d = 16 db + 4 g + r][head i]
+      f32x4 o = acc[db];
+      o.x *= f; o.y *= f; o.z *= f; o.w *= f;
+      *(f32x4*)&tile[wave][i][16 * db + 4 * g] = o;
+    }
+  }
+  __syncthreads();
+
+  for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
+    const int hh = e / kHeadDim, d = e % kHeadDim;
+    const int head = head0 + hh;
+    float a = 0.f, lsum = 0.f, mxx = lds_m[0][hh];
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) {
+      a += tile[w2][hh][d];
+      lsum += lds_l[w2][hh];
+      mxx = fmaxf(mxx, lds_m[w2][hh]);
+    }
+    if constexpr (DIRECT) {
+      p.out[((long)b * p.hq + head) * kHeadDim + d] = T::pack(lsum > 0.f ? a / lsum : 0.f);
+    } else {
+      const long pi = ((long)b * p.hq + head) * p.n_splits + split;
+      p.part_acc[pi * kHeadDim + d] = a;
+      if (d == 0) {
+        p.part_ml[pi * 2 + 0] = mxx;
+        p.part_ml[pi * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// log-sum-exp merge of the per-split partials: one workgroup of 128 threads per (head, batch).
+// The split weights are computed once into LDS; the accumulation loop then has no dependent
+// loads, so the partial rows of all splits are in flight together.
+constexpr int kMaxSplits = 256;
 template <typename T>
 __global__ void __launch_bounds__(kHeadDim) attn_combine_kernel(const float* part_acc,
                                                                 const float* part_ml,
                                                                 uint16_t* out, int hq, int n_splits) {
+  __shared__ float w_lds[kMaxSplits];
+  __shared__ float red[2][2];
   const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const long base = ((long)b * hq + head) * n_splits;
   float mx = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+  for (int s = d; s < n_splits; s += kHeadDim) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+  mx = wave_max(mx);
+  if ((d & (kWave - 1)) == 0) red[0][d >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(red[0][0], red[0][1]);
   const float m_use = (mx == -INFINITY) ? 0.f : mx;
-  float a = 0.f, lsum = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
+  float lpart = 0.f;
+  for (int s = d; s < n_splits; s += kHeadDim) {
     const float w = fast_exp2(part_ml[(base + s) * 2] - m_use);
-    lsum = fmaf(w, part_ml[(base + s) * 2 + 1], lsum);
-    a = fmaf(w, part_acc[(base + s) * kHeadDim + d], a);
+    w_lds[s] = w;
+    lpart = fmaf(w, part_ml[(base + s) * 2 + 1], lpart);
   }
+  lpart = wave_sum(lpart);
+  if ((d & (kWave - 1)) == 0) red[1][d >> 6] = lpart;
+  __syncthreads();
+  const float lsum = red[1][0] + red[1][1];
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  const float* pa = part_acc + base * kHeadDim + d;
+  int s = 0;
+  for (; s + 4 <= n_splits; s += 4) {
+    a0 = fmaf(w_lds[s + 0], pa[(long)(s + 0) * kHeadDim], a0);
+    a1 = fmaf(w_lds[s + 1], pa[(long)(s + 1) * kHeadDim], a1);
+    a2 = fmaf(w_lds[s + 2], pa[(long)(s + 2) * kHeadDim], a2);
+    a3 = fmaf(w_lds[s + 3], pa[(long)(s + 3) * kHeadDim], a3);
+  }
+  for (; s < n_splits; ++s) a0 = fmaf(w_lds[s], pa[(long)s * kHeadDim], a0);
+  const float a = (a0 + a1) + (a2 + a3);
   out[((long)b * hq + head) * kHeadDim + d] = T::pack(lsum > 0.f ? a / lsum : 0.f);
 }
 
@@ -428,6 +736,17 @@ constexpr int unroll_for(int nw) { return nw == 16 ? 2 : 4; }
 static int g_attn_waves = 0;  // 0: built-in choice; 4, 8 or 16 forces the workgroup size
 static int g_attn_head_parallel = 1;  // unsplit decodes at small batch: workgroup per query head
 static int g_attn_direct_tokens = 0;  // 0: built-in choice; longest sequence decoded unsplit
+// Shortest sequence that takes the matrix-core kernel; <= 0: never (the built-in choice: on
+// MI355X it measured 250 us against 176 us for the vector kernel at 32k context, batch 8 --
+// its per-block dependency chain (loads, LDS round trip, two MFMA chains, shuffles) is longer
+// than two waves per SIMD can hide -- so it stays an option for experiments).
+static int g_attn_mfma_tokens = 0;
+
+static inline bool attn_use_mfma(const AttnParams& p) {
+  if (g_attn_mfma_tokens <= 0) return false;
+  const int hint = p.seq_len > 0 ? p.seq_len : p.max_t;
+  return hint >= g_attn_mfma_tokens;
+}
 
 // waves per workgroup for a given number of query heads per KV head
 static inline int attn_waves_for(int g) {
@@ -447,7 +766,12 @@ template <typename T, int G>
 static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
   dim3 grid(p.n_splits, p.hq / G, batch);
   const int nw = attn_waves_for(G);
-  if constexpr (G <= 4) {
+  if (G == p.hq / p.hkv && attn_use_mfma(p)) {
+    if (p.n_splits == 1)
+      hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, true>), grid, dim3(8 * kWave), 0, s, p);
+    else
+      hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, false>), grid, dim3(8 * kWave), 0, s, p);
+  } else if constexpr (G <= 4) {
     if (nw == 16) launch_attn_nw<T, G, 16>(s, p, grid);
     else if (nw == 8) launch_attn_nw<T, G, 8>(s, p, grid);
     else launch_attn_nw<T, G, 4>(s, p, grid);
@@ -467,7 +791,7 @@ static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
 template <typename T>
 static int launch_attn_t(hipStream_t s, const AttnParams& p, int batch) {
   // unsplit and too few KV heads to occupy the GPU: one workgroup per query head
-  if (p.n_splits == 1 && g_attn_head_parallel && batch * p.hkv * 4 <= device_cus())
+  if (p.n_splits == 1 && g_attn_head_parallel && batch * p.hkv * 8 <= device_cus() && !attn_use_mfma(p))
     return launch_attn_g<T, 1>(s, p, batch);
   switch (p.hq / p.hkv) {
     case 1: return launch_attn_g<T, 1>(s, p, batch);
@@ -490,7 +814,8 @@ using namespace mui;
 
 static int g_attn_min_tokens = 0;  // 0: built-in choice; else fewest tokens worth a split
 
-extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens) {
+extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
+                                  int mfma_tokens) {
   if (!(waves_per_workgroup == 0 || waves_per_workgroup == 4 || waves_per_workgroup == 8 || waves_per_workgroup == 16))
     return MUI_ERR_INVALID_ARG;
   if (min_tokens_per_split < 0) return MUI_ERR_INVALID_ARG;
@@ -498,6 +823,7 @@ extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_sp
   g_attn_min_tokens = min_tokens_per_split;
   g_attn_head_parallel = direct_tokens >= 0;
   g_attn_direct_tokens = direct_tokens > 0 ? direct_tokens : 0;
+  g_attn_mfma_tokens = mfma_tokens;
   return MUI_OK;
 }
 
@@ -508,14 +834,14 @@ extern "C" int mui_flash_decode_splits(int batch, int n_q_heads, int n_kv_heads,
   // Splitting buys parallelism but every split beyond the first costs the combine launch
   // (~4 us) and partial traffic, so a split must carry a few passes of work. (Merging the
   // splits inside the kernel with a device-scope fence + counter was measured slower than
-  // the combine launch on MI355X.) The total is capped near 1.5 workgroups per CU: measured
-  // best at 32 splits for batch 1 and 4-8 splits for batch 8 with 8 KV heads.
+  // the combine launch on MI355X.) The total is one workgroup per CU: measured best at 32
+  // splits for batch 1 and 4 splits for batch 8 with 8 KV heads.
   // Short sequences at small batch: one unsplit workgroup per query head beats split + merge.
   const int direct = g_attn_direct_tokens > 0 ? g_attn_direct_tokens : 1024;
-  if (g_attn_head_parallel && seq_len_hint <= direct && batch * n_kv_heads * 4 <= device_cus()) return 1;
+  if (g_attn_head_parallel && seq_len_hint <= direct && batch * n_kv_heads * 8 <= device_cus()) return 1;
   const int min_tokens = g_attn_min_tokens > 0 ? g_attn_min_tokens : 2 * kBlock;
   const int max_useful = ceil_div(seq_len_hint, min_tokens);
-  int want = ceil_div(3 * device_cus() / 2, batch * n_kv_heads);
+  int want = device_cus() / (batch * n_kv_heads);  // one workgroup per CU, never a ragged second round
   if (want > 32) want = 32;
   int n = want < max_useful ? want : max_useful;
   if (n < 1) n = 1;
@@ -531,6 +857,7 @@ static int check_attn_shape(int dtype, int batch, int hq, int hkv, int head_dim,
                             int max_t) {
   if (!(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16)) return MUI_ERR_INVALID_ARG;
   if (batch <= 0 || hq <= 0 || hkv <= 0 || n_splits <= 0 || max_t <= 0) return MUI_ERR_INVALID_ARG;
+  if (n_splits > kMaxSplits) return MUI_ERR_UNSUPPORTED;
   if (head_dim != kHeadDim) return MUI_ERR_UNSUPPORTED;
   if (hq % hkv != 0) return MUI_ERR_INVALID_ARG;
   const int g = hq / hkv;

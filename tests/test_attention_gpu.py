@@ -20,6 +20,17 @@ D = 128
 ATOL = 2e-3
 
 
+@pytest.fixture(params=["auto", "matrix-core"], autouse=True)
+def attention_kernel_choice(request):
+    """Every test runs twice: with the built-in kernel choice, and with the matrix-core decode
+    kernel forced for every sequence length (it is otherwise reserved for long sequences)."""
+    lib = _lib.load()
+    if request.param == "matrix-core":
+        _lib.check(lib.mui_tune_attention(0, 0, 0, 1), "mui_tune_attention")
+    yield request.param
+    _lib.check(lib.mui_tune_attention(0, 0, 0, 0), "mui_tune_attention")
+
+
 def _gen(seed=0):
     g = torch.Generator(device="cpu")
     g.manual_seed(seed)
