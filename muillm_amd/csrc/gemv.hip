@@ -41,8 +41,16 @@ struct GemvParams {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 
+// The arguments are scalars, the ones every wave needs first in front: the first 16 dwords
+// of the kernel-argument segment are preloaded into SGPRs at wave launch (build flag
+// -amdgpu-kernarg-preload-count), so the first weight loads do not wait for a scalar load.
 template <typename T, int R, int CH, bool NORM, int EPI>
-__global__ void __launch_bounds__(kThreads) gemv_kernel(const GemvParams p) {
+__global__ void __launch_bounds__(kThreads) gemv_kernel(const uint16_t* a_w0, const uint16_t* a_w1, long a_pitch,
+                                                        const uint16_t* a_x, const uint16_t* a_gamma,
+                                                        uint16_t* a_y, int a_n, int a_k, float a_eps,
+                                                        const uint16_t* a_residual, const uint16_t* a_mul_bias,
+                                                        const uint16_t* a_add_bias) {
+  const GemvParams p = {a_w0, a_w1, a_pitch, a_x, a_gamma, a_mul_bias, a_add_bias, a_residual, a_y, a_n, a_k, a_eps};
   constexpr int OUT = (EPI == EPI_GATEUP) ? R / 2 : R;  // outputs per row group
   static_assert(EPI != EPI_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
 
@@ -208,9 +216,11 @@ static Tuning g_tune;
 template <typename T, int R, int CH, int EPI>
 static int launch_rc(hipStream_t s, const GemvParams& p, int grid) {
   if (p.gamma)
-    hipLaunchKernelGGL((gemv_kernel<T, R, CH, true, EPI>), dim3(grid), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((gemv_kernel<T, R, CH, true, EPI>), dim3(grid), dim3(kThreads), 0, s, p.w0, p.w1, p.pitch, p.x,
+                       p.gamma, p.y, p.n, p.k, p.eps, p.residual, p.mul_bias, p.add_bias);
   else
-    hipLaunchKernelGGL((gemv_kernel<T, R, CH, false, EPI>), dim3(grid), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((gemv_kernel<T, R, CH, false, EPI>), dim3(grid), dim3(kThreads), 0, s, p.w0, p.w1, p.pitch, p.x,
+                       p.gamma, p.y, p.n, p.k, p.eps, p.residual, p.mul_bias, p.add_bias);
   return launch_status();
 }
 

@@ -59,7 +59,13 @@ __device__ __forceinline__ void unpack16_u8(const u32x4 w, uint32_t flip, float 
 }
 
 template <typename T, int R, int CH, bool NORM, int EPI, int FMT>
-__global__ void __launch_bounds__(kThreads8) int8_gemv_kernel(const Int8Params p) {
+__global__ void __launch_bounds__(kThreads8) int8_gemv_kernel(
+    // scalars, hottest first: the first 16 argument dwords are preloaded into SGPRs at wave launch
+    const uint8_t* a_w0, const uint8_t* a_w1, long a_pitch, const uint16_t* a_x, const uint16_t* a_gamma,
+    uint16_t* a_y, int a_n, int a_k, const uint16_t* a_s0, const uint16_t* a_s1, long a_s_pitch,
+    int a_group_shift, float a_eps, const uint16_t* a_add_bias, const uint16_t* a_residual) {
+  const Int8Params p = {a_w0, a_w1, a_pitch, a_s0, a_s1, a_s_pitch, a_group_shift, a_x, a_gamma,
+                        a_add_bias, a_residual, a_y, a_n, a_k, a_eps};
   constexpr int OUT = (EPI == EPI8_GATEUP) ? R / 2 : R;
   static_assert(EPI != EPI8_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
   constexpr uint32_t kFlip = (FMT == FMT_CHANNEL) ? 0x80808080u : 0u;
@@ -284,9 +290,13 @@ static int g_int8_rows = 0;
 template <typename T, int R, int CH, int EPI, int FMT>
 static int launch8_rc(hipStream_t s, const Int8Params& p, int grid) {
   if (p.gamma)
-    hipLaunchKernelGGL((int8_gemv_kernel<T, R, CH, true, EPI, FMT>), dim3(grid), dim3(kThreads8), 0, s, p);
+    hipLaunchKernelGGL((int8_gemv_kernel<T, R, CH, true, EPI, FMT>), dim3(grid), dim3(kThreads8), 0, s, p.w0, p.w1,
+                       p.pitch, p.x, p.gamma, p.y, p.n, p.k, p.s0, p.s1, p.s_pitch, p.group_shift, p.eps, p.add_bias,
+                       p.residual);
   else
-    hipLaunchKernelGGL((int8_gemv_kernel<T, R, CH, false, EPI, FMT>), dim3(grid), dim3(kThreads8), 0, s, p);
+    hipLaunchKernelGGL((int8_gemv_kernel<T, R, CH, false, EPI, FMT>), dim3(grid), dim3(kThreads8), 0, s, p.w0, p.w1,
+                       p.pitch, p.x, p.gamma, p.y, p.n, p.k, p.s0, p.s1, p.s_pitch, p.group_shift, p.eps, p.add_bias,
+                       p.residual);
   return launch_status();
 }
 
