@@ -264,6 +264,28 @@ int mui_greedy_advance(mui_stream_t stream, int dtype, const void* logits, long 
                        long tokens_stride, int max_steps, int64_t* unfinished,
                        const int64_t* eos_ids, int n_eos, long pad_token);
 
+/* Sampling twin of mui_greedy_advance: tok = argmax_v(logits[b, v] / temperature - log q_v) with
+ * q_v ~ Exp(1), which is the draw of the reference's sync-free multinomial
+ * argmax(softmax(logits / temperature) / q) (muillm/sampling/multinomial.py:4-6) without
+ * materialising the probabilities; -inf logits (top-k / top-p filters) never win. The variates
+ * come from Philox4x32-10 keyed by `seed` with counter (v / 4, b, step[b] mod 2^32, 0), lane
+ * v % 4 of the block: u = ((bits >> 8) + 1) * 2^-24, q = -log u. Token store, eos/pad rule and
+ * counters exactly as mui_greedy_advance; replaying a captured launch draws fresh noise because
+ * step[b] advances on the device. temperature > 0. */
+int mui_sample_advance(mui_stream_t stream, int dtype, const void* logits, long row_stride,
+                       int rows, int vocab, float temperature, uint64_t seed, int64_t* next_ids,
+                       int64_t* position_ids, int64_t* cache_position, int64_t* step,
+                       int64_t* tokens_out, long tokens_stride, int max_steps, int64_t* unfinished,
+                       const int64_t* eos_ids, int n_eos, long pad_token);
+
+/* muillm_embedding_module_forward (csrc/module.cpp:320; csrc/embedding/embedding.cu:31-100; kernels
+ * csrc/embedding/embedding_xx16_kernels.cu:26-112): out[t, :] = table[ids[t], :] for a 16-bit
+ * [vocab, dim] table with row pitch row_pitch elements; ids int64, or int32 when ids_are_int32.
+ * Ids outside [0, vocab) are clamped (the reference reads out of bounds). out is dense
+ * [n_tokens, dim]. */
+int mui_embedding(mui_stream_t stream, int dtype, const void* table, long row_pitch,
+                  const void* ids, int ids_are_int32, void* out, int n_tokens, int dim, int vocab);
+
 /* ------------------------------------------------------------------------------------
  * Launch-shape knobs used by the benchmark sweeps (0 restores the built-in choice). They
  * have no counterpart in the reference, whose launch shapes are compile-time constants

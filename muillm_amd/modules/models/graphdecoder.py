@@ -20,9 +20,16 @@ from ..kvcache.cache_utils import MuiStaticCache, _next_pow2, create_static_cach
 
 
 class MuiGraphDecoder:
-    def __init__(self, lm, use_graph: bool = True, eos_token_ids=None, pad_token_id: int = 0):
+    def __init__(self, lm, use_graph: bool = True, eos_token_ids=None, pad_token_id: int = 0,
+                 do_sample: bool = False, temperature: float = 1.0, seed: int = 0):
+        """do_sample=True draws from softmax(logits / temperature) on the device (the reference's
+        sync-free multinomial, muillm/sampling/multinomial.py:4-6) instead of taking the argmax;
+        the draws are a function of (seed, batch row, step), so a run is reproducible."""
         self.lm = lm
         self.use_graph = use_graph
+        self.do_sample = do_sample
+        self.temperature = float(temperature)
+        self.seed = int(seed)
         self.eos_token_ids = list(eos_token_ids) if eos_token_ids is not None else None
         self.pad_token_id = int(pad_token_id)
         self.graph = None
@@ -48,10 +55,20 @@ class MuiGraphDecoder:
         out = self.lm(input_ids=self.ids, position_ids=self.pos, cache_position=self.cpos,
                       past_key_values=self.cache, use_cache=True, all_ones_mask=True, float_logits=False)
         logits = out.logits[:, -1, :]
-        muillm_ext.mui_greedy_advance(logits, self.ids, self.step, self.out_tokens, position_ids=self.pos,
-                                      cache_position=self.cpos, unfinished=self.unfinished,
-                                      eos_token_ids=self.eos, pad_token_id=self.pad_token_id)
+        self._advance(logits)
         return logits
+
+    def _advance(self, logits):
+        """Token choice + stop check + token store + counters: one launch, all on the device."""
+        if self.do_sample:
+            muillm_ext.mui_sample_advance(logits, self.ids, self.step, self.out_tokens, temperature=self.temperature,
+                                          seed=self.seed, position_ids=self.pos, cache_position=self.cpos,
+                                          unfinished=self.unfinished, eos_token_ids=self.eos,
+                                          pad_token_id=self.pad_token_id)
+        else:
+            muillm_ext.mui_greedy_advance(logits, self.ids, self.step, self.out_tokens, position_ids=self.pos,
+                                          cache_position=self.cpos, unfinished=self.unfinished,
+                                          eos_token_ids=self.eos, pad_token_id=self.pad_token_id)
 
     def _capture(self):
         self.cache.device_length_mode = True
@@ -99,16 +116,14 @@ class MuiGraphDecoder:
         if self._batch != batch or getattr(self, "_max_new", 0) < max_new_tokens:
             self._alloc_state(batch, max_new_tokens, device)
             self.graph = None
-        first = muillm_ext.mui_argmax(out.logits[:, -1, :])
-        self.ids.copy_(first.unsqueeze(1))
-        self.pos.fill_(prompt_len)
-        self.cpos.fill_(prompt_len)
-        self.step.fill_(1)
+        # the first new token goes through the same kernel as all later ones: the counters start
+        # one step back and the launch advances them to (prompt_len, prompt_len, 1)
+        self.pos.fill_(prompt_len - 1)
+        self.cpos.fill_(prompt_len - 1)
+        self.step.zero_()
         self.out_tokens.zero_()
-        self.out_tokens[:, 0] = first
         self.unfinished.fill_(1)
-        if self.eos is not None:
-            self.unfinished.copy_((first.unsqueeze(1) != self.eos.unsqueeze(0)).all(dim=1).to(torch.int64))
+        self._advance(out.logits[:, -1, :])
         return out.logits[:, -1, :]
 
     @torch.no_grad()

@@ -27,6 +27,7 @@ from ....replacement.replacementcontext import MuiReplacementContext
 from ...attention.rotaryembedding import MuiRotaryEmbedding
 from ...attention.sdpaattention import MuiSdpaAttention, _ignore_causal_mask_sdpa
 from ...decoder.decoder import MuiDecoderLayer
+from ...embedding import MuiEmbedding
 from ...gateupdownmlp import MuiGateUpDownMLP
 from ...kvcache.cache_utils import (MuiCache, MuiStaticCache, create_static_cache,
                                     grow_static_cache_if_needed)
@@ -113,7 +114,7 @@ class MuiLlamaModel(MuiModule):
         if device is None:
             raise ValueError("device was None")
         config = prev_model.config
-        embed_tokens = prev_model.embed_tokens.to(device)
+        embed_tokens = MuiEmbedding.replace(replacement_context, prev_model.embed_tokens)
         dtype = embed_tokens.weight.dtype
         layers = []
         for i in range(len(prev_model.layers)):
@@ -268,7 +269,7 @@ class MuiLlamaForCausalLM(MuiModule):
         def rnd_(p):
             p.data.normal_(0.0, init_std, generator=gen)
 
-        embed = nn.Embedding(config.vocab_size, hid, device=device, dtype=dtype)
+        embed = MuiEmbedding(engine_config, config.vocab_size, hid, device=device, dtype=dtype)
         rnd_(embed.weight)
         layers = []
         for i in range(config.num_hidden_layers):

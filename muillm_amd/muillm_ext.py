@@ -773,3 +773,94 @@ def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch
             tokens_out.stride(0), tokens_out.shape[1], _ptr(unfinished), _ptr(eos_token_ids), n_eos, int(pad_token_id)),
         "mui_greedy_advance",
     )
+
+
+def mui_sample_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch.Tensor, tokens_out: torch.Tensor,
+                       temperature: float = 1.0, seed: int = 0, position_ids: Optional[torch.Tensor] = None,
+                       cache_position: Optional[torch.Tensor] = None, unfinished: Optional[torch.Tensor] = None,
+                       eos_token_ids: Optional[torch.Tensor] = None, pad_token_id: int = 0) -> None:
+    """Sampling twin of mui_greedy_advance: draws each row's token from softmax(logits / temperature)
+    without a host sync or a probability tensor (argmax of logit / T - log q, q ~ Exp(1) from a
+    counter-based generator keyed by `seed` and the device-side step counter), then does the same
+    in-place bookkeeping. Logits filtered to -inf (top-k / top-p) are never drawn."""
+    _check_cuda(logits, "logits")
+    if logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    v = logits.shape[-1]
+    l2 = logits.reshape(-1, v)
+    rows = l2.shape[0]
+    if not temperature > 0:
+        raise ValueError("temperature must be positive (use mui_greedy_advance for greedy decoding)")
+    for name, tns, n in (("next_ids", next_ids, rows), ("step", step, rows), ("position_ids", position_ids, rows),
+                         ("cache_position", cache_position, 1), ("unfinished", unfinished, rows)):
+        if tns is None:
+            continue
+        _check_cuda(tns, name)
+        if tns.dtype != torch.int64 or tns.numel() != n or not tns.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous int64 tensor with {n} element(s)")
+    _check_cuda(tokens_out, "tokens_out")
+    if tokens_out.dtype != torch.int64 or tokens_out.dim() != 2 or tokens_out.shape[0] != rows or tokens_out.stride(1) != 1:
+        raise RuntimeError("tokens_out must be int64 [B, max_steps] with unit inner stride")
+    n_eos = 0
+    if eos_token_ids is not None:
+        _check_cuda(eos_token_ids, "eos_token_ids")
+        if eos_token_ids.dtype != torch.int64 or not eos_token_ids.is_contiguous():
+            raise RuntimeError("eos_token_ids must be a contiguous int64 tensor")
+        n_eos = eos_token_ids.numel()
+    check(
+        _lib.load().mui_sample_advance(
+            _stream(l2), _dtype_code(l2), l2.data_ptr(), l2.stride(0) if rows > 1 else v, rows, v,
+            float(temperature), int(seed) & 0xFFFFFFFFFFFFFFFF, next_ids.data_ptr(), _ptr(position_ids),
+            _ptr(cache_position), step.data_ptr(), tokens_out.data_ptr(), tokens_out.stride(0), tokens_out.shape[1],
+            _ptr(unfinished), _ptr(eos_token_ids), n_eos, int(pad_token_id)),
+        "mui_sample_advance",
+    )
+
+
+# --------------------------------------------------------------------------------------
+# embedding (csrc/module.cpp:314-320 of the reference)
+# --------------------------------------------------------------------------------------
+class MuiEmbeddingModule:
+    """Handle returned by muillm_embedding_module_init: aliases the weight table."""
+
+    def __init__(self, engine, weights: torch.Tensor):
+        self.engine = engine
+        self.weights = weights
+
+
+def muillm_embedding_module_init(engine, weights: torch.Tensor) -> MuiEmbeddingModule:
+    if weights.dim() != 2:
+        raise RuntimeError("embedding weights must be 2-D [num_embeddings, embedding_dim]")
+    return MuiEmbeddingModule(engine, weights)
+
+
+def muillm_embedding_module_deinit(module: MuiEmbeddingModule) -> None:
+    module.weights = None
+
+
+def muillm_embedding_forward(engine, weights: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """out[..., :] = weights[x[...], :] for a 16-bit CUDA table and int32/int64 CUDA ids."""
+    _check_cuda(weights, "weights")
+    _check_cuda(x, "x")
+    if weights.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("unsupported embedding type: only float16 and bfloat16 are supported")
+    if x.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("unsupported index type: only int32 and int64 are supported")
+    if weights.stride(1) != 1:
+        raise RuntimeError("weights must have unit inner stride")
+    xc = x.contiguous()
+    dim = weights.shape[1]
+    out = torch.empty(tuple(x.shape) + (dim,), dtype=weights.dtype, device=weights.device)
+    if xc.numel() == 0:
+        return out
+    check(
+        _lib.load().mui_embedding(_stream(weights), _dtype_code(weights), weights.data_ptr(), weights.stride(0),
+                                  xc.data_ptr(), 1 if x.dtype == torch.int32 else 0, out.data_ptr(), xc.numel(), dim,
+                                  weights.shape[0]),
+        "mui_embedding",
+    )
+    return out
+
+
+def muillm_embedding_module_forward(module: MuiEmbeddingModule, x: torch.Tensor) -> torch.Tensor:
+    return muillm_embedding_forward(module.engine, module.weights, x)

@@ -11,12 +11,15 @@ from ..modules.gateupdownmlp import MuiGateUpDownMLP
 from ..modules.linear import MuiLinear
 from ..modules.models.llama.model import (MuiLlamaForCausalLM, MuiLlamaModel, MuiMistralForCausalLM,
                                           MuiMistralModel)
+from ..modules.embedding import MuiEmbedding
 from ..modules.norm.rmsnorm import MuiRMSNorm
 from .replacementcontext import MuiReplacementContext
 
 _LAYER_REPLACEMENTS = {
     # Linear
     nn.Linear: MuiLinear,
+    # Embedding
+    nn.Embedding: MuiEmbedding,
     # MLPs
     _hf.MistralMLP: MuiGateUpDownMLP,
     _hf.LlamaMLP: MuiGateUpDownMLP,

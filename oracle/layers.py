@@ -17,6 +17,8 @@ import torch.nn.functional as F
 
 __all__ = [
     "greedy_advance",
+    "philox4x32_10",
+    "sample_scores",
     "rmsnorm",
     "linear",
     "multilinear",
@@ -447,3 +449,43 @@ def greedy_advance(logits, unfinished, eos_token_ids, pad_token_id: int, steps_d
         toks[r] = tok
         unf[r] = 1 if still else 0
     return toks, unf
+
+
+# ---------------------------------------------------------------------------------------
+# sync-free sampling
+# ---------------------------------------------------------------------------------------
+def philox4x32_10(counter, key):
+    """Philox4x32-10 block function (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy
+    as 1, 2, 3", SC'11; the generator behind torch's CUDA RNG as well). counter: 4 uint32, key: 2
+    uint32 -> 4 uint32. Pinned by the known-answer vectors of the Random123 distribution."""
+    m0, m1, w0, w1 = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85
+    c = [int(x) & 0xFFFFFFFF for x in counter]
+    k = [int(x) & 0xFFFFFFFF for x in key]
+    for _ in range(10):
+        p0, p1 = m0 * c[0], m1 * c[2]
+        c = [((p1 >> 32) ^ c[1] ^ k[0]) & 0xFFFFFFFF, p1 & 0xFFFFFFFF,
+             ((p0 >> 32) ^ c[3] ^ k[1]) & 0xFFFFFFFF, p0 & 0xFFFFFFFF]
+        k = [(k[0] + w0) & 0xFFFFFFFF, (k[1] + w1) & 0xFFFFFFFF]
+    return c
+
+
+def sample_scores(logits_row, temperature: float, seed: int, row: int, step: int):
+    """Scores whose argmax is the sampled token: logit / temperature - log q with q = -log u ~ Exp(1),
+    i.e. the draw argmax(softmax(logits / temperature) / q) of the reference's
+    muillm_multinomial_sample_one_no_sync (muillm/sampling/multinomial.py:4-6) in log space.
+    u for vocabulary entry v: Philox4x32-10 with key (seed low, seed high) and counter
+    (v // 4, row, step mod 2^32, 0), lane v % 4, u = ((bits >> 8) + 1) * 2^-24. float64. Loops:
+    small vocabularies only."""
+    import math
+
+    lg = logits_row.double()
+    out = torch.empty_like(lg)
+    blocks = {}
+    for v in range(lg.shape[0]):
+        c = v // 4
+        if c not in blocks:
+            blocks[c] = philox4x32_10([c, row, step & 0xFFFFFFFF, 0], [seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF])
+        u = ((blocks[c][v % 4] >> 8) + 1) * 2.0 ** -24
+        q = max(-math.log(u), 1e-30)
+        out[v] = float(lg[v]) / temperature - math.log(q)
+    return out

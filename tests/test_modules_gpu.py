@@ -246,6 +246,84 @@ def test_greedy_advance_kernel():
     assert torch.equal(out2[:, 0].cpu(), lg.float().argmax(-1).cpu())
 
 
+def test_embedding_kernel():
+    from muillm_amd.modules.embedding import MuiEmbedding
+    g = torch.Generator().manual_seed(11)
+    for dtype, vocab, dim in ((torch.float16, 1000, 4096), (torch.bfloat16, 77, 100)):
+        emb = MuiEmbedding(MuiEngineConfig(), vocab, dim, device=DEV, dtype=dtype)
+        emb.finalize_init()
+        for idt in (torch.int64, torch.int32):
+            ids = torch.randint(0, vocab, (3, 5), generator=g).to(idt).to(DEV)
+            out = emb(ids)
+            assert out.shape == (3, 5, dim)
+            assert torch.equal(out, torch.nn.functional.embedding(ids.long(), emb.weight))
+    # a strided view of a wider table (row pitch != dim) goes through the same kernel
+    from muillm_amd import muillm_ext
+    table = torch.randn(50, 256, generator=g).half().to(DEV)
+    ids = torch.tensor([0, 49, 7], device=DEV)
+    assert torch.equal(muillm_ext.muillm_embedding_forward(None, table[:, :128], ids), table[ids, :128])
+
+
+def test_sample_advance_kernel_matches_oracle_draws():
+    """Every draw of mui_sample_advance is the argmax of the oracle's scores for the same
+    (seed, row, step) -- up to fp32 rounding of the scores -- and the bookkeeping is the greedy one."""
+    from muillm_amd import muillm_ext
+    g = torch.Generator().manual_seed(12)
+    B, V, max_steps, seed, temp = 6, 203, 5, 0x1234567890ABCDEF, 0.8
+    ids = torch.zeros(B, 1, dtype=torch.int64, device=DEV)
+    step = torch.zeros(B, dtype=torch.int64, device=DEV)
+    toks = torch.full((B, max_steps), -1, dtype=torch.int64, device=DEV)
+    pos = torch.full((B, 1), 7, dtype=torch.int64, device=DEV)
+    cpos = torch.full((1,), 7, dtype=torch.int64, device=DEV)
+    for s_i in range(max_steps):
+        logits = (2.0 * torch.randn(B, V, generator=g)).half()
+        logits[:, 5] = float("-inf")  # a filtered token can never be drawn
+        muillm_ext.mui_sample_advance(logits.to(DEV), ids, step, toks, temperature=temp, seed=seed,
+                                      position_ids=pos, cache_position=cpos)
+        got = toks[:, s_i].cpu()
+        for b in range(B):
+            sc = oracle.sample_scores(logits[b], temp, seed, b, s_i)
+            assert got[b] != 5
+            assert float(sc.max() - sc[got[b]]) <= 1e-4 * max(1.0, float(sc.max().abs())), (s_i, b)
+        assert torch.equal(ids.cpu().view(-1), got) and int(cpos.item()) == 8 + s_i
+        assert torch.equal(step.cpu(), torch.full((B,), s_i + 1))
+
+
+def test_sample_advance_distribution_and_reproducibility():
+    from muillm_amd import muillm_ext
+    rows, V = 8192, 16
+    logits = torch.linspace(-2.0, 2.0, V).half()
+    probs = torch.softmax(logits.double() / 0.9, -1)
+    lg = logits.unsqueeze(0).expand(rows, V).contiguous().to(DEV)
+
+    def draw(seed, step0):
+        ids = torch.zeros(rows, dtype=torch.int64, device=DEV)
+        step = torch.full((rows,), step0, dtype=torch.int64, device=DEV)
+        out = torch.zeros(rows, step0 + 1, dtype=torch.int64, device=DEV)
+        muillm_ext.mui_sample_advance(lg, ids, step, out, temperature=0.9, seed=seed)
+        return ids.cpu()
+
+    a, a2, b, c = draw(1, 0), draw(1, 0), draw(2, 0), draw(1, 1)
+    assert torch.equal(a, a2)                                  # same (seed, row, step) -> same draw
+    assert not torch.equal(a, b) and not torch.equal(a, c)     # seed and step both matter
+    freq = torch.bincount(torch.cat([a, b, c]), minlength=V).double() / (3 * rows)
+    sigma = (probs * (1 - probs) / (3 * rows)).sqrt()
+    assert ((freq - probs).abs() <= 5 * sigma + 1e-4).all(), (freq, probs)
+
+
+def test_graph_decode_sampling_reproducible():
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=5, init_std=0.05)
+    ids = torch.randint(0, cfg.vocab_size, (2, 6), generator=torch.Generator().manual_seed(1)).to(DEV)
+    outs = []
+    for use_graph in (True, False, True):
+        dec = MuiGraphDecoder(lm, use_graph=use_graph, do_sample=True, temperature=1.0, seed=99)
+        outs.append(dec.generate(ids, 12).cpu())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])   # replayed == eager, run to run
+    greedy = MuiGraphDecoder(lm, use_graph=True).generate(ids, 12).cpu()
+    assert not torch.equal(outs[0], greedy)
+
+
 @pytest.mark.skipif(not _hf.HAVE_TRANSFORMERS, reason="transformers not installed")
 def test_init_engine_on_hf_llama_gpu_fp16():
     """Drop-in check: a HuggingFace Llama (fp16, GPU) before and after init_engine."""

@@ -284,3 +284,30 @@ def test_greedy_advance_rules():
     t = torch.zeros(2, 6); t[0, 2] = t[0, 4] = 1.0; t[1, :] = float("-inf")
     toks4, _ = oracle.greedy_advance(t, None, None, 0, 0, 10)
     assert toks4.tolist() == [2, 0]
+
+
+def test_philox_known_answers():
+    """Known-answer vectors of Philox4x32-10 from the Random123 distribution (kat_vectors)."""
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+        ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+        ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+         [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+    ]
+    for ctr, key, want in kat:
+        assert oracle.philox4x32_10(ctr, key) == want
+
+
+def test_sample_scores_distribution():
+    """argmax of the oracle's scores is a draw from softmax(logits / T): frequencies over many
+    (row, step) streams match the probabilities (a wrong sign or a missing log would not)."""
+    logits = torch.tensor([2.0, 1.0, 0.0, -1.0, float("-inf"), 0.5])
+    temp = 0.7
+    probs = torch.softmax(logits.double() / temp, -1)
+    counts = torch.zeros(6)
+    n = 3000
+    for i in range(n):
+        counts[int(oracle.sample_scores(logits, temp, seed=1234, row=i % 7, step=i // 7).argmax())] += 1
+    freq = counts / n
+    assert counts[4] == 0
+    assert (freq - probs.float()).abs().max() < 4 * float((probs * (1 - probs) / n).sqrt().max()) + 1e-3
