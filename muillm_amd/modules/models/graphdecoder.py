@@ -47,13 +47,15 @@ class MuiGraphDecoder:
                     if self.eos_token_ids else None)
         self.out_tokens = torch.zeros((batch, max_new_tokens), dtype=torch.int64, device=device)
         self.logits = None
+        self.mask4d = None  # static additive decode mask [B, 1, 1, capacity] when the prompts are padded
         self._batch = batch
         self._max_new = max_new_tokens
 
     def _step(self):
         """One decode step on the static buffers (this is what gets captured)."""
         out = self.lm(input_ids=self.ids, position_ids=self.pos, cache_position=self.cpos,
-                      past_key_values=self.cache, use_cache=True, all_ones_mask=True, float_logits=False)
+                      past_key_values=self.cache, use_cache=True, attention_mask=self.mask4d,
+                      all_ones_mask=self.mask4d is None, float_logits=False)
         logits = out.logits[:, -1, :]
         self._advance(logits)
         return logits
@@ -98,7 +100,11 @@ class MuiGraphDecoder:
             self.cache.cpp_module.seen_tokens = seen
 
     @torch.no_grad()
-    def prefill(self, input_ids: torch.LongTensor, max_new_tokens: int, cache: Optional[MuiStaticCache] = None):
+    def prefill(self, input_ids: torch.LongTensor, max_new_tokens: int, cache: Optional[MuiStaticCache] = None,
+                attention_mask: Optional[torch.Tensor] = None):
+        """attention_mask [B, prompt_len] of 0/1 marks LEFT padding (0 = pad): padded slots stay
+        masked for the whole generation and every row counts its rotary positions from its own
+        first real token, as HuggingFace's generate does."""
         lm = self.lm
         device = input_ids.device
         batch, prompt_len = input_ids.shape
@@ -111,14 +117,38 @@ class MuiGraphDecoder:
             self.graph = None
         self.cache = cache
         cache.device_length_mode = False
-        out = lm(input_ids=input_ids, past_key_values=cache, use_cache=True, all_ones_mask=True,
-                 num_logits_to_keep=1, float_logits=False)
+        padded = attention_mask is not None and not bool(torch.all(attention_mask == 1))
+        if padded:
+            am = attention_mask.to(device=device, dtype=torch.int64)
+            if bool((am[:, -1] == 0).any()):
+                raise ValueError("padding must be on the left: the last prompt position of every row must be real")
+            prompt_pos = (am.cumsum(-1) - 1).clamp_(min=0)
+            out = lm(input_ids=input_ids, attention_mask=am, position_ids=prompt_pos, past_key_values=cache,
+                     use_cache=True, all_ones_mask=False, num_logits_to_keep=1, float_logits=False)
+        else:
+            out = lm(input_ids=input_ids, past_key_values=cache, use_cache=True, all_ones_mask=True,
+                     num_logits_to_keep=1, float_logits=False)
         if self._batch != batch or getattr(self, "_max_new", 0) < max_new_tokens:
             self._alloc_state(batch, max_new_tokens, device)
             self.graph = None
+        had_mask = self.mask4d is not None
+        if padded:
+            mdtype = lm.model.mdtype
+            if self.mask4d is None or self.mask4d.shape[-1] != cache.max_cache_len:
+                self.mask4d = torch.zeros((batch, 1, 1, cache.max_cache_len), dtype=mdtype, device=device)
+                self.graph = None
+            self.mask4d.zero_()
+            self.mask4d[:, 0, 0, :prompt_len].masked_fill_(am == 0, torch.finfo(mdtype).min)
+        else:
+            self.mask4d = None
+        if had_mask != (self.mask4d is not None):
+            self.graph = None
         # the first new token goes through the same kernel as all later ones: the counters start
         # one step back and the launch advances them to (prompt_len, prompt_len, 1)
-        self.pos.fill_(prompt_len - 1)
+        if padded:
+            self.pos.copy_(am.sum(-1, keepdim=True) - 1)
+        else:
+            self.pos.fill_(prompt_len - 1)
         self.cpos.fill_(prompt_len - 1)
         self.step.zero_()
         self.out_tokens.zero_()
@@ -150,8 +180,8 @@ class MuiGraphDecoder:
 
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, max_new_tokens: int, cache: Optional[MuiStaticCache] = None,
-                 return_logits: bool = False):
-        first_logits = self.prefill(input_ids, max_new_tokens, cache)
+                 return_logits: bool = False, attention_mask: Optional[torch.Tensor] = None):
+        first_logits = self.prefill(input_ids, max_new_tokens, cache, attention_mask=attention_mask)
         hist = self.decode(max_new_tokens - 1, collect_logits=return_logits)
         tokens = torch.cat([input_ids, self.out_tokens[:, :max_new_tokens]], dim=1)
         if return_logits:

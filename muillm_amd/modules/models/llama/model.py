@@ -353,6 +353,32 @@ class MuiLlamaForCausalLM(MuiModule):
         return dec.generate(input_ids, max_new_tokens, cache=cache, return_logits=return_logits)
 
 
+    @torch.no_grad()
+    def generate(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
+                 max_new_tokens: int = 20, do_sample: bool = False, temperature: float = 1.0,
+                 eos_token_id=None, pad_token_id: Optional[int] = None, seed: int = 0, use_graph: bool = True,
+                 cache: Optional[MuiStaticCache] = None, **unused):
+        """HuggingFace-style entry point over the device-resident decode loop (the reference routes
+        generate() through its MuiGenerationMixin._sample, muillm/sampling/generation.py:77-408).
+        Greedy (do_sample=False) or temperature sampling; left-padded batches via attention_mask;
+        rows stop at eos_token_id (int or list) and are filled with pad_token_id afterwards.
+        Returns int64 [B, prompt_len + max_new_tokens]. Logit processors beyond temperature
+        (top-k, top-p, penalties) are not part of this loop."""
+        from ..graphdecoder import MuiGraphDecoder
+
+        dropped = {k: v for k, v in unused.items() if v is not None and k in ("top_k", "top_p", "repetition_penalty")}
+        if dropped:
+            raise NotImplementedError(f"generate(): unsupported options {sorted(dropped)}")
+        eos = None
+        if eos_token_id is not None:
+            eos = [int(eos_token_id)] if isinstance(eos_token_id, int) else [int(e) for e in eos_token_id]
+        if pad_token_id is None:
+            pad_token_id = eos[0] if eos else 0
+        dec = MuiGraphDecoder(self, use_graph=use_graph, eos_token_ids=eos, pad_token_id=pad_token_id,
+                              do_sample=do_sample, temperature=temperature, seed=seed)
+        return dec.generate(input_ids, max_new_tokens, cache=cache, attention_mask=attention_mask)
+
+
 # Mistral shares the Llama implementation (the reference's mistral/model.py is a renamed copy)
 MuiMistralModel = MuiLlamaModel
 MuiMistralForCausalLM = MuiLlamaForCausalLM

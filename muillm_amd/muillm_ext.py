@@ -654,6 +654,24 @@ def _decode(q, k, v, m, n_splits=None) -> torch.Tensor:
     return out
 
 
+def _mask_rows(mask: torch.Tensor, b: int, dtype) -> torch.Tensor:
+    """A [B, S] view with unit inner stride of a decode mask, without copying when possible."""
+    _check_cuda(mask, "mask")
+    if mask.dtype != dtype:
+        raise RuntimeError("mask must have the query dtype")
+    if mask.dim() == 4 and mask.shape[1] == 1 and mask.shape[2] == 1:
+        rows = mask[:, 0, 0, :]
+    elif mask.dim() == 2:
+        rows = mask
+    else:
+        rows = mask.reshape(b, -1)
+    if rows.shape[0] != b:
+        raise RuntimeError("mask must have one row per batch entry")
+    if rows.stride(1) != 1:
+        rows = rows.contiguous()
+    return rows
+
+
 def muillm_causal_transformer_decoding_no_mask(q, k, v, n_splits=None) -> torch.Tensor:
     """q [B, Hq, 1, D] contiguous (rotated), k/v [B, Hkv, S, D] cache views -> [B, 1, Hq*D]."""
     return _decode(q, k, v, None, n_splits)
@@ -690,7 +708,9 @@ def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_positi
     pos_bs = 1 if pos.numel() > 1 else 0
     mask_ptr, mask_bs = None, 0
     if mask is not None:
-        mask = mask.reshape(b, -1).contiguous()
+        # [B, 1, 1, S] (or [B, S]); a view into a wider static buffer is used in place: under graph
+        # replay the kernel reads up to the device-side sequence length, beyond the view's width
+        mask = _mask_rows(mask, b, q.dtype)
         mask_ptr, mask_bs = mask.data_ptr(), mask.stride(0)
     if n_splits is None:
         hint = seq_len if seq_len is not None else (seq_len_hint if seq_len_hint is not None else max_t)

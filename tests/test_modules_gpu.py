@@ -246,6 +246,49 @@ def test_greedy_advance_kernel():
     assert torch.equal(out2[:, 0].cpu(), lg.float().argmax(-1).cpu())
 
 
+def test_generate_left_padded_batch_matches_single_runs():
+    """Left-padded batch generation (static device-side mask + per-row rotary positions, graph
+    replay) must give every row the tokens it gets when generated alone without padding."""
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=8, init_std=0.08)
+    g = torch.Generator().manual_seed(2)
+    long_p = torch.randint(1, cfg.vocab_size, (1, 11), generator=g)
+    short_p = torch.randint(1, cfg.vocab_size, (1, 6), generator=g)
+    n_new = 10
+    alone = [lm.generate(p.to(DEV), max_new_tokens=n_new)[0, p.shape[1]:].cpu() for p in (long_p, short_p)]
+    batch = torch.zeros(2, 11, dtype=torch.int64)
+    mask = torch.zeros(2, 11, dtype=torch.int64)
+    batch[0], mask[0] = long_p[0], 1
+    batch[1, 5:], mask[1, 5:] = short_p[0], 1
+    for use_graph in (True, False):
+        out = lm.generate(batch.to(DEV), attention_mask=mask.to(DEV), max_new_tokens=n_new, use_graph=use_graph).cpu()
+        assert out.shape == (2, 11 + n_new)
+        for r in range(2):
+            got = out[r, 11:]
+            # fp16 reduction order differs between batch sizes: allow a late divergence, not an early one
+            agree = int((got == alone[r]).long().cumprod(0).sum())
+            assert agree >= n_new - 2, (use_graph, r, got, alone[r])
+
+
+def test_generate_stops_at_eos_and_pads():
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=9, init_std=0.08)
+    ids = torch.randint(1, cfg.vocab_size, (2, 7), generator=torch.Generator().manual_seed(3)).to(DEV)
+    free = lm.generate(ids, max_new_tokens=8).cpu()
+    eos = int(free[0, 7 + 3])                      # row 0 emits this at its 4th new token
+    first_hit = [int((free[r, 7:] == eos).nonzero()[0]) if bool((free[r, 7:] == eos).any()) else None for r in range(2)]
+    out = lm.generate(ids, max_new_tokens=8, eos_token_id=eos, pad_token_id=0).cpu()
+    for r in range(2):
+        h = first_hit[r]
+        if h is None:
+            assert torch.equal(out[r], free[r])
+        else:
+            assert torch.equal(out[r, : 7 + h + 1], free[r, : 7 + h + 1])   # identical up to and including eos
+            assert bool((out[r, 7 + h + 1:] == 0).all())                      # pad afterwards
+    with pytest.raises(NotImplementedError):
+        lm.generate(ids, max_new_tokens=2, top_k=5)
+
+
 def test_embedding_kernel():
     from muillm_amd.modules.embedding import MuiEmbedding
     g = torch.Generator().manual_seed(11)
