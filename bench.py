@@ -353,6 +353,8 @@ def main():
                     help="experiment: mui_tune_attention(waves per workgroup, min tokens per split, "
                          "longest unsplit sequence (-1 disables the head-parallel unsplit mode), shortest sequence for "
                          "the matrix-core kernel (-1 disables it))")
+    ap.add_argument("--only-kernel-table", action="store_true",
+                    help="only time the per-kernel table (for rocprofv3 kernel traces of the C1-C4 shapes)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
     args = ap.parse_args()
@@ -379,6 +381,9 @@ def main():
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
     torch.cuda.synchronize()
 
+    if args.only_kernel_table:
+        print(json.dumps({"kernels": kernel_table(lm)}))
+        return
     dt, dec = bench_decode(lm, args.steps, args.warmup)
     tokens_per_s = args.steps / dt
     hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size

@@ -267,3 +267,30 @@ def test_mlp_closed_forms():
     # Wg = 0 -> silu(0) = 0 -> out = residual ; Wu = 0 -> out = residual
     assert torch.equal(muillm_ext.muillm_gateupsilu_forward(None, None, 0.0, z, w, wd, r, x), r)
     assert torch.equal(muillm_ext.muillm_gateupsilu_forward(None, None, 0.0, w, z, wd, r, x), r)
+
+
+def test_lm_head_full_size_gather_property():
+    """At the full lm_head size (128256 x 4096, 1.05 GB) the oracle is too slow; a one-hot input
+    turns the GEMV into a column gather, which must be bit-exact, and linearity ties a random
+    input to two such runs (size-independent properties)."""
+    from muillm_amd import muillm_ext
+    g = torch.Generator(device="cuda").manual_seed(0)
+    n, k = 128256, 4096
+    w = torch.randn(n, k, device="cuda", dtype=torch.float16, generator=g) * 0.02
+    for j in (0, 1, 2047, 4095):
+        x = torch.zeros(1, k, device="cuda", dtype=torch.float16)
+        x[0, j] = 1.0
+        y = muillm_ext.muillm_linear_forward(None, x, w)
+        assert torch.equal(y[0], w[:, j])
+    # rows of ones -> sum of the inputs, for every one of the 128256 outputs
+    w1 = torch.ones(n, 64, device="cuda", dtype=torch.float16)
+    x = torch.randn(1, 64, device="cuda", dtype=torch.float16, generator=g)
+    y = muillm_ext.muillm_linear_forward(None, x, w1)
+    want = x.float().sum()
+    assert float((y.float() - want).abs().max()) <= 2e-3 * max(1.0, abs(float(want)))
+    # a random input against torch's fp32 matmul on a strided sample of rows
+    x = torch.randn(1, k, device="cuda", dtype=torch.float16, generator=g)
+    y = muillm_ext.muillm_linear_forward(None, x, w)
+    rows = torch.arange(0, n, 257, device="cuda")
+    ref = (w[rows].float() @ x[0].float())
+    assert float((y[0, rows].float() - ref).abs().max()) <= 1e-2 * float(ref.abs().max())
