@@ -301,10 +301,12 @@ int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
  * matrix-core kernel (default 0 = never: the vector kernel measured faster on MI355X) */
 int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
                        int mfma_tokens);
-/* fewest tokens that take the MFMA skinny-GEMM kernel instead of one GEMV per token (default 2;
- * MUI_MAX_TOKENS + 1 disables it); stream_b != 0 forces the variant that re-reads the token
- * operands per weight tile instead of keeping them in registers (K <= 4096 only) */
-int mui_tune_skinny(int min_tokens, int stream_b);
+/* fewest tokens that leave the one-GEMV-per-token loop (default 2; MUI_MAX_TOKENS + 1 keeps the
+ * loop); stream_b != 0 forces the MFMA variant that re-reads the token operands per weight tile
+ * instead of keeping them in registers (K <= 4096 only); multi_max_tokens: largest token count
+ * served by the multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 4,
+ * 1 = never) */
+int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 
 #ifdef __cplusplus
 }

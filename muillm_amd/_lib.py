@@ -74,7 +74,7 @@ _SIGNATURES = {
     "mui_embedding": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, c_int, c_int, c_int]),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
-    "mui_tune_skinny": (c_int, [c_int, c_int]),
+    "mui_tune_skinny": (c_int, [c_int, c_int, c_int]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

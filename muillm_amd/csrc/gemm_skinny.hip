@@ -85,38 +85,6 @@ __device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint1
   }
 }
 
-// B operand of one k-chunk: gamma * x rounded to the 16-bit type, sum of squares on the side.
-// fp16: packed multiply (one rounding, same result as the fp32 product rounded once) and a
-// packed dot for the squares.
-template <typename T, bool NORM>
-__device__ __forceinline__ u32x4 make_b(const u32x4 xv, const u32x4 gv, float& ss) {
-  if constexpr (!NORM) {
-    return xv;
-  } else if constexpr (T::kDtype == MUI_DTYPE_F16) {
-    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
-    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w};
-    uint32_t o[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const f16x2 xx = __builtin_bit_cast(f16x2, xw[i]);
-      ss = __builtin_amdgcn_fdot2(xx, xx, ss, false);
-      o[i] = __builtin_bit_cast(uint32_t, xx * __builtin_bit_cast(f16x2, gw[i]));
-    }
-    u32x4 b = {o[0], o[1], o[2], o[3]};
-    return b;
-  } else {
-    float xf[8], gf[8], o[8];
-    unpack8<T>(xv, xf);
-    unpack8<T>(gv, gf);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      ss = fmaf(xf[i], xf[i], ss);
-      o[i] = xf[i] * gf[i];
-    }
-    return pack8<T>(o);
-  }
-}
-
 template <typename T, int WF, bool NORM, int EPI>
 __global__ void __launch_bounds__(kSkThreads) gemm_skinny_kernel(const SkinnyParams p) {
   __shared__ float tile[kSkWaves][16][17];

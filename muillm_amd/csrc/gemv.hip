@@ -265,11 +265,15 @@ using namespace mui;
 
 // token count from which the MFMA skinny-GEMM kernel takes over (below: one GEMV per token)
 static int g_skinny_min_tokens = 2;
+// largest token count that takes the multi-token GEMV (gemv_multi.hip) instead of the MFMA kernel
+static int g_multi_max_tokens = 4;
 
-extern "C" int mui_tune_skinny(int min_tokens, int stream_b) {
+extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens) {
   if (min_tokens < 1 || min_tokens > MUI_MAX_TOKENS + 1) return MUI_ERR_INVALID_ARG;
+  if (multi_max_tokens < 0 || multi_max_tokens > 4) return MUI_ERR_INVALID_ARG;
   g_skinny_min_tokens = min_tokens;
   skinny_set_bstat(stream_b == 0);
+  g_multi_max_tokens = multi_max_tokens == 0 ? 4 : multi_max_tokens;
   return MUI_OK;
 }
 
@@ -310,6 +314,10 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
     sp.k = k_in;
     sp.tokens = tokens;
     sp.eps = epsilon;
+    if (tokens <= g_multi_max_tokens) {
+      const int st = launch_gemv_multi(s, dtype, SK_LINEAR, sp);
+      if (st != MUI_ERR_UNSUPPORTED) return st;
+    }
     return launch_skinny(s, dtype, WF_16BIT, SK_LINEAR, sp);
   }
   for (int tkn = 0; tkn < tokens; ++tkn) {
@@ -359,6 +367,10 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
     sp.k = k_in;
     sp.tokens = tokens;
     sp.eps = epsilon;
+    if (tokens <= g_multi_max_tokens) {
+      const int st = launch_gemv_multi(s, dtype, SK_GATEUP, sp);
+      if (st != MUI_ERR_UNSUPPORTED) return st;
+    }
     return launch_skinny(s, dtype, WF_16BIT, SK_GATEUP, sp);
   }
   for (int tkn = 0; tkn < tokens; ++tkn) {

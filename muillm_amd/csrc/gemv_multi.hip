@@ -1,0 +1,214 @@
+// Fused linears for 2..4 tokens with 16-bit weights: the single-token GEMV structure (256
+// threads, thread t owns 16-byte chunks t, t+256, ... of every row, R rows in flight, next row
+// group requested before the reduction, persistent balanced grid) with the token operands
+// gamma * x packed 16-bit in registers and one packed dot (v_dot2_f32_f16) per two weights and
+// token. The weights are streamed exactly once; at up to 4 tokens the vector ALUs stay far from
+// saturation, so the kernel runs at the single-token GEMV's HBM rate where the matrix-core
+// skinny GEMM (gemm_skinny.hip, used from 5 tokens) pays for its tile hand-offs.
+//
+// The reference has no kernel for this case (csrc/modules/linear_module.cpp:57-79 falls back to
+// RMSNorm + torch matmul + add; muillm/modules/gateupdownmlp.py:343-359).
+#include "skinny.cuh"
+
+namespace mui {
+
+constexpr int kMtThreads = 256;
+constexpr int kMtWaves = kMtThreads / kWave;
+
+template <typename T>
+__device__ __forceinline__ float dot2_mt(uint32_t a, uint32_t b, float c);
+template <>
+__device__ __forceinline__ float dot2_mt<F16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+template <>
+__device__ __forceinline__ float dot2_mt<BF16>(uint32_t a, uint32_t b, float c) {
+  c = fmaf(BF16::lo(a), BF16::lo(b), c);
+  return fmaf(BF16::hi(a), BF16::hi(b), c);
+}
+
+template <typename T, int R, int CH, bool NORM, int EPI, int TOK>
+__global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
+    // scalars, hottest first (preloaded into SGPRs at wave launch)
+    const uint16_t* w0, const uint16_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
+    uint16_t* y, int n, int k, int tokens, float eps, const uint16_t* residual,
+    const uint16_t* mul_bias, const uint16_t* add_bias) {
+  constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
+  static_assert(EPI != SK_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
+  __shared__ float red[2][kMtWaves][R][TOK];
+  __shared__ float red_ss[kMtWaves][TOK];
+
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int kc = k >> 3;
+  const int n_groups = (n + OUT - 1) / OUT;
+
+  int coff[CH];
+  bool cvalid[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const int c = t + kMtThreads * j;
+    cvalid[j] = c < kc;
+    coff[j] = cvalid[j] ? (c << 3) : 0;
+  }
+
+  u32x4 w[R][CH];
+  auto issue = [&](int rg) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int row;
+      const uint16_t* base;
+      if constexpr (EPI == SK_GATEUP) {
+        row = rg * OUT + (r >> 1);
+        base = (r & 1) ? w1 : w0;
+      } else {
+        row = rg * R + r;
+        base = w0;
+      }
+      row = row < n ? row : n - 1;
+      const uint16_t* rp = base + (long)row * pitch;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) w[r][j] = ld16_stream(rp + coff[j]);
+    }
+  };
+  int rg = blockIdx.x;
+  if (rg < n_groups) issue(rg);
+
+  // ---- token operands: gamma * x rounded once to the 16-bit type (zero past the row / batch) ----
+  u32x4 xq[TOK][CH];
+  float ss[TOK];
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) {
+    ss[tk] = 0.f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      u32x4 b = {0u, 0u, 0u, 0u};
+      if (cvalid[j] && tk < tokens) {
+        const u32x4 xv = ld16(x + (long)tk * k + coff[j]);
+        u32x4 gv = xv;
+        if constexpr (NORM) gv = ld16(gamma + coff[j]);
+        b = make_b<T, NORM>(xv, gv, ss[tk]);
+      }
+      xq[tk][j] = b;
+    }
+  }
+  float rs[TOK];
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) rs[tk] = 1.f;
+  if constexpr (NORM) {
+#pragma unroll
+    for (int tk = 0; tk < TOK; ++tk) {
+      const float s = wave_sum(ss[tk]);
+      if (lane == 0) red_ss[wave][tk] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tk = 0; tk < TOK; ++tk) {
+      const float tot = (red_ss[0][tk] + red_ss[1][tk]) + (red_ss[2][tk] + red_ss[3][tk]);
+      rs[tk] = rsqrtf(tot / (float)k + eps);
+    }
+  }
+
+  int buf = 0;
+  for (; rg < n_groups; rg += gridDim.x) {
+    float acc[R][TOK];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int tk = 0; tk < TOK; ++tk) {
+        float a = 0.f;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+          a = dot2_mt<T>(w[r][j].x, xq[tk][j].x, a);
+          a = dot2_mt<T>(w[r][j].y, xq[tk][j].y, a);
+          a = dot2_mt<T>(w[r][j].z, xq[tk][j].z, a);
+          a = dot2_mt<T>(w[r][j].w, xq[tk][j].w, a);
+        }
+        acc[r][tk] = a;
+      }
+    }
+    const int nxt = rg + gridDim.x;
+    if (nxt < n_groups) issue(nxt);  // keep the memory pipe full during the reduction
+
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int tk = 0; tk < TOK; ++tk) {
+        const float s = wave_sum(acc[r][tk]);
+        if (lane == 0) red[buf][wave][r][tk] = s;
+      }
+    __syncthreads();
+
+    if (t < OUT * TOK) {
+      const int o = t / TOK, tk = t % TOK;
+      const int row = rg * OUT + o;
+      if (row < n && tk < tokens) {
+        float rsv = rs[0];
+#pragma unroll
+        for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
+        auto total = [&](int r) {
+          return ((red[buf][0][r][tk] + red[buf][1][r][tk]) + (red[buf][2][r][tk] + red[buf][3][r][tk])) * rsv;
+        };
+        float v;
+        if constexpr (EPI == SK_GATEUP) {
+          v = silu_f32(total(2 * o)) * total(2 * o + 1);
+        } else {
+          v = total(o);
+          if (mul_bias) v *= T::one(mul_bias[row]);
+          if (add_bias) v += T::one(add_bias[row]);
+          if (residual) v += T::one(residual[(long)tk * n + row]);
+        }
+        y[(long)tk * n + row] = T::pack(v);
+      }
+    }
+    buf ^= 1;
+  }
+}
+
+template <typename T, int R, int CH, int EPI, int TOK>
+static int launch_mt_rc(hipStream_t s, const SkinnyParams& p, int grid) {
+#define MUI_MT_LAUNCH(NORMV)                                                                                   \
+  hipLaunchKernelGGL((gemv_multi_kernel<T, R, CH, NORMV, EPI, TOK>), dim3(grid), dim3(kMtThreads), 0, s,        \
+                     (const uint16_t*)p.w0, (const uint16_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k,        \
+                     p.tokens, p.eps, p.residual, p.mul_bias, p.add_bias)
+  if (p.gamma) MUI_MT_LAUNCH(true); else MUI_MT_LAUNCH(false);
+#undef MUI_MT_LAUNCH
+  return launch_status();
+}
+
+template <typename T, int EPI, int TOK>
+static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
+  const int ch = ceil_div(p.k >> 3, kMtThreads);
+  if (ch <= 2) {
+    constexpr int R = 4, OUT = (EPI == SK_GATEUP) ? 2 : 4;
+    const int grid = balanced_grid(ceil_div(p.n, OUT), 3);
+    if (ch <= 1) return launch_mt_rc<T, R, 1, EPI, TOK>(s, p, grid);
+    return launch_mt_rc<T, R, 2, EPI, TOK>(s, p, grid);
+  }
+  constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
+  const int grid = balanced_grid(ceil_div(p.n, OUT), 2);
+  if (ch <= 4) return launch_mt_rc<T, R, 4, EPI, TOK>(s, p, grid);
+  if (ch <= 7) return launch_mt_rc<T, R, 7, EPI, TOK>(s, p, grid);
+  return MUI_ERR_UNSUPPORTED;
+}
+
+int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p) {
+  if (p.tokens < 2 || p.tokens > 4) return MUI_ERR_UNSUPPORTED;
+#define MUI_MT_CASE(TT, EPIV)                                            \
+  if (epilogue == EPIV) {                                                \
+    if (p.tokens <= 2) return launch_mt_t<TT, EPIV, 2>(s, p);            \
+    return launch_mt_t<TT, EPIV, 4>(s, p);                               \
+  }
+  if (dtype == MUI_DTYPE_F16) {
+    MUI_MT_CASE(F16, SK_LINEAR)
+    MUI_MT_CASE(F16, SK_GATEUP)
+  } else if (dtype == MUI_DTYPE_BF16) {
+    MUI_MT_CASE(BF16, SK_LINEAR)
+    MUI_MT_CASE(BF16, SK_GATEUP)
+  }
+#undef MUI_MT_CASE
+  return MUI_ERR_INVALID_ARG;
+}
+
+}  // namespace mui
