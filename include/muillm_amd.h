@@ -304,8 +304,8 @@ int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int di
 /* fewest tokens that leave the one-GEMV-per-token loop (default 2; MUI_MAX_TOKENS + 1 keeps the
  * loop); stream_b != 0 forces the MFMA variant that re-reads the token operands per weight tile
  * instead of keeping them in registers (K <= 4096 only); multi_max_tokens: largest token count
- * served by the multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 4,
- * 1 = never) */
+ * served by the multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 8,
+ * where 5..8 tokens only qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
 int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 
 #ifdef __cplusplus

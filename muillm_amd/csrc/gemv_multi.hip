@@ -1,10 +1,10 @@
-// Fused linears for 2..4 tokens with 16-bit weights: the single-token GEMV structure (256
+// Fused linears for 2..4 tokens (up to 8 on tall matrices) with 16-bit weights: the single-token GEMV structure (256
 // threads, thread t owns 16-byte chunks t, t+256, ... of every row, R rows in flight, next row
 // group requested before the reduction, persistent balanced grid) with the token operands
 // gamma * x packed 16-bit in registers and one packed dot (v_dot2_f32_f16) per two weights and
 // token. The weights are streamed exactly once; at up to 4 tokens the vector ALUs stay far from
 // saturation, so the kernel runs at the single-token GEMV's HBM rate where the matrix-core
-// skinny GEMM (gemm_skinny.hip, used from 5 tokens) pays for its tile hand-offs.
+// skinny GEMM (gemm_skinny.hip, used otherwise from 5 tokens) pays for its tile hand-offs.
 //
 // The reference has no kernel for this case (csrc/modules/linear_module.cpp:57-79 falls back to
 // RMSNorm + torch matmul + add; muillm/modules/gateupdownmlp.py:343-359).
@@ -35,7 +35,8 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
     const uint16_t* mul_bias, const uint16_t* add_bias) {
   constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
   static_assert(EPI != SK_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
-  __shared__ float red[2][kMtWaves][R][TOK];
+  constexpr int NV = R * TOK;  // partial sums per row group: value r * TOK + token
+  __shared__ float red[2][kMtWaves * 4][NV];  // [buffer][wave * 4 + 16-lane row][value]
   __shared__ float red_ss[kMtWaves][TOK];
 
   const int t = threadIdx.x;
@@ -112,7 +113,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
 
   int buf = 0;
   for (; rg < n_groups; rg += gridDim.x) {
-    float acc[R][TOK];
+    float acc[NV];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
@@ -125,19 +126,16 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
           a = dot2_mt<T>(w[r][j].z, xq[tk][j].z, a);
           a = dot2_mt<T>(w[r][j].w, xq[tk][j].w, a);
         }
-        acc[r][tk] = a;
+        acc[r * TOK + tk] = a;
       }
     }
     const int nxt = rg + gridDim.x;
     if (nxt < n_groups) issue(nxt);  // keep the memory pipe full during the reduction
 
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int tk = 0; tk < TOK; ++tk) {
-        const float s = wave_sum(acc[r][tk]);
-        if (lane == 0) red[buf][wave][r][tk] = s;
-      }
+    // all NV sums of a 16-lane row in one multi-value DPP reduction; the 16 row partials
+    // (4 waves x 4 rows) are added by the epilogue threads
+    row16_reduce_scatter<NV>(acc, lane);
+    if ((lane & (16 / NV - 1)) == 0 || NV == 16) red[buf][t >> 4][(lane & 15) / (16 / NV)] = acc[0];
     __syncthreads();
 
     if (t < OUT * TOK) {
@@ -148,7 +146,10 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
 #pragma unroll
         for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
         auto total = [&](int r) {
-          return ((red[buf][0][r][tk] + red[buf][1][r][tk]) + (red[buf][2][r][tk] + red[buf][3][r][tk])) * rsv;
+          float v = 0.f;
+#pragma unroll
+          for (int q = 0; q < kMtWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
+          return v * rsv;
         };
         float v;
         if constexpr (EPI == SK_GATEUP) {
@@ -180,6 +181,16 @@ static int launch_mt_rc(hipStream_t s, const SkinnyParams& p, int grid) {
 template <typename T, int EPI, int TOK>
 static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
   const int ch = ceil_div(p.k >> 3, kMtThreads);
+  if constexpr (TOK == 8) {
+    // 8 tokens: 2 rows x 8 tokens = 16 partial sums per group; only rows of <= 2 chunks per thread
+    // and only tall matrices, where it measured faster than the matrix-core kernel (43 vs 48 us on
+    // the 2 x 14336 x 4096 gate/up shape; on par or slower at 6144 and 4096 rows)
+    if (ch > 2 || p.n < 8192) return MUI_ERR_UNSUPPORTED;
+    constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
+    const int grid = balanced_grid(ceil_div(p.n, OUT), 4);
+    if (ch <= 1) return launch_mt_rc<T, R, 1, EPI, TOK>(s, p, grid);
+    return launch_mt_rc<T, R, 2, EPI, TOK>(s, p, grid);
+  } else {
   if (ch <= 2) {
     constexpr int R = 4, OUT = (EPI == SK_GATEUP) ? 2 : 4;
     const int grid = balanced_grid(ceil_div(p.n, OUT), 3);
@@ -191,14 +202,16 @@ static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
   if (ch <= 4) return launch_mt_rc<T, R, 4, EPI, TOK>(s, p, grid);
   if (ch <= 7) return launch_mt_rc<T, R, 7, EPI, TOK>(s, p, grid);
   return MUI_ERR_UNSUPPORTED;
+  }
 }
 
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p) {
-  if (p.tokens < 2 || p.tokens > 4) return MUI_ERR_UNSUPPORTED;
+  if (p.tokens < 2 || p.tokens > 8) return MUI_ERR_UNSUPPORTED;
 #define MUI_MT_CASE(TT, EPIV)                                            \
   if (epilogue == EPIV) {                                                \
     if (p.tokens <= 2) return launch_mt_t<TT, EPIV, 2>(s, p);            \
-    return launch_mt_t<TT, EPIV, 4>(s, p);                               \
+    if (p.tokens <= 4) return launch_mt_t<TT, EPIV, 4>(s, p);            \
+    return launch_mt_t<TT, EPIV, 8>(s, p);                               \
   }
   if (dtype == MUI_DTYPE_F16) {
     MUI_MT_CASE(F16, SK_LINEAR)

@@ -65,7 +65,7 @@ int launch_skinny(hipStream_t s, int dtype, int weight_format, int epilogue, con
 // experiments: 0 disables the B-stationary persistent variant
 void skinny_set_bstat(int on);
 
-// 2..4 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
+// 2..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
 // in registers (gemv_multi.hip); returns MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
 
