@@ -427,8 +427,15 @@ static int launch_skinny_t(hipStream_t s, const SkinnyParams& p) {
 
 void skinny_set_bstat(int on) { g_skinny_bstat = on; }
 
+static int g_int8_multi = 1;  // 2..4 tokens of int8 weights: vector-ALU kernel (int8_multi.hip) first
+void skinny_set_int8_multi(int on) { g_int8_multi = on; }
+
 // entry used by gemv.hip / int8.hip for tokens >= 2
 int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams& p) {
+  if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4) {
+    const int st = launch_int8_multi(s, dtype, wf, epi, p);
+    if (st != MUI_ERR_UNSUPPORTED) return st;
+  }
 #define MUI_SK_CASE(TT, WFV, EPIV) \
   if (wf == WFV && epi == EPIV) return launch_skinny_t<TT, WFV, EPIV>(s, p);
   if (dtype == MUI_DTYPE_F16) {

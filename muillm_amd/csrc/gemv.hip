@@ -274,6 +274,7 @@ extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_token
   g_skinny_min_tokens = min_tokens;
   skinny_set_bstat(stream_b == 0);
   g_multi_max_tokens = multi_max_tokens == 0 ? 8 : multi_max_tokens;
+  skinny_set_int8_multi(g_multi_max_tokens >= 2);
   return MUI_OK;
 }
 

@@ -1,0 +1,270 @@
+// Weight-only int8 linears for 2..4 tokens (fp16 activations): the single-token int8 GEMV
+// structure (int8.hip) with the token operands gamma * x packed fp16 in registers.
+//
+// Dequantisation without a convert per weight: a byte b dropped into the mantissa of 1024.0
+// (0x6400 | b, two byte permutes per dword) IS the fp16 number 1024 + b, so
+//     sum_k (1024 + b_k) x_k  -  1024 sum_k x_k  =  sum_k b_k x_k
+// with one v_dot2_f32_f16 per two weights and token; the correction term is folded into the
+// accumulator's start value (per-channel format, where the sign bit is flipped first: offset
+// 1024 + 128) or applied per group together with (scale, min) (the reference's group format,
+// muillm/quantization/rtnquantizer.py:49-88). The products are exact in fp32 and the offset is
+// 16x the largest weight, so the cancellation costs about 4 bits of the fp32 accumulator.
+//
+// The reference has no kernel for more than one token (muillm/modules/quantized/int8linear.py:279-293
+// dequantises the whole matrix and calls F.linear).
+#include "skinny.cuh"
+
+namespace mui {
+
+constexpr int kI8mThreads = 256;
+constexpr int kI8mWaves = kI8mThreads / kWave;
+
+struct Int8MultiArgs {
+  const uint16_t* s0; const uint16_t* s1; long s_pitch; int group_shift;
+  const uint16_t* add_bias; const uint16_t* residual;
+};
+
+template <int R, int CH, bool NORM, int EPI, int WF, int TOK>
+__global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
+    // scalars, hottest first (preloaded into SGPRs at wave launch)
+    const uint8_t* w0, const uint8_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
+    uint16_t* y, int n, int k, int tokens, float eps, const Int8MultiArgs a) {
+  using T = F16;
+  constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
+  constexpr int NV = R * TOK;             // partial sums per row group
+  constexpr int NH = NV > 16 ? 2 : 1;     // reduced 16 at a time
+  constexpr int NVH = NV / NH;
+  constexpr uint32_t kFlip = (WF == WF_I8_CHANNEL) ? 0x80808080u : 0u;
+  constexpr float kOffset = (WF == WF_I8_CHANNEL) ? 1152.f : 1024.f;
+  static_assert(NV <= 32 && (R % 2 == 0), "shape");
+  __shared__ float red[2][kI8mWaves * 4][NV];
+  __shared__ float red_ss[kI8mWaves][TOK];
+
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int kc = k >> 4;  // 16-byte chunks (16 weights) per row
+  const int n_groups = (n + OUT - 1) / OUT;
+
+  int coff[CH];
+  bool cvalid[CH];
+#pragma unroll
+  for (int j = 0; j < CH; ++j) {
+    const int c = t + kI8mThreads * j;
+    cvalid[j] = c < kc;
+    coff[j] = cvalid[j] ? (c << 4) : 0;
+  }
+
+  u32x4 w[R][CH];
+  uint32_t sm[R][CH];  // group format: packed (scale, min) of the chunk's group
+  auto issue = [&](int rg) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int row;
+      const uint8_t* base;
+      const uint16_t* sbase;
+      if constexpr (EPI == SK_GATEUP) {
+        row = rg * OUT + (r >> 1);
+        base = (r & 1) ? w1 : w0;
+        sbase = (r & 1) ? a.s1 : a.s0;
+      } else {
+        row = rg * R + r;
+        base = w0;
+        sbase = a.s0;
+      }
+      row = row < n ? row : n - 1;
+      const uint8_t* rp = base + (long)row * pitch;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        w[r][j] = ld16_stream(rp + coff[j]);
+        if constexpr (WF == WF_U8_GROUP)
+          sm[r][j] = *(const uint32_t*)(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
+      }
+    }
+  };
+  int rg = blockIdx.x;
+  if (rg < n_groups) issue(rg);
+
+  // ---- token operands: gamma * x as packed fp16, the chunk's sum of them on the side ----
+  u32x4 xq[TOK][CH][2];
+  float xsum[TOK][CH];
+  float ss[TOK];
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) {
+    ss[tk] = 0.f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      xsum[tk][j] = 0.f;
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        u32x4 b = {0u, 0u, 0u, 0u};
+        if (cvalid[j] && tk < tokens) {
+          const u32x4 xv = ld16(x + (long)tk * k + coff[j] + 8 * hf);
+          u32x4 gv = xv;
+          if constexpr (NORM) gv = ld16(gamma + coff[j] + 8 * hf);
+          b = make_b<T, NORM>(xv, gv, ss[tk]);
+        }
+        xq[tk][j][hf] = b;
+        float bf[8];
+        unpack8<T>(b, bf);
+        xsum[tk][j] += ((bf[0] + bf[1]) + (bf[2] + bf[3])) + ((bf[4] + bf[5]) + (bf[6] + bf[7]));
+      }
+    }
+  }
+  float acc_init[TOK];  // per-channel: -(1024 + 128) * sum of this thread's operands
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) {
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) s += xsum[tk][j];
+    acc_init[tk] = -kOffset * s;
+  }
+  float rs[TOK];
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) rs[tk] = 1.f;
+  if constexpr (NORM) {
+#pragma unroll
+    for (int tk = 0; tk < TOK; ++tk) {
+      const float s = wave_sum(ss[tk]);
+      if (lane == 0) red_ss[wave][tk] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tk = 0; tk < TOK; ++tk) {
+      const float tot = (red_ss[0][tk] + red_ss[1][tk]) + (red_ss[2][tk] + red_ss[3][tk]);
+      rs[tk] = rsqrtf(tot / (float)k + eps);
+    }
+  }
+
+  int buf = 0;
+  for (; rg < n_groups; rg += gridDim.x) {
+    float acc[NH][NVH];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float ar[TOK];
+#pragma unroll
+      for (int tk = 0; tk < TOK; ++tk) ar[tk] = (WF == WF_I8_CHANNEL) ? acc_init[tk] : 0.f;
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        // 16 bytes -> 8 packed pairs (1024 + b): pairs 0..3 meet xq[..][0], pairs 4..7 meet xq[..][1]
+        const uint32_t wv[4] = {w[r][j].x ^ kFlip, w[r][j].y ^ kFlip, w[r][j].z ^ kFlip, w[r][j].w ^ kFlip};
+        uint32_t pr[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          pr[2 * d + 0] = __builtin_amdgcn_perm(0x64646464u, wv[d], 0x04010400u);
+          pr[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, wv[d], 0x04030402u);
+        }
+#pragma unroll
+        for (int tk = 0; tk < TOK; ++tk) {
+          float s = (WF == WF_I8_CHANNEL) ? ar[tk] : 0.f;
+          // components go through scalars: __builtin_bit_cast applied directly to a vector
+          // component (q.y) was compiled as a read of component 0 by this toolchain
+          const u32x4 q0 = xq[tk][j][0], q1 = xq[tk][j][1];
+          const uint32_t qa[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+          for (int d = 0; d < 8; ++d)
+            s = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pr[d]), __builtin_bit_cast(f16x2, qa[d]), s, false);
+          if constexpr (WF == WF_I8_CHANNEL) {
+            ar[tk] = s;
+          } else {
+            // w = u8 * scale + min over this chunk's group: scale * (s - 1024 xsum) + min * xsum
+            const float sc = T::lo(sm[r][j]), mn = T::hi(sm[r][j]);
+            ar[tk] = fmaf(sc, fmaf(-kOffset, xsum[tk][j], s), fmaf(mn, xsum[tk][j], ar[tk]));
+          }
+        }
+      }
+#pragma unroll
+      for (int tk = 0; tk < TOK; ++tk) {
+        const int v = r * TOK + tk;
+        acc[v / NVH][v % NVH] = ar[tk];
+      }
+    }
+    const int nxt = rg + gridDim.x;
+    if (nxt < n_groups) issue(nxt);
+
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      row16_reduce_scatter<NVH>(acc[h], lane);
+      if ((lane & (16 / NVH - 1)) == 0 || NVH == 16) red[buf][t >> 4][h * NVH + (lane & 15) / (16 / NVH)] = acc[h][0];
+    }
+    __syncthreads();
+
+    if (t < OUT * TOK) {
+      const int o = t / TOK, tk = t % TOK;
+      const int row = rg * OUT + o;
+      if (row < n && tk < tokens) {
+        float rsv = rs[0];
+#pragma unroll
+        for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
+        auto total = [&](int r) {
+          float v = 0.f;
+#pragma unroll
+          for (int q = 0; q < kI8mWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
+          return v * rsv;
+        };
+        float v;
+        if constexpr (EPI == SK_GATEUP) {
+          float g = total(2 * o), u = total(2 * o + 1);
+          if constexpr (WF == WF_I8_CHANNEL) {
+            g *= T::one(a.s0[(long)row * a.s_pitch]);
+            u *= T::one(a.s1[(long)row * a.s_pitch]);
+          }
+          v = silu_f32(g) * u;
+        } else {
+          v = total(o);
+          if constexpr (WF == WF_I8_CHANNEL) v *= T::one(a.s0[(long)row * a.s_pitch]);
+          if (a.add_bias) v += T::one(a.add_bias[row]);
+          if (a.residual) v += T::one(a.residual[(long)tk * n + row]);
+        }
+        y[(long)tk * n + row] = T::pack(v);
+      }
+    }
+    buf ^= 1;
+  }
+}
+
+template <int R, int CH, int EPI, int WF, int TOK>
+static int launch_i8m_rc(hipStream_t s, const SkinnyParams& p, int grid) {
+  Int8MultiArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual};
+#define MUI_I8M_LAUNCH(NORMV)                                                                              \
+  hipLaunchKernelGGL((int8_multi_kernel<R, CH, NORMV, EPI, WF, TOK>), dim3(grid), dim3(kI8mThreads), 0, s,  \
+                     (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k,      \
+                     p.tokens, p.eps, a)
+  if (p.gamma) MUI_I8M_LAUNCH(true); else MUI_I8M_LAUNCH(false);
+#undef MUI_I8M_LAUNCH
+  return launch_status();
+}
+
+template <int EPI, int WF, int TOK>
+static int launch_i8m_t(hipStream_t s, const SkinnyParams& p) {
+  const int ch = ceil_div(p.k >> 4, kI8mThreads);
+  if (ch <= 1) {
+    // short rows: 8 rows in flight at 2 tokens, 4 at 4 (at most 32 partial sums per group)
+    constexpr int R = (TOK <= 2) ? 8 : 4;
+    constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
+    return launch_i8m_rc<R, 1, EPI, WF, TOK>(s, p, balanced_grid(ceil_div(p.n, OUT), 3));
+  }
+  constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
+  const int grid = balanced_grid(ceil_div(p.n, OUT), 2);
+  if (ch <= 2) return launch_i8m_rc<R, 2, EPI, WF, TOK>(s, p, grid);
+  if (ch <= 4) return launch_i8m_rc<R, 4, EPI, WF, TOK>(s, p, grid);
+  return MUI_ERR_UNSUPPORTED;
+}
+
+int launch_int8_multi(hipStream_t s, int dtype, int wf, int epilogue, const SkinnyParams& p) {
+  if (dtype != MUI_DTYPE_F16 || p.tokens < 2 || p.tokens > 4) return MUI_ERR_UNSUPPORTED;
+  if (p.mul_bias) return MUI_ERR_UNSUPPORTED;
+#define MUI_I8M_CASE(WFV, EPIV)                                          \
+  if (wf == WFV && epilogue == EPIV) {                                   \
+    if (p.tokens <= 2) return launch_i8m_t<EPIV, WFV, 2>(s, p);          \
+    return launch_i8m_t<EPIV, WFV, 4>(s, p);                             \
+  }
+  MUI_I8M_CASE(WF_I8_CHANNEL, SK_LINEAR)
+  MUI_I8M_CASE(WF_I8_CHANNEL, SK_GATEUP)
+  MUI_I8M_CASE(WF_U8_GROUP, SK_LINEAR)
+  MUI_I8M_CASE(WF_U8_GROUP, SK_GATEUP)
+#undef MUI_I8M_CASE
+  return MUI_ERR_UNSUPPORTED;
+}
+
+}  // namespace mui
