@@ -292,6 +292,8 @@ int mui_embedding(mui_stream_t stream, int dtype, const void* table, long row_pi
  * (csrc/linear/linear_fp16_kernels.cu:646-654).
  * ---------------------------------------------------------------------------------- */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
+/* rows_per_group 16 / 17 instead switch the packed-dot kernel for a single fp16 token on
+ * (default) / off */
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the

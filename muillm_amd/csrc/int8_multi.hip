@@ -252,10 +252,11 @@ static int launch_i8m_t(hipStream_t s, const SkinnyParams& p) {
 }
 
 int launch_int8_multi(hipStream_t s, int dtype, int wf, int epilogue, const SkinnyParams& p) {
-  if (dtype != MUI_DTYPE_F16 || p.tokens < 2 || p.tokens > 4) return MUI_ERR_UNSUPPORTED;
+  if (dtype != MUI_DTYPE_F16 || p.tokens < 1 || p.tokens > 4) return MUI_ERR_UNSUPPORTED;
   if (p.mul_bias) return MUI_ERR_UNSUPPORTED;
 #define MUI_I8M_CASE(WFV, EPIV)                                          \
   if (wf == WFV && epilogue == EPIV) {                                   \
+    if (p.tokens <= 1) return launch_i8m_t<EPIV, WFV, 1>(s, p);          \
     if (p.tokens <= 2) return launch_i8m_t<EPIV, WFV, 2>(s, p);          \
     return launch_i8m_t<EPIV, WFV, 4>(s, p);                             \
   }

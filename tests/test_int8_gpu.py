@@ -88,7 +88,7 @@ def test_channel_gateup(n, k, tokens, packed):
     else:
         a = (qg.to(DEV), qu.to(DEV), sg.to(DEV), su.to(DEV))
     h = muillm_ext.mui_int8_channel_gateupsilu_forward(gamma.to(DEV), 1e-5, a[0], a[1], a[2], a[3], x.to(DEV))
-    assert_parity(h, ref, 1e-2, f"int8 gateup {n}x{k}", tight=6e-3 if tokens == 1 else 9e-3)
+    assert_parity(h, ref, 1e-2, f"int8 gateup {n}x{k}", tight=9e-3)  # activations enter the packed dot rounded to fp16
 
 
 def test_channel_closed_forms():
@@ -161,7 +161,7 @@ def test_group_gateup(n, k, gs):
     packed_w = torch.stack([qg, qu], dim=1).to(DEV)                                   # [N, 2, K]
     packed_s = torch.stack([smg.reshape(n, ng, 2), smu.reshape(n, ng, 2)], dim=1).to(DEV)  # [N, 2, G, 2]
     h = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, packed_w, packed_s, shift, x.to(DEV))
-    assert_parity(h, ref, 1e-2, f"int8 group gateup {n}x{k}", tight=6e-3)
+    assert_parity(h, ref, 1e-2, f"int8 group gateup {n}x{k}", tight=9e-3)
     dg, du = muillm_ext.muillm_int8_gateupsilu_dequantize_forward(packed_w, packed_s, shift)
     assert torch.equal(dg.cpu(), oracle.rtn_dequantize_group(qg, smg, gs))
     assert torch.equal(du.cpu(), oracle.rtn_dequantize_group(qu, smu, gs))
