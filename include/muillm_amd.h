@@ -291,6 +291,8 @@ int mui_embedding(mui_stream_t stream, int dtype, const void* table, long row_pi
  * have no counterpart in the reference, whose launch shapes are compile-time constants
  * (csrc/linear/linear_fp16_kernels.cu:646-654).
  * ---------------------------------------------------------------------------------- */
+/* rows_per_group 16 / 17 instead switch the packed-dot kernel for a single fp16 token of
+ * mui_linear on (default) / off */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
 /* rows_per_group 16 / 17 instead switch the packed-dot kernel for a single fp16 token on
  * (default) / off */

@@ -265,6 +265,12 @@ using namespace mui;
 
 // token count from which the MFMA skinny-GEMM kernel takes over (below: one GEMV per token)
 static int g_skinny_min_tokens = 2;
+// A single fp16 token of a plain linear also takes the packed-dot kernel of gemv_multi.hip
+// (gamma * x rounded once to fp16 like HuggingFace's normalised activations, half the multiply
+// instructions, half the operand registers): o_proj 8.2 -> 7.0 us, down 20.9 -> 19.2 us, decode
+// +3 % on MI355X. The gate/up kernel measured slower that way (36.2 vs 35.5 us) and stays on
+// gemv_kernel, as does bf16.
+static int g_gemv_dot2 = 1;
 // largest token count that takes the multi-token GEMV (gemv_multi.hip) instead of the MFMA kernel
 static int g_multi_max_tokens = 8;
 
@@ -279,6 +285,7 @@ extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_token
 }
 
 extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
+  if (rows_linear == 16 || rows_linear == 17) { g_gemv_dot2 = rows_linear == 16; return MUI_OK; }
   if (!(rows_linear == 0 || rows_linear == 2 || rows_linear == 4)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_tune.rows_linear = rows_linear;
@@ -301,7 +308,7 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
-  if (tokens >= g_skinny_min_tokens) {
+  if (tokens >= g_skinny_min_tokens || (g_gemv_dot2 && dtype == MUI_DTYPE_F16)) {
     SkinnyParams sp = {};
     sp.w0 = weights;
     sp.pitch = w_pitch;
@@ -319,7 +326,7 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
       const int st = launch_gemv_multi(s, dtype, SK_LINEAR, sp);
       if (st != MUI_ERR_UNSUPPORTED) return st;
     }
-    return launch_skinny(s, dtype, WF_16BIT, SK_LINEAR, sp);
+    if (tokens >= g_skinny_min_tokens) return launch_skinny(s, dtype, WF_16BIT, SK_LINEAR, sp);
   }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     GemvParams p;

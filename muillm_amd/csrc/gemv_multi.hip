@@ -206,9 +206,10 @@ static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
 }
 
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p) {
-  if (p.tokens < 2 || p.tokens > 8) return MUI_ERR_UNSUPPORTED;
+  if (p.tokens < 1 || p.tokens > 8) return MUI_ERR_UNSUPPORTED;
 #define MUI_MT_CASE(TT, EPIV)                                            \
   if (epilogue == EPIV) {                                                \
+    if (p.tokens <= 1) return launch_mt_t<TT, EPIV, 1>(s, p);            \
     if (p.tokens <= 2) return launch_mt_t<TT, EPIV, 2>(s, p);            \
     if (p.tokens <= 4) return launch_mt_t<TT, EPIV, 4>(s, p);            \
     return launch_mt_t<TT, EPIV, 8>(s, p);                               \
