@@ -189,8 +189,10 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
       const int tok = base + u * kWorkers + wk;
       valid[u] = (tok < t_end) && (tok != slot);
       const int tk = valid[u] ? tok : t_begin;  // t_begin < S: always a readable row
-      kreg[u] = ld16_stream(kc + (long)tk * p.c_ts);
-      vreg[u] = ld16_stream(vc + (long)tk * p.c_ts);
+      // split (long) sequences stream K/V once: non-temporal; the unsplit short case re-reads
+      // rows that the previous steps left in cache
+      kreg[u] = ld16_sel<!DIRECT>(kc + (long)tk * p.c_ts);
+      vreg[u] = ld16_sel<!DIRECT>(vc + (long)tk * p.c_ts);
       if (mrow != nullptr && valid[u]) {
         if (T::one(mrow[tok]) != 0.f) valid[u] = false;
       }
