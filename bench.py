@@ -98,6 +98,19 @@ def bench_int8_variant(config, steps, warmup):
             "format": "int8 per output channel + fp16 scale; lm_head fp16"}
 
 
+def measured_copy_ceiling():
+    """Device-to-device copy rate (read + write bytes per second) of torch's copy over 1 GiB
+    buffers, rotating over 3 source/destination pairs: a practical HBM ceiling to hold the
+    8 TB/s datasheet figure against."""
+    import torch
+
+    n = 1 << 29  # fp16 elements = 1 GiB
+    src = [torch.empty(n, device="cuda", dtype=torch.float16).fill_(1.0) for _ in range(3)]
+    dst = [torch.empty(n, device="cuda", dtype=torch.float16) for _ in range(3)]
+    us = _event_time_us(lambda i: dst[i % 3].copy_(src[i % 3]), iters=12, warm=3)
+    return round(2 * n * 2 / us / 1e3, 1)
+
+
 def gateup_roofline(lm):
     """Average launch duration of the fused gate/up+SiLU GEMV over the model's 32 distinct
     (cold) weight buffers, HIP events on the launch stream."""
@@ -414,6 +427,7 @@ def main():
         },
     }
     result["roofline"] = gateup_roofline(lm)
+    result["roofline"]["measured_copy_ceiling_GB/s"] = measured_copy_ceiling()
     if not args.no_kernel_table:
         result["kernels"] = kernel_table(lm)
     del dec
