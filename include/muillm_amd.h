@@ -41,7 +41,7 @@ extern "C" {
 #define MUI_DTYPE_BF16 1
 
 /* largest token batch the decode kernels accept in one call */
-#define MUI_MAX_TOKENS 8
+#define MUI_MAX_TOKENS 16
 
 typedef void* mui_stream_t; /* a hipStream_t; NULL is the default stream */
 

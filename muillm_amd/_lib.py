@@ -18,7 +18,7 @@ HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "muillm_amd.h")
 MUI_OK = 0
 MUI_DTYPE_F16 = 0
 MUI_DTYPE_BF16 = 1
-MUI_MAX_TOKENS = 8
+MUI_MAX_TOKENS = 16
 
 
 class MuiDeviceInfo(ctypes.Structure):

@@ -251,7 +251,7 @@ def muillm_gateupsilu_forward(engine, norm_weights, epsilon, gate_weights, up_we
                               residual, x) -> torch.Tensor:
     """out = Wd (silu(Wg xn) * (Wu xn)) + residual, argument order of csrc/module.cpp:182."""
     if not (kernel_dispatchable(x) and gate_weights.dtype == x.dtype):
-        raise RuntimeError("muillm_gateupsilu_forward needs 1..8 tokens of a 16-bit CUDA tensor")
+        raise RuntimeError("muillm_gateupsilu_forward needs 1..16 tokens of a 16-bit CUDA tensor")
     h = mui_gateup_silu(norm_weights, epsilon, gate_weights, up_weights, x)
     return muillm_linear_forward(engine, h, down_weights, residual=residual)
 

@@ -51,7 +51,7 @@ def test_channel_dequant_bit_exact(n, k):
 
 
 @pytest.mark.parametrize("n,k", SHAPES)
-@pytest.mark.parametrize("tokens", [1, 4])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("norm", [True, False])
 def test_channel_linear(n, k, tokens, norm):
     g = _gen(1)
@@ -71,7 +71,7 @@ def test_channel_linear(n, k, tokens, norm):
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (300, 1024), (5, 16)])
-@pytest.mark.parametrize("tokens", [1, 4])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("packed", [True, False])
 def test_channel_gateup(n, k, tokens, packed):
     g = _gen(2)
@@ -129,7 +129,7 @@ def test_group_dequant_bit_exact(n, k, gs):
 
 
 @pytest.mark.parametrize("n,k,gs", [(4096, 4096, 128), (4096, 14336, 1024), (6144, 4096, 64), (50, 256, 16)])
-@pytest.mark.parametrize("tokens", [1, 4])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 7, 16])
 def test_group_linear(n, k, gs, tokens):
     g = _gen(5)
     w = _mk((n, k), g, 0.02)

@@ -135,7 +135,7 @@ def test_linear_strided_weights():
         assert_parity(y, oracle.linear(x, big[:, s, :]), 1e-2, f"strided {s}", tight=4e-3)
 
 
-@pytest.mark.parametrize("tokens", [2, 3, 4, 8])
+@pytest.mark.parametrize("tokens", [2, 3, 4, 5, 8, 13, 16])
 @pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (100, 512)])
 def test_linear_small_batch(tokens, n, k):
     g = _gen(4)
@@ -171,7 +171,7 @@ def test_linear_abi_errors():
     assert lib.mui_linear(s, 0, None, 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 1) == -1
     assert lib.mui_linear(s, 7, w.data_ptr(), 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 1) == -1
     assert lib.mui_linear(s, 0, w.data_ptr(), 12, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 12, 1) == -2
-    assert lib.mui_linear(s, 0, w.data_ptr(), 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 9) == -2
+    assert lib.mui_linear(s, 0, w.data_ptr(), 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 17) == -2
     assert lib.mui_linear(s, 0, w.data_ptr() + 2, 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 4, 8, 1) == -4
     assert b"aligned" in lib.mui_status_string(-4)
     with pytest.raises(RuntimeError):
@@ -237,7 +237,7 @@ def test_gateup_silu(n, k, norm, packed):
     assert_parity(h, ref, 1e-2, f"gateup {n}x{k}", tight=6e-3)
 
 
-@pytest.mark.parametrize("tokens", [1, 2, 4, 8])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 8, 16])
 def test_mlp_config2(tokens):
     """Config 2: Mistral-7B-shaped MLP with fused norm and residual."""
     g = _gen(8)
