@@ -53,14 +53,14 @@ def _event_time_us(fn, iters, warm):
     return s.elapsed_time(e) * 1e3 / iters
 
 
-def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=True):
+def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=True, batch=1):
     import torch
 
     from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
 
     dev = "cuda"
     g = torch.Generator().manual_seed(0)
-    ids = torch.randint(0, lm.config.vocab_size, (1, prompt_len), generator=g).to(dev)
+    ids = torch.randint(0, lm.config.vocab_size, (batch, prompt_len), generator=g).to(dev)
     dec = MuiGraphDecoder(lm, use_graph=use_graph)
     dec.prefill(ids, steps + warmup + 1)
     dec.decode(warmup)  # captures the graph on first use, then W untimed replays
@@ -435,6 +435,11 @@ def main():
         dt_e, dec_e = bench_decode(lm, min(args.steps, 64), min(args.warmup, 8), use_graph=False)
         result["variants"] = {"fp16_eager_no_graph_tokens_per_s": round(min(args.steps, 64) / dt_e, 2)}
         del dec_e
+        for bsz in (4, 8):
+            dt_b, dec_b = bench_decode(lm, min(args.steps, 128), min(args.warmup, 8), batch=bsz)
+            result["variants"]["fp16_batch%d_aggregate_tokens_per_s" % bsz] = round(bsz * min(args.steps, 128) / dt_b, 1)
+            result["variants"]["fp16_batch%d_ms_per_step" % bsz] = round(dt_b / min(args.steps, 128) * 1e3, 4)
+            del dec_b
         del lm
         torch.cuda.empty_cache()
         result["variants"]["int8"] = bench_int8_variant(config, args.steps, args.warmup)
