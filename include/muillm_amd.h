@@ -238,6 +238,19 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
                           void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
                           int max_cache_len);
 
+/* Causal attention of `tokens` > 1 new query tokens per batch row (prefill, or a chunk of it)
+ * over a static cache that already holds their rotated keys and values:
+ *   out[b, t, h*D:(h+1)*D] = softmax_{s <= q_start + t}(q[b,h,t,:] . K[b, h/(Hq/Hkv), s, :] / sqrt(D)) V[...]
+ * q_rotated is dense [batch, n_q_heads, tokens, head_dim] (what mui_rope_kv_write produces), query t
+ * sits at key position q_start + t, keys are cache rows [0, seq_len), q_start + tokens <= seq_len.
+ * The reference hands T > 1 to torch's scaled_dot_product_attention
+ * (muillm/modules/attention/sdpaattention.py:221-245) after repeat_kv; here K/V are read per KV
+ * head and no mask tensor is built. No padding mask: padded batches keep the SDPA route. */
+int mui_prefill_attention(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
+                          const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                          long cache_token_stride, int seq_len, int q_start, void* out, int batch,
+                          int n_q_heads, int n_kv_heads, int tokens, int head_dim);
+
 /* Greedy token choice: out_index[r] = argmax_v logits[r, v] (lowest index on ties, NaN never
  * wins) for a 16-bit [rows, vocab] matrix with row pitch row_stride elements. Stands in for
  * the torch.argmax of the reference's greedy sampling branch

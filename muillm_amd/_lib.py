@@ -66,6 +66,8 @@ _SIGNATURES = {
     "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, _P,
                                       c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
                                       _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mui_prefill_attention": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, c_int, c_int, _P, c_int, c_int,
+                                      c_int, c_int, c_int]),
     "mui_argmax": (c_int, [_P, c_int, _P, c_long, _P, c_int, c_int]),
     "mui_greedy_advance": (c_int, [_P, c_int, _P, c_long, c_int, c_int, _P, _P, _P, _P, _P, c_long, c_int, _P, _P,
                                    c_int, c_long]),

@@ -637,6 +637,191 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Causal attention for T > 1 new tokens (prefill) on the matrix cores: the same formulation as
+// attn_decode_mfma_kernel with the 16 MFMA columns holding 16 consecutive QUERY POSITIONS of one
+// head instead of the heads of a group. grid = (ceil(T / 16), Hq, B), 4 waves; every wave walks
+// 32-token K/V blocks of the causal range [0, q_start + t0 + 16) and the waves are merged through
+// LDS. q is already rotated ([B, Hq, T, D] dense, as rope_kv_write_kernel leaves it) and the new
+// K/V rows are already in the cache. The reference hands this case to torch SDPA
+// (muillm/modules/attention/sdpaattention.py:221-245).
+// ---------------------------------------------------------------------------------------
+struct PrefillParams {
+  const uint16_t* q;        // [B, Hq, T, D]
+  const uint16_t* k_cache;  // [B, Hkv, >= S, D] by strides
+  const uint16_t* v_cache;
+  long c_bs, c_hs, c_ts;
+  uint16_t* out;            // [B, T, Hq * D]
+  int hq, hkv, tokens, seq_len, q_start;  // query t sits at key position q_start + t; keys [0, seq_len)
+  float scale_log2;
+};
+
+template <typename T, int NW>
+__global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const PrefillParams p) {
+  constexpr int kAttnThreads = NW * kWave;
+  constexpr int kBlock = NW * kMfTok;
+  __shared__ __attribute__((aligned(16))) uint16_t q_lds[16][kHeadDim];
+  __shared__ float lds_m[NW][16];
+  __shared__ float lds_l[NW][16];
+  constexpr int kVBytes = NW * kMfTok * kMfVStride * 2;
+  constexpr int kMergeBytes = NW * 16 * kHeadDim * 4;
+  __shared__ __attribute__((aligned(16))) char big_lds[kVBytes > kMergeBytes ? kVBytes : kMergeBytes];
+  uint16_t (*v_lds)[kMfVStride] = (uint16_t (*)[kMfVStride])(big_lds + (size_t)(threadIdx.x >> 6) * kMfTok * kMfVStride * 2);
+  float (*tile)[16][kHeadDim] = (float (*)[16][kHeadDim])big_lds;
+
+  const int t0 = blockIdx.x * 16, head = blockIdx.y, b = blockIdx.z;
+  const int kvh = head / (p.hq / p.hkv);
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int g = lane >> 4;
+  const int i = lane & 15;
+
+  // keys this tile can see: [0, kv_end); column i (query t0 + i) sees tokens < limit_i
+  int kv_end = p.q_start + t0 + 16;
+  kv_end = kv_end < p.seq_len ? kv_end : p.seq_len;
+  const bool col_ok = (t0 + i) < p.tokens;
+  int limit_i = p.q_start + t0 + i + 1;
+  limit_i = limit_i < p.seq_len ? limit_i : p.seq_len;
+  if (!col_ok) limit_i = 0;
+
+  const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
+  const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
+
+  struct Block {
+    u32x4 k[2][4];
+    u32x4 v[8];
+  };
+  auto load_block = [&](int base, Block& q) {
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int tok = base + 16 * h2 + i;
+      const uint16_t* rp = kc + (long)(tok < kv_end ? tok : 0) * p.c_ts + g * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q.k[h2][j] = ld16(rp + j * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int tok = base + 4 * u + g;
+      q.v[u] = ld16(vc + (long)(tok < kv_end ? tok : 0) * p.c_ts + i * 8);
+    }
+  };
+
+  Block ba, bb;
+  int base = wave * kMfTok;
+  bool have_a = base < kv_end;
+  if (have_a) load_block(base, ba);
+
+  for (int e = t; e < 16 * kHeadDim; e += kAttnThreads) {
+    const int qi = e / kHeadDim, d = e % kHeadDim;
+    uint16_t r = 0;
+    if (t0 + qi < p.tokens) r = p.q[(((long)b * p.hq + head) * p.tokens + t0 + qi) * kHeadDim + d];
+    q_lds[qi][d] = r;
+  }
+  __syncthreads();
+  u32x4 qreg[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) qreg[j] = *(const u32x4*)&q_lds[i][(g + 4 * j) * 8];
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto attend = [&](int base, Block& q) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
+    f32x4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      s1 = attn_mfma<T>(q.k[0][j], qreg[j], s1);
+      s2 = attn_mfma<T>(q.k[1][j], qreg[j], s2);
+    }
+    float sc[8];
+    float m_loc = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
+      const float raw = r < 4 ? s1[r] : s2[r - 4];
+      sc[r] = tok < limit_i ? raw * p.scale_log2 : -INFINITY;
+      m_loc = fmaxf(m_loc, sc[r]);
+    }
+    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
+    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+    const float m_new = fmaxf(m, m_loc);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = fast_exp2(m - m_use);
+    float pr[8];
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      pr[r] = fast_exp2(sc[r] - m_use);
+      psum += pr[r];
+    }
+    l = fmaf(l, corr, psum);
+    m = m_new;
+    u32x4 pb;
+    pb.x = (uint32_t)T::pack(pr[0]) | ((uint32_t)T::pack(pr[1]) << 16);
+    pb.y = (uint32_t)T::pack(pr[2]) | ((uint32_t)T::pack(pr[3]) << 16);
+    pb.z = (uint32_t)T::pack(pr[4]) | ((uint32_t)T::pack(pr[5]) << 16);
+    pb.w = (uint32_t)T::pack(pr[6]) | ((uint32_t)T::pack(pr[7]) << 16);
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const u32x2 lo = lds_read_tr16(&v_lds[4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x2 hi = lds_read_tr16(&v_lds[16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+      f32x4 a = acc[db];
+      a.x *= corr; a.y *= corr; a.z *= corr; a.w *= corr;
+      acc[db] = attn_mfma<T>(va, pb, a);
+    }
+  };
+
+  for (;;) {
+    if (!have_a) break;
+    const int nb = base + kBlock;
+    const bool have_b = nb < kv_end;
+    if (have_b) load_block(nb, bb);
+    attend(base, ba);
+    if (!have_b) break;
+    base = nb + kBlock;
+    have_a = base < kv_end;
+    if (have_a) load_block(base, ba);
+    attend(nb, bb);
+  }
+
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+
+  __syncthreads();
+  if (g == 0) lds_m[wave][i] = m;
+  __syncthreads();
+  float mx = -INFINITY;
+#pragma unroll
+  for (int w2 = 0; w2 < NW; ++w2) mx = fmaxf(mx, lds_m[w2][i]);
+  const float f = fast_exp2(m - ((mx == -INFINITY) ? 0.f : mx));
+  if (g == 0) lds_l[wave][i] = l * f;
+#pragma unroll
+  for (int db = 0; db < 8; ++db) {
+    f32x4 o = acc[db];
+    o.x *= f; o.y *= f; o.z *= f; o.w *= f;
+    *(f32x4*)&tile[wave][i][16 * db + 4 * g] = o;
+  }
+  __syncthreads();
+
+  for (int e = t; e < 16 * kHeadDim; e += kAttnThreads) {
+    const int qi = e / kHeadDim, d = e % kHeadDim;
+    if (t0 + qi >= p.tokens) continue;
+    float a = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) {
+      a += tile[w2][qi][d];
+      lsum += lds_l[w2][qi];
+    }
+    p.out[((long)b * p.tokens + t0 + qi) * ((long)p.hq * kHeadDim) + (long)head * kHeadDim + d] =
+        T::pack(lsum > 0.f ? a / lsum : 0.f);
+  }
+}
+
 // log-sum-exp merge of the per-split partials: one workgroup of 128 threads per (head, batch).
 // The split weights are computed once into LDS; the accumulation loop then has no dependent
 // loads, so the partial rows of all splits are in flight together.
@@ -994,5 +1179,35 @@ extern "C" int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, 
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MUI_DTYPE_F16) hipLaunchKernelGGL((rope_kv_write_kernel<F16>), grid, block, 0, s, p);
   else hipLaunchKernelGGL((rope_kv_write_kernel<BF16>), grid, block, 0, s, p);
+  return launch_status();
+}
+
+extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
+                                     const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                     long cache_token_stride, int seq_len, int q_start, void* out, int batch,
+                                     int n_q_heads, int n_kv_heads, int tokens, int head_dim) {
+  MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
+  MUI_CHECK_ARG(q_rotated && k_cache && v_cache && out);
+  MUI_CHECK_ARG(batch > 0 && n_q_heads > 0 && n_kv_heads > 0 && tokens > 0 && seq_len > 0 && q_start >= 0);
+  MUI_CHECK_ARG(q_start + tokens <= seq_len);
+  if (head_dim != kHeadDim) return MUI_ERR_UNSUPPORTED;
+  if (n_q_heads % n_kv_heads != 0) return MUI_ERR_INVALID_ARG;
+  if (batch > 65535 || n_q_heads > 65535) return MUI_ERR_UNSUPPORTED;
+  if ((cache_token_stride & 7) || (cache_head_stride & 7) || (cache_batch_stride & 7)) return MUI_ERR_ALIGNMENT;
+  if (!aligned16(k_cache) || !aligned16(v_cache)) return MUI_ERR_ALIGNMENT;
+  PrefillParams p = {};
+  p.q = (const uint16_t*)q_rotated;
+  p.k_cache = (const uint16_t*)k_cache;
+  p.v_cache = (const uint16_t*)v_cache;
+  p.c_bs = cache_batch_stride; p.c_hs = cache_head_stride; p.c_ts = cache_token_stride;
+  p.out = (uint16_t*)out;
+  p.hq = n_q_heads; p.hkv = n_kv_heads; p.tokens = tokens; p.seq_len = seq_len; p.q_start = q_start;
+  p.scale_log2 = kLog2e / sqrtf((float)head_dim);
+  dim3 grid(ceil_div(tokens, 16), n_q_heads, batch);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MUI_DTYPE_F16)
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4>), grid, dim3(4 * kWave), 0, s, p);
+  else
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<BF16, 4>), grid, dim3(4 * kWave), 0, s, p);
   return launch_status();
 }

@@ -212,6 +212,7 @@ struct Tuning {
   int wgs_per_cu = 0;   // 0 = pick per shape; else cap on workgroups per CU for persistent grids
 };
 static Tuning g_tune;
+int gemv_tuned_wgs_per_cu() { return g_tune.wgs_per_cu; }  // shared with gemv_multi.hip
 
 template <typename T, int R, int CH, int EPI>
 static int launch_rc(hipStream_t s, const GemvParams& p, int grid) {

@@ -193,12 +193,14 @@ static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
   } else {
   if (ch <= 2) {
     constexpr int R = 4, OUT = (EPI == SK_GATEUP) ? 2 : 4;
-    const int grid = balanced_grid(ceil_div(p.n, OUT), 3);
+    const int tuned = gemv_tuned_wgs_per_cu();
+    const int grid = balanced_grid(ceil_div(p.n, OUT), tuned > 0 ? tuned : 3);
     if (ch <= 1) return launch_mt_rc<T, R, 1, EPI, TOK>(s, p, grid);
     return launch_mt_rc<T, R, 2, EPI, TOK>(s, p, grid);
   }
   constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
-  const int grid = balanced_grid(ceil_div(p.n, OUT), 2);
+  const int tuned = gemv_tuned_wgs_per_cu();
+  const int grid = balanced_grid(ceil_div(p.n, OUT), tuned > 0 ? tuned : 2);
   if (ch <= 4) return launch_mt_rc<T, R, 4, EPI, TOK>(s, p, grid);
   if (ch <= 7) return launch_mt_rc<T, R, 7, EPI, TOK>(s, p, grid);
   return MUI_ERR_UNSUPPORTED;

@@ -68,6 +68,7 @@ void skinny_set_bstat(int on);
 // 2..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
 // in registers (gemv_multi.hip); returns MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
+int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 = built-in)
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 void skinny_set_int8_multi(int on);

@@ -4,6 +4,8 @@ from typing import Optional, Tuple
 
 import torch
 
+from ... import muillm_ext
+
 from .baseattention import MuiBaseAttention
 from .kvcache import repeat_kv
 
@@ -27,6 +29,23 @@ def _ignore_causal_mask_sdpa(attention_mask: Optional[torch.Tensor], inputs_shap
 
 
 class MuiSdpaAttention(MuiBaseAttention):
+    # measured on MI355X (32/8 heads x 128): 10 vs 38 us at 32 tokens, 44 vs 59 us at 512, 324 vs 180 us at 2048
+    prefill_kernel_max_tokens = 1024
+
+    def _prefill_kernel_ok(self, q, k, v, attention_mask, all_ones_mask, q_len) -> bool:
+        """T > 1 without padding (the mask, if any, is purely causal), 16-bit CUDA tensors,
+        head_dim 128, K/V being equally strided views with unit inner stride (the static cache)."""
+        if q_len <= 1 or not (all_ones_mask or attention_mask is None):
+            return False
+        if not (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype):
+            return False
+        if self.head_dim != 128 or k.shape[2] < q_len or self.training:
+            return False
+        if q_len > self.prefill_kernel_max_tokens:
+            return False  # long prompts: torch's flash attention is about 2x faster beyond ~1k tokens
+        return (k.stride() == v.stride() and k.stride(3) == 1 and all(st % 8 == 0 for st in k.stride()[:3])
+                and k.data_ptr() % 16 == 0 and v.data_ptr() % 16 == 0)
+
     def forward(self, query_states: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor,
                 attention_mask: Optional[torch.Tensor] = None, position_ids: Optional[torch.LongTensor] = None,
                 past_key_value=None, output_attentions: bool = False, use_cache: bool = False,
@@ -51,6 +70,9 @@ class MuiSdpaAttention(MuiBaseAttention):
             q, k, v = self.rotary_emb.apply_rotary_pos_emb_write_kv_cache(
                 q, k, position_ids, position_embeddings, v, past_key_value, cache_position)
             attn_output = self._decode_or_none(q, k, v, attention_mask, all_ones_mask, q_len)
+            if attn_output is None and self._prefill_kernel_ok(q, k, v, attention_mask, all_ones_mask, q_len):
+                # causal attention of the new tokens over the cache views that already hold them
+                attn_output = muillm_ext.mui_prefill_attention(q, k, v)
             if attn_output is None:
                 k = repeat_kv(k, self.num_key_value_groups)
                 v = repeat_kv(v, self.num_key_value_groups)

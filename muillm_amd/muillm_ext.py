@@ -884,3 +884,29 @@ def muillm_embedding_forward(engine, weights: torch.Tensor, x: torch.Tensor) -> 
 
 def muillm_embedding_module_forward(module: MuiEmbeddingModule, x: torch.Tensor) -> torch.Tensor:
     return muillm_embedding_forward(module.engine, module.weights, x)
+
+
+def mui_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_start: Optional[int] = None) -> torch.Tensor:
+    """Causal attention of T > 1 new tokens over cache views that already contain them.
+
+    q [B, Hq, T, D] rotated (made dense if it is not), k/v [B, Hkv, S, D] views of the static cache
+    (unit inner stride, equal strides); query t sits at key position q_start + t (default S - T).
+    Returns [B, T, Hq * D]."""
+    _check_cuda(q, "q")
+    _check_cuda(k, "k")
+    _check_cuda(v, "v")
+    b, hq, t, d = q.shape
+    hkv, s = k.shape[1], k.shape[2]
+    if q_start is None:
+        q_start = s - t
+    if q_start < 0 or q_start + t > s:
+        raise RuntimeError("the new tokens must lie inside the key sequence")
+    qc = q.contiguous()
+    cb, chs, cts = _cache_strides(k, v)
+    out = torch.empty((b, t, hq * d), dtype=q.dtype, device=q.device)
+    check(
+        _lib.load().mui_prefill_attention(_stream(qc), _dtype_code(qc), qc.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                          cb, chs, cts, s, int(q_start), out.data_ptr(), b, hq, hkv, t, d),
+        "mui_prefill_attention",
+    )
+    return out

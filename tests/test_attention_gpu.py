@@ -294,6 +294,57 @@ def test_fused_decode_sequence_matches_oracle_steps():
     assert (kd.cpu()[:, :, :seen].float() - kc[:, :, :seen].float()).abs().max() <= 8e-3
 
 
+# ------------------------------------------------------------------------------------
+# causal attention of T > 1 new tokens (prefill)
+# ------------------------------------------------------------------------------------
+def _causal_mask(t, s, q_start):
+    m = torch.zeros(1, 1, t, s, dtype=torch.float64)
+    key = torch.arange(s)[None, :]
+    qry = q_start + torch.arange(t)[:, None]
+    m[0, 0][key > qry] = float("-inf")
+    return m
+
+
+@pytest.mark.parametrize("b,hq,hkv,t,past", [
+    (1, 32, 8, 32, 0), (2, 8, 2, 5, 0), (1, 32, 8, 16, 100), (1, 4, 4, 77, 3), (3, 16, 2, 33, 31), (1, 32, 8, 300, 0),
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_prefill_attention(b, hq, hkv, t, past, dtype):
+    g = _gen(21)
+    s = past + t
+    cap = oracle.next_pow2(s)
+    q = _mk((b, hq, t, D), g, dtype=dtype)
+    kc = _mk((b, hkv, cap, D), g, dtype=dtype)
+    vc = _mk((b, hkv, cap, D), g, dtype=dtype)
+    kc[:, :, s:] = float("nan")  # rows beyond the sequence must never be read
+    vc[:, :, s:] = float("nan")
+    ref = oracle.decode_attention(q, kc[:, :, :s], vc[:, :, :s], _causal_mask(t, s, past))
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = muillm_ext.mui_prefill_attention(q.to(DEV), kd[:, :, :s], vd[:, :, :s])
+    assert out.shape == (b, t, hq * D) and torch.isfinite(out).all()
+    assert _max_abs(out, ref) <= (ATOL if dtype == torch.float16 else 1.6e-2)
+
+
+def test_prefill_attention_closed_forms():
+    g = _gen(22)
+    hq, hkv, t = 8, 2, 40
+    q = _mk((1, hq, t, D), g).to(DEV)
+    k = _mk((1, hkv, t, D), g).to(DEV)
+    v = _mk((1, hkv, t, D), g).to(DEV)
+    out = muillm_ext.mui_prefill_attention(q, k, v).view(t, hq, D)
+    # the first query sees only key 0 -> its value, exactly
+    assert torch.equal(out[0], v[0, :, 0].repeat_interleave(hq // hkv, dim=0))
+    # the last query row equals single-token decoding over the same keys
+    dec = muillm_ext.muillm_causal_transformer_decoding_no_mask(q[:, :, -1:].contiguous(), k, v).view(hq, D)
+    assert (out[-1].float() - dec.float()).abs().max() <= 1e-3
+    # changing a FUTURE key/value must not change earlier rows (causality)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, 30:] += 3.0
+    v2[:, :, 30:] -= 2.0
+    out2 = muillm_ext.mui_prefill_attention(q, k2, v2).view(t, hq, D)
+    assert torch.equal(out2[:30], out[:30]) and not torch.equal(out2[30:], out[30:])
+
+
 def test_attention_abi_errors():
     lib = _lib.load()
     s = torch.cuda.current_stream().cuda_stream
