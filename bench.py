@@ -442,6 +442,11 @@ def main():
             del dec_b
         del lm
         torch.cuda.empty_cache()
+        lm_bf = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.bfloat16, device="cuda", seed=0)
+        dt_bf, dec_bf = bench_decode(lm_bf, args.steps, args.warmup)
+        result["variants"]["bf16_tokens_per_s"] = round(args.steps / dt_bf, 2)
+        del dec_bf, lm_bf
+        torch.cuda.empty_cache()
         result["variants"]["int8"] = bench_int8_variant(config, args.steps, args.warmup)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(config)

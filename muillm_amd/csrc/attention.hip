@@ -70,10 +70,10 @@ template <>
 __device__ __forceinline__ float dot2_acc<F16>(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
 }
+typedef __bf16 bf16x2_at __attribute__((ext_vector_type(2)));
 template <>
 __device__ __forceinline__ float dot2_acc<BF16>(uint32_t a, uint32_t b, float c) {
-  c = fmaf(BF16::lo(a), BF16::lo(b), c);
-  return fmaf(BF16::hi(a), BF16::hi(b), c);
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_at, a), __builtin_bit_cast(bf16x2_at, b), c, false);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -50,11 +50,9 @@ struct BF16 {
   static __device__ __forceinline__ float one(uint16_t b) {
     return __builtin_bit_cast(float, ((uint32_t)b) << 16);
   }
+  // fp32 -> bf16, round-to-nearest-even: the hardware convert of gfx950 (v_cvt_pk_bf16_f32)
   static __device__ __forceinline__ uint16_t pack(float v) {
-    uint32_t u = __builtin_bit_cast(uint32_t, v);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)v);
   }
 };
 

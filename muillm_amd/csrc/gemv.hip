@@ -270,7 +270,7 @@ static int g_skinny_min_tokens = 2;
 // (gamma * x rounded once to fp16 like HuggingFace's normalised activations, half the multiply
 // instructions, half the operand registers): o_proj 8.2 -> 7.0 us, down 20.9 -> 19.2 us, decode
 // +3 % on MI355X. The gate/up kernel measured slower that way (36.2 vs 35.5 us) and stays on
-// gemv_kernel, as does bf16.
+// gemv_kernel. bf16 takes the same route with v_dot2_f32_bf16.
 static int g_gemv_dot2 = 1;
 // largest token count that takes the multi-token GEMV (gemv_multi.hip) instead of the MFMA kernel
 static int g_multi_max_tokens = 8;
@@ -309,7 +309,7 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
-  if (tokens >= g_skinny_min_tokens || (g_gemv_dot2 && dtype == MUI_DTYPE_F16)) {
+  if (tokens >= g_skinny_min_tokens || g_gemv_dot2) {
     SkinnyParams sp = {};
     sp.w0 = weights;
     sp.pitch = w_pitch;
@@ -364,7 +364,8 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
-  if (tokens >= g_skinny_min_tokens) {
+  // bf16 has no mixed-precision fma: a single bf16 token takes the packed-dot kernel here too
+  if (tokens >= g_skinny_min_tokens || (g_gemv_dot2 && dtype == MUI_DTYPE_BF16)) {
     SkinnyParams sp = {};
     sp.w0 = gate;
     sp.w1 = up;
@@ -380,7 +381,7 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
       const int st = launch_gemv_multi(s, dtype, SK_GATEUP, sp);
       if (st != MUI_ERR_UNSUPPORTED) return st;
     }
-    return launch_skinny(s, dtype, WF_16BIT, SK_GATEUP, sp);
+    if (tokens >= g_skinny_min_tokens) return launch_skinny(s, dtype, WF_16BIT, SK_GATEUP, sp);
   }
   for (int tkn = 0; tkn < tokens; ++tkn) {
     GemvParams p;

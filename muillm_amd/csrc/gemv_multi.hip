@@ -21,10 +21,10 @@ template <>
 __device__ __forceinline__ float dot2_mt<F16>(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
 }
+typedef __bf16 bf16x2_mt __attribute__((ext_vector_type(2)));
 template <>
 __device__ __forceinline__ float dot2_mt<BF16>(uint32_t a, uint32_t b, float c) {
-  c = fmaf(BF16::lo(a), BF16::lo(b), c);
-  return fmaf(BF16::hi(a), BF16::hi(b), c);
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_mt, a), __builtin_bit_cast(bf16x2_mt, b), c, false);
 }
 
 template <typename T, int R, int CH, bool NORM, int EPI, int TOK>
