@@ -56,3 +56,15 @@ def test_argument_validation_needs_no_gpu():
     assert lib.mui_rmsnorm(None, 0, None, None, 0.0, None, 1, 8) == -1
     assert lib.mui_gateup_silu(None, 0, None, None, 8, None, None, 0.0, None, 8, 8, 1) == -1
     assert lib.mui_device_info(0, None) == -1
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py drives one GPU: any other --gpus value exits with a message (no GPU needed for this)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr
