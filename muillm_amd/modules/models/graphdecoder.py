@@ -48,6 +48,7 @@ class MuiGraphDecoder:
         self.out_tokens = torch.zeros((batch, max_new_tokens), dtype=torch.int64, device=device)
         self.logits = None
         self.mask4d = None  # static additive decode mask [B, 1, 1, capacity] when the prompts are padded
+        self._stop_host = None  # pinned scalar for the sync-free stop check
         self._batch = batch
         self._max_new = max_new_tokens
 
@@ -151,38 +152,61 @@ class MuiGraphDecoder:
             self.pos.fill_(prompt_len - 1)
         self.cpos.fill_(prompt_len - 1)
         self.step.zero_()
-        self.out_tokens.zero_()
+        # columns never reached (early stop) read as padding
+        self.out_tokens.fill_(self.pad_token_id if self.eos is not None else 0)
         self.unfinished.fill_(1)
         self._advance(out.logits[:, -1, :])
         return out.logits[:, -1, :]
 
     @torch.no_grad()
-    def decode(self, n_steps: int, collect_logits: bool = False):
-        """Run n_steps decode steps from the current device state."""
+    def decode(self, n_steps: int, collect_logits: bool = False, stop_check_every: int = 0):
+        """Run up to n_steps decode steps from the current device state.
+
+        stop_check_every > 0 (and an eos criterion): every that many steps the count of unfinished
+        rows is copied to pinned host memory WITHOUT waiting for it; the loop ends once a copy that
+        has already landed reads zero. The host therefore never blocks on the GPU (the reference
+        gets the same effect with its Synchronizer, csrc/sync.cu:16-118, muillm/sampling/generation.py);
+        the few steps issued past the end only write pad tokens."""
         logits_hist = []
-        if self.use_graph:
-            if self.graph is None:
-                self._capture()
-            for _ in range(n_steps):
+        if self.use_graph and self.graph is None:
+            self._capture()
+        if not self.use_graph:
+            self.cache.device_length_mode = False
+        check = stop_check_every > 0 and self.eos is not None
+        pending = None  # (event, pinned host tensor) of the last stop-check copy
+        done = 0
+        for i in range(n_steps):
+            if check and pending is not None and pending[0].query():
+                if int(pending[1].item()) == 0:
+                    break
+                pending = None
+            if self.use_graph:
                 self.graph.replay()
-                if collect_logits:
-                    logits_hist.append(self.logits.clone())
-            self.cache._seen_tokens += n_steps
+                lg = self.logits
+            else:
+                lg = self._step()
+            done += 1
+            if collect_logits:
+                logits_hist.append(lg.clone())
+            if check and pending is None and (i + 1) % stop_check_every == 0:
+                if self._stop_host is None:
+                    self._stop_host = torch.zeros((), dtype=torch.int64, pin_memory=True)
+                self._stop_host.copy_(self.unfinished.sum(), non_blocking=True)
+                ev = torch.cuda.Event()
+                ev.record()
+                pending = (ev, self._stop_host)
+        if self.use_graph:
+            self.cache._seen_tokens += done
             if self.cache.cpp_module is not None:
                 self.cache.cpp_module.seen_tokens = self.cache._seen_tokens
-        else:
-            self.cache.device_length_mode = False
-            for _ in range(n_steps):
-                lg = self._step()
-                if collect_logits:
-                    logits_hist.append(lg.clone())
         return logits_hist
 
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, max_new_tokens: int, cache: Optional[MuiStaticCache] = None,
-                 return_logits: bool = False, attention_mask: Optional[torch.Tensor] = None):
+                 return_logits: bool = False, attention_mask: Optional[torch.Tensor] = None,
+                 stop_check_every: int = 0):
         first_logits = self.prefill(input_ids, max_new_tokens, cache, attention_mask=attention_mask)
-        hist = self.decode(max_new_tokens - 1, collect_logits=return_logits)
+        hist = self.decode(max_new_tokens - 1, collect_logits=return_logits, stop_check_every=stop_check_every)
         tokens = torch.cat([input_ids, self.out_tokens[:, :max_new_tokens]], dim=1)
         if return_logits:
             return tokens, torch.stack([first_logits] + hist, dim=1)

@@ -376,7 +376,9 @@ class MuiLlamaForCausalLM(MuiModule):
             pad_token_id = eos[0] if eos else 0
         dec = MuiGraphDecoder(self, use_graph=use_graph, eos_token_ids=eos, pad_token_id=pad_token_id,
                               do_sample=do_sample, temperature=temperature, seed=seed)
-        return dec.generate(input_ids, max_new_tokens, cache=cache, attention_mask=attention_mask)
+        # with an eos criterion the loop polls, without blocking, whether every row has finished
+        return dec.generate(input_ids, max_new_tokens, cache=cache, attention_mask=attention_mask,
+                            stop_check_every=8 if eos else 0)
 
 
 # Mistral shares the Llama implementation (the reference's mistral/model.py is a renamed copy)

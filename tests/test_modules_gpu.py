@@ -289,6 +289,26 @@ def test_generate_stops_at_eos_and_pads():
         lm.generate(ids, max_new_tokens=2, top_k=5)
 
 
+def test_generate_early_stop_without_host_sync():
+    """When every row has hit an eos token the loop ends early (asynchronous stop check); what it
+    emits is the free-running sequence up to each row's eos, then padding."""
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=10, init_std=0.08)
+    ids = torch.randint(1, cfg.vocab_size, (3, 5), generator=torch.Generator().manual_seed(4)).to(DEV)
+    n_new = 96
+    free = lm.generate(ids, max_new_tokens=n_new).cpu()
+    eos = sorted({int(free[r, 5 + 2]) for r in range(3)})  # every row emits one of these by its 3rd token
+    dec = MuiGraphDecoder(lm, use_graph=True, eos_token_ids=eos, pad_token_id=0)
+    out = dec.generate(ids, n_new, stop_check_every=8).cpu()
+    assert out.shape == free.shape
+    for r in range(3):
+        hits = [i for i in range(n_new) if int(free[r, 5 + i]) in eos]
+        h = hits[0]
+        assert h <= 2
+        assert torch.equal(out[r, : 5 + h + 1], free[r, : 5 + h + 1]) and bool((out[r, 5 + h + 1:] == 0).all())
+    assert dec.cache.get_seq_length() < 5 + n_new - 1   # the loop really stopped before the budget
+
+
 def test_embedding_kernel():
     from muillm_amd.modules.embedding import MuiEmbedding
     g = torch.Generator().manual_seed(11)
