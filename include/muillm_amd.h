@@ -304,11 +304,11 @@ int mui_embedding(mui_stream_t stream, int dtype, const void* table, long row_pi
  * have no counterpart in the reference, whose launch shapes are compile-time constants
  * (csrc/linear/linear_fp16_kernels.cu:646-654).
  * ---------------------------------------------------------------------------------- */
-/* rows_per_group 16 / 17 instead switch the packed-dot kernel for a single fp16 token of
- * mui_linear on (default) / off */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
-/* rows_per_group 16 / 17 instead switch the packed-dot kernel for a single fp16 token on
- * (default) / off */
+/* single-token routing: linear_on -> mui_linear (and bf16 mui_gateup_silu) through the packed-dot
+ * kernel of the multi-token GEMV (default on); int8_on -> a single fp16 token of the int8 entry
+ * points through the packed-dot int8 kernel (default on) */
+int mui_tune_packed_dot(int linear_on, int int8_on);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the

@@ -75,6 +75,7 @@ _SIGNATURES = {
                                    c_long, c_int, _P, _P, c_int, c_long]),
     "mui_embedding": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, c_int, c_int, c_int]),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
+    "mui_tune_packed_dot": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
     "mui_tune_skinny": (c_int, [c_int, c_int, c_int]),
 }

@@ -285,8 +285,13 @@ extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_token
   return MUI_OK;
 }
 
+extern "C" int mui_tune_packed_dot(int linear_on, int int8_on) {
+  g_gemv_dot2 = linear_on != 0;
+  int8_set_packed_dot(int8_on != 0);
+  return MUI_OK;
+}
+
 extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
-  if (rows_linear == 16 || rows_linear == 17) { g_gemv_dot2 = rows_linear == 16; return MUI_OK; }
   if (!(rows_linear == 0 || rows_linear == 2 || rows_linear == 4)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_tune.rows_linear = rows_linear;

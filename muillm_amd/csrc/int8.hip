@@ -353,11 +353,9 @@ static int check_int8_common(int dtype, const void* w, long pitch, const void* x
 
 using namespace mui;
 
+namespace mui { void int8_set_packed_dot(bool on) { g_int8_dot2 = on ? 1 : 0; } }
+
 extern "C" int mui_tune_int8(int rows, int wgs_per_cu) {
-  if (rows == 16 || rows == 17) {  // 16 / 17: single fp16 token through the packed-dot kernel on / off
-    g_int8_dot2 = rows == 16;
-    return MUI_OK;
-  }
   if (!(rows == 0 || rows == 2 || rows == 4 || rows == 8)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_int8_rows = rows;

@@ -72,5 +72,6 @@ int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 =
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 void skinny_set_int8_multi(int on);
+void int8_set_packed_dot(bool on);  // int8.hip: single fp16 token through int8_multi.hip
 
 }  // namespace mui
