@@ -312,7 +312,7 @@ int mui_tune_packed_dot(int linear_on, int int8_on);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the
- * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1024;
+ * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1536;
  * negative: never use the unsplit one-workgroup-per-query-head mode), and the shortest
  * sequence (or cache capacity, when the length is read on the device) that takes the
  * matrix-core kernel (default 0 = never: the vector kernel measured faster on MI355X) */

@@ -1024,7 +1024,7 @@ extern "C" int mui_flash_decode_splits(int batch, int n_q_heads, int n_kv_heads,
   // the combine launch on MI355X.) The total is one workgroup per CU: measured best at 32
   // splits for batch 1 and 4 splits for batch 8 with 8 KV heads.
   // Short sequences at small batch: one unsplit workgroup per query head beats split + merge.
-  const int direct = g_attn_direct_tokens > 0 ? g_attn_direct_tokens : 1024;
+  const int direct = g_attn_direct_tokens > 0 ? g_attn_direct_tokens : 1536;
   if (g_attn_head_parallel && seq_len_hint <= direct && batch * n_kv_heads * 8 <= device_cus()) return 1;
   const int min_tokens = g_attn_min_tokens > 0 ? g_attn_min_tokens : 2 * kBlock;
   const int max_useful = ceil_div(seq_len_hint, min_tokens);
