@@ -435,6 +435,11 @@ def main():
         dt_e, dec_e = bench_decode(lm, min(args.steps, 64), min(args.warmup, 8), use_graph=False)
         result["variants"] = {"fp16_eager_no_graph_tokens_per_s": round(min(args.steps, 64) / dt_e, 2)}
         del dec_e
+        for ctx in (4096,):
+            dt_c, dec_c = bench_decode(lm, 64, 8, prompt_len=ctx)
+            result["variants"]["fp16_context%d_tokens_per_s" % ctx] = round(64 / dt_c, 2)
+            del dec_c
+            torch.cuda.empty_cache()
         for bsz in (4, 8):
             dt_b, dec_b = bench_decode(lm, min(args.steps, 128), min(args.warmup, 8), batch=bsz)
             result["variants"]["fp16_batch%d_aggregate_tokens_per_s" % bsz] = round(bsz * min(args.steps, 128) / dt_b, 1)
