@@ -21,7 +21,8 @@ from ..kvcache.cache_utils import MuiStaticCache, _next_pow2, create_static_cach
 
 class MuiGraphDecoder:
     def __init__(self, lm, use_graph: bool = True, eos_token_ids=None, pad_token_id: int = 0,
-                 do_sample: bool = False, temperature: float = 1.0, seed: int = 0):
+                 do_sample: bool = False, temperature: float = 1.0, seed: int = 0,
+                 top_k: Optional[int] = None, top_p: Optional[float] = None):
         """do_sample=True draws from softmax(logits / temperature) on the device (the reference's
         sync-free multinomial, muillm/sampling/multinomial.py:4-6) instead of taking the argmax;
         the draws are a function of (seed, batch row, step), so a run is reproducible."""
@@ -30,6 +31,12 @@ class MuiGraphDecoder:
         self.do_sample = do_sample
         self.temperature = float(temperature)
         self.seed = int(seed)
+        # top-k / top-p filtering runs as torch ops (topk / sort) in front of the sampling kernel;
+        # those library calls stay out of HIP graphs, so the loop is eager when they are on
+        self.top_k = int(top_k) if top_k else None
+        self.top_p = float(top_p) if top_p is not None and top_p < 1.0 else None
+        if self.top_k or self.top_p:
+            self.use_graph = False
         self.eos_token_ids = list(eos_token_ids) if eos_token_ids is not None else None
         self.pad_token_id = int(pad_token_id)
         self.graph = None
@@ -64,6 +71,7 @@ class MuiGraphDecoder:
     def _advance(self, logits):
         """Token choice + stop check + token store + counters: one launch, all on the device."""
         if self.do_sample:
+            logits = self._filter_logits(logits)
             muillm_ext.mui_sample_advance(logits, self.ids, self.step, self.out_tokens, temperature=self.temperature,
                                           seed=self.seed, position_ids=self.pos, cache_position=self.cpos,
                                           unfinished=self.unfinished, eos_token_ids=self.eos,
@@ -72,6 +80,25 @@ class MuiGraphDecoder:
             muillm_ext.mui_greedy_advance(logits, self.ids, self.step, self.out_tokens, position_ids=self.pos,
                                           cache_position=self.cpos, unfinished=self.unfinished,
                                           eos_token_ids=self.eos, pad_token_id=self.pad_token_id)
+
+    def _filter_logits(self, logits):
+        """HuggingFace's TopKLogitsWarper / TopPLogitsWarper on the temperature-scaled distribution:
+        everything outside the k largest logits, or outside the smallest set of tokens whose
+        probability mass reaches top_p, becomes -inf (the sampling kernel never draws those)."""
+        if not (self.top_k or self.top_p):
+            return logits
+        lg = logits.float()
+        if self.top_k:
+            k = min(self.top_k, lg.shape[-1])
+            kth = torch.topk(lg, k, dim=-1).values[..., -1:]
+            lg = lg.masked_fill(lg < kth, float("-inf"))
+        if self.top_p:
+            srt, idx = torch.sort(lg / self.temperature, dim=-1, descending=False)
+            cum = torch.softmax(srt, dim=-1).cumsum(dim=-1)
+            drop = cum <= (1.0 - self.top_p)
+            drop[..., -1:] = False  # always keep the most likely token
+            lg = lg.masked_fill(drop.scatter(-1, idx, drop), float("-inf"))
+        return lg.to(logits.dtype)
 
     def _capture(self):
         self.cache.device_length_mode = True

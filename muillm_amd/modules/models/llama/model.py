@@ -356,17 +356,19 @@ class MuiLlamaForCausalLM(MuiModule):
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
                  max_new_tokens: int = 20, do_sample: bool = False, temperature: float = 1.0,
+                 top_k: Optional[int] = None, top_p: Optional[float] = None,
                  eos_token_id=None, pad_token_id: Optional[int] = None, seed: int = 0, use_graph: bool = True,
                  cache: Optional[MuiStaticCache] = None, **unused):
         """HuggingFace-style entry point over the device-resident decode loop (the reference routes
         generate() through its MuiGenerationMixin._sample, muillm/sampling/generation.py:77-408).
         Greedy (do_sample=False) or temperature sampling; left-padded batches via attention_mask;
         rows stop at eos_token_id (int or list) and are filled with pad_token_id afterwards.
-        Returns int64 [B, prompt_len + max_new_tokens]. Logit processors beyond temperature
-        (top-k, top-p, penalties) are not part of this loop."""
+        Returns int64 [B, prompt_len + max_new_tokens]. top_k / top_p filter the logits with torch
+        ops in front of the sampling kernel (the loop then runs eagerly instead of from the HIP
+        graph); other logit processors (penalties, ...) are not part of this loop."""
         from ..graphdecoder import MuiGraphDecoder
 
-        dropped = {k: v for k, v in unused.items() if v is not None and k in ("top_k", "top_p", "repetition_penalty")}
+        dropped = {k: v for k, v in unused.items() if v is not None and k in ("repetition_penalty", "num_beams")}
         if dropped:
             raise NotImplementedError(f"generate(): unsupported options {sorted(dropped)}")
         eos = None
@@ -375,7 +377,8 @@ class MuiLlamaForCausalLM(MuiModule):
         if pad_token_id is None:
             pad_token_id = eos[0] if eos else 0
         dec = MuiGraphDecoder(self, use_graph=use_graph, eos_token_ids=eos, pad_token_id=pad_token_id,
-                              do_sample=do_sample, temperature=temperature, seed=seed)
+                              do_sample=do_sample, temperature=temperature, seed=seed,
+                              top_k=top_k if do_sample else None, top_p=top_p if do_sample else None)
         # with an eos criterion the loop polls, without blocking, whether every row has finished
         return dec.generate(input_ids, max_new_tokens, cache=cache, attention_mask=attention_mask,
                             stop_check_every=8 if eos else 0)

@@ -286,7 +286,11 @@ def test_generate_stops_at_eos_and_pads():
             assert torch.equal(out[r, : 7 + h + 1], free[r, : 7 + h + 1])   # identical up to and including eos
             assert bool((out[r, 7 + h + 1:] == 0).all())                      # pad afterwards
     with pytest.raises(NotImplementedError):
-        lm.generate(ids, max_new_tokens=2, top_k=5)
+        lm.generate(ids, max_new_tokens=2, repetition_penalty=1.2)
+    # top_k = 1 sampling is greedy decoding; top_p -> 0 as well
+    k1 = lm.generate(ids, max_new_tokens=8, do_sample=True, top_k=1, seed=5).cpu()
+    p0 = lm.generate(ids, max_new_tokens=8, do_sample=True, top_p=1e-6, seed=6).cpu()
+    assert torch.equal(k1, free) and torch.equal(p0, free)
 
 
 def test_generate_early_stop_without_host_sync():
