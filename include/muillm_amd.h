@@ -319,10 +319,12 @@ int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
 int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
                        int mfma_tokens);
 /* fewest tokens that leave the one-GEMV-per-token loop (default 2; MUI_MAX_TOKENS + 1 keeps the
- * loop); stream_b != 0 forces the MFMA variant that re-reads the token operands per weight tile
- * instead of keeping them in registers (K <= 4096 only); multi_max_tokens: largest token count
- * served by the multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 8,
- * where 5..8 tokens only qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
+ * loop); stream_b selects older MFMA variants for 16-bit weights instead of the default one
+ * that turns contiguous row runs into operands through LDS: 2 = operands loaded in MFMA order
+ * straight from memory, token operands kept in registers (K <= 4096), 1 = the same with the
+ * token operands re-read per weight tile; multi_max_tokens: largest token count served by the
+ * multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 4; 5..8 only
+ * qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
 int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 
 #ifdef __cplusplus

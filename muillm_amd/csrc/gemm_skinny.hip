@@ -1,4 +1,7 @@
-// Small-batch (2..8 tokens) variants of the fused linears as skinny GEMMs on the matrix cores.
+// Small-batch (2..16 tokens) variants of the fused linears as skinny GEMMs on the matrix cores,
+// operands loaded in MFMA order straight from memory. Serves the 8-bit weight formats (whose
+// conversion happens in operand layout); 16-bit weights take gemm_skinny_lt.hip first, which
+// reads contiguous row runs and reorders them through LDS.
 //
 // The reference has no kernel for this case: anything but a single token falls back to an
 // RMSNorm kernel + torch matmul + residual add (csrc/modules/linear_module.cpp:57-79,
@@ -28,20 +31,6 @@ namespace mui {
 constexpr int kSkWaves = 8;
 constexpr int kSkThreads = kSkWaves * kWave;
 constexpr int kSkUnroll = 8;  // 16-byte weight loads in flight per lane
-
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-
-template <typename T>
-__device__ __forceinline__ f32x4 mfma16x16x32(u32x4 a, u32x4 b, f32x4 c);
-template <>
-__device__ __forceinline__ f32x4 mfma16x16x32<F16>(u32x4 a, u32x4 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-template <>
-__device__ __forceinline__ f32x4 mfma16x16x32<BF16>(u32x4 a, u32x4 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
 
 // 8 int8/uint8 weights (two dwords) -> the 16-bit MFMA operand.
 //   per-channel: exact integers (the row scale is applied in the epilogue). For fp16 the bytes
@@ -425,7 +414,9 @@ static int launch_skinny_t(hipStream_t s, const SkinnyParams& p) {
   return launch_status();
 }
 
+static int g_skinny_lt = 1;     // 16-bit weights: LDS-transposed operand kernel (gemm_skinny_lt.hip) first
 void skinny_set_bstat(int on) { g_skinny_bstat = on; }
+void skinny_set_lt(int on) { g_skinny_lt = on; }
 
 static int g_int8_multi = 1;  // 2..4 tokens of int8 weights: vector-ALU kernel (int8_multi.hip) first
 void skinny_set_int8_multi(int on) { g_int8_multi = on; }
@@ -434,6 +425,10 @@ void skinny_set_int8_multi(int on) { g_int8_multi = on; }
 int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams& p) {
   if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4) {
     const int st = launch_int8_multi(s, dtype, wf, epi, p);
+    if (st != MUI_ERR_UNSUPPORTED) return st;
+  }
+  if (wf == WF_16BIT && g_skinny_lt) {
+    const int st = launch_skinny_lt(s, dtype, epi, p);
     if (st != MUI_ERR_UNSUPPORTED) return st;
   }
 #define MUI_SK_CASE(TT, WFV, EPIV) \

@@ -1,10 +1,10 @@
-// Fused linears for 2..4 tokens (up to 8 on tall matrices) with 16-bit weights: the single-token GEMV structure (256
+// Fused linears for 1..4 tokens (opt-in up to 8 on tall matrices) with 16-bit weights: the single-token GEMV structure (256
 // threads, thread t owns 16-byte chunks t, t+256, ... of every row, R rows in flight, next row
 // group requested before the reduction, persistent balanced grid) with the token operands
 // gamma * x packed 16-bit in registers and one packed dot (v_dot2_f32_f16) per two weights and
 // token. The weights are streamed exactly once; at up to 4 tokens the vector ALUs stay far from
 // saturation, so the kernel runs at the single-token GEMV's HBM rate where the matrix-core
-// skinny GEMM (gemm_skinny.hip, used otherwise from 5 tokens) pays for its tile hand-offs.
+// skinny GEMM (gemm_skinny_lt.hip, used from 5 tokens) pays for its operand hand-offs.
 //
 // The reference has no kernel for this case (csrc/modules/linear_module.cpp:57-79 falls back to
 // RMSNorm + torch matmul + add; muillm/modules/gateupdownmlp.py:343-359).
@@ -183,8 +183,8 @@ static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
   const int ch = ceil_div(p.k >> 3, kMtThreads);
   if constexpr (TOK == 8) {
     // 8 tokens: 2 rows x 8 tokens = 16 partial sums per group; only rows of <= 2 chunks per thread
-    // and only tall matrices, where it measured faster than the matrix-core kernel (43 vs 48 us on
-    // the 2 x 14336 x 4096 gate/up shape; on par or slower at 6144 and 4096 rows)
+    // and only tall matrices. Opt-in (mui_tune_skinny): 43 us on the 2 x 14336 x 4096 gate/up
+    // shape against 40 us for the matrix-core kernel of gemm_skinny_lt.hip
     if (ch > 2 || p.n < 8192) return MUI_ERR_UNSUPPORTED;
     constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
     const int grid = balanced_grid(ceil_div(p.n, OUT), 4);

@@ -60,14 +60,34 @@ __device__ __forceinline__ u32x4 make_b(const u32x4 xv, const u32x4 gv, float& s
   }
 }
 
+// v_mfma_f32_16x16x32: A = 16 rows x 32 k, B = 32 k x 16 columns; lane l supplies 8 k-values
+// (k-chunk l / 16 of the step) of row / column l % 16
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template <typename T>
+__device__ __forceinline__ f32x4 mfma16x16x32(u32x4 a, u32x4 b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma16x16x32<F16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma16x16x32<BF16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
 // launches gemm_skinny_kernel<dtype, weight format, epilogue>; returns a MUI_* status
 int launch_skinny(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 // experiments: 0 disables the B-stationary persistent variant
 void skinny_set_bstat(int on);
+void skinny_set_lt(int on);  // 0: operands loaded straight from HBM in MFMA order (older kernels)
 
 // 2..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
 // in registers (gemv_multi.hip); returns MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
+// 5..16 tokens, 16-bit weights: weight rows read as whole 1 KB / 512 B runs and turned into
+// MFMA operands through wave-private LDS (gemm_skinny_lt.hip); MUI_ERR_UNSUPPORTED otherwise
+int launch_skinny_lt(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
 int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 = built-in)
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
