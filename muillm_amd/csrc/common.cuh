@@ -78,14 +78,26 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
 // loads. Weights are read exactly once per call, so they are streamed with the
 // non-temporal hint; small reused vectors (x, gamma) use ordinary cached loads.
 // ---------------------------------------------------------------------------------------
+// Every pointer these helpers see is device memory, so the global address space is named
+// explicitly: where the compiler cannot infer it (a pointer selected between two kernel
+// arguments, for instance) it would otherwise emit flat loads, which also occupy the LDS
+// counter and serialise against LDS traffic.
+typedef const __attribute__((address_space(1))) u32x4* global_u32x4_ptr;
+typedef const __attribute__((address_space(1))) u32x2* global_u32x2_ptr;
 __device__ __forceinline__ u32x4 ld16_stream(const void* p) {
-  return __builtin_nontemporal_load((const u32x4*)p);
+  return __builtin_nontemporal_load((global_u32x4_ptr)p);
 }
-__device__ __forceinline__ u32x4 ld16(const void* p) { return *(const u32x4*)p; }
+__device__ __forceinline__ u32x4 ld16(const void* p) { return *(global_u32x4_ptr)p; }
 __device__ __forceinline__ u32x2 ld8_stream(const void* p) {
-  return __builtin_nontemporal_load((const u32x2*)p);
+  return __builtin_nontemporal_load((global_u32x2_ptr)p);
 }
-__device__ __forceinline__ u32x2 ld8(const void* p) { return *(const u32x2*)p; }
+__device__ __forceinline__ u32x2 ld8(const void* p) { return *(global_u32x2_ptr)p; }
+__device__ __forceinline__ uint32_t ld4(const void* p) {
+  return *(const __attribute__((address_space(1))) uint32_t*)p;
+}
+__device__ __forceinline__ uint16_t ld2(const void* p) {
+  return *(const __attribute__((address_space(1))) uint16_t*)p;
+}
 
 template <bool STREAM>
 __device__ __forceinline__ u32x4 ld16_sel(const void* p) {

@@ -32,48 +32,6 @@ constexpr int kSkWaves = 8;
 constexpr int kSkThreads = kSkWaves * kWave;
 constexpr int kSkUnroll = 8;  // 16-byte weight loads in flight per lane
 
-// 8 int8/uint8 weights (two dwords) -> the 16-bit MFMA operand.
-//   per-channel: exact integers (the row scale is applied in the epilogue). For fp16 the bytes
-//   are dropped into the mantissa of 1024.0 (0x6400 | b = 1024 + b) with two byte permutes and
-//   the offset is removed with a packed subtract: 5 VALU ops per dword instead of a convert
-//   and a pack per weight.
-//   group format: u8 * scale + min, rounded once to the 16-bit type.
-template <typename T, int WF>
-__device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint16_t* srow, int elem, int group_shift) {
-  const uint32_t v[2] = {w0, w1};
-  if constexpr (WF == WF_I8_CHANNEL && T::kDtype == MUI_DTYPE_F16) {
-    u32x4 out;
-    const f16x2 off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128 (sign bit flipped below)
-    uint32_t o[4];
-#pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      const uint32_t u = v[m] ^ 0x80808080u;
-      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
-      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
-      o[2 * m + 0] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, lo) - off);
-      o[2 * m + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, hi) - off);
-    }
-    out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
-    return out;
-  } else {
-    float f[8];
-    if constexpr (WF == WF_I8_CHANNEL) {
-#pragma unroll
-      for (int m = 0; m < 2; ++m)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) f[4 * m + b] = (float)(int)(int8_t)((v[m] >> (8 * b)) & 0xffu);
-    } else {
-      const uint32_t pr = *(const uint32_t*)(srow + 2 * (elem >> group_shift));
-      const float sc = T::lo(pr), mn = T::hi(pr);
-#pragma unroll
-      for (int m = 0; m < 2; ++m)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) f[4 * m + b] = fmaf((float)((v[m] >> (8 * b)) & 0xffu), sc, mn);
-    }
-    return pack8<T>(f);
-  }
-}
-
 template <typename T, int WF, bool NORM, int EPI>
 __global__ void __launch_bounds__(kSkThreads) gemm_skinny_kernel(const SkinnyParams p) {
   __shared__ float tile[kSkWaves][16][17];
@@ -414,7 +372,7 @@ static int launch_skinny_t(hipStream_t s, const SkinnyParams& p) {
   return launch_status();
 }
 
-static int g_skinny_lt = 1;     // 16-bit weights: LDS-transposed operand kernel (gemm_skinny_lt.hip) first
+static int g_skinny_lt = 1;     // LDS-transposed operand kernel (gemm_skinny_lt.hip) first
 void skinny_set_bstat(int on) { g_skinny_bstat = on; }
 void skinny_set_lt(int on) { g_skinny_lt = on; }
 
@@ -427,8 +385,8 @@ int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams&
     const int st = launch_int8_multi(s, dtype, wf, epi, p);
     if (st != MUI_ERR_UNSUPPORTED) return st;
   }
-  if (wf == WF_16BIT && g_skinny_lt) {
-    const int st = launch_skinny_lt(s, dtype, epi, p);
+  if (g_skinny_lt) {
+    const int st = launch_skinny_lt(s, dtype, wf, epi, p);
     if (st != MUI_ERR_UNSUPPORTED) return st;
   }
 #define MUI_SK_CASE(TT, WFV, EPIV) \

@@ -1,23 +1,28 @@
-// Small-batch (5..16 tokens) fused linears with 16-bit weights on the matrix cores, with the
-// weight rows read the way the single-token GEMV reads them.
+// Small-batch (up to 16 tokens) fused linears on the matrix cores, with the weight rows read
+// the way the single-token GEMV reads them.
 //
-// An MFMA A operand wants lane l to hold 16 bytes of row l % 16, so loading operands straight
-// from HBM touches 16 rows x 64 bytes per instruction; measured on this part that pattern
-// streams 17-40 % slower than instructions that each cover one contiguous kilobyte (13.0 vs
-// 9.4 us for a 6144 x 4096 fp16 matrix). Here every load instruction covers 512-byte runs of two
-// rows; the registers are written to a wave-private LDS tile (row pitch +16
-// bytes: the 16 lanes of a b128 read phase hit 64 distinct banks) and read back in operand
-// order. LDS traffic is one write and one read per weight byte, far below its bandwidth, and
-// no workgroup barrier is involved: a wave only ever reads what it wrote itself.
+// An MFMA A operand wants lane l to hold the k-chunk l / 16 of row l % 16, so loading operands
+// straight from HBM touches 16 rows x 64 bytes per instruction; measured on this part that
+// pattern streams 17-40 % slower than instructions that cover contiguous runs of 512 bytes or
+// more (13.0 vs 9.4 us for a 6144 x 4096 fp16 matrix). Here every load instruction covers
+// contiguous runs (512 bytes of two rows with 16-bit weights, 256 bytes of four rows with 8-bit
+// weights); the registers are written to a wave-private LDS tile (row pitch +16 bytes: the
+// lanes of a read phase hit distinct banks) and read back in operand order. LDS traffic is one
+// write and one read per weight byte, far below its bandwidth, and no workgroup barrier is
+// involved: a wave only ever reads what it wrote itself. 8-bit weights cross LDS as bytes and
+// are converted to the 16-bit type in operand layout (per-channel: exact integers, the row scale
+// applied in the epilogue; group format: u8 * scale + min rounded once).
 //
-// A pass of a wave is 16 rows x 256 k-values (8 load instructions of two 512-byte runs, then 8
-// MFMAs): small enough that converting one pass overlaps the arrival of the next ones.
+// A pass of a wave is 16 rows x 256 k-values (then 8 MFMAs): small enough that converting one
+// pass overlaps the arrival of the next ones.
 //   B-stationary mode (K <= 4096, K % 256 == 0): wave w owns the same K range of every tile
 //     (two passes per tile); its B operands (gamma * x of the 16 token columns) are built once
-//     and stay in registers; four register sets = two tiles in flight.
-//   streaming mode (any K % 8 == 0, no fused norm): the wave walks its K range in passes and
-//     brings the token rows through LDS the same way as the weight rows; two register sets.
-// Both are persistent (one workgroup per CU, balanced tile counts).
+//     and stay in registers.
+//   streaming mode (longer rows, no fused norm): the wave walks its K range in passes and
+//     brings the token rows through LDS the same way as the weight rows.
+// Two register sets: the next pass is in flight while the current one is multiplied.
+// Both are persistent (one workgroup per CU, balanced tile counts). The number of passes of a
+// workgroup is a multiple of half the register sets (launcher).
 //
 // The reference has no kernel for this case (csrc/modules/linear_module.cpp:57-79 falls back to
 // RMSNorm + torch matmul + add; muillm/modules/gateupdownmlp.py:343-359).
@@ -27,27 +32,37 @@ namespace mui {
 
 constexpr int kLtWaves = 8;
 constexpr int kLtThreads = kLtWaves * kWave;
-constexpr int kLtSub = 256;                 // k-values per wave and pass
-constexpr int kLtPitch = kLtSub * 2 + 16;   // LDS row pitch in bytes
-constexpr int kLtLoads = 8;                 // load instructions per 16-row operand tile (2 rows each)
-constexpr int kLtSteps = kLtSub / 32;       // MFMAs per pass
+constexpr int kLtSub = 256;                  // k-values per wave and pass
+constexpr int kLtSteps = kLtSub / 32;        // MFMAs per pass
+constexpr int kLtXPitch = kLtSub * 2 + 16;   // LDS row pitch of a 16-bit operand tile, bytes
+constexpr int kLtXLoads = 8;                 // load instructions per 16-row tile of 16-bit values
 
-template <typename T, bool NORM, int EPI, bool BSTAT, bool FULL>
+template <typename T, int WF, bool NORM, int EPI, bool BSTAT, bool FULL>
 __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     // scalars, hottest first (the leading ones are preloaded into SGPRs at wave launch)
     const void* w0, const void* w1, long pitch, const uint16_t* x, int n, int k, int tokens, int n_tiles, int spw,
     const uint16_t* gamma, uint16_t* y, float eps, const uint16_t* residual, const uint16_t* mul_bias,
-    const uint16_t* add_bias) {
+    const uint16_t* add_bias, const uint16_t* s0, const uint16_t* s1, long s_pitch, int group_shift) {
   SkinnyParams p = {};
   p.w0 = w0; p.w1 = w1; p.pitch = pitch; p.x = x; p.n = n; p.k = k; p.tokens = tokens;
   p.gamma = gamma; p.y = y; p.eps = eps; p.residual = residual; p.mul_bias = mul_bias; p.add_bias = add_bias;
+  p.s0 = s0; p.s1 = s1; p.s_pitch = s_pitch; p.group_shift = group_shift;
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
-  constexpr int NOPS = BSTAT ? 1 : 2;   // operand tiles per wave in LDS: A, or A and B
-  constexpr int NSET = BSTAT ? 4 : 2;   // register sets = passes in flight per wave
-  constexpr int NB = BSTAT ? 1 : kLtLoads;
+  constexpr int WB = (WF == WF_16BIT) ? 2 : 1;   // bytes per weight
+  constexpr int ROWB = kLtSub * WB;              // bytes of a row segment of one pass
+  constexpr int PITCH = ROWB + 16;               // LDS row pitch of the weight tile
+  constexpr int RPI = 1024 / ROWB;               // rows covered by one load instruction (2 / 4)
+  constexpr int NLD = 16 / RPI;                  // load instructions per weight tile (8 / 4)
+  constexpr int LPR = kWave / RPI;               // lanes per row (32 / 16)
+  constexpr int KPC = 16 / WB;                   // k-values per 16-byte chunk (8 / 16)
+  constexpr int NOPS = BSTAT ? 1 : 2;            // operand tiles per wave in LDS: A, or A and B
+  // register sets = passes in flight per wave (four measured no faster with 8-bit weights and
+  // spill with 16-bit ones)
+  constexpr int NSET = 2;
+  constexpr int NB = BSTAT ? 1 : kLtXLoads;
   static_assert(BSTAT || !NORM, "streaming mode has no fused norm");
 
-  __shared__ __attribute__((aligned(16))) char op_lds[kLtWaves][NOPS][16 * kLtPitch];
+  __shared__ __attribute__((aligned(16))) char op_lds[kLtWaves][NOPS][16 * kLtXPitch];
   __shared__ float tile[2][kLtWaves][16][17];
   __shared__ float ss_part[kLtWaves][16];  // sum(x^2) of token j over wave w's K range
 
@@ -56,82 +71,117 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   const int wave = t >> 6;
   const int r16 = lane & 15;
   const int g = lane >> 4;
-  const int ld_row = lane >> 5;     // row inside a load instruction
-  const int ld_chunk = lane & 31;   // 16-byte chunk inside the 512-byte row segment
+  const int ld_row = lane / LPR;     // weight tile: row inside a load instruction
+  const int ld_chunk = lane % LPR;   //              16-byte chunk inside the row segment
+  const int xl_row = lane >> 5;      // 16-bit token tile: the same for two rows x 512 bytes
+  const int xl_chunk = lane & 31;
   char* la = &op_lds[wave][0][0];
   char* lb = &op_lds[wave][NOPS - 1][0];
 
-  // B-stationary: this wave's K range is jmax MFMA steps = jmax * 64 bytes of every row, walked
-  // in two passes of 8 steps; streaming: spw passes of 256 k-values per tile
+  // B-stationary: this wave's K range is jmax MFMA steps = 32 * jmax k-values of every row,
+  // walked in two passes of 8 steps; streaming: spw passes of 256 k-values per tile
   const int jmax = BSTAT ? (FULL ? 2 * kLtSteps : (p.k >> 8)) : 0;
   const int passes = BSTAT ? 2 : spw;
   const int my_tiles = blockIdx.x < n_tiles ? (n_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
   const int n_items = my_tiles * passes;  // pass i: tile blockIdx.x + (i / passes) * gridDim.x, sub-block i % passes
 
   auto row_base = [&](int tl, int q) -> const char* {
-    const int r = q * 2 + ld_row;  // row of the tile
+    const int r = q * RPI + ld_row;  // row of the tile
     int out_row;
     const void* wbase;
     if constexpr (EPI == SK_GATEUP) {
-      out_row = tl * 8 + q;
-      wbase = ld_row ? p.w1 : p.w0;
+      out_row = tl * 8 + (r >> 1);
+      wbase = (r & 1) ? p.w1 : p.w0;
     } else {
       out_row = tl * 16 + r;
       wbase = p.w0;
     }
     const int row_c = out_row < p.n ? out_row : p.n - 1;
-    return (const char*)wbase + (long)row_c * p.pitch * 2;
+    return (const char*)wbase + (long)row_c * p.pitch * WB;
+  };
+  // group format: (scale, min) pairs of the weight row behind tile row r16 (operand layout)
+  auto scale_row = [&](int tl) -> const uint16_t* {
+    if constexpr (WF != WF_U8_GROUP) return nullptr;
+    int out_row;
+    const uint16_t* sbase;
+    if constexpr (EPI == SK_GATEUP) {
+      out_row = tl * 8 + (r16 >> 1);
+      sbase = (r16 & 1) ? p.s1 : p.s0;
+    } else {
+      out_row = tl * 16 + r16;
+      sbase = p.s0;
+    }
+    const int row_c = out_row < p.n ? out_row : p.n - 1;
+    return sbase + (long)row_c * p.s_pitch;
   };
 
-  // Lanes, token rows and passes with nothing to fetch issue no load at all (measured: feeding
-  // them dummy addresses to keep the code branch-free costs more than the compiler's coarser
-  // load-counter waits behind the branches).
-  auto lane_k0 = [&](int i, bool& ok) -> int {  // first k-value of this lane's chunk in pass i
+  // first k-value of pass i of this wave
+  auto pass_k0 = [&](int i) -> int {
     const int sub = i % passes;
-    if constexpr (BSTAT) {
-      const int c = sub * 32 + ld_chunk;  // chunk inside the wave's range
-      ok = FULL || c < 4 * jmax;
-      return (wave * jmax * 4 + c) << 3;
-    } else {
-      const int k0 = ((wave * spw + sub) << 8) + (ld_chunk << 3);
-      ok = k0 < p.k;
-      return k0;
-    }
+    if constexpr (BSTAT) return wave * jmax * 32 + sub * kLtSub;
+    else return (wave * spw + sub) * kLtSub;
   };
+  // k-values of pass i that exist (B-stationary: inside the wave's range; streaming: inside the row)
+  auto pass_len = [&](int i) -> int {
+    if constexpr (BSTAT) return FULL ? kLtSub : jmax * 32 - (i % passes) * kLtSub;
+    else return p.k - pass_k0(i);
+  };
+
+  // No load of the steady state sits behind a branch: the compiler's load-counter waits are
+  // exact only in straight-line code (behind a branch it waits for everything outstanding,
+  // the newest prefetch included, which costs a full memory latency per pass). So nothing is
+  // predicated: lanes past the end of the K range read the start of their row instead and are
+  // zeroed on the way to LDS; token rows past the batch read the last token again (their
+  // output columns are never stored); the tail without refills is peeled off the loop.
   // Epilogue thread t < 16 * OUT handles token t / OUT, output t % OUT of the tile (consecutive
-  // threads write consecutive outputs of one token). Its residual value travels with the
-  // register set of the tile's last pass and is requested right after that pass's weights.
-  auto issue_residual = [&](int i, uint32_t& res) {  // 32-bit holder: never packed with another one
+  // threads write consecutive outputs of one token). Its residual value and per-channel scales
+  // travel with the register set of each pass, requested right after that pass's weights: a
+  // load inside the epilogue would be the youngest one outstanding, and waiting for it would
+  // wait for every prefetched pass.
+  struct Extras { uint32_t res, sc0, sc1; };  // 32-bit holders: never packed with one another
+  const int tok_last = p.tokens - 1;
+  auto issue_extras = [&](int i, Extras& e) {
+    const int tl = blockIdx.x + (i / passes) * gridDim.x;
+    int nn = tl * OUT + (t % OUT), j = t / OUT;
+    nn = nn < p.n ? nn : p.n - 1;
+    j = j < p.tokens ? j : tok_last;
     if constexpr (EPI == SK_LINEAR) {
-      const int tl = blockIdx.x + (i / passes) * gridDim.x;
-      const int n = tl * OUT + (t % OUT), j = t / OUT;
-      const bool want = p.residual && i < n_items && (i % passes) == passes - 1 && t < OUT * 16 && j < p.tokens && n < p.n;
-      if (want) res = p.residual[(long)j * p.n + n];
+      const uint16_t* rp = p.residual ? p.residual + ((long)j * p.n + nn) : p.x;
+      e.res = ld2(rp);
+    }
+    if constexpr (WF == WF_I8_CHANNEL) {
+      e.sc0 = ld2(p.s0 + (long)nn * p.s_pitch);
+      if constexpr (EPI == SK_GATEUP) e.sc1 = ld2(p.s1 + (long)nn * p.s_pitch);
     }
   };
-  auto issue = [&](int i, u32x4 (&a)[kLtLoads], u32x4 (&b)[NB]) {
-    if (i >= n_items) return;
-    const u32x4 zero = {0u, 0u, 0u, 0u};
+  // k-value of this lane's weight chunk in pass i, or -1 past the end of the range
+  auto weight_k = [&](int i) -> int {
+    const int kk = ld_chunk * KPC;
+    return (FULL || kk < pass_len(i)) ? pass_k0(i) + kk : -1;
+  };
+  auto issue = [&](int i, u32x4 (&a)[NLD], u32x4 (&b)[NB]) {  // needs i < n_items
     const int tl = blockIdx.x + (i / passes) * gridDim.x;
-    bool ok;
-    const int k0 = lane_k0(i, ok);
+    const int wk = weight_k(i);
+    const long woff = (long)(wk < 0 ? 0 : wk) * WB;
 #pragma unroll
-    for (int q = 0; q < kLtLoads; ++q) a[q] = ok ? ld16_stream(row_base(tl, q) + ((long)k0 << 1)) : zero;
+    for (int q = 0; q < NLD; ++q) a[q] = ld16_stream(row_base(tl, q) + woff);
     if constexpr (!BSTAT) {
+      const int xk = pass_k0(i) + xl_chunk * 8;
+      const int xoff = xk < p.k ? xk : 0;  // (the weights of those k-values are zeroed)
 #pragma unroll
-      for (int q = 0; q < kLtLoads; ++q) {
-        const int tok = q * 2 + ld_row;
-        b[q] = (ok && tok < p.tokens) ? ld16(p.x + (long)tok * p.k + k0) : zero;
+      for (int q = 0; q < kLtXLoads; ++q) {
+        const int tok = q * 2 + xl_row;
+        b[q] = ld16(p.x + (long)(tok < p.tokens ? tok : tok_last) * p.k + xoff);
       }
     }
   };
 
-  auto epilogue = [&](int tl, int buf, float res) {
+  auto epilogue = [&](int tl, int buf, const Extras& ex) {
     if (t < OUT * 16) {
       const int i = t % OUT;
       const int j = t / OUT;
-      const int n = tl * OUT + i;
-      if (j < p.tokens && n < p.n) {
+      const int nn = tl * OUT + i;
+      if (j < p.tokens && nn < p.n) {
         float rs = 1.f;
         if constexpr (NORM) {
           float tot = 0.f;
@@ -147,14 +197,20 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
         };
         float v;
         if constexpr (EPI == SK_GATEUP) {
-          v = silu_f32(total(2 * i) * rs) * (total(2 * i + 1) * rs);
+          float gt = total(2 * i) * rs, up = total(2 * i + 1) * rs;
+          if constexpr (WF == WF_I8_CHANNEL) {
+            gt *= T::one((uint16_t)ex.sc0);
+            up *= T::one((uint16_t)ex.sc1);
+          }
+          v = silu_f32(gt) * up;
         } else {
           v = total(i) * rs;
-          if (p.mul_bias) v *= T::one(p.mul_bias[n]);
-          if (p.add_bias) v += T::one(p.add_bias[n]);
-          if (p.residual) v += res;
+          if constexpr (WF == WF_I8_CHANNEL) v *= T::one((uint16_t)ex.sc0);
+          if (p.mul_bias) v *= T::one(p.mul_bias[nn]);
+          if (p.add_bias) v += T::one(p.add_bias[nn]);
+          if (p.residual) v += T::one((uint16_t)ex.res);
         }
-        p.y[(long)j * p.n + n] = T::pack(v);
+        p.y[(long)j * p.n + nn] = T::pack(v);
       }
     }
   };
@@ -162,44 +218,52 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   u32x4 bq[BSTAT ? 2 * kLtSteps : 1];
   f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};  // two chains: MFMAs back to back
   int buf = 0;
-  auto stage = [&](const u32x4 (&a)[kLtLoads], const u32x4 (&b)[NB]) {  // registers -> LDS tile
+  auto stage = [&](int i, const u32x4 (&a)[NLD], const u32x4 (&b)[NB]) {  // registers -> LDS tiles
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const bool ok = FULL || weight_k(i) >= 0;
 #pragma unroll
-    for (int q = 0; q < kLtLoads; ++q) *(u32x4*)(la + (q * 2 + ld_row) * kLtPitch + ld_chunk * 16) = a[q];
+    for (int q = 0; q < NLD; ++q) *(u32x4*)(la + (q * RPI + ld_row) * PITCH + ld_chunk * 16) = ok ? a[q] : zero;
     if constexpr (!BSTAT) {
 #pragma unroll
-      for (int q = 0; q < kLtLoads; ++q) *(u32x4*)(lb + (q * 2 + ld_row) * kLtPitch + ld_chunk * 16) = b[q];
+      for (int q = 0; q < kLtXLoads; ++q) *(u32x4*)(lb + (q * 2 + xl_row) * kLtXPitch + xl_chunk * 16) = b[q];
     }
     __builtin_amdgcn_wave_barrier();
   };
-  // operand order back into the registers the pass came from (all reads in flight at once)
-  auto gather = [&](u32x4 (&a)[kLtLoads], u32x4 (&b)[NB]) {
+  // one pass in operand order: 8 MFMA steps of 32 k-values (half: which half of the wave's range
+  // the pass covers in B-stationary mode; the register set fixes it)
+  // (the operands are read back into the registers the pass came from: NLD = 8 = steps with
+  // 16-bit weights, and the token tile of streaming mode has 8 loads as well)
+  auto multiply = [&](int i, const int half, u32x4 (&a16)[NLD], u32x4 (&bx)[NB]) {
+    u32x2 a8[WF == WF_16BIT ? 1 : kLtSteps];
 #pragma unroll
-    for (int s = 0; s < kLtSteps; ++s) a[s] = *(const u32x4*)(la + r16 * kLtPitch + (4 * s + g) * 16);
-    if constexpr (!BSTAT) {
-#pragma unroll
-      for (int s = 0; s < kLtSteps; ++s) b[s] = *(const u32x4*)(lb + r16 * kLtPitch + (4 * s + g) * 16);
+    for (int s = 0; s < kLtSteps; ++s) {  // all reads in flight at once
+      if constexpr (WF == WF_16BIT) a16[s] = *(const u32x4*)(la + r16 * PITCH + (4 * s + g) * 16);
+      else a8[s] = *(const u32x2*)(la + r16 * PITCH + (4 * s + g) * 8);
+      if constexpr (!BSTAT) bx[s] = *(const u32x4*)(lb + r16 * kLtXPitch + (4 * s + g) * 16);
     }
-  };
-  auto mma = [&](const u32x4 (&a)[kLtLoads], const u32x4 (&b)[NB], const int half) {
+    const uint16_t* srow = scale_row(blockIdx.x + (i / passes) * gridDim.x);
+    const int k0 = pass_k0(i);
 #pragma unroll
     for (int s = 0; s < kLtSteps; ++s) {
       if (BSTAT && !FULL && half * kLtSteps + s >= jmax) break;
-      u32x4 bv;
+      u32x4 av, bv;
+      if constexpr (WF == WF_16BIT) av = a16[s];
+      else av = convert_a<T, WF>(a8[s].x, a8[s].y, srow, k0 + 32 * s + 8 * g, p.group_shift);
       if constexpr (BSTAT) bv = bq[half * kLtSteps + s];
-      else bv = b[s];
-      if (s & 1) acc1 = mfma16x16x32<T>(a[s], bv, acc1);
-      else acc = mfma16x16x32<T>(a[s], bv, acc);
+      else bv = bx[s];
+      if (s & 1) acc1 = mfma16x16x32<T>(av, bv, acc1);
+      else acc = mfma16x16x32<T>(av, bv, acc);
     }
     __builtin_amdgcn_wave_barrier();
   };
-  auto finish = [&](int i, const uint32_t res_bits) {
-    if ((i % passes) == passes - 1 && i < n_items) {  // last pass of the tile: reduce over the waves
+  auto finish = [&](int i, const Extras& ex) {
+    if ((i % passes) == passes - 1) {  // last pass of the tile: reduce over the waves
 #pragma unroll
       for (int r = 0; r < 4; ++r) tile[buf][wave][4 * g + r][r16] = acc[r] + acc1[r];
       acc = f32x4{0.f, 0.f, 0.f, 0.f};
       acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
       __syncthreads();
-      epilogue(blockIdx.x + (i / passes) * gridDim.x, buf, T::one((uint16_t)res_bits));
+      epilogue(blockIdx.x + (i / passes) * gridDim.x, buf, ex);
       buf ^= 1;
     }
   };
@@ -213,104 +277,144 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   // behind them.
   u32x4 gv = {0u, 0u, 0u, 0u};
   u32x4 xv[BSTAT ? 16 : 1];
+  const bool b_ok = FULL || lane < 4 * jmax;
   if constexpr (BSTAT) {
-    const bool b_ok = FULL || lane < 4 * jmax;
-    const int e = (wave * jmax * 4 + lane) << 3;  // element offset of this lane's chunk inside a row
-    if constexpr (NORM) { if (b_ok) gv = ld16(p.gamma + e); }
+    const int e = b_ok ? (wave * jmax * 4 + lane) << 3 : 0;  // element offset of this lane's chunk inside a row
+    if constexpr (NORM) gv = ld16(p.gamma + e);
 #pragma unroll
-    for (int tk = 0; tk < 16; ++tk) {
-      xv[tk] = u32x4{0u, 0u, 0u, 0u};
-      if (b_ok && tk < p.tokens) xv[tk] = ld16(p.x + (long)tk * p.k + e);
-    }
+    for (int tk = 0; tk < 16; ++tk) xv[tk] = ld16(p.x + (long)(tk < p.tokens ? tk : tok_last) * p.k + e);
   }
-
-  // two passes go out before the build, the rest after it (the token rows, the build's
-  // registers and four register sets do not fit the register file together)
-  u32x4 as[NSET][kLtLoads], bs[NSET][NB];
-  uint32_t rs_bits[NSET] = {};
+  auto build_b = [&]() {
+    if constexpr (BSTAT) {
+      const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    issue(u, as[u], bs[u]);
-    issue_residual(u, rs_bits[u]);
-  }
-
-  if constexpr (BSTAT) {
+      for (int tk = 0; tk < 16; ++tk) {
+        float ss = 0.f;
+        xv[tk] = make_b<T, NORM>(b_ok ? xv[tk] : zero, gv, ss);
+        if constexpr (NORM) {
+          ss = wave_sum(ss);
+          if (lane == 0) ss_part[wave][tk] = ss;
+        }
+      }
 #pragma unroll
-    for (int tk = 0; tk < 16; ++tk) {
-      float ss = 0.f;
-      xv[tk] = make_b<T, NORM>(xv[tk], gv, ss);  // zero rows stay zero
-      if constexpr (NORM) {
-        ss = wave_sum(ss);
-        if (lane == 0) ss_part[wave][tk] = ss;
+      for (int h = 0; h < 2; ++h) {
+        if ((lane >> 5) == h) {
+#pragma unroll
+          for (int tk = 0; tk < 16; ++tk) *(u32x4*)(la + tk * kLtXPitch + xl_chunk * 16) = xv[tk];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < kLtSteps; ++j) bq[h * kLtSteps + j] = *(const u32x4*)(la + r16 * kLtXPitch + (4 * j + g) * 16);
+        __builtin_amdgcn_wave_barrier();
       }
     }
+  };
+
+  u32x4 as[NSET][NLD], bs[NSET][NB];
+  Extras ex[NSET] = {};
+  // pass i on register set U (U = i % NSET); REFILL: the set is requested again for pass i + NSET
+#define MUI_LT_PASS(i_, U, REFILL)                    \
+  {                                                   \
+    stage((i_), as[U], bs[U]);                        \
+    multiply((i_), (U) & 1, as[U], bs[U]);            \
+    if (REFILL) issue((i_) + NSET, as[U], bs[U]);     \
+    finish((i_), ex[U]);                              \
+    if (REFILL) issue_extras((i_) + NSET, ex[U]);     \
+  }
+
+  if (n_items >= NSET) {
+    // two passes go out before the build, the rest after it (the token rows, the build's
+    // registers and all register sets do not fit the register file together)
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      if ((lane >> 5) == h) {
-#pragma unroll
-        for (int tk = 0; tk < 16; ++tk) *(u32x4*)(la + tk * kLtPitch + ld_chunk * 16) = xv[tk];
-      }
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int j = 0; j < kLtSteps; ++j) bq[h * kLtSteps + j] = *(const u32x4*)(la + r16 * kLtPitch + (4 * j + g) * 16);
-      __builtin_amdgcn_wave_barrier();
+    for (int u = 0; u < 2; ++u) {
+      issue(u, as[u], bs[u]);
+      issue_extras(u, ex[u]);
     }
-  }
-
+    build_b();
 #pragma unroll
-  for (int u = 2; u < NSET; ++u) {
-    issue(u, as[u], bs[u]);
-    issue_residual(u, rs_bits[u]);
-  }
-
-  // passes in rounds of NSET
-  for (int i = 0; i < n_items; i += NSET) {
+    for (int u = 2; u < NSET; ++u) {
+      issue(u, as[u], bs[u]);
+      issue_extras(u, ex[u]);
+    }
+    // passes with a refill in rounds of NSET, a half round if their number asks for it (it is
+    // a multiple of NSET / 2), then the last NSET passes without refills
+    const int n_main = n_items - NSET;
+    int i = 0;
+    for (; i + NSET <= n_main; i += NSET) {
+#pragma unroll
+      for (int u = 0; u < NSET; ++u) MUI_LT_PASS(i + u, u, true)
+    }
+    if (i < n_main) {
+#pragma unroll
+      for (int u = 0; u < NSET / 2; ++u) MUI_LT_PASS(i + u, u, true)
+#pragma unroll
+      for (int v = 0; v < NSET; ++v) MUI_LT_PASS(i + NSET / 2 + v, (NSET / 2 + v) % NSET, false)
+    } else {
+#pragma unroll
+      for (int v = 0; v < NSET; ++v) MUI_LT_PASS(i + v, v, false)
+    }
+  } else {
+    // fewer passes than register sets (one small tile per workgroup): everything is requested
+    // up front and multiplied once it is there
 #pragma unroll
     for (int u = 0; u < NSET; ++u) {
-      const bool live = i + u < n_items;
-      if (live) {
-        stage(as[u], bs[u]);
-        gather(as[u], bs[u]);
-        mma(as[u], bs[u], u & 1);
+      if (u < n_items) {
+        issue(u, as[u], bs[u]);
+        issue_extras(u, ex[u]);
       }
-      issue(i + u + NSET, as[u], bs[u]);  // the set is free again
-      if (live) finish(i + u, rs_bits[u]);
-      issue_residual(i + u + NSET, rs_bits[u]);
+    }
+    build_b();
+#pragma unroll
+    for (int u = 0; u < NSET; ++u) {
+      if (u < n_items) MUI_LT_PASS(u, u, false)
     }
   }
+#undef MUI_LT_PASS
 }
 
-template <typename T, int EPI>
+template <typename T, int WF, int EPI>
 static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
   const int n_tiles = ceil_div(p.n, OUT);
   const int grid = balanced_grid(n_tiles, 1);  // ~150 KB of LDS: one workgroup per CU
-#define MUI_LT(NORMV, BSTATV, FULLV, SPW)                                                               \
-  hipLaunchKernelGGL((gemm_skinny_lt_kernel<T, NORMV, EPI, BSTATV, FULLV>), dim3(grid), dim3(kLtThreads), \
-                     0, s, p.w0, p.w1, p.pitch, p.x, p.n, p.k, p.tokens, n_tiles, SPW, p.gamma, p.y, p.eps,        \
-                     p.residual, p.mul_bias, p.add_bias)
+#define MUI_LT(NORMV, BSTATV, FULLV, SPW)                                                                   \
+  hipLaunchKernelGGL((gemm_skinny_lt_kernel<T, WF, NORMV, EPI, BSTATV, FULLV>), dim3(grid), dim3(kLtThreads), \
+                     0, s, p.w0, p.w1, p.pitch, p.x, p.n, p.k, p.tokens, n_tiles, SPW, p.gamma, p.y, p.eps,   \
+                     p.residual, p.mul_bias, p.add_bias, p.s0, p.s1, p.s_pitch, p.group_shift)
   if (p.k <= kLtWaves * 2 * kLtSub && p.k % 256 == 0) {
     const bool full = p.k == kLtWaves * 2 * kLtSub;
     if (p.gamma) { if (full) MUI_LT(true, true, true, 1); else MUI_LT(true, true, false, 1); }
     else { if (full) MUI_LT(false, true, true, 1); else MUI_LT(false, true, false, 1); }
     return launch_status();
   }
-  if (p.gamma || (p.k & 7)) return MUI_ERR_UNSUPPORTED;
-  const int spw = ceil_div(ceil_div(p.k, 256), kLtWaves);
+  // streaming: 16-byte chunks of weights and of token rows must not straddle the row end
+  if (p.gamma || (p.k % (WF == WF_16BIT ? 8 : 16))) return MUI_ERR_UNSUPPORTED;
+  const int spw = ceil_div(ceil_div(p.k, kLtSub), kLtWaves);
   MUI_LT(false, false, false, spw);
 #undef MUI_LT
   return launch_status();
 }
 
-int launch_skinny_lt(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p) {
+int launch_skinny_lt(hipStream_t s, int dtype, int wf, int epilogue, const SkinnyParams& p) {
   if (p.tokens < 1 || p.tokens > 16) return MUI_ERR_UNSUPPORTED;
+#define MUI_LT_CASE(TT, WFV, EPIV) \
+  if (wf == WFV && epilogue == EPIV) return launch_lt_t<TT, WFV, EPIV>(s, p);
   if (dtype == MUI_DTYPE_F16) {
-    if (epilogue == SK_LINEAR) return launch_lt_t<F16, SK_LINEAR>(s, p);
-    if (epilogue == SK_GATEUP) return launch_lt_t<F16, SK_GATEUP>(s, p);
+    MUI_LT_CASE(F16, WF_16BIT, SK_LINEAR)
+    MUI_LT_CASE(F16, WF_16BIT, SK_GATEUP)
+    MUI_LT_CASE(F16, WF_I8_CHANNEL, SK_LINEAR)
+    MUI_LT_CASE(F16, WF_I8_CHANNEL, SK_GATEUP)
+    MUI_LT_CASE(F16, WF_U8_GROUP, SK_LINEAR)
+    MUI_LT_CASE(F16, WF_U8_GROUP, SK_GATEUP)
   } else if (dtype == MUI_DTYPE_BF16) {
-    if (epilogue == SK_LINEAR) return launch_lt_t<BF16, SK_LINEAR>(s, p);
-    if (epilogue == SK_GATEUP) return launch_lt_t<BF16, SK_GATEUP>(s, p);
+    MUI_LT_CASE(BF16, WF_16BIT, SK_LINEAR)
+    MUI_LT_CASE(BF16, WF_16BIT, SK_GATEUP)
+    MUI_LT_CASE(BF16, WF_I8_CHANNEL, SK_LINEAR)
+    MUI_LT_CASE(BF16, WF_I8_CHANNEL, SK_GATEUP)
+    MUI_LT_CASE(BF16, WF_U8_GROUP, SK_LINEAR)
+    MUI_LT_CASE(BF16, WF_U8_GROUP, SK_GATEUP)
   }
+#undef MUI_LT_CASE
   return MUI_ERR_INVALID_ARG;
 }
 

@@ -76,6 +76,48 @@ __device__ __forceinline__ f32x4 mfma16x16x32<BF16>(u32x4 a, u32x4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// 8 int8/uint8 weights (two dwords) -> the 16-bit MFMA operand.
+//   per-channel: exact integers (the row scale is applied in the epilogue). For fp16 the bytes
+//   are dropped into the mantissa of 1024.0 (0x6400 | b = 1024 + b) with two byte permutes and
+//   the offset is removed with a packed subtract: 5 VALU ops per dword instead of a convert
+//   and a pack per weight.
+//   group format: u8 * scale + min, rounded once to the 16-bit type.
+template <typename T, int WF>
+__device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint16_t* srow, int elem, int group_shift) {
+  const uint32_t v[2] = {w0, w1};
+  if constexpr (WF == WF_I8_CHANNEL && T::kDtype == MUI_DTYPE_F16) {
+    u32x4 out;
+    const f16x2 off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128 (sign bit flipped below)
+    uint32_t o[4];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      const uint32_t u = v[m] ^ 0x80808080u;
+      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+      o[2 * m + 0] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, lo) - off);
+      o[2 * m + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, hi) - off);
+    }
+    out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
+    return out;
+  } else {
+    float f[8];
+    if constexpr (WF == WF_I8_CHANNEL) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) f[4 * m + b] = (float)(int)(int8_t)((v[m] >> (8 * b)) & 0xffu);
+    } else {
+      const uint32_t pr = ld4(srow + 2 * (elem >> group_shift));
+      const float sc = T::lo(pr), mn = T::hi(pr);
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) f[4 * m + b] = fmaf((float)((v[m] >> (8 * b)) & 0xffu), sc, mn);
+    }
+    return pack8<T>(f);
+  }
+}
+
 // launches gemm_skinny_kernel<dtype, weight format, epilogue>; returns a MUI_* status
 int launch_skinny(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 // experiments: 0 disables the B-stationary persistent variant
@@ -85,9 +127,9 @@ void skinny_set_lt(int on);  // 0: operands loaded straight from HBM in MFMA ord
 // 2..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
 // in registers (gemv_multi.hip); returns MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
-// 5..16 tokens, 16-bit weights: weight rows read as whole 1 KB / 512 B runs and turned into
-// MFMA operands through wave-private LDS (gemm_skinny_lt.hip); MUI_ERR_UNSUPPORTED otherwise
-int launch_skinny_lt(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
+// MFMA skinny GEMM whose weight rows are read as contiguous runs and turned into operands
+// through wave-private LDS (gemm_skinny_lt.hip); MUI_ERR_UNSUPPORTED for shapes it does not cover
+int launch_skinny_lt(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 = built-in)
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
