@@ -26,6 +26,8 @@
 //   slot that is being written.
 //   The sequence length can come from device memory (cache_position[0] + 1), which keeps
 //   the launch shape fixed under HIP-graph replay.
+#include <type_traits>
+
 #include "common.cuh"
 
 namespace mui {
@@ -183,18 +185,24 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
   const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs + dc * 8;
   const uint16_t* mrow = p.mask ? p.mask + (long)b * p.mask_bs : nullptr;
-  auto load_block = [&](int base, u32x4 (&kreg)[U], u32x4 (&vreg)[U], bool (&valid)[U]) {
+  // No K/V load sits behind a branch: the compiler's load-counter waits are exact only in
+  // straight-line code (behind a branch it waits for everything outstanding, the block just
+  // requested included, which would serialise the two register sets). Tokens past the end,
+  // the new slot and whole blocks past the last one read row 0 of the head instead (always
+  // there) and are marked invalid. MASKED adds the per-token mask read of padded batches.
+  auto load_block = [&](int base, bool live, u32x4 (&kreg)[U], u32x4 (&vreg)[U], bool (&valid)[U],
+                        auto masked) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int tok = base + u * kWorkers + wk;
-      valid[u] = (tok < t_end) && (tok != slot);
-      const int tk = valid[u] ? tok : t_begin;  // t_begin < S: always a readable row
+      valid[u] = live && (tok < t_end) && (tok != slot);
+      const int tk = valid[u] ? tok : 0;
       // split (long) sequences stream K/V once: non-temporal; the unsplit short case re-reads
       // rows that the previous steps left in cache
       kreg[u] = ld16_sel<!DIRECT>(kc + (long)tk * p.c_ts);
       vreg[u] = ld16_sel<!DIRECT>(vc + (long)tk * p.c_ts);
-      if (mrow != nullptr && valid[u]) {
-        if (T::one(mrow[tok]) != 0.f) valid[u] = false;
+      if constexpr (decltype(masked)::value) {
+        if (T::one(ld2(mrow + tk)) != 0.f) valid[u] = false;
       }
     }
   };
@@ -206,14 +214,18 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   // wraps around.
   const int n_blocks = t_end > t_begin ? (t_end - t_begin + kBlock - 1) / kBlock : 0;
   const int rot = n_blocks > 0 ? (int)((blockIdx.x * 7u + blockIdx.y * 13u + blockIdx.z * 29u) % (unsigned)n_blocks) : 0;
-  auto block_base = [&](int bi) {
+  auto block_base = [&](int bi) {  // any bi < 2 * n_blocks (blocks past the last one are not live)
     int blk = bi + rot;
     blk = blk >= n_blocks ? blk - n_blocks : blk;
     return t_begin + blk * kBlock;
   };
-  int bi = 0;
-  bool have_a = n_blocks > 0;
-  if (have_a) load_block(block_base(0), ka, va, valid_a);
+  auto fetch = [&](int bi, u32x4 (&kreg)[U], u32x4 (&vreg)[U], bool (&valid)[U], auto masked) {
+    const bool live = bi < n_blocks;
+    load_block(block_base(live ? bi : 0), live, kreg, vreg, valid, masked);
+  };
+  const bool use_mask = mrow != nullptr;
+  if (use_mask) fetch(0, ka, va, valid_a, std::true_type{});
+  else fetch(0, ka, va, valid_a, std::false_type{});
 
   // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once) ----
   for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
@@ -261,29 +273,26 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
     float madd[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) madd[u] = 0.f;
-    if constexpr (kPipe) {
-      // two register sets: the next block is in flight while the current one is consumed
-      for (;;) {
-        if (!have_a) break;
-        const bool have_b = bi + 1 < n_blocks;
-        if (have_b) load_block(block_base(bi + 1), kb, vb, valid_b);
-        attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
-        if (!have_b) break;
-        bi += 2;
-        have_a = bi < n_blocks;
-        if (have_a) load_block(block_base(bi), ka, va, valid_a);
-        attend_block<T, G, U>(kb, vb, valid_b, madd, qreg, p.scale_log2, m, l, acc);
+    auto sweep = [&](auto masked) {
+      if constexpr (kPipe) {
+        // two register sets: the next block is in flight while the current one is consumed
+        // (an odd block count ends with one block that is not live)
+        for (int bi = 0; bi < n_blocks; bi += 2) {
+          fetch(bi + 1, kb, vb, valid_b, masked);
+          attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
+          fetch(bi + 2, ka, va, valid_a, masked);
+          attend_block<T, G, U>(kb, vb, valid_b, madd, qreg, p.scale_log2, m, l, acc);
+        }
+      } else {
+        // 4 waves per SIMD overlap each other's loads; one register set keeps the kernel
+        // under 128 VGPRs
+        for (int bi = 0; bi < n_blocks; ++bi) {
+          attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
+          fetch(bi + 1, ka, va, valid_a, masked);
+        }
       }
-    } else {
-      // 4 waves per SIMD overlap each other's loads; one register set keeps the kernel
-      // under 128 VGPRs
-      while (have_a) {
-        attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
-        ++bi;
-        have_a = bi < n_blocks;
-        if (have_a) load_block(block_base(bi), ka, va, valid_a);
-      }
-    }
+    };
+    if (use_mask) sweep(std::true_type{}); else sweep(std::false_type{});
   }
 
   if (owner && wave == 0) {  // the new token, straight from LDS, on DPP row 0 of wave 0
