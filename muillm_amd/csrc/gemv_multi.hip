@@ -55,6 +55,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
   }
 
   u32x4 w[R][CH];
+  uint32_t res_w = 0;  // residual (16-bit pattern) that belongs to the weights in w
   auto issue = [&](int rg) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -71,6 +72,14 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
       const uint16_t* rp = base + (long)row * pitch;
 #pragma unroll
       for (int j = 0; j < CH; ++j) w[r][j] = ld16_stream(rp + coff[j]);
+    }
+    // the residual value of this group's epilogue thread rides along with the weights: loaded
+    // inside the epilogue it would add a memory round trip to the end of the kernel
+    if constexpr (EPI == SK_LINEAR) {
+      if (residual && t < OUT * TOK) {
+        const int row = rg * OUT + t / TOK, tk = t % TOK;
+        if (row < n && tk < tokens) res_w = ld2(residual + (long)tk * n + row);
+      }
     }
   };
   int rg = blockIdx.x;
@@ -129,6 +138,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
         acc[r * TOK + tk] = a;
       }
     }
+    const uint32_t res_cur = res_w;
     const int nxt = rg + gridDim.x;
     if (nxt < n_groups) issue(nxt);  // keep the memory pipe full during the reduction
 
@@ -158,7 +168,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
           v = total(o);
           if (mul_bias) v *= T::one(mul_bias[row]);
           if (add_bias) v += T::one(add_bias[row]);
-          if (residual) v += T::one(residual[(long)tk * n + row]);
+          if (residual) v += T::one((uint16_t)res_cur);
         }
         y[(long)tk * n + row] = T::pack(v);
       }

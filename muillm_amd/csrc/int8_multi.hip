@@ -57,6 +57,10 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
 
   u32x4 w[R][CH];
   uint32_t sm[R][CH];  // group format: packed (scale, min) of the chunk's group
+  // what the epilogue thread of a group needs from memory (residual, per-channel scales) rides
+  // along with the group's weights: loaded inside the epilogue it would add a memory round trip
+  // to the end of the kernel
+  uint32_t ep_res = 0, ep_s0 = 0, ep_s1 = 0;
   auto issue = [&](int rg) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -78,7 +82,19 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       for (int j = 0; j < CH; ++j) {
         w[r][j] = ld16_stream(rp + coff[j]);
         if constexpr (WF == WF_U8_GROUP)
-          sm[r][j] = *(const uint32_t*)(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
+          sm[r][j] = ld4(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
+      }
+    }
+    if (t < OUT * TOK) {
+      const int row = rg * OUT + t / TOK, tk = t % TOK;
+      if (row < n && tk < tokens) {
+        if constexpr (WF == WF_I8_CHANNEL) {
+          ep_s0 = ld2(a.s0 + (long)row * a.s_pitch);
+          if constexpr (EPI == SK_GATEUP) ep_s1 = ld2(a.s1 + (long)row * a.s_pitch);
+        }
+        if constexpr (EPI == SK_LINEAR) {
+          if (a.residual) ep_res = ld2(a.residual + (long)tk * n + row);
+        }
       }
     }
   };
@@ -179,6 +195,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
         acc[v / NVH][v % NVH] = ar[tk];
       }
     }
+    const uint32_t cur_res = ep_res, cur_s0 = ep_s0, cur_s1 = ep_s1;
     const int nxt = rg + gridDim.x;
     if (nxt < n_groups) issue(nxt);
 
@@ -206,15 +223,15 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
         if constexpr (EPI == SK_GATEUP) {
           float g = total(2 * o), u = total(2 * o + 1);
           if constexpr (WF == WF_I8_CHANNEL) {
-            g *= T::one(a.s0[(long)row * a.s_pitch]);
-            u *= T::one(a.s1[(long)row * a.s_pitch]);
+            g *= T::one((uint16_t)cur_s0);
+            u *= T::one((uint16_t)cur_s1);
           }
           v = silu_f32(g) * u;
         } else {
           v = total(o);
-          if constexpr (WF == WF_I8_CHANNEL) v *= T::one(a.s0[(long)row * a.s_pitch]);
+          if constexpr (WF == WF_I8_CHANNEL) v *= T::one((uint16_t)cur_s0);
           if (a.add_bias) v += T::one(a.add_bias[row]);
-          if (a.residual) v += T::one(a.residual[(long)tk * n + row]);
+          if (a.residual) v += T::one((uint16_t)cur_res);
         }
         y[(long)tk * n + row] = T::pack(v);
       }
