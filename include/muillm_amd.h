@@ -291,6 +291,59 @@ int mui_sample_advance(mui_stream_t stream, int dtype, const void* logits, long 
                        int64_t* tokens_out, long tokens_stride, int max_steps, int64_t* unfinished,
                        const int64_t* eos_ids, int n_eos, long pad_token);
 
+/* ------------------------------------------------------------------------------------
+ * decoder layers of one decode step in a single call
+ * ---------------------------------------------------------------------------------- */
+
+/* What MuiDecoderLayer.forward does for one token per batch row
+ * (muillm/modules/decoder/decoder.py:130-165), for all layers, enqueued by one call; the
+ * reference has a C++ layer loop only under tensor parallelism
+ * (csrc/modules/parallel_decoder_stack.cpp, csrc/modules/parallel_decoder_module.cpp:22-62).
+ * Per layer: qkv = Wqkv rmsnorm(h); attn = flash decoding with RoPE and cache write
+ * (mui_attn_decode_fused); h' = Wo attn + h; mid = silu(Wg n) * (Wu n) with n = rmsnorm(h');
+ * out = Wd mid + h'. All pointers are device memory of the 16-bit type `dtype`; the caller
+ * owns everything. */
+typedef struct mui_decoder_layer {
+  const void* input_norm;   /* [hidden] gamma of the RMSNorm fused into the QKV projection */
+  const void* qkv_weight;   /* [(Hq + 2 Hkv) * D, hidden], rows q | k | v */
+  long qkv_pitch;           /* row pitches in elements */
+  const void* o_weight;     /* [hidden, Hq * D] */
+  long o_pitch;
+  const void* post_norm;    /* [hidden] gamma of the RMSNorm fused into gate/up */
+  const void* gate_weight;  /* [intermediate, hidden] */
+  const void* up_weight;    /* [intermediate, hidden], same pitch (interleaved storage allowed) */
+  long gateup_pitch;
+  const void* down_weight;  /* [hidden, intermediate] */
+  long down_pitch;
+  void* k_cache;            /* [batch, Hkv, max_cache_len, D] with the strides below */
+  void* v_cache;
+} mui_decoder_layer_t;
+
+typedef struct mui_decoder_stack {
+  int dtype, n_layers, hidden, n_q_heads, n_kv_heads, head_dim, intermediate;
+  float norm_eps;
+  const mui_decoder_layer_t* layers; /* host array of n_layers entries */
+  const float* cos_table;            /* fp32 [positions, rope_row_stride] rotary tables */
+  const float* sin_table;
+  long rope_row_stride;
+  long cache_batch_stride, cache_head_stride, cache_token_stride; /* elements */
+  int max_cache_len;
+} mui_decoder_stack_t;
+
+/* Bytes of device workspace mui_decoder_stack_step needs (activations between the kernels
+ * and the flash-decoding partials for n_splits); 0 on bad arguments. */
+size_t mui_decoder_stack_workspace_bytes(const mui_decoder_stack_t* model, int batch, int n_splits);
+
+/* hidden_in [batch, hidden] (token embeddings) -> hidden_out [batch, hidden] (output of the
+ * last layer, before the final norm). position_ids, cache_position, seq_len, mask and
+ * n_splits as in mui_attn_decode_fused (n_splits from mui_flash_decode_splits). workspace:
+ * 256-byte aligned, mui_decoder_stack_workspace_bytes() bytes. batch <= MUI_MAX_TOKENS.
+ * Asynchronous on `stream`, allocates nothing: capturable into a HIP graph. */
+int mui_decoder_stack_step(mui_stream_t stream, const mui_decoder_stack_t* model, int batch,
+                           const void* hidden_in, void* hidden_out, const int64_t* position_ids,
+                           long position_batch_stride, const int64_t* cache_position, int seq_len,
+                           const void* mask, long mask_batch_stride, int n_splits, void* workspace);
+
 /* muillm_embedding_module_forward (csrc/module.cpp:320; csrc/embedding/embedding.cu:31-100; kernels
  * csrc/embedding/embedding_xx16_kernels.cu:26-112): out[t, :] = table[ids[t], :] for a 16-bit
  * [vocab, dim] table with row pitch row_pitch elements; ids int64, or int32 when ids_are_int32.

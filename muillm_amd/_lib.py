@@ -74,11 +74,32 @@ _SIGNATURES = {
     "mui_sample_advance": (c_int, [_P, c_int, _P, c_long, c_int, c_int, c_float, ctypes.c_uint64, _P, _P, _P, _P, _P,
                                    c_long, c_int, _P, _P, c_int, c_long]),
     "mui_embedding": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, c_int, c_int, c_int]),
+    "mui_decoder_stack_workspace_bytes": (ctypes.c_size_t, [_P, c_int, c_int]),
+    "mui_decoder_stack_step": (c_int, [_P, _P, c_int, _P, _P, _P, c_long, _P, c_int, _P, c_long, c_int, _P]),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_packed_dot": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
     "mui_tune_skinny": (c_int, [c_int, c_int, c_int]),
 }
+
+
+
+class MuiDecoderLayerDesc(ctypes.Structure):
+    """struct mui_decoder_layer of the public header."""
+    _fields_ = [("input_norm", _P), ("qkv_weight", _P), ("qkv_pitch", c_long), ("o_weight", _P),
+                ("o_pitch", c_long), ("post_norm", _P), ("gate_weight", _P), ("up_weight", _P),
+                ("gateup_pitch", c_long), ("down_weight", _P), ("down_pitch", c_long), ("k_cache", _P),
+                ("v_cache", _P)]
+
+
+class MuiDecoderStackDesc(ctypes.Structure):
+    """struct mui_decoder_stack of the public header."""
+    _fields_ = [("dtype", c_int), ("n_layers", c_int), ("hidden", c_int), ("n_q_heads", c_int),
+                ("n_kv_heads", c_int), ("head_dim", c_int), ("intermediate", c_int), ("norm_eps", c_float),
+                ("layers", ctypes.POINTER(MuiDecoderLayerDesc)), ("cos_table", _P), ("sin_table", _P),
+                ("rope_row_stride", c_long), ("cache_batch_stride", c_long), ("cache_head_stride", c_long),
+                ("cache_token_stride", c_long), ("max_cache_len", c_int)]
+
 
 _lib: Optional[ctypes.CDLL] = None
 

@@ -1,0 +1,132 @@
+"""All decoder layers of a decode step through one library call.
+
+The reference walks its layers from C++ only under tensor parallelism
+(muillm/modules/models/llama/model.py:331-358 -> csrc/modules/parallel_decoder_stack.cpp); on
+one GPU it calls its Python layer modules one by one (muillm/modules/decoder/decoder.py:130-165).
+Here `mui_decoder_stack_step` enqueues the same per-layer sequence for every layer, so a step
+that is not replayed from a HIP graph pays the host cost of one call instead of ~160.
+"""
+import ctypes
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from ... import _lib, muillm_ext
+from ..attention.baseattention import MuiBaseAttention
+from ..gateupdownmlp import MuiGateUpDownMLP
+from ..kvcache.cache_utils import MuiStaticCache
+from ..linear import MuiLinear
+from ..multilinear import MuiMultiLinear
+
+
+def _plain_linear(m, normalize: Optional[bool] = None) -> bool:
+    return (type(m) is MuiLinear and m.bias is None and m.weight.is_cuda and m.weight.stride(1) == 1
+            and (normalize is None or bool(m.normalize) == normalize))
+
+
+class MuiDecoderStack:
+    """Descriptor + workspace of `mui_decoder_stack_step` for one model, cache and batch size.
+
+    Holds plain pointers: it has to be rebuilt when the cache is re-allocated (`matches`)."""
+
+    def __init__(self, layers, rotary_emb, cache: MuiStaticCache, batch: int):
+        self.lib = _lib.load()
+        first = layers[0]
+        attn0: MuiBaseAttention = first.self_attn
+        w0 = first.qkv_proj.linear.weight
+        self.dtype, self.device = w0.dtype, w0.device
+        self.batch = batch
+        self.hidden = w0.shape[1]
+        self.hq, self.hkv, self.d = attn0.num_heads, attn0.num_key_value_heads, attn0.head_dim
+        self.cos32, self.sin32 = rotary_emb.cos32, rotary_emb.sin32
+        kc0 = cache.key_cache[0]
+        cb, chs, cts = kc0.stride(0), kc0.stride(1), kc0.stride(2)
+        self.max_cache_len = kc0.shape[2]
+        self._cache_ptrs = tuple(t.data_ptr() for t in cache.key_cache) + tuple(t.data_ptr() for t in cache.value_cache)
+        self._keep = []  # tensors the descriptor points into
+        arr = (_lib.MuiDecoderLayerDesc * len(layers))()
+        for i, layer in enumerate(layers):
+            qkv, attn, mlp = layer.qkv_proj.linear, layer.self_attn, layer.mlp
+            g, u, dn = mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight
+            kc, vc = cache.key_cache[attn.layer_idx], cache.value_cache[attn.layer_idx]
+            if (kc.stride(), vc.stride()) != (kc0.stride(), kc0.stride()):
+                raise ValueError("cache layers must share one layout")
+            arr[i] = _lib.MuiDecoderLayerDesc(
+                qkv.norm_weights.data_ptr(), qkv.weight.data_ptr(), qkv.weight.stride(0),
+                attn.o_proj.weight.data_ptr(), attn.o_proj.weight.stride(0),
+                mlp.norm_weights.data_ptr(), g.data_ptr(), u.data_ptr(), g.stride(0),
+                dn.data_ptr(), dn.stride(0), kc.data_ptr(), vc.data_ptr())
+            self._keep += [qkv.norm_weights, qkv.weight, attn.o_proj.weight, mlp.norm_weights, g, u, dn, kc, vc]
+        self._layers = arr
+        self.desc = _lib.MuiDecoderStackDesc(
+            muillm_ext._dtype_code(w0), len(layers), self.hidden, self.hq, self.hkv, self.d,
+            layers[0].mlp.gate_proj.weight.shape[0], float(first.qkv_proj.linear.variance_epsilon),
+            ctypes.cast(arr, ctypes.POINTER(_lib.MuiDecoderLayerDesc)), self.cos32.data_ptr(), self.sin32.data_ptr(),
+            self.cos32.stride(0), cb, chs, cts, self.max_cache_len)
+        self._ws = None
+        self._ws_splits = 0
+
+    @staticmethod
+    def eligible(layers, rotary_emb, cache, batch: int) -> bool:
+        """fp16 / bf16 Llama-shaped layers without biases on a static cache, head_dim 128."""
+        if not isinstance(cache, MuiStaticCache) or len(layers) == 0 or batch > _lib.MUI_MAX_TOKENS:
+            return False
+        if not getattr(rotary_emb, "dispatchable", False):
+            return False
+        eps = None
+        for layer in layers:
+            qkv, attn, mlp = getattr(layer, "qkv_proj", None), getattr(layer, "self_attn", None), getattr(layer, "mlp", None)
+            if type(qkv) is not MuiMultiLinear or not _plain_linear(qkv.linear, True):
+                return False
+            if not isinstance(attn, MuiBaseAttention) or not _plain_linear(attn.o_proj, False):
+                return False
+            if attn.head_dim != 128 or attn.num_key_value_groups not in (1, 2, 4, 8):
+                return False
+            if type(mlp) is not MuiGateUpDownMLP or not mlp.normalize or not isinstance(mlp.activation_function, nn.SiLU):
+                return False
+            if not all(_plain_linear(m, False) for m in (mlp.gate_proj, mlp.up_proj, mlp.down_proj)):
+                return False
+            if mlp.gate_proj.weight.stride(0) != mlp.up_proj.weight.stride(0):
+                return False
+            w = qkv.linear.weight
+            if w.dtype not in (torch.float16, torch.bfloat16) or cache.key_cache[attn.layer_idx].dtype != w.dtype:
+                return False
+            e = (float(qkv.linear.variance_epsilon), float(mlp.variance_epsilon))
+            if e[0] != e[1] or (eps is not None and e != eps):
+                return False
+            eps = e
+        return True
+
+    def matches(self, cache: MuiStaticCache, batch: int) -> bool:
+        ptrs = tuple(t.data_ptr() for t in cache.key_cache) + tuple(t.data_ptr() for t in cache.value_cache)
+        return batch == self.batch and ptrs == self._cache_ptrs
+
+    def step(self, hidden_in: torch.Tensor, position_ids: torch.Tensor, cache_position: torch.Tensor,
+             seq_len: Optional[int], mask: Optional[torch.Tensor]) -> torch.Tensor:
+        """hidden_in [B, 1, hidden] -> output of the last layer [B, 1, hidden]."""
+        lib, b = self.lib, self.batch
+        x = hidden_in.reshape(b, self.hidden)
+        if not x.is_contiguous():
+            x = x.contiguous()
+        hint = seq_len if seq_len is not None else self.max_cache_len
+        n_splits = lib.mui_flash_decode_splits(b, self.hq, self.hkv, int(hint))
+        if self._ws is None or n_splits > self._ws_splits:
+            nbytes = lib.mui_decoder_stack_workspace_bytes(ctypes.byref(self.desc), b, n_splits)
+            self._ws = torch.empty(nbytes + 256, dtype=torch.uint8, device=self.device)
+            self._ws_splits = n_splits
+        ws_ptr = (self._ws.data_ptr() + 255) & ~255
+        pos = position_ids.reshape(-1)
+        if pos.dtype != torch.int64 or cache_position.dtype != torch.int64:
+            raise RuntimeError("position_ids and cache_position must be int64")
+        mask_ptr, mask_bs = None, 0
+        if mask is not None:
+            mask = muillm_ext._mask_rows(mask, b, x.dtype)
+            mask_ptr, mask_bs = mask.data_ptr(), mask.stride(0)
+        out = torch.empty((b, 1, self.hidden), dtype=x.dtype, device=x.device)
+        muillm_ext.check(
+            lib.mui_decoder_stack_step(muillm_ext._stream(x), ctypes.byref(self.desc), b, x.data_ptr(), out.data_ptr(),
+                                       pos.data_ptr(), 1 if pos.numel() > 1 else 0, cache_position.data_ptr(),
+                                       -1 if seq_len is None else int(seq_len), mask_ptr, mask_bs, n_splits, ws_ptr),
+            "mui_decoder_stack_step")
+        return out

@@ -27,6 +27,7 @@ from ....replacement.replacementcontext import MuiReplacementContext
 from ...attention.rotaryembedding import MuiRotaryEmbedding
 from ...attention.sdpaattention import MuiSdpaAttention, _ignore_causal_mask_sdpa
 from ...decoder.decoder import MuiDecoderLayer
+from ...decoder.decoderstack import MuiDecoderStack
 from ...embedding import MuiEmbedding
 from ...gateupdownmlp import MuiGateUpDownMLP
 from ...kvcache.cache_utils import (MuiCache, MuiStaticCache, create_static_cache,
@@ -100,6 +101,9 @@ class MuiLlamaModel(MuiModule):
         self.layers = layers if isinstance(layers, nn.ModuleList) else nn.ModuleList(layers)
         self.norm = norm
         self.rotary_emb = rotary_emb
+        self.use_decoder_stack = True  # False: always walk the layer modules from Python
+        self._stack: Optional[MuiDecoderStack] = None
+        self._stack_eligible: Optional[bool] = None
 
     def finalize_init(self):
         self.mdevice = self.embed_tokens.weight.device
@@ -131,6 +135,21 @@ class MuiLlamaModel(MuiModule):
 
     def set_input_embeddings(self, value):
         self.embed_tokens = value
+
+    def _decode_stack(self, cache, batch_size: int, hidden_states) -> Optional[MuiDecoderStack]:
+        """The single-call layer stack for this cache and batch size, or None when the model does
+        not qualify (quantized layers, biases, foreign cache, ...); rebuilt when the cache moves."""
+        if not self.use_decoder_stack or not hidden_states.is_cuda or not isinstance(cache, MuiStaticCache):
+            return None
+        st = self._stack
+        if st is not None and st.matches(cache, batch_size):
+            return st
+        if self._stack_eligible is None or st is not None:
+            self._stack_eligible = MuiDecoderStack.eligible(self.layers, self.rotary_emb, cache, batch_size)
+        if not self._stack_eligible:
+            return None
+        self._stack = MuiDecoderStack(self.layers, self.rotary_emb, cache, batch_size)
+        return self._stack
 
     def _update_causal_mask(self, attention_mask, inputs_shape, cache_position, past_key_values,
                             output_attentions, all_ones_mask, past_seen_tokens: int):
@@ -212,7 +231,18 @@ class MuiLlamaModel(MuiModule):
 
         all_hidden_states = () if output_hidden_states else None
         all_self_attns = () if output_attentions else None
-        for decoder_layer in self.layers:
+        stack = None
+        if q_len == 1 and use_cache and not output_hidden_states and not output_attentions:
+            stack = self._decode_stack(past_key_values, batch_size, hidden_states)
+        if stack is not None:
+            # every layer through one library call (what the loop below does, layer by layer)
+            past_key_values._seen_tokens += 1
+            if past_key_values.cpp_module is not None:
+                past_key_values.cpp_module.seen_tokens = past_key_values._seen_tokens
+            seq_len = None if past_key_values.device_length_mode else past_key_values._seen_tokens
+            hidden_states = stack.step(hidden_states, position_ids, cache_position, seq_len,
+                                       None if all_ones_mask else causal_mask)
+        for decoder_layer in (self.layers if stack is None else ()):
             if output_hidden_states:
                 all_hidden_states += (hidden_states,)
             layer_outputs = decoder_layer(

@@ -188,6 +188,48 @@ def test_graph_decode_matches_eager(batch):
     assert dec.cache.get_seq_length() == 32 + n_new - 1
 
 
+@pytest.mark.parametrize("batch", [1, 3])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decoder_stack_call_matches_layer_modules(batch, dtype):
+    """mui_decoder_stack_step (all layers in one C call) runs the same kernels in the same order
+    as the layer modules: identical logits and cache contents, with and without padding masks,
+    also after the cache has grown (the descriptor is rebuilt)."""
+    cfg = _small_config(layers=3)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=dtype, device=DEV, seed=2, init_std=0.05)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, cfg.vocab_size, (batch, 11), generator=g).to(DEV)
+    results = {}
+    for use_stack in (False, True):
+        lm.model.use_decoder_stack = use_stack
+        out = lm(input_ids=ids)
+        cache = out.past_key_values
+        nxt = out.logits[:, -1].argmax(-1)
+        logits = []
+        for _ in range(9):  # crosses the 16 -> 32 capacity step
+            out = lm(input_ids=nxt.unsqueeze(1), past_key_values=cache)
+            logits.append(out.logits[:, -1].clone())
+            nxt = out.logits[:, -1].argmax(-1)
+        assert (lm.model._stack is not None) == use_stack or not use_stack
+        results[use_stack] = (torch.stack(logits), [k.clone() for k in cache.key_cache],
+                              [v.clone() for v in cache.value_cache], cache.get_seq_length())
+    assert lm.model._stack is not None, "the single-call path did not engage"
+    a, b2 = results[False], results[True]
+    assert a[3] == b2[3] == 20
+    assert torch.equal(a[0], b2[0])
+    for x, y in zip(a[1] + a[2], b2[1] + b2[2]):
+        assert torch.equal(x, y)
+    # left-padded batch through generate(): same tokens with and without the single call
+    if batch > 1:
+        mask = torch.ones_like(ids)
+        mask[0, :4] = 0
+        toks = {}
+        for use_stack in (False, True):
+            lm.model.use_decoder_stack = use_stack
+            toks[use_stack] = lm.generate(ids, attention_mask=mask, max_new_tokens=6, use_graph=False).cpu()
+        assert torch.equal(toks[False], toks[True])
+    lm.model.use_decoder_stack = True
+
+
 def test_argmax_kernel():
     from muillm_amd import muillm_ext
     g = torch.Generator().manual_seed(2)
