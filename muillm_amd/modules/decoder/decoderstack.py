@@ -45,6 +45,8 @@ class MuiDecoderStack:
         self.max_cache_len = kc0.shape[2]
         self._cache_ptrs = tuple(t.data_ptr() for t in cache.key_cache) + tuple(t.data_ptr() for t in cache.value_cache)
         self._keep = []  # tensors the descriptor points into
+        self._layer_list = layers
+        self._owners = []  # (module, attribute name, parameter object) the descriptor was built from
         arr = (_lib.MuiDecoderLayerDesc * len(layers))()
         for i, layer in enumerate(layers):
             qkv, attn, mlp = layer.qkv_proj.linear, layer.self_attn, layer.mlp
@@ -58,6 +60,11 @@ class MuiDecoderStack:
                 mlp.norm_weights.data_ptr(), g.data_ptr(), u.data_ptr(), g.stride(0),
                 dn.data_ptr(), dn.stride(0), kc.data_ptr(), vc.data_ptr())
             self._keep += [qkv.norm_weights, qkv.weight, attn.o_proj.weight, mlp.norm_weights, g, u, dn, kc, vc]
+            self._owners += [(layer, "qkv_proj", layer.qkv_proj), (layer, "self_attn", attn), (layer, "mlp", mlp),
+                             (layer.qkv_proj, "linear", qkv), (qkv, "weight", qkv.weight),
+                             (qkv, "norm_weights", qkv.norm_weights), (attn, "o_proj", attn.o_proj),
+                             (attn.o_proj, "weight", attn.o_proj.weight), (mlp, "norm_weights", mlp.norm_weights),
+                             (mlp.gate_proj, "weight", g), (mlp.up_proj, "weight", u), (mlp.down_proj, "weight", dn)]
         self._layers = arr
         self.desc = _lib.MuiDecoderStackDesc(
             muillm_ext._dtype_code(w0), len(layers), self.hidden, self.hq, self.hkv, self.d,
@@ -98,9 +105,17 @@ class MuiDecoderStack:
             eps = e
         return True
 
-    def matches(self, cache: MuiStaticCache, batch: int) -> bool:
+    def matches(self, layers, cache: MuiStaticCache, batch: int) -> bool:
+        """Still valid for this step? The cache tensors are where they were, and every module and
+        parameter the descriptor was built from is still the object in place (a later
+        quantize_layers / .to() / weight swap replaces them)."""
+        if batch != self.batch or layers is not self._layer_list or len(layers) * 12 != len(self._owners):
+            return False
+        for owner, name, obj in self._owners:
+            if getattr(owner, name, None) is not obj:
+                return False
         ptrs = tuple(t.data_ptr() for t in cache.key_cache) + tuple(t.data_ptr() for t in cache.value_cache)
-        return batch == self.batch and ptrs == self._cache_ptrs
+        return ptrs == self._cache_ptrs
 
     def step(self, hidden_in: torch.Tensor, position_ids: torch.Tensor, cache_position: torch.Tensor,
              seq_len: Optional[int], mask: Optional[torch.Tensor]) -> torch.Tensor:

@@ -103,7 +103,7 @@ class MuiLlamaModel(MuiModule):
         self.rotary_emb = rotary_emb
         self.use_decoder_stack = True  # False: always walk the layer modules from Python
         self._stack: Optional[MuiDecoderStack] = None
-        self._stack_eligible: Optional[bool] = None
+        self._stack_rejected = None
 
     def finalize_init(self):
         self.mdevice = self.embed_tokens.weight.device
@@ -142,13 +142,18 @@ class MuiLlamaModel(MuiModule):
         if not self.use_decoder_stack or not hidden_states.is_cuda or not isinstance(cache, MuiStaticCache):
             return None
         st = self._stack
-        if st is not None and st.matches(cache, batch_size):
+        if st is not None and st.matches(self.layers, cache, batch_size):
             return st
-        if self._stack_eligible is None or st is not None:
-            self._stack_eligible = MuiDecoderStack.eligible(self.layers, self.rotary_emb, cache, batch_size)
-        if not self._stack_eligible:
+        self._stack = None
+        # a model that did not qualify is not examined again until its modules or cache change
+        key = tuple(id(m) for l in self.layers for m in (getattr(l, "qkv_proj", None), getattr(l, "mlp", None)))
+        key += (id(cache), batch_size)
+        if key == self._stack_rejected:
             return None
-        self._stack = MuiDecoderStack(self.layers, self.rotary_emb, cache, batch_size)
+        if MuiDecoderStack.eligible(self.layers, self.rotary_emb, cache, batch_size):
+            self._stack = MuiDecoderStack(self.layers, self.rotary_emb, cache, batch_size)
+        else:
+            self._stack_rejected = key
         return self._stack
 
     def _update_causal_mask(self, attention_mask, inputs_shape, cache_position, past_key_values,

@@ -228,6 +228,25 @@ def test_decoder_stack_call_matches_layer_modules(batch, dtype):
             toks[use_stack] = lm.generate(ids, attention_mask=mask, max_new_tokens=6, use_graph=False).cpu()
         assert torch.equal(toks[False], toks[True])
     lm.model.use_decoder_stack = True
+    # a weight swapped after the descriptor was built is noticed (the descriptor is rebuilt)
+    if batch == 1:
+        out = lm(input_ids=ids)
+        cache = out.past_key_values
+        nxt = out.logits[:, -1].argmax(-1).unsqueeze(1)
+        before = lm(input_ids=nxt, past_key_values=cache).logits.clone()
+        old_stack = lm.model._stack
+        mlp = lm.model.layers[1].mlp
+        mlp.down_proj.weight = torch.nn.Parameter(torch.zeros_like(mlp.down_proj.weight), requires_grad=False)
+        cache.reset()
+        out = lm(input_ids=ids)
+        after = lm(input_ids=nxt, past_key_values=out.past_key_values).logits
+        assert lm.model._stack is not old_stack
+        assert not torch.equal(before, after)
+        lm.model.use_decoder_stack = False
+        cache2 = lm(input_ids=ids).past_key_values
+        ref = lm(input_ids=nxt, past_key_values=cache2).logits
+        lm.model.use_decoder_stack = True
+        assert torch.equal(after, ref)
 
 
 def test_argmax_kernel():
