@@ -366,9 +366,11 @@ int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the
  * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1536;
- * negative: never use the unsplit one-workgroup-per-query-head mode), and the shortest
- * sequence (or cache capacity, when the length is read on the device) that takes the
- * matrix-core kernel (default 0 = never: the vector kernel measured faster on MI355X) */
+ * negative: never use the unsplit one-workgroup-per-query-head mode), and mfma_tokens for the
+ * matrix-core decode kernel: 0 = default (whenever a workgroup handles a whole KV group, i.e.
+ * everywhere but in the unsplit one-workgroup-per-query-head mode), n > 0 = also instead of
+ * that mode for sequences (or cache capacities, when the length is read on the device) of at
+ * least n tokens, negative = never (vector-ALU kernel only) */
 int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
                        int mfma_tokens);
 /* fewest tokens that leave the one-GEMV-per-token loop (default 2; MUI_MAX_TOKENS + 1 keeps the

@@ -413,6 +413,7 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* lds_ptr) {
 }
 
 constexpr int kMfTok = 32;        // tokens per wave block
+constexpr int kMfKStride = 136;   // 16-bit elements per K tile row (256 + 16 bytes)
 constexpr int kMfVStride = 144;   // 16-bit elements per V tile row: 288 bytes keep the transposed reads spread over the banks
 
 template <typename T, int G, int NW, bool DIRECT>
@@ -429,6 +430,10 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
   constexpr int kMergeBytes = NW * G * kHeadDim * 4;
   __shared__ __attribute__((aligned(16))) char big_lds[kVBytes > kMergeBytes ? kVBytes : kMergeBytes];
   uint16_t (*v_lds)[kMfVStride] = (uint16_t (*)[kMfVStride])(big_lds + (size_t)(threadIdx.x >> 6) * kMfTok * kMfVStride * 2);
+  // K tile of the wave's block: rows of 256 + 16 bytes (the 16 lanes of an operand read phase
+  // hit 64 distinct banks)
+  __shared__ __attribute__((aligned(16))) uint16_t k_tiles[NW][kMfTok][kMfKStride];
+  uint16_t (*k_lds)[kMfKStride] = k_tiles[threadIdx.x >> 6];
   float (*tile)[G][kHeadDim] = (float (*)[G][kHeadDim])big_lds;
 
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
@@ -459,29 +464,31 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
   const uint16_t* mrow = p.mask ? p.mask + (long)b * p.mask_bs : nullptr;
   const int safe_row = t_begin < S ? t_begin : 0;  // a readable row for out-of-range lanes
 
+  // K and V are both loaded in the natural layout (a load instruction covers four whole token
+  // rows = 1 KB of a dense cache; loading K straight in operand layout would touch 16 rows x 64
+  // bytes per instruction, which streams markedly slower) and reach the MFMAs through LDS.
   struct Block {
-    u32x4 k[2][4];  // [token half][d step]: token base + 16 * half + i, chunk g + 4 * step
-    u32x4 v[8];     // token base + 4 * u + g, chunk i
+    u32x4 k[8];  // token base + 4 * u + g, chunk i
+    u32x4 v[8];
   };
   auto load_block = [&](int base, Block& q) {
 #pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-      const int tok = base + 16 * h2 + i;
-      const uint16_t* rp = kc + (long)(tok < t_end ? tok : safe_row) * p.c_ts + g * 8;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q.k[h2][j] = ld16(rp + j * 32);
-    }
-#pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int tok = base + 4 * u + g;
-      q.v[u] = ld16(vc + (long)(tok < t_end ? tok : safe_row) * p.c_ts + i * 8);
+      const long off = (long)(tok < t_end ? tok : safe_row) * p.c_ts + i * 8;
+      q.k[u] = ld16_sel<!DIRECT>(kc + off);
+      q.v[u] = ld16_sel<!DIRECT>(vc + off);
     }
   };
 
-  Block ba, bb;
-  int base = t_begin + wave * kMfTok;
-  bool have_a = base < t_end;
-  if (have_a) load_block(base, ba);
+  // (K/V loads are never behind a branch, see attn_decode_kernel: blocks past the end read the
+  // safe row and are masked out by their token indices)
+  // One register set: the LDS tiles hold the block being multiplied while the registers
+  // already receive the next one.
+  Block blk;
+  const int base0 = t_begin + wave * kMfTok;
+  const int n_blk = base0 < t_end ? (t_end - base0 + kBlock - 1) / kBlock : 0;  // blocks of this wave
+  load_block(base0, blk);
 
   // ---- rotate the G query heads into LDS (rows >= G stay zero: the padded MFMA columns) ----
   for (int e = t; e < 16 * kHeadDim; e += kAttnThreads) {
@@ -520,28 +527,28 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
 #pragma unroll
   for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  auto attend = [&](int base, Block& q) {
-    // the new token's row comes from LDS, never from the cache slot written above
-    if (owner && slot >= base && slot < base + kMfTok) {
+  auto park = [&](int base, const Block& q) {
+    // K and V (natural layout) into this wave's tiles
 #pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2)
-        if (base + 16 * h2 + i == slot) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) q.k[h2][j] = *(const u32x4*)&kn_lds[(g + 4 * j) * 8];
-        }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (base + 4 * u + g == slot) q.v[u] = *(const u32x4*)&vn_lds[i * 8];
+    for (int u = 0; u < 8; ++u) {
+      *(u32x4*)&k_lds[4 * u + g][i * 8] = q.k[u];
+      *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
     }
-    // park V (natural layout) in this wave's tile
-#pragma unroll
-    for (int u = 0; u < 8; ++u) *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
-
+    // the new token's row comes from LDS, never from the cache slot written above: it
+    // overwrites its row of the tiles (LDS operations of a wave execute in order)
+    if (owner && slot >= base && slot < base + kMfTok && g == 0) {
+      *(u32x4*)&k_lds[slot - base][i * 8] = *(const u32x4*)&kn_lds[i * 8];
+      *(u32x4*)&v_lds[slot - base][i * 8] = *(const u32x4*)&vn_lds[i * 8];
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto attend = [&](int base, auto masked) {
     f32x4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      s1 = attn_mfma<T>(q.k[0][j], qreg[j], s1);
-      s2 = attn_mfma<T>(q.k[1][j], qreg[j], s2);
+      // A operands: token 16 * half + i, chunk g + 4 * step
+      s1 = attn_mfma<T>(*(const u32x4*)&k_lds[i][(g + 4 * j) * 8], qreg[j], s1);
+      s2 = attn_mfma<T>(*(const u32x4*)&k_lds[16 + i][(g + 4 * j) * 8], qreg[j], s2);
     }
     float sc[8];
     float m_loc = -INFINITY;
@@ -549,7 +556,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
     for (int r = 0; r < 8; ++r) {
       const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
       bool ok = tok < t_end;
-      if (mrow != nullptr && ok) ok = T::one(mrow[tok]) == 0.f;
+      if constexpr (decltype(masked)::value) ok = ok && T::one(ld2(mrow + (ok ? tok : 0))) == 0.f;
       const float raw = r < 4 ? s1[r] : s2[r - 4];
       sc[r] = ok ? raw * p.scale_log2 : -INFINITY;
       m_loc = fmaxf(m_loc, sc[r]);
@@ -584,18 +591,16 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
     }
   };
 
-  for (;;) {
-    if (!have_a) break;
-    const int nb = base + kBlock;
-    const bool have_b = nb < t_end;
-    if (have_b) load_block(nb, bb);
-    attend(base, ba);
-    if (!have_b) break;
-    base = nb + kBlock;
-    have_a = base < t_end;
-    if (have_a) load_block(base, ba);
-    attend(nb, bb);
-  }
+  auto sweep = [&](auto masked) {
+    for (int kb = 0; kb < n_blk; ++kb) {
+      const int base = base0 + kb * kBlock;
+      park(base, blk);
+      load_block(base + kBlock, blk);
+      attend(base, masked);
+      __builtin_amdgcn_wave_barrier();  // the tiles are rewritten by the next park
+    }
+  };
+  if (mrow != nullptr) sweep(std::true_type{}); else sweep(std::false_type{});
 
   // ---- the wave's totals: l summed over the four lane groups (m is already shared) ----
   l += __shfl_xor(l, 16);
@@ -932,13 +937,13 @@ constexpr int unroll_for(int nw) { return nw == 16 ? 2 : 4; }
 static int g_attn_waves = 0;  // 0: built-in choice; 4, 8 or 16 forces the workgroup size
 static int g_attn_head_parallel = 1;  // unsplit decodes at small batch: workgroup per query head
 static int g_attn_direct_tokens = 0;  // 0: built-in choice; longest sequence decoded unsplit
-// Shortest sequence that takes the matrix-core kernel; <= 0: never (the built-in choice: on
-// MI355X it measured 250 us against 176 us for the vector kernel at 32k context, batch 8 --
-// its per-block dependency chain (loads, LDS round trip, two MFMA chains, shuffles) is longer
-// than two waves per SIMD can hide -- so it stays an option for experiments).
+// Matrix-core kernel (attn_decode_mfma_kernel). 0 = built-in choice: whenever a workgroup
+// handles a whole KV group, i.e. everywhere except the unsplit head-parallel mode of short
+// sequences (32k context: 30 vs 35 us at batch 1, 163 vs 174 us at batch 8; on par at 1k).
+// > 0: also instead of the head-parallel mode from that many tokens on; < 0: never.
 static int g_attn_mfma_tokens = 0;
 
-static inline bool attn_use_mfma(const AttnParams& p) {
+static inline bool attn_force_mfma(const AttnParams& p) {
   if (g_attn_mfma_tokens <= 0) return false;
   const int hint = p.seq_len > 0 ? p.seq_len : p.max_t;
   return hint >= g_attn_mfma_tokens;
@@ -962,7 +967,7 @@ template <typename T, int G>
 static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
   dim3 grid(p.n_splits, p.hq / G, batch);
   const int nw = attn_waves_for(G);
-  if (G == p.hq / p.hkv && attn_use_mfma(p)) {
+  if (G == p.hq / p.hkv && g_attn_mfma_tokens >= 0) {
     if (p.n_splits == 1)
       hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, true>), grid, dim3(8 * kWave), 0, s, p);
     else
@@ -987,7 +992,7 @@ static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
 template <typename T>
 static int launch_attn_t(hipStream_t s, const AttnParams& p, int batch) {
   // unsplit and too few KV heads to occupy the GPU: one workgroup per query head
-  if (p.n_splits == 1 && g_attn_head_parallel && batch * p.hkv * 8 <= device_cus() && !attn_use_mfma(p))
+  if (p.n_splits == 1 && g_attn_head_parallel && batch * p.hkv * 8 <= device_cus() && !attn_force_mfma(p))
     return launch_attn_g<T, 1>(s, p, batch);
   switch (p.hq / p.hkv) {
     case 1: return launch_attn_g<T, 1>(s, p, batch);

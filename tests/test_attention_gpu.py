@@ -20,13 +20,16 @@ D = 128
 ATOL = 2e-3
 
 
-@pytest.fixture(params=["auto", "matrix-core"], autouse=True)
+@pytest.fixture(params=["auto", "matrix-core", "vector"], autouse=True)
 def attention_kernel_choice(request):
-    """Every test runs twice: with the built-in kernel choice, and with the matrix-core decode
-    kernel forced for every sequence length (it is otherwise reserved for long sequences)."""
+    """Every test runs three times: with the built-in kernel choice (matrix-core decode kernel
+    except in the unsplit one-workgroup-per-query-head mode of short sequences), with the
+    matrix-core kernel forced everywhere, and with the vector-ALU kernel only."""
     lib = _lib.load()
     if request.param == "matrix-core":
         _lib.check(lib.mui_tune_attention(0, 0, 0, 1), "mui_tune_attention")
+    elif request.param == "vector":
+        _lib.check(lib.mui_tune_attention(0, 0, 0, -1), "mui_tune_attention")
     yield request.param
     _lib.check(lib.mui_tune_attention(0, 0, 0, 0), "mui_tune_attention")
 
