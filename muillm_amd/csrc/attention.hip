@@ -682,6 +682,8 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
   __shared__ __attribute__((aligned(16))) char big_lds[kVBytes > kMergeBytes ? kVBytes : kMergeBytes];
   uint16_t (*v_lds)[kMfVStride] = (uint16_t (*)[kMfVStride])(big_lds + (size_t)(threadIdx.x >> 6) * kMfTok * kMfVStride * 2);
   float (*tile)[16][kHeadDim] = (float (*)[16][kHeadDim])big_lds;
+  __shared__ __attribute__((aligned(16))) uint16_t k_tiles[NW][kMfTok][kMfKStride];
+  uint16_t (*k_lds)[kMfKStride] = k_tiles[threadIdx.x >> 6];
 
   const int t0 = blockIdx.x * 16, head = blockIdx.y, b = blockIdx.z;
   const int kvh = head / (p.hq / p.hkv);
@@ -702,29 +704,27 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
   const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
   const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
 
+  // K and V in their natural layout (four whole token rows per load instruction), through LDS
+  // tiles into the MFMAs; one register set, the tiles being the second buffer; no load behind a
+  // branch (see attn_decode_mfma_kernel)
   struct Block {
-    u32x4 k[2][4];
+    u32x4 k[8];  // token base + 4 * u + g, chunk i
     u32x4 v[8];
   };
   auto load_block = [&](int base, Block& q) {
 #pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-      const int tok = base + 16 * h2 + i;
-      const uint16_t* rp = kc + (long)(tok < kv_end ? tok : 0) * p.c_ts + g * 8;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q.k[h2][j] = ld16(rp + j * 32);
-    }
-#pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int tok = base + 4 * u + g;
-      q.v[u] = ld16(vc + (long)(tok < kv_end ? tok : 0) * p.c_ts + i * 8);
+      const long off = (long)(tok < kv_end ? tok : 0) * p.c_ts + i * 8;
+      q.k[u] = ld16(kc + off);
+      q.v[u] = ld16(vc + off);
     }
   };
 
-  Block ba, bb;
-  int base = wave * kMfTok;
-  bool have_a = base < kv_end;
-  if (have_a) load_block(base, ba);
+  Block blk;
+  const int base0 = wave * kMfTok;
+  const int n_blk = base0 < kv_end ? (kv_end - base0 + kBlock - 1) / kBlock : 0;
+  load_block(base0, blk);
 
   for (int e = t; e < 16 * kHeadDim; e += kAttnThreads) {
     const int qi = e / kHeadDim, d = e % kHeadDim;
@@ -742,14 +742,21 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
 #pragma unroll
   for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  auto attend = [&](int base, Block& q) {
+  auto park = [&](const Block& q) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
+    for (int u = 0; u < 8; ++u) {
+      *(u32x4*)&k_lds[4 * u + g][i * 8] = q.k[u];
+      *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+  auto attend = [&](int base) {
     f32x4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      s1 = attn_mfma<T>(q.k[0][j], qreg[j], s1);
-      s2 = attn_mfma<T>(q.k[1][j], qreg[j], s2);
+      // A operands: token 16 * half + i, chunk g + 4 * step
+      s1 = attn_mfma<T>(*(const u32x4*)&k_lds[i][(g + 4 * j) * 8], qreg[j], s1);
+      s2 = attn_mfma<T>(*(const u32x4*)&k_lds[16 + i][(g + 4 * j) * 8], qreg[j], s2);
     }
     float sc[8];
     float m_loc = -INFINITY;
@@ -790,17 +797,12 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
     }
   };
 
-  for (;;) {
-    if (!have_a) break;
-    const int nb = base + kBlock;
-    const bool have_b = nb < kv_end;
-    if (have_b) load_block(nb, bb);
-    attend(base, ba);
-    if (!have_b) break;
-    base = nb + kBlock;
-    have_a = base < kv_end;
-    if (have_a) load_block(base, ba);
-    attend(nb, bb);
+  for (int kb = 0; kb < n_blk; ++kb) {
+    const int base = base0 + kb * kBlock;
+    park(blk);
+    load_block(base + kBlock, blk);
+    attend(base);
+    __builtin_amdgcn_wave_barrier();  // the tiles are rewritten by the next park
   }
 
   l += __shfl_xor(l, 16);
