@@ -440,7 +440,7 @@ def main():
             result["variants"]["fp16_context%d_tokens_per_s" % ctx] = round(64 / dt_c, 2)
             del dec_c
             torch.cuda.empty_cache()
-        for bsz in (4, 8):
+        for bsz in (4, 8, 16):
             dt_b, dec_b = bench_decode(lm, min(args.steps, 128), min(args.warmup, 8), batch=bsz)
             result["variants"]["fp16_batch%d_aggregate_tokens_per_s" % bsz] = round(bsz * min(args.steps, 128) / dt_b, 1)
             result["variants"]["fp16_batch%d_ms_per_step" % bsz] = round(dt_b / min(args.steps, 128) * 1e3, 4)
