@@ -275,20 +275,29 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
     for (int u = 0; u < U; ++u) madd[u] = 0.f;
     auto sweep = [&](auto masked) {
       if constexpr (kPipe) {
-        // two register sets: the next block is in flight while the current one is consumed
-        // (an odd block count ends with one block that is not live)
-        for (int bi = 0; bi < n_blocks; bi += 2) {
+        // two register sets: the next block is in flight while the current one is consumed;
+        // the branch-free rounds run while both of their fetches are real, the last one or
+        // two blocks are peeled (short sequences consist of that tail only)
+        int bi = 0;
+        for (; bi + 2 < n_blocks; bi += 2) {
           fetch(bi + 1, kb, vb, valid_b, masked);
           attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
           fetch(bi + 2, ka, va, valid_a, masked);
           attend_block<T, G, U>(kb, vb, valid_b, madd, qreg, p.scale_log2, m, l, acc);
+        }
+        if (bi + 1 < n_blocks) {
+          fetch(bi + 1, kb, vb, valid_b, masked);
+          attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
+          attend_block<T, G, U>(kb, vb, valid_b, madd, qreg, p.scale_log2, m, l, acc);
+        } else if (bi < n_blocks) {
+          attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
         }
       } else {
         // 4 waves per SIMD overlap each other's loads; one register set keeps the kernel
         // under 128 VGPRs
         for (int bi = 0; bi < n_blocks; ++bi) {
           attend_block<T, G, U>(ka, va, valid_a, madd, qreg, p.scale_log2, m, l, acc);
-          fetch(bi + 1, ka, va, valid_a, masked);
+          if (bi + 1 < n_blocks) fetch(bi + 1, ka, va, valid_a, masked);
         }
       }
     };
