@@ -24,7 +24,7 @@ struct SkinnyParams {
   uint16_t* y;               // [tokens, n]
   int n;       // outputs (weight rows, or gate/up pairs)
   int k;
-  int tokens;  // 2..8 (1 works too)
+  int tokens;  // 1..16
   float eps;
 };
 
@@ -124,7 +124,7 @@ int launch_skinny(hipStream_t s, int dtype, int weight_format, int epilogue, con
 void skinny_set_bstat(int on);
 void skinny_set_lt(int on);  // 0: operands loaded straight from HBM in MFMA order (older kernels)
 
-// 2..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
+// 1..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
 // in registers (gemv_multi.hip); returns MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
 // MFMA skinny GEMM whose weight rows are read as contiguous runs and turned into operands
