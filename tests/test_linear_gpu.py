@@ -149,6 +149,44 @@ def test_linear_small_batch(tokens, n, k):
     assert_parity(y, ref, 1e-2, f"batch {tokens} {n}x{k}", tight=4e-3)
 
 
+@pytest.mark.parametrize("tokens", [5, 9, 16])
+@pytest.mark.parametrize("n,k", [(24, 256), (33, 3840), (64, 4104), (40, 8192), (17, 14336), (130, 2056), (9, 24)])
+@pytest.mark.parametrize("norm", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_small_batch_edge_shapes(tokens, n, k, norm, dtype):
+    """The matrix-core path at its seams: K below / at / above what a workgroup keeps stationary
+    (4096), K that is not a multiple of the 256-value pass, rows that do not fill a 16-row tile,
+    fused norm on long rows (the streaming mode has none and hands over to the direct-operand
+    kernel), with residual and both biases."""
+    g = _gen(40 + tokens)
+    w = _mk((n, k), g, 0.02, dtype=dtype)
+    x = _mk((tokens, k), g, dtype=dtype)
+    gamma = _mk((k,), g, 0.1, 1.0, dtype=dtype) if norm else None
+    r = _mk((tokens, n), g, dtype=dtype)
+    mb = _mk((n,), g, 0.1, 1.0, dtype=dtype)
+    ab = _mk((n,), g, 0.1, dtype=dtype)
+    ref = oracle.linear(x, w, gamma, 1e-5, ab, r, mul_bias=mb)
+    y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), None if gamma is None else gamma.to(DEV),
+                                         1e-5, mul_bias=mb.to(DEV), add_bias=ab.to(DEV), residual=r.to(DEV))
+    assert y.shape == (tokens, n) and y.dtype == dtype
+    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 3e-2, f"edge {tokens} {n}x{k} norm={norm} {dtype}")
+
+
+@pytest.mark.parametrize("tokens", [5, 16])
+@pytest.mark.parametrize("n,k", [(40, 256), (100, 3840), (24, 8192), (9, 2056)])
+@pytest.mark.parametrize("norm", [True, False])
+def test_gateup_small_batch_edge_shapes(tokens, n, k, norm):
+    g = _gen(60 + tokens)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0) if norm else None
+    ref = oracle.gateup_silu(x, wg, wu, gamma, 1e-5)
+    packed = torch.stack((wg, wu), dim=1).to(DEV)
+    h = muillm_ext.mui_gateup_silu(None if gamma is None else gamma.to(DEV), 1e-5, packed[:, 0], packed[:, 1], x.to(DEV))
+    assert h.shape == (tokens, n)
+    assert_parity(h, ref, 1e-2, f"gate/up edge {tokens} {n}x{k} norm={norm}")
+
+
 def test_linear_reference_recipe_batch4():
     """tests/test_linear.py:13-43 of the reference: randn weights (seed 0), rand inputs of
     batch 4, compared with allclose(rtol 1e-4, atol 1e-1)."""
