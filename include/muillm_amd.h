@@ -106,6 +106,14 @@ int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate, const void
                     long gu_pitch, const void* x, const void* norm_weights, float epsilon,
                     void* h, int n_inter, int k_in, int tokens);
 
+/* Activation step of the unfused MLP route for prompts longer than MUI_MAX_TOKENS tokens
+ * (muillm/modules/gateupdownmlp.py:343-359: two matmuls, SiLU, multiply): with the gate and up
+ * rows interleaved in one buffer, one matmul yields gate_up [rows, n, 2] and this call
+ * computes out[r, i] = silu(gate_up[r, i, 0]) * gate_up[r, i, 1] (fp32 math, one rounding).
+ * n % 8 == 0; 16-byte aligned buffers. */
+int mui_silu_mul_interleaved(mui_stream_t stream, int dtype, const void* gate_up, void* out,
+                             long rows, int n);
+
 /* ------------------------------------------------------------------------------------
  * int8 weight-only family
  * ---------------------------------------------------------------------------------- */

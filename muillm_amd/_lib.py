@@ -49,6 +49,7 @@ _SIGNATURES = {
     "mui_linear": (c_int, [_P, c_int, _P, c_long, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_int]),
     "mui_rmsnorm": (c_int, [_P, c_int, _P, _P, c_float, _P, c_int, c_int]),
     "mui_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
+    "mui_silu_mul_interleaved": (c_int, [_P, c_int, _P, _P, c_long, c_int]),
     "mui_int8_linear": (c_int, [_P, c_int, _P, c_long, _P, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int]),
     "mui_int8_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
     "mui_int8_group_linear": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int]),

@@ -103,3 +103,49 @@ extern "C" int mui_rmsnorm(mui_stream_t stream, int dtype, const void* weights, 
     return launch_rmsnorm<BF16>(s, (const uint16_t*)weights, (const uint16_t*)x, (uint16_t*)y, rows, k, epsilon);
   return MUI_ERR_INVALID_ARG;
 }
+
+// ---------------------------------------------------------------------------------------
+// SiLU(gate) * up on an interleaved [rows, n, 2] buffer (the output of ONE matmul with the
+// row-interleaved gate/up weights, used for prompts too long for the fused GEMV family):
+// out[r, i] = silu(gu[r, 2i]) * gu[r, 2i + 1], fp32 math, one rounding.
+// The reference runs two matmuls, an activation kernel and a multiply
+// (muillm/modules/gateupdownmlp.py:343-359).
+// ---------------------------------------------------------------------------------------
+namespace mui {
+template <typename T>
+__global__ void __launch_bounds__(256) silu_mul_interleaved_kernel(const uint16_t* gu, uint16_t* out, long total8) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long c = (long)blockIdx.x * blockDim.x + threadIdx.x; c < total8; c += stride) {
+    const u32x4 a = ld16(gu + c * 16), b = ld16(gu + c * 16 + 8);
+    float fa[8], fb[8], o[8];
+    unpack8<T>(a, fa);
+    unpack8<T>(b, fb);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[i] = silu_f32(fa[2 * i]) * fa[2 * i + 1];
+      o[4 + i] = silu_f32(fb[2 * i]) * fb[2 * i + 1];
+    }
+    *(u32x4*)(out + c * 8) = pack8<T>(o);
+  }
+}
+}  // namespace mui
+
+extern "C" int mui_silu_mul_interleaved(mui_stream_t stream, int dtype, const void* gate_up, void* out,
+                                        long rows, int n) {
+  MUI_CHECK_ARG(gate_up && out && rows > 0 && n > 0);
+  MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
+  if (n % 8) return MUI_ERR_UNSUPPORTED;
+  if ((((uintptr_t)gate_up | (uintptr_t)out) & 15u) != 0) return MUI_ERR_ALIGNMENT;
+  const long total8 = rows * (n / 8);
+  long blocks = (total8 + 255) / 256;
+  const long cap = (long)mui::device_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MUI_DTYPE_F16)
+    hipLaunchKernelGGL((mui::silu_mul_interleaved_kernel<mui::F16>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       (const uint16_t*)gate_up, (uint16_t*)out, total8);
+  else
+    hipLaunchKernelGGL((mui::silu_mul_interleaved_kernel<mui::BF16>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       (const uint16_t*)gate_up, (uint16_t*)out, total8);
+  return mui::launch_status();
+}

@@ -181,6 +181,14 @@ class MuiGateUpDownMLP(MuiModule):
                 h = input.to(torch.float32)
                 h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
                 input = self.norm_weights * h.to(input.dtype)
+        packed = self.gate_up_packed
+        if (packed is not None and input.is_cuda and input.dtype == packed.dtype and self.intermediate_size % 8 == 0
+                and self.gate_proj.bias is None and self.up_proj.bias is None
+                and self.gate_proj.weight.data_ptr() == packed.data_ptr()):
+            # long prompts: ONE matmul over the interleaved gate/up rows, one SiLU*mul kernel, and
+            # the residual in the epilogue of the down projection
+            gu = torch.nn.functional.linear(input, packed.view(2 * self.intermediate_size, self.hidden_size))
+            return self.down_proj(muillm_ext.mui_silu_mul_interleaved(gu), residual=residual)
         g = self.gate_proj(input)
         u = self.up_proj(input)
         output = self.down_proj(self.activation_function(g) * u)

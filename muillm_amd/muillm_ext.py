@@ -128,6 +128,11 @@ def _linear_unfused(x, weights, norm_weights, epsilon, mul_bias, add_bias, resid
     """The reference's non-single-token branch (csrc/modules/linear_module.cpp:57-79)."""
     if norm_weights is not None:
         x = muillm_rmsnorm_forward(norm_weights, x, epsilon) if (x.is_cuda and _is_16bit(x)) else _rmsnorm_torch(x, norm_weights, epsilon)
+    if residual is not None and mul_bias is None and x.is_cuda and _is_16bit(x) and residual.dtype == x.dtype:
+        # the residual (and bias) ride in the GEMM epilogue: one kernel, one rounding
+        out = torch.addmm(residual.reshape(-1, weights.shape[0]), x.reshape(-1, x.shape[-1]), weights.t())
+        out = out.reshape(x.shape[:-1] + (weights.shape[0],))
+        return out if add_bias is None else out + add_bias
     out = F.linear(x, weights, None)
     if mul_bias is not None:
         out = out * mul_bias
@@ -245,6 +250,17 @@ def mui_gateup_silu(norm_weights, epsilon, gate_weights, up_weights, x) -> torch
         "mui_gateup_silu",
     )
     return h
+
+
+def mui_silu_mul_interleaved(gate_up: torch.Tensor) -> torch.Tensor:
+    """[..., 2 * n] with (gate, up) pairs adjacent -> silu(gate) * up, [..., n]."""
+    _check_cuda(gate_up, "gate_up")
+    n = gate_up.shape[-1] // 2
+    gu = gate_up if gate_up.is_contiguous() else gate_up.contiguous()
+    out = torch.empty(gu.shape[:-1] + (n,), dtype=gu.dtype, device=gu.device)
+    check(_lib.load().mui_silu_mul_interleaved(_stream(gu), _dtype_code(gu), gu.data_ptr(), out.data_ptr(),
+                                               gu.numel() // (2 * n), n), "mui_silu_mul_interleaved")
+    return out
 
 
 def muillm_gateupsilu_forward(engine, norm_weights, epsilon, gate_weights, up_weights, down_weights,

@@ -187,6 +187,17 @@ def test_gateup_small_batch_edge_shapes(tokens, n, k, norm):
     assert_parity(h, ref, 1e-2, f"gate/up edge {tokens} {n}x{k} norm={norm}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,n", [(17, 64), (300, 14336), (5, 8)])
+def test_silu_mul_interleaved(rows, n, dtype):
+    g = _gen(70)
+    gu = _mk((rows, 2 * n), g, dtype=dtype)
+    ref = torch.nn.functional.silu(gu[:, 0::2].double()) * gu[:, 1::2].double()
+    out = muillm_ext.mui_silu_mul_interleaved(gu.to(DEV))
+    assert out.shape == (rows, n) and out.dtype == dtype
+    assert_parity(out, ref.float(), 1e-2, f"silu*mul {rows}x{n}")
+
+
 def test_linear_reference_recipe_batch4():
     """tests/test_linear.py:13-43 of the reference: randn weights (seed 0), rand inputs of
     batch 4, compared with allclose(rtol 1e-4, atol 1e-1)."""

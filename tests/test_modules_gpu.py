@@ -107,6 +107,31 @@ def test_multilinear_and_mlp_modules(ctx):
         assert_parity(out, oracle.gateupdown_mlp(xx, wg, wu, wd, norm_w, 1e-5, rr), 1e-2, f"MuiGateUpDownMLP b={tokens}")
 
 
+@pytest.mark.parametrize("tokens", [17, 100])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_mlp_module_long_prompt_route(ctx, tokens, dtype):
+    """More tokens than the fused GEMV family takes: one matmul over the interleaved gate/up rows,
+    the SiLU*mul kernel, residual in the down projection's epilogue."""
+    torch.manual_seed(11)
+    hid, inter = 256, 704
+    mlp = MuiGateUpDownMLP(MuiEngineConfig(), hid, inter, torch.nn.SiLU(), variance_epsilon=1e-5, normalize=True,
+                           device=DEV, dtype=dtype)
+    with torch.no_grad():
+        for lin in (mlp.gate_proj, mlp.up_proj, mlp.down_proj):
+            lin.weight.copy_(torch.randn_like(lin.weight) * 0.05)
+        mlp.norm_weights.copy_(1 + 0.1 * torch.randn_like(mlp.norm_weights))
+    mlp.finalize_init()
+    assert mlp.gate_up_packed is not None
+    x = torch.randn(2, tokens, hid, device=DEV, dtype=dtype)
+    r = torch.randn(2, tokens, hid, device=DEV, dtype=dtype)
+    ref = oracle.gateupdown_mlp(x.cpu(), mlp.gate_proj.weight.detach().cpu(), mlp.up_proj.weight.detach().cpu(),
+                     mlp.down_proj.weight.detach().cpu(), mlp.norm_weights.detach().cpu(), 1e-5, r.cpu())
+    with torch.no_grad():
+        y = mlp(x, residual=r)
+    assert y.shape == x.shape
+    assert_parity(y, ref, 2e-2 if dtype == torch.float16 else 4e-2, f"long-prompt MLP {tokens}")
+
+
 def _small_config(layers=2):
     return MuiDecoderConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=layers,
                             num_attention_heads=4, num_key_value_heads=2, vocab_size=1024,
