@@ -34,6 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 # (x2.0000 to KiB) and 114,783.2 for the GEMV; WRITE_SIZE reads 229,376.0 for the copy (x1.0) and 224.0 for
 # the GEMV. 235,038,826 B fetched + 229,417 B written.
 GATEUP_TRAFFIC_BYTES = 235038826 + 229417
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16 matrix-core peak
 BASELINE_TOKENS_PER_S = 210.0  # reference README: Llama-3-8B fp16 bs1 on 1x MI300X
 
 
@@ -187,9 +188,9 @@ def kernel_table(lm):
     stream = torch.cuda.current_stream().cuda_stream
     f16 = dict(device="cuda", dtype=torch.float16)
     gamma = (1 + 0.1 * torch.randn(hid)).half().cuda()
-    X, RES = torch.randn(8, hid, **f16), torch.randn(8, hid, **f16)
+    X, RES = torch.randn(16, hid, **f16), torch.randn(16, hid, **f16)
     HMID = torch.randn(8, inter, **f16)
-    Y = torch.empty(8 * max(v, inter), **f16)
+    Y = torch.empty(16 * max(v, inter), **f16)
     out = {}
 
     def add(name, fn, nbytes, ring, iters=10):
@@ -220,15 +221,23 @@ def kernel_table(lm):
     # ---- C2: the whole MLP (fused norm + gate/up + SiLU, then down + residual), 1..8 tokens
     gu = [(l.mlp.gate_proj.weight.data_ptr(), l.mlp.up_proj.weight.data_ptr(), l.mlp.gate_proj.weight.stride(0),
            l.mlp.norm_weights.data_ptr()) for l in layers]
-    hbuf = torch.empty(8, inter, **f16)
-    for b in (1, 2, 4, 8):
+    hbuf = torch.empty(16, inter, **f16)
+    for b in (1, 2, 4, 8, 16):
         def mlp(i, b=b):
             gp, up, pitch, nw = gu[i % nl]
             lib.mui_gateup_silu(stream, 0, gp, up, pitch, X.data_ptr(), nw, 1e-5, hbuf.data_ptr(), inter, hid, b)
             lib.mui_linear(stream, 0, dn[i % nl], inter, hbuf.data_ptr(), None, 0.0, None, None, RES.data_ptr(),
                            Y.data_ptr(), hid, inter, b)
-        add("C2_mlp_%dx%d_tokens%d" % (inter, hid, b), mlp,
-            3 * inter * hid * 2 + 2 * hid + b * (3 * hid * 2 + 2 * inter * 2), nl)
+        name = "C2_mlp_%dx%d_tokens%d" % (inter, hid, b)
+        add(name, mlp, 3 * inter * hid * 2 + 2 * hid + b * (3 * hid * 2 + 2 * inter * 2), nl)
+        # arithmetic rate of the batched call; from 5 tokens on it runs on the matrix cores (padded
+        # to 16 token columns), whose utilisation is this rate over the dense fp16 MFMA peak
+        tflops = 6.0 * inter * hid * b / out[name]["us"] / 1e6
+        out[name]["TFLOP/s"] = round(tflops, 1)
+        out[name]["compute_unit"] = "MFMA v_mfma_f32_16x16x32_f16" if b >= 5 else "vector ALUs"
+        if b >= 5:
+            out[name]["mfma_peak_frac"] = round(tflops / MFMA_FP16_PEAK_TFLOPS, 4)
+            out[name]["mfma_issued_frac"] = round(tflops * 16.0 / b / MFMA_FP16_PEAK_TFLOPS, 4)
 
     # ---- C3: int8 per-channel GEMVs (ring of random codes: speed does not depend on the values)
     def i8_ring(n, k):
