@@ -171,6 +171,35 @@ def pmc_probe(launches=6):
                                     "copy_bytes_read": dst.numel() * 2, "copy_bytes_written": dst.numel() * 2}}))
 
 
+def pmc_probe_batched(launches=6, tokens=8):
+    """Counter probe for the batched (matrix-core) MLP: a few launches of the fused gate/up and of
+    the down projection at `tokens` tokens, Llama-3-8B shape, over distinct weight buffers
+    (`rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES`,
+    and `--pmc FETCH_SIZE` for the traffic)."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    hid, inter = 4096, 14336
+    f16 = dict(device="cuda", dtype=torch.float16)
+    gu = [torch.randn(inter, 2, hid, **f16) * 0.02 for _ in range(launches)]
+    dn = [torch.randn(hid, inter, **f16) * 0.02 for _ in range(launches)]
+    x, gamma = torch.randn(tokens, hid, **f16), torch.ones(hid, **f16)
+    h, res, y = torch.empty(tokens, inter, **f16), torch.randn(tokens, hid, **f16), torch.empty(tokens, hid, **f16)
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    for w, d in zip(gu, dn):
+        _lib.check(lib.mui_gateup_silu(stream, 0, w[:, 0].data_ptr(), w[:, 1].data_ptr(), 2 * hid, x.data_ptr(),
+                                       gamma.data_ptr(), 1e-5, h.data_ptr(), inter, hid, tokens), "mui_gateup_silu")
+        _lib.check(lib.mui_linear(stream, 0, d.data_ptr(), inter, h.data_ptr(), None, 0.0, None, None, res.data_ptr(),
+                                  y.data_ptr(), hid, inter, tokens), "mui_linear")
+    torch.cuda.synchronize()
+    print(json.dumps({"pmc_probe_batched": {"launches": launches, "tokens": tokens,
+                                            "gateup_flops": 4 * inter * hid * tokens, "down_flops": 2 * inter * hid * tokens,
+                                            "gateup_weight_bytes": 4 * inter * hid, "down_weight_bytes": 2 * inter * hid}}))
+
+
 def kernel_table(lm):
     """GB/s of each fused kernel family at the benchmark shapes, HIP-event timed through the C ABI
     with pre-allocated outputs. Weights rotate over distinct buffers totalling >= 0.9 GB (the model's
@@ -379,6 +408,8 @@ def main():
                     help="only time the per-kernel table (for rocprofv3 kernel traces of the C1-C4 shapes)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
+    ap.add_argument("--pmc-probe-batched", action="store_true",
+                    help="launch the 8-token MLP kernels a few times and exit (for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (no tensor parallelism, no collectives); "
@@ -393,6 +424,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.pmc_probe:
         pmc_probe()
+        return
+    if args.pmc_probe_batched:
+        pmc_probe_batched()
         return
     if args.tune_attention:
         from muillm_amd import _lib
