@@ -200,6 +200,42 @@ def pmc_probe_batched(launches=6, tokens=8):
                                             "gateup_weight_bytes": 4 * inter * hid, "down_weight_bytes": 2 * inter * hid}}))
 
 
+def pmc_probe_attention(launches=3):
+    """Counter probe for flash decoding (`rocprofv3 --pmc FETCH_SIZE`): fused RoPE + cache write +
+    attention at 32k context, batch 8 and batch 1, over distinct caches."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    hq, hkv, d = 32, 8, 128
+    f16 = dict(device="cuda", dtype=torch.float16)
+    stream = torch.cuda.current_stream().cuda_stream
+    info = {}
+    for S, B in ((32768, 8), (32768, 1)):
+        caches = [(torch.randn(B, hkv, S, d, **f16), torch.randn(B, hkv, S, d, **f16)) for _ in range(launches)]
+        qkvx = torch.randn(B, (hq + 2 * hkv) * d, **f16)
+        cos, sin = [t.cuda() for t in _rope_tables_f32(S, d)]
+        pos = torch.full((B, 1), S - 1, dtype=torch.int64, device="cuda")
+        cpos = torch.full((1,), S - 1, dtype=torch.int64, device="cuda")
+        n_splits = lib.mui_flash_decode_splits(B, hq, hkv, S)
+        scratch = torch.empty(max(lib.mui_flash_decode_scratch_bytes(B, hq, d, n_splits), 16), dtype=torch.uint8, device="cuda")
+        o = torch.empty(B, hq * d, **f16)
+        qs = (hq + 2 * hkv) * d
+        torch.cuda.synchronize()
+        for kc, vc in caches:
+            _lib.check(lib.mui_attn_decode_fused(
+                stream, 0, qkvx.data_ptr(), qs, qkvx.data_ptr() + 2 * hq * d, qs, qkvx.data_ptr() + 2 * (hq + hkv) * d, qs,
+                cos.data_ptr(), sin.data_ptr(), d // 2, pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
+                hkv * S * d, S * d, d, None, 0, None, scratch.data_ptr(), n_splits, o.data_ptr(), B, hq, hkv, d, S),
+                "mui_attn_decode_fused")
+        torch.cuda.synchronize()
+        info["ctx%d_batch%d" % (S, B)] = {"kv_bytes": B * 2 * hkv * S * d * 2, "n_splits": n_splits}
+        del caches
+        torch.cuda.empty_cache()
+    print(json.dumps({"pmc_probe_attention": info}))
+
+
 def kernel_table(lm):
     """GB/s of each fused kernel family at the benchmark shapes, HIP-event timed through the C ABI
     with pre-allocated outputs. Weights rotate over distinct buffers totalling >= 0.9 GB (the model's
@@ -410,6 +446,8 @@ def main():
                     help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
     ap.add_argument("--pmc-probe-batched", action="store_true",
                     help="launch the 8-token MLP kernels a few times and exit (for rocprofv3 --pmc)")
+    ap.add_argument("--pmc-probe-attention", action="store_true",
+                    help="launch flash decoding at 32k context a few times and exit (for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (no tensor parallelism, no collectives); "
@@ -427,6 +465,9 @@ def main():
         return
     if args.pmc_probe_batched:
         pmc_probe_batched()
+        return
+    if args.pmc_probe_attention:
+        pmc_probe_attention()
         return
     if args.tune_attention:
         from muillm_amd import _lib
