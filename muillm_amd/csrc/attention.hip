@@ -8,7 +8,9 @@
 // Layout of the work (T = 1 new token per batch row, head_dim 128):
 //   grid = (splits of the cached sequence, blocks of G query heads, batch).
 //   Normally G = Hq/Hkv: a workgroup serves ALL query heads that share its KV head, so K and V
-//   are read from HBM exactly once (the reference re-reads them once per query head).
+//   are read from HBM exactly once (the reference re-reads them once per query head); that
+//   shape runs on the matrix cores (attn_decode_mfma_kernel below). What follows describes the
+//   vector-ALU kernel, which serves the other shape:
 //   Short sequences at small batch are latency-bound instead: there the launcher uses G = 1
 //   and no sequence split (one workgroup per query head, the few hundred KB of K/V re-read
 //   from cache by the heads of a group), which needs no second kernel to merge splits.
@@ -382,19 +384,24 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
 }
 
 // ---------------------------------------------------------------------------------------
-// Matrix-core formulation for long sequences. Same grid and merge as above with G = Hq/Hkv,
-// but a wave now owns blocks of 32 consecutive tokens:
+// Matrix-core formulation: the kernel the launcher uses whenever a workgroup serves a whole KV
+// group (G = Hq/Hkv; the vector kernel above keeps the unsplit G = 1 mode of short sequences).
+// Same grid and merge as above, but a wave now owns blocks of 32 consecutive tokens. K and V
+// are both loaded in their natural layout (lane = 16-byte chunk of a token row, four whole
+// rows per instruction), parked in wave-private LDS tiles and read from there: loading K
+// straight in MFMA operand layout touches 16 rows x 64 bytes per instruction and streams
+// markedly slower. One register set; the tiles hold the block being multiplied while the
+// registers receive the next one.
 //   scores   S^T[token, head] = K[token, :] . q[head, :]   two v_mfma_f32_16x16x32 chains over
-//            D = 128 (A = K rows loaded straight from the cache in operand layout: lane
-//            (g = lane / 16, i = lane % 16) holds 16-byte chunk g + 4j of token i; B = rotated
+//            D = 128 (A = K rows from the LDS tile in operand layout: lane
+//            (g = lane / 16, i = lane % 16) reads 16-byte chunk g + 4j of token i; B = rotated
 //            q of head i from LDS, zero for i >= G). C puts head i's scores of tokens 4g + r
 //            (r < 4) in lane (g, i): softmax needs one running max per lane column, shared by
 //            the four lane groups with two shuffles.
 //   output   O^T[d, head] += V^T[d, token] . P[token, head]   8 MFMAs (16 values of d each),
 //            contraction over the block's 32 tokens. P comes straight from the score
-//            registers (k-slots of lane group g = tokens 4g + r and 16 + 4g + r). V is loaded
-//            with the natural coalesced mapping, parked in a wave-private LDS tile and read
-//            back TRANSPOSED with ds_read_b64_tr_b16: within a 16-lane group, lane i receives
+//            registers (k-slots of lane group g = tokens 4g + r and 16 + 4g + r). V is read
+//            back from its tile TRANSPOSED with ds_read_b64_tr_b16: within a 16-lane group, lane i receives
 //            element i % 4 of the 8-byte rows addressed by lanes i/4, i/4 + 4, i/4 + 8,
 //            i/4 + 12, i.e. four tokens of one d when those lanes point at token rows
 //            4g .. 4g + 3 at column 16 * block + 4 * (lane % 4).
