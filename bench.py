@@ -258,10 +258,22 @@ def kernel_table(lm):
     Y = torch.empty(16 * max(v, inter), **f16)
     out = {}
 
-    def add(name, fn, nbytes, ring, iters=10):
+    sink = torch.zeros(64, dtype=torch.int32, device="cuda")
+
+    def add(name, fn, nbytes, ring, iters=10, reads=None):
+        """reads: [(buffer pointers, bytes), ...] = the matrices the call streams; the read probe
+        over the same buffers (one launch per matrix the call itself uses a launch for) gives the
+        least time those bytes can take on this device, launch latency included."""
         us = _event_time_us(fn, iters=max(iters * ring, 40), warm=max(ring, 8))
         out[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                      "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3)}
+        if reads:
+            def probe(i):
+                for ptrs, nb in reads:
+                    lib.mui_probe_read(stream, ptrs[i % len(ptrs)], nb, sink.data_ptr())
+            floor = _event_time_us(probe, iters=max(iters * ring, 40), warm=max(ring, 8))
+            out[name]["read_floor_us"] = round(floor, 2)
+            out[name]["vs_read_floor"] = round(floor / us, 3)
 
     def linear(w, xin, norm, resid, n, k, b=1):
         return lambda i: lib.mui_linear(stream, 0, w[i % len(w)], k, xin.data_ptr(), norm, 1e-5, None, None,
@@ -273,19 +285,22 @@ def kernel_table(lm):
     op = [l.self_attn.o_proj.weight.data_ptr() for l in layers]
     dn = [l.mlp.down_proj.weight.data_ptr() for l in layers]
     add("C1_norm_linear_residual_%dx%d" % (hid, hid), linear(op, X, gamma.data_ptr(), RES.data_ptr(), hid, hid),
-        2 * hid * hid + 2 * (4 * hid), nl)
+        2 * hid * hid + 2 * (4 * hid), nl, reads=[(op, 2 * hid * hid)])
     add("qkv_norm_gemv_%dx%d" % (n_qkv, hid), linear(qkv, X, gamma.data_ptr(), None, n_qkv, hid),
-        2 * n_qkv * hid + 2 * (2 * hid + n_qkv), nl)
+        2 * n_qkv * hid + 2 * (2 * hid + n_qkv), nl, reads=[(qkv, 2 * n_qkv * hid)])
     add("o_proj_gemv_residual_%dx%d" % (hid, hid), linear(op, X, None, RES.data_ptr(), hid, hid),
-        2 * hid * hid + 2 * (3 * hid), nl)
+        2 * hid * hid + 2 * (3 * hid), nl, reads=[(op, 2 * hid * hid)])
     add("down_gemv_residual_%dx%d" % (hid, inter), linear(dn, HMID, None, RES.data_ptr(), hid, inter),
-        2 * hid * inter + 2 * (inter + 2 * hid), nl)
+        2 * hid * inter + 2 * (inter + 2 * hid), nl, reads=[(dn, 2 * hid * inter)])
     add("lm_head_gemv_%dx%d" % (v, hid), linear([lm.lm_head.weight.data_ptr()], X, None, None, v, hid),
-        2 * v * hid + 2 * (hid + v), 1, iters=40)
+        2 * v * hid + 2 * (hid + v), 1, iters=40, reads=[([lm.lm_head.weight.data_ptr()], 2 * v * hid)])
 
     # ---- C2: the whole MLP (fused norm + gate/up + SiLU, then down + residual), 1..8 tokens
     gu = [(l.mlp.gate_proj.weight.data_ptr(), l.mlp.up_proj.weight.data_ptr(), l.mlp.gate_proj.weight.stride(0),
            l.mlp.norm_weights.data_ptr()) for l in layers]
+    # gate and up rows interleave in one packed buffer per layer, gate row 0 first
+    gu_base = [min(g[0], g[1]) for g in gu]
+    assert all(abs(g[0] - g[1]) == 2 * hid and g[2] == 2 * hid for g in gu)
     hbuf = torch.empty(16, inter, **f16)
     for b in (1, 2, 4, 8, 16):
         def mlp(i, b=b):
@@ -294,7 +309,8 @@ def kernel_table(lm):
             lib.mui_linear(stream, 0, dn[i % nl], inter, hbuf.data_ptr(), None, 0.0, None, None, RES.data_ptr(),
                            Y.data_ptr(), hid, inter, b)
         name = "C2_mlp_%dx%d_tokens%d" % (inter, hid, b)
-        add(name, mlp, 3 * inter * hid * 2 + 2 * hid + b * (3 * hid * 2 + 2 * inter * 2), nl)
+        add(name, mlp, 3 * inter * hid * 2 + 2 * hid + b * (3 * hid * 2 + 2 * inter * 2), nl,
+            reads=[(gu_base, 4 * inter * hid), (dn, 2 * hid * inter)])
         # arithmetic rate of the batched call; from 5 tokens on it runs on the matrix cores (padded
         # to 16 token columns), whose utilisation is this rate over the dense fp16 MFMA peak
         tflops = 6.0 * inter * hid * b / out[name]["us"] / 1e6
@@ -322,7 +338,8 @@ def kernel_table(lm):
                                     gamma.data_ptr() if norm else None, 1e-5, None,
                                     RES.data_ptr() if resid else None, Y.data_ptr(), n, k, b)
             add("C3_int8_%s_%dx%d_tokens%d" % (name, n, k, b), f,
-                n * k + 2 * n + 2 * hid * norm + b * 2 * (k + n + n * resid), len(ring))
+                n * k + 2 * n + 2 * hid * norm + b * 2 * (k + n + n * resid), len(ring),
+                reads=[([q.data_ptr() for q, _ in ring], n * k)])
             del ring
         ring = [(torch.randint(-127, 128, (inter, 2, hid), dtype=torch.int8, device="cuda"),
                  torch.rand(inter, 2, **f16) * 1e-3 + 1e-4) for _ in range(9)]
@@ -333,7 +350,8 @@ def kernel_table(lm):
                                      sc.data_ptr() + 2, 2, X.data_ptr(), gamma.data_ptr(), 1e-5, hbuf.data_ptr(),
                                      inter, hid, b)
         add("C3_int8_gateup_silu_%dx%d_tokens%d" % (2 * inter, hid, b), g,
-            2 * inter * hid + 4 * inter + 2 * hid + b * 2 * (hid + inter), len(ring))
+            2 * inter * hid + 4 * inter + 2 * hid + b * 2 * (hid + inter), len(ring),
+            reads=[([q.data_ptr() for q, _ in ring], 2 * inter * hid)])
         del ring
     torch.cuda.empty_cache()
 

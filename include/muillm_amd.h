@@ -390,6 +390,13 @@ int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int di
  * qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
 int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 
+/* Measurement aid without a counterpart in the reference: reads `bytes` (a multiple of 16, from
+ * a 16-byte aligned address) of device memory once with the access shape of the GEMV kernels and
+ * discards them. One launch takes the least time any kernel that must read that many bytes can
+ * take on this device, launch latency included. `sink` is any 256-byte device buffer (written
+ * only if the data matches a fixed 16-byte pattern). */
+int mui_probe_read(mui_stream_t stream, const void* src, uint64_t bytes, void* sink);
+
 #ifdef __cplusplus
 }
 #endif

@@ -82,25 +82,38 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
       }
     }
   };
-  int rg = blockIdx.x;
-  if (rg < n_groups) issue(rg);
-
-  // ---- token operands: gamma * x rounded once to the 16-bit type (zero past the row / batch) ----
+  // ---- token operands: gamma * x rounded once to the 16-bit type (zero past the row / batch).
+  // With a fused norm they are requested before the first weights: loads return in order, so the operand
+  // preparation and the norm's reduction then overlap the flight of the first row group instead
+  // of following it. No load sits behind a branch (clamped addresses, dead lanes zeroed by selects).
+  int rg = blockIdx.x;  // the grid never exceeds the number of row groups
+  if constexpr (!NORM) issue(rg);  // nothing to prepare: the weights go first
   u32x4 xq[TOK][CH];
+  u32x4 gq[CH];
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) {
+    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * k;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) xq[tk][j] = ld16(x + xrow + coff[j]);
+  }
+  if constexpr (NORM) {
+#pragma unroll
+    for (int j = 0; j < CH; ++j) gq[j] = ld16(gamma + coff[j]);
+  }
+  if constexpr (NORM) issue(rg);
+
   float ss[TOK];
 #pragma unroll
   for (int tk = 0; tk < TOK; ++tk) {
     ss[tk] = 0.f;
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      u32x4 b = {0u, 0u, 0u, 0u};
-      if (cvalid[j] && tk < tokens) {
-        const u32x4 xv = ld16(x + (long)tk * k + coff[j]);
-        u32x4 gv = xv;
-        if constexpr (NORM) gv = ld16(gamma + coff[j]);
-        b = make_b<T, NORM>(xv, gv, ss[tk]);
-      }
-      xq[tk][j] = b;
+      const bool live = cvalid[j] && tk < tokens;
+      float sq = 0.f;
+      const u32x4 b = make_b<T, NORM>(xq[tk][j], NORM ? gq[j] : xq[tk][j], sq);
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      xq[tk][j] = live ? b : zero;
+      ss[tk] += live ? sq : 0.f;
     }
   }
   float rs[TOK];

@@ -353,7 +353,10 @@ static int check_int8_common(int dtype, const void* w, long pitch, const void* x
 
 using namespace mui;
 
-namespace mui { void int8_set_packed_dot(bool on) { g_int8_dot2 = on ? 1 : 0; } }
+namespace mui {
+void int8_set_packed_dot(bool on) { g_int8_dot2 = on ? 1 : 0; }
+int int8_tuned_wgs_per_cu() { return g_int8_wgs_per_cu; }
+}  // namespace mui
 
 extern "C" int mui_tune_int8(int rows, int wgs_per_cu) {
   if (!(rows == 0 || rows == 2 || rows == 4 || rows == 8)) return MUI_ERR_INVALID_ARG;

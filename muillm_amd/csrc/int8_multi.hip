@@ -36,7 +36,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
   constexpr int NVH = NV / NH;
   constexpr uint32_t kFlip = (WF == WF_I8_CHANNEL) ? 0x80808080u : 0u;
   constexpr float kOffset = (WF == WF_I8_CHANNEL) ? 1152.f : 1024.f;
-  static_assert(NV <= 32 && (R % 2 == 0), "shape");
+  static_assert(NV <= 32 && (R % 2 == 0) && NVH <= 16, "shape");
   __shared__ float red[2][kI8mWaves * 4][NV];
   __shared__ float red_ss[kI8mWaves][TOK];
 
@@ -98,11 +98,32 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       }
     }
   };
-  int rg = blockIdx.x;
-  if (rg < n_groups) issue(rg);
-
-  // ---- token operands: gamma * x as packed fp16, the chunk's sum of them on the side ----
+  // ---- token operands: gamma * x as packed fp16, the chunk's sum of them on the side. With a fused norm they
+  // are requested before the first weights: loads return in order, so the operand preparation and
+  // the norm's reduction then overlap the flight of the first row group instead of following it.
+  // No load sits behind a branch (clamped addresses, dead lanes zeroed by selects).
+  int rg = blockIdx.x;  // the grid never exceeds the number of row groups
+  if constexpr (!NORM) issue(rg);  // nothing to prepare: the weights go first
   u32x4 xq[TOK][CH][2];
+  u32x4 gq[CH][2];
+#pragma unroll
+  for (int tk = 0; tk < TOK; ++tk) {
+    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * k;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) xq[tk][j][hf] = ld16(x + xrow + coff[j] + 8 * hf);
+    }
+  }
+  if constexpr (NORM) {
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) gq[j][hf] = ld16(gamma + coff[j] + 8 * hf);
+    }
+  }
+  if constexpr (NORM) issue(rg);
+
   float xsum[TOK][CH];
   float ss[TOK];
 #pragma unroll
@@ -111,15 +132,14 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       xsum[tk][j] = 0.f;
+      const bool live = cvalid[j] && tk < tokens;
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
-        u32x4 b = {0u, 0u, 0u, 0u};
-        if (cvalid[j] && tk < tokens) {
-          const u32x4 xv = ld16(x + (long)tk * k + coff[j] + 8 * hf);
-          u32x4 gv = xv;
-          if constexpr (NORM) gv = ld16(gamma + coff[j] + 8 * hf);
-          b = make_b<T, NORM>(xv, gv, ss[tk]);
-        }
+        float sq = 0.f;
+        u32x4 b = make_b<T, NORM>(xq[tk][j][hf], NORM ? gq[j][hf] : xq[tk][j][hf], sq);
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        b = live ? b : zero;
+        ss[tk] += live ? sq : 0.f;
         xq[tk][j][hf] = b;
         float bf[8];
         unpack8<T>(b, bf);
@@ -255,14 +275,15 @@ static int launch_i8m_rc(hipStream_t s, const SkinnyParams& p, int grid) {
 template <int EPI, int WF, int TOK>
 static int launch_i8m_t(hipStream_t s, const SkinnyParams& p) {
   const int ch = ceil_div(p.k >> 4, kI8mThreads);
+  const int per_cu = int8_tuned_wgs_per_cu();
   if (ch <= 1) {
     // short rows: 8 rows in flight at 2 tokens, 4 at 4 (at most 32 partial sums per group)
     constexpr int R = (TOK <= 2) ? 8 : 4;
     constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
-    return launch_i8m_rc<R, 1, EPI, WF, TOK>(s, p, balanced_grid(ceil_div(p.n, OUT), 3));
+    return launch_i8m_rc<R, 1, EPI, WF, TOK>(s, p, balanced_grid(ceil_div(p.n, OUT), per_cu > 0 ? per_cu : 3));
   }
   constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
-  const int grid = balanced_grid(ceil_div(p.n, OUT), 2);
+  const int grid = balanced_grid(ceil_div(p.n, OUT), per_cu > 0 ? per_cu : 2);
   if (ch <= 2) return launch_i8m_rc<R, 2, EPI, WF, TOK>(s, p, grid);
   if (ch <= 4) return launch_i8m_rc<R, 4, EPI, WF, TOK>(s, p, grid);
   return MUI_ERR_UNSUPPORTED;

@@ -130,6 +130,7 @@ int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams
 // MFMA skinny GEMM whose weight rows are read as contiguous runs and turned into operands
 // through wave-private LDS (gemm_skinny_lt.hip); MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_skinny_lt(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
+int int8_tuned_wgs_per_cu();  // mui_tune_int8's workgroups-per-CU override (0 = built-in)
 int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 = built-in)
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);

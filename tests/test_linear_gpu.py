@@ -343,3 +343,21 @@ def test_lm_head_full_size_gather_property():
     rows = torch.arange(0, n, 257, device="cuda")
     ref = (w[rows].float() @ x[0].float())
     assert float((y[0, rows].float() - ref).abs().max()) <= 1e-2 * float(ref.abs().max())
+
+
+def test_read_probe_reads_and_discards():
+    """The read probe leaves source and sink untouched (the sink is written only when the XOR of
+    everything a lane read equals a fixed pattern), covers sizes that are not a multiple of its
+    chunk, and rejects misaligned requests."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    sink = torch.zeros(64, dtype=torch.int32, device=DEV)
+    for nbytes in (16, 4096 * 8 + 48, 33554432):
+        src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=DEV)
+        keep = src.clone()
+        assert lib.mui_probe_read(stream, src.data_ptr(), nbytes, sink.data_ptr()) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(src, keep) and int(sink.abs().sum()) == 0
+    assert lib.mui_probe_read(stream, src.data_ptr() + 8, 64, sink.data_ptr()) != 0
+    assert lib.mui_probe_read(stream, src.data_ptr(), 24, sink.data_ptr()) != 0
+    assert lib.mui_probe_read(stream, None, 64, sink.data_ptr()) != 0
