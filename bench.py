@@ -89,12 +89,15 @@ def bench_int8_variant(config, steps, warmup):
     lm8 = init_engine(base, device="cuda", engine_config=MuiEngineConfig(qm))
     torch.cuda.synchronize()
     dt, dec = bench_decode(lm8, steps, warmup)
+    del dec
+    dt_eager, dec = bench_decode(lm8, steps, warmup, use_graph=False)
     hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
     hq, hkv, d = config.num_attention_heads, config.num_key_value_heads, hid // config.num_attention_heads
     wbytes = config.num_hidden_layers * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter) + 2 * v * hid
     del dec, lm8, base
     torch.cuda.empty_cache()
     return {"tokens_per_s": round(steps / dt, 2), "ms_per_step": round(dt / steps * 1e3, 4),
+            "eager_no_graph_tokens_per_s": round(steps / dt_eager, 2),
             "weight_bytes_per_token": wbytes, "hbm_floor_ms": round(wbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4),
             "format": "int8 per output channel + fp16 scale; lm_head fp16"}
 

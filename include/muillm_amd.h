@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define MUI_ABI_VERSION 1
+#define MUI_ABI_VERSION 2
 
 /* status codes (reference: TORCH_CHECK exceptions, csrc/linear/linear.cu:72-74;
  * muillm_error_t, csrc/base.h:4-7) */
@@ -309,7 +309,9 @@ int mui_sample_advance(mui_stream_t stream, int dtype, const void* logits, long 
  * (csrc/modules/parallel_decoder_stack.cpp, csrc/modules/parallel_decoder_module.cpp:22-62).
  * Per layer: qkv = Wqkv rmsnorm(h); attn = flash decoding with RoPE and cache write
  * (mui_attn_decode_fused); h' = Wo attn + h; mid = silu(Wg n) * (Wu n) with n = rmsnorm(h');
- * out = Wd mid + h'. All pointers are device memory of the 16-bit type `dtype`; the caller
+ * out = Wd mid + h'. Activations, norms, caches and 16-bit weights are device memory of the
+ * 16-bit type `dtype`; any projection may instead hold int8 weights with per-channel scales
+ * (muillm/modules/quantized/int8linear.py, int8gateupdownmlp.py in the reference). The caller
  * owns everything. */
 typedef struct mui_decoder_layer {
   const void* input_norm;   /* [hidden] gamma of the RMSNorm fused into the QKV projection */
@@ -325,6 +327,16 @@ typedef struct mui_decoder_layer {
   long down_pitch;
   void* k_cache;            /* [batch, Hkv, max_cache_len, D] with the strides below */
   void* v_cache;
+  /* Weight-only int8 projections (per-output-channel scales, the mui_int8_linear /
+   * mui_int8_gateup_silu format): a non-NULL scales pointer says that projection's weights are
+   * int8 codes (pitch in bytes) and are multiplied by these 16-bit scales; NULL = 16-bit
+   * weights. gate and up are int8 together or not at all. */
+  const void* qkv_scales;   /* [(Hq + 2 Hkv) * D] */
+  const void* o_scales;     /* [hidden] */
+  const void* gate_scales;  /* scale of row n at [n * gateup_scale_stride] */
+  const void* up_scales;
+  long gateup_scale_stride;
+  const void* down_scales;  /* [hidden] */
 } mui_decoder_layer_t;
 
 typedef struct mui_decoder_stack {

@@ -91,7 +91,8 @@ class MuiDecoderLayerDesc(ctypes.Structure):
     _fields_ = [("input_norm", _P), ("qkv_weight", _P), ("qkv_pitch", c_long), ("o_weight", _P),
                 ("o_pitch", c_long), ("post_norm", _P), ("gate_weight", _P), ("up_weight", _P),
                 ("gateup_pitch", c_long), ("down_weight", _P), ("down_pitch", c_long), ("k_cache", _P),
-                ("v_cache", _P)]
+                ("v_cache", _P), ("qkv_scales", _P), ("o_scales", _P), ("gate_scales", _P), ("up_scales", _P),
+                ("gateup_scale_stride", c_long), ("down_scales", _P)]
 
 
 class MuiDecoderStackDesc(ctypes.Structure):

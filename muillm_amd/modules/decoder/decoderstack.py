@@ -18,11 +18,29 @@ from ..gateupdownmlp import MuiGateUpDownMLP
 from ..kvcache.cache_utils import MuiStaticCache
 from ..linear import MuiLinear
 from ..multilinear import MuiMultiLinear
+from ..quantized.int8gateupdownmlp import MuiInt8GateUpDownMLP
+from ..quantized.int8linear import MuiInt8Linear
 
 
 def _plain_linear(m, normalize: Optional[bool] = None) -> bool:
+    """A bias-free MuiLinear, or a bias-free per-channel MuiInt8Linear."""
+    if type(m) is MuiInt8Linear:
+        return (m.per_channel and m.bias is None and m.dispatchable and m.weights_int8.is_contiguous()
+                and m.scales.is_contiguous() and (normalize is None or bool(m.normalize) == normalize))
     return (type(m) is MuiLinear and m.bias is None and m.weight.is_cuda and m.weight.stride(1) == 1
             and (normalize is None or bool(m.normalize) == normalize))
+
+
+def _linear_fields(m):
+    """(weight tensor, row pitch, scales tensor or None, [(owner, attribute, object)]) of a projection."""
+    if type(m) is MuiInt8Linear:
+        return m.weights_int8, m.weights_int8.stride(0), m.scales, [(m, "weights_int8", m.weights_int8),
+                                                                     (m, "scales", m.scales)]
+    return m.weight, m.weight.stride(0), None, [(m, "weight", m.weight)]
+
+
+def _ptr(t) -> Optional[int]:
+    return None if t is None else t.data_ptr()
 
 
 class MuiDecoderStack:
@@ -34,10 +52,9 @@ class MuiDecoderStack:
         self.lib = _lib.load()
         first = layers[0]
         attn0: MuiBaseAttention = first.self_attn
-        w0 = first.qkv_proj.linear.weight
-        self.dtype, self.device = w0.dtype, w0.device
+        self.dtype, self.device = first.qkv_proj.linear.norm_weights.dtype, first.qkv_proj.linear.norm_weights.device
         self.batch = batch
-        self.hidden = w0.shape[1]
+        self.hidden = first.qkv_proj.linear.in_features
         self.hq, self.hkv, self.d = attn0.num_heads, attn0.num_key_value_heads, attn0.head_dim
         self.cos32, self.sin32 = rotary_emb.cos32, rotary_emb.sin32
         kc0 = cache.key_cache[0]
@@ -46,29 +63,41 @@ class MuiDecoderStack:
         self._cache_ptrs = tuple(t.data_ptr() for t in cache.key_cache) + tuple(t.data_ptr() for t in cache.value_cache)
         self._keep = []  # tensors the descriptor points into
         self._layer_list = layers
-        self._owners = []  # (module, attribute name, parameter object) the descriptor was built from
+        self._owners = []  # (module, attribute name, object) the descriptor was built from
         arr = (_lib.MuiDecoderLayerDesc * len(layers))()
         for i, layer in enumerate(layers):
             qkv, attn, mlp = layer.qkv_proj.linear, layer.self_attn, layer.mlp
-            g, u, dn = mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight
             kc, vc = cache.key_cache[attn.layer_idx], cache.value_cache[attn.layer_idx]
             if (kc.stride(), vc.stride()) != (kc0.stride(), kc0.stride()):
                 raise ValueError("cache layers must share one layout")
+            qw, qp, qs, q_own = _linear_fields(qkv)
+            ow, op, osc, o_own = _linear_fields(attn.o_proj)
+            dw, dp, ds, d_own = _linear_fields(mlp.down_proj)
+            if type(mlp) is MuiInt8GateUpDownMLP:
+                gu, gs = mlp.gate_up_weights, mlp.gate_up_scales  # [inter, 2, hidden] codes, [inter, 2] scales
+                g_ptr, u_ptr, g_pitch = gu.data_ptr(), gu.data_ptr() + gu.stride(1), gu.stride(0)
+                gs_ptr, us_ptr, gs_stride = gs.data_ptr(), gs.data_ptr() + gs.element_size(), gs.stride(0)
+                gu_keep = [gu, gs]
+                gu_own = [(mlp, "gate_up_weights", gu), (mlp, "gate_up_scales", gs)]
+            else:
+                g, u = mlp.gate_proj.weight, mlp.up_proj.weight
+                g_ptr, u_ptr, g_pitch = g.data_ptr(), u.data_ptr(), g.stride(0)
+                gs_ptr, us_ptr, gs_stride = None, None, 0
+                gu_keep = [g, u]
+                gu_own = [(mlp.gate_proj, "weight", g), (mlp.up_proj, "weight", u)]
             arr[i] = _lib.MuiDecoderLayerDesc(
-                qkv.norm_weights.data_ptr(), qkv.weight.data_ptr(), qkv.weight.stride(0),
-                attn.o_proj.weight.data_ptr(), attn.o_proj.weight.stride(0),
-                mlp.norm_weights.data_ptr(), g.data_ptr(), u.data_ptr(), g.stride(0),
-                dn.data_ptr(), dn.stride(0), kc.data_ptr(), vc.data_ptr())
-            self._keep += [qkv.norm_weights, qkv.weight, attn.o_proj.weight, mlp.norm_weights, g, u, dn, kc, vc]
+                qkv.norm_weights.data_ptr(), qw.data_ptr(), qp, ow.data_ptr(), op,
+                mlp.norm_weights.data_ptr(), g_ptr, u_ptr, g_pitch, dw.data_ptr(), dp, kc.data_ptr(), vc.data_ptr(),
+                _ptr(qs), _ptr(osc), gs_ptr, us_ptr, gs_stride, _ptr(ds))
+            self._keep += [qkv.norm_weights, qw, qs, ow, osc, mlp.norm_weights, dw, ds, kc, vc] + gu_keep
             self._owners += [(layer, "qkv_proj", layer.qkv_proj), (layer, "self_attn", attn), (layer, "mlp", mlp),
-                             (layer.qkv_proj, "linear", qkv), (qkv, "weight", qkv.weight),
-                             (qkv, "norm_weights", qkv.norm_weights), (attn, "o_proj", attn.o_proj),
-                             (attn.o_proj, "weight", attn.o_proj.weight), (mlp, "norm_weights", mlp.norm_weights),
-                             (mlp.gate_proj, "weight", g), (mlp.up_proj, "weight", u), (mlp.down_proj, "weight", dn)]
+                             (layer.qkv_proj, "linear", qkv), (qkv, "norm_weights", qkv.norm_weights),
+                             (attn, "o_proj", attn.o_proj), (mlp, "norm_weights", mlp.norm_weights),
+                             (mlp, "down_proj", mlp.down_proj)] + q_own + o_own + d_own + gu_own
         self._layers = arr
         self.desc = _lib.MuiDecoderStackDesc(
-            muillm_ext._dtype_code(w0), len(layers), self.hidden, self.hq, self.hkv, self.d,
-            layers[0].mlp.gate_proj.weight.shape[0], float(first.qkv_proj.linear.variance_epsilon),
+            muillm_ext._dtype_code(first.qkv_proj.linear.norm_weights), len(layers), self.hidden, self.hq, self.hkv,
+            self.d, first.mlp.intermediate_size, float(first.qkv_proj.linear.variance_epsilon),
             ctypes.cast(arr, ctypes.POINTER(_lib.MuiDecoderLayerDesc)), self.cos32.data_ptr(), self.sin32.data_ptr(),
             self.cos32.stride(0), cb, chs, cts, self.max_cache_len)
         self._ws = None
@@ -76,12 +105,13 @@ class MuiDecoderStack:
 
     @staticmethod
     def eligible(layers, rotary_emb, cache, batch: int) -> bool:
-        """fp16 / bf16 Llama-shaped layers without biases on a static cache, head_dim 128."""
+        """fp16 / bf16 Llama-shaped layers without biases on a static cache, head_dim 128; every
+        projection either 16-bit or per-channel int8."""
         if not isinstance(cache, MuiStaticCache) or len(layers) == 0 or batch > _lib.MUI_MAX_TOKENS:
             return False
         if not getattr(rotary_emb, "dispatchable", False):
             return False
-        eps = None
+        eps, dtype = None, None
         for layer in layers:
             qkv, attn, mlp = getattr(layer, "qkv_proj", None), getattr(layer, "self_attn", None), getattr(layer, "mlp", None)
             if type(qkv) is not MuiMultiLinear or not _plain_linear(qkv.linear, True):
@@ -90,15 +120,30 @@ class MuiDecoderStack:
                 return False
             if attn.head_dim != 128 or attn.num_key_value_groups not in (1, 2, 4, 8):
                 return False
-            if type(mlp) is not MuiGateUpDownMLP or not mlp.normalize or not isinstance(mlp.activation_function, nn.SiLU):
+            if type(mlp) is MuiGateUpDownMLP:
+                if not all(_plain_linear(m, False) and type(m) is MuiLinear for m in (mlp.gate_proj, mlp.up_proj)):
+                    return False
+                if mlp.gate_proj.weight.stride(0) != mlp.up_proj.weight.stride(0):
+                    return False
+            elif type(mlp) is MuiInt8GateUpDownMLP:
+                if not (mlp.per_channel and mlp.dispatchable and mlp.gate_up_weights.is_contiguous()
+                        and mlp.gate_up_scales.is_contiguous()):
+                    return False
+            else:
                 return False
-            if not all(_plain_linear(m, False) for m in (mlp.gate_proj, mlp.up_proj, mlp.down_proj)):
+            if not mlp.normalize or not isinstance(mlp.activation_function, nn.SiLU):
                 return False
-            if mlp.gate_proj.weight.stride(0) != mlp.up_proj.weight.stride(0):
+            if not _plain_linear(mlp.down_proj, False):
                 return False
-            w = qkv.linear.weight
-            if w.dtype not in (torch.float16, torch.bfloat16) or cache.key_cache[attn.layer_idx].dtype != w.dtype:
+            w = qkv.linear.norm_weights
+            if w is None or mlp.norm_weights is None or w.dtype not in (torch.float16, torch.bfloat16):
                 return False
+            if cache.key_cache[attn.layer_idx].dtype != w.dtype or (dtype is not None and w.dtype != dtype):
+                return False
+            dtype = w.dtype
+            for m in (qkv.linear, attn.o_proj, mlp.down_proj):
+                if (m.scales.dtype if type(m) is MuiInt8Linear else m.weight.dtype) != dtype:
+                    return False
             e = (float(qkv.linear.variance_epsilon), float(mlp.variance_epsilon))
             if e[0] != e[1] or (eps is not None and e != eps):
                 return False
@@ -109,7 +154,7 @@ class MuiDecoderStack:
         """Still valid for this step? The cache tensors are where they were, and every module and
         parameter the descriptor was built from is still the object in place (a later
         quantize_layers / .to() / weight swap replaces them)."""
-        if batch != self.batch or layers is not self._layer_list or len(layers) * 12 != len(self._owners):
+        if batch != self.batch or layers is not self._layer_list:
             return False
         for owner, name, obj in self._owners:
             if getattr(owner, name, None) is not obj:

@@ -274,6 +274,45 @@ def test_decoder_stack_call_matches_layer_modules(batch, dtype):
         assert torch.equal(after, ref)
 
 
+@pytest.mark.parametrize("modules", [["qkv_proj", "o_proj", "mlp"], ["mlp"], ["o_proj"]])
+@pytest.mark.parametrize("batch", [1, 3])
+def test_decoder_stack_call_int8_layers(modules, batch):
+    """Per-channel int8 projections (all of them, or only some: the rest stay fp16) go through the
+    single call too: same logits and cache contents as the layer modules called one by one; the
+    group format keeps the per-layer calls."""
+    cfg = _small_config(layers=2)
+    base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=5,
+                                           init_std=0.05, finalize=False)
+    qm = Int8WeightOnlyQuantizationMethod(group_size=0, modules=modules)
+    lm = init_engine(copy.deepcopy(base), device=DEV, engine_config=MuiEngineConfig(qm))
+    g = torch.Generator().manual_seed(6)
+    ids = torch.randint(0, cfg.vocab_size, (batch, 9), generator=g).to(DEV)
+    results = {}
+    with torch.no_grad():
+        for use_stack in (False, True):
+            lm.model.use_decoder_stack = use_stack
+            out = lm(input_ids=ids)
+            cache = out.past_key_values
+            nxt = out.logits[:, -1].argmax(-1)
+            logits = []
+            for _ in range(5):
+                out = lm(input_ids=nxt.unsqueeze(1), past_key_values=cache)
+                logits.append(out.logits[:, -1].clone())
+                nxt = out.logits[:, -1].argmax(-1)
+            results[use_stack] = (torch.stack(logits), [k.clone() for k in cache.key_cache + cache.value_cache])
+    assert lm.model._stack is not None, "the single-call path did not engage"
+    assert torch.equal(results[False][0], results[True][0])
+    for x, y in zip(results[False][1], results[True][1]):
+        assert torch.equal(x, y)
+    # the reference's group format is not part of the single call
+    qg = Int8WeightOnlyQuantizationMethod(group_size=128, modules=modules)
+    lg = init_engine(base, device=DEV, engine_config=MuiEngineConfig(qg))
+    with torch.no_grad():
+        out = lg(input_ids=ids)
+        lg(input_ids=out.logits[:, -1].argmax(-1).unsqueeze(1), past_key_values=out.past_key_values)
+    assert lg.model._stack is None
+
+
 def test_argmax_kernel():
     from muillm_amd import muillm_ext
     g = torch.Generator().manual_seed(2)
