@@ -172,7 +172,8 @@ int mui_int8_group_dequantize(mui_stream_t stream, int dtype, const void* weight
                               void* out, long out_pitch, int n, int k);
 
 /* ------------------------------------------------------------------------------------
- * RoPE, static KV cache, decode attention (head_dim 128; Hq/Hkv in {1, 2, 4, 8})
+ * RoPE, static KV cache, decode attention (head_dim 128; any whole number of query heads per KV
+ * head: 1..8 read K/V once per KV head, other ratios once per query head)
  *
  * Common conventions: q/k/v inputs and the cache have unit inner stride; all other strides
  * are in elements. cos/sin tables are fp32 [max_position, rope_row_stride] with

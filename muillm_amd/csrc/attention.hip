@@ -981,15 +981,17 @@ static void launch_attn_nw(hipStream_t s, const AttnParams& p, dim3 grid) {
     hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, false>), grid, dim3(NW * kWave), 0, s, p);
 }
 
-template <typename T, int G>
+template <typename T, int G, bool MFMA_ONLY = false>
 static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
   dim3 grid(p.n_splits, p.hq / G, batch);
   const int nw = attn_waves_for(G);
-  if (G == p.hq / p.hkv && g_attn_mfma_tokens >= 0) {
+  if (MFMA_ONLY || (G == p.hq / p.hkv && g_attn_mfma_tokens >= 0)) {
     if (p.n_splits == 1)
       hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, true>), grid, dim3(8 * kWave), 0, s, p);
     else
       hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, false>), grid, dim3(8 * kWave), 0, s, p);
+  } else if constexpr (MFMA_ONLY) {
+    return MUI_ERR_UNSUPPORTED;
   } else if constexpr (G <= 4) {
     if (nw == 16) launch_attn_nw<T, G, 16>(s, p, grid);
     else if (nw == 8) launch_attn_nw<T, G, 8>(s, p, grid);
@@ -1017,8 +1019,15 @@ static int launch_attn_t(hipStream_t s, const AttnParams& p, int batch) {
     case 2: return launch_attn_g<T, 2>(s, p, batch);
     case 4: return launch_attn_g<T, 4>(s, p, batch);
     case 8: return launch_attn_g<T, 8>(s, p, batch);
-    default: return MUI_ERR_UNSUPPORTED;
+    // other group sizes: the matrix-core kernel pads the heads of a group to 16 columns anyway
+    case 3: if (g_attn_mfma_tokens >= 0) return launch_attn_g<T, 3, true>(s, p, batch); break;
+    case 5: if (g_attn_mfma_tokens >= 0) return launch_attn_g<T, 5, true>(s, p, batch); break;
+    case 6: if (g_attn_mfma_tokens >= 0) return launch_attn_g<T, 6, true>(s, p, batch); break;
+    case 7: if (g_attn_mfma_tokens >= 0) return launch_attn_g<T, 7, true>(s, p, batch); break;
+    default: break;
   }
+  // any other ratio: one workgroup per query head (K/V re-read by the heads of a group)
+  return launch_attn_g<T, 1>(s, p, batch);
 }
 
 static int launch_attn(hipStream_t s, int dtype, const AttnParams& p, int batch) {
@@ -1079,9 +1088,7 @@ static int check_attn_shape(int dtype, int batch, int hq, int hkv, int head_dim,
   if (n_splits > kMaxSplits) return MUI_ERR_UNSUPPORTED;
   if (head_dim != kHeadDim) return MUI_ERR_UNSUPPORTED;
   if (hq % hkv != 0) return MUI_ERR_INVALID_ARG;
-  const int g = hq / hkv;
-  if (!(g == 1 || g == 2 || g == 4 || g == 8)) return MUI_ERR_UNSUPPORTED;
-  if (batch > 65535 || hkv > 65535) return MUI_ERR_UNSUPPORTED;
+  if (batch > 65535 || hq > 65535) return MUI_ERR_UNSUPPORTED;
   return MUI_OK;
 }
 

@@ -18,8 +18,9 @@
 //   B-stationary mode (K <= 4096, K % 256 == 0): wave w owns the same K range of every tile
 //     (two passes per tile); its B operands (gamma * x of the 16 token columns) are built once
 //     and stay in registers.
-//   streaming mode (longer rows, no fused norm): the wave walks its K range in passes and
-//     brings the token rows through LDS the same way as the weight rows.
+//   streaming mode (longer rows): the wave walks its K range in passes and brings the token rows
+//     through LDS the same way as the weight rows (a fused norm multiplies them by gamma on the
+//     way and gathers sum(x^2) during the first tile).
 // Two register sets: the next pass is in flight while the current one is multiplied.
 // Both are persistent (one workgroup per CU, balanced tile counts). The number of passes of a
 // workgroup is a multiple of half the register sets (launcher).
@@ -60,7 +61,6 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   // spill with 16-bit ones)
   constexpr int NSET = 2;
   constexpr int NB = BSTAT ? 1 : kLtXLoads;
-  static_assert(BSTAT || !NORM, "streaming mode has no fused norm");
 
   __shared__ __attribute__((aligned(16))) char op_lds[kLtWaves][NOPS][16 * kLtXPitch];
   __shared__ float tile[2][kLtWaves][16][17];
@@ -159,7 +159,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     const int kk = ld_chunk * KPC;
     return (FULL || kk < pass_len(i)) ? pass_k0(i) + kk : -1;
   };
-  auto issue = [&](int i, u32x4 (&a)[NLD], u32x4 (&b)[NB]) {  // needs i < n_items
+  auto issue = [&](int i, u32x4 (&a)[NLD], u32x4 (&b)[NB], u32x4& gm) {  // needs i < n_items
     const int tl = blockIdx.x + (i / passes) * gridDim.x;
     const int wk = weight_k(i);
     const long woff = (long)(wk < 0 ? 0 : wk) * WB;
@@ -168,6 +168,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     if constexpr (!BSTAT) {
       const int xk = pass_k0(i) + xl_chunk * 8;
       const int xoff = xk < p.k ? xk : 0;  // (the weights of those k-values are zeroed)
+      if constexpr (NORM) gm = ld16(p.gamma + xoff);
 #pragma unroll
       for (int q = 0; q < kLtXLoads; ++q) {
         const int tok = q * 2 + xl_row;
@@ -218,14 +219,26 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   u32x4 bq[BSTAT ? 2 * kLtSteps : 1];
   f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};  // two chains: MFMAs back to back
   int buf = 0;
-  auto stage = [&](int i, const u32x4 (&a)[NLD], const u32x4 (&b)[NB]) {  // registers -> LDS tiles
+  // streaming mode with a fused norm: sum(x^2) of tokens 2 q + xl_row over this lane's chunks,
+  // gathered during the wave's passes over the first tile (later tiles read the same token rows)
+  float ssx[(NORM && !BSTAT) ? kLtXLoads : 1] = {};
+  auto stage = [&](int i, const u32x4 (&a)[NLD], const u32x4 (&b)[NB], const u32x4& gm) {  // registers -> LDS tiles
     const u32x4 zero = {0u, 0u, 0u, 0u};
     const bool ok = FULL || weight_k(i) >= 0;
 #pragma unroll
     for (int q = 0; q < NLD; ++q) *(u32x4*)(la + (q * RPI + ld_row) * PITCH + ld_chunk * 16) = ok ? a[q] : zero;
     if constexpr (!BSTAT) {
+      const bool count = NORM && i < passes && pass_k0(i) + xl_chunk * 8 < p.k;
 #pragma unroll
-      for (int q = 0; q < kLtXLoads; ++q) *(u32x4*)(lb + (q * 2 + xl_row) * kLtXPitch + xl_chunk * 16) = b[q];
+      for (int q = 0; q < kLtXLoads; ++q) {
+        u32x4 v = b[q];
+        if constexpr (NORM) {
+          float sq = 0.f;
+          v = make_b<T, true>(v, gm, sq);
+          ssx[q] += count ? sq : 0.f;
+        }
+        *(u32x4*)(lb + (q * 2 + xl_row) * kLtXPitch + xl_chunk * 16) = v;
+      }
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -262,6 +275,18 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
       for (int r = 0; r < 4; ++r) tile[buf][wave][4 * g + r][r16] = acc[r] + acc1[r];
       acc = f32x4{0.f, 0.f, 0.f, 0.f};
       acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (NORM && !BSTAT) {
+        if (i < passes) {  // first tile done: this wave has seen its whole K range of every token
+#pragma unroll
+          for (int q = 0; q < kLtXLoads; ++q) {
+            const float even = wave_sum(lane < 32 ? ssx[q] : 0.f), odd = wave_sum(lane < 32 ? 0.f : ssx[q]);
+            if (lane == 0) {
+              ss_part[wave][2 * q] = even;
+              ss_part[wave][2 * q + 1] = odd;
+            }
+          }
+        }
+      }
       __syncthreads();
       epilogue(blockIdx.x + (i / passes) * gridDim.x, buf, ex);
       buf ^= 1;
@@ -311,13 +336,14 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   };
 
   u32x4 as[NSET][NLD], bs[NSET][NB];
+  u32x4 gs[NSET] = {};  // streaming mode with a fused norm: gamma chunk of the pass
   Extras ex[NSET] = {};
   // pass i on register set U (U = i % NSET); REFILL: the set is requested again for pass i + NSET
 #define MUI_LT_PASS(i_, U, REFILL)                    \
   {                                                   \
-    stage((i_), as[U], bs[U]);                        \
+    stage((i_), as[U], bs[U], gs[U]);                 \
     multiply((i_), (U) & 1, as[U], bs[U]);            \
-    if (REFILL) issue((i_) + NSET, as[U], bs[U]);     \
+    if (REFILL) issue((i_) + NSET, as[U], bs[U], gs[U]); \
     finish((i_), ex[U]);                              \
     if (REFILL) issue_extras((i_) + NSET, ex[U]);     \
   }
@@ -327,13 +353,13 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     // registers and all register sets do not fit the register file together)
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      issue(u, as[u], bs[u]);
+      issue(u, as[u], bs[u], gs[u]);
       issue_extras(u, ex[u]);
     }
     build_b();
 #pragma unroll
     for (int u = 2; u < NSET; ++u) {
-      issue(u, as[u], bs[u]);
+      issue(u, as[u], bs[u], gs[u]);
       issue_extras(u, ex[u]);
     }
     // passes with a refill in rounds of NSET, a half round if their number asks for it (it is
@@ -359,7 +385,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
 #pragma unroll
     for (int u = 0; u < NSET; ++u) {
       if (u < n_items) {
-        issue(u, as[u], bs[u]);
+        issue(u, as[u], bs[u], gs[u]);
         issue_extras(u, ex[u]);
       }
     }
@@ -388,9 +414,9 @@ static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
     return launch_status();
   }
   // streaming: 16-byte chunks of weights and of token rows must not straddle the row end
-  if (p.gamma || (p.k % (WF == WF_16BIT ? 8 : 16))) return MUI_ERR_UNSUPPORTED;
+  if (p.k % (WF == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
   const int spw = ceil_div(ceil_div(p.k, kLtSub), kLtWaves);
-  MUI_LT(false, false, false, spw);
+  if (p.gamma) MUI_LT(true, false, false, spw); else MUI_LT(false, false, false, spw);
 #undef MUI_LT
   return launch_status();
 }

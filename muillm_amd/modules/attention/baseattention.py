@@ -71,7 +71,7 @@ class MuiBaseAttention(MuiModule):
     def _fused_decode_ok(self, query_states, past_key_value, q_len: int) -> bool:
         return (q_len == 1 and isinstance(past_key_value, MuiStaticCache) and query_states.is_cuda
                 and query_states.dtype in (torch.float16, torch.bfloat16) and self.head_dim == 128
-                and self.num_key_value_groups in (1, 2, 4, 8) and self.rotary_emb.dispatchable
+                and self.rotary_emb.dispatchable
                 and past_key_value.key_cache[self.layer_idx].dtype == query_states.dtype)
 
     def _fused_decode(self, query_states, key_states, value_states, attention_mask, position_ids,
@@ -95,8 +95,7 @@ class MuiBaseAttention(MuiModule):
 
     def _decode_or_none(self, q, k, v, attention_mask, all_ones_mask, q_len):
         """The two-step decode path (already rotated q, cache views) for T == 1."""
-        if q_len == 1 and q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and self.head_dim == 128 \
-                and self.num_key_value_groups in (1, 2, 4, 8):
+        if q_len == 1 and q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and self.head_dim == 128:
             if all_ones_mask or (attention_mask is None):
                 return mui_causally_decode(q.contiguous(), k, v)
             return mui_causally_decode_masked(q.contiguous(), k, v, attention_mask)

@@ -118,7 +118,7 @@ class MuiDecoderStack:
                 return False
             if not isinstance(attn, MuiBaseAttention) or not _plain_linear(attn.o_proj, False):
                 return False
-            if attn.head_dim != 128 or attn.num_key_value_groups not in (1, 2, 4, 8):
+            if attn.head_dim != 128:
                 return False
             if type(mlp) is MuiGateUpDownMLP:
                 if not all(_plain_linear(m, False) and type(m) is MuiLinear for m in (mlp.gate_proj, mlp.up_proj)):

@@ -129,6 +129,9 @@ def test_static_cache_prefill_then_decode():
     (1, 32, 8, 1, 16), (1, 32, 8, 5, 8), (1, 32, 8, 63, 64), (2, 32, 8, 64, 128), (1, 32, 8, 65, 128),
     (1, 32, 8, 1024, 1024), (3, 32, 8, 1000, 1024), (8, 32, 8, 1024, 2048),
     (1, 8, 8, 300, 512), (1, 16, 8, 300, 512), (2, 64, 8, 300, 512),
+    # other GQA ratios: 3, 5, 6, 7 (matrix-core kernel) and 12, 16 (one workgroup per query head)
+    (1, 24, 8, 300, 512), (2, 20, 4, 700, 1024), (1, 12, 2, 300, 512), (1, 14, 2, 2000, 2048),
+    (1, 12, 1, 300, 512), (1, 32, 2, 2000, 2048),
 ])
 @pytest.mark.parametrize("splits", [None, 1, 7])
 def test_flash_decode(b, hq, hkv, s, cap, splits):
@@ -216,8 +219,18 @@ def test_fused_decode(b, s, cap, device_len, dtype):
     """Config 4 recipe: cache pre-filled for s-1 positions, new token at position s-1."""
     if dtype == torch.bfloat16 and s > 1024:
         pytest.skip("bf16 twin covered at the smaller shapes")
+    _fused_decode_case(b, s, cap, device_len, dtype, 32, 8)
+
+
+@pytest.mark.parametrize("hq,hkv", [(24, 8), (20, 4), (12, 2), (14, 2), (32, 2), (12, 1)])
+@pytest.mark.parametrize("b,s,cap", [(1, 257, 512), (2, 3000, 4096)])
+def test_fused_decode_other_group_sizes(hq, hkv, b, s, cap):
+    """Query heads per KV head other than 1, 2, 4, 8 (Llama-3.2-3B has 3): unsplit and split."""
+    _fused_decode_case(b, s, cap, True, torch.float16, hq, hkv)
+
+
+def _fused_decode_case(b, s, cap, device_len, dtype, hq, hkv):
     g = _gen(7)
-    hq, hkv = 32, 8
     cos, sin = oracle.rope_tables(500000.0, D, cap)
     qkv = _mk((b, 1, (hq + 2 * hkv) * D), g, dtype=dtype)
     kc = torch.zeros(b, hkv, cap, D, dtype=dtype)

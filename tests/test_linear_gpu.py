@@ -136,7 +136,7 @@ def test_linear_strided_weights():
 
 
 @pytest.mark.parametrize("tokens", [2, 3, 4, 5, 8, 13, 16])
-@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (100, 512)])
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336), (100, 512), (8208, 5120)])
 def test_linear_small_batch(tokens, n, k):
     g = _gen(4)
     w = _mk((n, k), g, 0.02)
@@ -156,8 +156,8 @@ def test_linear_small_batch(tokens, n, k):
 def test_linear_small_batch_edge_shapes(tokens, n, k, norm, dtype):
     """The matrix-core path at its seams: K below / at / above what a workgroup keeps stationary
     (4096), K that is not a multiple of the 256-value pass, rows that do not fill a 16-row tile,
-    fused norm on long rows (the streaming mode has none and hands over to the direct-operand
-    kernel), with residual and both biases."""
+    fused norm on long rows (the streaming mode applies gamma on the way to LDS and gathers
+    sum(x^2) during its first tile), with residual and both biases."""
     g = _gen(40 + tokens)
     w = _mk((n, k), g, 0.02, dtype=dtype)
     x = _mk((tokens, k), g, dtype=dtype)
@@ -173,7 +173,7 @@ def test_linear_small_batch_edge_shapes(tokens, n, k, norm, dtype):
 
 
 @pytest.mark.parametrize("tokens", [5, 16])
-@pytest.mark.parametrize("n,k", [(40, 256), (100, 3840), (24, 8192), (9, 2056)])
+@pytest.mark.parametrize("n,k", [(40, 256), (100, 3840), (24, 8192), (9, 2056), (4100, 5120)])
 @pytest.mark.parametrize("norm", [True, False])
 def test_gateup_small_batch_edge_shapes(tokens, n, k, norm):
     g = _gen(60 + tokens)
