@@ -310,7 +310,6 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
   if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
   if (w_pitch < k_in) return MUI_ERR_INVALID_ARG;
   if ((k_in & 7) || (w_pitch & 7)) return MUI_ERR_UNSUPPORTED;
-  if (k_in > 8 * 8 * kThreads) return MUI_ERR_UNSUPPORTED;
   if (!aligned16(weights) || !aligned16(x) || (norm_weights && !aligned16(norm_weights)))
     return MUI_ERR_ALIGNMENT;
 
@@ -335,6 +334,7 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
     }
     if (tokens >= g_skinny_min_tokens) return launch_skinny(s, dtype, WF_16BIT, SK_LINEAR, sp);
   }
+  if (k_in > 8 * 8 * kThreads) return MUI_ERR_UNSUPPORTED;  // the per-token kernel below: 8 chunks per thread
   for (int tkn = 0; tkn < tokens; ++tkn) {
     GemvParams p;
     p.w0 = (const uint16_t*)weights;
@@ -364,7 +364,6 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
   if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
   if (gu_pitch < k_in) return MUI_ERR_INVALID_ARG;
   if ((k_in & 7) || (gu_pitch & 7)) return MUI_ERR_UNSUPPORTED;
-  if (k_in > 8 * 8 * kThreads) return MUI_ERR_UNSUPPORTED;
   if (!aligned16(gate) || !aligned16(up) || !aligned16(x) ||
       (norm_weights && !aligned16(norm_weights)))
     return MUI_ERR_ALIGNMENT;
@@ -389,6 +388,7 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
     }
     if (tokens >= g_skinny_min_tokens) return launch_skinny(s, dtype, WF_16BIT, SK_GATEUP, sp);
   }
+  if (k_in > 8 * 8 * kThreads) return MUI_ERR_UNSUPPORTED;  // the per-token kernel below: 8 chunks per thread
   for (int tkn = 0; tkn < tokens; ++tkn) {
     GemvParams p;
     p.w0 = (const uint16_t*)gate;

@@ -32,7 +32,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
     // scalars, hottest first (preloaded into SGPRs at wave launch)
     const uint16_t* w0, const uint16_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
     uint16_t* y, int n, int k, int tokens, float eps, const uint16_t* residual,
-    const uint16_t* mul_bias, const uint16_t* add_bias) {
+    const uint16_t* mul_bias, const uint16_t* add_bias, long x_pitch) {
   constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
   static_assert(EPI != SK_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
   constexpr int NV = R * TOK;  // partial sums per row group: value r * TOK + token
@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
   u32x4 gq[CH];
 #pragma unroll
   for (int tk = 0; tk < TOK; ++tk) {
-    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * k;
+    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * x_pitch;
 #pragma unroll
     for (int j = 0; j < CH; ++j) xq[tk][j] = ld16(x + xrow + coff[j]);
   }
@@ -195,7 +195,7 @@ static int launch_mt_rc(hipStream_t s, const SkinnyParams& p, int grid) {
 #define MUI_MT_LAUNCH(NORMV)                                                                                   \
   hipLaunchKernelGGL((gemv_multi_kernel<T, R, CH, NORMV, EPI, TOK>), dim3(grid), dim3(kMtThreads), 0, s,        \
                      (const uint16_t*)p.w0, (const uint16_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k,        \
-                     p.tokens, p.eps, p.residual, p.mul_bias, p.add_bias)
+                     p.tokens, p.eps, p.residual, p.mul_bias, p.add_bias, p.x_pitch > 0 ? p.x_pitch : (long)p.k)
   if (p.gamma) MUI_MT_LAUNCH(true); else MUI_MT_LAUNCH(false);
 #undef MUI_MT_LAUNCH
   return launch_status();
@@ -230,8 +230,29 @@ static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
   }
 }
 
+// longest row one launch covers: 7 chunks of 8 values per thread
+constexpr int kMtMaxK = 7 * 8 * kMtThreads;
+
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p) {
   if (p.tokens < 1 || p.tokens > 8) return MUI_ERR_UNSUPPORTED;
+  if (p.k > kMtMaxK) {
+    // Longer rows (down projections of 70B-class models): K segments, one launch each, every
+    // launch after the first adding to y through the residual operand (the thread that loads
+    // y[t, n] is the one that stores it). A fused norm needs the whole row and is not split.
+    if (epilogue != SK_LINEAR || p.gamma) return MUI_ERR_UNSUPPORTED;
+    SkinnyParams q = p;
+    q.x_pitch = p.x_pitch > 0 ? p.x_pitch : (long)p.k;
+    for (int done = 0; done < p.k; done += kMtMaxK) {
+      q.k = p.k - done < kMtMaxK ? p.k - done : kMtMaxK;
+      q.w0 = (const uint16_t*)p.w0 + done;
+      q.x = p.x + done;
+      q.residual = done == 0 ? p.residual : p.y;
+      q.add_bias = done + q.k == p.k ? p.add_bias : nullptr;
+      const int st = launch_gemv_multi(s, dtype, epilogue, q);
+      if (st != MUI_OK) return st;
+    }
+    return MUI_OK;
+  }
 #define MUI_MT_CASE(TT, EPIV)                                            \
   if (epilogue == EPIV) {                                                \
     if (p.tokens <= 1) return launch_mt_t<TT, EPIV, 1>(s, p);            \

@@ -344,7 +344,6 @@ static int check_int8_common(int dtype, const void* w, long pitch, const void* x
   if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
   if (pitch < k) return MUI_ERR_INVALID_ARG;
   if ((k & 15) || (pitch & 15)) return MUI_ERR_UNSUPPORTED;
-  if (k > 16 * 4 * kThreads8) return MUI_ERR_UNSUPPORTED;
   if (!aligned16(w) || !aligned16(x) || (gamma && !aligned16(gamma))) return MUI_ERR_ALIGNMENT;
   return MUI_OK;
 }

@@ -21,7 +21,7 @@ constexpr int kI8mWaves = kI8mThreads / kWave;
 
 struct Int8MultiArgs {
   const uint16_t* s0; const uint16_t* s1; long s_pitch; int group_shift;
-  const uint16_t* add_bias; const uint16_t* residual;
+  const uint16_t* add_bias; const uint16_t* residual; long x_pitch;
 };
 
 template <int R, int CH, bool NORM, int EPI, int WF, int TOK>
@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
   u32x4 gq[CH][2];
 #pragma unroll
   for (int tk = 0; tk < TOK; ++tk) {
-    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * k;
+    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * a.x_pitch;
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
 #pragma unroll
@@ -262,7 +262,8 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
 
 template <int R, int CH, int EPI, int WF, int TOK>
 static int launch_i8m_rc(hipStream_t s, const SkinnyParams& p, int grid) {
-  Int8MultiArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual};
+  Int8MultiArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual,
+                     p.x_pitch > 0 ? p.x_pitch : (long)p.k};
 #define MUI_I8M_LAUNCH(NORMV)                                                                              \
   hipLaunchKernelGGL((int8_multi_kernel<R, CH, NORMV, EPI, WF, TOK>), dim3(grid), dim3(kI8mThreads), 0, s,  \
                      (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k,      \
@@ -289,9 +290,32 @@ static int launch_i8m_t(hipStream_t s, const SkinnyParams& p) {
   return MUI_ERR_UNSUPPORTED;
 }
 
+// longest row one launch covers: 4 chunks of 16 weights per thread
+constexpr int kI8mMaxK = 4 * 16 * kI8mThreads;
+
 int launch_int8_multi(hipStream_t s, int dtype, int wf, int epilogue, const SkinnyParams& p) {
   if (dtype != MUI_DTYPE_F16 || p.tokens < 1 || p.tokens > 4) return MUI_ERR_UNSUPPORTED;
   if (p.mul_bias) return MUI_ERR_UNSUPPORTED;
+  if (p.k > kI8mMaxK) {
+    // Longer rows: K segments, one launch each, every launch after the first adding to y through
+    // the residual operand (row scale and (scale, min) pairs are linear in the segment sums; a
+    // segment starts on a group boundary). A fused norm needs the whole row and is not split.
+    if (epilogue != SK_LINEAR || p.gamma) return MUI_ERR_UNSUPPORTED;
+    if (wf == WF_U8_GROUP && (p.group_shift > 14)) return MUI_ERR_UNSUPPORTED;
+    SkinnyParams q = p;
+    q.x_pitch = p.x_pitch > 0 ? p.x_pitch : (long)p.k;
+    for (int done = 0; done < p.k; done += kI8mMaxK) {
+      q.k = p.k - done < kI8mMaxK ? p.k - done : kI8mMaxK;
+      q.w0 = (const uint8_t*)p.w0 + done;
+      q.x = p.x + done;
+      if (wf == WF_U8_GROUP) q.s0 = p.s0 + 2 * (done >> p.group_shift);
+      q.residual = done == 0 ? p.residual : p.y;
+      q.add_bias = done + q.k == p.k ? p.add_bias : nullptr;
+      const int st = launch_int8_multi(s, dtype, wf, epilogue, q);
+      if (st != MUI_OK) return st;
+    }
+    return MUI_OK;
+  }
 #define MUI_I8M_CASE(WFV, EPIV)                                          \
   if (wf == WFV && epilogue == EPIV) {                                   \
     if (p.tokens <= 1) return launch_i8m_t<EPIV, WFV, 1>(s, p);          \

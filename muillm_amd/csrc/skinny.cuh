@@ -16,7 +16,8 @@ struct SkinnyParams {
   const uint16_t* s1;
   long s_pitch;
   int group_shift;
-  const uint16_t* x;    // [tokens, k]
+  const uint16_t* x;    // [tokens, k], token rows x_pitch elements apart (0: k)
+  long x_pitch;         // honoured by the 1..4-token kernels (their K-segment calls); others need 0
   const uint16_t* gamma;
   const uint16_t* mul_bias;
   const uint16_t* add_bias;

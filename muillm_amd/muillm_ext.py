@@ -170,6 +170,9 @@ def muillm_linear_forward(
 
     if not (kernel_dispatchable(x) and weights.dtype == x.dtype):
         return _linear_unfused(x, weights, norm_weights, epsilon, mul_bias, add_bias, residual)
+    if k > 16384 and norm_weights is not None and _num_tokens(x) == 1:
+        # a fused norm needs the whole row in one pass of the single-token kernel
+        return _linear_unfused(x, weights, norm_weights, epsilon, mul_bias, add_bias, residual)
 
     _check_cuda(weights, "weights")
     pitch = _row_pitch(weights, "weights")
@@ -291,8 +294,9 @@ def _byte_pitch(w: torch.Tensor, name: str) -> int:
 
 
 def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
+    # rows longer than 16384: fp16 activations only (K segments / the streaming matrix-core kernel)
     return x.is_cuda and _is_16bit(x) and 1 <= _num_tokens(x) <= MUI_MAX_TOKENS and x.shape[-1] % 16 == 0 \
-        and x.shape[-1] <= 16384
+        and (x.shape[-1] <= 16384 or x.dtype == torch.float16)
 
 
 def mui_int8_channel_dequantize_forward(weights_i8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:

@@ -70,6 +70,22 @@ def test_channel_linear(n, k, tokens, norm):
     assert oracle.rel_err(y.cpu(), full) < 3e-2
 
 
+@pytest.mark.parametrize("tokens", [1, 3, 8])
+@pytest.mark.parametrize("k", [28672, 16400])
+def test_channel_linear_rows_longer_than_one_pass(tokens, k):
+    """K = 28672 (down projection of a 70B-class model): K segments accumulating through the
+    residual operand at up to 4 tokens, the streaming matrix-core kernel beyond."""
+    g = _gen(11)
+    n = 40
+    w = _mk((n, k), g, 0.02)
+    q, s = oracle.rtn_quantize_channel(w)
+    x = _mk((tokens, k), g)
+    r = _mk((tokens, n), g)
+    ref = oracle.int8_channel_linear(x, q, s, None, 0.0, None, r)
+    y = muillm_ext.mui_int8_channel_linear_forward(x.to(DEV), q.to(DEV), s.to(DEV), None, 0.0, None, r.to(DEV))
+    assert_parity(y, ref, 1e-2, f"int8 long rows {tokens} x {k}", tight=4e-3)
+
+
 @pytest.mark.parametrize("n,k", [(14336, 4096), (300, 1024), (5, 16)])
 @pytest.mark.parametrize("tokens", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("packed", [True, False])

@@ -198,6 +198,26 @@ def test_silu_mul_interleaved(rows, n, dtype):
     assert_parity(out, ref.float(), 1e-2, f"silu*mul {rows}x{n}")
 
 
+@pytest.mark.parametrize("tokens", [1, 3, 8])
+@pytest.mark.parametrize("k", [28672, 16392])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_rows_longer_than_one_pass(tokens, k, dtype):
+    """Down projections of 70B-class models (K = 28672): up to 4 tokens go through K segments that
+    accumulate through the residual operand, more tokens through the streaming matrix-core kernel."""
+    g = _gen(80 + tokens)
+    n = 72
+    w = _mk((n, k), g, 0.02, dtype=dtype)
+    x = _mk((tokens, k), g, dtype=dtype)
+    r = _mk((tokens, n), g, dtype=dtype)
+    mb = _mk((n,), g, 0.1, 1.0, dtype=dtype)
+    ab = _mk((n,), g, 0.1, dtype=dtype)
+    ref = oracle.linear(x, w, None, 0.0, ab, r, mul_bias=mb)
+    y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), mul_bias=mb.to(DEV), add_bias=ab.to(DEV),
+                                         residual=r.to(DEV))
+    assert y.shape == (tokens, n) and y.dtype == dtype
+    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 3e-2, f"long rows {tokens} x {k} {dtype}")
+
+
 def test_linear_reference_recipe_batch4():
     """tests/test_linear.py:13-43 of the reference: randn weights (seed 0), rand inputs of
     batch 4, compared with allclose(rtol 1e-4, atol 1e-1)."""
