@@ -314,12 +314,12 @@ def kernel_table(lm):
         name = "C2_mlp_%dx%d_tokens%d" % (inter, hid, b)
         add(name, mlp, 3 * inter * hid * 2 + 2 * hid + b * (3 * hid * 2 + 2 * inter * 2), nl,
             reads=[(gu_base, 4 * inter * hid), (dn, 2 * hid * inter)])
-        # arithmetic rate of the batched call; from 5 tokens on it runs on the matrix cores (padded
+        # arithmetic rate of the batched call; from 3 tokens on it runs on the matrix cores (padded
         # to 16 token columns), whose utilisation is this rate over the dense fp16 MFMA peak
         tflops = 6.0 * inter * hid * b / out[name]["us"] / 1e6
         out[name]["TFLOP/s"] = round(tflops, 1)
-        out[name]["compute_unit"] = "MFMA v_mfma_f32_16x16x32_f16" if b >= 5 else "vector ALUs"
-        if b >= 5:
+        out[name]["compute_unit"] = "MFMA v_mfma_f32_16x16x32_f16" if b >= 3 else "vector ALUs"
+        if b >= 3:
             out[name]["mfma_peak_frac"] = round(tflops / MFMA_FP16_PEAK_TFLOPS, 4)
             out[name]["mfma_issued_frac"] = round(tflops * 16.0 / b / MFMA_FP16_PEAK_TFLOPS, 4)
 

@@ -399,7 +399,7 @@ int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int di
  * that turns contiguous row runs into operands through LDS: 2 = operands loaded in MFMA order
  * straight from memory, token operands kept in registers (K <= 4096), 1 = the same with the
  * token operands re-read per weight tile; multi_max_tokens: largest token count served by the
- * multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 4; 5..8 only
+ * multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 2; 5..8 only
  * qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
 int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 

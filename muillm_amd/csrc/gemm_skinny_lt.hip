@@ -305,19 +305,20 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   // order, so the build only waits for the L2-resident token rows, not for the weight passes
   // behind them.
   u32x4 gv = {0u, 0u, 0u, 0u};
-  u32x4 xv[BSTAT ? 16 : 1];
+  constexpr int XT = HB ? 8 : 16;  // token rows brought in (B-stationary mode: built into operands)
+  u32x4 xv[BSTAT ? XT : 1];
   const bool b_ok = FULL || lane < 4 * jmax;
   if constexpr (BSTAT) {
     const int e = b_ok ? (wave * jmax * 4 + lane) << 3 : 0;  // element offset of this lane's chunk inside a row
     if constexpr (NORM) gv = ld16(p.gamma + e);
 #pragma unroll
-    for (int tk = 0; tk < 16; ++tk) xv[tk] = ld16(p.x + (long)(tk < p.tokens ? tk : tok_last) * p.k + e);
+    for (int tk = 0; tk < XT; ++tk) xv[tk] = ld16(p.x + (long)(tk < p.tokens ? tk : tok_last) * p.k + e);
   }
   auto build_b = [&]() {
     if constexpr (BSTAT) {
       const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int tk = 0; tk < 16; ++tk) {
+      for (int tk = 0; tk < XT; ++tk) {
         float ss = 0.f;
         xv[tk] = make_b<T, NORM>(b_ok ? xv[tk] : zero, gv, ss);
         if constexpr (NORM) {
@@ -329,7 +330,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
       for (int h = 0; h < 2; ++h) {
         if ((lane >> 5) == h) {
 #pragma unroll
-          for (int tk = 0; tk < 16; ++tk) *(u32x4*)(la + tk * kLtXPitch + xl_chunk * 16) = xv[tk];
+          for (int tk = 0; tk < XT; ++tk) *(u32x4*)(la + tk * kLtXPitch + xl_chunk * 16) = xv[tk];
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -413,8 +414,12 @@ static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
                      p.residual, p.mul_bias, p.add_bias, p.s0, p.s1, p.s_pitch, p.group_shift)
   if (p.k <= kLtWaves * 2 * kLtSub && p.k % 256 == 0) {
     const bool full = p.k == kLtWaves * 2 * kLtSub;
-    if (p.gamma) { if (full) MUI_LT(true, true, true, false, 1); else MUI_LT(true, true, false, false, 1); }
-    else { if (full) MUI_LT(false, true, true, false, 1); else MUI_LT(false, true, false, false, 1); }
+    const bool hb = p.tokens <= 8;
+#define MUI_LT_HB(NORMV, FULLV) \
+  { if (hb) MUI_LT(NORMV, true, FULLV, true, 1); else MUI_LT(NORMV, true, FULLV, false, 1); }
+    if (p.gamma) { if (full) MUI_LT_HB(true, true) else MUI_LT_HB(true, false) }
+    else { if (full) MUI_LT_HB(false, true) else MUI_LT_HB(false, false) }
+#undef MUI_LT_HB
     return launch_status();
   }
   // streaming: 16-byte chunks of weights and of token rows must not straddle the row end

@@ -273,7 +273,8 @@ static int g_skinny_min_tokens = 2;
 // gemv_kernel. bf16 takes the same route with v_dot2_f32_bf16.
 static int g_gemv_dot2 = 1;
 // largest token count that takes the multi-token GEMV (gemv_multi.hip) instead of the MFMA kernel
-static int g_multi_max_tokens = 4;
+// (3-4 tokens measured 1.8 us per decoder layer slower on it than on the MFMA kernel)
+static int g_multi_max_tokens = 2;
 
 extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens) {
   if (min_tokens < 1 || min_tokens > MUI_MAX_TOKENS + 1) return MUI_ERR_INVALID_ARG;
@@ -281,7 +282,7 @@ extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_token
   g_skinny_min_tokens = min_tokens;
   skinny_set_bstat(stream_b != 1);
   skinny_set_lt(stream_b == 0);
-  g_multi_max_tokens = multi_max_tokens == 0 ? 4 : multi_max_tokens;
+  g_multi_max_tokens = multi_max_tokens == 0 ? 2 : multi_max_tokens;
   skinny_set_int8_multi(g_multi_max_tokens >= 2);
   return MUI_OK;
 }

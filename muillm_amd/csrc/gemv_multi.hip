@@ -1,10 +1,10 @@
-// Fused linears for 1..4 tokens (opt-in up to 8 on tall matrices) with 16-bit weights: the single-token GEMV structure (256
-// threads, thread t owns 16-byte chunks t, t+256, ... of every row, R rows in flight, next row
-// group requested before the reduction, persistent balanced grid) with the token operands
-// gamma * x packed 16-bit in registers and one packed dot (v_dot2_f32_f16) per two weights and
-// token. The weights are streamed exactly once; at up to 4 tokens the vector ALUs stay far from
-// saturation, so the kernel runs at the single-token GEMV's HBM rate where the matrix-core
-// skinny GEMM (gemm_skinny_lt.hip, used from 5 tokens) pays for its operand hand-offs.
+// Fused linears for 1..2 tokens (3..4 and, on tall matrices, up to 8 on request) with 16-bit
+// weights: the single-token GEMV structure (256 threads, thread t owns 16-byte chunks t, t+256, ...
+// of every row, R rows in flight, next row group requested before the reduction, persistent
+// balanced grid) with the token operands gamma * x packed 16-bit in registers and one packed dot
+// (v_dot2_f32_f16) per two weights and token. The weights are streamed exactly once. From 3
+// tokens on the matrix-core skinny GEMM (gemm_skinny_lt.hip) is the default: it measured 0.2-1 us
+// per call faster there once it brought in only 8 token rows for up to 8 tokens.
 //
 // The reference has no kernel for this case (csrc/modules/linear_module.cpp:57-79 falls back to
 // RMSNorm + torch matmul + add; muillm/modules/gateupdownmlp.py:343-359).
