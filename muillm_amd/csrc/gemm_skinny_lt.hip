@@ -39,7 +39,7 @@ constexpr int kLtSteps = kLtSub / 32;        // MFMAs per pass
 constexpr int kLtXPitch = kLtSub * 2 + 16;   // LDS row pitch of a 16-bit operand tile, bytes
 constexpr int kLtXLoads = 8;                 // load instructions per 16-row tile of 16-bit values
 
-template <typename T, int WF, bool NORM, int EPI, bool BSTAT, bool FULL, bool HB>
+template <typename T, int WF, bool NORM, int EPI, bool BSTAT, bool FULL, bool HB, bool BIGP>
 __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     // scalars, hottest first (the leading ones are preloaded into SGPRs at wave launch)
     const void* w0, const void* w1, long pitch, const uint16_t* x, int n, int k, int tokens, int n_tiles, int spw,
@@ -51,7 +51,18 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   p.s0 = s0; p.s1 = s1; p.s_pitch = s_pitch; p.group_shift = group_shift;
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
   constexpr int WB = (WF == WF_16BIT) ? 2 : 1;   // bytes per weight
-  constexpr int ROWB = kLtSub * WB;              // bytes of a row segment of one pass
+  // k-values per wave and pass: 256 (512 bytes of a 16-bit row). Per-channel int8 weights in
+  // B-stationary mode can take 512 (BIGP), so that a pass again covers 512 contiguous bytes of
+  // each row and a load instruction two rows of them: with 256-byte runs and half the bytes in
+  // flight the int8 gate/up shape (7 tiles per workgroup) ran 33.7 us, with 512 it runs 27.9 us.
+  // With one or two tiles per workgroup the finer passes overlap better (QKV 8.9 vs 10.8 us), so
+  // the launcher picks by tiles per workgroup. (The group format stays at 256: its scale
+  // operands do not fit the register file beside the larger pass.)
+  constexpr int SUB = BIGP ? 2 * kLtSub : kLtSub;
+  static_assert(!BIGP || (BSTAT && WF == WF_I8_CHANNEL), "large passes: per-channel int8, B-stationary");
+  constexpr int STEPS = SUB / 32;                // MFMAs per pass
+  constexpr int PB = 2 * kLtSub / SUB;           // B-stationary: passes per tile (2 or 1)
+  constexpr int ROWB = SUB * WB;                 // bytes of a row segment of one pass
   constexpr int PITCH = ROWB + 16;               // LDS row pitch of the weight tile
   constexpr int RPI = 1024 / ROWB;               // rows covered by one load instruction (2 / 4)
   constexpr int NLD = 16 / RPI;                  // load instructions per weight tile (8 / 4)
@@ -83,9 +94,9 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   char* lb = &op_lds[wave][NOPS - 1][0];
 
   // B-stationary: this wave's K range is jmax MFMA steps = 32 * jmax k-values of every row,
-  // walked in two passes of 8 steps; streaming: spw passes of 256 k-values per tile
+  // walked in PB passes of STEPS steps; streaming: spw passes of 256 k-values per tile
   const int jmax = BSTAT ? (FULL ? 2 * kLtSteps : (p.k >> 8)) : 0;
-  const int passes = BSTAT ? 2 : spw;
+  const int passes = BSTAT ? PB : spw;
   const int my_tiles = blockIdx.x < n_tiles ? (n_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
   const int n_items = my_tiles * passes;  // pass i: tile blockIdx.x + (i / passes) * gridDim.x, sub-block i % passes
 
@@ -122,12 +133,12 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   // first k-value of pass i of this wave
   auto pass_k0 = [&](int i) -> int {
     const int sub = i % passes;
-    if constexpr (BSTAT) return wave * jmax * 32 + sub * kLtSub;
-    else return (wave * spw + sub) * kLtSub;
+    if constexpr (BSTAT) return wave * jmax * 32 + sub * SUB;
+    else return (wave * spw + sub) * SUB;
   };
   // k-values of pass i that exist (B-stationary: inside the wave's range; streaming: inside the row)
   auto pass_len = [&](int i) -> int {
-    if constexpr (BSTAT) return FULL ? kLtSub : jmax * 32 - (i % passes) * kLtSub;
+    if constexpr (BSTAT) return FULL ? SUB : jmax * 32 - (i % passes) * SUB;
     else return p.k - pass_k0(i);
   };
 
@@ -246,14 +257,14 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     }
     __builtin_amdgcn_wave_barrier();
   };
-  // one pass in operand order: 8 MFMA steps of 32 k-values (half: which half of the wave's range
-  // the pass covers in B-stationary mode; the register set fixes it)
+  // one pass in operand order: STEPS MFMA steps of 32 k-values (half: which part of the wave's
+  // range the pass covers in B-stationary mode; the register set fixes it)
   // (the operands are read back into the registers the pass came from: NLD = 8 = steps with
   // 16-bit weights, and the token tile of streaming mode has 8 loads as well)
   auto multiply = [&](int i, const int half, u32x4 (&a16)[NLD], u32x4 (&bx)[NB]) {
-    u32x2 a8[WF == WF_16BIT ? 1 : kLtSteps];
+    u32x2 a8[WF == WF_16BIT ? 1 : STEPS];
 #pragma unroll
-    for (int s = 0; s < kLtSteps; ++s) {  // all reads in flight at once
+    for (int s = 0; s < STEPS; ++s) {  // all reads in flight at once
       if constexpr (WF == WF_16BIT) a16[s] = *(const u32x4*)(la + r16 * PITCH + (4 * s + g) * 16);
       else a8[s] = *(const u32x2*)(la + r16 * PITCH + (4 * s + g) * 8);
       if constexpr (!BSTAT) bx[s] = *(const u32x4*)(lb + r16 * kLtXPitch + (4 * s + g) * 16);
@@ -261,12 +272,12 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     const uint16_t* srow = scale_row(blockIdx.x + (i / passes) * gridDim.x);
     const int k0 = pass_k0(i);
 #pragma unroll
-    for (int s = 0; s < kLtSteps; ++s) {
-      if (BSTAT && !FULL && half * kLtSteps + s >= jmax) break;
+    for (int s = 0; s < STEPS; ++s) {
+      if (BSTAT && !FULL && half * STEPS + s >= jmax) break;
       u32x4 av, bv;
       if constexpr (WF == WF_16BIT) av = a16[s];
       else av = convert_a<T, WF>(a8[s].x, a8[s].y, srow, k0 + 32 * s + 8 * g, p.group_shift);
-      if constexpr (BSTAT) bv = bq[half * kLtSteps + s];
+      if constexpr (BSTAT) bv = bq[half * STEPS + s];
       else bv = bx[s];
       if (s & 1) acc1 = mfma16x16x32<T>(av, bv, acc1);
       else acc = mfma16x16x32<T>(av, bv, acc);
@@ -347,7 +358,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
 #define MUI_LT_PASS(i_, U, REFILL)                    \
   {                                                   \
     stage((i_), as[U], bs[U], gs[U]);                 \
-    multiply((i_), (U) & 1, as[U], bs[U]);            \
+    multiply((i_), (U) % PB, as[U], bs[U]);           \
     if (REFILL) issue((i_) + NSET, as[U], bs[U], gs[U]); \
     finish((i_), ex[U]);                              \
     if (REFILL) issue_extras((i_) + NSET, ex[U]);     \
@@ -408,15 +419,23 @@ static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
   const int n_tiles = ceil_div(p.n, OUT);
   const int grid = balanced_grid(n_tiles, 1);  // ~150 KB of LDS: one workgroup per CU
-#define MUI_LT(NORMV, BSTATV, FULLV, HBV, SPW)                                                                  \
-  hipLaunchKernelGGL((gemm_skinny_lt_kernel<T, WF, NORMV, EPI, BSTATV, FULLV, HBV>), dim3(grid), dim3(kLtThreads), \
+#define MUI_LT(NORMV, BSTATV, FULLV, HBV, BIGV, SPW)                                                                  \
+  hipLaunchKernelGGL((gemm_skinny_lt_kernel<T, WF, NORMV, EPI, BSTATV, FULLV, HBV, BIGV>), dim3(grid), dim3(kLtThreads), \
                      0, s, p.w0, p.w1, p.pitch, p.x, p.n, p.k, p.tokens, n_tiles, SPW, p.gamma, p.y, p.eps,   \
                      p.residual, p.mul_bias, p.add_bias, p.s0, p.s1, p.s_pitch, p.group_shift)
   if (p.k <= kLtWaves * 2 * kLtSub && p.k % 256 == 0) {
     const bool full = p.k == kLtWaves * 2 * kLtSub;
     const bool hb = p.tokens <= 8;
-#define MUI_LT_HB(NORMV, FULLV) \
-  { if (hb) MUI_LT(NORMV, true, FULLV, true, 1); else MUI_LT(NORMV, true, FULLV, false, 1); }
+    const bool big = WF == WF_I8_CHANNEL && n_tiles >= 3 * grid;
+#define MUI_LT_HB(NORMV, FULLV)                                                                              \
+  {                                                                                                          \
+    if constexpr (WF == WF_I8_CHANNEL) {                                                                     \
+      if (big) { if (hb) MUI_LT(NORMV, true, FULLV, true, true, 1); else MUI_LT(NORMV, true, FULLV, false, true, 1); } \
+      else { if (hb) MUI_LT(NORMV, true, FULLV, true, false, 1); else MUI_LT(NORMV, true, FULLV, false, false, 1); }   \
+    } else {                                                                                                 \
+      if (hb) MUI_LT(NORMV, true, FULLV, true, false, 1); else MUI_LT(NORMV, true, FULLV, false, false, 1);  \
+    }                                                                                                        \
+  }
     if (p.gamma) { if (full) MUI_LT_HB(true, true) else MUI_LT_HB(true, false) }
     else { if (full) MUI_LT_HB(false, true) else MUI_LT_HB(false, false) }
 #undef MUI_LT_HB
@@ -426,8 +445,8 @@ static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
   if (p.k % (WF == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
   const int spw = ceil_div(ceil_div(p.k, kLtSub), kLtWaves);
   const bool hb = p.tokens <= 8;
-  if (p.gamma) { if (hb) MUI_LT(true, false, false, true, spw); else MUI_LT(true, false, false, false, spw); }
-  else { if (hb) MUI_LT(false, false, false, true, spw); else MUI_LT(false, false, false, false, spw); }
+  if (p.gamma) { if (hb) MUI_LT(true, false, false, true, false, spw); else MUI_LT(true, false, false, false, false, spw); }
+  else { if (hb) MUI_LT(false, false, false, true, false, spw); else MUI_LT(false, false, false, false, false, spw); }
 #undef MUI_LT
   return launch_status();
 }
