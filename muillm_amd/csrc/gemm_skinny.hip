@@ -381,9 +381,11 @@ void skinny_set_int8_multi(int on) { g_int8_multi = on; }
 
 // entry used by gemv.hip / int8.hip for tokens >= 2
 int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams& p) {
-  // int8 at up to 4 tokens: the vector-ALU kernel, except long rows at 3-4 tokens where the
-  // matrix-core kernel measured faster (down 4096 x 14336 at 4 tokens: 15.6 vs 16.4 us)
-  if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4 && !(g_skinny_lt && p.tokens >= 3 && p.k > 8192)) {
+  // int8 at up to 4 tokens: the vector-ALU kernel, except at 3-4 tokens long rows (down 4096 x
+  // 14336 at 4 tokens: 13.6 vs 16.4 us) and tall gate/up matrices (2 x 14336 x 4096: a steady
+  // 27 us against 27-34 us), where the matrix-core kernel measured faster
+  const bool lt_first = g_skinny_lt && p.tokens >= 3 && (p.k > 8192 || (epi == SK_GATEUP && p.n >= 8192));
+  if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4 && !lt_first) {
     const int st = launch_int8_multi(s, dtype, wf, epi, p);
     if (st != MUI_ERR_UNSUPPORTED) return st;
   }

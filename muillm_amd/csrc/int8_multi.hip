@@ -98,17 +98,17 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       }
     }
   };
-  // ---- token operands: gamma * x as packed fp16, the chunk's sum of them on the side. With a fused norm they
-  // are requested before the first weights: loads return in order, so the operand preparation and
-  // the norm's reduction then overlap the flight of the first row group instead of following it.
-  // No load sits behind a branch (clamped addresses, dead lanes zeroed by selects).
+  // ---- token operands: gamma * x as packed fp16, the chunk's sum of them on the side. They are
+  // requested before the first weights: loads return in order, so the operand preparation (and a
+  // fused norm's reduction) then overlaps the flight of the first row group instead of following
+  // it (QKV with fused norm 7.5 -> 6.4 us at one token). No load sits behind a branch (clamped
+  // addresses, dead lanes zeroed by selects).
   int rg = blockIdx.x;  // the grid never exceeds the number of row groups
-  if constexpr (!NORM) issue(rg);  // nothing to prepare: the weights go first
   u32x4 xq[TOK][CH][2];
   u32x4 gq[CH][2];
 #pragma unroll
   for (int tk = 0; tk < TOK; ++tk) {
-    const long xrow = (long)(tk < tokens ? tk : tokens - 1) * a.x_pitch;
+    const long xrow = tk == 0 ? 0 : (long)(tk < tokens ? tk : tokens - 1) * a.x_pitch;
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
 #pragma unroll
@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       for (int hf = 0; hf < 2; ++hf) gq[j][hf] = ld16(gamma + coff[j] + 8 * hf);
     }
   }
-  if constexpr (NORM) issue(rg);
+  issue(rg);
 
   float xsum[TOK][CH];
   float ss[TOK];
