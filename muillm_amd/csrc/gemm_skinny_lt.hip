@@ -106,7 +106,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     const void* wbase;
     if constexpr (EPI == SK_GATEUP) {
       out_row = tl * 8 + (r >> 1);
-      wbase = (r & 1) ? p.w1 : p.w0;
+      wbase = (r & 1) ? w1 : w0;
     } else {
       out_row = tl * 16 + r;
       wbase = p.w0;
@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     const uint16_t* sbase;
     if constexpr (EPI == SK_GATEUP) {
       out_row = tl * 8 + (r16 >> 1);
-      sbase = (r16 & 1) ? p.s1 : p.s0;
+      sbase = (r16 & 1) ? s1 : s0;
     } else {
       out_row = tl * 16 + r16;
       sbase = p.s0;
