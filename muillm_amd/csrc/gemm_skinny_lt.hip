@@ -296,7 +296,10 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
       if (BSTAT && !FULL && half * STEPS + s >= jmax) break;
       u32x4 av, bv;
       if constexpr (WF == WF_16BIT) av = a16[s];
-      else av = convert_a<T, WF>(a8[s].x, a8[s].y, srow, k0 + 32 * s + 8 * g, p.group_shift);
+      else {
+        const int ke = k0 + 32 * s + 8 * g;  // (clamped: the scale pair of a k past the row end is never used)
+        av = convert_a<T, WF>(a8[s].x, a8[s].y, srow, ke < p.k ? ke : p.k - 1, p.group_shift);
+      }
       if constexpr (BSTAT) bv = bq[half * STEPS + s];
       else bv = bx[s];
       if (s & 1) acc1 = mfma16x16x32<T>(av, bv, acc1);
