@@ -26,6 +26,8 @@
 extern "C" {
 #endif
 
+/* bumped whenever a struct below changes layout or an entry point changes its arguments;
+ * mui_abi_version() returns the value the library was built with */
 #define MUI_ABI_VERSION 2
 
 /* status codes (reference: TORCH_CHECK exceptions, csrc/linear/linear.cu:72-74;

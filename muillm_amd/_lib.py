@@ -104,6 +104,8 @@ class MuiDecoderStackDesc(ctypes.Structure):
                 ("cache_token_stride", c_long), ("max_cache_len", c_int)]
 
 
+MUI_ABI_VERSION = 2  # MUI_ABI_VERSION of the public header: layout of the structs above
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -134,6 +136,10 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
+    if lib.mui_abi_version() != MUI_ABI_VERSION:
+        raise MuiLibraryError(
+            f"{LIB_PATH} has ABI version {lib.mui_abi_version()}, this package expects {MUI_ABI_VERSION} "
+            "(the descriptor structs differ): rebuild it with `make -C muillm_amd/csrc`.")
     _lib = lib
     return lib
 

@@ -42,7 +42,7 @@ def test_no_framework_types_in_header():
 
 def test_status_strings_and_version():
     lib = _lib.load()
-    assert lib.mui_abi_version() == 2
+    assert lib.mui_abi_version() == _lib.MUI_ABI_VERSION == 2
     assert _lib.status_string(0) == "ok"
     for code in (-1, -2, -3, -4, -5):
         assert _lib.status_string(code) not in ("ok", "unknown status")
