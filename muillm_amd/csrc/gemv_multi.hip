@@ -226,9 +226,13 @@ static int launch_mt_t(hipStream_t s, const SkinnyParams& p) {
   }
   constexpr int R = 2, OUT = (EPI == SK_GATEUP) ? 1 : 2;
   const int tuned = gemv_tuned_wgs_per_cu();
-  // long rows: 2 workgroups per CU; one token: 4 (18.35 against 18.65 us on 4096 x 14336; with the
-  // operand registers of 4 tokens the same choice measured 22.3 against 21.3 us)
-  const int grid = balanced_grid(ceil_div(p.n, OUT), tuned > 0 ? tuned : (TOK == 1 ? 4 : 2));
+  // long rows: 2 workgroups per CU. One token, rows of 5+ chunks per thread and a row-group count
+  // that fills 4 workgroups per CU evenly: 4 (18.35 against 18.65 us on 4096 x 14336). Elsewhere 4
+  // measured slower (15360 x 5120: 26.6 against 24.9 us; 5120 x 13824, whose 2560 groups do not
+  // split evenly: 23.1 against 22.0 us; with the operand registers of 4 tokens 22.3 against 21.3 us).
+  const int n_groups = ceil_div(p.n, OUT);
+  const bool four = TOK == 1 && ch > 4 && n_groups % (device_cus() * 4) == 0;
+  const int grid = balanced_grid(n_groups, tuned > 0 ? tuned : (four ? 4 : 2));
   if (ch <= 4) return launch_mt_rc<T, R, 4, EPI, TOK>(s, p, grid);
   if (ch <= 7) return launch_mt_rc<T, R, 7, EPI, TOK>(s, p, grid);
   return MUI_ERR_UNSUPPORTED;
