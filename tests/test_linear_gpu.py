@@ -381,3 +381,25 @@ def test_read_probe_reads_and_discards():
     assert lib.mui_probe_read(stream, src.data_ptr() + 8, 64, sink.data_ptr()) != 0
     assert lib.mui_probe_read(stream, src.data_ptr(), 24, sink.data_ptr()) != 0
     assert lib.mui_probe_read(stream, None, 64, sink.data_ptr()) != 0
+
+
+@pytest.mark.parametrize("tokens", [17, 32])
+def test_short_prompt_goes_through_the_fused_kernels_in_chunks(tokens):
+    """17..32 tokens: two calls of the 16-token kernels instead of norm + library GEMM + add."""
+    assert muillm_ext.FUSED_CHUNK_MAX_TOKENS == 32
+    g = _gen(90 + tokens)
+    n, k = 520, 1024
+    w = _mk((n, k), g, 0.02)
+    x = _mk((2, tokens // 2 if tokens % 2 == 0 else 1, k), g) if tokens % 2 == 0 else _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    r = _mk(tuple(x.shape[:-1]) + (n,), g)
+    assert muillm_ext.kernel_dispatchable(x.to(DEV))
+    ref = oracle.linear(x, w, gamma, 1e-5, None, r)
+    y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), gamma.to(DEV), 1e-5, residual=r.to(DEV))
+    assert y.shape == r.shape
+    assert_parity(y, ref, 1e-2, f"chunked linear {tokens}", tight=4e-3)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    packed = torch.stack((wg, wu), dim=1).to(DEV)
+    h = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, packed[:, 0], packed[:, 1], x.to(DEV))
+    assert_parity(h, oracle.gateup_silu(x, wg, wu, gamma, 1e-5), 1e-2, f"chunked gate/up {tokens}")
+    assert not muillm_ext.kernel_dispatchable(torch.zeros(33, k, dtype=torch.float16, device=DEV))
