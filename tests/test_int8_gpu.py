@@ -200,3 +200,29 @@ def test_int8_abi_errors():
     xx = _mk((24,), g)
     yy = muillm_ext.mui_int8_channel_linear_forward(xx.to(DEV), q.to(DEV), s_.to(DEV))
     assert_parity(yy, oracle.int8_channel_linear(xx, q, s_), 1e-2, "K=24")
+
+
+@pytest.mark.parametrize("tokens", [17, 40, 64])
+def test_channel_linear_and_gateup_in_chunks(tokens):
+    """17..64 tokens go through the 16-token int8 kernels in chunks (the alternative would be
+    dequantising the whole matrix for a library GEMM)."""
+    assert muillm_ext.INT8_CHUNK_MAX_TOKENS == 64
+    g = _gen(31)
+    n, k = 264, 1024
+    w = _mk((n, k), g, 0.02)
+    q, s = oracle.rtn_quantize_channel(w)
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    r = _mk((tokens, n), g)
+    assert muillm_ext.int8_kernel_dispatchable(x.to(DEV))
+    ref = oracle.int8_channel_linear(x, q, s, gamma, 1e-5, None, r)
+    y = muillm_ext.mui_int8_channel_linear_forward(x.to(DEV), q.to(DEV), s.to(DEV), gamma.to(DEV), 1e-5, None, r.to(DEV))
+    assert y.shape == (tokens, n)
+    assert_parity(y, ref, 1e-2, f"int8 chunks {tokens}", tight=4e-3)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    (qg, sg), (qu, su) = oracle.rtn_quantize_channel(wg), oracle.rtn_quantize_channel(wu)
+    h = muillm_ext.mui_int8_channel_gateupsilu_forward(gamma.to(DEV), 1e-5, qg.to(DEV), qu.to(DEV), sg.to(DEV),
+                                                       su.to(DEV), x.to(DEV))
+    ref_h = oracle.gateup_silu(x, oracle.rtn_dequantize_channel(qg, sg), oracle.rtn_dequantize_channel(qu, su), gamma, 1e-5)
+    assert_parity(h, ref_h, 1e-2, f"int8 gate/up chunks {tokens}")
+    assert not muillm_ext.int8_kernel_dispatchable(torch.zeros(65, k, dtype=torch.float16, device=DEV))
