@@ -188,6 +188,39 @@ def test_model_prefill_and_decode_vs_oracle():
     assert cache.get_max_length() == 32  # grew by the power-of-two schedule
 
 
+def test_model_three_query_heads_per_kv_head_and_chunked_prompt():
+    """A 6 / 2-head decoder (ratio 3, as in Llama-3.2-3B) with a 17-token prompt (the fused linears
+    run in two chunks): prefill and greedy decode against the oracle, through the layer modules and
+    through the single-call stack."""
+    cfg = MuiDecoderConfig(hidden_size=768, intermediate_size=1536, num_hidden_layers=2, num_attention_heads=6,
+                           num_key_value_heads=2, vocab_size=512, max_position_embeddings=256,
+                           rope_theta=500000.0, rms_norm_eps=1e-5)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=7,
+                                         init_std=0.05)
+    params = _oracle_params(lm)
+    d = 128
+    cos, sin = oracle.rope_tables(cfg.rope_theta, d, cfg.max_position_embeddings)
+    ids = torch.randint(0, cfg.vocab_size, (1, 17), generator=torch.Generator().manual_seed(7))
+    for use_stack in (False, True):
+        lm.model.use_decoder_stack = use_stack
+        kcs = [torch.zeros(1, 2, 64, d, dtype=torch.float16) for _ in range(2)]
+        vcs = [torch.zeros(1, 2, 64, d, dtype=torch.float16) for _ in range(2)]
+        ref_logits, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, 6, 2)
+        with torch.no_grad():
+            out = lm(input_ids=ids.to(DEV))
+        assert_parity(out.logits, ref_logits, 1e-2, "prefill logits (ratio 3)")
+        cache = out.past_key_values
+        nxt = ref_logits[:, -1].argmax(-1)
+        for step in range(4):
+            ref_logits, seen = oracle.decoder_model_step(nxt.unsqueeze(1), params, kcs, vcs, cos, sin, seen, 6, 2)
+            with torch.no_grad():
+                out = lm(input_ids=nxt.unsqueeze(1).to(DEV), past_key_values=cache)
+            assert_parity(out.logits, ref_logits, 1e-2, f"decode step {step} (ratio 3, stack={use_stack})")
+            nxt = ref_logits[:, -1].argmax(-1)
+        assert (lm.model._stack is not None) == use_stack
+    lm.model.use_decoder_stack = True
+
+
 @pytest.mark.parametrize("batch", [1, 2])
 def test_graph_decode_matches_eager(batch):
     cfg = _small_config(layers=3)
