@@ -115,6 +115,22 @@ def measured_copy_ceiling():
     return round(2 * n * 2 / us / 1e3, 1)
 
 
+def measured_read_ceiling():
+    """Read-only rate of the library's probe kernel (the GEMVs' access shape, nothing but loads)
+    over 1 GiB buffers, rotating over 3 of them: what a kernel that only has to read can reach."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    n = 1 << 30
+    src = [torch.empty(n, device="cuda", dtype=torch.uint8).fill_(1) for _ in range(3)]
+    sink = torch.zeros(64, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    us = _event_time_us(lambda i: lib.mui_probe_read(stream, src[i % 3].data_ptr(), n, sink.data_ptr()), iters=12, warm=3)
+    return round(n / us / 1e3, 1)
+
+
 def gateup_roofline(lm):
     """Average launch duration of the fused gate/up+SiLU GEMV over the model's 32 distinct
     (cold) weight buffers, HIP events on the launch stream."""
@@ -533,6 +549,7 @@ def main():
     }
     result["roofline"] = gateup_roofline(lm)
     result["roofline"]["measured_copy_ceiling_GB/s"] = measured_copy_ceiling()
+    result["roofline"]["measured_read_ceiling_GB/s"] = measured_read_ceiling()
     if not args.no_kernel_table:
         result["kernels"] = kernel_table(lm)
     del dec
