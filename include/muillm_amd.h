@@ -7,7 +7,9 @@
  *   - enqueues asynchronously on that stream and never synchronises or allocates;
  *   - owns nothing: outputs and scratch are caller-allocated;
  *   - returns MUI_OK (0) or a negative MUI_ERR_* code (mui_status_string() names it);
- *   - validates shapes/alignment on the host before launching anything.
+ *   - validates shapes/alignment on the host before launching anything;
+ *   - keeps no state between calls (the sweep aids that do are declared apart, in
+ *     muillm_amd_tune.h).
  *
  * The comment above each declaration names the entry of the reference's pybind11
  * module `muillm_ext` (Epliz/muiLLM, csrc/module.cpp) that it stands in for.
@@ -374,43 +376,6 @@ int mui_decoder_stack_step(mui_stream_t stream, const mui_decoder_stack_t* model
  * [n_tokens, dim]. */
 int mui_embedding(mui_stream_t stream, int dtype, const void* table, long row_pitch,
                   const void* ids, int ids_are_int32, void* out, int n_tokens, int dim, int vocab);
-
-/* ------------------------------------------------------------------------------------
- * Launch-shape knobs used by the benchmark sweeps (0 restores the built-in choice). They
- * have no counterpart in the reference, whose launch shapes are compile-time constants
- * (csrc/linear/linear_fp16_kernels.cu:646-654).
- * ---------------------------------------------------------------------------------- */
-int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
-/* single-token routing: linear_on -> mui_linear (and bf16 mui_gateup_silu) through the packed-dot
- * kernel of the multi-token GEMV (default on); int8_on -> a single fp16 token of the int8 entry
- * points through the packed-dot int8 kernel (default on) */
-int mui_tune_packed_dot(int linear_on, int int8_on);
-int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
-/* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
- * fewest cached tokens that justify one more sequence split (default: two passes), and the
- * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1536;
- * negative: never use the unsplit one-workgroup-per-query-head mode), and mfma_tokens for the
- * matrix-core decode kernel: 0 = default (whenever a workgroup handles a whole KV group, i.e.
- * everywhere but in the unsplit one-workgroup-per-query-head mode), n > 0 = also instead of
- * that mode for sequences (or cache capacities, when the length is read on the device) of at
- * least n tokens, negative = never (vector-ALU kernel only) */
-int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
-                       int mfma_tokens);
-/* fewest tokens that leave the one-GEMV-per-token loop (default 2; MUI_MAX_TOKENS + 1 keeps the
- * loop); stream_b selects older MFMA variants for 16-bit weights instead of the default one
- * that turns contiguous row runs into operands through LDS: 2 = operands loaded in MFMA order
- * straight from memory, token operands kept in registers (K <= 4096), 1 = the same with the
- * token operands re-read per weight tile; multi_max_tokens: largest token count served by the
- * multi-token GEMV rather than the MFMA kernel (16-bit weights; 0 = default 2; 5..8 only
- * qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
-int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
-
-/* Measurement aid without a counterpart in the reference: reads `bytes` (a multiple of 16, from
- * a 16-byte aligned address) of device memory once with the access shape of the GEMV kernels and
- * discards them. One launch takes the least time any kernel that must read that many bytes can
- * take on this device, launch latency included. `sink` is any 256-byte device buffer (written
- * only if the data matches a fixed 16-byte pattern). */
-int mui_probe_read(mui_stream_t stream, const void* src, uint64_t bytes, void* sink);
 
 #ifdef __cplusplus
 }

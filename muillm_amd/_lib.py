@@ -14,6 +14,8 @@ from typing import Dict, List, Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmuillm_amd.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "muillm_amd.h")
+# measurement aids (process-global launch-shape overrides, bandwidth probe): not product ABI
+TUNE_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "muillm_amd_tune.h")
 
 MUI_OK = 0
 MUI_DTYPE_F16 = 0
@@ -109,12 +111,18 @@ MUI_ABI_VERSION = 2  # MUI_ABI_VERSION of the public header: layout of the struc
 _lib: Optional[ctypes.CDLL] = None
 
 
-def declared_functions(header_path: str = HEADER_PATH) -> List[str]:
-    """Names of the functions the public header declares."""
-    with open(header_path, "r") as f:
-        text = f.read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mui_[a-z0-9_]+)\s*\(", text)))
+def header_text(*paths: str) -> str:
+    """Concatenated text of the given headers (default: both) with comments removed."""
+    out = []
+    for path in paths or (HEADER_PATH, TUNE_HEADER_PATH):
+        with open(path, "r") as f:
+            out.append(re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S))
+    return "\n".join(out)
+
+
+def declared_functions(*paths: str) -> List[str]:
+    """Names of the functions the given headers (default: product + tuning header) declare."""
+    return sorted(set(re.findall(r"\b(mui_[a-z0-9_]+)\s*\(", header_text(*paths))))
 
 
 def load() -> ctypes.CDLL:

@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include "../../include/muillm_amd.h"
+#include "../../include/muillm_amd_tune.h"
 
 namespace mui {
 

@@ -23,8 +23,7 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 
 def test_signature_arity_matches_header():
-    with open(_lib.HEADER_PATH) as f:
-        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    text = _lib.header_text()
     for name, (_, argtypes) in _lib._SIGNATURES.items():
         m = re.search(r"\b%s\s*\(([^;]*?)\)\s*;" % name, text, flags=re.S)
         assert m, name
@@ -34,10 +33,17 @@ def test_signature_arity_matches_header():
 
 
 def test_no_framework_types_in_header():
-    with open(_lib.HEADER_PATH) as f:
-        text = f.read()
+    text = _lib.header_text()
     for banned in ("torch", "at::", "Tensor", "hipStream_t stream", "#include <hip"):
-        assert banned not in re.sub(r"/\*.*?\*/", "", text, flags=re.S), banned
+        assert banned not in text, banned
+
+
+def test_product_header_holds_no_process_global_knobs():
+    """The stateless product ABI and the sweep aids live in separate headers."""
+    product = _lib.declared_functions(_lib.HEADER_PATH)
+    aids = _lib.declared_functions(_lib.TUNE_HEADER_PATH)
+    assert not [n for n in product if n.startswith("mui_tune") or n.startswith("mui_probe")]
+    assert aids and all(n.startswith("mui_tune") or n.startswith("mui_probe") for n in aids)
 
 
 def test_status_strings_and_version():

@@ -6,6 +6,7 @@ slot is untouched.  The reference has no test for these kernels; the recipes her
 closed forms of softmax attention plus the prefill-then-decode sequence of the reference's
 static-cache test (tests/test_static_kvcache.py:52-112 there)."""
 
+import functools
 import math
 
 import pytest
@@ -217,9 +218,17 @@ def test_flash_decode_masked():
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_fused_decode(b, s, cap, device_len, dtype):
     """Config 4 recipe: cache pre-filled for s-1 positions, new token at position s-1."""
-    if dtype == torch.bfloat16 and s > 1024:
-        pytest.skip("bf16 twin covered at the smaller shapes")
     _fused_decode_case(b, s, cap, device_len, dtype, 32, 8)
+
+
+@pytest.mark.parametrize("b,s", [(1, 16384), (8, 16384), (1, 32768), (8, 32768)])
+def test_fused_decode_long_context(b, s):
+    """Config 4 at its long contexts, batch 1 and 8, through the entry point the decoder calls
+    (RoPE + cache write + split flash decoding + merge); fp16, and bf16 at batch 1. Every batch
+    row is checked against the oracle."""
+    _fused_decode_case(b, s, s, True, torch.float16, 32, 8)
+    if b == 1:
+        _fused_decode_case(b, s, s, False, torch.bfloat16, 32, 8)
 
 
 @pytest.mark.parametrize("hq,hkv", [(24, 8), (20, 4), (12, 2), (14, 2), (32, 2), (12, 1)])
@@ -229,7 +238,10 @@ def test_fused_decode_other_group_sizes(hq, hkv, b, s, cap):
     _fused_decode_case(b, s, cap, True, torch.float16, hq, hkv)
 
 
-def _fused_decode_case(b, s, cap, device_len, dtype, hq, hkv):
+@functools.lru_cache(maxsize=8)
+def _fused_decode_inputs(b, s, cap, dtype, hq, hkv):
+    """Seeded inputs and the oracle's result of one fused-decode case (kept for the runs of the
+    same case under the other kernel choices: the long contexts take seconds to generate)."""
     g = _gen(7)
     cos, sin = oracle.rope_tables(500000.0, D, cap)
     qkv = _mk((b, 1, (hq + 2 * hkv) * D), g, dtype=dtype)
@@ -248,6 +260,11 @@ def _fused_decode_case(b, s, cap, device_len, dtype, hq, hkv):
     kref, vref = kc.clone(), vc.clone()
     kk, vv, _ = oracle.static_cache_update(kref, vref, rk, v, cpos, s - 1)
     ref = oracle.decode_attention(rq, kk, vv)
+    return cos, sin, qkv, kc, vc, pos, cpos, v, rk, ref
+
+
+def _fused_decode_case(b, s, cap, device_len, dtype, hq, hkv):
+    cos, sin, qkv, kc, vc, pos, cpos, v, rk, ref = _fused_decode_inputs(b, s, cap, dtype, hq, hkv)
 
     qkv_d, kd, vd = qkv.to(DEV), kc.to(DEV), vc.to(DEV)
     qd = qkv_d[:, 0, : hq * D]

@@ -1,0 +1,131 @@
+"""Parity at the sizes the benchmark is quoted on (Llama-3-8B shape: hidden 4096, intermediate
+14336, 32 query / 8 KV heads of 128, RMSNorm eps 1e-5, weights ~ N(0, 0.02)):
+
+* one full-shape decoder layer (+ embedding, final norm and a small lm_head) against the CPU
+  oracle, 32-token prompt then single-token decode steps: fp16, bf16 and per-channel int8;
+* the whole 32-layer model: tokens and logits of HIP-graph replay == eager decode, bit for bit,
+  for a 32-token prompt + 32 greedy steps (fp16, bf16, per-channel int8).
+
+The second test follows the recipe of the reference's static-cache test (prefill, then
+single-token steps over a growing static cache, tests/test_static_kvcache.py:52-112 there)."""
+
+import copy
+
+import pytest
+import torch
+
+import oracle
+from muillm_amd.engine import init_engine
+from muillm_amd.engineconfig import MuiEngineConfig
+from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
+from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
+from muillm_amd.modules.quantized.int8gateupdownmlp import MuiInt8GateUpDownMLP
+from muillm_amd.modules.quantized.int8linear import MuiInt8Linear
+from muillm_amd.quantization.quantizationmethod import Int8WeightOnlyQuantizationMethod
+from tests.util import assert_parity
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+HQ, HKV, D = 32, 8, 128
+
+
+def _cfg(layers, vocab):
+    return MuiDecoderConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=layers,
+                            num_attention_heads=HQ, num_key_value_heads=HKV, vocab_size=vocab,
+                            max_position_embeddings=512, rope_theta=500000.0, rms_norm_eps=1e-5)
+
+
+def _exact_channel_weights(q, s):
+    """q * s without the 16-bit rounding of a dense dequantisation: what the int8 GEMV accumulates."""
+    return q.detach().cpu().double() * s.detach().cpu().double()[:, None]
+
+
+def _oracle_params(lm):
+    """Weights of a (possibly int8) MuiLlamaForCausalLM as CPU tensors in the oracle's layout."""
+    cfg = lm.config
+    layers = []
+    for layer in lm.model.layers:
+        qkv, o, mlp = layer.qkv_proj.linear, layer.self_attn.o_proj, layer.mlp
+        if isinstance(qkv, MuiInt8Linear):
+            w = _exact_channel_weights(qkv.weights_int8, qkv.scales)
+        else:
+            w = qkv.weight.detach().cpu()
+        wo = _exact_channel_weights(o.weights_int8, o.scales) if isinstance(o, MuiInt8Linear) else o.weight.detach().cpu()
+        if isinstance(mlp, MuiInt8GateUpDownMLP):
+            wg = _exact_channel_weights(mlp.gate_up_weights[:, 0], mlp.gate_up_scales[:, 0])
+            wu = _exact_channel_weights(mlp.gate_up_weights[:, 1], mlp.gate_up_scales[:, 1])
+            wd = _exact_channel_weights(mlp.down_proj.weights_int8, mlp.down_proj.scales)
+        else:
+            wg, wu, wd = (m.weight.detach().cpu() for m in (mlp.gate_proj, mlp.up_proj, mlp.down_proj))
+        layers.append(dict(ln1=qkv.norm_weights.detach().cpu(), wq=w[: HQ * D], wk=w[HQ * D : (HQ + HKV) * D],
+                           wv=w[(HQ + HKV) * D :], wo=wo, ln2=mlp.norm_weights.detach().cpu(), wg=wg, wu=wu, wd=wd,
+                           eps=cfg.rms_norm_eps))
+    return dict(embed=lm.model.embed_tokens.weight.detach().cpu(), layers=layers,
+                norm=lm.model.norm.weight.detach().cpu(), lm_head=lm.lm_head.weight.detach().cpu(),
+                eps=cfg.rms_norm_eps)
+
+
+def _build(layers, vocab, dtype, int8, seed):
+    cfg = _cfg(layers, vocab)
+    if not int8:
+        return MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=dtype, device=DEV, seed=seed,
+                                               init_std=0.02)
+    base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=dtype, device=DEV, seed=seed,
+                                           init_std=0.02, finalize=False)
+    qm = Int8WeightOnlyQuantizationMethod(group_size=0, modules=["qkv_proj", "o_proj", "mlp"])
+    return init_engine(base, device=DEV, engine_config=MuiEngineConfig(qm))
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "int8"])
+def test_full_shape_decoder_layer_vs_oracle(kind):
+    """Gate: logits within 1e-2 (fp16, int8 weights with fp16 activations) / 3e-2 (bf16: 8-bit
+    significands at five rounding points per layer) of the oracle, max error over max |ref|."""
+    dtype = torch.bfloat16 if kind == "bf16" else torch.float16
+    lm = _build(1, 2048, dtype, kind == "int8", seed=21)
+    with torch.no_grad():
+        # norm gammas away from 1 so that a dropped or misplaced gamma shows
+        for layer in lm.model.layers:
+            layer.qkv_proj.linear.norm_weights.copy_(1 + 0.1 * torch.randn(4096, generator=torch.Generator().manual_seed(1)))
+            layer.mlp.norm_weights.copy_(1 + 0.1 * torch.randn(4096, generator=torch.Generator().manual_seed(2)))
+    params = _oracle_params(lm)
+    cos, sin = oracle.rope_tables(500000.0, D, 512)
+    ids = torch.randint(0, 2048, (1, 32), generator=torch.Generator().manual_seed(3))
+    kcs = [torch.zeros(1, HKV, 64, D, dtype=dtype)]
+    vcs = [torch.zeros(1, HKV, 64, D, dtype=dtype)]
+    tol = 3e-2 if kind == "bf16" else 1e-2
+    ref, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, HQ, HKV, store_dtype=dtype)
+    with torch.no_grad():
+        out = lm(input_ids=ids.to(DEV))
+    assert_parity(out.logits, ref, tol, f"{kind} full-shape prefill logits")
+    cache = out.past_key_values
+    nxt = ref[:, -1].argmax(-1)
+    for step in range(3):
+        ref, seen = oracle.decoder_model_step(nxt.unsqueeze(1), params, kcs, vcs, cos, sin, seen, HQ, HKV,
+                                              store_dtype=dtype)
+        with torch.no_grad():
+            out = lm(input_ids=nxt.unsqueeze(1).to(DEV), past_key_values=cache)
+        assert_parity(out.logits, ref, tol, f"{kind} full-shape decode step {step}")
+        nxt = ref[:, -1].argmax(-1)
+    # the layer's cache rows equal the oracle's within one 16-bit ulp of rounding flips
+    kd = cache.key_cache[0][:, :, :seen].float().cpu()
+    assert float((kd - kcs[0][:, :, :seen].float()).abs().max()) <= (0.05 if kind == "bf16" else 0.01)
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "int8"])
+def test_full_model_graph_replay_equals_eager(kind):
+    """The 32-layer, vocabulary-128256 model the headline number is quoted on: 32-token prompt,
+    32 greedy steps; tokens and per-step logits identical between HIP-graph replay and eager."""
+    dtype = torch.bfloat16 if kind == "bf16" else torch.float16
+    lm = _build(32, 128256, dtype, kind == "int8", seed=0)
+    ids = torch.randint(0, 128256, (1, 32), generator=torch.Generator().manual_seed(0)).to(DEV)
+    n_new = 32
+    eager, eager_logits = lm.generate_greedy(ids, n_new, use_graph=False, return_logits=True)
+    dec = MuiGraphDecoder(lm, use_graph=True)
+    graph, graph_logits = dec.generate(ids, n_new, return_logits=True)
+    assert eager.shape == (1, 32 + n_new)
+    assert torch.isfinite(eager_logits).all()
+    assert torch.equal(eager, graph), "graph replay and eager decode disagree"
+    assert torch.equal(eager_logits, graph_logits)
+    assert len(set(eager[0, 32:].tolist())) > 1, "degenerate generation"
+    del lm, dec
+    torch.cuda.empty_cache()
