@@ -78,8 +78,12 @@ def _build(layers, vocab, dtype, int8, seed):
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16", "int8"])
 def test_full_shape_decoder_layer_vs_oracle(kind):
-    """Gate: logits within 1e-2 (fp16, int8 weights with fp16 activations) / 3e-2 (bf16: 8-bit
-    significands at five rounding points per layer) of the oracle, max error over max |ref|."""
+    """Gate: logits within 1e-2 (fp16, int8 weights with fp16 activations) of the oracle, max error
+    over max |ref| and elementwise. bf16: 3e-2 on the max form and 5e-2 elementwise -- the bf16
+    kernels feed gamma * x, rounded once to bf16, to the packed dot / matrix-core instructions (the
+    HuggingFace layers round the normalised activations to bf16 as well), the oracle keeps them
+    exact: a 2^-9 relative perturbation of every operand of five chained projections, which over
+    65536 logits puts a handful beyond 3 % of the logits' rms."""
     dtype = torch.bfloat16 if kind == "bf16" else torch.float16
     lm = _build(1, 2048, dtype, kind == "int8", seed=21)
     with torch.no_grad():
@@ -93,10 +97,11 @@ def test_full_shape_decoder_layer_vs_oracle(kind):
     kcs = [torch.zeros(1, HKV, 64, D, dtype=dtype)]
     vcs = [torch.zeros(1, HKV, 64, D, dtype=dtype)]
     tol = 3e-2 if kind == "bf16" else 1e-2
+    elem = 5e-2 if kind == "bf16" else None
     ref, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, HQ, HKV, store_dtype=dtype)
     with torch.no_grad():
         out = lm(input_ids=ids.to(DEV))
-    assert_parity(out.logits, ref, tol, f"{kind} full-shape prefill logits")
+    assert_parity(out.logits, ref, tol, f"{kind} full-shape prefill logits", elementwise=elem)
     cache = out.past_key_values
     nxt = ref[:, -1].argmax(-1)
     for step in range(3):
@@ -104,7 +109,7 @@ def test_full_shape_decoder_layer_vs_oracle(kind):
                                               store_dtype=dtype)
         with torch.no_grad():
             out = lm(input_ids=nxt.unsqueeze(1).to(DEV), past_key_values=cache)
-        assert_parity(out.logits, ref, tol, f"{kind} full-shape decode step {step}")
+        assert_parity(out.logits, ref, tol, f"{kind} full-shape decode step {step}", elementwise=elem)
         nxt = ref[:, -1].argmax(-1)
     # the layer's cache rows equal the oracle's within one 16-bit ulp of rounding flips
     kd = cache.key_cache[0][:, :, :seen].float().cpu()
