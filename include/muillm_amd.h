@@ -40,6 +40,7 @@ extern "C" {
 #define MUI_ERR_LAUNCH (-3)      /* hipGetLastError() after the launch was not hipSuccess */
 #define MUI_ERR_ALIGNMENT (-4)   /* a pointer or row pitch is not 16-byte aligned */
 #define MUI_ERR_DEVICE (-5)      /* device query failed / not a gfx950 device */
+#define MUI_ERR_SCRATCH_LIMIT (-6) /* needs more scratch than the library's built-in array holds */
 
 #define MUI_DTYPE_F16 0
 #define MUI_DTYPE_BF16 1
@@ -231,6 +232,26 @@ int mui_flash_decode(mui_stream_t stream, int dtype, const void* q, const void* 
                      long cache_token_stride, const void* mask, long mask_batch_stride, int seq_len,
                      void* scratch, int n_splits, void* out, int batch, int n_q_heads,
                      int n_kv_heads, int head_dim, int max_cache_len);
+
+/* mui_flash_decode for callers that cannot allocate device memory (code under HIP-graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the
+ * reference, whose flash decoding allocates its partials inside every call
+ * (csrc/attention/flash_decoding.cu:156-158). Same arguments and results as mui_flash_decode
+ * minus `scratch`: the split partials go to an array built into the library
+ * (MUI_FLASH_DECODE_STATIC_SCRATCH_BYTES per GPU, held until the process ends), so the call
+ * performs no allocation of any kind. A shape whose partials
+ * (mui_flash_decode_scratch_bytes(batch, n_q_heads, head_dim, n_splits)) exceed that size is
+ * refused with MUI_ERR_SCRATCH_LIMIT; at batch * n_q_heads * n_splits <= 8065 it fits. All calls
+ * on one GPU share the array: calls that overlap in time on one GPU (different streams) race;
+ * calls on one stream, or serialised by events, are safe. The device that is current at the
+ * call must be the one the pointers belong to. */
+#define MUI_FLASH_DECODE_STATIC_SCRATCH_BYTES (4u << 20)
+size_t mui_flash_decode_static_scratch_limit(void);
+int mui_flash_decode_static(mui_stream_t stream, int dtype, const void* q, const void* k_cache,
+                            const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                            long cache_token_stride, const void* mask, long mask_batch_stride,
+                            int seq_len, int n_splits, void* out, int batch, int n_q_heads,
+                            int n_kv_heads, int head_dim, int max_cache_len);
 
 /* One call for what the reference does in three (muillm_rotary_embedding_module_forward
  * csrc/module.cpp:381 -> RoPE + cache write kernel, then the two flash-decoding kernels,

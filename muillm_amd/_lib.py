@@ -66,6 +66,9 @@ _SIGNATURES = {
     "mui_flash_decode_scratch_bytes": (ctypes.c_size_t, [c_int, c_int, c_int, c_int]),
     "mui_flash_decode": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, _P, c_long, c_int, _P,
                                  c_int, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mui_flash_decode_static_scratch_limit": (ctypes.c_size_t, []),
+    "mui_flash_decode_static": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, _P, c_long, c_int,
+                                        c_int, _P, c_int, c_int, c_int, c_int, c_int]),
     "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, _P,
                                       c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
                                       _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),

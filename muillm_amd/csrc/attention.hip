@@ -28,6 +28,7 @@
 //   slot that is being written.
 //   The sequence length can come from device memory (cache_position[0] + 1), which keeps
 //   the launch shape fixed under HIP-graph replay.
+#include <mutex>
 #include <type_traits>
 
 #include "common.cuh"
@@ -1125,6 +1126,58 @@ extern "C" int mui_flash_decode(mui_stream_t stream, int dtype, const void* q, c
   p.max_t = max_cache_len;
   p.scale_log2 = kLog2e / sqrtf((float)head_dim);
   return launch_attn((hipStream_t)stream, dtype, p, batch);
+}
+
+// ---------------------------------------------------------------------------------------
+// mui_flash_decode for callers that cannot allocate: the split partials live in a file-scope
+// device array. Every GPU the library runs on holds its own copy of it, at its own address,
+// until the process ends.
+// ---------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = MUI_FLASH_DECODE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` per HIP ordinal. In host code the array's name is only a handle
+// for hipGetSymbolAddress, never an address a kernel may use.
+constexpr int kMaxDevices = 64;
+static void* g_static_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_static_scratch_lock;
+
+static int static_scratch_for_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MUI_ERR_DEVICE;
+  std::lock_guard<std::mutex> guard(g_static_scratch_lock);
+  if (!g_static_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return MUI_ERR_DEVICE;
+    g_static_scratch_ptr[dev] = ptr;
+  }
+  *out = g_static_scratch_ptr[dev];
+  return MUI_OK;
+}
+
+extern "C" size_t mui_flash_decode_static_scratch_limit(void) { return kStaticScratchBytes; }
+
+extern "C" int mui_flash_decode_static(mui_stream_t stream, int dtype, const void* q, const void* k_cache,
+                                       const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                       long cache_token_stride, const void* mask, long mask_batch_stride,
+                                       int seq_len, int n_splits, void* out, int batch, int n_q_heads,
+                                       int n_kv_heads, int head_dim, int max_cache_len) {
+  int st = check_attn_shape(dtype, batch, n_q_heads, n_kv_heads, head_dim, n_splits, max_cache_len);
+  if (st != MUI_OK) return st;
+  // partials of (batch, query head, split): beyond the array's size the call is refused, it
+  // never falls back to an allocation
+  if (mui_flash_decode_scratch_bytes(batch, n_q_heads, head_dim, n_splits) > kStaticScratchBytes)
+    return MUI_ERR_SCRATCH_LIMIT;
+  void* ptr = nullptr;
+  if (n_splits > 1) {
+    st = static_scratch_for_current_device(&ptr);
+    if (st != MUI_OK) return st;
+  }
+  // Nothing in the array has to start at zero: every (row, head, split) slot the merge kernel
+  // reads is written by the pass before it, empty splits included.
+  return mui_flash_decode(stream, dtype, q, k_cache, v_cache, cache_batch_stride, cache_head_stride,
+                          cache_token_stride, mask, mask_batch_stride, seq_len, ptr, n_splits, out, batch,
+                          n_q_heads, n_kv_heads, head_dim, max_cache_len);
 }
 
 extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,

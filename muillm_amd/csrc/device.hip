@@ -15,6 +15,7 @@ extern "C" const char* mui_status_string(int status) {
     case MUI_ERR_LAUNCH: return "kernel launch failed";
     case MUI_ERR_ALIGNMENT: return "pointer or row pitch is not 16-byte aligned";
     case MUI_ERR_DEVICE: return "device query failed";
+    case MUI_ERR_SCRATCH_LIMIT: return "shape needs more scratch than the library's built-in array holds";
     default: return "unknown status";
   }
 }
