@@ -245,7 +245,7 @@ def pmc_probe_attention(launches=3):
         for kc, vc in caches:
             _lib.check(lib.mui_attn_decode_fused(
                 stream, 0, qkvx.data_ptr(), qs, qkvx.data_ptr() + 2 * hq * d, qs, qkvx.data_ptr() + 2 * (hq + hkv) * d, qs,
-                cos.data_ptr(), sin.data_ptr(), d // 2, pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
+                cos.data_ptr(), sin.data_ptr(), d // 2, cos.shape[0], pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
                 hkv * S * d, S * d, d, None, 0, None, scratch.data_ptr(), n_splits, o.data_ptr(), B, hq, hkv, d, S),
                 "mui_attn_decode_fused")
         torch.cuda.synchronize()
@@ -394,7 +394,7 @@ def kernel_table(lm):
             kc, vc = caches[i % len(caches)]
             lib.mui_attn_decode_fused(stream, 0, qkvx.data_ptr(), qs, qkvx.data_ptr() + 2 * hq * d, qs,
                                       qkvx.data_ptr() + 2 * (hq + hkv) * d, qs, cos.data_ptr(), sin.data_ptr(), d // 2,
-                                      pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
+                                      cos.shape[0], pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
                                       hkv * S * d, S * d, d, None, 0, None, scratch.data_ptr(), n_splits, o.data_ptr(),
                                       B, hq, hkv, d, S)
         add("C4_rope_cachewrite_flashdecode_ctx%d_batch%d_splits%d" % (S, B, n_splits), att, kvbytes + 4 * B * hq * d, cnt)

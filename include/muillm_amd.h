@@ -30,7 +30,7 @@ extern "C" {
 
 /* bumped whenever a struct below changes layout or an entry point changes its arguments;
  * mui_abi_version() returns the value the library was built with */
-#define MUI_ABI_VERSION 2
+#define MUI_ABI_VERSION 3
 
 /* status codes (reference: TORCH_CHECK exceptions, csrc/linear/linear.cu:72-74;
  * muillm_error_t, csrc/base.h:4-7) */
@@ -181,12 +181,16 @@ int mui_int8_group_dequantize(mui_stream_t stream, int dtype, const void* weight
  * head: 1..8 read K/V once per KV head, other ratios once per query head)
  *
  * Common conventions: q/k/v inputs and the cache have unit inner stride; all other strides
- * are in elements. cos/sin tables are fp32 [max_position, rope_row_stride] with
+ * are in elements. cos/sin tables are fp32 [rope_rows, rope_row_stride] with
  * rope_row_stride >= head_dim/2 and column f (f < head_dim/2) holding cos/sin(pos * inv_freq[f])
  * (the first half of the reference's cos_cached/sin_cached rows,
  * muillm/modules/attention/rotaryembedding.py:313-337); rotation is the HF rotate-half form
  * q' = q*cos + rotate_half(q)*sin in fp32, rounded once. position_ids / cache_position are
- * int64 device arrays like the reference's (csrc/rope/rotary.cu:209-211). The cache is
+ * int64 device arrays like the reference's (csrc/rope/rotary.cu:209-211). Positions are read on
+ * the device, so the table height rope_rows travels with the tables: a position outside
+ * [0, rope_rows) uses the nearest table row instead of reading past the tables (the reference
+ * reads out of bounds, csrc/rope/rotary_fp16_kernels.cu:674-685); callers that can know the
+ * positions on the host should refuse such a request before it gets here. The cache is
  * [batch, n_kv_heads, max_cache_len, head_dim] (muillm/modules/kvcache/cache_utils.py:113-204).
  * ---------------------------------------------------------------------------------- */
 
@@ -204,8 +208,9 @@ int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, long q_batc
                       long q_token_stride, long q_head_stride, const void* k, long k_batch_stride,
                       long k_token_stride, long k_head_stride, const void* v, long v_batch_stride,
                       long v_token_stride, long v_head_stride, const float* cos_table,
-                      const float* sin_table, int rope_row_stride, const int64_t* position_ids,
-                      long position_batch_stride, const int64_t* cache_position, void* q_out,
+                      const float* sin_table, int rope_row_stride, int rope_rows,
+                      const int64_t* position_ids, long position_batch_stride,
+                      const int64_t* cache_position, void* q_out,
                       void* k_out, void* v_out, long out_batch_stride, long out_head_stride,
                       long out_token_stride, int batch, int tokens, int n_q_heads, int n_kv_heads,
                       int head_dim, int max_cache_len);
@@ -264,7 +269,7 @@ int mui_flash_decode_static(mui_stream_t stream, int dtype, const void* q, const
 int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
                           const void* k_new, long k_batch_stride, const void* v_new,
                           long v_batch_stride, const float* cos_table, const float* sin_table,
-                          int rope_row_stride, const int64_t* position_ids,
+                          int rope_row_stride, int rope_rows, const int64_t* position_ids,
                           long position_batch_stride, const int64_t* cache_position, int seq_len,
                           void* k_cache, void* v_cache, long cache_batch_stride,
                           long cache_head_stride, long cache_token_stride, const void* mask,
@@ -369,9 +374,10 @@ typedef struct mui_decoder_stack {
   int dtype, n_layers, hidden, n_q_heads, n_kv_heads, head_dim, intermediate;
   float norm_eps;
   const mui_decoder_layer_t* layers; /* host array of n_layers entries */
-  const float* cos_table;            /* fp32 [positions, rope_row_stride] rotary tables */
+  const float* cos_table;            /* fp32 [rope_rows, rope_row_stride] rotary tables */
   const float* sin_table;
   long rope_row_stride;
+  long rope_rows;
   long cache_batch_stride, cache_head_stride, cache_token_stride; /* elements */
   int max_cache_len;
 } mui_decoder_stack_t;

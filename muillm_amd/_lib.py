@@ -59,7 +59,7 @@ _SIGNATURES = {
     "mui_int8_dequantize": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, c_int, c_int]),
     "mui_int8_group_dequantize": (c_int, [_P, c_int, _P, c_long, _P, c_long, c_int, _P, c_long, c_int, c_int]),
     "mui_rope_kv_write": (c_int, [_P, c_int, _P, c_long, c_long, c_long, _P, c_long, c_long, c_long,
-                                  _P, c_long, c_long, c_long, _P, _P, c_int, _P, c_long, _P, _P, _P, _P,
+                                  _P, c_long, c_long, c_long, _P, _P, c_int, c_int, _P, c_long, _P, _P, _P, _P,
                                   c_long, c_long, c_long, c_int, c_int, c_int, c_int, c_int, c_int]),
     "mui_flash_decode_splits": (c_int, [c_int, c_int, c_int, c_int]),
     "mui_tune_attention": (c_int, [c_int, c_int, c_int, c_int]),
@@ -69,7 +69,7 @@ _SIGNATURES = {
     "mui_flash_decode_static_scratch_limit": (ctypes.c_size_t, []),
     "mui_flash_decode_static": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, _P, c_long, c_int,
                                         c_int, _P, c_int, c_int, c_int, c_int, c_int]),
-    "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, _P,
+    "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, c_int, _P,
                                       c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
                                       _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),
     "mui_prefill_attention": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, c_int, c_int, _P, c_int, c_int,
@@ -105,11 +105,11 @@ class MuiDecoderStackDesc(ctypes.Structure):
     _fields_ = [("dtype", c_int), ("n_layers", c_int), ("hidden", c_int), ("n_q_heads", c_int),
                 ("n_kv_heads", c_int), ("head_dim", c_int), ("intermediate", c_int), ("norm_eps", c_float),
                 ("layers", ctypes.POINTER(MuiDecoderLayerDesc)), ("cos_table", _P), ("sin_table", _P),
-                ("rope_row_stride", c_long), ("cache_batch_stride", c_long), ("cache_head_stride", c_long),
+                ("rope_row_stride", c_long), ("rope_rows", c_long), ("cache_batch_stride", c_long), ("cache_head_stride", c_long),
                 ("cache_token_stride", c_long), ("max_cache_len", c_int)]
 
 
-MUI_ABI_VERSION = 2  # MUI_ABI_VERSION of the public header: layout of the structs above
+MUI_ABI_VERSION = 3  # MUI_ABI_VERSION of the public header: layout of the structs above
 
 _lib: Optional[ctypes.CDLL] = None
 

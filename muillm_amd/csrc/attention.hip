@@ -52,6 +52,7 @@ struct AttnParams {
   const float* cos;       // [max_pos, rope_stride] fp32 tables, or null (no rotation)
   const float* sin;
   int rope_stride;
+  int rope_rows;          // height of the tables: positions are clamped into [0, rope_rows)
   const int64_t* position_ids;  // rotary position of the new token per batch row, or null
   long pos_bs;
   const int64_t* cache_position;  // device scalar: cache slot of the new token
@@ -170,7 +171,8 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   const int slot = has_new ? (int)p.cache_position[0] : -1;
   int S = p.seq_len >= 0 ? p.seq_len : slot + 1;
   S = S < p.max_t ? S : p.max_t;
-  const long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+  long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+  pos = pos < 0 ? 0 : (pos >= p.rope_rows ? p.rope_rows - 1 : pos);  // never index past the tables
 
   constexpr int kBlock = kWorkers * U;  // tokens per workgroup iteration
   int chunk = (S + p.n_splits - 1) / p.n_splits;
@@ -465,7 +467,8 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
   const int slot = has_new ? (int)p.cache_position[0] : -1;
   int S = p.seq_len >= 0 ? p.seq_len : slot + 1;
   S = S < p.max_t ? S : p.max_t;
-  const long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+  long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+  pos = pos < 0 ? 0 : (pos >= p.rope_rows ? p.rope_rows - 1 : pos);  // never index past the tables
 
   int chunk = (S + p.n_splits - 1) / p.n_splits;
   chunk = ((chunk + kBlock - 1) / kBlock) * kBlock;
@@ -905,6 +908,7 @@ struct RopeParams {
   const uint16_t* k; long k_bs, k_ts, k_hs;   // may be null
   const uint16_t* v; long v_bs, v_ts, v_hs;   // may be null
   const float* cos; const float* sin; int rope_stride;  // null: no rotation (plain cache update)
+  int rope_rows;                              // height of the tables (positions are clamped to it)
   const int64_t* position_ids; long pos_bs;   // [B, T] (pos_bs = 0 broadcasts one row)
   const int64_t* cache_position;              // [T] slots; null: k_out/v_out are dense [B, Hkv, T, D]
   uint16_t* q_out;                            // dense [B, Hq, T, D]
@@ -918,7 +922,8 @@ __global__ void __launch_bounds__(kHeadDim) rope_kv_write_kernel(const RopeParam
   const float* cos_row = nullptr;
   const float* sin_row = nullptr;
   if (p.cos) {
-    const long pos = p.position_ids[(long)b * p.pos_bs + tkn];
+    long pos = p.position_ids[(long)b * p.pos_bs + tkn];
+    pos = pos < 0 ? 0 : (pos >= p.rope_rows ? p.rope_rows - 1 : pos);
     cos_row = p.cos + pos * p.rope_stride;
     sin_row = p.sin + pos * p.rope_stride;
   }
@@ -1183,7 +1188,7 @@ extern "C" int mui_flash_decode_static(mui_stream_t stream, int dtype, const voi
 extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
                                      const void* k_new, long k_batch_stride, const void* v_new,
                                      long v_batch_stride, const float* cos_table, const float* sin_table,
-                                     int rope_row_stride, const int64_t* position_ids,
+                                     int rope_row_stride, int rope_rows, const int64_t* position_ids,
                                      long position_batch_stride, const int64_t* cache_position,
                                      int seq_len, void* k_cache, void* v_cache, long cache_batch_stride,
                                      long cache_head_stride, long cache_token_stride, const void* mask,
@@ -1195,7 +1200,7 @@ extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void*
   MUI_CHECK_ARG(q && k_new && v_new && k_cache && v_cache && out && cache_position);
   MUI_CHECK_ARG((cos_table == nullptr) == (sin_table == nullptr));
   MUI_CHECK_ARG(seq_len <= max_cache_len);
-  if (cos_table && rope_row_stride < head_dim / 2) return MUI_ERR_INVALID_ARG;
+  if (cos_table && (rope_row_stride < head_dim / 2 || rope_rows <= 0)) return MUI_ERR_INVALID_ARG;
   if (n_splits > 1 && !scratch) return MUI_ERR_INVALID_ARG;
   if ((cache_token_stride & 7) || (cache_head_stride & 7) || (cache_batch_stride & 7)) return MUI_ERR_ALIGNMENT;
   if (!aligned16(k_cache) || !aligned16(v_cache)) return MUI_ERR_ALIGNMENT;
@@ -1212,6 +1217,7 @@ extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void*
   p.cos = cos_table;
   p.sin = sin_table;
   p.rope_stride = rope_row_stride;
+  p.rope_rows = rope_rows;
   p.position_ids = position_ids;
   p.pos_bs = position_batch_stride;
   p.cache_position = cache_position;
@@ -1240,7 +1246,7 @@ extern "C" int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, 
                                  long k_batch_stride, long k_token_stride, long k_head_stride,
                                  const void* v, long v_batch_stride, long v_token_stride,
                                  long v_head_stride, const float* cos_table, const float* sin_table,
-                                 int rope_row_stride, const int64_t* position_ids,
+                                 int rope_row_stride, int rope_rows, const int64_t* position_ids,
                                  long position_batch_stride, const int64_t* cache_position, void* q_out,
                                  void* k_out, void* v_out, long out_batch_stride, long out_head_stride,
                                  long out_token_stride, int batch, int tokens, int n_q_heads,
@@ -1253,13 +1259,13 @@ extern "C" int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, 
   MUI_CHECK_ARG(!k || k_out);
   MUI_CHECK_ARG(!v || v_out);
   if (head_dim != kHeadDim) return MUI_ERR_UNSUPPORTED;
-  if (cos_table && rope_row_stride < head_dim / 2) return MUI_ERR_INVALID_ARG;
+  if (cos_table && (rope_row_stride < head_dim / 2 || rope_rows <= 0)) return MUI_ERR_INVALID_ARG;
   if (tokens > 65535 || batch > 65535) return MUI_ERR_UNSUPPORTED;
   RopeParams p = {};
   p.q = (const uint16_t*)q; p.q_bs = q_batch_stride; p.q_ts = q_token_stride; p.q_hs = q_head_stride;
   p.k = (const uint16_t*)k; p.k_bs = k_batch_stride; p.k_ts = k_token_stride; p.k_hs = k_head_stride;
   p.v = (const uint16_t*)v; p.v_bs = v_batch_stride; p.v_ts = v_token_stride; p.v_hs = v_head_stride;
-  p.cos = cos_table; p.sin = sin_table; p.rope_stride = rope_row_stride;
+  p.cos = cos_table; p.sin = sin_table; p.rope_stride = rope_row_stride; p.rope_rows = rope_rows;
   p.position_ids = position_ids; p.pos_bs = position_batch_stride;
   p.cache_position = cache_position;
   p.q_out = (uint16_t*)q_out; p.k_out = (uint16_t*)k_out; p.v_out = (uint16_t*)v_out;

@@ -77,7 +77,7 @@ extern "C" int mui_decoder_stack_step(mui_stream_t stream, const mui_decoder_sta
     if (st != MUI_OK) return st;
     const char* q = w.qkv;
     st = mui_attn_decode_fused(stream, m->dtype, q, qkv_n, q + (size_t)qd * 2, qkv_n,
-                               q + (size_t)(qd + kvd) * 2, qkv_n, m->cos_table, m->sin_table, (int)m->rope_row_stride,
+                               q + (size_t)(qd + kvd) * 2, qkv_n, m->cos_table, m->sin_table, (int)m->rope_row_stride, (int)m->rope_rows,
                                position_ids, position_batch_stride, cache_position, seq_len, L.k_cache,
                                L.v_cache, m->cache_batch_stride, m->cache_head_stride, m->cache_token_stride,
                                mask, mask_batch_stride, nullptr, w.scratch, n_splits, w.attn, batch,

@@ -99,7 +99,7 @@ class MuiDecoderStack:
             muillm_ext._dtype_code(first.qkv_proj.linear.norm_weights), len(layers), self.hidden, self.hq, self.hkv,
             self.d, first.mlp.intermediate_size, float(first.qkv_proj.linear.variance_epsilon),
             ctypes.cast(arr, ctypes.POINTER(_lib.MuiDecoderLayerDesc)), self.cos32.data_ptr(), self.sin32.data_ptr(),
-            self.cos32.stride(0), cb, chs, cts, self.max_cache_len)
+            self.cos32.stride(0), self.cos32.shape[0], cb, chs, cts, self.max_cache_len)
         self._ws = None
         self._ws_splits = 0
 

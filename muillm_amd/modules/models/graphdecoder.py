@@ -40,6 +40,7 @@ class MuiGraphDecoder:
         self.eos_token_ids = list(eos_token_ids) if eos_token_ids is not None else None
         self.pad_token_id = int(pad_token_id)
         self.graph = None
+        self._graph_key = None  # what the captured graph has baked in (see _capture_key)
         self.cache: Optional[MuiStaticCache] = None
         self._batch = None
 
@@ -100,6 +101,15 @@ class MuiGraphDecoder:
             lg = lg.masked_fill(drop.scatter(-1, idx, drop), float("-inf"))
         return lg.to(logits.dtype)
 
+    def _capture_key(self):
+        """Everything a captured step holds by address or by value: the cache tensors (re-allocated
+        when the cache grows, which also changes the head stride and the capacity the kernels
+        clamp to), the batch size and whether a padding mask is part of the step."""
+        c = self.cache
+        return (id(c), self._batch, c.max_cache_len, tuple(t.data_ptr() for t in c.key_cache),
+                tuple(t.data_ptr() for t in c.value_cache),
+                None if self.mask4d is None else self.mask4d.data_ptr())
+
     def _capture(self):
         self.cache.device_length_mode = True
         seen = self.cache._seen_tokens
@@ -115,6 +125,7 @@ class MuiGraphDecoder:
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             self.logits = self._step()
+        self._graph_key = self._capture_key()
         # capture does not execute: the device state is as restored; the host counter moved once
         self.cache._seen_tokens = seen
         if self.cache.cpp_module is not None:
@@ -136,16 +147,26 @@ class MuiGraphDecoder:
         lm = self.lm
         device = input_ids.device
         batch, prompt_len = input_ids.shape
-        total = prompt_len + max_new_tokens
+        padded = attention_mask is not None and not bool(torch.all(attention_mask == 1))
+        # a cache that already holds tokens continues after them (multi-turn): slots and rotary
+        # positions are offset by what it has seen
+        past = 0 if cache is None else cache.get_seq_length()
+        if past and padded:
+            raise ValueError("a left-padded prompt needs an empty cache (call cache.reset() first)")
+        total = past + prompt_len + max_new_tokens
+        max_pos = lm.model.rotary_emb.max_seq_len_cached
+        if total > max_pos:
+            raise ValueError(f"cached tokens + prompt + max_new_tokens = {total} exceeds the {max_pos} rotary "
+                             "positions of this model (max_position_embeddings)")
         if cache is None:
             cache = create_static_cache(lm.engine_config, lm.config, batch, total, device, lm.model.mdtype)
-        elif cache.max_cache_len < total:
-            cache.grow_cache(total, max(lm.config.max_position_embeddings, _next_pow2(total)))
-        if self.cache is not cache or self._batch != batch:
-            self.graph = None
+        else:
+            if batch > cache.max_batch_size:
+                raise ValueError(f"batch {batch} exceeds the cache's max_batch_size {cache.max_batch_size}")
+            if cache.max_cache_len < total:
+                cache.grow_cache(total, max(lm.config.max_position_embeddings, _next_pow2(total)))
         self.cache = cache
         cache.device_length_mode = False
-        padded = attention_mask is not None and not bool(torch.all(attention_mask == 1))
         if padded:
             am = attention_mask.to(device=device, dtype=torch.int64)
             if bool((am[:, -1] == 0).any()):
@@ -159,25 +180,24 @@ class MuiGraphDecoder:
         if self._batch != batch or getattr(self, "_max_new", 0) < max_new_tokens:
             self._alloc_state(batch, max_new_tokens, device)
             self.graph = None
-        had_mask = self.mask4d is not None
         if padded:
             mdtype = lm.model.mdtype
             if self.mask4d is None or self.mask4d.shape[-1] != cache.max_cache_len:
                 self.mask4d = torch.zeros((batch, 1, 1, cache.max_cache_len), dtype=mdtype, device=device)
-                self.graph = None
             self.mask4d.zero_()
             self.mask4d[:, 0, 0, :prompt_len].masked_fill_(am == 0, torch.finfo(mdtype).min)
         else:
             self.mask4d = None
-        if had_mask != (self.mask4d is not None):
+        # a captured step is only good for the buffers it was recorded on
+        if self.graph is not None and self._graph_key != self._capture_key():
             self.graph = None
         # the first new token goes through the same kernel as all later ones: the counters start
         # one step back and the launch advances them to (prompt_len, prompt_len, 1)
         if padded:
             self.pos.copy_(am.sum(-1, keepdim=True) - 1)
         else:
-            self.pos.fill_(prompt_len - 1)
-        self.cpos.fill_(prompt_len - 1)
+            self.pos.fill_(past + prompt_len - 1)
+        self.cpos.fill_(past + prompt_len - 1)
         self.step.zero_()
         # columns never reached (early stop) read as padding
         self.out_tokens.fill_(self.pad_token_id if self.eos is not None else 0)

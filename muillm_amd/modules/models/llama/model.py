@@ -1,6 +1,7 @@
 """MuiLlamaModel / MuiLlamaForCausalLM -- the decoder harness around the fused layers
-(muillm/modules/models/llama/model.py:75-873 of the reference; the Mistral file there is a
-rename of the Llama one and is aliased here).
+(muillm/modules/models/llama/model.py:75-873 of the reference; its Mistral file differs in
+feeding config.sliding_window into the mask -- here the Mistral names alias the Llama classes,
+which serve sequences up to the window and refuse longer ones).
 
 Semantics kept from the reference: embed -> N x MuiDecoderLayer -> final MuiRMSNorm ->
 lm_head (MuiLinear) -> fp32 logits; a MuiStaticCache with power-of-two capacity is created
@@ -200,6 +201,19 @@ class MuiLlamaModel(MuiModule):
             past_key_values = None  # foreign cache types are dropped, a static cache is built instead
         past_seen_tokens = past_key_values.get_seq_length() if past_key_values is not None else 0
         tot_seq_len = past_seen_tokens + q_len
+        # the rotary tables have max_position_embeddings rows and the kernels index them with
+        # device-side positions: refuse here what would run past them
+        if tot_seq_len > self.rotary_emb.max_seq_len_cached:
+            raise ValueError(f"{tot_seq_len} tokens exceed the {self.rotary_emb.max_seq_len_cached} rotary positions "
+                             "of this model (max_position_embeddings)")
+        if isinstance(past_key_values, MuiStaticCache) and batch_size > past_key_values.max_batch_size:
+            raise ValueError(f"batch {batch_size} exceeds the cache's max_batch_size {past_key_values.max_batch_size}")
+        # Mistral's sliding-window attention (the reference feeds config.sliding_window into its mask,
+        # muillm/modules/models/mistral/model.py:484,593-602) is not built: inside the window it is
+        # plain causal attention, beyond it this refuses instead of attending to keys it should not
+        window = getattr(self.config, "sliding_window", None)
+        if window and tot_seq_len > int(window):
+            raise NotImplementedError(f"sliding-window attention: {tot_seq_len} tokens exceed sliding_window={window}")
 
         if use_cache:
             if past_key_values is None:
@@ -382,11 +396,29 @@ class MuiLlamaForCausalLM(MuiModule):
 
         use_graph=True captures one decode step (model forward, argmax, position bookkeeping,
         all on the device) into a HIP graph and replays it; False runs the same step eagerly."""
-        from ..graphdecoder import MuiGraphDecoder
-
-        dec = MuiGraphDecoder(self, use_graph=use_graph)
+        dec = self._decoder_for(use_graph=use_graph)
+        cache = self._reusable_cache(dec, cache, input_ids)
         return dec.generate(input_ids, max_new_tokens, cache=cache, return_logits=return_logits)
 
+    def _decoder_for(self, **options):
+        """The MuiGraphDecoder for these options; the last one is kept, so that repeated generate()
+        calls replay the graph captured by the first instead of warming up and capturing again."""
+        from ..graphdecoder import MuiGraphDecoder
+
+        key = tuple(sorted((k, tuple(v) if isinstance(v, (list, tuple)) else v) for k, v in options.items()))
+        if self._graph_decoder is None or self._graph_decoder[0] != key:
+            self._graph_decoder = (key, MuiGraphDecoder(self, **options))
+        return self._graph_decoder[1]
+
+    @staticmethod
+    def _reusable_cache(dec, cache, input_ids):
+        """Without a cache from the caller, a kept decoder starts again on its own (emptied) cache
+        when the batch size fits: same buffers, so its captured graph stays valid."""
+        if cache is None and dec.cache is not None and dec.cache.max_batch_size == input_ids.shape[0] \
+                and dec.cache.key_cache[0].device == input_ids.device:
+            dec.cache.reset()
+            return dec.cache
+        return cache
 
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
@@ -401,8 +433,6 @@ class MuiLlamaForCausalLM(MuiModule):
         Returns int64 [B, prompt_len + max_new_tokens]. top_k / top_p filter the logits with torch
         ops in front of the sampling kernel (the loop then runs eagerly instead of from the HIP
         graph); other logit processors (penalties, ...) are not part of this loop."""
-        from ..graphdecoder import MuiGraphDecoder
-
         dropped = {k: v for k, v in unused.items() if v is not None and k in ("repetition_penalty", "num_beams")}
         if dropped:
             raise NotImplementedError(f"generate(): unsupported options {sorted(dropped)}")
@@ -411,14 +441,16 @@ class MuiLlamaForCausalLM(MuiModule):
             eos = [int(eos_token_id)] if isinstance(eos_token_id, int) else [int(e) for e in eos_token_id]
         if pad_token_id is None:
             pad_token_id = eos[0] if eos else 0
-        dec = MuiGraphDecoder(self, use_graph=use_graph, eos_token_ids=eos, pad_token_id=pad_token_id,
-                              do_sample=do_sample, temperature=temperature, seed=seed,
-                              top_k=top_k if do_sample else None, top_p=top_p if do_sample else None)
+        dec = self._decoder_for(use_graph=use_graph, eos_token_ids=eos, pad_token_id=pad_token_id,
+                                do_sample=do_sample, temperature=temperature, seed=seed,
+                                top_k=top_k if do_sample else None, top_p=top_p if do_sample else None)
+        cache = self._reusable_cache(dec, cache, input_ids)
         # with an eos criterion the loop polls, without blocking, whether every row has finished
         return dec.generate(input_ids, max_new_tokens, cache=cache, attention_mask=attention_mask,
                             stop_check_every=8 if eos else 0)
 
 
-# Mistral shares the Llama implementation (the reference's mistral/model.py is a renamed copy)
+# Mistral shares the Llama implementation up to config.sliding_window tokens (forward() refuses
+# longer sequences: the reference's mistral/model.py:484,593-602 masks keys outside the window)
 MuiMistralModel = MuiLlamaModel
 MuiMistralForCausalLM = MuiLlamaForCausalLM

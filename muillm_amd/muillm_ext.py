@@ -69,6 +69,24 @@ def _num_tokens(x: torch.Tensor) -> int:
     return x.numel() // x.shape[-1]
 
 
+def _check_activations(x: torch.Tensor, k: int, what: str, max_tokens: int, *others) -> None:
+    """What every fused entry point needs of its operands before raw pointers go to a kernel: a
+    16-bit CUDA activation tensor with k features and a token count the kernels take, and every
+    other operand on the same device. The kernels read k values per token: a shorter x would be
+    read out of bounds."""
+    _check_cuda(x, what + " input")
+    if not _is_16bit(x):
+        raise RuntimeError(f"{what}: activations must be fp16 or bf16, got {x.dtype}")
+    if x.dim() < 1 or x.shape[-1] != k:
+        raise RuntimeError(f"{what}: input has {x.shape[-1] if x.dim() else 0} features but the weights expect {k}")
+    tokens = _num_tokens(x)
+    if not 1 <= tokens <= max_tokens:
+        raise RuntimeError(f"{what}: {tokens} tokens, the fused kernels take 1..{max_tokens}")
+    for o in others:
+        if o is not None and (not o.is_cuda or o.device != x.device):
+            raise RuntimeError(f"{what}: every operand must live on the activations' device {x.device}")
+
+
 # Short prompts: up to this many tokens go through the fused kernels in chunks of MUI_MAX_TOKENS
 # (each chunk reads the weights once more, which still beats norm + library GEMM + add for a few
 # chunks: a Llama-3-8B-shaped model prefills 32 tokens in 6.3 ms against 8.4 ms; from a third chunk
@@ -254,6 +272,12 @@ def mui_gateup_silu(norm_weights, epsilon, gate_weights, up_weights, x) -> torch
     pitch = _row_pitch(gate_weights, "gate_weights")
     if _row_pitch(up_weights, "up_weights") != pitch:
         raise RuntimeError("gate and up weights must share one row pitch")
+    _check_activations(x, k, "mui_gateup_silu", max(MUI_MAX_TOKENS, FUSED_CHUNK_MAX_TOKENS), gate_weights,
+                       up_weights, norm_weights)
+    if gate_weights.dtype != x.dtype or up_weights.dtype != x.dtype or \
+            (norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k)):
+        raise RuntimeError("mui_gateup_silu: weights and norm weights must have the activations' dtype "
+                           "(norm weights: one value per input feature)")
     x = x.contiguous()
     tokens = _num_tokens(x)
     h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
@@ -387,6 +411,17 @@ def mui_int8_channel_gateupsilu_forward(norm_weights, epsilon, gate_i8, up_i8, g
     sstride = gate_scales.stride(0) if gate_scales.numel() > 1 else 1
     if (up_scales.stride(0) if up_scales.numel() > 1 else 1) != sstride:
         raise RuntimeError("gate and up scales must share one stride")
+    _check_activations(x, k, "mui_int8_channel_gateupsilu_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS),
+                       gate_i8, up_i8, gate_scales, up_scales, norm_weights)
+    if not int8_kernel_dispatchable(x):
+        raise RuntimeError("mui_int8_channel_gateupsilu_forward: the int8 kernels need k % 16 == 0 "
+                           "(and fp16 activations beyond 16384 features)")
+    if gate_i8.dtype != torch.int8 or up_i8.dtype != torch.int8:
+        raise RuntimeError("per-channel gate/up weights must be int8")
+    if gate_scales.dtype != x.dtype or up_scales.dtype != x.dtype or gate_scales.numel() != n or up_scales.numel() != n:
+        raise RuntimeError("gate/up scales must be one value per row in the activation dtype")
+    if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
+        raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
     x = x.contiguous()
     tokens = _num_tokens(x)
     h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
@@ -433,6 +468,12 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
     if weights.dtype != torch.uint8:
         raise RuntimeError("group-quantised weights must be uint8")
     _check_contiguous(scales_min_vals, "scales_min_vals")
+    _check_activations(x, k, "muillm_int8_linear_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS), weights,
+                       scales_min_vals, norm_weights, add_bias, residual)
+    if scales_min_vals.dtype != x.dtype or scales_min_vals.numel() != 2 * n * (k >> group_size_shift):
+        raise RuntimeError("scales_min_vals must be [N * K / group, 2] (scale, min) pairs in the activation dtype")
+    if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
+        raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
     x = x.contiguous()
     tokens = _num_tokens(x)
     if add_bias is not None and add_bias.numel() == tokens * n and residual is None and tokens > 1:
@@ -464,6 +505,17 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
     if two != 2:
         raise RuntimeError("gate_up_weights must be [N, 2, K]")
     g = k >> group_size_shift
+    _check_activations(x, k, "muillm_int8_gateupsilu_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS),
+                       gate_up_weights, gate_up_scales_min_vals, norm_weights)
+    if not int8_kernel_dispatchable(x) or group_size_shift < 4:
+        raise RuntimeError("muillm_int8_gateupsilu_forward: the int8 kernels need k % 16 == 0 and groups of >= 16")
+    if gate_up_weights.dtype != torch.uint8 or not gate_up_weights.is_contiguous():
+        raise RuntimeError("gate_up_weights must be a contiguous uint8 tensor")
+    if gate_up_scales_min_vals.dtype != x.dtype or gate_up_scales_min_vals.numel() != n * 2 * g * 2 \
+            or not gate_up_scales_min_vals.is_contiguous():
+        raise RuntimeError("gate_up_scales_min_vals must hold N * 2 * K / group (scale, min) pairs in the activation dtype")
+    if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
+        raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
     smv = gate_up_scales_min_vals.reshape(n, 2, g, 2)
     x = x.contiguous()
     tokens = _num_tokens(x)
@@ -552,6 +604,8 @@ def mui_rope_kv_write(q, k, v, cos, sin, position_ids, cache_position, k_out, v_
         if out_ref.dim() != 4 or out_ref.stride(3) != 1:
             raise RuntimeError("k/v outputs must be [B, H, T, D] with unit inner stride")
         ob, oh, ot = out_ref.stride(0), out_ref.stride(1), out_ref.stride(2)
+        if b > out_ref.shape[0]:
+            raise RuntimeError(f"batch {b} exceeds the batch capacity {out_ref.shape[0]} of the k/v outputs")
         if k_out is not None and v_out is not None and k_out.stride() != v_out.stride():
             raise RuntimeError("k and v outputs must share strides")
     else:
@@ -563,6 +617,7 @@ def mui_rope_kv_write(q, k, v, cos, sin, position_ids, cache_position, k_out, v_
             _stream(ref_t), _dtype_code(ref_t),
             _ptr(q), qs[0], qs[1], qs[2], _ptr(k), ks[0], ks[1], ks[2], _ptr(v), vs[0], vs[1], vs[2],
             _ptr(cos32), _ptr(sin32), cos32.stride(0) if cos32 is not None else 0,
+            cos32.shape[0] if cos32 is not None else 0,
             _ptr(pos), pos_bs, _ptr(cache_position), _ptr(q_out), _ptr(k_out), _ptr(v_out), ob, oh, ot,
             b, t, hq, hkv, d, int(max_cache_len)),
         "mui_rope_kv_write",
@@ -753,6 +808,8 @@ def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_positi
     the split count then comes from seq_len_hint (default: cache capacity)."""
     lib = _lib.load()
     b = q.shape[0]
+    if b > k_cache.shape[0] or b > v_cache.shape[0]:
+        raise RuntimeError(f"batch {b} exceeds the cache's batch capacity {k_cache.shape[0]}")
     q2, k2, v2 = q.reshape(b, -1), k.reshape(b, -1), v.reshape(b, -1)
     for name, tns in (("q", q2), ("k", k2), ("v", v2)):
         _check_cuda(tns, name)
@@ -782,6 +839,7 @@ def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_positi
         lib.mui_attn_decode_fused(
             _stream(q2), _dtype_code(q2), q2.data_ptr(), bs(q2), k2.data_ptr(), bs(k2), v2.data_ptr(), bs(v2),
             _ptr(cos32), _ptr(sin32), cos32.stride(0) if cos32 is not None else 0,
+            cos32.shape[0] if cos32 is not None else 0,
             pos.data_ptr(), pos_bs, cache_position.data_ptr(), -1 if seq_len is None else int(seq_len),
             k_cache.data_ptr(), v_cache.data_ptr(), cb, chs, cts, mask_ptr, mask_bs, _ptr(q_out),
             _ptr(scratch), n_splits, out.data_ptr(), b, hq, hkv, d, max_t),

@@ -48,7 +48,7 @@ def test_product_header_holds_no_process_global_knobs():
 
 def test_status_strings_and_version():
     lib = _lib.load()
-    assert lib.mui_abi_version() == _lib.MUI_ABI_VERSION == 2
+    assert lib.mui_abi_version() == _lib.MUI_ABI_VERSION == 3
     assert _lib.status_string(0) == "ok"
     for code in (-1, -2, -3, -4, -5):
         assert _lib.status_string(code) not in ("ok", "unknown status")

@@ -393,3 +393,53 @@ def test_attention_abi_errors():
     assert lib.mui_flash_decode_scratch_bytes(2, 32, 128, 4) == 2 * 32 * 4 * 130 * 4
     with pytest.raises(RuntimeError):
         muillm_ext.muillm_causal_transformer_decoding_no_mask(torch.zeros(1, 32, 2, 128, dtype=torch.float16, device=DEV), kc, kc)
+
+
+def test_rope_positions_outside_the_tables_and_batch_capacity():
+    """Positions are read on the device, so the kernels get the table height: a position beyond
+    the tables uses the last row instead of reading past it; a batch larger than the cache is
+    refused by the wrappers; a table height of zero by the C ABI."""
+    lib = _lib.load()
+    g = _gen(12)
+    rows = 64
+    cos, sin = oracle.rope_tables(500000.0, D, rows)
+    q, k = _mk((1, 4, 1, D), g).to(DEV), _mk((1, 1, 1, D), g).to(DEV)
+    last = torch.full((1, 1), rows - 1, dtype=torch.int64, device=DEV)
+    beyond = torch.full((1, 1), rows + 1000, dtype=torch.int64, device=DEV)
+    negative = torch.full((1, 1), -5, dtype=torch.int64, device=DEV)
+    zero = torch.zeros((1, 1), dtype=torch.int64, device=DEV)
+    q_last, k_last = muillm_ext.muillm_rope_forward_no_cache(last, cos.to(DEV), sin.to(DEV), q, k)
+    q_far, k_far = muillm_ext.muillm_rope_forward_no_cache(beyond, cos.to(DEV), sin.to(DEV), q, k)
+    q_neg, _ = muillm_ext.muillm_rope_forward_no_cache(negative, cos.to(DEV), sin.to(DEV), q, k)
+    q_zero, _ = muillm_ext.muillm_rope_forward_no_cache(zero, cos.to(DEV), sin.to(DEV), q, k)
+    assert torch.equal(q_far, q_last) and torch.equal(k_far, k_last) and torch.equal(q_neg, q_zero)
+    # fused decode entry: same clamp
+    kc = torch.zeros(1, 1, 16, D, dtype=torch.float16, device=DEV)
+    vc = torch.zeros_like(kc)
+    cpos = torch.zeros(1, dtype=torch.int64, device=DEV)
+    qkv = _mk((1, 6 * D), g).to(DEV)
+    outs = []
+    for pos in (last, beyond):
+        kc.zero_(); vc.zero_()
+        outs.append((muillm_ext.mui_attention_decode_fused(qkv[:, : 4 * D], qkv[:, 4 * D : 5 * D], qkv[:, 5 * D :],
+                                                           cos.to(DEV), sin.to(DEV), pos, cpos, kc, vc, seq_len=1),
+                     kc.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    # wrappers refuse a batch the cache cannot hold
+    qkv2 = _mk((2, 6 * D), g).to(DEV)
+    with pytest.raises(RuntimeError, match="batch"):
+        muillm_ext.mui_attention_decode_fused(qkv2[:, : 4 * D], qkv2[:, 4 * D : 5 * D], qkv2[:, 5 * D :], cos.to(DEV),
+                                              sin.to(DEV), torch.zeros(2, 1, dtype=torch.int64, device=DEV), cpos,
+                                              kc, vc, seq_len=1)
+    with pytest.raises(RuntimeError, match="batch"):
+        muillm_ext.muillm_static_kvcache_update(kc, vc, _mk((2, 1, 1, D), g).to(DEV), _mk((2, 1, 1, D), g).to(DEV),
+                                                cpos, 1)
+    # C ABI: tables without a height are an invalid argument
+    s = torch.cuda.current_stream().cuda_stream
+    c32, s32 = cos.to(DEV), sin.to(DEV)
+    out = torch.zeros(1, 4 * D, dtype=torch.float16, device=DEV)
+    st = lib.mui_attn_decode_fused(s, 0, qkv.data_ptr(), 6 * D, qkv.data_ptr() + 8 * D, 6 * D, qkv.data_ptr() + 10 * D,
+                                   6 * D, c32.data_ptr(), s32.data_ptr(), D // 2, 0, zero.data_ptr(), 1, cpos.data_ptr(),
+                                   1, kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1), kc.stride(2), None, 0,
+                                   None, None, 1, out.data_ptr(), 1, 4, 1, D, 16)
+    assert st == -1

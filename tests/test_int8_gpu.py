@@ -226,3 +226,38 @@ def test_channel_linear_and_gateup_in_chunks(tokens):
     ref_h = oracle.gateup_silu(x, oracle.rtn_dequantize_channel(qg, sg), oracle.rtn_dequantize_channel(qu, su), gamma, 1e-5)
     assert_parity(h, ref_h, 1e-2, f"int8 gate/up chunks {tokens}")
     assert not muillm_ext.int8_kernel_dispatchable(torch.zeros(65, k, dtype=torch.float16, device=DEV))
+
+
+def test_wrappers_refuse_mismatched_operands():
+    """The drop-in entry points hand raw pointers to the kernels: a short activation row, a CPU
+    tensor, scales in another 16-bit type or too many tokens are refused with RuntimeError."""
+    g = _gen(41)
+    n, k = 64, 256
+    q, s = oracle.rtn_quantize_channel(_mk((n, k), g, 0.02))
+    qd, sd = q.to(DEV), s.to(DEV)
+    x = _mk((1, k), g).to(DEV)
+    with pytest.raises(RuntimeError, match="features"):
+        muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd, sd, x[:, : k - 16])
+    with pytest.raises(RuntimeError, match="CUDA"):
+        muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd, sd, x.cpu())
+    with pytest.raises(RuntimeError, match="dtype"):
+        muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd.bfloat16(), sd.bfloat16(), x)
+    with pytest.raises(RuntimeError, match="tokens"):
+        muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd, sd, _mk((100, k), g).to(DEV))
+    qu, smv = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), 128)
+    qu, smv = qu.to(DEV), smv.to(DEV)
+    with pytest.raises(RuntimeError, match="dtype"):
+        muillm_ext.muillm_int8_linear_forward(x.bfloat16(), qu, smv, 7)        # bf16 activations, fp16 (scale, min)
+    packed = torch.stack([qu, qu], dim=1).contiguous()
+    psmv = torch.stack([smv.reshape(n, -1, 2)] * 2, dim=1).contiguous()
+    with pytest.raises(RuntimeError, match="features"):
+        muillm_ext.muillm_int8_gateupsilu_forward(None, 0.0, packed, psmv, 7, x[:, : k - 16])
+    with pytest.raises(RuntimeError, match="tokens"):
+        muillm_ext.muillm_int8_gateupsilu_forward(None, 0.0, packed, psmv, 7, _mk((100, k), g).to(DEV))
+    w = _mk((n, k), g, 0.02).to(DEV)
+    with pytest.raises(RuntimeError, match="features"):
+        muillm_ext.mui_gateup_silu(None, 0.0, w, w, x[:, : k - 8])
+    with pytest.raises(RuntimeError, match="dtype"):
+        muillm_ext.mui_gateup_silu(None, 0.0, w, w, x.bfloat16())
+    with pytest.raises(RuntimeError, match="CUDA"):
+        muillm_ext.muillm_gateupsilu_forward(None, None, 0.0, w, w, w[:k, :n] if False else w, None, x.cpu())

@@ -292,3 +292,76 @@ def test_replace_layers_leaves_unknown_modules(ctx):
     m = Odd()
     out = replace_layers(m, MuiReplacementContext(ctx.engine_config, m, "cpu"))
     assert isinstance(out.lin, MuiLinear) and isinstance(out.act, nn.GELU) and type(out.keep) is nn.Linear
+
+
+# ------------------------------------------------------------------------------------
+# guards of the decode loop (host logic; nothing here provokes an out-of-range read)
+# ------------------------------------------------------------------------------------
+def _tiny_lm(max_pos=32, **extra):
+    cfg = MuiDecoderConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                           num_key_value_heads=1, vocab_size=64, max_position_embeddings=max_pos)
+    for k, v in extra.items():
+        setattr(cfg, k, v)
+    return MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float32, device="cpu", seed=0,
+                                           init_std=0.05)
+
+
+def test_forward_refuses_positions_beyond_the_rotary_tables():
+    lm = _tiny_lm(max_pos=32)
+    ids = torch.randint(0, 64, (1, 30))
+    with torch.no_grad():
+        out = lm(input_ids=ids)
+        lm(input_ids=ids[:, :2], past_key_values=out.past_key_values)      # 32 tokens: the last table row
+        with pytest.raises(ValueError, match="rotary positions"):
+            lm(input_ids=ids[:, :1], past_key_values=out.past_key_values)  # 33rd token
+        with pytest.raises(ValueError, match="rotary positions"):
+            lm(input_ids=torch.randint(0, 64, (1, 33)))
+
+
+def test_forward_refuses_a_batch_larger_than_the_cache():
+    lm = _tiny_lm()
+    cache = create_static_cache(MuiEngineConfig(), lm.config, max_batch_size=1, seq_len=16, device="cpu",
+                                dtype=torch.float32)
+    with torch.no_grad(), pytest.raises(ValueError, match="max_batch_size"):
+        lm(input_ids=torch.randint(0, 64, (2, 4)), past_key_values=cache)
+
+
+def test_sliding_window_is_refused_beyond_the_window():
+    lm = _tiny_lm(max_pos=64, sliding_window=8)
+    with torch.no_grad():
+        out = lm(input_ids=torch.randint(0, 64, (1, 8)))                    # inside the window: plain causal
+        with pytest.raises(NotImplementedError, match="sliding"):
+            lm(input_ids=torch.randint(0, 64, (1, 1)), past_key_values=out.past_key_values)
+
+
+def test_graph_decoder_prefill_guards_and_capture_key():
+    """MuiGraphDecoder.prefill refuses, before any kernel runs, what the rotary tables or the cache
+    cannot hold; the key of a captured step changes when the cache is re-allocated. (The decode
+    loop itself needs the GPU kernels: its continuation test lives in test_modules_gpu.py.)"""
+    from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
+
+    lm = _tiny_lm(max_pos=64)
+    dec = MuiGraphDecoder(lm, use_graph=False)
+    ids = torch.randint(0, 64, (1, 6))
+    with pytest.raises(ValueError, match="rotary positions"):
+        dec.prefill(ids, 60)
+    cache = create_static_cache(MuiEngineConfig(), lm.config, max_batch_size=1, seq_len=8, device="cpu",
+                                dtype=torch.float32)
+    with pytest.raises(ValueError, match="max_batch_size"):
+        dec.prefill(torch.randint(0, 64, (2, 6)), 4, cache=cache)
+    with torch.no_grad():
+        lm(input_ids=ids, past_key_values=cache)                            # the cache now holds 6 tokens
+    with pytest.raises(ValueError, match="rotary positions"):
+        dec.prefill(ids, 53, cache=cache)                                   # 6 + 6 + 53 > 64
+    with pytest.raises(ValueError, match="empty cache"):
+        dec.prefill(ids, 2, cache=cache, attention_mask=torch.tensor([[0, 1, 1, 1, 1, 1]]))
+    dec.cache, dec._batch, dec.mask4d = cache, 1, None
+    before = dec._capture_key()
+    assert dec._capture_key() == before
+    cache.grow_cache(20, 64)                                                # 8 -> 32 slots: new tensors
+    after = dec._capture_key()
+    assert after != before, "a re-allocated cache must invalidate a captured step"
+    dec.mask4d = torch.zeros(1, 1, 1, 32)
+    assert dec._capture_key() != after                                      # a padding mask is part of the step
+    dec._batch = 2
+    assert dec._capture_key()[1] == 2

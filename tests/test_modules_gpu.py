@@ -246,6 +246,57 @@ def test_graph_decode_matches_eager(batch):
     assert dec.cache.get_seq_length() == 32 + n_new - 1
 
 
+def test_graph_decoder_reuse_after_cache_growth_and_multi_turn():
+    """One decoder object, one cache object, a second generation that needs a larger cache: the
+    cache tensors are re-allocated, so the captured step must be recorded again (a stale graph
+    would read the old tensors). And a cache that already holds a first turn is continued, not
+    overwritten: two turns == one generation over the concatenated prompt."""
+    cfg = _small_config(layers=2)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=4,
+                                         init_std=0.05)
+    g = torch.Generator().manual_seed(5)
+    short = torch.randint(0, cfg.vocab_size, (1, 8), generator=g).to(DEV)
+    long_p = torch.randint(0, cfg.vocab_size, (1, 40), generator=g).to(DEV)
+    dec = MuiGraphDecoder(lm, use_graph=True)
+    first = dec.generate(short, 8)                          # capacity 16
+    cache = dec.cache
+    ptr = cache.key_cache[0].data_ptr()
+    graph = dec.graph
+    assert graph is not None
+    cache.reset()
+    second = dec.generate(long_p, 8, cache=cache)           # needs 48 slots: grows to 64, new tensors
+    assert cache.key_cache[0].data_ptr() != ptr and cache.get_max_length() == 64
+    assert dec.graph is not graph, "the graph captured on the old cache tensors was replayed"
+    assert torch.equal(second, lm.generate_greedy(long_p, 8, use_graph=False))
+    assert torch.equal(first, lm.generate_greedy(short, 8, use_graph=False))
+    # same buffers again: the captured step is kept
+    graph = dec.graph
+    cache.reset()
+    third = dec.generate(short, 8, cache=cache)
+    assert dec.graph is graph and torch.equal(third, first)
+    # multi-turn: the second prompt continues after the 8 + 8 - 1 tokens the cache holds
+    turn2 = dec.generate(short, 6, cache=cache)
+    assert cache.get_seq_length() == 15 + 8 + 6 - 1 and int(dec.cpos) == 15 + 8 + 6 - 1
+    eager = MuiGraphDecoder(lm, use_graph=False)
+    eager.generate(short, 8)                                # the same first turn, eagerly
+    c2 = eager.cache
+    with torch.no_grad():
+        out = lm(input_ids=short, past_key_values=c2)       # second turn through plain forward calls
+        toks = [out.logits[:, -1].argmax(-1)]
+        for _ in range(5):
+            out = lm(input_ids=toks[-1].unsqueeze(1), past_key_values=c2)
+            toks.append(out.logits[:, -1].argmax(-1))
+    assert torch.equal(turn2[:, 8:], torch.stack(toks, dim=1))
+    # generate() keeps its decoder: the second call replays the first call's graph
+    lm.generate(short, max_new_tokens=8)
+    kept = lm._graph_decoder[1]
+    g0 = kept.graph
+    out = lm.generate(short, max_new_tokens=8)
+    assert lm._graph_decoder[1] is kept and kept.graph is g0 and torch.equal(out, first)
+    with pytest.raises(ValueError, match="rotary positions"):
+        lm.generate(long_p, max_new_tokens=cfg.max_position_embeddings)
+
+
 @pytest.mark.parametrize("batch", [1, 3])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_decoder_stack_call_matches_layer_modules(batch, dtype):
