@@ -163,6 +163,18 @@ int mui_int8_group_gateup_silu(mui_stream_t stream, int dtype, const void* gate_
                                const void* x, const void* norm_weights, float epsilon, void* h,
                                int n_inter, int k_in, int tokens);
 
+/* The reference packs gate and up per element: gate_up_weights uint8 [n_inter, k_in, 2] and
+ * gate_up_scales_min_vals 16-bit [n_inter * G, 2, 2] (group, gate|up, scale|min)
+ * (muillm/modules/quantized/int8gateupdownmlp.py:211-230; read that way by
+ * csrc/int8_gateup_kernels.cu:255-296). The kernels here stream row-interleaved buffers,
+ * [n_inter, 2, k_in] and [n_inter, 2, G, 2]. This call converts the first form into the second,
+ * once per weight (out of place; smv_* may both be NULL to convert only the codes), so that
+ * tensors made by the reference's Python classes can be handed to mui_int8_group_gateup_silu /
+ * mui_int8_group_dequantize. k_in % 16 == 0, group size >= 16. */
+int mui_int8_repack_gateup(mui_stream_t stream, const void* gate_up_nk2, const void* smv_ng22,
+                           int group_size_shift, void* gate_up_n2k, void* smv_n2g2, int n_inter,
+                           int k_in);
+
 /* Dense dequantisation of the per-channel format (the non-single-token branch of
  * muillm/modules/quantized/int8linear.py:279-293): out[n, k] = T(float(q[n,k]) * float(s[n])),
  * bit-identical to torch's q.to(T) * s[:, None]. scale of row n at scales[n * scale_stride]. */
@@ -341,9 +353,9 @@ int mui_sample_advance(mui_stream_t stream, int dtype, const void* logits, long 
  * Per layer: qkv = Wqkv rmsnorm(h); attn = flash decoding with RoPE and cache write
  * (mui_attn_decode_fused); h' = Wo attn + h; mid = silu(Wg n) * (Wu n) with n = rmsnorm(h');
  * out = Wd mid + h'. Activations, norms, caches and 16-bit weights are device memory of the
- * 16-bit type `dtype`; any projection may instead hold int8 weights with per-channel scales
- * (muillm/modules/quantized/int8linear.py, int8gateupdownmlp.py in the reference). The caller
- * owns everything. */
+ * 16-bit type `dtype`; any projection may instead hold int8 weights, with per-channel scales or
+ * in the reference's group-wise (scale, min) format (muillm/modules/quantized/int8linear.py,
+ * int8gateupdownmlp.py, muillm/quantization/rtnquantizer.py:49-88). The caller owns everything. */
 typedef struct mui_decoder_layer {
   const void* input_norm;   /* [hidden] gamma of the RMSNorm fused into the QKV projection */
   const void* qkv_weight;   /* [(Hq + 2 Hkv) * D, hidden], rows q | k | v */
@@ -368,6 +380,13 @@ typedef struct mui_decoder_layer {
   const void* up_scales;
   long gateup_scale_stride;
   const void* down_scales;  /* [hidden] */
+  /* 0: the *_scales above are per-channel scales. s >= 4: the int8 projections of this layer are in
+   * the reference's group format instead (muillm/quantization/rtnquantizer.py:49-88; the
+   * mui_int8_group_linear / mui_int8_group_gateup_silu format): uint8 codes, groups of 2^s inputs,
+   * and every non-NULL *_scales pointer addresses 16-bit (scale, min) pairs, [rows * G, 2] with
+   * G = inputs >> s; for gate and up the pairs of row n start at gate_scales / up_scales +
+   * n * gateup_scale_stride elements. */
+  int int8_group_size_shift;
 } mui_decoder_layer_t;
 
 typedef struct mui_decoder_stack {

@@ -56,6 +56,7 @@ _SIGNATURES = {
     "mui_int8_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
     "mui_int8_group_linear": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, _P, c_float, _P, _P, _P, c_int, c_int, c_int]),
     "mui_int8_group_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_long, c_int, _P, _P, c_float, _P, c_int, c_int, c_int]),
+    "mui_int8_repack_gateup": (c_int, [_P, _P, _P, c_int, _P, _P, c_int, c_int]),
     "mui_int8_dequantize": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, c_int, c_int]),
     "mui_int8_group_dequantize": (c_int, [_P, c_int, _P, c_long, _P, c_long, c_int, _P, c_long, c_int, c_int]),
     "mui_rope_kv_write": (c_int, [_P, c_int, _P, c_long, c_long, c_long, _P, c_long, c_long, c_long,
@@ -97,7 +98,7 @@ class MuiDecoderLayerDesc(ctypes.Structure):
                 ("o_pitch", c_long), ("post_norm", _P), ("gate_weight", _P), ("up_weight", _P),
                 ("gateup_pitch", c_long), ("down_weight", _P), ("down_pitch", c_long), ("k_cache", _P),
                 ("v_cache", _P), ("qkv_scales", _P), ("o_scales", _P), ("gate_scales", _P), ("up_scales", _P),
-                ("gateup_scale_stride", c_long), ("down_scales", _P)]
+                ("gateup_scale_stride", c_long), ("down_scales", _P), ("int8_group_size_shift", c_int)]
 
 
 class MuiDecoderStackDesc(ctypes.Structure):

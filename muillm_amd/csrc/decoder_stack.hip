@@ -7,8 +7,9 @@
 // goes through its Python modules (muillm/modules/decoder/decoder.py:130-165). Here the same
 // order is enqueued by one C call, which removes the per-launch host work of an interpreter
 // loop (about 160 launches per token) when the step is not replayed from a HIP graph. Each
-// projection takes 16-bit weights or int8 codes with per-channel scales
-// (muillm/modules/quantized/int8linear.py:279-293, int8gateupdownmlp.py in the reference).
+// projection takes 16-bit weights or int8 codes, the latter with per-channel scales or in the
+// reference's group-wise (scale, min) format (muillm/modules/quantized/int8linear.py:279-293,
+// int8gateupdownmlp.py, muillm/quantization/rtnquantizer.py:49-88).
 #include "common.cuh"
 
 using namespace mui;
@@ -69,11 +70,16 @@ extern "C" int mui_decoder_stack_step(mui_stream_t stream, const mui_decoder_sta
   for (int l = 0; l < m->n_layers; ++l) {
     const mui_decoder_layer_t& L = m->layers[l];
     char* out = (l + 1 == m->n_layers) ? (char*)hidden_out : w.h_b;
-    int st = L.qkv_scales
-                 ? mui_int8_linear(stream, m->dtype, L.qkv_weight, L.qkv_pitch, L.qkv_scales, h, L.input_norm,
-                                   m->norm_eps, nullptr, nullptr, w.qkv, qkv_n, m->hidden, batch)
-                 : mui_linear(stream, m->dtype, L.qkv_weight, L.qkv_pitch, h, L.input_norm, m->norm_eps, nullptr,
-                              nullptr, nullptr, w.qkv, qkv_n, m->hidden, batch);
+    const int gs = L.int8_group_size_shift;  // 0: per-channel scales; else the reference's group format
+    if (gs < 0) return MUI_ERR_INVALID_ARG;
+    int st = !L.qkv_scales
+                 ? mui_linear(stream, m->dtype, L.qkv_weight, L.qkv_pitch, h, L.input_norm, m->norm_eps, nullptr,
+                              nullptr, nullptr, w.qkv, qkv_n, m->hidden, batch)
+             : gs ? mui_int8_group_linear(stream, m->dtype, L.qkv_weight, L.qkv_pitch, L.qkv_scales, gs, h,
+                                          L.input_norm, m->norm_eps, nullptr, nullptr, w.qkv, qkv_n, m->hidden,
+                                          batch)
+                  : mui_int8_linear(stream, m->dtype, L.qkv_weight, L.qkv_pitch, L.qkv_scales, h, L.input_norm,
+                                    m->norm_eps, nullptr, nullptr, w.qkv, qkv_n, m->hidden, batch);
     if (st != MUI_OK) return st;
     const char* q = w.qkv;
     st = mui_attn_decode_fused(stream, m->dtype, q, qkv_n, q + (size_t)qd * 2, qkv_n,
@@ -83,23 +89,30 @@ extern "C" int mui_decoder_stack_step(mui_stream_t stream, const mui_decoder_sta
                                mask, mask_batch_stride, nullptr, w.scratch, n_splits, w.attn, batch,
                                m->n_q_heads, m->n_kv_heads, m->head_dim, m->max_cache_len);
     if (st != MUI_OK) return st;
-    st = L.o_scales ? mui_int8_linear(stream, m->dtype, L.o_weight, L.o_pitch, L.o_scales, w.attn, nullptr, 0.f,
+    st = !L.o_scales ? mui_linear(stream, m->dtype, L.o_weight, L.o_pitch, w.attn, nullptr, 0.f, nullptr, nullptr, h,
+                                  w.h_a, m->hidden, qd, batch)
+         : gs ? mui_int8_group_linear(stream, m->dtype, L.o_weight, L.o_pitch, L.o_scales, gs, w.attn, nullptr, 0.f,
                                       nullptr, h, w.h_a, m->hidden, qd, batch)
-                    : mui_linear(stream, m->dtype, L.o_weight, L.o_pitch, w.attn, nullptr, 0.f, nullptr, nullptr, h,
-                                 w.h_a, m->hidden, qd, batch);
+              : mui_int8_linear(stream, m->dtype, L.o_weight, L.o_pitch, L.o_scales, w.attn, nullptr, 0.f, nullptr, h,
+                                w.h_a, m->hidden, qd, batch);
     if (st != MUI_OK) return st;
     if ((L.gate_scales == nullptr) != (L.up_scales == nullptr)) return MUI_ERR_INVALID_ARG;
-    st = L.gate_scales
-             ? mui_int8_gateup_silu(stream, m->dtype, L.gate_weight, L.up_weight, L.gateup_pitch, L.gate_scales,
-                                    L.up_scales, L.gateup_scale_stride, w.h_a, L.post_norm, m->norm_eps, w.mid,
-                                    m->intermediate, m->hidden, batch)
-             : mui_gateup_silu(stream, m->dtype, L.gate_weight, L.up_weight, L.gateup_pitch, w.h_a, L.post_norm,
-                               m->norm_eps, w.mid, m->intermediate, m->hidden, batch);
+    st = !L.gate_scales
+             ? mui_gateup_silu(stream, m->dtype, L.gate_weight, L.up_weight, L.gateup_pitch, w.h_a, L.post_norm,
+                               m->norm_eps, w.mid, m->intermediate, m->hidden, batch)
+         : gs ? mui_int8_group_gateup_silu(stream, m->dtype, L.gate_weight, L.up_weight, L.gateup_pitch,
+                                           L.gate_scales, L.up_scales, L.gateup_scale_stride, gs, w.h_a,
+                                           L.post_norm, m->norm_eps, w.mid, m->intermediate, m->hidden, batch)
+              : mui_int8_gateup_silu(stream, m->dtype, L.gate_weight, L.up_weight, L.gateup_pitch, L.gate_scales,
+                                     L.up_scales, L.gateup_scale_stride, w.h_a, L.post_norm, m->norm_eps, w.mid,
+                                     m->intermediate, m->hidden, batch);
     if (st != MUI_OK) return st;
-    st = L.down_scales ? mui_int8_linear(stream, m->dtype, L.down_weight, L.down_pitch, L.down_scales, w.mid,
-                                         nullptr, 0.f, nullptr, w.h_a, out, m->hidden, m->intermediate, batch)
-                       : mui_linear(stream, m->dtype, L.down_weight, L.down_pitch, w.mid, nullptr, 0.f, nullptr,
-                                    nullptr, w.h_a, out, m->hidden, m->intermediate, batch);
+    st = !L.down_scales ? mui_linear(stream, m->dtype, L.down_weight, L.down_pitch, w.mid, nullptr, 0.f, nullptr,
+                                     nullptr, w.h_a, out, m->hidden, m->intermediate, batch)
+         : gs ? mui_int8_group_linear(stream, m->dtype, L.down_weight, L.down_pitch, L.down_scales, gs, w.mid,
+                                      nullptr, 0.f, nullptr, w.h_a, out, m->hidden, m->intermediate, batch)
+              : mui_int8_linear(stream, m->dtype, L.down_weight, L.down_pitch, L.down_scales, w.mid, nullptr, 0.f,
+                                nullptr, w.h_a, out, m->hidden, m->intermediate, batch);
     if (st != MUI_OK) return st;
     h = out;
   }

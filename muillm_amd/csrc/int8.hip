@@ -571,3 +571,67 @@ extern "C" int mui_int8_group_dequantize(mui_stream_t stream, int dtype, const v
     return MUI_ERR_INVALID_ARG;
   return launch_status();
 }
+
+// ---------------------------------------------------------------------------------------
+// One-time conversion of the reference's packed gate/up format into the row-interleaved one the
+// kernels stream: weights [N, K, 2] (gate and up of one input feature adjacent,
+// muillm/modules/quantized/int8gateupdownmlp.py:211-230) -> [N, 2, K]; (scale, min) pairs
+// [N * G, 2, 2] (group, gate|up, scale|min) -> [N, 2, G, 2]. One thread moves 16 input bytes
+// (8 gate + 8 up codes); the first N * G * 2 threads also move one (scale, min) pair each.
+// ---------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) int8_repack_gateup_kernel(const uint8_t* in, const uint32_t* smv_in,
+                                                                 uint8_t* out, uint32_t* smv_out, int n, int k,
+                                                                 int groups) {
+  const long total = (long)n * (k >> 3);  // 16-byte input chunks
+  const long pairs = (long)n * groups * 2;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long row = idx / (k >> 3);
+    const int c = (int)(idx - row * (k >> 3));  // covers input features 8c .. 8c+7
+    const u32x4 v = *(const u32x4*)(in + row * 2L * k + ((long)c << 4));
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t g[2], u[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      // dword = (g0, u0, g1, u1): even bytes are gate codes, odd bytes up codes
+      g[h] = __builtin_amdgcn_perm(w[2 * h + 1], w[2 * h], 0x06040200u);
+      u[h] = __builtin_amdgcn_perm(w[2 * h + 1], w[2 * h], 0x07050301u);
+    }
+    uint32_t* go = (uint32_t*)(out + row * 2L * k + ((long)c << 3));
+    uint32_t* uo = (uint32_t*)(out + row * 2L * k + k + ((long)c << 3));
+    go[0] = g[0]; go[1] = g[1];
+    uo[0] = u[0]; uo[1] = u[1];
+    if (smv_in && idx < pairs) {
+      // idx enumerates the input pairs (row, group, which)
+      const long r = idx / (2L * groups);
+      const int rem = (int)(idx - r * 2L * groups);
+      const int grp = rem >> 1, which = rem & 1;
+      smv_out[(r * 2 + which) * groups + grp] = smv_in[idx];
+    }
+  }
+}
+
+extern "C" int mui_int8_repack_gateup(mui_stream_t stream, const void* gate_up_nk2, const void* smv_ng22,
+                                      int group_size_shift, void* gate_up_n2k, void* smv_n2g2, int n_inter,
+                                      int k_in) {
+  MUI_CHECK_ARG(gate_up_nk2 && gate_up_n2k && n_inter > 0 && k_in > 0);
+  MUI_CHECK_ARG((smv_ng22 == nullptr) == (smv_n2g2 == nullptr));
+  MUI_CHECK_ARG(gate_up_nk2 != gate_up_n2k && (smv_ng22 == nullptr || smv_ng22 != smv_n2g2));
+  if (k_in & 15) return MUI_ERR_UNSUPPORTED;
+  int groups = 0;
+  if (smv_ng22) {
+    if (group_size_shift < 4 || group_size_shift > 30 || (k_in & ((1 << group_size_shift) - 1)))
+      return MUI_ERR_UNSUPPORTED;
+    groups = k_in >> group_size_shift;
+    if (((uintptr_t)smv_ng22 & 3) || ((uintptr_t)smv_n2g2 & 3)) return MUI_ERR_ALIGNMENT;
+  }
+  if (!aligned16(gate_up_nk2) || !aligned16(gate_up_n2k)) return MUI_ERR_ALIGNMENT;
+  // every (scale, min) pair needs a thread: 2 G pairs per row against K / 8 chunks per row
+  if (2L * groups > (k_in >> 3)) return MUI_ERR_UNSUPPORTED;
+  const long chunks = (long)n_inter * (k_in >> 3);
+  const int grid = (int)((chunks + 255) / 256 < 65536 ? (chunks + 255) / 256 : 65536);
+  hipLaunchKernelGGL(int8_repack_gateup_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)gate_up_nk2, (const uint32_t*)smv_ng22, (uint8_t*)gate_up_n2k,
+                     (uint32_t*)smv_n2g2, n_inter, k_in, groups);
+  return launch_status();
+}

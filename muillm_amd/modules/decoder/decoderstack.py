@@ -22,20 +22,38 @@ from ..quantized.int8gateupdownmlp import MuiInt8GateUpDownMLP
 from ..quantized.int8linear import MuiInt8Linear
 
 
+def _group_shift(m) -> int:
+    """0 for a 16-bit or per-channel int8 module, the group size's log2 for the group format."""
+    if type(m) is MuiInt8Linear and not m.per_channel:
+        return int(m.quantizer.group_size_shift)
+    if type(m) is MuiInt8GateUpDownMLP and not m.per_channel:
+        return int(m.group_size_shift)
+    return 0
+
+
 def _plain_linear(m, normalize: Optional[bool] = None) -> bool:
-    """A bias-free MuiLinear, or a bias-free per-channel MuiInt8Linear."""
+    """A bias-free MuiLinear, or a bias-free MuiInt8Linear (per-channel, or the group format with
+    groups of at least 16 that divide the rows)."""
     if type(m) is MuiInt8Linear:
-        return (m.per_channel and m.bias is None and m.dispatchable and m.weights_int8.is_contiguous()
-                and m.scales.is_contiguous() and (normalize is None or bool(m.normalize) == normalize))
+        if m.bias is not None or not m.dispatchable or (normalize is not None and bool(m.normalize) != normalize):
+            return False
+        if m.per_channel:
+            return m.weights_int8.is_contiguous() and m.scales.is_contiguous()
+        return (m.quantizer.group_size_shift >= 4 and m.in_features % 16 == 0 and m.weights_uint8.is_contiguous()
+                and m.scales_min_vals.is_contiguous())
     return (type(m) is MuiLinear and m.bias is None and m.weight.is_cuda and m.weight.stride(1) == 1
             and (normalize is None or bool(m.normalize) == normalize))
 
 
 def _linear_fields(m):
-    """(weight tensor, row pitch, scales tensor or None, [(owner, attribute, object)]) of a projection."""
+    """(weight tensor, row pitch, scales tensor or None, [(owner, attribute, object)]) of a projection;
+    "scales" are per-channel scales or, in the group format, the (scale, min) pairs."""
     if type(m) is MuiInt8Linear:
-        return m.weights_int8, m.weights_int8.stride(0), m.scales, [(m, "weights_int8", m.weights_int8),
-                                                                     (m, "scales", m.scales)]
+        if m.per_channel:
+            return m.weights_int8, m.weights_int8.stride(0), m.scales, [(m, "weights_int8", m.weights_int8),
+                                                                         (m, "scales", m.scales)]
+        return m.weights_uint8, m.weights_uint8.stride(0), m.scales_min_vals, [
+            (m, "weights_uint8", m.weights_uint8), (m, "scales_min_vals", m.scales_min_vals)]
     return m.weight, m.weight.stride(0), None, [(m, "weight", m.weight)]
 
 
@@ -73,12 +91,18 @@ class MuiDecoderStack:
             qw, qp, qs, q_own = _linear_fields(qkv)
             ow, op, osc, o_own = _linear_fields(attn.o_proj)
             dw, dp, ds, d_own = _linear_fields(mlp.down_proj)
+            shift = max(_group_shift(m) for m in (qkv, attn.o_proj, mlp, mlp.down_proj))
             if type(mlp) is MuiInt8GateUpDownMLP:
-                gu, gs = mlp.gate_up_weights, mlp.gate_up_scales  # [inter, 2, hidden] codes, [inter, 2] scales
+                gu = mlp.gate_up_weights  # [inter, 2, hidden] codes
                 g_ptr, u_ptr, g_pitch = gu.data_ptr(), gu.data_ptr() + gu.stride(1), gu.stride(0)
-                gs_ptr, us_ptr, gs_stride = gs.data_ptr(), gs.data_ptr() + gs.element_size(), gs.stride(0)
+                if mlp.per_channel:
+                    gs, gs_name = mlp.gate_up_scales, "gate_up_scales"  # [inter, 2] scales
+                else:
+                    gs, gs_name = mlp.gate_up_scales_min_vals, "gate_up_scales_min_vals"  # [inter, 2, G, 2] pairs
+                gs_ptr, us_ptr = gs.data_ptr(), gs.data_ptr() + gs.stride(1) * gs.element_size()
+                gs_stride = gs.stride(0)
                 gu_keep = [gu, gs]
-                gu_own = [(mlp, "gate_up_weights", gu), (mlp, "gate_up_scales", gs)]
+                gu_own = [(mlp, "gate_up_weights", gu), (mlp, gs_name, gs)]
             else:
                 g, u = mlp.gate_proj.weight, mlp.up_proj.weight
                 g_ptr, u_ptr, g_pitch = g.data_ptr(), u.data_ptr(), g.stride(0)
@@ -88,7 +112,7 @@ class MuiDecoderStack:
             arr[i] = _lib.MuiDecoderLayerDesc(
                 qkv.norm_weights.data_ptr(), qw.data_ptr(), qp, ow.data_ptr(), op,
                 mlp.norm_weights.data_ptr(), g_ptr, u_ptr, g_pitch, dw.data_ptr(), dp, kc.data_ptr(), vc.data_ptr(),
-                _ptr(qs), _ptr(osc), gs_ptr, us_ptr, gs_stride, _ptr(ds))
+                _ptr(qs), _ptr(osc), gs_ptr, us_ptr, gs_stride, _ptr(ds), shift)
             self._keep += [qkv.norm_weights, qw, qs, ow, osc, mlp.norm_weights, dw, ds, kc, vc] + gu_keep
             self._owners += [(layer, "qkv_proj", layer.qkv_proj), (layer, "self_attn", attn), (layer, "mlp", mlp),
                              (layer.qkv_proj, "linear", qkv), (qkv, "norm_weights", qkv.norm_weights),
@@ -106,7 +130,7 @@ class MuiDecoderStack:
     @staticmethod
     def eligible(layers, rotary_emb, cache, batch: int) -> bool:
         """fp16 / bf16 Llama-shaped layers without biases on a static cache, head_dim 128; every
-        projection either 16-bit or per-channel int8."""
+        projection 16-bit or int8 (per-channel, or the reference's group format)."""
         if not isinstance(cache, MuiStaticCache) or len(layers) == 0 or batch > _lib.MUI_MAX_TOKENS:
             return False
         if not getattr(rotary_emb, "dispatchable", False):
@@ -126,8 +150,10 @@ class MuiDecoderStack:
                 if mlp.gate_proj.weight.stride(0) != mlp.up_proj.weight.stride(0):
                     return False
             elif type(mlp) is MuiInt8GateUpDownMLP:
-                if not (mlp.per_channel and mlp.dispatchable and mlp.gate_up_weights.is_contiguous()
-                        and mlp.gate_up_scales.is_contiguous()):
+                if not (mlp.dispatchable and mlp.gate_up_weights.is_contiguous()):
+                    return False
+                sc = mlp.gate_up_scales if mlp.per_channel else mlp.gate_up_scales_min_vals
+                if not sc.is_contiguous() or (not mlp.per_channel and mlp.group_size_shift < 4):
                     return False
             else:
                 return False
@@ -142,8 +168,18 @@ class MuiDecoderStack:
                 return False
             dtype = w.dtype
             for m in (qkv.linear, attn.o_proj, mlp.down_proj):
-                if (m.scales.dtype if type(m) is MuiInt8Linear else m.weight.dtype) != dtype:
+                if type(m) is MuiInt8Linear:
+                    wd = m.scales.dtype if m.per_channel else m.scales_min_vals.dtype
+                else:
+                    wd = m.weight.dtype
+                if wd != dtype:
                     return False
+            # the int8 projections of a layer share one format: all per-channel, or all in the group
+            # format with one group size (the layer descriptor carries a single shift)
+            int8_mods = [m for m in (qkv.linear, attn.o_proj, mlp, mlp.down_proj)
+                         if type(m) in (MuiInt8Linear, MuiInt8GateUpDownMLP)]
+            if len({_group_shift(m) for m in int8_mods}) > 1:
+                return False
             e = (float(qkv.linear.variance_epsilon), float(mlp.variance_epsilon))
             if e[0] != e[1] or (eps is not None and e != eps):
                 return False

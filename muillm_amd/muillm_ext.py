@@ -495,15 +495,68 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
     return y
 
 
+# Row-interleaved twins of gate/up buffers that arrived in the reference's per-element packing,
+# keyed by the identity and version of the source tensors (bounded: one entry per quantised MLP).
+_REPACKED_GATEUP: "OrderedDict" = None
+_REPACKED_GATEUP_MAX = 256
+
+
+def _is_reference_gateup_packing(gate_up_weights: torch.Tensor) -> bool:
+    """[N, K, 2] (the reference's per-element interleave) as opposed to [N, 2, K]."""
+    return gate_up_weights.dim() == 3 and gate_up_weights.shape[2] == 2 and gate_up_weights.shape[1] != 2
+
+
+def _row_interleaved_gateup(gate_up_weights: torch.Tensor, gate_up_scales_min_vals: torch.Tensor,
+                            group_size_shift: int):
+    """(weights [N, 2, K], scales_min_vals [N, 2, G, 2]) of a gate/up pair in either packing.
+
+    The reference's own tensors ([N, K, 2] + [N*G, 2, 2], int8gateupdownmlp.py:211-230) are
+    converted on first use by mui_int8_repack_gateup and the result is kept for as long as the
+    source tensors are unchanged (same storage, same version counter), so a reference module that
+    calls this entry point every step pays the conversion once. The twin costs as much device
+    memory as the original."""
+    global _REPACKED_GATEUP
+    if not _is_reference_gateup_packing(gate_up_weights):
+        if gate_up_weights.dim() != 3 or gate_up_weights.shape[1] != 2:
+            raise RuntimeError("gate_up_weights must be [N, 2, K] (row-interleaved) or [N, K, 2] (the reference's)")
+        return gate_up_weights, gate_up_scales_min_vals
+    from collections import OrderedDict
+
+    if _REPACKED_GATEUP is None:
+        _REPACKED_GATEUP = OrderedDict()
+    w, smv = gate_up_weights, gate_up_scales_min_vals
+    _check_cuda(w, "gate_up_weights")
+    _check_cuda(smv, "gate_up_scales_min_vals")
+    n, k, _ = w.shape
+    g = k >> group_size_shift
+    if w.dtype != torch.uint8 or not w.is_contiguous() or not smv.is_contiguous() or smv.numel() != n * g * 4:
+        raise RuntimeError("reference packing: gate_up_weights uint8 [N, K, 2] and gate_up_scales_min_vals "
+                           "[N * K / group, 2, 2], both contiguous")
+    key = (w.data_ptr(), smv.data_ptr(), w._version, smv._version, n, k, int(group_size_shift), smv.dtype)
+    hit = _REPACKED_GATEUP.get(key)
+    if hit is not None:
+        _REPACKED_GATEUP.move_to_end(key)
+        return hit
+    out_w = torch.empty((n, 2, k), dtype=torch.uint8, device=w.device)
+    out_smv = torch.empty((n, 2, g, 2), dtype=smv.dtype, device=smv.device)
+    check(_lib.load().mui_int8_repack_gateup(_stream(w), w.data_ptr(), smv.data_ptr(), int(group_size_shift),
+                                             out_w.data_ptr(), out_smv.data_ptr(), n, k), "mui_int8_repack_gateup")
+    _REPACKED_GATEUP[key] = (out_w, out_smv)
+    while len(_REPACKED_GATEUP) > _REPACKED_GATEUP_MAX:
+        _REPACKED_GATEUP.popitem(last=False)
+    return out_w, out_smv
+
+
 def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_up_scales_min_vals,
                                    group_size_shift, x) -> torch.Tensor:
-    """csrc/module.cpp:248. gate_up_weights is the packed uint8 buffer [N, 2, K] (row n of gate,
-    then row n of up) and gate_up_scales_min_vals is [N, 2, G, 2]; the reference packs per
-    element ([N, K, 2], int8gateupdownmlp.py:211-230), this build per row so that each row
-    stays one contiguous 128-bit-loadable stream."""
+    """csrc/module.cpp:248. Takes the reference's packing -- gate_up_weights uint8 [N, K, 2],
+    gate_up_scales_min_vals [N*G, 2, 2] (int8gateupdownmlp.py:211-230) -- or this build's
+    row-interleaved one, [N, 2, K] (row n of gate, then row n of up) with [N, 2, G, 2], which
+    keeps each row one contiguous 128-bit-loadable stream; the first is converted once (see
+    _row_interleaved_gateup)."""
+    gate_up_weights, gate_up_scales_min_vals = _row_interleaved_gateup(gate_up_weights, gate_up_scales_min_vals,
+                                                                       group_size_shift)
     n, two, k = gate_up_weights.shape
-    if two != 2:
-        raise RuntimeError("gate_up_weights must be [N, 2, K]")
     g = k >> group_size_shift
     _check_activations(x, k, "muillm_int8_gateupsilu_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS),
                        gate_up_weights, gate_up_scales_min_vals, norm_weights)
@@ -535,7 +588,10 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
 
 
 def muillm_int8_gateupsilu_dequantize_forward(gate_up_weights, gate_up_scales_min_vals, group_size_shift):
-    """csrc/module.cpp:247: packed [N, 2, K] uint8 -> (gate, up) dense 16-bit matrices."""
+    """csrc/module.cpp:247: packed uint8 gate/up ([N, K, 2] as in the reference, or [N, 2, K]) ->
+    (gate, up) dense 16-bit matrices."""
+    gate_up_weights, gate_up_scales_min_vals = _row_interleaved_gateup(gate_up_weights, gate_up_scales_min_vals,
+                                                                       group_size_shift)
     n, _, k = gate_up_weights.shape
     g = k >> group_size_shift
     smv = gate_up_scales_min_vals.reshape(n, 2, g, 2)

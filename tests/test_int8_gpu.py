@@ -181,6 +181,32 @@ def test_group_gateup(n, k, gs):
     dg, du = muillm_ext.muillm_int8_gateupsilu_dequantize_forward(packed_w, packed_s, shift)
     assert torch.equal(dg.cpu(), oracle.rtn_dequantize_group(qg, smg, gs))
     assert torch.equal(du.cpu(), oracle.rtn_dequantize_group(qu, smu, gs))
+    # the reference's own packing (muillm/modules/quantized/int8gateupdownmlp.py:211-230: codes
+    # concatenated on a new last axis, (scale, min) rows on a new middle axis) gives the same bits
+    ref_w = torch.cat([qg[:, :, None], qu[:, :, None]], dim=2).to(DEV)               # [N, K, 2]
+    ref_s = torch.cat([smg[:, None, :], smu[:, None, :]], dim=1).to(DEV)             # [N*G, 2, 2]
+    assert ref_w.shape == (n, k, 2) and ref_s.shape == (n * ng, 2, 2)
+    h_ref = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, ref_w, ref_s, shift, x.to(DEV))
+    assert torch.equal(h_ref, h)
+    rg, ru = muillm_ext.muillm_int8_gateupsilu_dequantize_forward(ref_w, ref_s, shift)
+    assert torch.equal(rg, dg) and torch.equal(ru, du)
+    # converted once: a second call finds the row-interleaved twin; an in-place edit of the source drops it
+    twins = len(muillm_ext._REPACKED_GATEUP)
+    muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, ref_w, ref_s, shift, x.to(DEV))
+    assert len(muillm_ext._REPACKED_GATEUP) == twins
+    ref_w[0, 0, 0] += 1
+    h_edit = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, ref_w, ref_s, shift, x.to(DEV))
+    assert len(muillm_ext._REPACKED_GATEUP) == twins + 1 and not torch.equal(h_edit[..., 0], h[..., 0])
+    # the conversion itself, through the C ABI, against torch's permute
+    lib = _lib.load()
+    out_w = torch.empty((n, 2, k), dtype=torch.uint8, device=DEV)
+    out_s = torch.empty((n, 2, ng, 2), dtype=torch.float16, device=DEV)
+    st = lib.mui_int8_repack_gateup(torch.cuda.current_stream().cuda_stream, ref_w.data_ptr(), ref_s.data_ptr(), shift,
+                                    out_w.data_ptr(), out_s.data_ptr(), n, k)
+    assert st == 0
+    assert torch.equal(out_w, ref_w.permute(0, 2, 1)) and torch.equal(out_s, ref_s.reshape(n, ng, 2, 2).permute(0, 2, 1, 3))
+    assert lib.mui_int8_repack_gateup(None, ref_w.data_ptr(), ref_s.data_ptr(), 3, out_w.data_ptr(), out_s.data_ptr(), n, k) == -2
+    assert lib.mui_int8_repack_gateup(None, ref_w.data_ptr(), None, shift, out_w.data_ptr(), out_s.data_ptr(), n, k) == -1
 
 
 def test_int8_abi_errors():

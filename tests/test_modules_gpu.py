@@ -360,14 +360,16 @@ def test_decoder_stack_call_matches_layer_modules(batch, dtype):
 
 @pytest.mark.parametrize("modules", [["qkv_proj", "o_proj", "mlp"], ["mlp"], ["o_proj"]])
 @pytest.mark.parametrize("batch", [1, 3])
-def test_decoder_stack_call_int8_layers(modules, batch):
-    """Per-channel int8 projections (all of them, or only some: the rest stay fp16) go through the
-    single call too: same logits and cache contents as the layer modules called one by one; the
-    group format keeps the per-layer calls."""
+@pytest.mark.parametrize("group_size", [0, 128])
+def test_decoder_stack_call_int8_layers(modules, batch, group_size):
+    """int8 projections -- per-channel (group_size 0) or the reference's group-wise (scale, min)
+    format -- all of them, or only some (the rest stay fp16), go through the single call too: same
+    logits and cache contents as the layer modules called one by one, and the same tokens from
+    HIP-graph replay."""
     cfg = _small_config(layers=2)
     base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=5,
                                            init_std=0.05, finalize=False)
-    qm = Int8WeightOnlyQuantizationMethod(group_size=0, modules=modules)
+    qm = Int8WeightOnlyQuantizationMethod(group_size=group_size, modules=modules)
     lm = init_engine(copy.deepcopy(base), device=DEV, engine_config=MuiEngineConfig(qm))
     g = torch.Generator().manual_seed(6)
     ids = torch.randint(0, cfg.vocab_size, (batch, 9), generator=g).to(DEV)
@@ -388,13 +390,19 @@ def test_decoder_stack_call_int8_layers(modules, batch):
     assert torch.equal(results[False][0], results[True][0])
     for x, y in zip(results[False][1], results[True][1]):
         assert torch.equal(x, y)
-    # the reference's group format is not part of the single call
-    qg = Int8WeightOnlyQuantizationMethod(group_size=128, modules=modules)
-    lg = init_engine(base, device=DEV, engine_config=MuiEngineConfig(qg))
-    with torch.no_grad():
-        out = lg(input_ids=ids)
-        lg(input_ids=out.logits[:, -1].argmax(-1).unsqueeze(1), past_key_values=out.past_key_values)
-    assert lg.model._stack is None
+    eager = lm.generate_greedy(ids, 6, use_graph=False)
+    assert torch.equal(lm.generate_greedy(ids, 6, use_graph=True), eager)
+    # a layer that mixes the two int8 formats keeps the per-layer calls (one descriptor, one format)
+    if group_size and len(modules) == 3:
+        mixed = init_engine(copy.deepcopy(base), device=DEV, engine_config=MuiEngineConfig(
+            Int8WeightOnlyQuantizationMethod(group_size=0, modules=["o_proj"])))
+        from muillm_amd.quantization.quantizedreplacements import quantize_layers
+        mixed = quantize_layers(mixed, MuiEngineConfig(Int8WeightOnlyQuantizationMethod(group_size=128, modules=["mlp"])),
+                                device=DEV)
+        with torch.no_grad():
+            out = mixed(input_ids=ids)
+            mixed(input_ids=out.logits[:, -1].argmax(-1).unsqueeze(1), past_key_values=out.past_key_values)
+        assert mixed.model._stack is None
 
 
 def test_argmax_kernel():
