@@ -73,9 +73,10 @@ def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=True, batch=1):
     return dt, dec
 
 
-def bench_int8_variant(config, steps, warmup):
-    """The same decode benchmark with the decoder layers quantised to int8 (symmetric per output
-    channel; lm_head stays 16-bit, as the reference's module-name filter would leave it)."""
+def bench_int8_variant(config, steps, warmup, group_size=0):
+    """The same decode benchmark with the decoder layers quantised to int8 (group_size 0: symmetric
+    per output channel; else the reference's group-wise uint8 + (scale, min) format; lm_head stays
+    16-bit, as the reference's module-name filter would leave it)."""
     import torch
 
     from muillm_amd.engine import init_engine
@@ -83,7 +84,7 @@ def bench_int8_variant(config, steps, warmup):
     from muillm_amd.modules.models.llama.model import MuiLlamaForCausalLM
     from muillm_amd.quantization.quantizationmethod import Int8WeightOnlyQuantizationMethod
 
-    qm = Int8WeightOnlyQuantizationMethod(group_size=0, modules=["qkv_proj", "o_proj", "mlp"])
+    qm = Int8WeightOnlyQuantizationMethod(group_size=group_size, modules=["qkv_proj", "o_proj", "mlp"])
     base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0,
                                            finalize=False)
     lm8 = init_engine(base, device="cuda", engine_config=MuiEngineConfig(qm))
@@ -93,13 +94,16 @@ def bench_int8_variant(config, steps, warmup):
     dt_eager, dec = bench_decode(lm8, steps, warmup, use_graph=False)
     hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
     hq, hkv, d = config.num_attention_heads, config.num_key_value_heads, hid // config.num_attention_heads
-    wbytes = config.num_hidden_layers * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter) + 2 * v * hid
+    codes = config.num_hidden_layers * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter)
+    # per-channel: one fp16 scale per row (negligible); group format: 4 bytes of (scale, min) per group
+    wbytes = codes + (codes // group_size * 4 if group_size else 0) + 2 * v * hid
     del dec, lm8, base
     torch.cuda.empty_cache()
     return {"tokens_per_s": round(steps / dt, 2), "ms_per_step": round(dt / steps * 1e3, 4),
             "eager_no_graph_tokens_per_s": round(steps / dt_eager, 2),
             "weight_bytes_per_token": wbytes, "hbm_floor_ms": round(wbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4),
-            "format": "int8 per output channel + fp16 scale; lm_head fp16"}
+            "format": ("uint8 + fp16 (scale, min) per group of %d inputs (the reference's RTN format); lm_head fp16" % group_size)
+            if group_size else "int8 per output channel + fp16 scale; lm_head fp16"}
 
 
 def measured_copy_ceiling():
@@ -217,6 +221,58 @@ def pmc_probe_batched(launches=6, tokens=8):
     print(json.dumps({"pmc_probe_batched": {"launches": launches, "tokens": tokens,
                                             "gateup_flops": 4 * inter * hid * tokens, "down_flops": 2 * inter * hid * tokens,
                                             "gateup_weight_bytes": 4 * inter * hid, "down_weight_bytes": 2 * inter * hid}}))
+
+
+def pmc_probe_int8(launches=4):
+    """Counter probe for the int8 GEMVs of a Llama-3-8B layer (per-channel format): QKV, o_proj, down
+    and gate/up at 1 and at 4 tokens, `launches` launches each over distinct weight buffers, then as
+    many launches of an elementwise copy of 117,440,512 B for the counters' units
+    (`rocprofv3 --pmc FETCH_SIZE`; `--pmc SQ_WAVES SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_VMEM_RD`;
+    `--pmc SQ_BUSY_CU_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY GRBM_GUI_ACTIVE`)."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    hid, inter, n_qkv = 4096, 14336, 6144
+    f16 = dict(device="cuda", dtype=torch.float16)
+    stream = torch.cuda.current_stream().cuda_stream
+    gamma = torch.ones(hid, **f16)
+    X, RES, HM = torch.randn(4, hid, **f16), torch.randn(4, hid, **f16), torch.randn(4, inter, **f16)
+    Y = torch.empty(4 * inter, **f16)
+    shapes = (("qkv", n_qkv, hid, True, False), ("o_proj", hid, hid, False, True), ("down", hid, inter, False, True))
+    info = {}
+    for b in (1, 4):
+        for name, n, k, norm, resid in shapes:
+            ws = [(torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda"), torch.rand(n, **f16) * 1e-3 + 1e-4)
+                  for _ in range(launches)]
+            xin = X if k == hid else HM
+            torch.cuda.synchronize()
+            for q, sc in ws:
+                _lib.check(lib.mui_int8_linear(stream, 0, q.data_ptr(), k, sc.data_ptr(), xin.data_ptr(),
+                                               gamma.data_ptr() if norm else None, 1e-5, None,
+                                               RES.data_ptr() if resid else None, Y.data_ptr(), n, k, b), "mui_int8_linear")
+            torch.cuda.synchronize()
+            info["%s_tokens%d" % (name, b)] = {"weight_bytes": n * k, "weights": n * k}
+            del ws
+        ws = [(torch.randint(-127, 128, (inter, 2, hid), dtype=torch.int8, device="cuda"),
+               torch.rand(inter, 2, **f16) * 1e-3 + 1e-4) for _ in range(launches)]
+        torch.cuda.synchronize()
+        for q, sc in ws:
+            _lib.check(lib.mui_int8_gateup_silu(stream, 0, q.data_ptr(), q.data_ptr() + hid, 2 * hid, sc.data_ptr(),
+                                                sc.data_ptr() + 2, 2, X.data_ptr(), gamma.data_ptr(), 1e-5, Y.data_ptr(),
+                                                inter, hid, b), "mui_int8_gateup_silu")
+        torch.cuda.synchronize()
+        info["gateup_tokens%d" % b] = {"weight_bytes": 2 * inter * hid, "weights": 2 * inter * hid}
+        del ws
+    src = [torch.randn(inter * hid, **f16) for _ in range(2)]
+    dst = torch.empty(inter * hid, **f16)
+    for i in range(launches):
+        torch.mul(src[i % 2], 1.0, out=dst)
+    torch.cuda.synchronize()
+    info["copy"] = {"bytes_read": dst.numel() * 2, "bytes_written": dst.numel() * 2}
+    print(json.dumps({"pmc_probe_int8": {"launches": launches, "order": "tokens 1: qkv, o_proj, down, gateup; tokens 4: same; copy",
+                                         "calls": info}}))
 
 
 def pmc_probe_attention(launches=3):
@@ -374,6 +430,44 @@ def kernel_table(lm):
         del ring
     torch.cuda.empty_cache()
 
+    # ---- C3g: the same GEMVs on the reference's own format (uint8 codes + fp16 (scale, min) per group
+    # of 128 inputs, muillm/quantization/rtnquantizer.py:49-88)
+    gshift, gsz = 7, 128
+
+    def g_ring(n, k):
+        cnt = max(2, int(0.95e9 // (n * k)) + 1)
+        return [(torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda"),
+                 torch.rand(n * (k // gsz), 2, **f16) * 1e-3 + 1e-4) for _ in range(cnt)]
+
+    for b in (1, 4):
+        for name, n, k, norm, resid in (("qkv", n_qkv, hid, True, False), ("o_proj", hid, hid, False, True),
+                                        ("down", hid, inter, False, True)):
+            ring = g_ring(n, k)
+            xin = X if k == hid else HMID
+
+            def fg(i, ring=ring, xin=xin, n=n, k=k, norm=norm, resid=resid, b=b):
+                q, smv = ring[i % len(ring)]
+                lib.mui_int8_group_linear(stream, 0, q.data_ptr(), k, smv.data_ptr(), gshift, xin.data_ptr(),
+                                          gamma.data_ptr() if norm else None, 1e-5, None,
+                                          RES.data_ptr() if resid else None, Y.data_ptr(), n, k, b)
+            add("C3g_group128_%s_%dx%d_tokens%d" % (name, n, k, b), fg,
+                n * k + 4 * n * (k // gsz) + 2 * hid * norm + b * 2 * (k + n + n * resid), len(ring),
+                reads=[([q.data_ptr() for q, _ in ring], n * k)])
+            del ring
+        ring = [(torch.randint(0, 256, (inter, 2, hid), dtype=torch.uint8, device="cuda"),
+                 torch.rand(inter, 2, hid // gsz, 2, **f16) * 1e-3 + 1e-4) for _ in range(9)]
+
+        def gg(i, ring=ring, b=b):
+            q, smv = ring[i % len(ring)]
+            lib.mui_int8_group_gateup_silu(stream, 0, q.data_ptr(), q.data_ptr() + hid, 2 * hid, smv.data_ptr(),
+                                           smv.data_ptr() + 2 * 2 * (hid // gsz), 4 * (hid // gsz), gshift,
+                                           X.data_ptr(), gamma.data_ptr(), 1e-5, hbuf.data_ptr(), inter, hid, b)
+        add("C3g_group128_gateup_silu_%dx%d_tokens%d" % (2 * inter, hid, b), gg,
+            2 * inter * hid + 8 * inter * (hid // gsz) + 2 * hid + b * 2 * (hid + inter), len(ring),
+            reads=[([q.data_ptr() for q, _ in ring], 2 * inter * hid)])
+        del ring
+    torch.cuda.empty_cache()
+
     # ---- C4: fused RoPE + cache write + flash decoding, GQA 32/8 x 128 (bytes = the K/V rows read)
     hq, hkv, d = 32, 8, 128
     for S, B in ((1024, 1), (4096, 1), (16384, 1), (32768, 1), (1024, 8), (4096, 8), (32768, 8)):
@@ -453,15 +547,40 @@ def cpu_baseline(config, layers_sample=4, steps_sample=100, ctx_len=64):
             for p in layers:
                 h = layer_step(p, h, ctx_len + s)
         t_layers = (time.perf_counter() - t0) / (steps_sample * layers_sample)
-        oracle.linear(h0, lm_head, torch.ones(hid).half(), 1e-5, reference_path=True)
-        t0 = time.perf_counter()
-        oracle.linear(h0, lm_head, torch.ones(hid).half(), 1e-5, reference_path=True)
-        t_head = time.perf_counter() - t0
+        ones = torch.ones(hid).half()
+        oracle.linear(h0, lm_head, ones, 1e-5, reference_path=True)
+        head_times = []
+        for _ in range(11):  # median of 11 calls: a single call varies 2x from run to run
+            t0 = time.perf_counter()
+            oracle.linear(h0, lm_head, ones, 1e-5, reference_path=True)
+            head_times.append(time.perf_counter() - t0)
+        t_head = sorted(head_times)[len(head_times) // 2]
     per_token = t_layers * config.num_hidden_layers + t_head
+    layer_bytes = 2 * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter)
+    head_bytes = 2 * v * hid
     return {"value": round(1.0 / per_token, 4), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{layers_sample} decoder layers x {steps_sample} decode steps (ctx {ctx_len}) + 1 lm_head call of the "
-                      f"reference's PyTorch fallback path in fp16 on CPU, extrapolated to {config.num_hidden_layers} layers",
-            "s_per_layer": round(t_layers, 4), "s_lm_head": round(t_head, 4), "host_cpus": os.cpu_count()}
+            "sample": f"{layers_sample} decoder layers x {steps_sample} decode steps (ctx {ctx_len}) + median of 11 lm_head "
+                      f"calls of the reference's PyTorch fallback path in fp16 on CPU, extrapolated to "
+                      f"{config.num_hidden_layers} layers",
+            "s_per_layer": round(t_layers, 5), "s_lm_head": round(t_head, 5),
+            "s_lm_head_min_max": [round(min(head_times), 5), round(max(head_times), 5)],
+            "layer_weight_GB/s": round(layer_bytes / t_layers / 1e9, 1),
+            "lm_head_weight_GB/s": round(head_bytes / t_head / 1e9, 1),
+            "cpu_model": _cpu_model(), "host_cpus": os.cpu_count()}
+
+
+def _cpu_model():
+    """The host CPU's model string (/proc/cpuinfo), for reading the baseline figure."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+
+    return platform.processor() or platform.machine()
 
 
 def main():
@@ -483,6 +602,8 @@ def main():
                     help="only launch the gate/up GEMV and a calibration copy a few times (for rocprofv3 --pmc runs)")
     ap.add_argument("--pmc-probe-batched", action="store_true",
                     help="launch the 8-token MLP kernels a few times and exit (for rocprofv3 --pmc)")
+    ap.add_argument("--pmc-probe-int8", action="store_true",
+                    help="launch the int8 GEMVs of a Llama-3-8B layer at 1 and 4 tokens a few times and exit (for rocprofv3 --pmc)")
     ap.add_argument("--pmc-probe-attention", action="store_true",
                     help="launch flash decoding at 32k context a few times and exit (for rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -502,6 +623,9 @@ def main():
         return
     if args.pmc_probe_batched:
         pmc_probe_batched()
+        return
+    if args.pmc_probe_int8:
+        pmc_probe_int8()
         return
     if args.pmc_probe_attention:
         pmc_probe_attention()
@@ -575,6 +699,7 @@ def main():
         del dec_bf, lm_bf
         torch.cuda.empty_cache()
         result["variants"]["int8"] = bench_int8_variant(config, args.steps, args.warmup)
+        result["variants"]["int8_group128"] = bench_int8_variant(config, args.steps, args.warmup, group_size=128)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(config)
         result["cpu_baseline"]["gpu_over_cpu"] = round(tokens_per_s / result["cpu_baseline"]["value"], 1)

@@ -45,7 +45,8 @@ extern "C" {
 #define MUI_DTYPE_F16 0
 #define MUI_DTYPE_BF16 1
 
-/* largest token batch the decode kernels accept in one call */
+/* largest token batch of the weight-streaming decode kernels (and of mui_decoder_stack_step); the
+ * linear entry points take more tokens than this through their tiled GEMM */
 #define MUI_MAX_TOKENS 16
 
 typedef void* mui_stream_t; /* a hipStream_t; NULL is the default stream */
@@ -84,7 +85,10 @@ int mui_device_info(int device, mui_device_info_t* out);
  * W is [n_out, k_in] with row pitch `w_pitch` elements (w_pitch == k_in when dense);
  * x is [tokens, k_in]; y, residual are [tokens, n_out]; norm_weights is [k_in];
  * mul_bias, add_bias are [n_out]. norm_weights, mul_bias, add_bias, residual may be NULL.
- * tokens in 1..MUI_MAX_TOKENS. epsilon is added to the mean (HuggingFace convention).
+ * tokens >= 1: up to MUI_MAX_TOKENS the weight-streaming decode kernels (weights read once per
+ * call), beyond that a tiled matrix-core GEMM (weights read once per 128 tokens) -- the reference
+ * hands every multi-token call to the framework's GEMM after a separate RMSNorm kernel
+ * (csrc/modules/linear_module.cpp:57-79). epsilon is added to the mean (HuggingFace convention).
  * Requirements: k_in % 8 == 0, W and x 16-byte aligned, w_pitch % 8 == 0.
  * y may alias residual. */
 int mui_linear(mui_stream_t stream, int dtype, const void* weights, long w_pitch,
@@ -105,7 +109,7 @@ int mui_rmsnorm(mui_stream_t stream, int dtype, const void* weights, const void*
  * G and U are [n_inter, k_in] with a common row pitch `gu_pitch` elements. They may be two
  * separate dense matrices (gu_pitch == k_in) or the two interleaved halves of one packed
  * [n_inter, 2, k_in] buffer (up == gate + k_in, gu_pitch == 2 * k_in), which is the layout
- * the Python layer repacks to. xn as in mui_linear. h is [tokens, n_inter].
+ * the Python layer repacks to. xn and the token range as in mui_linear. h is [tokens, n_inter].
  * The second half (down projection + residual) is mui_linear with residual. */
 int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate, const void* up,
                     long gu_pitch, const void* x, const void* norm_weights, float epsilon,
@@ -128,6 +132,9 @@ int mui_silu_mul_interleaved(mui_stream_t stream, int dtype, const void* gate_up
  *   weights_i8 int8 [n_out, k_in] (row pitch w_pitch bytes), scales 16-bit [n_out],
  *   w[n, k] = q[n, k] * scales[n];   y = W xn + add_bias + residual   (xn as in mui_linear).
  * The reference passes the residual through add_bias (int8linear.py:53-57); here both exist.
+ * Any tokens >= 1 (as mui_linear: beyond MUI_MAX_TOKENS the tiled GEMM converts the codes on their
+ * way to LDS; the reference dequantises the whole matrix and calls the framework's GEMM,
+ * muillm/modules/quantized/int8linear.py:279-293).
  * Requirements: k_in % 16 == 0, k_in <= 16384, 16-byte aligned rows. */
 int mui_int8_linear(mui_stream_t stream, int dtype, const void* weights_i8, long w_pitch,
                     const void* scales, const void* x, const void* norm_weights, float epsilon,

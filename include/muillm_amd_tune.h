@@ -44,6 +44,12 @@ int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int di
  * qualify on matrices of >= 8192 rows with K <= 4096; 1 = never) */
 int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 
+/* Prompt GEMM (more than MUI_MAX_TOKENS tokens): tile = 0 built-in choice, 1 = 128 rows x 128
+ * tokens, 2 = 64 x 128, 3 = 32 x 64 (linear only); wide_max_tokens = longest prompt served by the
+ * weight-streaming 16-rows-per-workgroup kernel instead of the LDS-tiled one (0 restores the
+ * built-in choice; at most 128; negative: never) */
+int mui_tune_prefill(int tile, int wide_max_tokens);
+
 /* Measurement aid without a counterpart in the reference: reads `bytes` (a multiple of 16, from
  * a 16-byte aligned address) of device memory once with the access shape of the GEMV kernels and
  * discards them. One launch takes the least time any kernel that must read that many bytes can

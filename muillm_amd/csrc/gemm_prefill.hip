@@ -1,0 +1,334 @@
+// Linear layers for more than MUI_MAX_TOKENS tokens (prompts): a tiled matrix-core GEMM with the
+// same fused prologue / epilogues as the decode GEMVs.
+//
+// The reference hands every multi-token call to the framework's GEMM after a standalone RMSNorm
+// kernel (csrc/modules/linear_module.cpp:57-79; muillm/modules/linear.py:324-333;
+// muillm/modules/gateupdownmlp.py:343-359: norm, two matmuls, SiLU, multiply, matmul, add;
+// int8: dequantise the whole matrix first, muillm/modules/quantized/int8linear.py:279-293).
+// Here one kernel does y = (W . (gamma * x)) * rsqrt(mean(x^2) + eps) [* scale] [* mul_bias]
+// [+ add_bias] [+ residual], or h = silu(G xn) * (U xn), for 16-bit or per-channel int8 weights.
+//
+// Work layout (wave64, v_mfma_f32_16x16x32):
+//   a workgroup of 4 waves (2 x 2) owns a tile of weight rows x tokens and walks K in steps: the
+//   weight tile (int8 rows converted on the way) and the token tile (gamma * x rounded once to
+//   the 16-bit type, sum of squares gathered on the side) are staged through LDS with a padded
+//   pitch (conflict-free 128-bit reads); the loads of step s + 1 are in flight while step s is
+//   multiplied. Three tile shapes: 128 rows x 128 tokens x 64 k (each wave 4 x 4 MFMA tiles) when
+//   that still gives two workgroups per CU; else 64 x 128 x 128; else 32 x 64 x 256 -- the
+//   smaller the grid, the longer the k-step, so that enough weight bytes are in flight per CU.
+//   Under the gate/up epilogue half of a wave's rows are gate rows and the other half the up
+//   rows of the same outputs, so SiLU * mul happens in registers.
+//   Token tiles of one row tile are placed on the same XCD (workgroup id modulo 8) so that the
+//   re-reads of its weights hit that XCD's L2.
+#include "skinny.cuh"
+
+namespace mui {
+
+constexpr int kPfThreads = 256;  // 4 waves: 2 (rows) x 2 (tokens)
+
+struct PrefillGemmParams {
+  const uint8_t* w0;      // linear: matrix; gate/up: gate rows
+  const uint8_t* w1;      // gate/up: up rows
+  long pitch;             // weight row pitch in bytes
+  const uint16_t* s0;     // per-channel int8: scale of row n at s0[n * s_pitch]
+  const uint16_t* s1;
+  long s_pitch;
+  const uint16_t* x;      // [tokens, k] dense
+  const uint16_t* gamma;
+  const uint16_t* mul_bias;
+  const uint16_t* add_bias;
+  const uint16_t* residual;  // [tokens, n] dense
+  uint16_t* y;               // [tokens, n] dense
+  int n;        // outputs (weight rows; gate/up pairs)
+  int k;
+  int tokens;
+  float eps;
+  int n_tiles;  // row tiles
+  int t_tiles;  // token tiles
+};
+
+// WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile is 32 WR weight rows x 32 WT tokens;
+// KS k-values per step.
+template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int KS>
+__global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillGemmParams p) {
+  constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
+  constexpr int PITCH = KS + 8;          // LDS row pitch in 16-bit elements: conflict-free 128-bit reads
+  constexpr int CPR = KS / 8;            // 16-byte chunks of 8 elements per row and step
+  constexpr int OUT_TILE = (EPI == SK_GATEUP) ? ROWS / 2 : ROWS;  // outputs per workgroup
+  constexpr int XCH = TOKS * CPR / kPfThreads;                     // token loads per thread and step
+  constexpr int WCH = (WF == WF_16BIT) ? ROWS * CPR / kPfThreads : ROWS * (KS / 16) / kPfThreads;
+  static_assert(EPI != SK_GATEUP || WR % 2 == 0, "gate/up needs an even number of row tiles per wave");
+  static_assert(XCH >= 1 && WCH >= 1 && kPfThreads % CPR == 0, "tile shape");
+  __shared__ __align__(16) uint16_t w_lds[ROWS * PITCH];
+  __shared__ __align__(16) uint16_t x_lds[TOKS * PITCH];
+  __shared__ float rs_lds[TOKS];
+
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int wr = wave >> 1;  // which half of the rows
+  const int wt = wave & 1;   // which half of the tokens
+
+  // workgroup -> (row tile, token tile): consecutive workgroup ids are dealt round-robin to the
+  // 8 XCDs, so ids that share id % 8 share an L2; give each XCD whole row tiles
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int tile_n = (slot / p.t_tiles) * 8 + xcd;
+  const int tile_t = slot % p.t_tiles;
+  if (tile_n >= p.n_tiles) return;  // uniform for the workgroup, before any barrier
+  const int o0 = tile_n * OUT_TILE;  // first output of the tile
+  const int t0 = tile_t * TOKS;      // first token of the tile
+
+  // local weight row r -> matrix row. linear: o0 + r. gate/up: of a wave's 16 WR rows the first
+  // half are gate rows, the second half the up rows of the same outputs
+  auto weight_row_ptr = [&](int r) -> const uint8_t* {
+    if constexpr (EPI == SK_GATEUP) {
+      constexpr int HALF = 8 * WR;  // outputs per wave
+      const int h = r / (2 * HALF), within = r % (2 * HALF);
+      int o = o0 + h * HALF + within % HALF;
+      o = o < p.n ? o : p.n - 1;
+      return (within >= HALF ? p.w1 : p.w0) + (long)o * p.pitch;
+    } else {
+      int o = o0 + r;
+      o = o < p.n ? o : p.n - 1;
+      return p.w0 + (long)o * p.pitch;
+    }
+  };
+
+  // ---- staging assignment: 16-byte chunk c = t + 256 i of a tile is row c / chunks-per-row,
+  // column c % chunks-per-row (the column is the same for every i)
+  const int xcol = t % CPR;
+  const uint16_t* xrow[XCH];
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) {
+    int tk = t0 + (t + kPfThreads * i) / CPR;
+    tk = tk < p.tokens ? tk : p.tokens - 1;
+    xrow[i] = p.x + (long)tk * p.k;
+  }
+  constexpr int WCPR = (WF == WF_16BIT) ? CPR : KS / 16;  // weight chunks per row (int8: 16 codes each)
+  const int wcol = t % WCPR;
+  const uint8_t* wrow[WCH];
+#pragma unroll
+  for (int i = 0; i < WCH; ++i) wrow[i] = weight_row_ptr((t + kPfThreads * i) / WCPR);
+
+  u32x4 wreg[WCH], xreg[XCH], greg;
+  auto load_step = [&](int k0) {
+    // chunks past the end of the row read the row's first chunk and are zeroed on the way to LDS
+    const int xk = k0 + xcol * 8;
+    const int xoff = xk + 8 <= p.k ? xk : 0;
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) xreg[i] = ld16(xrow[i] + xoff);
+    if constexpr (NORM) greg = ld16(p.gamma + xoff);
+    if constexpr (WF == WF_16BIT) {
+#pragma unroll
+      for (int i = 0; i < WCH; ++i) wreg[i] = ld16_stream(wrow[i] + 2L * xoff);
+    } else {
+      const int wk = k0 + wcol * 16;
+      const int woff = wk + 16 <= p.k ? wk : 0;
+#pragma unroll
+      for (int i = 0; i < WCH; ++i) wreg[i] = ld16_stream(wrow[i] + woff);
+    }
+  };
+
+  float ss[XCH];
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) ss[i] = 0.f;
+  auto store_step = [&](int k0) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const bool xlive = k0 + xcol * 8 + 8 <= p.k;
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      float sq = 0.f;
+      u32x4 b = make_b<T, NORM>(xreg[i], NORM ? greg : xreg[i], sq);
+      b = xlive ? b : zero;
+      ss[i] += xlive ? sq : 0.f;
+      *(u32x4*)&x_lds[((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = b;
+    }
+    if constexpr (WF == WF_16BIT) {
+#pragma unroll
+      for (int i = 0; i < WCH; ++i)
+        *(u32x4*)&w_lds[((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = xlive ? wreg[i] : zero;
+    } else {
+      const bool wlive = k0 + wcol * 16 + 16 <= p.k;
+#pragma unroll
+      for (int i = 0; i < WCH; ++i) {
+        const u32x4 lo = convert_a<T, WF>(wreg[i].x, wreg[i].y, nullptr, 0, 0);
+        const u32x4 hi = convert_a<T, WF>(wreg[i].z, wreg[i].w, nullptr, 0, 0);
+        uint16_t* dst = &w_lds[((t + kPfThreads * i) / WCPR) * PITCH + wcol * 16];
+        *(u32x4*)dst = wlive ? lo : zero;
+        *(u32x4*)(dst + 8) = wlive ? hi : zero;
+      }
+    }
+  };
+
+  f32x4 acc[WR][WT];
+#pragma unroll
+  for (int i = 0; i < WR; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (t < TOKS) rs_lds[t] = 0.f;
+
+  const int n_steps = (p.k + KS - 1) / KS;
+  const int a_base = (wr * 16 * WR + (lane & 15)) * PITCH + (lane >> 4) * 8;
+  const int b_base = (wt * 16 * WT + (lane & 15)) * PITCH + (lane >> 4) * 8;
+  load_step(0);
+  for (int s = 0; s < n_steps; ++s) {
+    __syncthreads();  // the previous step's operands have been read
+    store_step(s * KS);
+    __syncthreads();
+    // requested now, consumed after this step's multiplications (the last iteration re-reads
+    // step 0, which keeps the loads out of a branch)
+    load_step(s + 1 < n_steps ? (s + 1) * KS : 0);
+#pragma unroll
+    for (int ks = 0; ks < KS / 32; ++ks) {
+      u32x4 a[WR], b[WT];
+#pragma unroll
+      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[a_base + i * 16 * PITCH + ks * 32];
+#pragma unroll
+      for (int j = 0; j < WT; ++j) b[j] = *(const u32x4*)&x_lds[b_base + j * 16 * PITCH + ks * 32];
+#pragma unroll
+      for (int i = 0; i < WR; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) acc[i][j] = mfma16x16x32<T>(a[i], b[j], acc[i][j]);
+    }
+  }
+
+  // ---- per-token rsqrt(mean(x^2) + eps): every thread adds the squares it staged to its tokens
+  if constexpr (NORM) {
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) atomicAdd(&rs_lds[(t + kPfThreads * i) / CPR], ss[i]);
+    __syncthreads();
+    if (t < TOKS) rs_lds[t] = rsqrtf(rs_lds[t] / (float)p.k + p.eps);
+    __syncthreads();
+  }
+
+  // ---- epilogue. acc[i][j][e]: token t0 + 16 WT wt + 16 j + lane % 16, local row 16 WR wr + 16 i +
+  // 4 (lane / 16) + e
+  const int tok_l = wt * 16 * WT + (lane & 15);
+  const int sub = (lane >> 4) * 4;
+  constexpr int OT = (EPI == SK_GATEUP) ? WR / 2 : WR;  // output row tiles per wave
+#pragma unroll
+  for (int j = 0; j < WT; ++j) {
+    const int tl = tok_l + 16 * j;
+    const int tok = t0 + tl;
+    if (tok >= p.tokens) continue;
+    const float rs = NORM ? rs_lds[tl] : 1.f;
+#pragma unroll
+    for (int i = 0; i < OT; ++i) {
+      const int o = o0 + wr * 16 * OT + 16 * i + sub;
+      if (o >= p.n) continue;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int oe = o + e < p.n ? o + e : p.n - 1;
+        if constexpr (EPI == SK_GATEUP) {
+          float g = acc[i][j][e] * rs, u = acc[i + OT][j][e] * rs;
+          if constexpr (WF == WF_I8_CHANNEL) {
+            g *= T::one(p.s0[(long)oe * p.s_pitch]);
+            u *= T::one(p.s1[(long)oe * p.s_pitch]);
+          }
+          v[e] = silu_f32(g) * u;
+        } else {
+          float r = acc[i][j][e] * rs;
+          if constexpr (WF == WF_I8_CHANNEL) r *= T::one(p.s0[(long)oe * p.s_pitch]);
+          if (p.mul_bias) r *= T::one(p.mul_bias[oe]);
+          if (p.add_bias) r += T::one(p.add_bias[oe]);
+          if (p.residual) r += T::one(p.residual[(long)tok * p.n + oe]);
+          v[e] = r;
+        }
+      }
+      uint16_t* dst = p.y + (long)tok * p.n + o;
+      if (o + 3 < p.n && (p.n & 3) == 0) {
+        u32x2 pk;
+        pk.x = (uint32_t)T::pack(v[0]) | ((uint32_t)T::pack(v[1]) << 16);
+        pk.y = (uint32_t)T::pack(v[2]) | ((uint32_t)T::pack(v[3]) << 16);
+        *(u32x2*)dst = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (o + e < p.n) dst[e] = T::pack(v[e]);
+      }
+    }
+  }
+}
+
+static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64
+
+template <typename T, int WF, int EPI, int WR, int WT, int KS>
+static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
+  constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
+  p.n_tiles = ceil_div(p.n, EPI == SK_GATEUP ? ROWS / 2 : ROWS);
+  p.t_tiles = ceil_div(p.tokens, TOKS);
+  // whole row tiles per XCD: the grid covers ceil(n_tiles / 8) * 8 row tiles, the surplus exits
+  const long grid = (long)ceil_div(p.n_tiles, 8) * 8 * p.t_tiles;
+  if (grid > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
+  if (p.gamma)
+    hipLaunchKernelGGL((prefill_gemm_kernel<T, WF, true, EPI, WR, WT, KS>), dim3((int)grid), dim3(kPfThreads), 0, s, p);
+  else
+    hipLaunchKernelGGL((prefill_gemm_kernel<T, WF, false, EPI, WR, WT, KS>), dim3((int)grid), dim3(kPfThreads), 0, s, p);
+  return launch_status();
+}
+
+template <typename T, int WF, int EPI>
+static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
+  // The largest tile that still yields a workgroup per CU: big tiles re-read x and the weights
+  // least, but a grid smaller than the chip leaves the weight stream to too few CUs (measured on
+  // the Llama-3-8B shapes: 32 x 64 wins up to 256 tokens on the 4096-row matrices, 64 x 128 at
+  // 512, 128 x 128 from 2048; the 28672 gate/up rows take 64 x 128 up to 128 tokens, then 128 x 128).
+  const long rows = (EPI == SK_GATEUP) ? 2L * p.n : p.n;
+  const long want = device_cus();
+  auto tiles = [&](int r, int tk) { return (long)ceil_div((int)rows, r) * ceil_div(p.tokens, tk); };
+  int which = g_prefill_tile;
+  if (which == 0) which = tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
+  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 64>(s, p);
+  if constexpr (EPI == SK_GATEUP) {
+    return launch_prefill_cfg<T, WF, EPI, 2, 4, 128>(s, p);
+  } else {
+    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 128>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 1, 2, 256>(s, p);
+  }
+}
+
+constexpr int kWideDefaultMaxTokens = 0;  // 0: the built-in rule below
+static int g_wide_max_tokens = kWideDefaultMaxTokens;  // longest prompt taken by gemm_wide.hip
+
+// Any number of tokens >= 1 (meant for more than MUI_MAX_TOKENS), 16-bit weights or per-channel
+// int8 codes; SkinnyParams as for the decode kernels (x, residual and y dense).
+int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const SkinnyParams& q) {
+  if (q.tokens < 1 || q.n < 1 || q.k < 1) return MUI_ERR_INVALID_ARG;
+  // short prompts are bound by the weight stream: few rows per workgroup, K split over the waves,
+  // no LDS tiling (gemm_wide.hip)
+  // (gemm_wide.hip); it wins while its grid is a single round of workgroups and the token tiles few
+  const bool wide_default = q.tokens <= 64 && epilogue == SK_LINEAR && ceil_div(q.n, 16) <= device_cus();
+  if (g_wide_max_tokens == kWideDefaultMaxTokens ? wide_default : q.tokens <= g_wide_max_tokens)
+    return launch_gemm_wide(s, dtype, wf, epilogue, q);
+  if (!(wf == WF_16BIT || wf == WF_I8_CHANNEL)) return MUI_ERR_UNSUPPORTED;
+  if (q.k % (wf == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
+  if (q.x_pitch != 0 && q.x_pitch != q.k) return MUI_ERR_UNSUPPORTED;
+  PrefillGemmParams p = {};
+  const long esz = (wf == WF_16BIT) ? 2 : 1;
+  p.w0 = (const uint8_t*)q.w0; p.w1 = (const uint8_t*)q.w1; p.pitch = q.pitch * esz;
+  p.s0 = q.s0; p.s1 = q.s1; p.s_pitch = q.s_pitch;
+  p.x = q.x; p.gamma = q.gamma; p.mul_bias = q.mul_bias; p.add_bias = q.add_bias; p.residual = q.residual;
+  p.y = q.y; p.n = q.n; p.k = q.k; p.tokens = q.tokens; p.eps = q.eps;
+#define MUI_PF_CASE(TT, WFV, EPIV) \
+  if (dtype == TT::kDtype && wf == WFV && epilogue == EPIV) return launch_prefill_t<TT, WFV, EPIV>(s, p);
+  MUI_PF_CASE(F16, WF_16BIT, SK_LINEAR)
+  MUI_PF_CASE(F16, WF_16BIT, SK_GATEUP)
+  MUI_PF_CASE(F16, WF_I8_CHANNEL, SK_LINEAR)
+  MUI_PF_CASE(F16, WF_I8_CHANNEL, SK_GATEUP)
+  MUI_PF_CASE(BF16, WF_16BIT, SK_LINEAR)
+  MUI_PF_CASE(BF16, WF_16BIT, SK_GATEUP)
+  MUI_PF_CASE(BF16, WF_I8_CHANNEL, SK_LINEAR)
+  MUI_PF_CASE(BF16, WF_I8_CHANNEL, SK_GATEUP)
+#undef MUI_PF_CASE
+  return MUI_ERR_INVALID_ARG;
+}
+
+}  // namespace mui
+
+extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
+  if (tile < 0 || tile > 3 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_tile = tile;
+  mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
+  return MUI_OK;
+}

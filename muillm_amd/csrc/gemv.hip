@@ -308,13 +308,20 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
   MUI_CHECK_ARG(weights && x && y);
   MUI_CHECK_ARG(n_out > 0 && k_in > 0 && tokens > 0);
   MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
-  if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
   if (w_pitch < k_in) return MUI_ERR_INVALID_ARG;
   if ((k_in & 7) || (w_pitch & 7)) return MUI_ERR_UNSUPPORTED;
   if (!aligned16(weights) || !aligned16(x) || (norm_weights && !aligned16(norm_weights)))
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
+  if (tokens > MUI_MAX_TOKENS) {  // a prompt: the tiled matrix-core GEMM
+    SkinnyParams sp = {};
+    sp.w0 = weights; sp.pitch = w_pitch; sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.mul_bias = (const uint16_t*)mul_bias; sp.add_bias = (const uint16_t*)add_bias;
+    sp.residual = (const uint16_t*)residual; sp.y = (uint16_t*)y; sp.n = n_out; sp.k = k_in; sp.tokens = tokens;
+    sp.eps = epsilon;
+    return launch_prefill_gemm(s, dtype, WF_16BIT, SK_LINEAR, sp);
+  }
   if (tokens >= g_skinny_min_tokens || g_gemv_dot2) {
     SkinnyParams sp = {};
     sp.w0 = weights;
@@ -362,7 +369,6 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
   MUI_CHECK_ARG(gate && up && x && h);
   MUI_CHECK_ARG(n_inter > 0 && k_in > 0 && tokens > 0);
   MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
-  if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
   if (gu_pitch < k_in) return MUI_ERR_INVALID_ARG;
   if ((k_in & 7) || (gu_pitch & 7)) return MUI_ERR_UNSUPPORTED;
   if (!aligned16(gate) || !aligned16(up) || !aligned16(x) ||
@@ -370,6 +376,13 @@ extern "C" int mui_gateup_silu(mui_stream_t stream, int dtype, const void* gate,
     return MUI_ERR_ALIGNMENT;
 
   hipStream_t s = (hipStream_t)stream;
+  if (tokens > MUI_MAX_TOKENS) {  // a prompt: the tiled matrix-core GEMM
+    SkinnyParams sp = {};
+    sp.w0 = gate; sp.w1 = up; sp.pitch = gu_pitch; sp.x = (const uint16_t*)x;
+    sp.gamma = (const uint16_t*)norm_weights; sp.y = (uint16_t*)h; sp.n = n_inter; sp.k = k_in;
+    sp.tokens = tokens; sp.eps = epsilon;
+    return launch_prefill_gemm(s, dtype, WF_16BIT, SK_GATEUP, sp);
+  }
   // bf16 has no mixed-precision fma: a single bf16 token takes the packed-dot kernel here too
   if (tokens >= g_skinny_min_tokens || (g_gemv_dot2 && dtype == MUI_DTYPE_BF16)) {
     SkinnyParams sp = {};

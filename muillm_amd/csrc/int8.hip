@@ -323,7 +323,7 @@ template <typename T, int EPI, int FMT>
 static int launch8_t(hipStream_t s, const Int8Params& p) {
   const int ch = ceil_div(p.k >> 4, kThreads8);
   int rows = g_int8_rows;
-  if (rows == 0) rows = ch > 1 ? 4 : 8;
+  if (rows == 0 || rows == 16) rows = ch > 1 ? 4 : 8;
   if (rows == 8 && ch == 1) return launch8_r<T, 8, EPI, FMT>(s, p, ch);
   if (rows >= 4 && ch <= 2) return launch8_r<T, 4, EPI, FMT>(s, p, ch);
   return launch8_r<T, 2, EPI, FMT>(s, p, ch);
@@ -337,11 +337,11 @@ static int launch8(hipStream_t s, int dtype, const Int8Params& p) {
 }
 
 static int check_int8_common(int dtype, const void* w, long pitch, const void* x,
-                             const void* gamma, int n, int k, int tokens) {
+                             const void* gamma, int n, int k, int tokens, bool any_token_count = false) {
   if (!(w && x)) return MUI_ERR_INVALID_ARG;
   if (!(n > 0 && k > 0 && tokens > 0)) return MUI_ERR_INVALID_ARG;
   if (!(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16)) return MUI_ERR_INVALID_ARG;
-  if (tokens > MUI_MAX_TOKENS) return MUI_ERR_UNSUPPORTED;
+  if (tokens > MUI_MAX_TOKENS && !any_token_count) return MUI_ERR_UNSUPPORTED;
   if (pitch < k) return MUI_ERR_INVALID_ARG;
   if ((k & 15) || (pitch & 15)) return MUI_ERR_UNSUPPORTED;
   if (!aligned16(w) || !aligned16(x) || (gamma && !aligned16(gamma))) return MUI_ERR_ALIGNMENT;
@@ -355,10 +355,11 @@ using namespace mui;
 namespace mui {
 void int8_set_packed_dot(bool on) { g_int8_dot2 = on ? 1 : 0; }
 int int8_tuned_wgs_per_cu() { return g_int8_wgs_per_cu; }
+int int8_tuned_rows() { return g_int8_rows; }
 }  // namespace mui
 
 extern "C" int mui_tune_int8(int rows, int wgs_per_cu) {
-  if (!(rows == 0 || rows == 2 || rows == 4 || rows == 8)) return MUI_ERR_INVALID_ARG;
+  if (!(rows == 0 || rows == 2 || rows == 4 || rows == 8 || rows == 16)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_int8_rows = rows;
   g_int8_wgs_per_cu = wgs_per_cu;
@@ -369,10 +370,18 @@ extern "C" int mui_int8_linear(mui_stream_t stream, int dtype, const void* weigh
                                const void* scales, const void* x, const void* norm_weights,
                                float epsilon, const void* add_bias, const void* residual, void* y,
                                int n_out, int k_in, int tokens) {
-  int st = check_int8_common(dtype, weights_i8, w_pitch, x, norm_weights, n_out, k_in, tokens);
+  int st = check_int8_common(dtype, weights_i8, w_pitch, x, norm_weights, n_out, k_in, tokens, true);
   if (st != MUI_OK) return st;
   MUI_CHECK_ARG(scales && y);
   hipStream_t s = (hipStream_t)stream;
+  if (tokens > MUI_MAX_TOKENS) {  // a prompt: the tiled matrix-core GEMM, codes converted on the way to LDS
+    SkinnyParams sp = {};
+    sp.w0 = weights_i8; sp.pitch = w_pitch; sp.s0 = (const uint16_t*)scales; sp.s_pitch = 1;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.add_bias = (const uint16_t*)add_bias; sp.residual = (const uint16_t*)residual;
+    sp.y = (uint16_t*)y; sp.n = n_out; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_prefill_gemm(s, dtype, WF_I8_CHANNEL, SK_LINEAR, sp);
+  }
   if (tokens >= 2 || (g_int8_dot2 && dtype == MUI_DTYPE_F16)) {
     SkinnyParams sp = {};
     sp.w0 = weights_i8; sp.pitch = w_pitch; sp.s0 = (const uint16_t*)scales; sp.s_pitch = 1;
@@ -406,11 +415,19 @@ extern "C" int mui_int8_gateup_silu(mui_stream_t stream, int dtype, const void* 
                                     const void* up_scales, long scale_stride, const void* x,
                                     const void* norm_weights, float epsilon, void* h, int n_inter,
                                     int k_in, int tokens) {
-  int st = check_int8_common(dtype, gate_i8, gu_pitch, x, norm_weights, n_inter, k_in, tokens);
+  int st = check_int8_common(dtype, gate_i8, gu_pitch, x, norm_weights, n_inter, k_in, tokens, true);
   if (st != MUI_OK) return st;
   MUI_CHECK_ARG(up_i8 && gate_scales && up_scales && h && scale_stride >= 1);
   if (!aligned16(up_i8)) return MUI_ERR_ALIGNMENT;
   hipStream_t s = (hipStream_t)stream;
+  if (tokens > MUI_MAX_TOKENS) {
+    SkinnyParams sp = {};
+    sp.w0 = gate_i8; sp.w1 = up_i8; sp.pitch = gu_pitch;
+    sp.s0 = (const uint16_t*)gate_scales; sp.s1 = (const uint16_t*)up_scales; sp.s_pitch = scale_stride;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.y = (uint16_t*)h; sp.n = n_inter; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_prefill_gemm(s, dtype, WF_I8_CHANNEL, SK_GATEUP, sp);
+  }
   if (tokens >= 2 || (g_int8_dot2 && dtype == MUI_DTYPE_F16)) {
     SkinnyParams sp = {};
     sp.w0 = gate_i8; sp.w1 = up_i8; sp.pitch = gu_pitch;

@@ -278,6 +278,12 @@ static int launch_i8m_t(hipStream_t s, const SkinnyParams& p) {
   const int ch = ceil_div(p.k >> 4, kI8mThreads);
   const int per_cu = int8_tuned_wgs_per_cu();
   if (ch <= 1) {
+    if constexpr (TOK == 1) {
+      if (int8_tuned_rows() == 16) {
+        constexpr int R = 16, OUT = (EPI == SK_GATEUP) ? R / 2 : R;
+        return launch_i8m_rc<R, 1, EPI, WF, TOK>(s, p, balanced_grid(ceil_div(p.n, OUT), per_cu > 0 ? per_cu : 2));
+      }
+    }
     // short rows: 8 rows in flight at 2 tokens, 4 at 4 (at most 32 partial sums per group)
     constexpr int R = (TOK <= 2) ? 8 : 4;
     constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;

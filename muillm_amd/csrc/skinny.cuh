@@ -119,6 +119,10 @@ __device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint1
   }
 }
 
+// tiled matrix-core GEMM for prompts (gemm_prefill.hip): any token count, 16-bit or per-channel int8
+int launch_prefill_gemm(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
+// 17..128 tokens: 16 weight rows per workgroup, K split over its waves, token columns in up to 8 MFMA tiles (gemm_wide.hip)
+int launch_gemm_wide(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 // launches gemm_skinny_kernel<dtype, weight format, epilogue>; returns a MUI_* status
 int launch_skinny(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 // experiments: 0 disables the B-stationary persistent variant
@@ -132,6 +136,7 @@ int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams
 // through wave-private LDS (gemm_skinny_lt.hip); MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_skinny_lt(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 int int8_tuned_wgs_per_cu();  // mui_tune_int8's workgroups-per-CU override (0 = built-in)
+int int8_tuned_rows();        // mui_tune_int8's rows-per-group override (0 = built-in)
 int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 = built-in)
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);

@@ -7,11 +7,12 @@ muillm_amd.modules read like the reference's, but every function here only valid
 tensors, allocates the output with torch and hands raw device pointers plus the current HIP
 stream to libmuillm_amd.so.
 
-Dispatch rule (csrc/modules/linear_module.cpp:39-80): the fused kernels serve 16-bit CUDA
-tensors holding 1..MUI_MAX_TOKENS tokens (up to FUSED_CHUNK_MAX_TOKENS in chunks); anything else
-(longer prefill, fp32) takes the
-reference's own unfused route -- RMSNorm kernel, torch matmul, residual add -- on the same
-device.  There is no CPU fallback for CUDA inputs and no silent one for a missing library.
+Dispatch rule (csrc/modules/linear_module.cpp:39-80 hands everything but a single token to the
+framework's GEMM): here the library's kernels serve 16-bit CUDA tensors of any token count --
+1..MUI_MAX_TOKENS tokens the weight-streaming decode kernels (up to FUSED_CHUNK_MAX_TOKENS in
+chunks), longer prompts the tiled matrix-core GEMM behind the same entry points. Only fp32 and CPU
+tensors take the reference's unfused route (RMSNorm, torch matmul, residual add).  There is no
+CPU fallback for CUDA inputs and no silent one for a missing library.
 """
 
 from __future__ import annotations
@@ -69,6 +70,9 @@ def _num_tokens(x: torch.Tensor) -> int:
     return x.numel() // x.shape[-1]
 
 
+_MAX_CALL_TOKENS = 1 << 20  # tokens one library call may carry (a sanity bound, not a kernel limit)
+
+
 def _check_activations(x: torch.Tensor, k: int, what: str, max_tokens: int, *others) -> None:
     """What every fused entry point needs of its operands before raw pointers go to a kernel: a
     16-bit CUDA activation tensor with k features and a token count the kernels take, and every
@@ -87,17 +91,23 @@ def _check_activations(x: torch.Tensor, k: int, what: str, max_tokens: int, *oth
             raise RuntimeError(f"{what}: every operand must live on the activations' device {x.device}")
 
 
-# Short prompts: up to this many tokens go through the fused kernels in chunks of MUI_MAX_TOKENS
-# (each chunk reads the weights once more, which still beats norm + library GEMM + add for a few
-# chunks: a Llama-3-8B-shaped model prefills 32 tokens in 6.3 ms against 8.4 ms; from a third chunk
-# on the library GEMM wins, 9.0 against 8.3 ms at 40 tokens).
+# Short prompts: up to this many tokens go through the decode kernels in chunks of MUI_MAX_TOKENS
+# (each chunk streams the weights once more with the GEMVs' long contiguous runs); longer ones take
+# the tiled matrix-core GEMM of the same entry points in one call (weights read once per 128 tokens).
 FUSED_CHUNK_MAX_TOKENS = 32
 
 
 def kernel_dispatchable(x: torch.Tensor) -> bool:
-    """True when the fused decode kernels take this input (in chunks beyond MUI_MAX_TOKENS)."""
-    return (x.is_cuda and _is_16bit(x) and 1 <= _num_tokens(x) <= max(MUI_MAX_TOKENS, FUSED_CHUNK_MAX_TOKENS)
-            and x.shape[-1] % 8 == 0)
+    """True when the library's kernels take this input: any number of 16-bit CUDA tokens."""
+    return x.is_cuda and _is_16bit(x) and _num_tokens(x) >= 1 and x.shape[-1] % 8 == 0
+
+
+def _token_calls(tokens: int, chunk_max: int):
+    """(first token, count) of the library calls that cover `tokens` rows: chunks of MUI_MAX_TOKENS
+    for the decode kernels up to chunk_max tokens, one call (the tiled GEMM) beyond."""
+    if tokens > chunk_max:
+        return [(0, tokens)]
+    return [(off, min(MUI_MAX_TOKENS, tokens - off)) for off in range(0, tokens, MUI_MAX_TOKENS)]
 
 
 # --------------------------------------------------------------------------------------
@@ -197,9 +207,10 @@ def muillm_linear_forward(
 
     if not (kernel_dispatchable(x) and weights.dtype == x.dtype):
         return _linear_unfused(x, weights, norm_weights, epsilon, mul_bias, add_bias, residual)
-    if k > 16384 and norm_weights is not None and _num_tokens(x) == 1:
-        # a fused norm needs the whole row in one pass of the single-token kernel
-        return _linear_unfused(x, weights, norm_weights, epsilon, mul_bias, add_bias, residual)
+    if k > 16384 and norm_weights is not None and _num_tokens(x) <= FUSED_CHUNK_MAX_TOKENS:
+        # a fused norm needs the whole row in one pass of the 1..4-token kernels: norm kernel first
+        x = muillm_rmsnorm_forward(norm_weights, x, epsilon)
+        norm_weights = None
 
     _check_cuda(weights, "weights")
     pitch = _row_pitch(weights, "weights")
@@ -219,13 +230,13 @@ def muillm_linear_forward(
         residual = residual.contiguous()
     y = torch.empty(out_shape, dtype=x.dtype, device=x.device)
     lib, stream, code, esz = _lib.load(), _stream(x), _dtype_code(x), x.element_size()
-    for off in range(0, tokens, MUI_MAX_TOKENS):  # one call up to MUI_MAX_TOKENS, else chunks
+    for off, cnt in _token_calls(tokens, FUSED_CHUNK_MAX_TOKENS):
         check(
             lib.mui_linear(
                 stream, code, weights.data_ptr(), pitch, x.data_ptr() + off * k * esz,
                 _ptr(norm_weights), float(epsilon), _ptr(mul_bias), _ptr(add_bias),
                 None if residual is None else residual.data_ptr() + off * n * esz,
-                y.data_ptr() + off * n * esz, n, k, min(MUI_MAX_TOKENS, tokens - off),
+                y.data_ptr() + off * n * esz, n, k, cnt,
             ),
             "mui_linear",
         )
@@ -272,8 +283,7 @@ def mui_gateup_silu(norm_weights, epsilon, gate_weights, up_weights, x) -> torch
     pitch = _row_pitch(gate_weights, "gate_weights")
     if _row_pitch(up_weights, "up_weights") != pitch:
         raise RuntimeError("gate and up weights must share one row pitch")
-    _check_activations(x, k, "mui_gateup_silu", max(MUI_MAX_TOKENS, FUSED_CHUNK_MAX_TOKENS), gate_weights,
-                       up_weights, norm_weights)
+    _check_activations(x, k, "mui_gateup_silu", _MAX_CALL_TOKENS, gate_weights, up_weights, norm_weights)
     if gate_weights.dtype != x.dtype or up_weights.dtype != x.dtype or \
             (norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k)):
         raise RuntimeError("mui_gateup_silu: weights and norm weights must have the activations' dtype "
@@ -282,12 +292,12 @@ def mui_gateup_silu(norm_weights, epsilon, gate_weights, up_weights, x) -> torch
     tokens = _num_tokens(x)
     h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
     lib, stream, code, esz = _lib.load(), _stream(x), _dtype_code(x), x.element_size()
-    for off in range(0, tokens, MUI_MAX_TOKENS):  # one call up to MUI_MAX_TOKENS, else chunks
+    for off, cnt in _token_calls(tokens, FUSED_CHUNK_MAX_TOKENS):
         check(
             lib.mui_gateup_silu(
                 stream, code, gate_weights.data_ptr(), up_weights.data_ptr(), pitch,
                 x.data_ptr() + off * k * esz, _ptr(norm_weights), float(epsilon),
-                h.data_ptr() + off * n * esz, n, k, min(MUI_MAX_TOKENS, tokens - off),
+                h.data_ptr() + off * n * esz, n, k, cnt,
             ),
             "mui_gateup_silu",
         )
@@ -309,7 +319,7 @@ def muillm_gateupsilu_forward(engine, norm_weights, epsilon, gate_weights, up_we
                               residual, x) -> torch.Tensor:
     """out = Wd (silu(Wg xn) * (Wu xn)) + residual, argument order of csrc/module.cpp:182."""
     if not (kernel_dispatchable(x) and gate_weights.dtype == x.dtype):
-        raise RuntimeError("muillm_gateupsilu_forward needs a 16-bit CUDA tensor of at most %d tokens" % max(MUI_MAX_TOKENS, FUSED_CHUNK_MAX_TOKENS))
+        raise RuntimeError("muillm_gateupsilu_forward needs fp16 / bf16 CUDA tensors with k % 8 == 0")
     h = mui_gateup_silu(norm_weights, epsilon, gate_weights, up_weights, x)
     return muillm_linear_forward(engine, h, down_weights, residual=residual)
 
@@ -332,22 +342,21 @@ def _byte_pitch(w: torch.Tensor, name: str) -> int:
     return w.stride(0) if w.shape[0] > 1 else max(w.stride(0), w.shape[1])
 
 
-# int8 weights: the alternative to chunks is dequantising the whole matrix for a library GEMM,
-# so chunks of MUI_MAX_TOKENS pay off for longer prompts than with 16-bit weights (an int8
-# Llama-3-8B-shaped model prefills 32 tokens in 5.7 ms against 10.4 ms, 64 in 8.9 against 10.3 ms,
-# 96 in 12.9 against 11.0 ms).
+# int8 weights: the decode kernels take chunks of MUI_MAX_TOKENS up to this many tokens; beyond, the
+# tiled matrix-core GEMM converts the codes on their way to LDS (per-channel format) or runs on the
+# matrix dequantised by the library's kernel (group format).
 INT8_CHUNK_MAX_TOKENS = 64
 
 
 def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
     # rows longer than 16384: fp16 activations only (K segments / the streaming matrix-core kernel)
-    return x.is_cuda and _is_16bit(x) and 1 <= _num_tokens(x) <= max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS) \
+    return x.is_cuda and _is_16bit(x) and _num_tokens(x) >= 1 \
         and x.shape[-1] % 16 == 0 and (x.shape[-1] <= 16384 or x.dtype == torch.float16)
 
 
 def _token_chunks(tokens: int):
-    """(first token, count) of the calls that cover `tokens` rows, MUI_MAX_TOKENS at a time."""
-    return [(off, min(MUI_MAX_TOKENS, tokens - off)) for off in range(0, tokens, MUI_MAX_TOKENS)]
+    """(first token, count) of the int8 calls that cover `tokens` rows."""
+    return _token_calls(tokens, INT8_CHUNK_MAX_TOKENS)
 
 
 def mui_int8_channel_dequantize_forward(weights_i8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
@@ -411,7 +420,7 @@ def mui_int8_channel_gateupsilu_forward(norm_weights, epsilon, gate_i8, up_i8, g
     sstride = gate_scales.stride(0) if gate_scales.numel() > 1 else 1
     if (up_scales.stride(0) if up_scales.numel() > 1 else 1) != sstride:
         raise RuntimeError("gate and up scales must share one stride")
-    _check_activations(x, k, "mui_int8_channel_gateupsilu_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS),
+    _check_activations(x, k, "mui_int8_channel_gateupsilu_forward", _MAX_CALL_TOKENS,
                        gate_i8, up_i8, gate_scales, up_scales, norm_weights)
     if not int8_kernel_dispatchable(x):
         raise RuntimeError("mui_int8_channel_gateupsilu_forward: the int8 kernels need k % 16 == 0 "
@@ -468,8 +477,13 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
     if weights.dtype != torch.uint8:
         raise RuntimeError("group-quantised weights must be uint8")
     _check_contiguous(scales_min_vals, "scales_min_vals")
-    _check_activations(x, k, "muillm_int8_linear_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS), weights,
+    _check_activations(x, k, "muillm_int8_linear_forward", _MAX_CALL_TOKENS, weights,
                        scales_min_vals, norm_weights, add_bias, residual)
+    if _num_tokens(x) > INT8_CHUNK_MAX_TOKENS:
+        # a prompt: the reference's route (dequantise the matrix, then a GEMM,
+        # muillm/modules/quantized/int8linear.py:279-293) on this library's kernels
+        w = muillm_int8_dequantize_forward(weights, scales_min_vals, group_size_shift)
+        return muillm_linear_forward(None, x, w, norm_weights, epsilon, None, add_bias, residual)
     if scales_min_vals.dtype != x.dtype or scales_min_vals.numel() != 2 * n * (k >> group_size_shift):
         raise RuntimeError("scales_min_vals must be [N * K / group, 2] (scale, min) pairs in the activation dtype")
     if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
@@ -558,7 +572,7 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
                                                                        group_size_shift)
     n, two, k = gate_up_weights.shape
     g = k >> group_size_shift
-    _check_activations(x, k, "muillm_int8_gateupsilu_forward", max(MUI_MAX_TOKENS, INT8_CHUNK_MAX_TOKENS),
+    _check_activations(x, k, "muillm_int8_gateupsilu_forward", _MAX_CALL_TOKENS,
                        gate_up_weights, gate_up_scales_min_vals, norm_weights)
     if not int8_kernel_dispatchable(x) or group_size_shift < 4:
         raise RuntimeError("muillm_int8_gateupsilu_forward: the int8 kernels need k % 16 == 0 and groups of >= 16")
@@ -569,6 +583,10 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
         raise RuntimeError("gate_up_scales_min_vals must hold N * 2 * K / group (scale, min) pairs in the activation dtype")
     if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
         raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
+    if _num_tokens(x) > INT8_CHUNK_MAX_TOKENS:
+        # a prompt: dequantise gate and up once, then the tiled GEMM with the SiLU * mul epilogue
+        gd, ud = muillm_int8_gateupsilu_dequantize_forward(gate_up_weights, gate_up_scales_min_vals, group_size_shift)
+        return mui_gateup_silu(norm_weights, epsilon, gd, ud, x)
     smv = gate_up_scales_min_vals.reshape(n, 2, g, 2)
     x = x.contiguous()
     tokens = _num_tokens(x)

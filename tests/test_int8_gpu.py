@@ -251,7 +251,9 @@ def test_channel_linear_and_gateup_in_chunks(tokens):
                                                        su.to(DEV), x.to(DEV))
     ref_h = oracle.gateup_silu(x, oracle.rtn_dequantize_channel(qg, sg), oracle.rtn_dequantize_channel(qu, su), gamma, 1e-5)
     assert_parity(h, ref_h, 1e-2, f"int8 gate/up chunks {tokens}")
-    assert not muillm_ext.int8_kernel_dispatchable(torch.zeros(65, k, dtype=torch.float16, device=DEV))
+    # longer prompts stay on the library's kernels too (the tiled GEMM of the same entry points)
+    assert muillm_ext.int8_kernel_dispatchable(torch.zeros(65, k, dtype=torch.float16, device=DEV))
+    assert muillm_ext._token_chunks(64) == [(0, 16), (16, 16), (32, 16), (48, 16)] and muillm_ext._token_chunks(65) == [(0, 65)]
 
 
 def test_wrappers_refuse_mismatched_operands():
@@ -269,7 +271,7 @@ def test_wrappers_refuse_mismatched_operands():
     with pytest.raises(RuntimeError, match="dtype"):
         muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd.bfloat16(), sd.bfloat16(), x)
     with pytest.raises(RuntimeError, match="tokens"):
-        muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd, sd, _mk((100, k), g).to(DEV))
+        muillm_ext.mui_int8_channel_gateupsilu_forward(None, 0.0, qd, qd, sd, sd, torch.zeros(0, k, dtype=torch.float16, device=DEV))
     qu, smv = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), 128)
     qu, smv = qu.to(DEV), smv.to(DEV)
     with pytest.raises(RuntimeError, match="dtype"):
@@ -279,7 +281,7 @@ def test_wrappers_refuse_mismatched_operands():
     with pytest.raises(RuntimeError, match="features"):
         muillm_ext.muillm_int8_gateupsilu_forward(None, 0.0, packed, psmv, 7, x[:, : k - 16])
     with pytest.raises(RuntimeError, match="tokens"):
-        muillm_ext.muillm_int8_gateupsilu_forward(None, 0.0, packed, psmv, 7, _mk((100, k), g).to(DEV))
+        muillm_ext.muillm_int8_gateupsilu_forward(None, 0.0, packed, psmv, 7, torch.zeros(0, k, dtype=torch.float16, device=DEV))
     w = _mk((n, k), g, 0.02).to(DEV)
     with pytest.raises(RuntimeError, match="features"):
         muillm_ext.mui_gateup_silu(None, 0.0, w, w, x[:, : k - 8])

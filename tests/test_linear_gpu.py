@@ -238,7 +238,7 @@ def test_linear_abi_errors():
     assert lib.mui_linear(s, 0, None, 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 1) == -1
     assert lib.mui_linear(s, 7, w.data_ptr(), 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 1) == -1
     assert lib.mui_linear(s, 0, w.data_ptr(), 12, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 12, 1) == -2
-    assert lib.mui_linear(s, 0, w.data_ptr(), 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 17) == -2
+    assert lib.mui_linear(s, 0, w.data_ptr(), 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 8, 16, 0) == -1
     assert lib.mui_linear(s, 0, w.data_ptr() + 2, 16, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), 4, 8, 1) == -4
     assert b"aligned" in lib.mui_status_string(-4)
     with pytest.raises(RuntimeError):
@@ -400,4 +400,7 @@ def test_short_prompt_goes_through_the_fused_kernels_in_chunks(tokens):
     packed = torch.stack((wg, wu), dim=1).to(DEV)
     h = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, packed[:, 0], packed[:, 1], x.to(DEV))
     assert_parity(h, oracle.gateup_silu(x, wg, wu, gamma, 1e-5), 1e-2, f"chunked gate/up {tokens}")
-    assert not muillm_ext.kernel_dispatchable(torch.zeros(33, k, dtype=torch.float16, device=DEV))
+    # longer prompts stay on the library's kernels too (the tiled GEMM of the same entry points)
+    assert muillm_ext.kernel_dispatchable(torch.zeros(33, k, dtype=torch.float16, device=DEV))
+    assert muillm_ext._token_calls(32, 32) == [(0, 16), (16, 16)] and muillm_ext._token_calls(33, 32) == [(0, 33)]
+    assert not muillm_ext.kernel_dispatchable(torch.zeros(33, k, dtype=torch.float32, device=DEV))

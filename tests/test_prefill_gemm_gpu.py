@@ -1,0 +1,197 @@
+"""GPU parity of the linear entry points at prompt sizes (more than MUI_MAX_TOKENS tokens): the
+tiled matrix-core GEMM with fused RMSNorm prologue and residual / bias / SiLU*mul epilogues, for
+16-bit weights and int8 weights, against the CPU oracle.
+
+The reference hands these calls to the framework's GEMM (csrc/modules/linear_module.cpp:57-79);
+its own tests compare batch-4 layers with HuggingFace at allclose(rtol 1e-4, atol 1e-1)
+(tests/test_linear.py, tests/test_gateupdownmlp.py there).  Gate here: the fp16/bf16 output
+gate of the decode kernels (max error over max |ref| <= 1e-2 fp16 / 2e-2 bf16, elementwise form
+included), plus that reference tolerance."""
+
+import functools
+
+import pytest
+import torch
+
+import oracle
+from muillm_amd import _lib, muillm_ext
+from tests.util import assert_parity, reference_allclose
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(params=["auto", "wide", "tile-128x128", "tile-64x128", "tile-32x64"], autouse=True)
+def prompt_kernel_choice(request):
+    """Every test runs with the built-in kernel choice and with each prompt kernel forced: the
+    16-rows-per-workgroup kernel without LDS tiling (up to 128 tokens; longer prompts keep the
+    built-in choice) and the three shapes of the LDS-tiled kernel (the gate/up epilogue has no
+    32 x 64 shape and takes 64 x 128 then)."""
+    lib = _lib.load()
+    knobs = {"auto": (0, 0), "wide": (0, 128), "tile-128x128": (1, -1), "tile-64x128": (2, -1), "tile-32x64": (3, -1)}
+    _lib.check(lib.mui_tune_prefill(*knobs[request.param]), "mui_tune_prefill")
+    yield request.param
+    _lib.check(lib.mui_tune_prefill(0, 0), "mui_tune_prefill")
+
+
+@functools.lru_cache(maxsize=64)
+def _oracle_linear_case(tokens, n, k, norm, res, bias):
+    """Seeded inputs and the oracle's result, shared by the runs of a case under each kernel choice."""
+    g = _gen(0)
+    w = _mk((n, k), g, 0.02)
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0) if norm else None
+    r = _mk((tokens, n), g) if res else None
+    b = _mk((n,), g, 0.5) if bias else None
+    return w, x, gamma, r, b, oracle.linear(x, w, gamma, 1e-5, b, r)
+
+
+def _gen(seed):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def _mk(shape, g, std=1.0, mean=0.0, dtype=torch.float16):
+    return (mean + std * torch.randn(shape, generator=g)).to(dtype)
+
+
+@pytest.mark.parametrize("tokens", [33, 64, 128, 512])
+@pytest.mark.parametrize("n,k,norm,res,bias", [
+    (4096, 4096, True, True, False),     # config 1 as a prompt
+    (6144, 4096, True, False, False),    # fused QKV
+    (4096, 14336, False, True, False),   # down projection
+    (1000, 2056, True, True, True),      # rows not a multiple of the tile, K not a multiple of the step
+    (130, 72, False, False, True),       # smaller than one tile / barely over one step
+    (33, 8, True, True, False),          # a single k-chunk, odd row count (scalar stores)
+])
+def test_linear_prompt(tokens, n, k, norm, res, bias):
+    if tokens == 512 and n * k > 4096 * 4096:
+        tokens = 300  # keeps the float64 oracle quick; still three token tiles with a ragged last one
+    w, x, gamma, r, b, ref = _oracle_linear_case(tokens, n, k, norm, res, bias)
+    y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), None if gamma is None else gamma.to(DEV), 1e-5,
+                                         None, None if b is None else b.to(DEV), None if r is None else r.to(DEV))
+    assert y.shape == (tokens, n)
+    assert_parity(y, ref, 1e-2, f"prompt linear {tokens}x{n}x{k}", tight=5e-3)
+    assert reference_allclose(y, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tokens", [33, 128, 257])
+def test_linear_prompt_mul_bias_and_bf16(tokens, dtype):
+    g = _gen(1)
+    n, k = 520, 1024
+    w, x = _mk((n, k), g, 0.02, dtype=dtype), _mk((2, tokens, k), g, dtype=dtype)   # [B, T, K] input
+    gamma, mb = _mk((k,), g, 0.1, 1.0, dtype=dtype), _mk((n,), g, 0.2, 1.0, dtype=dtype)
+    ab, r = _mk((n,), g, 0.5, dtype=dtype), _mk((2, tokens, n), g, dtype=dtype)
+    ref = (oracle.linear(x, w, gamma, 1e-5).double() * mb.double() + ab.double() + r.double())
+    y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), gamma.to(DEV), 1e-5, mb.to(DEV), ab.to(DEV), r.to(DEV))
+    assert y.shape == (2, tokens, n) and y.dtype == dtype
+    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 2e-2, f"prompt linear mul_bias {dtype}")
+
+
+@pytest.mark.parametrize("tokens", [33, 64, 128, 512])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (700, 520)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gateup_prompt(tokens, n, k, dtype):
+    if n * k > 4096 * 4096 and (dtype == torch.bfloat16 or tokens == 512):
+        tokens = min(tokens, 200)
+    g = _gen(2)
+    wg, wu = _mk((n, k), g, 0.02, dtype=dtype), _mk((n, k), g, 0.02, dtype=dtype)
+    x, gamma = _mk((tokens, k), g, dtype=dtype), _mk((k,), g, 0.1, 1.0, dtype=dtype)
+    ref = oracle.gateup_silu(x, wg, wu, gamma, 1e-5)
+    packed = torch.stack([wg, wu], dim=1).contiguous().to(DEV)   # the module's interleaved [N, 2, K] buffer
+    h = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, packed[:, 0], packed[:, 1], x.to(DEV))
+    # bf16: gamma * x is rounded to 8 significant bits before the matrix cores see it, and SiLU * mul
+    # multiplies two such results: 2.5e-2 on the max form, 4e-2 on the elementwise form
+    assert_parity(h, ref, 1e-2 if dtype == torch.float16 else 2.5e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype}",
+                  elementwise=None if dtype == torch.float16 else 4e-2)
+    h2 = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, wg.to(DEV), wu.to(DEV), x.to(DEV))  # two dense matrices
+    assert torch.equal(h, h2)
+
+
+def test_mlp_prompt_matches_chunked_decode_kernels():
+    """The whole MLP at 40 tokens: the tiled GEMM against the same call cut into 16-token chunks of
+    the decode kernels (two independent kernel families) and against the oracle."""
+    g = _gen(3)
+    hid, inter, tokens = 1024, 2816, 40
+    wg, wu, wd = _mk((inter, hid), g, 0.02), _mk((inter, hid), g, 0.02), _mk((hid, inter), g, 0.02)
+    x, r, gamma = _mk((tokens, hid), g), _mk((tokens, hid), g), _mk((hid,), g, 0.1, 1.0)
+    ref = oracle.gateupdown_mlp(x, wg, wu, wd, gamma, 1e-5, r)
+    args = (gamma.to(DEV), 1e-5, wg.to(DEV), wu.to(DEV), wd.to(DEV), r.to(DEV), x.to(DEV))
+    out = muillm_ext.muillm_gateupsilu_forward(None, *args)
+    old = muillm_ext.FUSED_CHUNK_MAX_TOKENS
+    try:
+        muillm_ext.FUSED_CHUNK_MAX_TOKENS = 64
+        chunked = muillm_ext.muillm_gateupsilu_forward(None, *args)
+    finally:
+        muillm_ext.FUSED_CHUNK_MAX_TOKENS = old
+    assert_parity(out, ref, 1e-2, "prompt MLP (tiled GEMM)")
+    assert_parity(chunked, ref, 1e-2, "prompt MLP (decode kernels in chunks)")
+    assert float((out.float() - chunked.float()).abs().max()) <= 2e-2
+
+
+@pytest.mark.parametrize("tokens", [65, 128, 300])
+@pytest.mark.parametrize("n,k", [(6144, 4096), (4096, 14336), (200, 528)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_int8_channel_linear_prompt(tokens, n, k, dtype):
+    g = _gen(4)
+    w = _mk((n, k), g, 0.02)
+    q, s = oracle.rtn_quantize_channel(w)
+    s = s.to(dtype)
+    x, gamma, r = _mk((tokens, k), g, dtype=dtype), _mk((k,), g, 0.1, 1.0, dtype=dtype), _mk((tokens, n), g, dtype=dtype)
+    wexact = q.double() * s.double()[:, None]
+    ref = oracle.linear(x, wexact, gamma, 1e-5, None, r)
+    y = muillm_ext.mui_int8_channel_linear_forward(x.to(DEV), q.to(DEV), s.to(DEV), gamma.to(DEV), 1e-5, None, r.to(DEV))
+    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 2e-2, f"int8 prompt linear {tokens}x{n}x{k} {dtype}")
+
+
+@pytest.mark.parametrize("tokens", [65, 200])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (136, 272)])
+def test_int8_channel_gateup_prompt(tokens, n, k):
+    g = _gen(5)
+    qg, sg = oracle.rtn_quantize_channel(_mk((n, k), g, 0.02))
+    qu, su = oracle.rtn_quantize_channel(_mk((n, k), g, 0.02))
+    x, gamma = _mk((tokens, k), g), _mk((k,), g, 0.1, 1.0)
+    ref = oracle.gateup_silu(x, qg.double() * sg.double()[:, None], qu.double() * su.double()[:, None], gamma, 1e-5)
+    pw = torch.stack([qg, qu], dim=1).contiguous().to(DEV)
+    ps = torch.stack([sg, su], dim=1).contiguous().to(DEV)
+    h = muillm_ext.mui_int8_channel_gateupsilu_forward(gamma.to(DEV), 1e-5, pw[:, 0], pw[:, 1], ps[:, 0], ps[:, 1], x.to(DEV))
+    assert_parity(h, ref, 1e-2, f"int8 prompt gate/up {tokens}x{n}x{k}")
+
+
+@pytest.mark.parametrize("tokens", [65, 150])
+def test_int8_group_format_prompt(tokens):
+    """The reference's group format at prompt sizes: dequantised by the library's kernel (bit-exact
+    definition), then the tiled GEMM -- the reference's own route (int8linear.py:279-293)."""
+    g = _gen(6)
+    n, k, gs = 1040, 1024, 128
+    qw, smv = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
+    x, gamma, r = _mk((tokens, k), g), _mk((k,), g, 0.1, 1.0), _mk((tokens, n), g)
+    wd = oracle.rtn_dequantize_group(qw, smv, gs)               # what the dequantisation kernel produces
+    ref = oracle.linear(x, wd, gamma, 1e-5, None, r)
+    y = muillm_ext.muillm_int8_linear_forward(x.to(DEV), qw.to(DEV), smv.to(DEV), 7, gamma.to(DEV), 1e-5,
+                                              residual=r.to(DEV))
+    assert_parity(y, ref, 1e-2, "group-format prompt linear")
+    qu, smu = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
+    pw = torch.stack([qw, qu], dim=1).contiguous().to(DEV)
+    ps = torch.stack([smv.reshape(n, -1, 2), smu.reshape(n, -1, 2)], dim=1).contiguous().to(DEV)
+    h = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, pw, ps, 7, x.to(DEV))
+    refh = oracle.gateup_silu(x, wd, oracle.rtn_dequantize_group(qu, smu, gs), gamma, 1e-5)
+    assert_parity(h, refh, 1e-2, "group-format prompt gate/up")
+
+
+def test_prompt_abi_direct_and_errors():
+    """Straight through the C ABI (ctypes): 48 tokens, and the argument checks of the tiled path."""
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    g = _gen(7)
+    n, k, tokens = 256, 512, 48
+    w, x, r = _mk((n, k), g, 0.02).to(DEV), _mk((tokens, k), g).to(DEV), _mk((tokens, n), g).to(DEV)
+    y = torch.zeros(tokens, n, dtype=torch.float16, device=DEV)
+    st = lib.mui_linear(s, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, r.data_ptr(), y.data_ptr(), n, k, tokens)
+    assert st == 0
+    assert_parity(y, oracle.linear(x.cpu(), w.cpu(), residual=r.cpu()), 1e-2, "ABI prompt linear")
+    assert lib.mui_linear(s, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), n, 12, tokens) == -2
+    assert lib.mui_linear(s, 0, w.data_ptr() + 2, k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), n, k, tokens) == -4
+    assert lib.mui_linear(s, 7, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), n, k, tokens) == -1
