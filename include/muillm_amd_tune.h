@@ -50,6 +50,10 @@ int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
  * built-in choice; at most 128; negative: never) */
 int mui_tune_prefill(int tile, int wide_max_tokens);
 
+/* Prompt attention (mui_prefill_attention): fewest query tokens that take the kernel sharing each
+ * K/V block between all query heads of a KV head (0 = built-in choice, negative = never) */
+int mui_tune_prefill_attention(int group_kernel_min_tokens);
+
 /* Measurement aid without a counterpart in the reference: reads `bytes` (a multiple of 16, from
  * a 16-byte aligned address) of device memory once with the access shape of the GEMV kernels and
  * discards them. One launch takes the least time any kernel that must read that many bytes can

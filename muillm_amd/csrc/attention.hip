@@ -858,6 +858,200 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Causal attention for long prompts: every K/V row that crosses LDS serves 32 query positions of
+// ALL query heads of its KV head.
+//
+// grid = (position tiles, Hkv, B), heaviest (last) position tile first. A workgroup has one wave
+// per (query head of the KV group, block of 32 query positions): NW = 4 waves for 1, 2 or 4 heads
+// per KV head (4, 2, 1 position blocks), 8 waves for 8. The workgroup walks the causal key range
+// in blocks of 64 tokens: all threads load the block's K and V rows in their natural layout (whole
+// 256-byte rows, the next block in flight while the current one is multiplied) into ONE LDS tile
+// pair that every wave reads -- K as MFMA A operands, V transposed with ds_read_b64_tr_b16, as
+// in attn_decode_mfma_kernel. Per 32 tokens a wave issues 32 MFMAs (two query tiles of 16
+// positions share each operand read), keeps its own online softmax (fp32, one rescale per 32
+// tokens) and needs no merge with other waves. K/V are read from HBM/L2 once per 32 query
+// positions of a KV head (attn_prefill_mfma_kernel: once per 16 positions of every query head).
+// The reference hands this case to torch SDPA after repeat_kv
+// (muillm/modules/attention/sdpaattention.py:221-245).
+// ---------------------------------------------------------------------------------------
+constexpr int kPgTok = 64;  // tokens per LDS block
+
+template <typename T, int G>
+__global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) attn_prefill_group_kernel(const PrefillParams p) {
+  constexpr int NW = (G == 8) ? 8 : 4;
+  constexpr int kThreads = NW * kWave;
+  constexpr int PB = NW / G;           // blocks of 32 query positions per workgroup
+  constexpr int POS = PB * 32;
+  constexpr int LCH = kPgTok * 16 / kThreads;  // 16-byte chunks of K (and of V) per thread and block
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[kPgTok][kMfKStride];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds[kPgTok][kMfVStride];
+
+  const int tile = gridDim.x - 1 - blockIdx.x;  // long key ranges first
+  const int kvh = blockIdx.y, b = blockIdx.z;
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  const int g = lane >> 4;
+  const int i = lane & 15;
+  const int head = kvh * G + (wave % G);
+  const int tpos = tile * POS + (wave / G) * 32;  // first query position of this wave
+
+  // keys the workgroup can see: [0, kv_end); query column i of tile qt sees tokens < limit[qt]
+  int kv_end = p.q_start + tile * POS + POS;
+  kv_end = kv_end < p.seq_len ? kv_end : p.seq_len;
+  int limit[2], wave_end = 0;
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const int pos = tpos + 16 * qt + i;
+    int lim = p.q_start + pos + 1;
+    lim = lim < p.seq_len ? lim : p.seq_len;
+    limit[qt] = pos < p.tokens ? lim : 0;
+  }
+  {
+    int last = tpos + 31 < p.tokens - 1 ? tpos + 31 : p.tokens - 1;  // last live position of the wave
+    wave_end = last >= tpos ? p.q_start + last + 1 : 0;
+    wave_end = wave_end < p.seq_len ? wave_end : p.seq_len;
+  }
+
+  const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
+  const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
+
+  u32x4 kreg[LCH], vreg[LCH];
+  auto load_block = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < LCH; ++u) {
+      const int c = t + kThreads * u;
+      const int tok = base + (c >> 4);
+      // rows past the key range read row 0 (their scores are masked): no load behind a branch
+      const long off = (long)(tok < kv_end ? tok : 0) * p.c_ts + (c & 15) * 8;
+      kreg[u] = ld16(kc + off);
+      vreg[u] = ld16(vc + off);
+    }
+  };
+  auto park = [&]() {
+#pragma unroll
+    for (int u = 0; u < LCH; ++u) {
+      const int c = t + kThreads * u;
+      *(u32x4*)&k_lds[c >> 4][(c & 15) * 8] = kreg[u];
+      *(u32x4*)&v_lds[c >> 4][(c & 15) * 8] = vreg[u];
+    }
+  };
+
+  const int n_blk = (kv_end + kPgTok - 1) / kPgTok;
+  load_block(0);
+
+  // B operands: rotated q of this wave's head, positions tpos + 16 qt + i, chunk g + 4 j
+  u32x4 qreg[2][4];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    int pos = tpos + 16 * qt + i;
+    pos = pos < p.tokens ? pos : p.tokens - 1;
+    const uint16_t* qrow = p.q + (((long)b * p.hq + head) * p.tokens + pos) * kHeadDim;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) qreg[qt][j] = ld16(qrow + (g + 4 * j) * 8);
+  }
+
+  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  f32x4 acc[2][8];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int db = 0; db < 8; ++db) acc[qt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // one 32-token half of the LDS block (rows r0 .. r0 + 31), key positions base ..
+  auto attend = [&](int r0, int base) {
+    f32x4 s1[2], s2[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) { s1[qt] = f32x4{0.f, 0.f, 0.f, 0.f}; s2[qt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const u32x4 ka1 = *(const u32x4*)&k_lds[r0 + i][(g + 4 * j) * 8];
+      const u32x4 ka2 = *(const u32x4*)&k_lds[r0 + 16 + i][(g + 4 * j) * 8];
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        s1[qt] = attn_mfma<T>(ka1, qreg[qt][j], s1[qt]);
+        s2[qt] = attn_mfma<T>(ka2, qreg[qt][j], s2[qt]);
+      }
+    }
+    u32x4 pb[2];
+    float corr[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      float sc[8];
+      float m_loc = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
+        const float raw = r < 4 ? s1[qt][r] : s2[qt][r - 4];
+        sc[r] = tok < limit[qt] ? raw * p.scale_log2 : -INFINITY;
+        m_loc = fmaxf(m_loc, sc[r]);
+      }
+      m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
+      m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+      const float m_new = fmaxf(m[qt], m_loc);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      corr[qt] = fast_exp2(m[qt] - m_use);
+      float pr[8];
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        pr[r] = fast_exp2(sc[r] - m_use);
+        psum += pr[r];
+      }
+      l[qt] = fmaf(l[qt], corr[qt], psum);
+      m[qt] = m_new;
+      pb[qt].x = (uint32_t)T::pack(pr[0]) | ((uint32_t)T::pack(pr[1]) << 16);
+      pb[qt].y = (uint32_t)T::pack(pr[2]) | ((uint32_t)T::pack(pr[3]) << 16);
+      pb[qt].z = (uint32_t)T::pack(pr[4]) | ((uint32_t)T::pack(pr[5]) << 16);
+      pb[qt].w = (uint32_t)T::pack(pr[6]) | ((uint32_t)T::pack(pr[7]) << 16);
+    }
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const u32x2 lo = lds_read_tr16(&v_lds[r0 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x2 hi = lds_read_tr16(&v_lds[r0 + 16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        f32x4 a = acc[qt][db];
+        a.x *= corr[qt]; a.y *= corr[qt]; a.z *= corr[qt]; a.w *= corr[qt];
+        acc[qt][db] = attn_mfma<T>(va, pb[qt], a);
+      }
+    }
+  };
+
+  for (int kb = 0; kb < n_blk; ++kb) {
+    const int base = kb * kPgTok;
+    __syncthreads();  // every wave is done with the previous block
+    park();
+    __syncthreads();
+    load_block(base + kPgTok);  // in flight while this block is multiplied
+    // a wave whose last query cannot see the half skips it (uniform per wave; LDS reads only)
+    if (base < wave_end) attend(0, base);
+    if (base + 32 < wave_end) attend(32, base + 32);
+  }
+
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    float lt = l[qt];
+    lt += __shfl_xor(lt, 16);
+    lt += __shfl_xor(lt, 32);
+    const int pos = tpos + 16 * qt + i;
+    if (pos >= p.tokens) continue;
+    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    uint16_t* orow = p.out + ((long)b * p.tokens + pos) * ((long)p.hq * kHeadDim) + (long)head * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      // acc[qt][db][e]: d = 16 db + 4 g + e of query column i
+      const f32x4 o = acc[qt][db];
+      u32x2 pk;
+      pk.x = (uint32_t)T::pack(o.x * inv) | ((uint32_t)T::pack(o.y * inv) << 16);
+      pk.y = (uint32_t)T::pack(o.z * inv) | ((uint32_t)T::pack(o.w * inv) << 16);
+      *(u32x2*)(orow + 16 * db + 4 * g) = pk;
+    }
+  }
+}
+
 // log-sum-exp merge of the per-split partials: one workgroup of 128 threads per (head, batch).
 // The split weights are computed once into LDS; the accumulation loop then has no dependent
 // loads, so the partial rows of all splits are in flight together.
@@ -1047,6 +1241,14 @@ static int launch_attn(hipStream_t s, int dtype, const AttnParams& p, int batch)
 using namespace mui;
 
 static int g_attn_min_tokens = 0;  // 0: built-in choice; else fewest tokens worth a split
+// prompt attention: 0 = built-in choice (the KV-group kernel from 512 query tokens), n > 0 = from n
+// tokens, negative = never
+static int g_prefill_group_tokens = 0;
+
+extern "C" int mui_tune_prefill_attention(int group_kernel_min_tokens) {
+  g_prefill_group_tokens = group_kernel_min_tokens;
+  return MUI_OK;
+}
 
 extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
                                   int mfma_tokens) {
@@ -1301,8 +1503,28 @@ extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void*
   p.out = (uint16_t*)out;
   p.hq = n_q_heads; p.hkv = n_kv_heads; p.tokens = tokens; p.seq_len = seq_len; p.q_start = q_start;
   p.scale_log2 = kLog2e / sqrtf((float)head_dim);
-  dim3 grid(ceil_div(tokens, 16), n_q_heads, batch);
   hipStream_t s = (hipStream_t)stream;
+  // Long prompts with 1, 2, 4 or 8 query heads per KV head: K/V rows cross LDS once per 32 query
+  // positions of the whole KV group. Short prompts keep the kernel that splits the key range of
+  // 16 query positions over four waves (more workgroups, shorter chains).
+  const int group = n_q_heads / n_kv_heads;
+  const bool grouped = (group == 1 || group == 2 || group == 4 || group == 8) &&
+                       (g_prefill_group_tokens > 0 ? tokens >= g_prefill_group_tokens : g_prefill_group_tokens == 0 && tokens >= 512);
+  if (grouped) {
+#define MUI_PG_LAUNCH(TT, GG)                                                                          \
+    hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG>), dim3(ceil_div(tokens, 128 / (GG == 8 ? 4 : GG)), n_kv_heads, batch), \
+                       dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p)
+    if (dtype == MUI_DTYPE_F16) {
+      if (group == 1) MUI_PG_LAUNCH(F16, 1); else if (group == 2) MUI_PG_LAUNCH(F16, 2);
+      else if (group == 4) MUI_PG_LAUNCH(F16, 4); else MUI_PG_LAUNCH(F16, 8);
+    } else {
+      if (group == 1) MUI_PG_LAUNCH(BF16, 1); else if (group == 2) MUI_PG_LAUNCH(BF16, 2);
+      else if (group == 4) MUI_PG_LAUNCH(BF16, 4); else MUI_PG_LAUNCH(BF16, 8);
+    }
+#undef MUI_PG_LAUNCH
+    return launch_status();
+  }
+  dim3 grid(ceil_div(tokens, 16), n_q_heads, batch);
   if (dtype == MUI_DTYPE_F16)
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4>), grid, dim3(4 * kWave), 0, s, p);
   else

@@ -49,7 +49,15 @@ struct PrefillGemmParams {
 
 // WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile is 32 WR weight rows x 32 WT tokens;
 // KS k-values per step.
-template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int KS>
+// dynamically sized LDS: two stages of the 128 x 128 tile exceed the 64 KB a kernel may declare statically
+extern __shared__ __align__(16) unsigned char pf_smem[];
+
+template <int WR, int WT, int KS, int NBUF>
+constexpr size_t prefill_lds_bytes() {
+  return (size_t)NBUF * (32 * WR + 32 * WT) * (KS + 8) * 2 + 32 * WT * 4;
+}
+
+template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int KS, int NBUF>
 __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillGemmParams p) {
   constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
   constexpr int PITCH = KS + 8;          // LDS row pitch in 16-bit elements: conflict-free 128-bit reads
@@ -59,9 +67,13 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   constexpr int WCH = (WF == WF_16BIT) ? ROWS * CPR / kPfThreads : ROWS * (KS / 16) / kPfThreads;
   static_assert(EPI != SK_GATEUP || WR % 2 == 0, "gate/up needs an even number of row tiles per wave");
   static_assert(XCH >= 1 && WCH >= 1 && kPfThreads % CPR == 0, "tile shape");
-  __shared__ __align__(16) uint16_t w_lds[ROWS * PITCH];
-  __shared__ __align__(16) uint16_t x_lds[TOKS * PITCH];
-  __shared__ float rs_lds[TOKS];
+  // NBUF == 2: step s + 1 is written to the other LDS stage while step s is multiplied, one
+  // barrier per step instead of two
+  typedef uint16_t WStage[ROWS * PITCH];
+  typedef uint16_t XStage[TOKS * PITCH];
+  WStage* w_lds = (WStage*)pf_smem;
+  XStage* x_lds = (XStage*)(pf_smem + (size_t)NBUF * sizeof(WStage));
+  float* rs_lds = (float*)(pf_smem + (size_t)NBUF * (sizeof(WStage) + sizeof(XStage)));
 
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
@@ -132,7 +144,7 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   float ss[XCH];
 #pragma unroll
   for (int i = 0; i < XCH; ++i) ss[i] = 0.f;
-  auto store_step = [&](int k0) {
+  auto store_step = [&](int k0, int buf) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
     const bool xlive = k0 + xcol * 8 + 8 <= p.k;
 #pragma unroll
@@ -141,19 +153,19 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
       u32x4 b = make_b<T, NORM>(xreg[i], NORM ? greg : xreg[i], sq);
       b = xlive ? b : zero;
       ss[i] += xlive ? sq : 0.f;
-      *(u32x4*)&x_lds[((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = b;
+      *(u32x4*)&x_lds[buf][((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = b;
     }
     if constexpr (WF == WF_16BIT) {
 #pragma unroll
       for (int i = 0; i < WCH; ++i)
-        *(u32x4*)&w_lds[((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = xlive ? wreg[i] : zero;
+        *(u32x4*)&w_lds[buf][((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = xlive ? wreg[i] : zero;
     } else {
       const bool wlive = k0 + wcol * 16 + 16 <= p.k;
 #pragma unroll
       for (int i = 0; i < WCH; ++i) {
         const u32x4 lo = convert_a<T, WF>(wreg[i].x, wreg[i].y, nullptr, 0, 0);
         const u32x4 hi = convert_a<T, WF>(wreg[i].z, wreg[i].w, nullptr, 0, 0);
-        uint16_t* dst = &w_lds[((t + kPfThreads * i) / WCPR) * PITCH + wcol * 16];
+        uint16_t* dst = &w_lds[buf][((t + kPfThreads * i) / WCPR) * PITCH + wcol * 16];
         *(u32x4*)dst = wlive ? lo : zero;
         *(u32x4*)(dst + 8) = wlive ? hi : zero;
       }
@@ -170,25 +182,39 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   const int n_steps = (p.k + KS - 1) / KS;
   const int a_base = (wr * 16 * WR + (lane & 15)) * PITCH + (lane >> 4) * 8;
   const int b_base = (wt * 16 * WT + (lane & 15)) * PITCH + (lane >> 4) * 8;
-  load_step(0);
-  for (int s = 0; s < n_steps; ++s) {
-    __syncthreads();  // the previous step's operands have been read
-    store_step(s * KS);
-    __syncthreads();
-    // requested now, consumed after this step's multiplications (the last iteration re-reads
-    // step 0, which keeps the loads out of a branch)
-    load_step(s + 1 < n_steps ? (s + 1) * KS : 0);
+  auto multiply = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < KS / 32; ++ks) {
       u32x4 a[WR], b[WT];
 #pragma unroll
-      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[a_base + i * 16 * PITCH + ks * 32];
+      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[buf][a_base + i * 16 * PITCH + ks * 32];
 #pragma unroll
-      for (int j = 0; j < WT; ++j) b[j] = *(const u32x4*)&x_lds[b_base + j * 16 * PITCH + ks * 32];
+      for (int j = 0; j < WT; ++j) b[j] = *(const u32x4*)&x_lds[buf][b_base + j * 16 * PITCH + ks * 32];
 #pragma unroll
       for (int i = 0; i < WR; ++i)
 #pragma unroll
         for (int j = 0; j < WT; ++j) acc[i][j] = mfma16x16x32<T>(a[i], b[j], acc[i][j]);
+    }
+  };
+  // loads past the last step re-read step 0 (never stored): that keeps them out of branches
+  load_step(0);
+  if constexpr (NBUF == 2) {
+    store_step(0, 0);
+    load_step(1 < n_steps ? KS : 0);
+    __syncthreads();
+    for (int s = 0; s < n_steps; ++s) {
+      multiply(s & 1);
+      if (s + 1 < n_steps) store_step((s + 1) * KS, (s + 1) & 1);  // uniform; the registers hold step s + 1
+      load_step(s + 2 < n_steps ? (s + 2) * KS : 0);
+      __syncthreads();
+    }
+  } else {
+    for (int s = 0; s < n_steps; ++s) {
+      __syncthreads();  // the previous step's operands have been read
+      store_step(s * KS, 0);
+      __syncthreads();
+      load_step(s + 1 < n_steps ? (s + 1) * KS : 0);  // in flight during this step's multiplications
+      multiply(0);
     }
   }
 
@@ -253,7 +279,7 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
 
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64
 
-template <typename T, int WF, int EPI, int WR, int WT, int KS>
+template <typename T, int WF, int EPI, int WR, int WT, int KS, int NBUF>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
   p.n_tiles = ceil_div(p.n, EPI == SK_GATEUP ? ROWS / 2 : ROWS);
@@ -261,30 +287,43 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   // whole row tiles per XCD: the grid covers ceil(n_tiles / 8) * 8 row tiles, the surplus exits
   const long grid = (long)ceil_div(p.n_tiles, 8) * 8 * p.t_tiles;
   if (grid > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
-  if (p.gamma)
-    hipLaunchKernelGGL((prefill_gemm_kernel<T, WF, true, EPI, WR, WT, KS>), dim3((int)grid), dim3(kPfThreads), 0, s, p);
-  else
-    hipLaunchKernelGGL((prefill_gemm_kernel<T, WF, false, EPI, WR, WT, KS>), dim3((int)grid), dim3(kPfThreads), 0, s, p);
-  return launch_status();
+  constexpr size_t lds = prefill_lds_bytes<WR, WT, KS, NBUF>();
+  auto launch = [&](auto kernel) {
+    if constexpr (lds > 65536) {
+      // more dynamic LDS than the default limit: raised once per kernel (and device)
+      static int raised_for = -1;
+      int dev = 0;
+      if (hipGetDevice(&dev) != hipSuccess) return MUI_ERR_DEVICE;
+      if (raised_for != dev) {
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+          return MUI_ERR_LAUNCH;
+        raised_for = dev;
+      }
+    }
+    hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(kPfThreads), lds, s, p);
+    return launch_status();
+  };
+  if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, KS, NBUF>);
+  return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, KS, NBUF>);
 }
 
 template <typename T, int WF, int EPI>
 static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
-  // The largest tile that still yields a workgroup per CU: big tiles re-read x and the weights
-  // least, but a grid smaller than the chip leaves the weight stream to too few CUs (measured on
-  // the Llama-3-8B shapes: 32 x 64 wins up to 256 tokens on the 4096-row matrices, 64 x 128 at
-  // 512, 128 x 128 from 2048; the 28672 gate/up rows take 64 x 128 up to 128 tokens, then 128 x 128).
+  // The largest tile that still yields three workgroups per four CUs: big tiles re-read x and the
+  // weights least, but a grid much smaller than the chip leaves the weight stream to too few CUs
+  // (measured on the Llama-3-8B shapes: 32 x 64 wins up to 256 tokens on the 4096-row matrices,
+  // 64 x 128 at 512, 128 x 128 from 2048; the 28672 gate/up rows take 128 x 128 throughout).
   const long rows = (EPI == SK_GATEUP) ? 2L * p.n : p.n;
-  const long want = device_cus();
+  const long want = 3L * device_cus() / 4;
   auto tiles = [&](int r, int tk) { return (long)ceil_div((int)rows, r) * ceil_div(p.tokens, tk); };
   int which = g_prefill_tile;
   if (which == 0) which = tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
-  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 64>(s, p);
+  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 64, 2>(s, p);
   if constexpr (EPI == SK_GATEUP) {
-    return launch_prefill_cfg<T, WF, EPI, 2, 4, 128>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 2, 4, 128, 1>(s, p);
   } else {
-    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 128>(s, p);
-    return launch_prefill_cfg<T, WF, EPI, 1, 2, 256>(s, p);
+    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 128, 1>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 1, 2, 256, 1>(s, p);
   }
 }
 

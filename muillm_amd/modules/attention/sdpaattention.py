@@ -29,9 +29,11 @@ def _ignore_causal_mask_sdpa(attention_mask: Optional[torch.Tensor], inputs_shap
 
 
 class MuiSdpaAttention(MuiBaseAttention):
-    # measured on MI355X (32/8 heads x 128) against repeat_kv + torch SDPA: 10 vs 38 us at 32 tokens,
-    # 30 vs 58 us at 512, 208 vs 182 us at 2048, 1930 vs 1418 us at 8192
-    prefill_kernel_max_tokens = 1536
+    # Unpadded prompts of any length run the library's causal kernels (measured on MI355X, 32/8 heads
+    # x 128, against repeat_kv + torch SDPA: 12 vs 36 us at 128 tokens, 22 vs 52 us at 512, 105 vs
+    # 165 us at 2048, 0.95 vs 1.37 ms at 8192); None = no limit, a number restores the SDPA route
+    # beyond that many tokens
+    prefill_kernel_max_tokens = None
 
     def _prefill_kernel_ok(self, q, k, v, attention_mask, all_ones_mask, q_len) -> bool:
         """T > 1 without padding (the mask, if any, is purely causal), 16-bit CUDA tensors,
@@ -42,8 +44,8 @@ class MuiSdpaAttention(MuiBaseAttention):
             return False
         if self.head_dim != 128 or k.shape[2] < q_len or self.training:
             return False
-        if q_len > self.prefill_kernel_max_tokens:
-            return False  # long prompts: torch's flash attention is about 2x faster beyond ~1k tokens
+        if self.prefill_kernel_max_tokens is not None and q_len > self.prefill_kernel_max_tokens:
+            return False
         return (k.stride() == v.stride() and k.stride(3) == 1 and all(st % 8 == 0 for st in k.stride()[:3])
                 and k.data_ptr() % 16 == 0 and v.data_ptr() % 16 == 0)
 

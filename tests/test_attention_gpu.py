@@ -358,6 +358,65 @@ def test_prefill_attention(b, hq, hkv, t, past, dtype):
     assert _max_abs(out, ref) <= (ATOL if dtype == torch.float16 else 1.6e-2)
 
 
+@pytest.mark.parametrize("choice", ["auto", "kv-group", "per-head"])
+@pytest.mark.parametrize("b,hq,hkv,t,past", [
+    (1, 32, 8, 2048, 0),     # the kernel shared by the four query heads of a KV head
+    (1, 32, 8, 1000, 24),    # ragged: not a multiple of the 32-position blocks, continues a cache
+    (2, 8, 8, 130, 5),       # one query head per KV head: four position blocks per workgroup
+    (1, 16, 8, 260, 0),      # two
+    (1, 64, 8, 140, 0),      # eight (8 waves)
+    (1, 24, 8, 300, 0),      # three: no kv-group variant, the per-head kernel serves it
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_prefill_attention_long_prompts(b, hq, hkv, t, past, dtype, choice):
+    """Prompt attention under each kernel choice (built-in; K/V shared by the query heads of a KV
+    head; one workgroup per 16 positions of one head), a sample of query rows against the oracle."""
+    if dtype == torch.bfloat16 and t > 1000:
+        t = 520
+    lib = _lib.load()
+    _lib.check(lib.mui_tune_prefill_attention({"auto": 0, "kv-group": 1, "per-head": -1}[choice]), "tune")
+    try:
+        g = _gen(23)
+        s = past + t
+        cap = oracle.next_pow2(s)
+        q = _mk((b, hq, t, D), g, dtype=dtype)
+        kc = _mk((b, hkv, cap, D), g, dtype=dtype)
+        vc = _mk((b, hkv, cap, D), g, dtype=dtype)
+        kc[:, :, s:] = float("nan")  # rows beyond the sequence must never be read
+        vc[:, :, s:] = float("nan")
+        kd, vd = kc.to(DEV), vc.to(DEV)
+        out = muillm_ext.mui_prefill_attention(q.to(DEV), kd[:, :, :s], vd[:, :, :s])
+        assert out.shape == (b, t, hq * D) and torch.isfinite(out).all()
+        rows = sorted(set(list(range(0, min(t, 40))) + list(range(t // 2 - 20, t // 2 + 20)) + list(range(t - 40, t))))
+        rows = torch.tensor([r for r in rows if 0 <= r < t])
+        mask = _causal_mask(t, s, past)[:, :, rows]
+        ref = oracle.decode_attention(q[:, :, rows], kc[:, :, :s], vc[:, :, :s], mask)
+        assert _max_abs(out[:, rows], ref) <= (ATOL if dtype == torch.float16 else 1.6e-2)
+    finally:
+        _lib.check(lib.mui_tune_prefill_attention(0), "tune")
+
+
+def test_prefill_attention_8k_rows_vs_oracle_and_kernels_agree():
+    """An 8192-token prompt (32 / 8 heads): sampled rows against the oracle, and the two prompt
+    kernels against each other on every row."""
+    lib = _lib.load()
+    g = _gen(24)
+    t = 8192
+    q, kc, vc = _mk((1, 32, t, D), g), _mk((1, 8, t, D), g), _mk((1, 8, t, D), g)
+    qd, kd, vd = q.to(DEV), kc.to(DEV), vc.to(DEV)
+    outs = {}
+    for name, knob in (("kv-group", 1), ("per-head", -1)):
+        _lib.check(lib.mui_tune_prefill_attention(knob), "tune")
+        try:
+            outs[name] = muillm_ext.mui_prefill_attention(qd, kd, vd)
+        finally:
+            _lib.check(lib.mui_tune_prefill_attention(0), "tune")
+    assert float((outs["kv-group"].float() - outs["per-head"].float()).abs().max()) <= 2 * ATOL
+    rows = torch.tensor(list(range(0, 24)) + list(range(4085, 4110)) + list(range(t - 24, t)))
+    ref = oracle.decode_attention(q[:, :, rows], kc, vc, _causal_mask(t, t, 0)[:, :, rows])
+    assert _max_abs(outs["kv-group"][:, rows], ref) <= ATOL
+
+
 def test_prefill_attention_closed_forms():
     g = _gen(22)
     hq, hkv, t = 8, 2, 40
