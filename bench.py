@@ -73,6 +73,32 @@ def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=True, batch=1):
     return dt, dec
 
 
+def bench_prefill(lm, tokens, iters=3):
+    """Prefill of one `tokens`-token prompt (batch 1, last-token logits only): every linear layer on
+    the library's prompt kernels (fused-norm matrix-core GEMMs), causal attention on its prompt
+    attention kernel. Returns ms and the arithmetic rate over the dense fp16 MFMA peak."""
+    import torch
+
+    cfg = lm.config
+    ids = torch.randint(0, cfg.vocab_size, (1, tokens), generator=torch.Generator().manual_seed(1)).to("cuda")
+    with torch.no_grad():
+        for _ in range(2):
+            lm(input_ids=ids, num_logits_to_keep=1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            lm(input_ids=ids, num_logits_to_keep=1)
+        torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / iters * 1e3
+    hid, inter = cfg.hidden_size, cfg.intermediate_size
+    hq, hkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, hid // cfg.num_attention_heads
+    linear_flops = 2.0 * tokens * cfg.num_hidden_layers * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter)
+    attn_flops = 4.0 * hq * d * tokens * tokens / 2 * cfg.num_hidden_layers
+    tflops = (linear_flops + attn_flops) / ms / 1e9
+    return {"ms": round(ms, 3), "tokens_per_s": round(tokens / ms * 1e3, 1), "TFLOP/s": round(tflops, 1),
+            "mfma_peak_frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4)}
+
+
 def bench_int8_variant(config, steps, warmup, group_size=0):
     """The same decode benchmark with the decoder layers quantised to int8 (group_size 0: symmetric
     per output channel; else the reference's group-wise uint8 + (scale, min) format; lm_head stays
@@ -685,6 +711,9 @@ def main():
             dt_c, dec_c = bench_decode(lm, 64, 8, prompt_len=ctx)
             result["variants"]["fp16_context%d_tokens_per_s" % ctx] = round(64 / dt_c, 2)
             del dec_c
+            torch.cuda.empty_cache()
+        for ptoks in (512, 4096):
+            result["variants"]["prefill_%d" % ptoks] = bench_prefill(lm, ptoks)
             torch.cuda.empty_cache()
         for bsz in (4, 8, 16):
             dt_b, dec_b = bench_decode(lm, min(args.steps, 128), min(args.warmup, 8), batch=bsz)

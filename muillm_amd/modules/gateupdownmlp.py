@@ -20,6 +20,7 @@ from ..memorymanagement.gc import trigger_gc
 from ..replacement.replacementcontext import MuiReplacementContext
 from .linear import MuiLinear
 from .module import MuiModule
+from ._fusion import AbsorbedNorm
 from .norm.rmsnorm import MuiRMSNorm, _MuiRMSNorm
 
 
@@ -136,7 +137,7 @@ class MuiGateUpDownMLP(MuiModule):
             normalize, variance_epsilon, norm_weights = True, prev_module.variance_epsilon, None
         elif prev_layernorm_module is not None:
             normalize = True
-            variance_epsilon = MuiRMSNorm._extract_eps(prev_layernorm_module)
+            variance_epsilon = AbsorbedNorm.of(prev_layernorm_module).eps
             norm_weights = prev_layernorm_module.weight
         else:
             normalize, variance_epsilon, norm_weights = False, 0.0, None

@@ -1,5 +1,12 @@
-"""MuiLinear -- muillm/modules/linear.py:19-333: nn.Linear with an optional fused input
-RMSNorm and a fused residual add."""
+"""MuiLinear: nn.Linear that can apply the RMSNorm in front of it and add a residual behind it,
+all inside one kernel (API of muillm/modules/linear.py:19-333 in the reference: replace /
+copy_module / finalize_init / finalize_deinit / forward(input, residual), `normalize`,
+`variance_epsilon`, `norm_weights`).
+
+The gain vector stays a separate parameter (multiplying it into the matrix would change the
+rounding). One deliberate difference from the reference: the epsilon passed to the constructor
+survives copy_module (there it falls back to 0 whenever norm weights are handed over,
+linear.py:272-309)."""
 from typing import Optional, Union
 
 import torch
@@ -11,18 +18,21 @@ from .. import muillm_ext
 from .._hf import LlamaRMSNorm, MistralRMSNorm
 from ..engineconfig import MuiEngineConfig
 from ..replacement.replacementcontext import MuiReplacementContext
+from ._fusion import AbsorbedNorm, fill_parameter, is_kernel_dtype, rmsnorm_reference
 from .module import MuiModule
 from .norm.rmsnorm import MuiRMSNorm, _MuiRMSNorm
 
 
 class _MuiLinear(torch.autograd.Function):
+    """The library call as an autograd node without a backward (inference only)."""
+
     @staticmethod
     def forward(ctx, module, x, residual):
         return muillm_ext.muillm_linear_module_forward(module, x, residual=residual)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("MuiLinear backward is not implemented")
+        raise NotImplementedError("inference only: MuiLinear has no backward")
 
 
 class MuiLinear(MuiModule, nn.Linear):
@@ -32,121 +42,101 @@ class MuiLinear(MuiModule, nn.Linear):
         nn.Linear.__init__(self, in_features=in_features, out_features=out_features, bias=bias,
                            device=device, dtype=dtype)
         self.cpp_engine = engine_config.cpp_engine
-        self.device = self.weight.device
-        self.dtype = self.weight.dtype
-        self.normalize = normalize
+        self.device, self.dtype = self.weight.device, self.weight.dtype
+        self.normalize = bool(normalize)
         self.variance_epsilon = variance_epsilon
-        self.norm_weights = nn.Parameter(torch.ones(in_features, dtype=dtype, device=device)) if normalize else None
-        self._check_dispatchable()
-        # the kernel-side handle is created at the end of all layer replacements
-        self.cpp_module = None
+        self.norm_weights = None
+        if self.normalize:
+            self.norm_weights = nn.Parameter(torch.ones(in_features, dtype=dtype, device=device))
+        self.dispatchable = is_kernel_dtype(self.weight)
+        self.cpp_module = None  # the library-side handle; made by finalize_init once every layer is in place
 
-    def _check_dispatchable(self):
-        self.dispatchable = self.weight.is_cuda and self.weight.dtype in (torch.float16, torch.bfloat16)
-
+    # ---- life cycle --------------------------------------------------------------------------
     def finalize_init(self):
-        if self.cpp_module is not None:
-            muillm_ext.muillm_linear_module_deinit(self.cpp_module)
+        self.finalize_deinit()
+        self.dispatchable = is_kernel_dtype(self.weight)
         self.cpp_module = muillm_ext.muillm_linear_module_init(
             self.cpp_engine, self.weight, self.norm_weights, self.variance_epsilon, None, self.bias)
-        self._check_dispatchable()
 
     def finalize_deinit(self):
-        cpp_module = self.__dict__.get("cpp_module", None)
-        if cpp_module is not None:
-            muillm_ext.muillm_linear_module_deinit(cpp_module)
+        handle = self.__dict__.get("cpp_module")
+        if handle is not None:
+            muillm_ext.muillm_linear_module_deinit(handle)
             self.cpp_module = None
 
-    @staticmethod
-    def _set_requires_grads(param: nn.Parameter, requires_grads: bool) -> None:
-        if param is not None:
-            param.requires_grad = requires_grads
-
+    # ---- construction from other layers ------------------------------------------------------
     @staticmethod
     def replace(replacement_context: MuiReplacementContext, prev_module: Union["MuiLinear", nn.Linear],
                 prev_layernorm_module: Union[MuiRMSNorm, LlamaRMSNorm, MistralRMSNorm] = None) -> "MuiLinear":
-        engine_config = replacement_context.engine_config
+        """A MuiLinear holding prev_module's parameters; with prev_layernorm_module, that norm is
+        absorbed (the caller drops the norm layer). A MuiLinear passes through unchanged unless a
+        norm is to be absorbed into it."""
         device = replacement_context.device
         if device is None:
-            raise ValueError("device was None")
-        if isinstance(prev_module, MuiLinear) and (prev_layernorm_module is None):
+            raise ValueError("the replacement context names no target device")
+        already_ours = isinstance(prev_module, MuiLinear)
+        if already_ours and prev_layernorm_module is None:
             return prev_module
         if not isinstance(prev_module, nn.Linear):
-            raise ValueError(f"Unsupported replacement to MuiLinear: {prev_module.__class__.__name__}")
-        prev_module = replacement_context.to_local_module(prev_module).to(device)
+            raise ValueError(f"MuiLinear can stand in for nn.Linear layers, not for {type(prev_module).__name__}")
+        if already_ours and prev_module.normalize and prev_layernorm_module is not None:
+            raise ValueError("this MuiLinear already applies a norm; a second one cannot be absorbed")
+
+        source = replacement_context.to_local_module(prev_module).to(device)
+        absorbed = None
         if prev_layernorm_module is not None:
-            prev_layernorm_module = replacement_context.to_local_module(prev_layernorm_module).to(device)
+            absorbed = AbsorbedNorm.of(replacement_context.to_local_module(prev_layernorm_module).to(device))
+        carries_norm = already_ours and source.normalize
+        eps = absorbed.eps if absorbed is not None else (source.variance_epsilon if carries_norm else 0.0)
 
-        if isinstance(prev_module, MuiLinear) and prev_module.normalize:
-            if prev_layernorm_module is not None:
-                raise ValueError("both norm weights in MuiLinear and layernorm module provided")
-            normalize, variance_epsilon, norm_weights = True, prev_module.variance_epsilon, None
-        elif prev_layernorm_module is not None:
-            normalize = True
-            variance_epsilon = MuiRMSNorm._extract_eps(prev_layernorm_module)
-            norm_weights = prev_layernorm_module.weight
-        else:
-            normalize, variance_epsilon, norm_weights = False, 0.0, None
+        layer = MuiLinear(replacement_context.engine_config, in_features=source.in_features,
+                          out_features=source.out_features, bias=source.bias is not None, variance_epsilon=eps,
+                          normalize=absorbed is not None or carries_norm, dtype=source.weight.dtype, device=device)
+        layer.copy_module(source, norm_weights=None if absorbed is None else absorbed.gain, device=device)
+        return layer
 
-        new_module = MuiLinear(
-            engine_config=engine_config, in_features=prev_module.in_features,
-            out_features=prev_module.out_features, bias=prev_module.bias is not None,
-            variance_epsilon=variance_epsilon, normalize=normalize,
-            dtype=prev_module.weight.dtype, device=device)
-        new_module.copy_module(prev_module=prev_module, norm_weights=norm_weights, device=device)
-        return new_module
-
-    def _set_weights(self, weights: torch.Tensor, requires_grads: Optional[bool] = None) -> None:
-        rg = weights.requires_grad if requires_grads is None else requires_grads
-        self.weight.data.copy_(weights.data)
-        MuiLinear._set_requires_grads(self.weight, rg)
-
-    def _set_bias(self, bias: torch.Tensor, requires_grads: Optional[bool] = None) -> None:
-        if bias is not None:
-            rg = bias.requires_grad if requires_grads is None else requires_grads
-            self.bias.data.copy_(bias.data)
-            MuiLinear._set_requires_grads(self.bias, rg)
-        else:
-            self.bias = None
-
-    def _set_norm_weights(self, norm_weights: torch.Tensor, requires_grads: Optional[bool] = None) -> None:
-        rg = norm_weights.requires_grad if requires_grads is None else requires_grads
-        self.norm_weights.data.copy_(norm_weights.data)
-        MuiLinear._set_requires_grads(self.norm_weights, rg)
+    def load_tensors(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     norm_weights: Optional[torch.Tensor] = None, weight_requires_grad: Optional[bool] = None,
+                     bias_requires_grad: Optional[bool] = None) -> None:
+        """Fill the parameters in place from plain tensors (shapes must match the constructor's)."""
+        fill_parameter(self.weight, weight, weight_requires_grad)
+        if self.bias is not None:
+            if bias is None:
+                raise ValueError("this layer was built with a bias but none was supplied")
+            fill_parameter(self.bias, bias, bias_requires_grad)
+        elif bias is not None:
+            raise ValueError("this layer was built without a bias")
+        if norm_weights is not None:
+            if self.norm_weights is None:
+                raise ValueError("this layer was built without a fused norm")
+            fill_parameter(self.norm_weights, norm_weights)
 
     def copy_module(self, prev_module: Union["MuiLinear", nn.Linear], norm_weights: torch.Tensor = None,
                     device=None):
-        """Copies weights/bias (and norm weights). Unlike the reference (linear.py:272-309) the
-        epsilon given to the constructor is kept instead of being reset to 0."""
+        """Take over prev_module's matrix and bias, plus a gain vector: either norm_weights or the
+        one prev_module (a MuiLinear) already carries, never both."""
         if device is None:
-            raise ValueError("device was None")
-        self._set_weights(prev_module.weight)
-        if prev_module.bias is not None:
-            self._set_bias(prev_module.bias)
-        if isinstance(prev_module, MuiLinear):
-            if (prev_module.norm_weights is not None) and (norm_weights is not None):
-                raise ValueError("both norm weights in MuiLinear and norm_weight provided")
-            if prev_module.normalize:
-                norm_weights = prev_module.norm_weights
-        elif not isinstance(prev_module, nn.Linear):
-            raise ValueError(f"Unsupported replacement: {prev_module.__class__.__name__}")
-        if norm_weights is not None:
-            # the norm weights stay separate from the matrix (folding them in is numerically unstable)
-            self._set_norm_weights(norm_weights)
+            raise ValueError("copy_module needs the target device")
+        if not isinstance(prev_module, nn.Linear):
+            raise ValueError(f"cannot copy from {type(prev_module).__name__}")
+        own_gain = prev_module.norm_weights if isinstance(prev_module, MuiLinear) and prev_module.normalize else None
+        if own_gain is not None and norm_weights is not None:
+            raise ValueError("two gain vectors: the source layer carries one and another was passed")
+        self.load_tensors(prev_module.weight, prev_module.bias if self.bias is not None else None,
+                          norm_weights if norm_weights is not None else own_gain)
         self.to(device=device)
-        self._check_dispatchable()
+        self.dispatchable = is_kernel_dtype(self.weight)
 
+    # ---- forward -----------------------------------------------------------------------------
     def forward(self, input: Tensor, residual: Optional[Tensor] = None) -> Tensor:
         if self.cpp_module is not None:
             return _MuiLinear.apply(self.cpp_module, input, residual)
+        # before finalize_init: plain torch, with the library's norm kernel where it applies
+        x = input
         if self.normalize:
-            if self.dispatchable and input.is_cuda:
-                input = _MuiRMSNorm.apply(input, self.norm_weights, self.variance_epsilon)
+            if self.dispatchable and x.is_cuda:
+                x = _MuiRMSNorm.apply(x, self.norm_weights, self.variance_epsilon)
             else:
-                h = input.to(torch.float32)
-                h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
-                input = self.norm_weights * h.to(input.dtype)
-        output = F.linear(input, self.weight, self.bias)
-        if residual is not None:
-            output = output + residual
-        return output
+                x = rmsnorm_reference(x, self.norm_weights, self.variance_epsilon)
+        y = F.linear(x, self.weight, self.bias)
+        return y if residual is None else y + residual

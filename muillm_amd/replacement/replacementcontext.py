@@ -1,25 +1,26 @@
-"""MuiReplacementContext -- muillm/replacement/replacementcontext.py:7-42."""
+"""MuiReplacementContext: what every replace() receives (API of
+muillm/replacement/replacementcontext.py:7-42 in the reference: engine_config, model, device,
+to_local_module)."""
 import torch.nn as nn
 
 from ..engineconfig import MuiEngineConfig
 
 
 class MuiReplacementContext:
-    """What a replace() call needs: the engine config, the model being rewritten and the
-    target device."""
-
     def __init__(self, engine_config: MuiEngineConfig, model: nn.Module, device: str = "cuda"):
         self.engine_config = engine_config
-        self.model = model
-        self.device = device
+        self.model = model      # the tree being rewritten (None when layers are converted on their own)
+        self.device = device    # where converted layers end up
 
-    def _get_module_name(self, module: nn.Module) -> str:
-        for name, mod in self.model.named_modules():
-            if mod is module:
-                return name
-        raise ValueError(f"Module {module} not found in the model.")
+    def qualified_name(self, module: nn.Module) -> str:
+        """Dotted name of `module` inside the model."""
+        if self.model is not None:
+            for name, candidate in self.model.named_modules():
+                if candidate is module:
+                    return name
+        raise ValueError(f"{type(module).__name__} is not part of the model being converted")
 
     def to_local_module(self, module: nn.Module) -> nn.Module:
-        """The reference converts DTensor-sharded HF modules to local ones here; with one GPU
-        every module already is local."""
+        """Hook for sharded checkpoints: the reference gathers DTensor-sharded HuggingFace modules
+        here. One GPU: every module is local already."""
         return module
