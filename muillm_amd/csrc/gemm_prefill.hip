@@ -54,13 +54,16 @@ extern __shared__ __align__(16) unsigned char pf_smem[];
 
 template <int WR, int WT, int KS, int NBUF>
 constexpr size_t prefill_lds_bytes() {
-  return (size_t)NBUF * (32 * WR + 32 * WT) * (KS + 8) * 2 + 32 * WT * 4;
+  return (size_t)NBUF * (32 * WR + 32 * WT) * KS * 2 + 32 * WT * 4;
 }
 
 template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int KS, int NBUF>
 __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillGemmParams p) {
   constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
-  constexpr int PITCH = KS + 8;          // LDS row pitch in 16-bit elements: conflict-free 128-bit reads
+  // LDS rows are unpadded; 16-byte chunk c of row r lives at chunk c ^ swz(r), chosen so that the
+  // 16 lanes of a 128-bit access (16 consecutive rows of one logical chunk when reading operands,
+  // 16 consecutive chunks when staging) fall into 16 different groups of four banks
+  constexpr int PITCH = KS;
   constexpr int CPR = KS / 8;            // 16-byte chunks of 8 elements per row and step
   constexpr int OUT_TILE = (EPI == SK_GATEUP) ? ROWS / 2 : ROWS;  // outputs per workgroup
   constexpr int XCH = TOKS * CPR / kPfThreads;                     // token loads per thread and step
@@ -80,6 +83,8 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   const int wave = t >> 6;
   const int wr = wave >> 1;  // which half of the rows
   const int wt = wave & 1;   // which half of the tokens
+  // bank group of (row r, chunk c) is (r * chunks-per-row + c) mod 16
+  auto swz = [](int r) { return CPR == 8 ? ((r >> 1) & 7) : (r & 15); };
 
   // workgroup -> (row tile, token tile): consecutive workgroup ids are dealt round-robin to the
   // 8 XCDs, so ids that share id % 8 share an L2; give each XCD whole row tiles
@@ -122,52 +127,61 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
 #pragma unroll
   for (int i = 0; i < WCH; ++i) wrow[i] = weight_row_ptr((t + kPfThreads * i) / WCPR);
 
-  u32x4 wreg[WCH], xreg[XCH], greg;
-  auto load_step = [&](int k0) {
+  const int n_steps = (p.k + KS - 1) / KS;
+  // one k-step of the tile in registers, on its way from global memory to LDS
+  struct Stage { u32x4 w[WCH], x[XCH], g; };
+  auto load_step = [&](int step, Stage& r) {
+    // steps past the last one re-read step 0 (never stored): that keeps the loads out of branches;
     // chunks past the end of the row read the row's first chunk and are zeroed on the way to LDS
+    const int k0 = step < n_steps ? step * KS : 0;
     const int xk = k0 + xcol * 8;
     const int xoff = xk + 8 <= p.k ? xk : 0;
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) xreg[i] = ld16(xrow[i] + xoff);
-    if constexpr (NORM) greg = ld16(p.gamma + xoff);
+    for (int i = 0; i < XCH; ++i) r.x[i] = ld16(xrow[i] + xoff);
+    if constexpr (NORM) r.g = ld16(p.gamma + xoff);
     if constexpr (WF == WF_16BIT) {
 #pragma unroll
-      for (int i = 0; i < WCH; ++i) wreg[i] = ld16_stream(wrow[i] + 2L * xoff);
+      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wrow[i] + 2L * xoff);
     } else {
       const int wk = k0 + wcol * 16;
       const int woff = wk + 16 <= p.k ? wk : 0;
 #pragma unroll
-      for (int i = 0; i < WCH; ++i) wreg[i] = ld16_stream(wrow[i] + woff);
+      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wrow[i] + woff);
     }
   };
 
   float ss[XCH];
 #pragma unroll
   for (int i = 0; i < XCH; ++i) ss[i] = 0.f;
-  auto store_step = [&](int k0, int buf) {
+  auto store_step = [&](int step, int buf, const Stage& r) {
+    const int k0 = step * KS;
     const u32x4 zero = {0u, 0u, 0u, 0u};
     const bool xlive = k0 + xcol * 8 + 8 <= p.k;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
       float sq = 0.f;
-      u32x4 b = make_b<T, NORM>(xreg[i], NORM ? greg : xreg[i], sq);
+      u32x4 b = make_b<T, NORM>(r.x[i], NORM ? r.g : r.x[i], sq);
       b = xlive ? b : zero;
       ss[i] += xlive ? sq : 0.f;
-      *(u32x4*)&x_lds[buf][((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = b;
+      const int row = (t + kPfThreads * i) / CPR;
+      *(u32x4*)&x_lds[buf][row * PITCH + ((xcol ^ swz(row)) * 8)] = b;
     }
     if constexpr (WF == WF_16BIT) {
 #pragma unroll
-      for (int i = 0; i < WCH; ++i)
-        *(u32x4*)&w_lds[buf][((t + kPfThreads * i) / CPR) * PITCH + xcol * 8] = xlive ? wreg[i] : zero;
+      for (int i = 0; i < WCH; ++i) {
+        const int row = (t + kPfThreads * i) / CPR;
+        *(u32x4*)&w_lds[buf][row * PITCH + ((xcol ^ swz(row)) * 8)] = xlive ? r.w[i] : zero;
+      }
     } else {
       const bool wlive = k0 + wcol * 16 + 16 <= p.k;
 #pragma unroll
       for (int i = 0; i < WCH; ++i) {
-        const u32x4 lo = convert_a<T, WF>(wreg[i].x, wreg[i].y, nullptr, 0, 0);
-        const u32x4 hi = convert_a<T, WF>(wreg[i].z, wreg[i].w, nullptr, 0, 0);
-        uint16_t* dst = &w_lds[buf][((t + kPfThreads * i) / WCPR) * PITCH + wcol * 16];
-        *(u32x4*)dst = wlive ? lo : zero;
-        *(u32x4*)(dst + 8) = wlive ? hi : zero;
+        const u32x4 lo = convert_a<T, WF>(r.w[i].x, r.w[i].y, nullptr, 0, 0);
+        const u32x4 hi = convert_a<T, WF>(r.w[i].z, r.w[i].w, nullptr, 0, 0);
+        const int row = (t + kPfThreads * i) / WCPR;
+        uint16_t* dst = &w_lds[buf][row * PITCH];
+        *(u32x4*)(dst + (((2 * wcol) ^ swz(row)) * 8)) = wlive ? lo : zero;
+        *(u32x4*)(dst + (((2 * wcol + 1) ^ swz(row)) * 8)) = wlive ? hi : zero;
       }
     }
   };
@@ -179,41 +193,45 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
     for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   if (t < TOKS) rs_lds[t] = 0.f;
 
-  const int n_steps = (p.k + KS - 1) / KS;
-  const int a_base = (wr * 16 * WR + (lane & 15)) * PITCH + (lane >> 4) * 8;
-  const int b_base = (wt * 16 * WT + (lane & 15)) * PITCH + (lane >> 4) * 8;
+  const int a_base = (wr * 16 * WR + (lane & 15)) * PITCH;  // rows 16 i + lane % 16: the swizzle depends on the lane only
+  const int b_base = (wt * 16 * WT + (lane & 15)) * PITCH;
+  const int lsw = swz(lane & 15), lg = lane >> 4;
   auto multiply = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < KS / 32; ++ks) {
       u32x4 a[WR], b[WT];
 #pragma unroll
-      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[buf][a_base + i * 16 * PITCH + ks * 32];
+      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[buf][a_base + i * 16 * PITCH + (((ks * 4 + lg) ^ lsw) * 8)];
 #pragma unroll
-      for (int j = 0; j < WT; ++j) b[j] = *(const u32x4*)&x_lds[buf][b_base + j * 16 * PITCH + ks * 32];
+      for (int j = 0; j < WT; ++j) b[j] = *(const u32x4*)&x_lds[buf][b_base + j * 16 * PITCH + (((ks * 4 + lg) ^ lsw) * 8)];
 #pragma unroll
       for (int i = 0; i < WR; ++i)
 #pragma unroll
         for (int j = 0; j < WT; ++j) acc[i][j] = mfma16x16x32<T>(a[i], b[j], acc[i][j]);
     }
   };
-  // loads past the last step re-read step 0 (never stored): that keeps them out of branches
-  load_step(0);
+  Stage r0;
+  load_step(0, r0);
   if constexpr (NBUF == 2) {
-    store_step(0, 0);
-    load_step(1 < n_steps ? KS : 0);
+    // two LDS stages: while step s is multiplied, step s + 1 moves from the registers to the
+    // other stage and step s + 2 is in flight from memory; one barrier per step. (A second
+    // register stage, two steps in flight, pushed the kernel past 256 registers per lane: one
+    // workgroup per CU instead of two, 686 -> 846 us on 2048 x 28672 x 4096.)
+    store_step(0, 0, r0);
+    load_step(1, r0);
     __syncthreads();
     for (int s = 0; s < n_steps; ++s) {
       multiply(s & 1);
-      if (s + 1 < n_steps) store_step((s + 1) * KS, (s + 1) & 1);  // uniform; the registers hold step s + 1
-      load_step(s + 2 < n_steps ? (s + 2) * KS : 0);
+      if (s + 1 < n_steps) store_step(s + 1, (s + 1) & 1, r0);  // uniform branch, no loads inside
+      load_step(s + 2, r0);
       __syncthreads();
     }
   } else {
     for (int s = 0; s < n_steps; ++s) {
       __syncthreads();  // the previous step's operands have been read
-      store_step(s * KS, 0);
+      store_step(s, 0, r0);
       __syncthreads();
-      load_step(s + 1 < n_steps ? (s + 1) * KS : 0);  // in flight during this step's multiplications
+      load_step(s + 1, r0);  // in flight during this step's multiplications
       multiply(0);
     }
   }
