@@ -301,6 +301,179 @@ def pmc_probe_int8(launches=4):
                                          "calls": info}}))
 
 
+def _graph_chain_us(launch, n=400, replays=10):
+    """Average cost of one launch in a HIP graph of `n` copies of `launch(stream)` on one stream
+    (every kernel waits for the one before it), over `replays` replays."""
+    import torch
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = torch.cuda.current_stream().cuda_stream
+        for _ in range(n):
+            launch(st)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(replays):
+        graph.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return round(a.elapsed_time(b) * 1e3 / (replays * n), 3)
+
+
+def probe_kernel_boundary():
+    """What one dependent kernel costs inside a replayed HIP graph when it has next to nothing to do:
+    the read probe over 16 B and over 64 KiB, and a 256 x 256 GEMV (alone, and two of them feeding each
+    other). This is the part of every launch of a decode step that no kernel code can remove."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    f16 = dict(device="cuda", dtype=torch.float16)
+    sink = torch.zeros(64, dtype=torch.int32, device="cuda")
+    src = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    w, x, y = torch.randn(256, 256, **f16), torch.randn(256, **f16), torch.empty(256, **f16)
+
+    def gemv(st, a, b):
+        lib.mui_linear(st, 0, w.data_ptr(), 256, a.data_ptr(), None, 0.0, None, None, None, b.data_ptr(), 256, 256, 1)
+
+    out = {
+        "read_probe_16B_us": _graph_chain_us(lambda st: lib.mui_probe_read(st, src.data_ptr(), 16, sink.data_ptr())),
+        "read_probe_64KiB_us": _graph_chain_us(lambda st: lib.mui_probe_read(st, src.data_ptr(), 65536, sink.data_ptr())),
+        "gemv_256x256_us": _graph_chain_us(lambda st: gemv(st, x, y)),
+        "gemv_256x256_feeding_each_other_us": _graph_chain_us(lambda st: (gemv(st, x, y), gemv(st, y, x)), n=200) / 2,
+    }
+    print(json.dumps({"probe_kernel_boundary": out}))
+
+
+def probe_flash_splits():
+    """Fused RoPE + cache write + flash decoding at batch 1 (32 / 8 heads x 128) over the number of
+    sequence splits, 1k to 32k context, K/V rotated over distinct buffers (> 1 GB per ring)."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    f16 = dict(device="cuda", dtype=torch.float16)
+    hq, hkv, d, B = 32, 8, 128, 1
+    qs = (hq + 2 * hkv) * d
+    table = {}
+    for S in (1024, 4096, 16384, 32768):
+        kvbytes = B * 2 * hkv * S * d * 2
+        cnt = max(2, min(64, int(1.0e9 // kvbytes) + 1))
+        caches = [(torch.randn(B, hkv, S, d, **f16), torch.randn(B, hkv, S, d, **f16)) for _ in range(cnt)]
+        qkvx = torch.randn(B, qs, **f16)
+        cos, sin = [t.cuda() for t in _rope_tables_f32(S, d)]
+        pos = torch.full((B, 1), S - 1, dtype=torch.int64, device="cuda")
+        cpos = torch.full((1,), S - 1, dtype=torch.int64, device="cuda")
+        o = torch.empty(B, hq * d, **f16)
+        row = {"kv_bytes": kvbytes, "auto_splits": lib.mui_flash_decode_splits(B, hq, hkv, S)}
+        for ns in (1, 8, 16, 32, 48, 64, 128):
+            if ns > 1 and S // ns < 32:
+                continue
+            scratch = torch.empty(max(lib.mui_flash_decode_scratch_bytes(B, hq, d, ns), 16), dtype=torch.uint8, device="cuda")
+
+            def att(i):
+                kc, vc = caches[i % len(caches)]
+                _lib.check(lib.mui_attn_decode_fused(
+                    stream, 0, qkvx.data_ptr(), qs, qkvx.data_ptr() + 2 * hq * d, qs, qkvx.data_ptr() + 2 * (hq + hkv) * d, qs,
+                    cos.data_ptr(), sin.data_ptr(), d // 2, cos.shape[0], pos.data_ptr(), 1, cpos.data_ptr(), S,
+                    kc.data_ptr(), vc.data_ptr(), hkv * S * d, S * d, d, None, 0, None, scratch.data_ptr(), ns, o.data_ptr(),
+                    B, hq, hkv, d, S), "mui_attn_decode_fused")
+
+            row["splits_%d_us" % ns] = round(_event_time_us(att, 10 * cnt, cnt), 2)
+        table["context_%d" % S] = row
+        del caches
+        torch.cuda.empty_cache()
+    print(json.dumps({"probe_flash_splits": table}))
+
+
+_PROMPT_SHAPES = (("qkv", 6144, 4096, False), ("o_proj", 4096, 4096, False), ("gateup", 14336, 4096, True),
+                  ("down", 4096, 14336, False))
+
+
+def _prompt_gemm_call(lib, stream, w, x, y, n, k, tokens, gateup):
+    from muillm_amd import _lib
+
+    if gateup:
+        _lib.check(lib.mui_gateup_silu(stream, 0, w.data_ptr(), w.data_ptr() + 2 * k, 2 * k, x.data_ptr(), None, 0.0,
+                                       y.data_ptr(), n, k, tokens), "mui_gateup_silu")
+    else:
+        _lib.check(lib.mui_linear(stream, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(),
+                                  n, k, tokens), "mui_linear")
+
+
+def probe_prompt(counters_only=False):
+    """The prompt kernels at the Llama-3-8B shapes. Timing mode: every projection at 64 to 4096 tokens
+    through the C ABI (weights rotated over > 1 GB) beside torch.matmul on the same operands, and causal
+    attention at 512 to 8192 tokens beside repeat_kv + torch SDPA. Counter mode (for `rocprofv3 --pmc`):
+    three launches of the gate/up projection at 2048 tokens and of attention at 4096 tokens."""
+    import torch
+    import torch.nn.functional as F
+
+    from muillm_amd import _lib, muillm_ext
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    f16 = dict(device="cuda", dtype=torch.float16)
+    hq, hkv, d = 32, 8, 128
+    if counters_only:
+        n, k, tokens = 14336, 4096, 2048
+        w = torch.randn(2 * n, k, **f16) * 0.02
+        x, y = torch.randn(tokens, k, **f16), torch.empty(tokens, n, **f16)
+        q = torch.randn(1, hq, 4096, d, **f16)
+        kk, vv = torch.randn(1, hkv, 4096, d, **f16), torch.randn(1, hkv, 4096, d, **f16)
+        for _ in range(3):
+            _prompt_gemm_call(lib, stream, w, x, y, n, k, tokens, True)
+        for _ in range(3):
+            muillm_ext.mui_prefill_attention(q, kk, vv)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe_prompt": {"gateup_flops_per_launch": 2.0 * tokens * 2 * n * k,
+                                               "attention_flops_per_launch": 4.0 * hq * d * 4096 * 4096 / 2}}))
+        return
+    out = {"linears": {}, "attention": {}}
+    for name, n, k, gateup in _PROMPT_SHAPES:
+        rows = 2 * n if gateup else n
+        ring = [torch.randn(rows, k, **f16) * 0.02 for _ in range(max(2, int(1e9 // (2 * rows * k)) + 1))]
+        for tokens in (64, 128, 256, 512, 2048, 4096):
+            x, y = torch.randn(tokens, k, **f16), torch.empty(tokens, n, **f16)
+            yt = torch.empty(tokens, rows, **f16)
+            us = _event_time_us(lambda i: _prompt_gemm_call(lib, stream, ring[i % len(ring)], x, y, n, k, tokens, gateup), 20, 3)
+            us_t = _event_time_us(lambda i: torch.matmul(x, ring[i % len(ring)].t(), out=yt), 20, 3)
+            flops = 2.0 * tokens * rows * k
+            out["linears"]["%s_tokens%d" % (name, tokens)] = {
+                "us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1),
+                "mfma_peak_frac": round(flops / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4), "torch_matmul_us": round(us_t, 1)}
+        del ring
+        torch.cuda.empty_cache()
+    for tokens in (512, 1024, 2048, 4096, 8192):
+        q = torch.randn(1, hq, tokens, d, **f16)
+        kk, vv = torch.randn(1, hkv, tokens, d, **f16), torch.randn(1, hkv, tokens, d, **f16)
+
+        def sdpa(i):
+            ke = kk[:, :, None].expand(1, hkv, hq // hkv, tokens, d).reshape(1, hq, tokens, d)
+            ve = vv[:, :, None].expand(1, hkv, hq // hkv, tokens, d).reshape(1, hq, tokens, d)
+            return F.scaled_dot_product_attention(q, ke, ve, is_causal=True)
+
+        us = _event_time_us(lambda i: muillm_ext.mui_prefill_attention(q, kk, vv), 10, 2)
+        us_t = _event_time_us(sdpa, 10, 2)
+        flops = 4.0 * hq * d * tokens * tokens / 2
+        out["attention"]["tokens%d" % tokens] = {"us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1),
+                                                 "mfma_peak_frac": round(flops / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4),
+                                                 "torch_repeat_kv_sdpa_us": round(us_t, 1)}
+    print(json.dumps({"probe_prompt": out}))
+
+
 def pmc_probe_attention(launches=3):
     """Counter probe for flash decoding (`rocprofv3 --pmc FETCH_SIZE`): fused RoPE + cache write +
     attention at 32k context, batch 8 and batch 1, over distinct caches."""
@@ -632,6 +805,15 @@ def main():
                     help="launch the int8 GEMVs of a Llama-3-8B layer at 1 and 4 tokens a few times and exit (for rocprofv3 --pmc)")
     ap.add_argument("--pmc-probe-attention", action="store_true",
                     help="launch flash decoding at 32k context a few times and exit (for rocprofv3 --pmc)")
+    ap.add_argument("--probe-kernel-boundary", action="store_true",
+                    help="time chains of near-empty dependent kernels in a replayed HIP graph and exit")
+    ap.add_argument("--probe-flash-splits", action="store_true",
+                    help="time fused flash decoding at batch 1 over the number of sequence splits and exit")
+    ap.add_argument("--probe-prompt", action="store_true",
+                    help="time the prompt GEMMs and prompt attention at the Llama-3-8B shapes beside torch and exit")
+    ap.add_argument("--pmc-probe-prompt", action="store_true",
+                    help="launch the gate/up prompt GEMM (2048 tokens) and prompt attention (4096) three times and exit "
+                         "(for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (no tensor parallelism, no collectives); "
@@ -655,6 +837,15 @@ def main():
         return
     if args.pmc_probe_attention:
         pmc_probe_attention()
+        return
+    if args.probe_kernel_boundary:
+        probe_kernel_boundary()
+        return
+    if args.probe_flash_splits:
+        probe_flash_splits()
+        return
+    if args.probe_prompt or args.pmc_probe_prompt:
+        probe_prompt(counters_only=args.pmc_probe_prompt)
         return
     if args.tune_attention:
         from muillm_amd import _lib

@@ -9,13 +9,16 @@
 // [+ add_bias] [+ residual], or h = silu(G xn) * (U xn), for 16-bit or per-channel int8 weights.
 //
 // Work layout (wave64, v_mfma_f32_16x16x32):
-//   a workgroup of 4 waves (2 x 2) owns a tile of weight rows x tokens and walks K in steps: the
-//   weight tile (int8 rows converted on the way) and the token tile (gamma * x rounded once to
-//   the 16-bit type, sum of squares gathered on the side) are staged through LDS with a padded
-//   pitch (conflict-free 128-bit reads); the loads of step s + 1 are in flight while step s is
-//   multiplied. Three tile shapes: 128 rows x 128 tokens x 64 k (each wave 4 x 4 MFMA tiles) when
-//   that still gives two workgroups per CU; else 64 x 128 x 128; else 32 x 64 x 256 -- the
-//   smaller the grid, the longer the k-step, so that enough weight bytes are in flight per CU.
+//   a workgroup owns a tile of weight rows x tokens and walks K in steps: the weight tile (int8
+//   rows converted on the way) and the token tile (gamma * x rounded once to the 16-bit type, sum
+//   of squares gathered on the side) are staged through LDS in unpadded rows whose 16-byte
+//   chunks are XOR-swizzled (conflict-free 128-bit reads and writes); the loads of step s + 2 are
+//   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
+//   Four tile shapes: 256 rows x 256 tokens x 64 k with eight waves (4 x 2, each 4 x 8 MFMA
+//   tiles: 12 KB of LDS reads per 32 matrix instructions) when the grid still covers most of the
+//   chip; else 128 x 128 x 64 with four waves (2 x 2, each 4 x 4 tiles); else 64 x 128 x 128;
+//   else 32 x 64 x 256 -- the smaller the grid, the longer the k-step, so that enough weight
+//   bytes are in flight per CU.
 //   Under the gate/up epilogue half of a wave's rows are gate rows and the other half the up
 //   rows of the same outputs, so SiLU * mul happens in registers.
 //   Token tiles of one row tile are placed on the same XCD (workgroup id modulo 8) so that the
@@ -24,7 +27,6 @@
 
 namespace mui {
 
-constexpr int kPfThreads = 256;  // 4 waves: 2 (rows) x 2 (tokens)
 
 struct PrefillGemmParams {
   const uint8_t* w0;      // linear: matrix; gate/up: gate rows
@@ -47,19 +49,20 @@ struct PrefillGemmParams {
   int t_tiles;  // token tiles
 };
 
-// WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile is 32 WR weight rows x 32 WT tokens;
-// KS k-values per step.
+// NWR x NWT waves per workgroup, WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile is
+// 16 WR NWR weight rows x 16 WT NWT tokens; KS k-values per step.
 // dynamically sized LDS: two stages of the 128 x 128 tile exceed the 64 KB a kernel may declare statically
 extern __shared__ __align__(16) unsigned char pf_smem[];
 
-template <int WR, int WT, int KS, int NBUF>
+template <int ROWS, int TOKS, int KS, int NBUF>
 constexpr size_t prefill_lds_bytes() {
-  return (size_t)NBUF * (32 * WR + 32 * WT) * KS * 2 + 32 * WT * 4;
+  return (size_t)NBUF * (ROWS + TOKS) * KS * 2 + TOKS * 4;
 }
 
-template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int KS, int NBUF>
-__global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillGemmParams p) {
-  constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
+template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int KS, int NBUF>
+__global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const PrefillGemmParams p) {
+  constexpr int kPfThreads = 64 * NWR * NWT;
+  constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   // LDS rows are unpadded; 16-byte chunk c of row r lives at chunk c ^ swz(r), chosen so that the
   // 16 lanes of a 128-bit access (16 consecutive rows of one logical chunk when reading operands,
   // 16 consecutive chunks when staging) fall into 16 different groups of four banks
@@ -81,8 +84,8 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t >> 6;
-  const int wr = wave >> 1;  // which half of the rows
-  const int wt = wave & 1;   // which half of the tokens
+  const int wr = wave / NWT;  // which band of the rows
+  const int wt = wave % NWT;  // which band of the tokens
   // bank group of (row r, chunk c) is (r * chunks-per-row + c) mod 16
   auto swz = [](int r) { return CPR == 8 ? ((r >> 1) & 7) : (r & 15); };
 
@@ -96,36 +99,47 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   const int t0 = tile_t * TOKS;      // first token of the tile
 
   // local weight row r -> matrix row. linear: o0 + r. gate/up: of a wave's 16 WR rows the first
-  // half are gate rows, the second half the up rows of the same outputs
-  auto weight_row_ptr = [&](int r) -> const uint8_t* {
+  // half are gate rows, the second half the up rows of the same outputs. Rows past the matrix read
+  // its last row (their outputs are never stored). Kept as 32-bit indices: the addresses are
+  // formed at the loads, 64-bit pointers per staged chunk would cost twice the registers.
+  auto weight_row = [&](int r, bool& up) -> int {
+    int o;
     if constexpr (EPI == SK_GATEUP) {
       constexpr int HALF = 8 * WR;  // outputs per wave
       const int h = r / (2 * HALF), within = r % (2 * HALF);
-      int o = o0 + h * HALF + within % HALF;
-      o = o < p.n ? o : p.n - 1;
-      return (within >= HALF ? p.w1 : p.w0) + (long)o * p.pitch;
+      o = o0 + h * HALF + within % HALF;
+      up = within >= HALF;
     } else {
-      int o = o0 + r;
-      o = o < p.n ? o : p.n - 1;
-      return p.w0 + (long)o * p.pitch;
+      o = o0 + r;
+      up = false;
     }
+    return o < p.n ? o : p.n - 1;
   };
 
-  // ---- staging assignment: 16-byte chunk c = t + 256 i of a tile is row c / chunks-per-row,
+  // ---- staging assignment: 16-byte chunk c = t + threads * i of a tile is row c / chunks-per-row,
   // column c % chunks-per-row (the column is the same for every i)
   const int xcol = t % CPR;
-  const uint16_t* xrow[XCH];
+  int xtok[XCH];
 #pragma unroll
   for (int i = 0; i < XCH; ++i) {
-    int tk = t0 + (t + kPfThreads * i) / CPR;
-    tk = tk < p.tokens ? tk : p.tokens - 1;
-    xrow[i] = p.x + (long)tk * p.k;
+    const int tk = t0 + (t + kPfThreads * i) / CPR;
+    xtok[i] = tk < p.tokens ? tk : p.tokens - 1;
   }
   constexpr int WCPR = (WF == WF_16BIT) ? CPR : KS / 16;  // weight chunks per row (int8: 16 codes each)
   const int wcol = t % WCPR;
-  const uint8_t* wrow[WCH];
+  int wrow[WCH];     // matrix row; bit 30 set: a row of the up matrix
 #pragma unroll
-  for (int i = 0; i < WCH; ++i) wrow[i] = weight_row_ptr((t + kPfThreads * i) / WCPR);
+  for (int i = 0; i < WCH; ++i) {
+    bool up;
+    const int o = weight_row((t + kPfThreads * i) / WCPR, up);
+    wrow[i] = o | (up ? (1 << 30) : 0);
+  }
+  auto wptr = [&](int i) -> const uint8_t* {
+    if constexpr (EPI == SK_GATEUP)
+      return ((wrow[i] >> 30) ? p.w1 : p.w0) + (long)(wrow[i] & ((1 << 30) - 1)) * p.pitch;
+    else
+      return p.w0 + (long)wrow[i] * p.pitch;
+  };
 
   const int n_steps = (p.k + KS - 1) / KS;
   // one k-step of the tile in registers, on its way from global memory to LDS
@@ -137,16 +151,16 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
     const int xk = k0 + xcol * 8;
     const int xoff = xk + 8 <= p.k ? xk : 0;
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) r.x[i] = ld16(xrow[i] + xoff);
+    for (int i = 0; i < XCH; ++i) r.x[i] = ld16(p.x + (long)xtok[i] * p.k + xoff);
     if constexpr (NORM) r.g = ld16(p.gamma + xoff);
     if constexpr (WF == WF_16BIT) {
 #pragma unroll
-      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wrow[i] + 2L * xoff);
+      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wptr(i) + 2L * xoff);
     } else {
       const int wk = k0 + wcol * 16;
       const int woff = wk + 16 <= p.k ? wk : 0;
 #pragma unroll
-      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wrow[i] + woff);
+      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wptr(i) + woff);
     }
   };
 
@@ -191,7 +205,7 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   for (int i = 0; i < WR; ++i)
 #pragma unroll
     for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  if (t < TOKS) rs_lds[t] = 0.f;
+  for (int i = t; i < TOKS; i += kPfThreads) rs_lds[i] = 0.f;
 
   const int a_base = (wr * 16 * WR + (lane & 15)) * PITCH;  // rows 16 i + lane % 16: the swizzle depends on the lane only
   const int b_base = (wt * 16 * WT + (lane & 15)) * PITCH;
@@ -213,17 +227,18 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   Stage r0;
   load_step(0, r0);
   if constexpr (NBUF == 2) {
-    // two LDS stages: while step s is multiplied, step s + 1 moves from the registers to the
-    // other stage and step s + 2 is in flight from memory; one barrier per step. (A second
-    // register stage, two steps in flight, pushed the kernel past 256 registers per lane: one
-    // workgroup per CU instead of two, 686 -> 846 us on 2048 x 28672 x 4096.)
+    // two LDS stages: step s + 1 moves from the registers to the other stage and step s + 2 is
+    // requested from memory before step s is multiplied, so that the LDS writes and the loads
+    // proceed under the matrix instructions; one barrier per step. (A second register stage, two
+    // steps in flight, pushed the 128 x 128 tile past 256 registers per lane: one workgroup per
+    // CU instead of two, 686 -> 846 us on 2048 x 28672 x 4096.)
     store_step(0, 0, r0);
     load_step(1, r0);
     __syncthreads();
     for (int s = 0; s < n_steps; ++s) {
-      multiply(s & 1);
       if (s + 1 < n_steps) store_step(s + 1, (s + 1) & 1, r0);  // uniform branch, no loads inside
       load_step(s + 2, r0);
+      multiply(s & 1);
       __syncthreads();
     }
   } else {
@@ -241,7 +256,7 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
 #pragma unroll
     for (int i = 0; i < XCH; ++i) atomicAdd(&rs_lds[(t + kPfThreads * i) / CPR], ss[i]);
     __syncthreads();
-    if (t < TOKS) rs_lds[t] = rsqrtf(rs_lds[t] / (float)p.k + p.eps);
+    for (int i = t; i < TOKS; i += kPfThreads) rs_lds[i] = rsqrtf(rs_lds[i] / (float)p.k + p.eps);
     __syncthreads();
   }
 
@@ -295,17 +310,17 @@ __global__ void __launch_bounds__(kPfThreads) prefill_gemm_kernel(const PrefillG
   }
 }
 
-static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64
+static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256
 
-template <typename T, int WF, int EPI, int WR, int WT, int KS, int NBUF>
+template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int KS, int NBUF>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
-  constexpr int ROWS = 32 * WR, TOKS = 32 * WT;
+  constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   p.n_tiles = ceil_div(p.n, EPI == SK_GATEUP ? ROWS / 2 : ROWS);
   p.t_tiles = ceil_div(p.tokens, TOKS);
   // whole row tiles per XCD: the grid covers ceil(n_tiles / 8) * 8 row tiles, the surplus exits
   const long grid = (long)ceil_div(p.n_tiles, 8) * 8 * p.t_tiles;
   if (grid > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
-  constexpr size_t lds = prefill_lds_bytes<WR, WT, KS, NBUF>();
+  constexpr size_t lds = prefill_lds_bytes<ROWS, TOKS, KS, NBUF>();
   auto launch = [&](auto kernel) {
     if constexpr (lds > 65536) {
       // more dynamic LDS than the default limit: raised once per kernel (and device)
@@ -318,30 +333,33 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
         raised_for = dev;
       }
     }
-    hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(kPfThreads), lds, s, p);
+    hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(64 * NWR * NWT), lds, s, p);
     return launch_status();
   };
-  if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, KS, NBUF>);
-  return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, KS, NBUF>);
+  if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, KS, NBUF>);
+  return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, KS, NBUF>);
 }
 
 template <typename T, int WF, int EPI>
 static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
-  // The largest tile that still yields three workgroups per four CUs: big tiles re-read x and the
-  // weights least, but a grid much smaller than the chip leaves the weight stream to too few CUs
-  // (measured on the Llama-3-8B shapes: 32 x 64 wins up to 256 tokens on the 4096-row matrices,
-  // 64 x 128 at 512, 128 x 128 from 2048; the 28672 gate/up rows take 128 x 128 throughout).
+  // Big tiles re-read x and the weights least and keep the LDS traffic per matrix instruction
+  // low, but a grid much smaller than the chip leaves the work to too few CUs. Measured on the
+  // Llama-3-8B shapes: 256 x 256 (eight waves of 64 x 128) wins once it yields five workgroups
+  // per eight CUs (gate/up from 512 tokens: 129 vs 187 us; QKV at 2048: 123 vs 176 us; down at
+  // 4096: 434 vs 746 us); below that 128 x 128 while it yields three per four CUs, then 64 x 128,
+  // then 32 x 64 (up to 256 tokens on the 4096-row matrices).
   const long rows = (EPI == SK_GATEUP) ? 2L * p.n : p.n;
   const long want = 3L * device_cus() / 4;
   auto tiles = [&](int r, int tk) { return (long)ceil_div((int)rows, r) * ceil_div(p.tokens, tk); };
   int which = g_prefill_tile;
-  if (which == 0) which = tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
-  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 64, 2>(s, p);
+  if (which == 0) which = tiles(256, 256) >= 5L * device_cus() / 8 ? 4 : tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
+  if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 64, 2>(s, p);
+  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 64, 2>(s, p);
   if constexpr (EPI == SK_GATEUP) {
-    return launch_prefill_cfg<T, WF, EPI, 2, 4, 128, 1>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 128, 1>(s, p);
   } else {
-    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 128, 1>(s, p);
-    return launch_prefill_cfg<T, WF, EPI, 1, 2, 256, 1>(s, p);
+    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 128, 1>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 1, 2, 2, 2, 256, 1>(s, p);
   }
 }
 
@@ -384,7 +402,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 }  // namespace mui
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
-  if (tile < 0 || tile > 3 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  if (tile < 0 || tile > 4 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;
