@@ -49,8 +49,9 @@ struct PrefillGemmParams {
   int t_tiles;  // token tiles
 };
 
-// NWR x NWT waves per workgroup, WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile is
-// 16 WR NWR weight rows x 16 WT NWT tokens; KS k-values per step.
+// NWR x NWT x NWK waves per workgroup, WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile
+// is 16 WR NWR weight rows x 16 WT NWT tokens; KS k-values per step, of which the NWK wave groups
+// take every NWK-th 32-value chunk each (their partial tiles are added through LDS at the end).
 // dynamically sized LDS: two stages of the 128 x 128 tile exceed the 64 KB a kernel may declare statically
 extern __shared__ __align__(16) unsigned char pf_smem[];
 
@@ -59,9 +60,10 @@ constexpr size_t prefill_lds_bytes() {
   return (size_t)NBUF * (ROWS + TOKS) * KS * 2 + TOKS * 4;
 }
 
-template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int KS, int NBUF>
-__global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const PrefillGemmParams p) {
-  constexpr int kPfThreads = 64 * NWR * NWT;
+template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
+__global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(const PrefillGemmParams p) {
+  constexpr int kPfThreads = 64 * NWR * NWT * NWK;
+  static_assert((KS / 32) % NWK == 0 && WT % NWK == 0, "k-split of the waves");
   constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   // LDS rows are unpadded; 16-byte chunk c of row r lives at chunk c ^ swz(r), chosen so that the
   // 16 lanes of a 128-bit access (16 consecutive rows of one logical chunk when reading operands,
@@ -84,8 +86,9 @@ __global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const Pref
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t >> 6;
-  const int wr = wave / NWT;  // which band of the rows
-  const int wt = wave % NWT;  // which band of the tokens
+  const int wk = wave / (NWR * NWT);         // which share of every k-step
+  const int wr = (wave % (NWR * NWT)) / NWT;  // which band of the rows
+  const int wt = wave % NWT;                  // which band of the tokens
   // bank group of (row r, chunk c) is (r * chunks-per-row + c) mod 16
   auto swz = [](int r) { return CPR == 8 ? ((r >> 1) & 7) : (r & 15); };
 
@@ -212,7 +215,8 @@ __global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const Pref
   const int lsw = swz(lane & 15), lg = lane >> 4;
   auto multiply = [&](int buf) {
 #pragma unroll
-    for (int ks = 0; ks < KS / 32; ++ks) {
+    for (int kk = 0; kk < KS / 32 / NWK; ++kk) {
+      const int ks = kk * NWK + wk;
       u32x4 a[WR], b[WT];
 #pragma unroll
       for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[buf][a_base + i * 16 * PITCH + (((ks * 4 + lg) ^ lsw) * 8)];
@@ -229,9 +233,11 @@ __global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const Pref
   if constexpr (NBUF == 2) {
     // two LDS stages: step s + 1 moves from the registers to the other stage and step s + 2 is
     // requested from memory before step s is multiplied, so that the LDS writes and the loads
-    // proceed under the matrix instructions; one barrier per step. (A second register stage, two
-    // steps in flight, pushed the 128 x 128 tile past 256 registers per lane: one workgroup per
-    // CU instead of two, 686 -> 846 us on 2048 x 28672 x 4096.)
+    // proceed under the matrix instructions; one barrier per step. (A second register stage
+    // pushes the 128 x 128 tile past 256 registers per lane: one workgroup per CU instead of two,
+    // 686 -> 846 us on 2048 x 28672 x 4096; on the tiles whose waves split K, which have the
+    // registers to spare, it bought nothing either: 46 vs 41 us on 256 x 6144 x 4096 -- the
+    // staging rate of a CU, about 35 GB/s from L2 in every shape, is the limit, not the latency.)
     store_step(0, 0, r0);
     load_step(1, r0);
     __syncthreads();
@@ -251,6 +257,48 @@ __global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const Pref
     }
   }
 
+  // ---- waves that split K: wave group g keeps token tiles [g JW, (g + 1) JW) of its tile and
+  // receives the other groups' partial sums for them through LDS (the stage buffers are free: the
+  // loop ended with a barrier)
+  constexpr int JW = WT / NWK;
+  if constexpr (NWK > 1) {
+    // NWK - 1 rounds: in round r group g hands the tiles of group (g + r) % NWK to it and takes its
+    // own from group (g - r) % NWK; one area per wave
+    constexpr int AREA = WR * JW * 64;  // f32x4 slots per wave and round
+    static_assert((size_t)NWK * NWR * NWT * AREA * 16 <= (size_t)NBUF * (ROWS + TOKS) * KS * 2,
+                  "the partial tiles of a round must fit the stage buffers");
+    f32x4* red = (f32x4*)pf_smem;
+    const int wrt = wave % (NWR * NWT);
+#pragma unroll
+    for (int r = 1; r < NWK; ++r) {
+      const int to = (wk + r) % NWK, from = (wk + NWK - r) % NWK;
+      f32x4* out = red + ((long)wrt * NWK + wk) * AREA;
+#pragma unroll
+      for (int d = 0; d < NWK; ++d) {
+        if (d != to) continue;  // uniform per wave; d is a constant inside
+#pragma unroll
+        for (int i = 0; i < WR; ++i)
+#pragma unroll
+          for (int jj = 0; jj < JW; ++jj) out[(i * JW + jj) * 64 + lane] = acc[i][d * JW + jj];
+      }
+      __syncthreads();
+      const f32x4* in = red + ((long)wrt * NWK + from) * AREA;
+#pragma unroll
+      for (int d = 0; d < NWK; ++d) {
+        if (d != wk) continue;
+#pragma unroll
+        for (int i = 0; i < WR; ++i)
+#pragma unroll
+          for (int jj = 0; jj < JW; ++jj) {
+            const f32x4 v = in[(i * JW + jj) * 64 + lane];
+            f32x4& a = acc[i][d * JW + jj];
+            a = f32x4{a.x + v.x, a.y + v.y, a.z + v.z, a.w + v.w};
+          }
+      }
+      __syncthreads();
+    }
+  }
+
   // ---- per-token rsqrt(mean(x^2) + eps): every thread adds the squares it staged to its tokens
   if constexpr (NORM) {
 #pragma unroll
@@ -267,6 +315,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const Pref
   constexpr int OT = (EPI == SK_GATEUP) ? WR / 2 : WR;  // output row tiles per wave
 #pragma unroll
   for (int j = 0; j < WT; ++j) {
+    if (NWK > 1 && j / JW != wk) continue;  // another wave group finishes this token tile
     const int tl = tok_l + 16 * j;
     const int tok = t0 + tl;
     if (tok >= p.tokens) continue;
@@ -310,9 +359,10 @@ __global__ void __launch_bounds__(64 * NWR * NWT) prefill_gemm_kernel(const Pref
   }
 }
 
-static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256
+static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
+                                // 5 = 64 x 128 with the waves splitting K, 6 = 32 x 64 likewise
 
-template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int KS, int NBUF>
+template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   p.n_tiles = ceil_div(p.n, EPI == SK_GATEUP ? ROWS / 2 : ROWS);
@@ -333,11 +383,11 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
         raised_for = dev;
       }
     }
-    hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(64 * NWR * NWT), lds, s, p);
+    hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(64 * NWR * NWT * NWK), lds, s, p);
     return launch_status();
   };
-  if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, KS, NBUF>);
-  return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, KS, NBUF>);
+  if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
+  return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
 }
 
 template <typename T, int WF, int EPI>
@@ -352,14 +402,27 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   const long want = 3L * device_cus() / 4;
   auto tiles = [&](int r, int tk) { return (long)ceil_div((int)rows, r) * ceil_div(p.tokens, tk); };
   int which = g_prefill_tile;
-  if (which == 0) which = tiles(256, 256) >= 5L * device_cus() / 8 ? 4 : tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
-  if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 64, 2>(s, p);
-  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 64, 2>(s, p);
+  if (which == 0) {
+    // few output tiles (short prompts on the 4096-row matrices): one workgroup per tile whose four
+    // waves each hold the whole tile and split every k-step between them -- the LDS traffic per
+    // matrix instruction of a four times larger tile. They pay while the grid is a single round
+    // of workgroups (their 96 KB of LDS leave one per CU): 32 x 64 for up to 64 tokens on 8192 rows
+    // (o_proj at 128 tokens 21.7 vs 28.3 us, down 60 vs 91 us), 64 x 128 when that fills more
+    // than half of the CUs (down at 512 tokens 116 vs 184 us, QKV at 256 41 vs 57 us).
+    const long cus = device_cus();
+    if (EPI == SK_LINEAR && tiles(32, 64) <= cus) which = 6;
+    else if (EPI == SK_LINEAR && tiles(64, 128) <= cus && 2 * tiles(64, 128) > cus) which = 5;
+    else which = tiles(256, 256) >= 5 * cus / 8 ? 4 : tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
+  }
+  if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2>(s, p);
+  if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 8, 1, 1, 4, 128, 2>(s, p);   // 64 x 128, waves split K
+  if (which == 6) return launch_prefill_cfg<T, WF, EPI, 2, 4, 1, 1, 4, 256, 2>(s, p);   // 32 x 64, waves split K
+  if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 1, 64, 2>(s, p);
   if constexpr (EPI == SK_GATEUP) {
-    return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 128, 1>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 1, 128, 1>(s, p);
   } else {
-    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 128, 1>(s, p);
-    return launch_prefill_cfg<T, WF, EPI, 1, 2, 2, 2, 256, 1>(s, p);
+    if (which == 2) return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 1, 128, 1>(s, p);
+    return launch_prefill_cfg<T, WF, EPI, 1, 2, 2, 2, 1, 256, 1>(s, p);
   }
 }
 
@@ -370,10 +433,11 @@ static int g_wide_max_tokens = kWideDefaultMaxTokens;  // longest prompt taken b
 // int8 codes; SkinnyParams as for the decode kernels (x, residual and y dense).
 int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const SkinnyParams& q) {
   if (q.tokens < 1 || q.n < 1 || q.k < 1) return MUI_ERR_INVALID_ARG;
-  // short prompts are bound by the weight stream: few rows per workgroup, K split over the waves,
-  // no LDS tiling (gemm_wide.hip)
-  // (gemm_wide.hip); it wins while its grid is a single round of workgroups and the token tiles few
-  const bool wide_default = q.tokens <= 64 && epilogue == SK_LINEAR && ceil_div(q.n, 16) <= device_cus();
+  // the shortest prompts are bound by the weight stream: 16 rows per workgroup, K split over the
+  // waves, no LDS tiling (gemm_wide.hip). It wins while its grid is a single round of workgroups
+  // and the token tiles are few: up to 40 tokens (o_proj at 33 tokens 16.0 vs 20.4 us for the
+  // smallest LDS tile, 19.6 vs 20.6 at 48, 23.1 vs 21.2 at 64)
+  const bool wide_default = q.tokens <= 40 && epilogue == SK_LINEAR && ceil_div(q.n, 16) <= device_cus();
   if (g_wide_max_tokens == kWideDefaultMaxTokens ? wide_default : q.tokens <= g_wide_max_tokens)
     return launch_gemm_wide(s, dtype, wf, epilogue, q);
   if (!(wf == WF_16BIT || wf == WF_I8_CHANNEL)) return MUI_ERR_UNSUPPORTED;
@@ -402,7 +466,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 }  // namespace mui
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
-  if (tile < 0 || tile > 4 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  if (tile < 0 || tile > 6 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;
