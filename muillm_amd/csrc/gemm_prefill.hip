@@ -28,26 +28,6 @@
 namespace mui {
 
 
-struct PrefillGemmParams {
-  const uint8_t* w0;      // linear: matrix; gate/up: gate rows
-  const uint8_t* w1;      // gate/up: up rows
-  long pitch;             // weight row pitch in bytes
-  const uint16_t* s0;     // per-channel int8: scale of row n at s0[n * s_pitch]
-  const uint16_t* s1;
-  long s_pitch;
-  const uint16_t* x;      // [tokens, k] dense
-  const uint16_t* gamma;
-  const uint16_t* mul_bias;
-  const uint16_t* add_bias;
-  const uint16_t* residual;  // [tokens, n] dense
-  uint16_t* y;               // [tokens, n] dense
-  int n;        // outputs (weight rows; gate/up pairs)
-  int k;
-  int tokens;
-  float eps;
-  int n_tiles;  // row tiles
-  int t_tiles;  // token tiles
-};
 
 // NWR x NWT x NWK waves per workgroup, WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile
 // is 16 WR NWR weight rows x 16 WT NWT tokens; KS k-values per step, of which the NWK wave groups
@@ -65,6 +45,11 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
   constexpr int kPfThreads = 64 * NWR * NWT * NWK;
   static_assert((KS / 32) % NWK == 0 && WT % NWK == 0, "k-split of the waves");
   constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
+  // The big tiles run in grids of several rounds in which the token tiles of a row tile share its
+  // weights through L2: ordinary loads (gate/up at 4096 tokens 893 -> 865 us, down at 2048 350 ->
+  // 312 us against non-temporal ones). The small tiles of short prompts stream the weights about
+  // once: non-temporal (down at 512 tokens 116 vs 133 us).
+  constexpr bool kStreamW = ROWS * TOKS < 128 * 128;
   // LDS rows are unpadded; 16-byte chunk c of row r lives at chunk c ^ swz(r), chosen so that the
   // 16 lanes of a 128-bit access (16 consecutive rows of one logical chunk when reading operands,
   // 16 consecutive chunks when staging) fall into 16 different groups of four banks
@@ -158,12 +143,12 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
     if constexpr (NORM) r.g = ld16(p.gamma + xoff);
     if constexpr (WF == WF_16BIT) {
 #pragma unroll
-      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wptr(i) + 2L * xoff);
+      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_sel<kStreamW>(wptr(i) + 2L * xoff);
     } else {
       const int wk = k0 + wcol * 16;
       const int woff = wk + 16 <= p.k ? wk : 0;
 #pragma unroll
-      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_stream(wptr(i) + woff);
+      for (int i = 0; i < WCH; ++i) r.w[i] = ld16_sel<kStreamW>(wptr(i) + woff);
     }
   };
 

@@ -29,6 +29,28 @@ struct SkinnyParams {
   float eps;
 };
 
+// Operands of the prompt GEMM (gemm_prefill.hip)
+struct PrefillGemmParams {
+  const uint8_t* w0;      // linear: matrix; gate/up: gate rows
+  const uint8_t* w1;      // gate/up: up rows
+  long pitch;             // weight row pitch in bytes
+  const uint16_t* s0;     // per-channel int8: scale of row n at s0[n * s_pitch]
+  const uint16_t* s1;
+  long s_pitch;
+  const uint16_t* x;      // [tokens, k] dense
+  const uint16_t* gamma;
+  const uint16_t* mul_bias;
+  const uint16_t* add_bias;
+  const uint16_t* residual;  // [tokens, n] dense
+  uint16_t* y;               // [tokens, n] dense
+  int n;        // outputs (weight rows; gate/up pairs)
+  int k;
+  int tokens;
+  float eps;
+  int n_tiles;  // row tiles
+  int t_tiles;  // token tiles
+};
+
 // B operand of one k-chunk: gamma * x rounded to the 16-bit type, sum of squares on the side.
 // fp16: packed multiply (one rounding, same result as the fp32 product rounded once) and a
 // packed dot for the squares.
