@@ -303,11 +303,23 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
  * sits at key position q_start + t, keys are cache rows [0, seq_len), q_start + tokens <= seq_len.
  * The reference hands T > 1 to torch's scaled_dot_product_attention
  * (muillm/modules/attention/sdpaattention.py:221-245) after repeat_kv; here K/V are read per KV
- * head and no mask tensor is built. No padding mask: padded batches keep the SDPA route. */
+ * head and no mask tensor is built. */
 int mui_prefill_attention(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
                           const void* v_cache, long cache_batch_stride, long cache_head_stride,
                           long cache_token_stride, int seq_len, int q_start, void* out, int batch,
                           int n_q_heads, int n_kv_heads, int tokens, int head_dim);
+
+/* The same with a key-padding mask (padded batches of prompts): key_mask is [batch, >= seq_len
+ * rounded up to a multiple of 4] 16-bit entries, rows mask_batch_stride entries apart, 8-byte
+ * aligned; a key whose entry is not zero is hidden from every query, on top of causality (what the
+ * reference's additive 4-D mask amounts to when it is built from a 2-D attention mask,
+ * muillm/modules/models/llama/model.py:437-613). A query whose every visible key is hidden gets
+ * zeros. Reference route: torch SDPA with the 4-D mask (muillm/modules/attention/sdpaattention.py:221-245). */
+int mui_prefill_attention_masked(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
+                                 const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                 long cache_token_stride, int seq_len, int q_start, const void* key_mask,
+                                 long mask_batch_stride, void* out, int batch, int n_q_heads,
+                                 int n_kv_heads, int tokens, int head_dim);
 
 /* Greedy token choice: out_index[r] = argmax_v logits[r, v] (lowest index on ties, NaN never
  * wins) for a 16-bit [rows, vocab] matrix with row pitch row_stride elements. Stands in for

@@ -75,6 +75,8 @@ _SIGNATURES = {
                                       _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),
     "mui_prefill_attention": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, c_int, c_int, _P, c_int, c_int,
                                       c_int, c_int, c_int]),
+    "mui_prefill_attention_masked": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, c_int, c_int, _P, c_long, _P,
+                                             c_int, c_int, c_int, c_int, c_int]),
     "mui_argmax": (c_int, [_P, c_int, _P, c_long, _P, c_int, c_int]),
     "mui_greedy_advance": (c_int, [_P, c_int, _P, c_long, c_int, c_int, _P, _P, _P, _P, _P, c_long, c_int, _P, _P,
                                    c_int, c_long]),

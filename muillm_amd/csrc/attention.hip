@@ -688,9 +688,17 @@ struct PrefillParams {
   uint16_t* out;            // [B, T, Hq * D]
   int hq, hkv, tokens, seq_len, q_start;  // query t sits at key position q_start + t; keys [0, seq_len)
   float scale_log2;
+  const uint16_t* key_mask;  // optional [B, >= seq_len rounded up to 8]: non-zero = key hidden from every query
+  long mask_bs;
 };
 
-template <typename T, int NW>
+// four consecutive 16-bit mask entries -> is entry r hidden (anything but +-0)
+__device__ __forceinline__ bool key_hidden(const u32x2 m4, int r) {
+  const uint32_t w = (r & 2) ? m4.y : m4.x;
+  return (((r & 1) ? (w >> 16) : w) & 0x7fffu) != 0u;
+}
+
+template <typename T, int NW, bool MASKED>
 __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const PrefillParams p) {
   constexpr int kAttnThreads = NW * kWave;
   constexpr int kBlock = NW * kMfTok;
@@ -730,7 +738,9 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
   struct Block {
     u32x4 k[8];  // token base + 4 * u + g, chunk i
     u32x4 v[8];
+    u32x2 hidden[2];  // MASKED: mask entries of tokens base + 4 g .. + 3 and base + 16 + 4 g .. + 3
   };
+  const uint16_t* mrow = MASKED ? p.key_mask + (long)b * p.mask_bs : nullptr;
   auto load_block = [&](int base, Block& q) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -738,6 +748,11 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
       const long off = (long)(tok < kv_end ? tok : 0) * p.c_ts + i * 8;
       q.k[u] = ld16(kc + off);
       q.v[u] = ld16(vc + off);
+    }
+    if constexpr (MASKED) {  // groups past the key range read the row's first entries (those tokens are out of range anyway)
+      const int m0 = base + 4 * g, m1 = base + 16 + 4 * g;
+      q.hidden[0] = ld8(mrow + (m0 < kv_end ? m0 : 0));
+      q.hidden[1] = ld8(mrow + (m1 < kv_end ? m1 : 0));
     }
   };
 
@@ -762,12 +777,14 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
 #pragma unroll
   for (int db = 0; db < 8; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  u32x2 hidden_now[2] = {u32x2{0u, 0u}, u32x2{0u, 0u}};  // mask entries of the block in the LDS tiles
   auto park = [&](const Block& q) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       *(u32x4*)&k_lds[4 * u + g][i * 8] = q.k[u];
       *(u32x4*)&v_lds[4 * u + g][i * 8] = q.v[u];
     }
+    if constexpr (MASKED) { hidden_now[0] = q.hidden[0]; hidden_now[1] = q.hidden[1]; }
     __builtin_amdgcn_wave_barrier();
   };
   auto attend = [&](int base) {
@@ -784,7 +801,9 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
     for (int r = 0; r < 8; ++r) {
       const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
       const float raw = r < 4 ? s1[r] : s2[r - 4];
-      sc[r] = tok < limit_i ? raw * p.scale_log2 : -INFINITY;
+      bool seen = tok < limit_i;
+      if constexpr (MASKED) seen = seen && !key_hidden(hidden_now[r >> 2], r & 3);
+      sc[r] = seen ? raw * p.scale_log2 : -INFINITY;
       m_loc = fmaxf(m_loc, sc[r]);
     }
     m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
@@ -877,7 +896,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
 // ---------------------------------------------------------------------------------------
 constexpr int kPgTok = 64;  // tokens per LDS block
 
-template <typename T, int G>
+template <typename T, int G, bool MASKED>
 __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) attn_prefill_group_kernel(const PrefillParams p) {
   constexpr int NW = (G == 8) ? 8 : 4;
   constexpr int kThreads = NW * kWave;
@@ -886,6 +905,7 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
   constexpr int LCH = kPgTok * 16 / kThreads;  // 16-byte chunks of K (and of V) per thread and block
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[kPgTok][kMfKStride];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds[kPgTok][kMfVStride];
+  __shared__ __attribute__((aligned(16))) uint16_t hidden_lds[MASKED ? kPgTok : 8];  // mask entries of the block
 
   const int tile = gridDim.x - 1 - blockIdx.x;  // long key ranges first
   const int kvh = blockIdx.y, b = blockIdx.z;
@@ -918,6 +938,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
   const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
 
   u32x4 kreg[LCH], vreg[LCH];
+  u32x2 hreg = {0u, 0u};
+  const uint16_t* mrow = MASKED ? p.key_mask + (long)b * p.mask_bs : nullptr;
   auto load_block = [&](int base) {
 #pragma unroll
     for (int u = 0; u < LCH; ++u) {
@@ -928,6 +950,10 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
       kreg[u] = ld16(kc + off);
       vreg[u] = ld16(vc + off);
     }
+    if constexpr (MASKED) {  // every thread reads the four entries of group t % 16 (no load behind a branch); 16 threads keep them
+      const int m0 = base + 4 * (t & 15);
+      hreg = ld8(mrow + (m0 < kv_end ? m0 : 0));
+    }
   };
   auto park = [&]() {
 #pragma unroll
@@ -935,6 +961,9 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
       const int c = t + kThreads * u;
       *(u32x4*)&k_lds[c >> 4][(c & 15) * 8] = kreg[u];
       *(u32x4*)&v_lds[c >> 4][(c & 15) * 8] = vreg[u];
+    }
+    if constexpr (MASKED) {
+      if (t < 16) *(u32x2*)&hidden_lds[4 * t] = hreg;
     }
   };
 
@@ -976,6 +1005,11 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     }
     u32x4 pb[2];
     float corr[2];
+    u32x2 hid[2] = {u32x2{0u, 0u}, u32x2{0u, 0u}};
+    if constexpr (MASKED) {
+      hid[0] = *(const u32x2*)&hidden_lds[r0 + 4 * g];
+      hid[1] = *(const u32x2*)&hidden_lds[r0 + 16 + 4 * g];
+    }
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
       float sc[8];
@@ -984,7 +1018,9 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
       for (int r = 0; r < 8; ++r) {
         const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
         const float raw = r < 4 ? s1[qt][r] : s2[qt][r - 4];
-        sc[r] = tok < limit[qt] ? raw * p.scale_log2 : -INFINITY;
+        bool seen = tok < limit[qt];
+        if constexpr (MASKED) seen = seen && !key_hidden(hid[r >> 2], r & 3);
+        sc[r] = seen ? raw * p.scale_log2 : -INFINITY;
         m_loc = fmaxf(m_loc, sc[r]);
       }
       m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
@@ -1482,10 +1518,11 @@ extern "C" int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, 
   return launch_status();
 }
 
-extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
-                                     const void* v_cache, long cache_batch_stride, long cache_head_stride,
-                                     long cache_token_stride, int seq_len, int q_start, void* out, int batch,
-                                     int n_q_heads, int n_kv_heads, int tokens, int head_dim) {
+static int prefill_attention_impl(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
+                                  const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                  long cache_token_stride, int seq_len, int q_start, const void* key_mask,
+                                  long mask_batch_stride, void* out, int batch, int n_q_heads, int n_kv_heads,
+                                  int tokens, int head_dim) {
   MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
   MUI_CHECK_ARG(q_rotated && k_cache && v_cache && out);
   MUI_CHECK_ARG(batch > 0 && n_q_heads > 0 && n_kv_heads > 0 && tokens > 0 && seq_len > 0 && q_start >= 0);
@@ -1495,6 +1532,10 @@ extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void*
   if (batch > 65535 || n_q_heads > 65535) return MUI_ERR_UNSUPPORTED;
   if ((cache_token_stride & 7) || (cache_head_stride & 7) || (cache_batch_stride & 7)) return MUI_ERR_ALIGNMENT;
   if (!aligned16(k_cache) || !aligned16(v_cache)) return MUI_ERR_ALIGNMENT;
+  if (key_mask) {  // read four entries at a time
+    if (((uintptr_t)key_mask & 7) || (mask_batch_stride & 3)) return MUI_ERR_ALIGNMENT;
+    if (mask_batch_stride < (long)((seq_len + 3) / 4) * 4) return MUI_ERR_INVALID_ARG;
+  }
   PrefillParams p = {};
   p.q = (const uint16_t*)q_rotated;
   p.k_cache = (const uint16_t*)k_cache;
@@ -1503,6 +1544,8 @@ extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void*
   p.out = (uint16_t*)out;
   p.hq = n_q_heads; p.hkv = n_kv_heads; p.tokens = tokens; p.seq_len = seq_len; p.q_start = q_start;
   p.scale_log2 = kLog2e / sqrtf((float)head_dim);
+  p.key_mask = (const uint16_t*)key_mask; p.mask_bs = mask_batch_stride;
+  const bool masked = key_mask != nullptr;
   hipStream_t s = (hipStream_t)stream;
   // Long prompts with 1, 2, 4 or 8 query heads per KV head: K/V rows cross LDS once per 32 query
   // positions of the whole KV group. Short prompts keep the kernel that splits the key range of
@@ -1512,8 +1555,11 @@ extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void*
                        (g_prefill_group_tokens > 0 ? tokens >= g_prefill_group_tokens : g_prefill_group_tokens == 0 && tokens >= 512);
   if (grouped) {
 #define MUI_PG_LAUNCH(TT, GG)                                                                          \
-    hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG>), dim3(ceil_div(tokens, 128 / (GG == 8 ? 4 : GG)), n_kv_heads, batch), \
-                       dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p)
+    do {                                                                                                 \
+      const dim3 pg_grid(ceil_div(tokens, 128 / (GG == 8 ? 4 : GG)), n_kv_heads, batch);                  \
+      if (masked) hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, true>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p); \
+      else hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, false>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p);       \
+    } while (0)
     if (dtype == MUI_DTYPE_F16) {
       if (group == 1) MUI_PG_LAUNCH(F16, 1); else if (group == 2) MUI_PG_LAUNCH(F16, 2);
       else if (group == 4) MUI_PG_LAUNCH(F16, 4); else MUI_PG_LAUNCH(F16, 8);
@@ -1525,9 +1571,32 @@ extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void*
     return launch_status();
   }
   dim3 grid(ceil_div(tokens, 16), n_q_heads, batch);
-  if (dtype == MUI_DTYPE_F16)
-    hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4>), grid, dim3(4 * kWave), 0, s, p);
-  else
-    hipLaunchKernelGGL((attn_prefill_mfma_kernel<BF16, 4>), grid, dim3(4 * kWave), 0, s, p);
+  if (dtype == MUI_DTYPE_F16) {
+    if (masked) hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4, true>), grid, dim3(4 * kWave), 0, s, p);
+    else hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4, false>), grid, dim3(4 * kWave), 0, s, p);
+  } else {
+    if (masked) hipLaunchKernelGGL((attn_prefill_mfma_kernel<BF16, 4, true>), grid, dim3(4 * kWave), 0, s, p);
+    else hipLaunchKernelGGL((attn_prefill_mfma_kernel<BF16, 4, false>), grid, dim3(4 * kWave), 0, s, p);
+  }
   return launch_status();
+}
+
+extern "C" int mui_prefill_attention(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
+                                     const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                     long cache_token_stride, int seq_len, int q_start, void* out, int batch,
+                                     int n_q_heads, int n_kv_heads, int tokens, int head_dim) {
+  return prefill_attention_impl(stream, dtype, q_rotated, k_cache, v_cache, cache_batch_stride, cache_head_stride,
+                                cache_token_stride, seq_len, q_start, nullptr, 0, out, batch, n_q_heads, n_kv_heads,
+                                tokens, head_dim);
+}
+
+extern "C" int mui_prefill_attention_masked(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
+                                            const void* v_cache, long cache_batch_stride, long cache_head_stride,
+                                            long cache_token_stride, int seq_len, int q_start, const void* key_mask,
+                                            long mask_batch_stride, void* out, int batch, int n_q_heads,
+                                            int n_kv_heads, int tokens, int head_dim) {
+  MUI_CHECK_ARG(key_mask);
+  return prefill_attention_impl(stream, dtype, q_rotated, k_cache, v_cache, cache_batch_stride, cache_head_stride,
+                                cache_token_stride, seq_len, q_start, key_mask, mask_batch_stride, out, batch,
+                                n_q_heads, n_kv_heads, tokens, head_dim);
 }

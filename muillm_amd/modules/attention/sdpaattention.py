@@ -1,5 +1,7 @@
-"""MuiSdpaAttention -- muillm/modules/attention/sdpaattention.py:27-256: as MuiBaseAttention
-but multi-token inputs (prefill) go through torch's scaled_dot_product_attention."""
+"""MuiSdpaAttention -- muillm/modules/attention/sdpaattention.py:27-256: as MuiBaseAttention;
+multi-token inputs (prefill) run the library's causal kernels (with the key padding of a padded
+batch when the model hands it over), torch's scaled_dot_product_attention only for masks of another
+kind, fp32 or CPU tensors."""
 from typing import Optional, Tuple
 
 import torch
@@ -35,10 +37,11 @@ class MuiSdpaAttention(MuiBaseAttention):
     # beyond that many tokens
     prefill_kernel_max_tokens = None
 
-    def _prefill_kernel_ok(self, q, k, v, attention_mask, all_ones_mask, q_len) -> bool:
-        """T > 1 without padding (the mask, if any, is purely causal), 16-bit CUDA tensors,
-        head_dim 128, K/V being equally strided views with unit inner stride (the static cache)."""
-        if q_len <= 1 or not (all_ones_mask or attention_mask is None):
+    def _prefill_kernel_ok(self, q, k, v, attention_mask, all_ones_mask, q_len, key_padding_mask=None) -> bool:
+        """T > 1 whose mask is causal, or causal plus a key-padding mask handed over as such
+        (key_padding_mask: what the model built its 4-D mask from), 16-bit CUDA tensors, head_dim
+        128, K/V being equally strided views with unit inner stride (the static cache)."""
+        if q_len <= 1 or not (all_ones_mask or attention_mask is None or key_padding_mask is not None):
             return False
         if not (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype):
             return False
@@ -73,9 +76,11 @@ class MuiSdpaAttention(MuiBaseAttention):
             q, k, v = self.rotary_emb.apply_rotary_pos_emb_write_kv_cache(
                 q, k, position_ids, position_embeddings, v, past_key_value, cache_position)
             attn_output = self._decode_or_none(q, k, v, attention_mask, all_ones_mask, q_len)
-            if attn_output is None and self._prefill_kernel_ok(q, k, v, attention_mask, all_ones_mask, q_len):
+            key_padding_mask = None if all_ones_mask else kwargs.get("key_padding_mask")
+            if attn_output is None and self._prefill_kernel_ok(q, k, v, attention_mask, all_ones_mask, q_len,
+                                                               key_padding_mask):
                 # causal attention of the new tokens over the cache views that already hold them
-                attn_output = muillm_ext.mui_prefill_attention(q, k, v)
+                attn_output = muillm_ext.mui_prefill_attention(q, k, v, key_mask=key_padding_mask)
             if attn_output is None:
                 k = repeat_kv(k, self.num_key_value_groups)
                 v = repeat_kv(v, self.num_key_value_groups)

@@ -72,7 +72,8 @@ class MuiDecoderLayer(MuiModule):
             query_states=q, key_states=k, value_states=v, attention_mask=attention_mask,
             position_ids=position_ids, past_key_value=past_key_value, output_attentions=output_attentions,
             use_cache=use_cache, cache_position=cache_position, position_embeddings=position_embeddings,
-            all_ones_mask=all_ones_mask, residual=hidden_states)
+            all_ones_mask=all_ones_mask, residual=hidden_states,
+            key_padding_mask=kwargs.get("key_padding_mask"))
         result = [self.mlp(after_attention, residual=after_attention)]
         if output_attentions:
             result.append(attention_weights)

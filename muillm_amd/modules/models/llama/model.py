@@ -237,6 +237,13 @@ class MuiLlamaModel(MuiModule):
             causal_mask = None
         elif causal_mask is not None:
             causal_mask = causal_mask[:, :, :, :tot_seq_len]
+        # a padded prompt whose 4-D mask was built right here from a 2-D one: the attention layers
+        # get the key padding as such and keep the library's prompt kernel (a 4-D mask from the
+        # caller may hold anything and stays with SDPA)
+        key_padding_mask = None
+        if (causal_mask is not None and q_len > 1 and attention_mask is not None and attention_mask.dim() == 2
+                and torch.device(self.mdevice).type == "cuda" and self.mdtype in (torch.float16, torch.bfloat16)):
+            key_padding_mask = muillm_ext.key_padding_mask16(attention_mask, self.mdtype, tot_seq_len)
         position_ids = position_ids.contiguous()
 
         if inputs_embeds is None:
@@ -268,7 +275,7 @@ class MuiLlamaModel(MuiModule):
                 hidden_states=hidden_states, attention_mask=causal_mask, position_ids=position_ids,
                 past_key_value=past_key_values if use_cache else None, output_attentions=output_attentions,
                 use_cache=use_cache, cache_position=cache_position, position_embeddings=position_embeddings,
-                all_ones_mask=all_ones_mask)
+                all_ones_mask=all_ones_mask, key_padding_mask=key_padding_mask)
             hidden_states = layer_outputs[0]
             if output_attentions:
                 all_self_attns += (layer_outputs[1],)

@@ -1077,12 +1077,25 @@ def muillm_embedding_module_forward(module: MuiEmbeddingModule, x: torch.Tensor)
     return muillm_embedding_forward(module.engine, module.weights, x)
 
 
-def mui_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_start: Optional[int] = None) -> torch.Tensor:
+def key_padding_mask16(attention_mask: torch.Tensor, dtype: torch.dtype, seq_len: Optional[int] = None) -> torch.Tensor:
+    """The [B, S] 0 / 1 attention mask of a padded batch as mui_prefill_attention's key mask: 16-bit,
+    1 where the key is padding, rows padded with zeros to a multiple of 8 entries (the kernel reads
+    four entries at a time)."""
+    b, s_mask = attention_mask.shape
+    s = s_mask if seq_len is None else max(int(seq_len), s_mask)
+    out = torch.zeros((b, (s + 7) // 8 * 8), dtype=dtype, device=attention_mask.device)
+    out[:, :s_mask] = (attention_mask == 0).to(dtype)
+    return out
+
+
+def mui_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_start: Optional[int] = None,
+                          key_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of T > 1 new tokens over cache views that already contain them.
 
     q [B, Hq, T, D] rotated (made dense if it is not), k/v [B, Hkv, S, D] views of the static cache
     (unit inner stride, equal strides); query t sits at key position q_start + t (default S - T).
-    Returns [B, T, Hq * D]."""
+    key_mask (padded batches, see key_padding_mask16): [B, >= S rounded up to 4] in q's dtype, non-zero
+    hides the key from every query. Returns [B, T, Hq * D]."""
     _check_cuda(q, "q")
     _check_cuda(k, "k")
     _check_cuda(v, "v")
@@ -1095,6 +1108,18 @@ def mui_prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_s
     qc = q.contiguous()
     cb, chs, cts = _cache_strides(k, v)
     out = torch.empty((b, t, hq * d), dtype=q.dtype, device=q.device)
+    if key_mask is not None:
+        _check_cuda(key_mask, "key_mask")
+        if key_mask.dtype != q.dtype or key_mask.dim() != 2 or key_mask.shape[0] != b or key_mask.stride(1) != 1 \
+                or key_mask.shape[1] < (s + 3) // 4 * 4 or key_mask.device != q.device:
+            raise RuntimeError("key_mask must be [batch, >= keys rounded up to 4] in the activations' dtype, on their device")
+        check(
+            _lib.load().mui_prefill_attention_masked(_stream(qc), _dtype_code(qc), qc.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                     cb, chs, cts, s, int(q_start), key_mask.data_ptr(), key_mask.stride(0),
+                                                     out.data_ptr(), b, hq, hkv, t, d),
+            "mui_prefill_attention_masked",
+        )
+        return out
     check(
         _lib.load().mui_prefill_attention(_stream(qc), _dtype_code(qc), qc.data_ptr(), k.data_ptr(), v.data_ptr(),
                                           cb, chs, cts, s, int(q_start), out.data_ptr(), b, hq, hkv, t, d),

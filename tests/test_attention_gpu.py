@@ -396,6 +396,72 @@ def test_prefill_attention_long_prompts(b, hq, hkv, t, past, dtype, choice):
         _lib.check(lib.mui_tune_prefill_attention(0), "tune")
 
 
+@pytest.mark.parametrize("choice", ["kv-group", "per-head"])
+@pytest.mark.parametrize("b,hq,hkv,t,past,padding", [
+    (3, 32, 8, 200, 0, "left"),      # the reference's padded batches (tokenizer padding on the left)
+    (2, 32, 8, 610, 0, "left"),
+    (2, 8, 8, 97, 7, "right"),       # ragged, continues a cache, padding behind the prompt
+    (2, 16, 8, 300, 0, "holes"),     # arbitrary hidden keys
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_prefill_attention_key_padding_mask(b, hq, hkv, t, past, padding, dtype, choice):
+    """Prompt attention with a key-padding mask (mui_prefill_attention_masked) under both prompt
+    kernels against the oracle with the additive 4-D mask the reference would build
+    (muillm/modules/models/llama/model.py:437-613): every row that sees a key; rows that see none
+    (padding queries of a left-padded row) come out as zeros."""
+    lib = _lib.load()
+    _lib.check(lib.mui_tune_prefill_attention({"kv-group": 1, "per-head": -1}[choice]), "tune")
+    try:
+        g = _gen(29)
+        s = past + t
+        q = _mk((b, hq, t, D), g, dtype=dtype)
+        kc = _mk((b, hkv, s, D), g, dtype=dtype)
+        vc = _mk((b, hkv, s, D), g, dtype=dtype)
+        keep = torch.ones(b, s, dtype=torch.long)
+        for row in range(b):
+            n_pad = (37 * (row + 1)) % (t // 2)
+            if padding == "left":
+                keep[row, :n_pad] = 0
+            elif padding == "right":
+                keep[row, s - n_pad:] = 0
+            else:
+                keep[row, torch.randperm(s, generator=g)[:n_pad]] = 0
+        key_mask = muillm_ext.key_padding_mask16(keep.to(DEV), dtype)
+        assert key_mask.shape[1] % 8 == 0 and key_mask.shape[1] >= s
+        out = muillm_ext.mui_prefill_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), key_mask=key_mask)
+        assert out.shape == (b, t, hq * D) and torch.isfinite(out).all()
+        mask4 = _causal_mask(t, s, past).expand(b, 1, t, s).clone()
+        mask4 = mask4.masked_fill(keep[:, None, None, :] == 0, float("-inf"))
+        sees_a_key = torch.isfinite(mask4).any(dim=-1)[:, 0]          # [b, t]
+        safe = mask4.clone()
+        safe[~sees_a_key[:, None].expand(b, 1, t)] = 0.0                # any finite row: those outputs are not compared
+        ref = oracle.decode_attention(q, kc, vc, safe).reshape(b, t, hq * D)
+        got = out.cpu().float()
+        err = (got - ref.float()).abs().amax(dim=-1)                   # [b, t]
+        assert float(err[sees_a_key].max()) <= (ATOL if dtype == torch.float16 else 1.6e-2)
+        if (~sees_a_key).any():
+            assert float(got[~sees_a_key].abs().max()) == 0.0
+    finally:
+        _lib.check(lib.mui_tune_prefill_attention(0), "tune")
+
+
+def test_prefill_attention_masked_abi_errors():
+    lib = _lib.load()
+    q = torch.zeros(1, 8, 32, D, dtype=torch.float16, device=DEV)
+    kv = torch.zeros(1, 8, 32, D, dtype=torch.float16, device=DEV)
+    out = torch.empty(1, 32, 8 * D, dtype=torch.float16, device=DEV)
+    mask = torch.zeros(1, 32, dtype=torch.float16, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    args = (st, 0, q.data_ptr(), kv.data_ptr(), kv.data_ptr(), 8 * 32 * D, 32 * D, D, 32, 0)
+    tail = (out.data_ptr(), 1, 8, 8, 32, D)
+    assert lib.mui_prefill_attention_masked(*args, None, 32, *tail) == -1             # no mask
+    assert lib.mui_prefill_attention_masked(*args, mask.data_ptr() + 2, 32, *tail) == -4  # misaligned
+    assert lib.mui_prefill_attention_masked(*args, mask.data_ptr(), 30, *tail) == -4   # stride not a multiple of 4
+    assert lib.mui_prefill_attention_masked(*args, mask.data_ptr(), 28, *tail) == -1   # rows shorter than the keys
+    with pytest.raises(RuntimeError, match="key_mask"):
+        muillm_ext.mui_prefill_attention(q, kv, kv, key_mask=mask.to(torch.bfloat16))
+
+
 def test_prefill_attention_8k_rows_vs_oracle_and_kernels_agree():
     """An 8192-token prompt (32 / 8 heads): sampled rows against the oracle, and the two prompt
     kernels against each other on every row."""

@@ -487,6 +487,35 @@ def test_generate_left_padded_batch_matches_single_runs():
             assert agree >= n_new - 2, (use_graph, r, got, alone[r])
 
 
+def test_padded_prompt_runs_on_the_library_attention_kernel(monkeypatch):
+    """A left-padded batch of prompts must not reach torch's scaled_dot_product_attention (the
+    reference's route for masked prompts): the 2-D attention mask travels to the layers as a key
+    padding mask and the library's prompt kernel applies it. Logits of the real tokens must match
+    the rows run alone."""
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=12, init_std=0.08)
+    g = torch.Generator().manual_seed(4)
+    long_p = torch.randint(1, cfg.vocab_size, (1, 40), generator=g)
+    short_p = torch.randint(1, cfg.vocab_size, (1, 23), generator=g)
+    with torch.no_grad():
+        alone = [lm(input_ids=p.to(DEV)).logits[0, -1].float().cpu() for p in (long_p, short_p)]
+    batch = torch.zeros(2, 40, dtype=torch.int64)
+    mask = torch.zeros(2, 40, dtype=torch.int64)
+    batch[0], mask[0] = long_p[0], 1
+    batch[1, 17:], mask[1, 17:] = short_p[0], 1
+    pos = (mask.cumsum(-1) - 1).clamp(min=0)
+
+    def no_sdpa(*args, **kwargs):
+        raise AssertionError("the padded prompt fell back to torch SDPA")
+
+    monkeypatch.setattr(torch.nn.functional, "scaled_dot_product_attention", no_sdpa)
+    with torch.no_grad():
+        out = lm(input_ids=batch.to(DEV), attention_mask=mask.to(DEV), position_ids=pos.to(DEV)).logits[:, -1].float().cpu()
+    assert torch.isfinite(out).all()
+    for r in range(2):
+        assert float((out[r] - alone[r]).abs().max()) <= 3e-2 * float(alone[r].abs().max()) + 1e-3
+
+
 def test_generate_stops_at_eos_and_pads():
     cfg = _small_config()
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=9, init_std=0.08)
