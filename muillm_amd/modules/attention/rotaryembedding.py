@@ -89,6 +89,50 @@ class _MuiRotaryNoCache(torch.autograd.Function):
         raise NotImplementedError("rotary backward not implemented")
 
 
+def is_hf_static_cache(cache) -> bool:
+    """A HuggingFace StaticCache of either generation (see _hf_static_cache_layer)."""
+    if cache is None or isinstance(cache, MuiCache):
+        return False
+    layers = getattr(cache, "layers", None)
+    if isinstance(layers, (list, tuple)) and len(layers) > 0:
+        return all(type(layer).__name__ == "StaticLayer" for layer in layers)
+    return isinstance(getattr(cache, "key_cache", None), list) and hasattr(cache, "max_cache_len")
+
+
+def _hf_static_cache_layer(cache, layer_idx: int, k: torch.Tensor, v: torch.Tensor, cache_position=None):
+    """(k_cache, v_cache, seen tokens after this update) of a HuggingFace StaticCache, or None for
+    any other object. Two generations of that class are recognised by their attributes: per-layer
+    objects (`cache.layers[i]` of type StaticLayer with `keys` / `values` / `max_cache_len`, allocated
+    on first use, a device-side `cumulative_length`) and the older lists `key_cache` / `value_cache`
+    with `max_cache_len`. The seen-token count is read from cache_position by the first layer (one
+    device-to-host copy per forward; the reference keeps a counter on the cache object,
+    rotaryembedding.py:394-396 there, which a reset of the cache would leave stale) and kept on the
+    cache object for the other layers; the per-layer length counter of the newer class is advanced
+    as its own update() would."""
+    new_tokens = k.shape[-2]
+    layers = getattr(cache, "layers", None)
+    if isinstance(layers, (list, tuple)) and layer_idx < len(layers) and type(layers[layer_idx]).__name__ == "StaticLayer":
+        layer = layers[layer_idx]
+        if not getattr(layer, "is_initialized", True):
+            layer.lazy_initialization(k, v)
+        k_cache, v_cache = layer.keys, layer.values
+        if isinstance(getattr(layer, "cumulative_length", None), torch.Tensor):
+            layer.cumulative_length.add_(new_tokens)
+    elif isinstance(getattr(cache, "key_cache", None), list) and hasattr(cache, "max_cache_len") \
+            and layer_idx < len(cache.key_cache) and not isinstance(cache, MuiCache):
+        k_cache, v_cache = cache.key_cache[layer_idx], cache.value_cache[layer_idx]
+    else:
+        return None
+    if not (torch.is_tensor(k_cache) and k_cache.dim() == 4 and k_cache.shape == v_cache.shape
+            and k_cache.dtype == k.dtype and k_cache.device == k.device and k_cache.stride(3) == 1):
+        return None
+    if cache_position is None:
+        raise ValueError("cache_position is needed")
+    if layer_idx == 0 or not hasattr(cache, "_mui_seen_tokens"):
+        cache._mui_seen_tokens = int(cache_position.reshape(-1)[-1]) + 1
+    return k_cache, v_cache, min(int(cache._mui_seen_tokens), k_cache.shape[2])
+
+
 class _MuiRotaryCacheModule(torch.autograd.Function):
     @staticmethod
     def forward(ctx, module, cache, q, k, v, position_ids, cos_sin, cache_positions):
@@ -206,6 +250,13 @@ class MuiRotaryEmbedding(MuiModule):
                     raise ValueError("cache_position is needed")
                 return _MuiRotaryCacheModule.apply(self.cpp_module, cache.cpp_module, q, k, v, position_ids,
                                                    position_embeddings, cache_position)
+            hf_static = _hf_static_cache_layer(cache, self.layer_idx, k, v, cache_position)
+            if hf_static is not None:
+                # HuggingFace's StaticCache (muillm/modules/attention/rotaryembedding.py:392-418 of the
+                # reference): its per-layer buffers are written in place by the same kernel
+                k_cache, v_cache, seen = hf_static
+                return muillm_ext.muillm_rope_forward_static_cache(
+                    position_ids, self.cos32, self.sin32, q, k, v, k_cache, v_cache, cache_position, seen)
             raise ValueError(f"Unsupported cache type: {type(cache).__name__}")
 
         if position_embeddings is None:

@@ -25,7 +25,7 @@ from ...._hf import (LlamaForCausalLM, LlamaModel, MistralForCausalLM, MistralMo
 from ....engineconfig import MuiEngineConfig
 from ....memorymanagement.gc import trigger_gc
 from ....replacement.replacementcontext import MuiReplacementContext
-from ...attention.rotaryembedding import MuiRotaryEmbedding
+from ...attention.rotaryembedding import MuiRotaryEmbedding, is_hf_static_cache
 from ...attention.sdpaattention import MuiSdpaAttention, _ignore_causal_mask_sdpa
 from ...decoder.decoder import MuiDecoderLayer
 from ...decoder.decoderstack import MuiDecoderStack
@@ -197,9 +197,12 @@ class MuiLlamaModel(MuiModule):
                 "You cannot specify both input_ids and inputs_embeds at the same time, and must specify either one")
         inputs_shape = input_ids.shape if input_ids is not None else inputs_embeds.shape
         batch_size, q_len = inputs_shape[0], inputs_shape[1]
-        if past_key_values is not None and not isinstance(past_key_values, MuiCache):
-            past_key_values = None  # foreign cache types are dropped, a static cache is built instead
-        past_seen_tokens = past_key_values.get_seq_length() if past_key_values is not None else 0
+        if past_key_values is not None and not isinstance(past_key_values, MuiCache) \
+                and not is_hf_static_cache(past_key_values):
+            past_key_values = None  # other foreign cache types are dropped, a static cache is built instead
+        # (a HuggingFace StaticCache is written in place by the rotary / cache-write kernel; its layers
+        # take the per-layer route, the single-call decode step needs a MuiStaticCache)
+        past_seen_tokens = int(past_key_values.get_seq_length()) if past_key_values is not None else 0
         tot_seq_len = past_seen_tokens + q_len
         # the rotary tables have max_position_embeddings rows and the kernels index them with
         # device-side positions: refuse here what would run past them

@@ -516,6 +516,52 @@ def test_padded_prompt_runs_on_the_library_attention_kernel(monkeypatch):
         assert float((out[r] - alone[r]).abs().max()) <= 3e-2 * float(alone[r].abs().max()) + 1e-3
 
 
+def test_hf_static_cache_as_input_cache():
+    """A HuggingFace StaticCache handed to the model (the reference dispatches that type too,
+    muillm/modules/attention/rotaryembedding.py:392-418): prefill and three decode steps must give
+    the logits of the same run on a MuiStaticCache, and the HF object must end up holding the
+    rotated keys."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import LlamaConfig, StaticCache
+    from muillm_amd.modules.kvcache.cache_utils import create_static_cache
+
+    cfg = _small_config()
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=13, init_std=0.08)
+    hf_cfg = LlamaConfig(hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size,
+                         num_hidden_layers=cfg.num_hidden_layers, num_attention_heads=cfg.num_attention_heads,
+                         num_key_value_heads=cfg.num_key_value_heads, vocab_size=cfg.vocab_size,
+                         max_position_embeddings=cfg.max_position_embeddings)
+    try:
+        hf_cache = StaticCache(config=hf_cfg, max_cache_len=64)
+    except TypeError:
+        pytest.skip("this transformers version builds StaticCache differently")
+    mui_cache = create_static_cache(MuiEngineConfig(), cfg, 1, 64, DEV, torch.float16)
+    ids = torch.randint(1, cfg.vocab_size, (1, 9), generator=torch.Generator().manual_seed(5)).to(DEV)
+
+    def run(cache):
+        outs = []
+        with torch.no_grad():
+            o = lm(input_ids=ids, past_key_values=cache, use_cache=True,
+                   cache_position=torch.arange(9, device=DEV))
+            outs.append(o.logits[0, -1].float().cpu())
+            tok = o.logits[:, -1].argmax(-1, keepdim=True)
+            for step in range(3):
+                o = lm(input_ids=tok, past_key_values=cache, use_cache=True,
+                       cache_position=torch.tensor([9 + step], device=DEV),
+                       position_ids=torch.tensor([[9 + step]], device=DEV))
+                outs.append(o.logits[0, -1].float().cpu())
+                tok = o.logits[:, -1].argmax(-1, keepdim=True)
+        return outs
+
+    ref = run(mui_cache)
+    got = run(hf_cache)
+    for a, b in zip(got, ref):
+        assert float((a - b).abs().max()) <= 2e-2 * float(b.abs().max()) + 1e-3
+    layer0 = hf_cache.layers[0] if hasattr(hf_cache, "layers") else None
+    keys = layer0.keys if layer0 is not None else hf_cache.key_cache[0]
+    assert bool(keys[:, :, :12].abs().sum() > 0) and bool((keys[:, :, 12:] == 0).all())
+
+
 def test_generate_stops_at_eos_and_pads():
     cfg = _small_config()
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=9, init_std=0.08)
