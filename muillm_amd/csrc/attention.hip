@@ -933,6 +933,9 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     wave_end = last >= tpos ? p.q_start + last + 1 : 0;
     wave_end = wave_end < p.seq_len ? wave_end : p.seq_len;
   }
+  // keys below this are seen by every query of the wave: no causal test needed for such blocks
+  int wave_all_see = p.q_start + tpos + 1;
+  wave_all_see = wave_all_see < p.seq_len ? wave_all_see : p.seq_len;
 
   const uint16_t* kc = p.k_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
   const uint16_t* vc = p.v_cache + (long)b * p.c_bs + (long)kvh * p.c_hs;
@@ -988,8 +991,9 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
 #pragma unroll
     for (int db = 0; db < 8; ++db) acc[qt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // one 32-token half of the LDS block (rows r0 .. r0 + 31), key positions base ..
-  auto attend = [&](int r0, int base) {
+  // one 32-token half of the LDS block (rows r0 .. r0 + 31), key positions base ..; below_diag: every
+  // query of the wave sees every key of the half (no causal test, the common case)
+  auto attend = [&](int r0, int base, auto below_diag) {
     f32x4 s1[2], s2[2];
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) { s1[qt] = f32x4{0.f, 0.f, 0.f, 0.f}; s2[qt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
@@ -1018,9 +1022,13 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
       for (int r = 0; r < 8; ++r) {
         const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
         const float raw = r < 4 ? s1[qt][r] : s2[qt][r - 4];
-        bool seen = tok < limit[qt];
-        if constexpr (MASKED) seen = seen && !key_hidden(hid[r >> 2], r & 3);
-        sc[r] = seen ? raw * p.scale_log2 : -INFINITY;
+        if constexpr (decltype(below_diag)::value && !MASKED) {
+          sc[r] = raw * p.scale_log2;
+        } else {
+          bool seen = tok < limit[qt];
+          if constexpr (MASKED) seen = seen && !key_hidden(hid[r >> 2], r & 3);
+          sc[r] = seen ? raw * p.scale_log2 : -INFINITY;
+        }
         m_loc = fmaxf(m_loc, sc[r]);
       }
       m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
@@ -1042,17 +1050,25 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
       pb[qt].z = (uint32_t)T::pack(pr[4]) | ((uint32_t)T::pack(pr[5]) << 16);
       pb[qt].w = (uint32_t)T::pack(pr[6]) | ((uint32_t)T::pack(pr[7]) << 16);
     }
+    // the running maxima settle after the first blocks: the 64 accumulator rescalings are skipped
+    // whenever no lane of the wave raised its maximum (exp2(0) is exactly 1)
+    if (__builtin_amdgcn_ballot_w64(corr[0] != 1.f || corr[1] != 1.f) != 0) {
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int db = 0; db < 8; ++db) {
+          f32x4 a = acc[qt][db];
+          a.x *= corr[qt]; a.y *= corr[qt]; a.z *= corr[qt]; a.w *= corr[qt];
+          acc[qt][db] = a;
+        }
+    }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
       const u32x2 lo = lds_read_tr16(&v_lds[r0 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
       const u32x2 hi = lds_read_tr16(&v_lds[r0 + 16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
       const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        f32x4 a = acc[qt][db];
-        a.x *= corr[qt]; a.y *= corr[qt]; a.z *= corr[qt]; a.w *= corr[qt];
-        acc[qt][db] = attn_mfma<T>(va, pb[qt], a);
-      }
+      for (int qt = 0; qt < 2; ++qt) acc[qt][db] = attn_mfma<T>(va, pb[qt], acc[qt][db]);
     }
   };
 
@@ -1063,8 +1079,10 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     __syncthreads();
     load_block(base + kPgTok);  // in flight while this block is multiplied
     // a wave whose last query cannot see the half skips it (uniform per wave; LDS reads only)
-    if (base < wave_end) attend(0, base);
-    if (base + 32 < wave_end) attend(32, base + 32);
+    if (base + 32 <= wave_all_see) attend(0, base, std::true_type{});
+    else if (base < wave_end) attend(0, base, std::false_type{});
+    if (base + 64 <= wave_all_see) attend(32, base + 32, std::true_type{});
+    else if (base + 32 < wave_end) attend(32, base + 32, std::false_type{});
   }
 
 #pragma unroll
