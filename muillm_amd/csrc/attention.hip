@@ -1016,39 +1016,38 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     }
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
-      float sc[8];
-      float m_loc = -INFINITY;
+      // raw scores; the scale (positive) goes into the exponent's fma: p = 2^(raw * scale - m)
+      float raw[8];
+      float m_raw = -INFINITY;
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         const int tok = base + (r < 4 ? 4 * g + r : 16 + 4 * g + (r - 4));
-        const float raw = r < 4 ? s1[qt][r] : s2[qt][r - 4];
-        if constexpr (decltype(below_diag)::value && !MASKED) {
-          sc[r] = raw * p.scale_log2;
-        } else {
+        raw[r] = r < 4 ? s1[qt][r] : s2[qt][r - 4];
+        if constexpr (!(decltype(below_diag)::value && !MASKED)) {
           bool seen = tok < limit[qt];
           if constexpr (MASKED) seen = seen && !key_hidden(hid[r >> 2], r & 3);
-          sc[r] = seen ? raw * p.scale_log2 : -INFINITY;
+          raw[r] = seen ? raw[r] : -INFINITY;
         }
-        m_loc = fmaxf(m_loc, sc[r]);
+        m_raw = fmaxf(m_raw, raw[r]);
       }
-      m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
-      m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
-      const float m_new = fmaxf(m[qt], m_loc);
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 16));
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32));
+      const float m_new = fmaxf(m[qt], m_raw * p.scale_log2);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
       corr[qt] = fast_exp2(m[qt] - m_use);
       float pr[8];
       float psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
-        pr[r] = fast_exp2(sc[r] - m_use);
+        pr[r] = fast_exp2(fmaf(raw[r], p.scale_log2, -m_use));
         psum += pr[r];
       }
       l[qt] = fmaf(l[qt], corr[qt], psum);
       m[qt] = m_new;
-      pb[qt].x = (uint32_t)T::pack(pr[0]) | ((uint32_t)T::pack(pr[1]) << 16);
-      pb[qt].y = (uint32_t)T::pack(pr[2]) | ((uint32_t)T::pack(pr[3]) << 16);
-      pb[qt].z = (uint32_t)T::pack(pr[4]) | ((uint32_t)T::pack(pr[5]) << 16);
-      pb[qt].w = (uint32_t)T::pack(pr[6]) | ((uint32_t)T::pack(pr[7]) << 16);
+      pb[qt].x = T::pack2(pr[0], pr[1]);
+      pb[qt].y = T::pack2(pr[2], pr[3]);
+      pb[qt].z = T::pack2(pr[4], pr[5]);
+      pb[qt].w = T::pack2(pr[6], pr[7]);
     }
     // the running maxima settle after the first blocks: the 64 accumulator rescalings are skipped
     // whenever no lane of the wave raised its maximum (exp2(0) is exactly 1)

@@ -38,6 +38,12 @@ struct F16 {
   static __device__ __forceinline__ uint16_t pack(float v) {
     return __builtin_bit_cast(uint16_t, (_Float16)v);
   }
+  // two values -> one packed word (a in the low half): one v_cvt_pk_f16_f32, same rounding
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
 };
 
 struct BF16 {
@@ -54,6 +60,12 @@ struct BF16 {
   // fp32 -> bf16, round-to-nearest-even: the hardware convert of gfx950 (v_cvt_pk_bf16_f32)
   static __device__ __forceinline__ uint16_t pack(float v) {
     return __builtin_bit_cast(uint16_t, (__bf16)v);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   }
 };
 
