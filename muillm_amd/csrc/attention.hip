@@ -1071,6 +1071,80 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     }
   };
 
+  // a whole 64-token block that every query of the wave sees (the bulk of a long prompt): all 32
+  // score MFMAs first, ONE online-softmax step over the 16 scores per lane and query tile, then all
+  // 32 value MFMAs -- half the shuffles, rescale tests and exponentials of the running maxima of
+  // two 32-token steps, and the softmax arithmetic of one query tile can run under the matrix
+  // instructions of the other
+  auto attend_block = [&]() {
+    f32x4 sc4[2][4];  // [query tile][rows 0-15, 16-31, 32-47, 48-63 of the block]
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int h = 0; h < 4; ++h) sc4[qt][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const u32x4 ka = *(const u32x4*)&k_lds[16 * h + i][(g + 4 * j) * 8];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) sc4[qt][h] = attn_mfma<T>(ka, qreg[qt][j], sc4[qt][h]);
+      }
+    }
+    u32x4 pb[2][2];
+    float corr[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      float m_raw = -INFINITY;
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m_raw = fmaxf(m_raw, sc4[qt][h][r]);
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 16));
+      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32));
+      const float m_new = fmaxf(m[qt], m_raw * p.scale_log2);  // finite: the block is fully visible
+      corr[qt] = fast_exp2(m[qt] - m_new);
+      float pr[4][4];
+      float psum = 0.f;
+#pragma unroll
+      for (int h = 0; h < 4; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          pr[h][r] = fast_exp2(fmaf(sc4[qt][h][r], p.scale_log2, -m_new));
+          psum += pr[h][r];
+        }
+      l[qt] = fmaf(l[qt], corr[qt], psum);
+      m[qt] = m_new;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {  // B operand of a 32-token half: tokens 4 g + r, then 16 + 4 g + r
+        pb[qt][half].x = T::pack2(pr[2 * half][0], pr[2 * half][1]);
+        pb[qt][half].y = T::pack2(pr[2 * half][2], pr[2 * half][3]);
+        pb[qt][half].z = T::pack2(pr[2 * half + 1][0], pr[2 * half + 1][1]);
+        pb[qt][half].w = T::pack2(pr[2 * half + 1][2], pr[2 * half + 1][3]);
+      }
+    }
+    if (__builtin_amdgcn_ballot_w64(corr[0] != 1.f || corr[1] != 1.f) != 0) {
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int db = 0; db < 8; ++db) {
+          f32x4 a = acc[qt][db];
+          a.x *= corr[qt]; a.y *= corr[qt]; a.z *= corr[qt]; a.w *= corr[qt];
+          acc[qt][db] = a;
+        }
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int db = 0; db < 8; ++db) {
+        const u32x2 lo = lds_read_tr16(&v_lds[32 * half + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+        const u32x2 hi = lds_read_tr16(&v_lds[32 * half + 16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+        const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) acc[qt][db] = attn_mfma<T>(va, pb[qt][half], acc[qt][db]);
+      }
+  };
+
   for (int kb = 0; kb < n_blk; ++kb) {
     const int base = kb * kPgTok;
     __syncthreads();  // every wave is done with the previous block
@@ -1078,10 +1152,14 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     __syncthreads();
     load_block(base + kPgTok);  // in flight while this block is multiplied
     // a wave whose last query cannot see the half skips it (uniform per wave; LDS reads only)
-    if (base + 32 <= wave_all_see) attend(0, base, std::true_type{});
-    else if (base < wave_end) attend(0, base, std::false_type{});
-    if (base + 64 <= wave_all_see) attend(32, base + 32, std::true_type{});
-    else if (base + 32 < wave_end) attend(32, base + 32, std::false_type{});
+    if (!MASKED && base + 64 <= wave_all_see) {
+      attend_block();
+    } else {
+      if (base + 32 <= wave_all_see) attend(0, base, std::true_type{});
+      else if (base < wave_end) attend(0, base, std::false_type{});
+      if (base + 64 <= wave_all_see) attend(32, base + 32, std::true_type{});
+      else if (base + 32 < wave_end) attend(32, base + 32, std::false_type{});
+    }
   }
 
 #pragma unroll
