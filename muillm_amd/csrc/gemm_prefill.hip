@@ -14,11 +14,15 @@
 //   of squares gathered on the side) are staged through LDS in unpadded rows whose 16-byte
 //   chunks are XOR-swizzled (conflict-free 128-bit reads and writes); the loads of step s + 2 are
 //   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
-//   Four tile shapes: 256 rows x 256 tokens x 64 k with eight waves (4 x 2, each 4 x 8 MFMA
+//   Tile shapes: 256 rows x 256 tokens x 64 k with eight waves (4 x 2, each 4 x 8 MFMA
 //   tiles: 12 KB of LDS reads per 32 matrix instructions) when the grid still covers most of the
 //   chip; else 128 x 128 x 64 with four waves (2 x 2, each 4 x 4 tiles); else 64 x 128 x 128;
 //   else 32 x 64 x 256 -- the smaller the grid, the longer the k-step, so that enough weight
-//   bytes are in flight per CU.
+//   bytes are in flight per CU. For grids of at most one workgroup per CU (short prompts on
+//   matrices of a few thousand rows) two more shapes, 64 x 128 x 128 and 32 x 64 x 256, whose four
+//   waves each hold the WHOLE tile and take every fourth 32-value chunk of a k-step: the LDS
+//   traffic per matrix instruction of a tile four times the size; their partial tiles are
+//   exchanged through LDS in three rounds at the end.
 //   Under the gate/up epilogue half of a wave's rows are gate rows and the other half the up
 //   rows of the same outputs, so SiLU * mul happens in registers.
 //   Token tiles of one row tile are placed on the same XCD (workgroup id modulo 8) so that the
