@@ -32,8 +32,8 @@ def _ignore_causal_mask_sdpa(attention_mask: Optional[torch.Tensor], inputs_shap
 
 class MuiSdpaAttention(MuiBaseAttention):
     # Unpadded prompts of any length run the library's causal kernels (measured on MI355X, 32/8 heads
-    # x 128, against repeat_kv + torch SDPA: 12 vs 36 us at 128 tokens, 22 vs 52 us at 512, 105 vs
-    # 165 us at 2048, 0.95 vs 1.37 ms at 8192); None = no limit, a number restores the SDPA route
+    # x 128, against repeat_kv + torch SDPA: 12 vs 36 us at 128 tokens, 20 vs 52 us at 512, 90 vs
+    # 170 us at 2048, 0.77 vs 1.37 ms at 8192); None = no limit, a number restores the SDPA route
     # beyond that many tokens
     prefill_kernel_max_tokens = None
 
