@@ -16,7 +16,10 @@
 //   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
 //   Tile shapes: 256 rows x 256 tokens x 64 k with eight waves (4 x 2, each 4 x 8 MFMA
 //   tiles: 12 KB of LDS reads per 32 matrix instructions) when the grid still covers most of the
-//   chip; else 128 x 128 x 64 with four waves (2 x 2, each 4 x 4 tiles); else 64 x 128 x 128;
+//   chip, or 192 x 256 / 128 x 256 (eight waves, 2 x 4) when that takes fewer rounds of
+//   workgroups; else 128 x 128 x 64 or 96 x 128 x 64 with four waves (2 x 2), or 128 x 128 x 128
+//   with eight waves (two token halves, each split four ways along K) for a round or two of
+//   workgroups; else 64 x 128 x 128;
 //   else 32 x 64 x 256 -- the smaller the grid, the longer the k-step, so that enough weight
 //   bytes are in flight per CU. For grids of at most one workgroup per CU (short prompts on
 //   matrices of a few thousand rows) two more shapes, 64 x 128 x 128 and 32 x 64 x 256, whose four
@@ -64,6 +67,8 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
   constexpr int WCH = (WF == WF_16BIT) ? ROWS * CPR / kPfThreads : ROWS * (KS / 16) / kPfThreads;
   static_assert(EPI != SK_GATEUP || WR % 2 == 0, "gate/up needs an even number of row tiles per wave");
   static_assert(XCH >= 1 && WCH >= 1 && kPfThreads % CPR == 0, "tile shape");
+  static_assert(TOKS * CPR % kPfThreads == 0 && ROWS * ((WF == WF_16BIT) ? CPR : KS / 16) % kPfThreads == 0,
+                "every thread stages the same number of chunks");
   // NBUF == 2: step s + 1 is written to the other LDS stage while step s is multiplied, one
   // barrier per step instead of two
   typedef uint16_t WStage[ROWS * PITCH];
@@ -349,7 +354,9 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
 }
 
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
-                                // 5 = 64 x 128 with the waves splitting K, 6 = 32 x 64 likewise
+                                // 5 = 64 x 128 with the waves splitting K, 6 = 32 x 64 likewise,
+                                // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
+                                // 10 = 96 x 128 (linear only)
 
 template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
@@ -382,13 +389,18 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
 template <typename T, int WF, int EPI>
 static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   // Big tiles re-read x and the weights least and keep the LDS traffic per matrix instruction
-  // low, but a grid much smaller than the chip leaves the work to too few CUs. Measured on the
-  // Llama-3-8B shapes: 256 x 256 (eight waves of 64 x 128) wins once it yields five workgroups
-  // per eight CUs (gate/up from 512 tokens: 129 vs 187 us; QKV at 2048: 123 vs 176 us; down at
-  // 4096: 434 vs 746 us); below that 128 x 128 while it yields three per four CUs, then 64 x 128,
-  // then 32 x 64 (up to 256 tokens on the 4096-row matrices).
+  // low, but a grid much smaller than the chip leaves the work to too few CUs, and a grid of one
+  // and a bit rounds of workgroups costs two rounds. Each shape has a cost per round of
+  // workgroups (microseconds at K = 4096 on MI355X; only the ratios matter); the number of
+  // rounds the grid needs decides between them. Measured on the Llama-3-8B shapes: QKV at 1536
+  // tokens is 144 tiles of 256 x 256 (109 us) but 192 of 192 x 256 (100 us; the built-in choice
+  // before took 134); o_proj and down at 2048 tokens are 128 tiles of 256 x 256 (112 / 363 us)
+  // and 256 of 128 x 256 (78 / 270 us); QKV at 512 is 192 tiles of 128 x 128 (68 us), 256 of
+  // 96 x 128 (62 us). Below three workgroups of 128 x 128 per four CUs: 64 x 128, then 32 x 64 (up
+  // to 256 tokens on the 4096-row matrices).
   const long rows = (EPI == SK_GATEUP) ? 2L * p.n : p.n;
-  const long want = 3L * device_cus() / 4;
+  const long cus = device_cus();
+  const long want = 3L * cus / 4;
   auto tiles = [&](int r, int tk) { return (long)ceil_div((int)rows, r) * ceil_div(p.tokens, tk); };
   int which = g_prefill_tile;
   if (which == 0) {
@@ -398,12 +410,49 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
     // of workgroups (their 96 KB of LDS leave one per CU): 32 x 64 for up to 64 tokens on 8192 rows
     // (o_proj at 128 tokens 21.7 vs 28.3 us, down 60 vs 91 us), 64 x 128 when that fills more
     // than half of the CUs (down at 512 tokens 116 vs 184 us, QKV at 256 41 vs 57 us).
-    const long cus = device_cus();
     if (EPI == SK_LINEAR && tiles(32, 64) <= cus) which = 6;
     else if (EPI == SK_LINEAR && tiles(64, 128) <= cus && 2 * tiles(64, 128) > cus) which = 5;
-    else which = tiles(256, 256) >= 5 * cus / 8 ? 4 : tiles(128, 128) >= want ? 1 : (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
+    else if (tiles(256, 256) >= 5 * cus / 8 || 2 * tiles(128, 128) >= cus) {
+      // one workgroup per CU (eight waves): rounds x cost, a little more per round once the
+      // rounds follow each other (their weights compete for the L2)
+      auto whole = [&](long n_tiles, float one, float many) {
+        const long r = (n_tiles + cus - 1) / cus;
+        return (float)r * (r > 1 ? many : one);
+      };
+      // two workgroups per CU (four waves): up to `cus` tiles run one per CU, the next `cus` join them
+      auto pairs = [&](long n_tiles, float single, float twin) {
+        const long full = n_tiles / (2 * cus), rest = n_tiles % (2 * cus);
+        const float last = rest == 0 ? 0.f : rest <= cus ? single : single + (twin - single) * (float)(rest - cus) / (float)cus;
+        return (float)full * twin + last;
+      };
+      float best = whole(tiles(256, 256), 108.f, 116.f);
+      which = 4;
+      auto offer = [&](int id, float cost) {
+        if (cost < best * 0.97f) { best = cost; which = id; }  // bigger tiles win ties
+      };
+      // (int8 rows are staged in 16-byte chunks of 16 codes: 192 and 96 rows do not divide evenly among the threads)
+      if (WF == WF_16BIT) offer(8, whole(tiles(192, 256), 100.f, 103.f));
+      offer(7, whole(tiles(128, 256), 73.f, 76.f));
+      offer(1, pairs(tiles(128, 128), 68.f, 92.f));
+      if (EPI == SK_LINEAR && WF == WF_16BIT) offer(10, pairs(tiles(96, 128), 60.f, 76.f));
+      // 128 x 128 on eight waves that split K: the fastest single tile (QKV at 512 tokens 46 vs
+      // 62 us, o_proj at 1024 45 vs 68 us, down at 1024 143 vs 219 us), one per CU
+      offer(9, whole(tiles(128, 128), 45.f, 42.f));
+    } else {
+      which = (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
+    }
   }
   if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2>(s, p);
+  if constexpr (WF == WF_16BIT) {
+    if (which == 8) return launch_prefill_cfg<T, WF, EPI, 6, 4, 2, 4, 1, 64, 2>(s, p);  // 192 x 256, eight waves of 96 x 64
+    if constexpr (EPI == SK_LINEAR) {
+      if (which == 10) return launch_prefill_cfg<T, WF, EPI, 3, 4, 2, 2, 1, 64, 2>(s, p);  // 96 x 128, four waves of 48 x 64
+    }
+  }
+  if (which == 8) which = 7;   // int8 weights
+  if (which == 10) which = 1;  // int8 weights, gate/up
+  if (which == 7) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2>(s, p);   // 128 x 256, eight waves of 64 x 64
+  if (which == 9) return launch_prefill_cfg<T, WF, EPI, 8, 4, 1, 2, 4, 128, 2>(s, p);   // 128 x 128, eight waves: 2 token halves x 4 shares of K
   if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 8, 1, 1, 4, 128, 2>(s, p);   // 64 x 128, waves split K
   if (which == 6) return launch_prefill_cfg<T, WF, EPI, 2, 4, 1, 1, 4, 256, 2>(s, p);   // 32 x 64, waves split K
   if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 1, 64, 2>(s, p);
@@ -455,7 +504,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 }  // namespace mui
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
-  if (tile < 0 || tile > 6 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  if (tile < 0 || tile > 10 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;

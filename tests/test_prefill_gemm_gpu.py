@@ -21,14 +21,16 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
-@pytest.fixture(params=["auto", "wide", "tile-256x256", "tile-128x128", "tile-64x128", "tile-32x64", "ksplit-64x128", "ksplit-32x64"], autouse=True)
+@pytest.fixture(params=["auto", "wide", "tile-256x256", "tile-128x128", "tile-64x128", "tile-32x64", "ksplit-64x128", "ksplit-32x64", "tile-128x256", "tile-192x256", "tile-96x128", "ksplit-128x128"], autouse=True)
 def prompt_kernel_choice(request):
     """Every test runs with the built-in kernel choice and with each prompt kernel forced: the
     16-rows-per-workgroup kernel without LDS tiling (up to 128 tokens; longer prompts keep the
-    built-in choice) and the four shapes of the LDS-tiled kernel (the gate/up epilogue has no
-    32 x 64 shape and takes 64 x 128 then)."""
+    built-in choice) and the shapes of the LDS-tiled kernel (the gate/up epilogue has no
+    32 x 64 and 96 x 128 shapes and takes 64 x 128 / 128 x 128 then; int8 weights have no 192- and
+    96-row shapes and take 128 x 256 / 128 x 128)."""
     lib = _lib.load()
-    knobs = {"auto": (0, 0), "wide": (0, 128), "tile-256x256": (4, -1), "ksplit-64x128": (5, -1), "ksplit-32x64": (6, -1), "tile-128x128": (1, -1), "tile-64x128": (2, -1), "tile-32x64": (3, -1)}
+    knobs = {"auto": (0, 0), "wide": (0, 128), "tile-256x256": (4, -1), "ksplit-64x128": (5, -1), "ksplit-32x64": (6, -1), "tile-128x128": (1, -1), "tile-64x128": (2, -1), "tile-32x64": (3, -1),
+             "tile-128x256": (7, -1), "tile-192x256": (8, -1), "tile-96x128": (10, -1), "ksplit-128x128": (9, -1)}
     _lib.check(lib.mui_tune_prefill(*knobs[request.param]), "mui_tune_prefill")
     yield request.param
     _lib.check(lib.mui_tune_prefill(0, 0), "mui_tune_prefill")
