@@ -21,11 +21,12 @@
 //   with eight waves (two token halves, each split four ways along K) for a round or two of
 //   workgroups; else 64 x 128 x 128;
 //   else 32 x 64 x 256 -- the smaller the grid, the longer the k-step, so that enough weight
-//   bytes are in flight per CU. For grids of at most one workgroup per CU (short prompts on
-//   matrices of a few thousand rows) two more shapes, 64 x 128 x 128 and 32 x 64 x 256, whose four
-//   waves each hold the WHOLE tile and take every fourth 32-value chunk of a k-step: the LDS
-//   traffic per matrix instruction of a tile four times the size; their partial tiles are
-//   exchanged through LDS in three rounds at the end.
+//   bytes are in flight per CU. For grids of about one workgroup per CU (short prompts on
+//   matrices of a few thousand rows) shapes whose waves split K: 32 x 64 x 256 on four waves that
+//   each hold the WHOLE tile and take every fourth 32-value chunk of a k-step, 64 x 128 x 128 and
+//   128 x 128 x 128 on eight waves (two token halves, four shares of K): the LDS traffic per
+//   matrix instruction of a larger tile; the partial tiles are exchanged through LDS in three
+//   rounds at the end.
 //   Under the gate/up epilogue half of a wave's rows are gate rows and the other half the up
 //   rows of the same outputs, so SiLU * mul happens in registers.
 //   Token tiles of one row tile are placed on the same XCD (workgroup id modulo 8) so that the
@@ -354,7 +355,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
 }
 
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
-                                // 5 = 64 x 128 with the waves splitting K, 6 = 32 x 64 likewise,
+                                // 5 = 64 x 128 on eight waves that split K four ways, 6 = 32 x 64 on four waves that split K,
                                 // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
                                 // 10 = 96 x 128 (linear only)
 
@@ -404,15 +405,14 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   auto tiles = [&](int r, int tk) { return (long)ceil_div((int)rows, r) * ceil_div(p.tokens, tk); };
   int which = g_prefill_tile;
   if (which == 0) {
-    // few output tiles (short prompts on the 4096-row matrices): one workgroup per tile whose four
-    // waves each hold the whole tile and split every k-step between them -- the LDS traffic per
-    // matrix instruction of a four times larger tile. They pay while the grid is a single round
-    // of workgroups (their 96 KB of LDS leave one per CU): 32 x 64 for up to 64 tokens on 8192 rows
-    // (o_proj at 128 tokens 21.7 vs 28.3 us, down 60 vs 91 us), 64 x 128 when that fills more
-    // than half of the CUs (down at 512 tokens 116 vs 184 us, QKV at 256 41 vs 57 us).
+    // few output tiles (short prompts on the 4096-row matrices): one workgroup per tile whose
+    // waves split every k-step between them -- four waves that each hold the whole 32 x 64 tile,
+    // or eight waves in two token halves of a 64 x 128 or 128 x 128 tile: the LDS traffic per
+    // matrix instruction of a larger tile, and enough waves per CU although the grid is a single
+    // round of workgroups (their 96-128 KB of LDS leave one per CU). 32 x 64 for up to 64 tokens
+    // on 8192 rows (o_proj at 128 tokens 21.7 vs 28.3 us, down 60 vs 91 us).
     if (EPI == SK_LINEAR && tiles(32, 64) <= cus) which = 6;
-    else if (EPI == SK_LINEAR && tiles(64, 128) <= cus && 2 * tiles(64, 128) > cus) which = 5;
-    else if (tiles(256, 256) >= 5 * cus / 8 || 2 * tiles(128, 128) >= cus) {
+    else if (tiles(256, 256) >= 5 * cus / 8 || 2 * tiles(64, 128) > cus) {
       // one workgroup per CU (eight waves): rounds x cost, a little more per round once the
       // rounds follow each other (their weights compete for the L2)
       auto whole = [&](long n_tiles, float one, float many) {
@@ -438,6 +438,9 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
       // 128 x 128 on eight waves that split K: the fastest single tile (QKV at 512 tokens 46 vs
       // 62 us, o_proj at 1024 45 vs 68 us, down at 1024 143 vs 219 us), one per CU
       offer(9, whole(tiles(128, 128), 45.f, 42.f));
+      // 64 x 128 likewise (o_proj at 512 tokens 33 us, down 100 us, QKV at 256 34 us; four waves
+      // that each held the whole tile took 40 / 118 / 41 us)
+      offer(5, whole(tiles(64, 128), 33.5f, 32.f));
     } else {
       which = (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
     }
@@ -453,7 +456,7 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   if (which == 10) which = 1;  // int8 weights, gate/up
   if (which == 7) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2>(s, p);   // 128 x 256, eight waves of 64 x 64
   if (which == 9) return launch_prefill_cfg<T, WF, EPI, 8, 4, 1, 2, 4, 128, 2>(s, p);   // 128 x 128, eight waves: 2 token halves x 4 shares of K
-  if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 8, 1, 1, 4, 128, 2>(s, p);   // 64 x 128, waves split K
+  if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 4, 1, 2, 4, 128, 2>(s, p);   // 64 x 128, eight waves: 2 token halves x 4 shares of K
   if (which == 6) return launch_prefill_cfg<T, WF, EPI, 2, 4, 1, 1, 4, 256, 2>(s, p);   // 32 x 64, waves split K
   if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 1, 64, 2>(s, p);
   if constexpr (EPI == SK_GATEUP) {
