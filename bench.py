@@ -445,7 +445,7 @@ def probe_prompt(counters_only=False):
     for name, n, k, gateup in _PROMPT_SHAPES:
         rows = 2 * n if gateup else n
         ring = [torch.randn(rows, k, **f16) * 0.02 for _ in range(max(2, int(1e9 // (2 * rows * k)) + 1))]
-        for tokens in (64, 128, 256, 512, 2048, 4096):
+        for tokens in (64, 128, 256, 512, 1024, 2048, 4096):
             x, y = torch.randn(tokens, k, **f16), torch.empty(tokens, n, **f16)
             yt = torch.empty(tokens, rows, **f16)
             us = _event_time_us(lambda i: _prompt_gemm_call(lib, stream, ring[i % len(ring)], x, y, n, k, tokens, gateup), 20, 3)
@@ -471,7 +471,47 @@ def probe_prompt(counters_only=False):
         out["attention"]["tokens%d" % tokens] = {"us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1),
                                                  "mfma_peak_frac": round(flops / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4),
                                                  "torch_repeat_kv_sdpa_us": round(us_t, 1)}
+    out["whole_model_ms"] = _probe_prompt_whole_model()
     print(json.dumps({"probe_prompt": out}))
+
+
+def _probe_prompt_whole_model():
+    """Prefill of the 8B-shaped model (embedding to last-token logits) on the library's prompt kernels,
+    and with every linear layer of more than 32 tokens handed to torch instead (rmsnorm kernel +
+    F.linear, the reference's route for multi-token inputs) -- attention on the library's kernel in
+    both. Same process, alternating."""
+    import torch
+
+    from muillm_amd import muillm_ext
+    from muillm_amd.engineconfig import MuiEngineConfig
+    from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
+
+    cfg = MuiDecoderConfig.llama3_8b(max_position_embeddings=16384)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device="cuda", seed=0)
+    dispatchable = muillm_ext.kernel_dispatchable
+
+    def run(tokens, iters=3):
+        ids = torch.randint(0, cfg.vocab_size, (1, tokens), device="cuda")
+        with torch.no_grad():
+            for _ in range(2):
+                lm(input_ids=ids, num_logits_to_keep=1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                lm(input_ids=ids, num_logits_to_keep=1)
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters * 1e3
+
+    res = {}
+    for tokens in (64, 128, 512, 2048, 4096, 8192):
+        ours = run(tokens)
+        muillm_ext.kernel_dispatchable = lambda x: dispatchable(x) and muillm_ext._num_tokens(x) <= 32
+        try:
+            theirs = run(tokens)
+        finally:
+            muillm_ext.kernel_dispatchable = dispatchable
+        res["tokens%d" % tokens] = {"library_kernels": round(ours, 2), "torch_gemm_route": round(theirs, 2)}
+    return res
 
 
 def pmc_probe_attention(launches=3):
