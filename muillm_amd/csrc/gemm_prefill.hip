@@ -14,9 +14,8 @@
 //   of squares gathered on the side) are staged through LDS in unpadded rows whose 16-byte
 //   chunks are XOR-swizzled (conflict-free 128-bit reads and writes); the loads of step s + 2 are
 //   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
-//   Tile shapes: 256 rows x 256 tokens x 64 k with eight waves (4 x 2, each 4 x 8 MFMA
-//   tiles: 12 KB of LDS reads per 32 matrix instructions) when the grid still covers most of the
-//   chip, or 192 x 256 / 128 x 256 (eight waves, 2 x 4) when that takes fewer rounds of
+//   Tile shapes: 256 rows x 256 tokens x 64 k with sixteen waves (4 x 4, each 4 x 4 MFMA
+//   tiles) when the grid still covers most of the chip, or 192 x 256 / 128 x 256 (eight waves, 2 x 4) when that takes fewer rounds of
 //   workgroups; else 128 x 128 x 64 or 96 x 128 x 64 with four waves (2 x 2), or 128 x 128 x 128
 //   with eight waves (two token halves, each split four ways along K) for a round or two of
 //   workgroups; else 64 x 128 x 128;
@@ -425,38 +424,47 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
         const float last = rest == 0 ? 0.f : rest <= cus ? single : single + (twin - single) * (float)(rest - cus) / (float)cus;
         return (float)full * twin + last;
       };
-      float best = whole(tiles(256, 256), 108.f, 116.f);
+      float best = whole(tiles(256, 256), 100.f, 111.f);
       which = 4;
       auto offer = [&](int id, float cost) {
         if (cost < best * 0.97f) { best = cost; which = id; }  // bigger tiles win ties
       };
       // (int8 rows are staged in 16-byte chunks of 16 codes: 192 and 96 rows do not divide evenly among the threads)
       if (WF == WF_16BIT) offer(8, whole(tiles(192, 256), 100.f, 103.f));
-      offer(7, whole(tiles(128, 256), 73.f, 76.f));
+      offer(7, whole(tiles(128, 256), WF == WF_16BIT ? 67.f : 73.f, WF == WF_16BIT ? 70.f : 76.f));
       offer(1, pairs(tiles(128, 128), 68.f, 92.f));
       if (EPI == SK_LINEAR && WF == WF_16BIT) offer(10, pairs(tiles(96, 128), 60.f, 76.f));
-      // 128 x 128 on eight waves that split K: the fastest single tile (QKV at 512 tokens 46 vs
-      // 62 us, o_proj at 1024 45 vs 68 us, down at 1024 143 vs 219 us), one per CU
-      offer(9, whole(tiles(128, 128), 45.f, 42.f));
-      // 64 x 128 likewise (o_proj at 512 tokens 33 us, down 100 us, QKV at 256 34 us; four waves
+      // 128 x 128 on waves that split K: the fastest single tile (QKV at 512 tokens 43 vs 62 us,
+      // o_proj at 1024 44 vs 68 us, down at 1024 139 vs 219 us), one per CU
+      offer(9, whole(tiles(128, 128), 42.f, 40.f));
+      // 64 x 128 likewise (o_proj at 512 tokens 32 us, down 99 us, QKV at 256 33 us; four waves
       // that each held the whole tile took 40 / 118 / 41 us)
-      offer(5, whole(tiles(64, 128), 33.5f, 32.f));
+      offer(5, whole(tiles(64, 128), 32.5f, 31.f));
     } else {
       which = (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
     }
   }
-  if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2>(s, p);
+  // Sixteen waves per workgroup (four per SIMD, at most 128 registers each) on all but the smallest
+  // shapes: 3-16 % ahead of eight waves with twice the wave tile, although a wave then reads 8
+  // instead of 6 KB of operands per 16 matrix instructions -- more waves to fill the gaps between
+  // a step's phases (256 x 256: o_proj at 2048 tokens 115 -> 104 us, down 375 -> 323 us, gate/up at
+  // 4096 881 -> 854 us; 128 x 256: 75 -> 68 us per round; 128 x 128 splitting K: 46 -> 42 us).
+  // int8 rows hold a quarter of the 16-byte chunks per k-step: where sixteen waves would leave
+  // threads without a chunk to stage, the int8 kernels keep eight.
+  if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 4, 4, 4, 1, 64, 2>(s, p);      // 256 x 256, 4 x 4 waves of 64 x 64
   if constexpr (WF == WF_16BIT) {
-    if (which == 8) return launch_prefill_cfg<T, WF, EPI, 6, 4, 2, 4, 1, 64, 2>(s, p);  // 192 x 256, eight waves of 96 x 64
+    if (which == 8) return launch_prefill_cfg<T, WF, EPI, 6, 4, 2, 4, 1, 64, 2>(s, p);    // 192 x 256, 2 x 4 waves of 96 x 64
+    if (which == 7) return launch_prefill_cfg<T, WF, EPI, 2, 4, 4, 4, 1, 64, 2>(s, p);    // 128 x 256, 4 x 4 waves of 32 x 64
+    if (which == 5) return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 4, 128, 2>(s, p);   // 64 x 128, 2 x 2 waves x 4 shares of K
     if constexpr (EPI == SK_LINEAR) {
-      if (which == 10) return launch_prefill_cfg<T, WF, EPI, 3, 4, 2, 2, 1, 64, 2>(s, p);  // 96 x 128, four waves of 48 x 64
+      if (which == 10) return launch_prefill_cfg<T, WF, EPI, 3, 4, 2, 2, 1, 64, 2>(s, p);  // 96 x 128, 2 x 2 waves of 48 x 64
     }
   }
   if (which == 8) which = 7;   // int8 weights
   if (which == 10) which = 1;  // int8 weights, gate/up
-  if (which == 7) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2>(s, p);   // 128 x 256, eight waves of 64 x 64
-  if (which == 9) return launch_prefill_cfg<T, WF, EPI, 8, 4, 1, 2, 4, 128, 2>(s, p);   // 128 x 128, eight waves: 2 token halves x 4 shares of K
-  if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 4, 1, 2, 4, 128, 2>(s, p);   // 64 x 128, eight waves: 2 token halves x 4 shares of K
+  if (which == 7) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2>(s, p);      // 128 x 256, 2 x 4 waves of 64 x 64
+  if (which == 9) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 4, 128, 2>(s, p);     // 128 x 128, 2 x 2 waves x 4 shares of K
+  if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 4, 1, 2, 4, 128, 2>(s, p);     // 64 x 128, 2 token halves x 4 shares of K
   if (which == 6) return launch_prefill_cfg<T, WF, EPI, 2, 4, 1, 1, 4, 256, 2>(s, p);   // 32 x 64, waves split K
   if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 1, 64, 2>(s, p);
   if constexpr (EPI == SK_GATEUP) {
