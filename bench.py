@@ -75,8 +75,8 @@ def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=True, batch=1):
 
 def bench_prefill(lm, tokens, iters=3):
     """Prefill of one `tokens`-token prompt (batch 1, last-token logits only): every linear layer on
-    the library's prompt kernels (fused-norm matrix-core GEMMs), causal attention on its prompt
-    attention kernel. Returns ms and the arithmetic rate over the dense fp16 MFMA peak."""
+    the library's prompt kernels (rmsnorm launch + tiled matrix-core GEMM), causal attention on its
+    prompt attention kernel. Returns ms and the arithmetic rate over the dense fp16 MFMA peak."""
     import torch
 
     cfg = lm.config
