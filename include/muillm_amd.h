@@ -96,6 +96,23 @@ int mui_linear(mui_stream_t stream, int dtype, const void* weights, long w_pitch
                const void* mul_bias, const void* add_bias, const void* residual,
                void* y, int n_out, int k_in, int tokens);
 
+/* mui_linear with a scratch buffer for prompts. No counterpart in the reference (which allocates
+ * inside its calls, csrc/linear/linear.cu:178-189). With more than MUI_MAX_TOKENS tokens on a matrix of
+ * few rows and a long K (the down projection up to about 256 tokens) one workgroup per output tile
+ * would leave most of the chip idle: given a workspace, K is shared between several workgroups per
+ * tile, which exchange fp32 partial tiles through it (4096 x 14336 at 64 tokens: 44 instead of
+ * 59 us, at 256 tokens 57 instead of 109 us). workspace: mui_linear_workspace_bytes() bytes of device memory, 256-byte aligned,
+ * zero-filled ONCE by the caller before its first use (the kernels leave its counters at zero);
+ * calls that may overlap on the device (different streams) need a workspace each. workspace may
+ * be NULL (workspace_bytes 0): then, or when norm_weights is given, or for shapes that do not
+ * profit, the call is mui_linear. Results do not depend on which workgroup arrives last (the
+ * partials are added in a fixed order). */
+size_t mui_linear_workspace_bytes(void);
+int mui_linear_ws(mui_stream_t stream, int dtype, const void* weights, long w_pitch,
+                  const void* x, const void* norm_weights, float epsilon,
+                  const void* mul_bias, const void* add_bias, const void* residual,
+                  void* y, int n_out, int k_in, int tokens, void* workspace, size_t workspace_bytes);
+
 /* muillm_rmsnorm_forward (csrc/module.cpp:251; csrc/norm/rmsnorm.cu:31-85; kernel
  * csrc/norm/rmsnorm_fp16_kernels.cu:35-126).
  *   y[r, :] = weights * x[r, :] * rsqrt(mean(x[r, :]^2) + epsilon), rows r < rows.

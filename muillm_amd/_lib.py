@@ -49,6 +49,9 @@ _SIGNATURES = {
     "mui_status_string": (c_char_p, [c_int]),
     "mui_device_info": (c_int, [c_int, ctypes.POINTER(MuiDeviceInfo)]),
     "mui_linear": (c_int, [_P, c_int, _P, c_long, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_int]),
+    "mui_linear_ws": (c_int, [_P, c_int, _P, c_long, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_int, _P,
+                              ctypes.c_size_t]),
+    "mui_linear_workspace_bytes": (ctypes.c_size_t, []),
     "mui_rmsnorm": (c_int, [_P, c_int, _P, _P, c_float, _P, c_int, c_int]),
     "mui_gateup_silu": (c_int, [_P, c_int, _P, _P, c_long, _P, _P, c_float, _P, c_int, c_int, c_int]),
     "mui_silu_mul_interleaved": (c_int, [_P, c_int, _P, _P, c_long, c_int]),

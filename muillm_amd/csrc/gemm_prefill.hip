@@ -47,9 +47,31 @@ constexpr size_t prefill_lds_bytes() {
   return (size_t)NBUF * (ROWS + TOKS) * KS * 2 + TOKS * 4;
 }
 
-template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
+// partial tiles between workgroups: agent-scope relaxed atomics (write-through stores, loads that
+// bypass the non-coherent caches; the XCDs do not share an L2)
+__device__ __forceinline__ void xs_store(float* dst, f32x4 v) {
+  __hip_atomic_store((uint64_t*)dst, ((uint64_t)__float_as_uint(v.y) << 32) | __float_as_uint(v.x), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((uint64_t*)dst + 1, ((uint64_t)__float_as_uint(v.w) << 32) | __float_as_uint(v.z),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 xs_load(const float* src) {
+  const uint64_t a = __hip_atomic_load((const uint64_t*)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t b = __hip_atomic_load((const uint64_t*)src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return f32x4{__uint_as_float((uint32_t)a), __uint_as_float((uint32_t)(a >> 32)), __uint_as_float((uint32_t)b),
+               __uint_as_float((uint32_t)(b >> 32))};
+}
+
+// XS: K is also split over p.k_splits workgroups per tile (short prompts on matrices of few row
+// tiles, where one workgroup per tile would leave most CUs idle and a long K to each): every
+// workgroup delivers its partial tile in fp32 and counts itself in; whoever arrives last adds the
+// partials up in index order (the same sum whichever workgroup that is) and runs the epilogue.
+// Nobody waits for anybody.
+template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF,
+          bool XS = false>
 __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(const PrefillGemmParams p) {
   constexpr int kPfThreads = 64 * NWR * NWT * NWK;
+  static_assert(!XS || (!NORM && EPI == SK_LINEAR && NBUF == 2), "workgroups that split K: plain linear, two stages");
   static_assert((KS / 32) % NWK == 0 && WT % NWK == 0, "k-split of the waves");
   constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   // The big tiles run in grids of several rounds in which the token tiles of a row tile share its
@@ -88,9 +110,13 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
 
   // workgroup -> (row tile, token tile): consecutive workgroup ids are dealt round-robin to the
   // 8 XCDs, so ids that share id % 8 share an L2; give each XCD whole row tiles
+  // (XS: the share of K is the fastest index -- with 8 shares it is the XCD, whose L2 then holds
+  // one k-range of x for all row tiles)
+  const int xs_share = XS ? (int)(blockIdx.x % (unsigned)p.k_splits) : 0;
+  const int xs_tile = XS ? (int)(blockIdx.x / (unsigned)p.k_splits) : 0;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int tile_n = (slot / p.t_tiles) * 8 + xcd;
-  const int tile_t = slot % p.t_tiles;
+  const int tile_n = XS ? xs_tile / p.t_tiles : (slot / p.t_tiles) * 8 + xcd;
+  const int tile_t = XS ? xs_tile % p.t_tiles : slot % p.t_tiles;
   if (tile_n >= p.n_tiles) return;  // uniform for the workgroup, before any barrier
   const int o0 = tile_n * OUT_TILE;  // first output of the tile
   const int t0 = tile_t * TOKS;      // first token of the tile
@@ -222,8 +248,11 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
         for (int j = 0; j < WT; ++j) acc[i][j] = mfma16x16x32<T>(a[i], b[j], acc[i][j]);
     }
   };
+  // k-steps of this workgroup: all of them, or its share
+  const int sb = XS ? (int)((long)n_steps * xs_share / p.k_splits) : 0;
+  const int se = XS ? (int)((long)n_steps * (xs_share + 1) / p.k_splits) : n_steps;
   Stage r0;
-  load_step(0, r0);
+  load_step(sb, r0);
   if constexpr (NBUF == 2) {
     // two LDS stages: step s + 1 moves from the registers to the other stage and step s + 2 is
     // requested from memory before step s is multiplied, so that the LDS writes and the loads
@@ -232,13 +261,13 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
     // 686 -> 846 us on 2048 x 28672 x 4096; on the tiles whose waves split K, which have the
     // registers to spare, it bought nothing either: 46 vs 41 us on 256 x 6144 x 4096 -- the
     // staging rate of a CU, about 35 GB/s from L2 in every shape, is the limit, not the latency.)
-    store_step(0, 0, r0);
-    load_step(1, r0);
+    store_step(sb, 0, r0);
+    load_step(sb + 1, r0);
     __syncthreads();
-    for (int s = 0; s < n_steps; ++s) {
-      if (s + 1 < n_steps) store_step(s + 1, (s + 1) & 1, r0);  // uniform branch, no loads inside
+    for (int s = sb; s < se; ++s) {
+      if (s + 1 < se) store_step(s + 1, (s + 1 - sb) & 1, r0);  // uniform branch, no loads inside
       load_step(s + 2, r0);
-      multiply(s & 1);
+      multiply((s - sb) & 1);
       __syncthreads();
     }
   } else {
@@ -291,6 +320,44 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
       }
       __syncthreads();
     }
+  }
+
+  // ---- workgroups that split K: deliver, count, and the last one adds up
+  if constexpr (XS) {
+    constexpr int SLOT = (kPfThreads / 64) * WR * JW * 64 * 4;  // floats per partial tile
+    float* mine = p.part + ((long)xs_tile * p.k_splits + xs_share) * SLOT;
+#pragma unroll
+    for (int j = 0; j < WT; ++j) {
+      if (NWK > 1 && j / JW != wk) continue;  // tiles of another wave group (already handed over)
+#pragma unroll
+      for (int i = 0; i < WR; ++i) xs_store(mine + (((wave * WR + i) * JW + j % JW) * 64 + lane) * 4, acc[i][j]);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's stores have arrived
+    __syncthreads();                                    // ... and everybody's
+    __shared__ unsigned xs_arrived;
+    if (t == 0) xs_arrived = __hip_atomic_fetch_add(&p.part_count[xs_tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (xs_arrived + 1 != (unsigned)p.k_splits) return;  // uniform: somebody else finishes the tile
+#pragma unroll
+    for (int j = 0; j < WT; ++j) {
+      if (NWK > 1 && j / JW != wk) continue;
+#pragma unroll
+      for (int i = 0; i < WR; ++i) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int c = 0; c < p.k_splits; ++c) {
+      const float* theirs = p.part + ((long)xs_tile * p.k_splits + c) * SLOT;
+#pragma unroll
+      for (int j = 0; j < WT; ++j) {
+        if (NWK > 1 && j / JW != wk) continue;
+#pragma unroll
+        for (int i = 0; i < WR; ++i) {
+          const f32x4 v = xs_load(theirs + (((wave * WR + i) * JW + j % JW) * 64 + lane) * 4);
+          f32x4& a = acc[i][j];
+          a = f32x4{a.x + v.x, a.y + v.y, a.z + v.z, a.w + v.w};
+        }
+      }
+    }
+    if (t == 0) __hip_atomic_store(&p.part_count[xs_tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   // ---- per-token rsqrt(mean(x^2) + eps): every thread adds the squares it staged to its tokens
@@ -384,6 +451,55 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   };
   if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
   return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
+}
+
+// Workspace of the K split over workgroups (mui_linear_ws): arrival counters, then partial tiles
+constexpr int kXsMaxTiles = 1024;                              // counters
+constexpr int kXsMaxWorkgroups = 512;                          // partial tiles
+constexpr size_t kXsSlotBytes = 128 * 128 * sizeof(float);     // one 128 x 128 partial tile
+constexpr size_t kXsCounterBytes = kXsMaxTiles * sizeof(unsigned);
+size_t prefill_workspace_bytes() { return kXsCounterBytes + kXsMaxWorkgroups * kXsSlotBytes; }
+
+// shares of K per 128 x 128 tile worth taking, or 0: the grid of whole tiles leaves at least three
+// quarters of the CUs idle and every share keeps at least twelve k-steps of 128 -- the exchange
+// (write-through of the partial tile, the counter, the last workgroup's reads) costs 10-15 us, so
+// it pays on long rows only. Measured on MI355X: down 4096 x 14336 at 64 tokens 59 -> 44 us, at 256
+// tokens 109 -> 57 us (8 and 4 shares); o_proj 4096 x 4096 at 64 tokens would go 20 -> 31 us.
+static int xs_shares(const PrefillGemmParams& p) {
+  const long tiles = (long)ceil_div(p.n, 128) * ceil_div(p.tokens, 128);
+  const long cus = device_cus();
+  if (tiles > kXsMaxTiles) return 0;
+  long c = cus / tiles;
+  const long steps = ceil_div(p.k, 128);
+  if (c > steps / 12) c = steps / 12;
+  if (c > 8) c = 8;
+  if (tiles * c > kXsMaxWorkgroups) c = kXsMaxWorkgroups / tiles;
+  return c >= 4 ? (int)c : 0;
+}
+
+template <typename T>
+static int launch_prefill_xs(hipStream_t s, PrefillGemmParams p, int shares, void* workspace) {
+  constexpr int WR = 4, WT = 4, NWR = 2, NWT = 2, NWK = 4, KS = 128;  // the K-splitting 128 x 128 tile
+  constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
+  static_assert((size_t)ROWS * TOKS * sizeof(float) == kXsSlotBytes, "partial tile size");
+  p.n_tiles = ceil_div(p.n, ROWS);
+  p.t_tiles = ceil_div(p.tokens, TOKS);
+  p.k_splits = shares;
+  p.part_count = (unsigned*)workspace;
+  p.part = (float*)((char*)workspace + kXsCounterBytes);
+  const long grid = (long)p.n_tiles * p.t_tiles * shares;
+  constexpr size_t lds = prefill_lds_bytes<ROWS, TOKS, KS, 2>();
+  auto kernel = prefill_gemm_kernel<T, WF_16BIT, false, SK_LINEAR, WR, WT, NWR, NWT, NWK, KS, 2, true>;
+  static int raised_for = -1;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MUI_ERR_DEVICE;
+  if (raised_for != dev) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return MUI_ERR_LAUNCH;
+    raised_for = dev;
+  }
+  hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(64 * NWR * NWT * NWK), lds, s, p);
+  return launch_status();
 }
 
 template <typename T, int WF, int EPI>
@@ -486,18 +602,30 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
   // waves, no LDS tiling (gemm_wide.hip). It wins while its grid is a single round of workgroups
   // and the token tiles are few: up to 40 tokens (o_proj at 33 tokens 16.0 vs 20.4 us for the
   // smallest LDS tile, 19.6 vs 20.6 at 48, 23.1 vs 21.2 at 64)
-  const bool wide_default = q.tokens <= 40 && epilogue == SK_LINEAR && ceil_div(q.n, 16) <= device_cus();
-  if (g_wide_max_tokens == kWideDefaultMaxTokens ? wide_default : q.tokens <= g_wide_max_tokens)
-    return launch_gemm_wide(s, dtype, wf, epilogue, q);
-  if (!(wf == WF_16BIT || wf == WF_I8_CHANNEL)) return MUI_ERR_UNSUPPORTED;
-  if (q.k % (wf == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
-  if (q.x_pitch != 0 && q.x_pitch != q.k) return MUI_ERR_UNSUPPORTED;
   PrefillGemmParams p = {};
   const long esz = (wf == WF_16BIT) ? 2 : 1;
   p.w0 = (const uint8_t*)q.w0; p.w1 = (const uint8_t*)q.w1; p.pitch = q.pitch * esz;
   p.s0 = q.s0; p.s1 = q.s1; p.s_pitch = q.s_pitch;
   p.x = q.x; p.gamma = q.gamma; p.mul_bias = q.mul_bias; p.add_bias = q.add_bias; p.residual = q.residual;
   p.y = q.y; p.n = q.n; p.k = q.k; p.tokens = q.tokens; p.eps = q.eps;
+  // a caller-provided workspace lets a long K be shared between workgroups when the tiles are few
+  // (in front of the 16-rows-per-workgroup kernel only for K beyond 8192: down at 33 tokens 31 vs 50 us)
+  const bool wide_default = q.tokens <= 40 && epilogue == SK_LINEAR && ceil_div(q.n, 16) <= device_cus();
+  const bool wide = g_wide_max_tokens == kWideDefaultMaxTokens ? wide_default : q.tokens <= g_wide_max_tokens;
+  if (q.workspace && g_prefill_tile == 0 && g_wide_max_tokens == kWideDefaultMaxTokens && wf == WF_16BIT &&
+      epilogue == SK_LINEAR && !q.gamma && q.k % 8 == 0 && (q.x_pitch == 0 || q.x_pitch == q.k) &&
+      ((uintptr_t)q.workspace & 255u) == 0 && q.workspace_bytes >= prefill_workspace_bytes() &&
+      (!wide || q.k > 8192)) {
+    const int shares = xs_shares(p);
+    if (shares) {
+      if (dtype == MUI_DTYPE_F16) return launch_prefill_xs<F16>(s, p, shares, q.workspace);
+      if (dtype == MUI_DTYPE_BF16) return launch_prefill_xs<BF16>(s, p, shares, q.workspace);
+    }
+  }
+  if (wide) return launch_gemm_wide(s, dtype, wf, epilogue, q);
+  if (!(wf == WF_16BIT || wf == WF_I8_CHANNEL)) return MUI_ERR_UNSUPPORTED;
+  if (q.k % (wf == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
+  if (q.x_pitch != 0 && q.x_pitch != q.k) return MUI_ERR_UNSUPPORTED;
 #define MUI_PF_CASE(TT, WFV, EPIV) \
   if (dtype == TT::kDtype && wf == WFV && epilogue == EPIV) return launch_prefill_t<TT, WFV, EPIV>(s, p);
   MUI_PF_CASE(F16, WF_16BIT, SK_LINEAR)

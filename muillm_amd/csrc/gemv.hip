@@ -301,11 +301,23 @@ extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
   return MUI_OK;
 }
 
+extern "C" size_t mui_linear_workspace_bytes(void) { return prefill_workspace_bytes(); }
+
 extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, long w_pitch,
                           const void* x, const void* norm_weights, float epsilon,
                           const void* mul_bias, const void* add_bias, const void* residual,
                           void* y, int n_out, int k_in, int tokens) {
+  return mui_linear_ws(stream, dtype, weights, w_pitch, x, norm_weights, epsilon, mul_bias, add_bias, residual, y,
+                       n_out, k_in, tokens, nullptr, 0);
+}
+
+extern "C" int mui_linear_ws(mui_stream_t stream, int dtype, const void* weights, long w_pitch,
+                             const void* x, const void* norm_weights, float epsilon,
+                             const void* mul_bias, const void* add_bias, const void* residual,
+                             void* y, int n_out, int k_in, int tokens, void* workspace,
+                             size_t workspace_bytes) {
   MUI_CHECK_ARG(weights && x && y);
+  MUI_CHECK_ARG(workspace || workspace_bytes == 0);
   MUI_CHECK_ARG(n_out > 0 && k_in > 0 && tokens > 0);
   MUI_CHECK_ARG(dtype == MUI_DTYPE_F16 || dtype == MUI_DTYPE_BF16);
   if (w_pitch < k_in) return MUI_ERR_INVALID_ARG;
@@ -320,6 +332,7 @@ extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, l
     sp.mul_bias = (const uint16_t*)mul_bias; sp.add_bias = (const uint16_t*)add_bias;
     sp.residual = (const uint16_t*)residual; sp.y = (uint16_t*)y; sp.n = n_out; sp.k = k_in; sp.tokens = tokens;
     sp.eps = epsilon;
+    sp.workspace = workspace; sp.workspace_bytes = workspace_bytes;
     return launch_prefill_gemm(s, dtype, WF_16BIT, SK_LINEAR, sp);
   }
   if (tokens >= g_skinny_min_tokens || g_gemv_dot2) {

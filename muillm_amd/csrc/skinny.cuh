@@ -27,6 +27,8 @@ struct SkinnyParams {
   int k;
   int tokens;  // 1..16
   float eps;
+  void* workspace;         // optional scratch of the prompt GEMM (mui_linear_ws), zeroed once by the caller
+  size_t workspace_bytes;
 };
 
 // Operands of the prompt GEMM (gemm_prefill.hip)
@@ -49,6 +51,10 @@ struct PrefillGemmParams {
   float eps;
   int n_tiles;  // row tiles
   int t_tiles;  // token tiles
+  // K split over workgroups (prefill_gemm_kernel<..., XS = true>): partial tiles and arrival counters
+  int k_splits;
+  float* part;            // [tiles * k_splits] partial tiles in fp32
+  unsigned* part_count;   // [tiles], zero between launches
 };
 
 // B operand of one k-chunk: gamma * x rounded to the 16-bit type, sum of squares on the side.
@@ -143,6 +149,7 @@ __device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint1
 
 // tiled matrix-core GEMM for prompts (gemm_prefill.hip): any token count, 16-bit or per-channel int8
 int launch_prefill_gemm(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
+size_t prefill_workspace_bytes();  // what SkinnyParams::workspace must hold for the prompt GEMM to use it
 // 17..128 tokens: 16 weight rows per workgroup, K split over its waves, token columns in up to 8 MFMA tiles (gemm_wide.hip)
 int launch_gemm_wide(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 // launches gemm_skinny_kernel<dtype, weight format, epilogue>; returns a MUI_* status

@@ -118,6 +118,22 @@ def _norm_first(x: torch.Tensor, norm_weights: Optional[torch.Tensor], epsilon: 
     return x, norm_weights
 
 
+# Scratch of the prompt GEMM (mui_linear_ws), one per device and stream: calls on one stream follow
+# each other and can share it, calls on different streams may overlap. Zero-filled once.
+_PROMPT_WORKSPACES: dict = {}
+
+
+def _prompt_workspace(x: torch.Tensor) -> Optional[torch.Tensor]:
+    key = (x.device.index, torch.cuda.current_stream(x.device).cuda_stream)
+    ws = _PROMPT_WORKSPACES.get(key)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None  # no allocation inside a capture: the call runs without the workspace
+        ws = torch.zeros(_lib.load().mui_linear_workspace_bytes(), dtype=torch.uint8, device=x.device)
+        _PROMPT_WORKSPACES[key] = ws
+    return ws
+
+
 def _token_calls(tokens: int, chunk_max: int):
     """(first token, count) of the library calls that cover `tokens` rows: chunks of MUI_MAX_TOKENS
     for the decode kernels up to chunk_max tokens, one call (the tiled GEMM) beyond."""
@@ -247,13 +263,15 @@ def muillm_linear_forward(
         residual = residual.contiguous()
     y = torch.empty(out_shape, dtype=x.dtype, device=x.device)
     lib, stream, code, esz = _lib.load(), _stream(x), _dtype_code(x), x.element_size()
+    ws = _prompt_workspace(x) if tokens > FUSED_CHUNK_MAX_TOKENS else None
     for off, cnt in _token_calls(tokens, FUSED_CHUNK_MAX_TOKENS):
         check(
-            lib.mui_linear(
+            lib.mui_linear_ws(
                 stream, code, weights.data_ptr(), pitch, x.data_ptr() + off * k * esz,
                 _ptr(norm_weights), float(epsilon), _ptr(mul_bias), _ptr(add_bias),
                 None if residual is None else residual.data_ptr() + off * n * esz,
                 y.data_ptr() + off * n * esz, n, k, cnt,
+                None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(),
             ),
             "mui_linear",
         )
