@@ -402,15 +402,16 @@ _PROMPT_SHAPES = (("qkv", 6144, 4096, False), ("o_proj", 4096, 4096, False), ("g
                   ("down", 4096, 14336, False))
 
 
-def _prompt_gemm_call(lib, stream, w, x, y, n, k, tokens, gateup):
+def _prompt_gemm_call(lib, stream, w, x, y, n, k, tokens, gateup, ws=None):
     from muillm_amd import _lib
 
     if gateup:
         _lib.check(lib.mui_gateup_silu(stream, 0, w.data_ptr(), w.data_ptr() + 2 * k, 2 * k, x.data_ptr(), None, 0.0,
                                        y.data_ptr(), n, k, tokens), "mui_gateup_silu")
     else:
-        _lib.check(lib.mui_linear(stream, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(),
-                                  n, k, tokens), "mui_linear")
+        _lib.check(lib.mui_linear_ws(stream, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(),
+                                     n, k, tokens, None if ws is None else ws.data_ptr(),
+                                     0 if ws is None else ws.numel()), "mui_linear_ws")
 
 
 def probe_prompt(counters_only=False):
@@ -442,13 +443,14 @@ def probe_prompt(counters_only=False):
                                                "attention_flops_per_launch": 4.0 * hq * d * 4096 * 4096 / 2}}))
         return
     out = {"linears": {}, "attention": {}}
+    ws = torch.zeros(lib.mui_linear_workspace_bytes(), dtype=torch.uint8, device="cuda")  # as the host layer passes it
     for name, n, k, gateup in _PROMPT_SHAPES:
         rows = 2 * n if gateup else n
         ring = [torch.randn(rows, k, **f16) * 0.02 for _ in range(max(2, int(1e9 // (2 * rows * k)) + 1))]
         for tokens in (64, 128, 256, 512, 1024, 2048, 4096):
             x, y = torch.randn(tokens, k, **f16), torch.empty(tokens, n, **f16)
             yt = torch.empty(tokens, rows, **f16)
-            us = _event_time_us(lambda i: _prompt_gemm_call(lib, stream, ring[i % len(ring)], x, y, n, k, tokens, gateup), 20, 3)
+            us = _event_time_us(lambda i: _prompt_gemm_call(lib, stream, ring[i % len(ring)], x, y, n, k, tokens, gateup, ws), 20, 3)
             us_t = _event_time_us(lambda i: torch.matmul(x, ring[i % len(ring)].t(), out=yt), 20, 3)
             flops = 2.0 * tokens * rows * k
             out["linears"]["%s_tokens%d" % (name, tokens)] = {
