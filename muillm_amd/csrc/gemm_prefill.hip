@@ -423,7 +423,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
                                 // 5 = 64 x 128 on eight waves that split K four ways, 6 = 32 x 64 on four waves that split K,
                                 // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
-                                // 10 = 96 x 128 (linear only)
+                                // 10 = 96 x 128 (linear only), 11 = 128 x 64 on sixteen waves that split K four ways
 
 template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
@@ -553,6 +553,9 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
       // 128 x 128 on waves that split K: the fastest single tile (QKV at 512 tokens 43 vs 62 us,
       // o_proj at 1024 44 vs 68 us, down at 1024 139 vs 219 us), one per CU
       offer(9, whole(tiles(128, 128), 42.f, 40.f));
+      // the same with 64-token tiles: half the token bytes per workgroup for prompts of up to 64
+      // tokens (gate/up at 64 tokens 57 -> 50 us)
+      offer(11, whole(tiles(128, 64), 37.f, 36.5f));
       // 64 x 128 likewise (o_proj at 512 tokens 32 us, down 99 us, QKV at 256 33 us; four waves
       // that each held the whole tile took 40 / 118 / 41 us)
       offer(5, whole(tiles(64, 128), 32.5f, 31.f));
@@ -580,6 +583,7 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   if (which == 10) which = 1;  // int8 weights, gate/up
   if (which == 7) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2>(s, p);      // 128 x 256, 2 x 4 waves of 64 x 64
   if (which == 9) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 4, 128, 2>(s, p);     // 128 x 128, 2 x 2 waves x 4 shares of K
+  if (which == 11) return launch_prefill_cfg<T, WF, EPI, 2, 4, 4, 1, 4, 128, 2>(s, p);    // 128 x 64, 4 x 1 waves x 4 shares of K
   if (which == 5) return launch_prefill_cfg<T, WF, EPI, 4, 4, 1, 2, 4, 128, 2>(s, p);     // 64 x 128, 2 token halves x 4 shares of K
   if (which == 6) return launch_prefill_cfg<T, WF, EPI, 2, 4, 1, 1, 4, 256, 2>(s, p);   // 32 x 64, waves split K
   if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 1, 64, 2>(s, p);
@@ -643,7 +647,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 }  // namespace mui
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
-  if (tile < 0 || tile > 10 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  if (tile < 0 || tile > 11 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;
