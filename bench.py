@@ -477,6 +477,29 @@ def probe_prompt(counters_only=False):
     print(json.dumps({"probe_prompt": out}))
 
 
+def trace_prefill(tokens, passes=3):
+    """Prefill passes of the 8B-shaped fp16 model (embedding to last-token logits) for a kernel trace:
+    two warm-up passes, then `passes` passes with a device synchronisation after each."""
+    import torch
+
+    from muillm_amd.engineconfig import MuiEngineConfig
+    from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
+
+    cfg = MuiDecoderConfig.llama3_8b(max_position_embeddings=16384)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device="cuda", seed=0)
+    ids = torch.randint(0, cfg.vocab_size, (1, tokens), device="cuda")
+    with torch.no_grad():
+        for _ in range(2):
+            lm(input_ids=ids, num_logits_to_keep=1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(passes):
+            lm(input_ids=ids, num_logits_to_keep=1)
+            torch.cuda.synchronize()
+    print(json.dumps({"trace_prefill": {"tokens": tokens, "passes": passes,
+                                        "ms_per_pass": round((time.perf_counter() - t0) / passes * 1e3, 3)}}))
+
+
 def _probe_prompt_whole_model():
     """Prefill of the 8B-shaped model (embedding to last-token logits) on the library's prompt kernels,
     and with every linear layer of more than 32 tokens handed to torch instead (rmsnorm kernel +
@@ -853,6 +876,8 @@ def main():
                     help="time fused flash decoding at batch 1 over the number of sequence splits and exit")
     ap.add_argument("--probe-prompt", action="store_true",
                     help="time the prompt GEMMs and prompt attention at the Llama-3-8B shapes beside torch and exit")
+    ap.add_argument("--trace-prefill", type=int, default=0, metavar="TOKENS",
+                    help="a few prefill passes of the 8B-shaped model at this prompt length (for rocprofv3 --kernel-trace)")
     ap.add_argument("--pmc-probe-prompt", action="store_true",
                     help="launch the gate/up prompt GEMM (2048 tokens) and prompt attention (4096) three times and exit "
                          "(for rocprofv3 --pmc)")
@@ -888,6 +913,9 @@ def main():
         return
     if args.probe_prompt or args.pmc_probe_prompt:
         probe_prompt(counters_only=args.pmc_probe_prompt)
+        return
+    if args.trace_prefill:
+        trace_prefill(args.trace_prefill)
         return
     if args.tune_attention:
         from muillm_amd import _lib
