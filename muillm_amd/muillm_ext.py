@@ -9,8 +9,9 @@ stream to libmuillm_amd.so.
 
 Dispatch rule (csrc/modules/linear_module.cpp:39-80 hands everything but a single token to the
 framework's GEMM): here the library's kernels serve 16-bit CUDA tensors of any token count --
-1..MUI_MAX_TOKENS tokens the weight-streaming decode kernels (up to FUSED_CHUNK_MAX_TOKENS in
-chunks), longer prompts the tiled matrix-core GEMM behind the same entry points. Only fp32 and CPU
+1..MUI_MAX_TOKENS tokens the weight-streaming decode kernels, more tokens the tiled matrix-core GEMM
+behind the same entry points (FUSED_CHUNK_MAX_TOKENS can send short prompts through the decode
+kernels in chunks instead). Only fp32 and CPU
 tensors take the reference's unfused route (RMSNorm, torch matmul, residual add).  There is no
 CPU fallback for CUDA inputs and no silent one for a missing library.
 """
@@ -91,10 +92,11 @@ def _check_activations(x: torch.Tensor, k: int, what: str, max_tokens: int, *oth
             raise RuntimeError(f"{what}: every operand must live on the activations' device {x.device}")
 
 
-# Short prompts: up to this many tokens go through the decode kernels in chunks of MUI_MAX_TOKENS
-# (each chunk streams the weights once more with the GEMVs' long contiguous runs); longer ones take
-# the tiled matrix-core GEMM of the same entry points in one call (weights read once per 128 tokens).
-FUSED_CHUNK_MAX_TOKENS = 32
+# Up to this many tokens go through the decode kernels in chunks of MUI_MAX_TOKENS (each chunk
+# streams the weights once more); more take the tiled matrix-core GEMM of the same entry points in
+# one call. MUI_MAX_TOKENS = no chunking: an 8B-shaped prefill of 17-32 tokens takes 5.4-5.5 ms on the
+# GEMM against 5.8-6.3 ms in two chunks.
+FUSED_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
 
 
 def kernel_dispatchable(x: torch.Tensor) -> bool:
@@ -379,9 +381,12 @@ def _byte_pitch(w: torch.Tensor, name: str) -> int:
 
 
 # int8 weights: the decode kernels take chunks of MUI_MAX_TOKENS up to this many tokens; beyond, the
-# tiled matrix-core GEMM converts the codes on their way to LDS (per-channel format) or runs on the
-# matrix dequantised by the library's kernel (group format).
-INT8_CHUNK_MAX_TOKENS = 64
+# tiled matrix-core GEMM converts the codes on their way to LDS (per-channel format: no chunking,
+# 64 tokens of an 8B-shaped prefill take 5.6 ms on the GEMM against 8.9 ms in four chunks) or runs
+# on the matrix dequantised by the library's kernel (group format: dequantising every matrix costs
+# about 4 ms per 8B-shaped pass, two chunks of the decode kernels less).
+INT8_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
+INT8_GROUP_CHUNK_MAX_TOKENS = 32
 
 
 def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
@@ -390,9 +395,9 @@ def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
         and x.shape[-1] % 16 == 0 and (x.shape[-1] <= 16384 or x.dtype == torch.float16)
 
 
-def _token_chunks(tokens: int):
+def _token_chunks(tokens: int, group_format: bool = False):
     """(first token, count) of the int8 calls that cover `tokens` rows."""
-    return _token_calls(tokens, INT8_CHUNK_MAX_TOKENS)
+    return _token_calls(tokens, INT8_GROUP_CHUNK_MAX_TOKENS if group_format else INT8_CHUNK_MAX_TOKENS)
 
 
 def mui_int8_channel_dequantize_forward(weights_i8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
@@ -517,7 +522,7 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
     _check_contiguous(scales_min_vals, "scales_min_vals")
     _check_activations(x, k, "muillm_int8_linear_forward", _MAX_CALL_TOKENS, weights,
                        scales_min_vals, norm_weights, add_bias, residual)
-    if _num_tokens(x) > INT8_CHUNK_MAX_TOKENS:
+    if _num_tokens(x) > INT8_GROUP_CHUNK_MAX_TOKENS:
         # a prompt: the reference's route (dequantise the matrix, then a GEMM,
         # muillm/modules/quantized/int8linear.py:279-293) on this library's kernels
         w = muillm_int8_dequantize_forward(weights, scales_min_vals, group_size_shift)
@@ -534,7 +539,7 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
         residual = residual.contiguous()
     y = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
     esz = x.element_size()
-    for off, cnt in _token_chunks(tokens):
+    for off, cnt in _token_chunks(tokens, group_format=True):
         check(
             _lib.load().mui_int8_group_linear(_stream(x), _dtype_code(x), weights.data_ptr(),
                                               _byte_pitch(weights, "weights"), scales_min_vals.data_ptr(),
@@ -621,7 +626,7 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
         raise RuntimeError("gate_up_scales_min_vals must hold N * 2 * K / group (scale, min) pairs in the activation dtype")
     if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
         raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
-    if _num_tokens(x) > INT8_CHUNK_MAX_TOKENS:
+    if _num_tokens(x) > INT8_GROUP_CHUNK_MAX_TOKENS:
         # a prompt: dequantise gate and up once, then the tiled GEMM with the SiLU * mul epilogue
         gd, ud = muillm_int8_gateupsilu_dequantize_forward(gate_up_weights, gate_up_scales_min_vals, group_size_shift)
         return mui_gateup_silu(norm_weights, epsilon, gd, ud, x)
@@ -631,7 +636,7 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
     h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
     gw, uw = gate_up_weights[:, 0, :], gate_up_weights[:, 1, :]
     esz = x.element_size()
-    for off, cnt in _token_chunks(tokens):
+    for off, cnt in _token_chunks(tokens, group_format=True):
         check(
             _lib.load().mui_int8_group_gateup_silu(_stream(x), _dtype_code(x), gw.data_ptr(), uw.data_ptr(),
                                                    2 * k, smv[:, 0].data_ptr(), smv[:, 1].data_ptr(), 4 * g,

@@ -228,11 +228,14 @@ def test_int8_abi_errors():
     assert_parity(yy, oracle.int8_channel_linear(xx, q, s_), 1e-2, "K=24")
 
 
+@pytest.mark.parametrize("chunk_max", [16, 64])
 @pytest.mark.parametrize("tokens", [17, 40, 64])
-def test_channel_linear_and_gateup_in_chunks(tokens):
-    """17..64 tokens go through the 16-token int8 kernels in chunks (the alternative would be
-    dequantising the whole matrix for a library GEMM)."""
-    assert muillm_ext.INT8_CHUNK_MAX_TOKENS == 64
+def test_channel_linear_and_gateup_short_prompts(tokens, chunk_max, monkeypatch):
+    """17..64 tokens: the tiled GEMM converting the codes on the way (the default), or the 16-token
+    int8 kernels in chunks when the chunk limit is raised -- never a dequantised matrix for a
+    library GEMM."""
+    assert muillm_ext.INT8_CHUNK_MAX_TOKENS == 16 and muillm_ext.INT8_GROUP_CHUNK_MAX_TOKENS == 32
+    monkeypatch.setattr(muillm_ext, "INT8_CHUNK_MAX_TOKENS", chunk_max)
     g = _gen(31)
     n, k = 264, 1024
     w = _mk((n, k), g, 0.02)
@@ -253,7 +256,8 @@ def test_channel_linear_and_gateup_in_chunks(tokens):
     assert_parity(h, ref_h, 1e-2, f"int8 gate/up chunks {tokens}")
     # longer prompts stay on the library's kernels too (the tiled GEMM of the same entry points)
     assert muillm_ext.int8_kernel_dispatchable(torch.zeros(65, k, dtype=torch.float16, device=DEV))
-    assert muillm_ext._token_chunks(64) == [(0, 16), (16, 16), (32, 16), (48, 16)] and muillm_ext._token_chunks(65) == [(0, 65)]
+    assert muillm_ext._token_calls(64, 64) == [(0, 16), (16, 16), (32, 16), (48, 16)] and muillm_ext._token_calls(65, 64) == [(0, 65)]
+    assert muillm_ext._token_chunks(32, group_format=True) == [(0, 16), (16, 16)] and muillm_ext._token_chunks(33, group_format=True) == [(0, 33)]
 
 
 def test_wrappers_refuse_mismatched_operands():

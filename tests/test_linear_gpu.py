@@ -381,10 +381,13 @@ def test_read_probe_reads_and_discards():
     assert lib.mui_probe_read(stream, None, 64, sink.data_ptr()) != 0
 
 
+@pytest.mark.parametrize("chunk_max", [16, 32])
 @pytest.mark.parametrize("tokens", [17, 32])
-def test_short_prompt_goes_through_the_fused_kernels_in_chunks(tokens):
-    """17..32 tokens: two calls of the 16-token kernels instead of norm + library GEMM + add."""
-    assert muillm_ext.FUSED_CHUNK_MAX_TOKENS == 32
+def test_short_prompt_on_the_library_kernels(tokens, chunk_max, monkeypatch):
+    """17..32 tokens: the tiled GEMM in one call (the default: FUSED_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS),
+    or two calls of the 16-token kernels when the chunk limit is raised -- never norm + library GEMM + add."""
+    assert muillm_ext.FUSED_CHUNK_MAX_TOKENS == 16
+    monkeypatch.setattr(muillm_ext, "FUSED_CHUNK_MAX_TOKENS", chunk_max)
     g = _gen(90 + tokens)
     n, k = 520, 1024
     w = _mk((n, k), g, 0.02)
