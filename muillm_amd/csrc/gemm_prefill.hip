@@ -6,7 +6,9 @@
 // muillm/modules/gateupdownmlp.py:343-359: norm, two matmuls, SiLU, multiply, matmul, add;
 // int8: dequantise the whole matrix first, muillm/modules/quantized/int8linear.py:279-293).
 // Here one kernel does y = (W . (gamma * x)) * rsqrt(mean(x^2) + eps) [* scale] [* mul_bias]
-// [+ add_bias] [+ residual], or h = silu(G xn) * (U xn), for 16-bit or per-channel int8 weights.
+// [+ add_bias] [+ residual], or h = silu(G xn) * (U xn), for 16-bit or per-channel int8 weights
+// (gamma optional: the host layer normalises prompts with one rmsnorm launch in front, which is
+// cheaper than redoing the norm in every row tile).
 //
 // Work layout (wave64, v_mfma_f32_16x16x32):
 //   a workgroup owns a tile of weight rows x tokens and walks K in steps: the weight tile (int8
@@ -14,18 +16,18 @@
 //   of squares gathered on the side) are staged through LDS in unpadded rows whose 16-byte
 //   chunks are XOR-swizzled (conflict-free 128-bit reads and writes); the loads of step s + 2 are
 //   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
-//   Tile shapes: 256 rows x 256 tokens x 64 k with sixteen waves (4 x 4, each 4 x 4 MFMA
-//   tiles) when the grid still covers most of the chip, or 192 x 256 / 128 x 256 (eight waves, 2 x 4) when that takes fewer rounds of
-//   workgroups; else 128 x 128 x 64 or 96 x 128 x 64 with four waves (2 x 2), or 128 x 128 x 128
-//   with eight waves (two token halves, each split four ways along K) for a round or two of
-//   workgroups; else 64 x 128 x 128;
-//   else 32 x 64 x 256 -- the smaller the grid, the longer the k-step, so that enough weight
-//   bytes are in flight per CU. For grids of about one workgroup per CU (short prompts on
-//   matrices of a few thousand rows) shapes whose waves split K: 32 x 64 x 256 on four waves that
-//   each hold the WHOLE tile and take every fourth 32-value chunk of a k-step, 64 x 128 x 128 and
-//   128 x 128 x 128 on eight waves (two token halves, four shares of K): the LDS traffic per
-//   matrix instruction of a larger tile; the partial tiles are exchanged through LDS in three
-//   rounds at the end.
+//   Tile shapes, chosen per call by rounds of workgroups x cost per round (launch_prefill_t):
+//   256 rows x 256 tokens x 64 k and 128 x 256 x 64 on sixteen waves (4 x 4), 192 x 256 x 64 on
+//   eight (2 x 4) while the grid covers most of the chip; 128 x 128 x 64 and 96 x 128 x 64 on four
+//   waves (2 x 2), two workgroups per CU; 64 x 128 x 128 and 32 x 64 x 256 with a single LDS stage
+//   for small matrices. For grids of a round or two of workgroups (short prompts, matrices of a few
+//   thousand rows) shapes whose waves ALSO split K, each taking every fourth 32-value chunk of a
+//   k-step: 128 x 128 x 128, 128 x 64 x 128 and 64 x 128 x 128 on sixteen waves, 32 x 64 x 256 on
+//   eight -- the LDS traffic per matrix instruction of a larger tile and four waves per SIMD
+//   although there is one workgroup per CU; their partial tiles are exchanged through LDS in three
+//   rounds at the end. (int8 weights keep eight / four waves where more would leave threads
+//   without a chunk to stage.) With a caller-provided workspace a long K is shared between
+//   workgroups as well (XS below).
 //   Under the gate/up epilogue half of a wave's rows are gate rows and the other half the up
 //   rows of the same outputs, so SiLU * mul happens in registers.
 //   Token tiles of one row tile are placed on the same XCD (workgroup id modulo 8) so that the
@@ -33,8 +35,6 @@
 #include "skinny.cuh"
 
 namespace mui {
-
-
 
 // NWR x NWT x NWK waves per workgroup, WR x WT MFMA tiles (16 x 16) per wave: the workgroup tile
 // is 16 WR NWR weight rows x 16 WT NWT tokens; KS k-values per step, of which the NWK wave groups
