@@ -84,6 +84,41 @@ __device__ __forceinline__ float dot2_acc<BF16>(uint32_t a, uint32_t b, float c)
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Maximum / sum over the four 16-lane rows of a wave (lanes i, i + 16, i + 32, i + 48), the same
+// value in all four: gfx950's row-swap instructions exchange rows between two registers in the
+// vector ALU, without the LDS round trip of ds_bpermute that a shuffle by 16 or 32 lanes costs.
+// (permlane16_swap: rows 1, 3 of the first operand <-> rows 0, 2 of the second; permlane32_swap:
+// upper half of the first <-> lower half of the second.) The additions pair the rows as the two
+// shuffles did -- (r0 + r1) + (r2 + r3) --, so the results are bit-identical.
+__device__ __forceinline__ float rows_max(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned w = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned w = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+// The two registers of one swap: OFF = 16 -> a = rows (0, 0, 2, 2), b = rows (1, 1, 3, 3) of v;
+// OFF = 32 -> a = rows (0, 1, 0, 1), b = rows (2, 3, 2, 3). Every row sees its own value in one of
+// them and its partner's (lane ^ OFF) in the other, in the same order in all rows.
+template <int OFF>
+__device__ __forceinline__ void rows_pair(float v, float& a, float& b) {
+  const unsigned u = __float_as_uint(v);
+  if constexpr (OFF == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+  } else {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+  }
+}
+
 // rotate-half RoPE of element d of a 128-wide head held at `src` (16-bit), fp32 math:
 //   r = x * cos[d mod 64] + (d < 64 ? -x[d+64] : x[d-64]) * sin[d mod 64]
 template <typename T>
@@ -320,22 +355,30 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
     attend_block<T, G, 1>(kreg, vreg, valid, madd, qreg, p.scale_log2, m, l, acc);
   }
 
-  // ---- stage 1: merge the 4 workers (DPP rows) of each wave with cross-row shuffles; every
-  //      row ends up with the wave's combined (m, l, acc) ----
-#pragma unroll
-  for (int off = 16; off <= 32; off <<= 1) {
+  // ---- stage 1: merge the 4 workers (DPP rows) of each wave with row swaps in the vector ALU
+  //      (no LDS round trips); every row ends up with the wave's combined (m, l, acc) ----
+  auto merge_rows = [&](auto off_tag) {
+    constexpr int OFF = decltype(off_tag)::value;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const float mo = __shfl_xor(m[g], off);
-      const float mn = fmaxf(m[g], mo);
+      float ma, mb, la, lb;
+      rows_pair<OFF>(m[g], ma, mb);
+      rows_pair<OFF>(l[g], la, lb);
+      const float mn = fmaxf(ma, mb);
       const float mu = (mn == -INFINITY) ? 0.f : mn;
-      const float fs = fast_exp2(m[g] - mu), fo = fast_exp2(mo - mu);
-      l[g] = l[g] * fs + __shfl_xor(l[g], off) * fo;
+      const float fa = fast_exp2(ma - mu), fb = fast_exp2(mb - mu);
+      l[g] = la * fa + lb * fb;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[g][i] = acc[g][i] * fs + __shfl_xor(acc[g][i], off) * fo;
+      for (int i = 0; i < 8; ++i) {
+        float xa, xb;
+        rows_pair<OFF>(acc[g][i], xa, xb);
+        acc[g][i] = xa * fa + xb * fb;
+      }
       m[g] = mn;
     }
-  }
+  };
+  merge_rows(std::integral_constant<int, 16>{});
+  merge_rows(std::integral_constant<int, 32>{});
   // ---- stage 2: merge the NW waves through LDS ----
   if (lane == 0) {
 #pragma unroll
@@ -581,8 +624,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
       sc[r] = ok ? raw * p.scale_log2 : -INFINITY;
       m_loc = fmaxf(m_loc, sc[r]);
     }
-    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
-    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+    m_loc = rows_max(m_loc);
     const float m_new = fmaxf(m, m_loc);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     const float corr = fast_exp2(m - m_use);
@@ -623,8 +665,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
   if (mrow != nullptr) sweep(std::true_type{}); else sweep(std::false_type{});
 
   // ---- the wave's totals: l summed over the four lane groups (m is already shared) ----
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
+  l = rows_sum(l);
 
   // ---- merge the NW waves through LDS (the V tiles are dead: every wave has finished) ----
   __syncthreads();
@@ -713,7 +754,8 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
   __shared__ __attribute__((aligned(16))) uint16_t k_tiles[NW][kMfTok][kMfKStride];
   uint16_t (*k_lds)[kMfKStride] = k_tiles[threadIdx.x >> 6];
 
-  const int t0 = blockIdx.x * 16, head = blockIdx.y, b = blockIdx.z;
+  // grid = (Hq * B, position tiles): x is handed out first, so every head's long tiles start first
+  const int t0 = (gridDim.y - 1 - blockIdx.y) * 16, head = blockIdx.x % p.hq, b = blockIdx.x / p.hq;
   const int kvh = head / (p.hq / p.hkv);
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
@@ -806,8 +848,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
       sc[r] = seen ? raw * p.scale_log2 : -INFINITY;
       m_loc = fmaxf(m_loc, sc[r]);
     }
-    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16));
-    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32));
+    m_loc = rows_max(m_loc);
     const float m_new = fmaxf(m, m_loc);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     const float corr = fast_exp2(m - m_use);
@@ -844,8 +885,7 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
     __builtin_amdgcn_wave_barrier();  // the tiles are rewritten by the next park
   }
 
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
+  l = rows_sum(l);
 
   __syncthreads();
   if (g == 0) lds_m[wave][i] = m;
@@ -881,7 +921,11 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
 // Causal attention for long prompts: every K/V row that crosses LDS serves 32 query positions of
 // ALL query heads of its KV head.
 //
-// grid = (position tiles, Hkv, B), heaviest (last) position tile first. A workgroup has one wave
+// grid = (Hkv * B, position tiles): workgroups are handed out x first, so the heaviest (last)
+// position tile of EVERY KV head starts before any lighter tile -- with the tiles of one head
+// after another the last heads' long tiles started when the chip was half done (64 % of the CU
+// time busy at 4096 tokens) --, and with Hkv * B a multiple of the eight XCDs each XCD's L2 sees
+// the K/V of its own heads only. A workgroup has one wave
 // per (query head of the KV group, block of 32 query positions): NW = 4 waves for 1, 2 or 4 heads
 // per KV head (4, 2, 1 position blocks), 8 waves for 8. The workgroup walks the causal key range
 // in blocks of 64 tokens: all threads load the block's K and V rows in their natural layout (whole
@@ -907,8 +951,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
   __shared__ __attribute__((aligned(16))) uint16_t v_lds[kPgTok][kMfVStride];
   __shared__ __attribute__((aligned(16))) uint16_t hidden_lds[MASKED ? kPgTok : 8];  // mask entries of the block
 
-  const int tile = gridDim.x - 1 - blockIdx.x;  // long key ranges first
-  const int kvh = blockIdx.y, b = blockIdx.z;
+  const int tile = gridDim.y - 1 - blockIdx.y;  // long key ranges first
+  const int kvh = blockIdx.x % p.hkv, b = blockIdx.x / p.hkv;
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t >> 6;
@@ -1030,8 +1074,7 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
         }
         m_raw = fmaxf(m_raw, raw[r]);
       }
-      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 16));
-      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32));
+      m_raw = rows_max(m_raw);
       const float m_new = fmaxf(m[qt], m_raw * p.scale_log2);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
       corr[qt] = fast_exp2(m[qt] - m_use);
@@ -1082,6 +1125,9 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
       for (int h = 0; h < 4; ++h) sc4[qt][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // the wave that multiplies goes first: the other wave of the SIMD fits its softmax arithmetic
+    // between the matrix instructions
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -1091,6 +1137,20 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
         for (int qt = 0; qt < 2; ++qt) sc4[qt][h] = attn_mfma<T>(ka, qreg[qt][j], sc4[qt][h]);
       }
     }
+    // pinned order: the K operands of two k-slices requested up front, then eight matrix
+    // instructions per four further reads (left alone the compiler reuses one operand register
+    // set and waits for an LDS read right before half of the multiplies)
+    {
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      __builtin_amdgcn_sched_barrier(0x6);  // only scalar and vector ALU work may move across
+    }
+    __builtin_amdgcn_s_setprio(0);
     u32x4 pb[2][2];
     float corr[2];
 #pragma unroll
@@ -1100,8 +1160,7 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
       for (int h = 0; h < 4; ++h)
 #pragma unroll
         for (int r = 0; r < 4; ++r) m_raw = fmaxf(m_raw, sc4[qt][h][r]);
-      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 16));
-      m_raw = fmaxf(m_raw, __shfl_xor(m_raw, 32));
+      m_raw = rows_max(m_raw);
       const float m_new = fmaxf(m[qt], m_raw * p.scale_log2);  // finite: the block is fully visible
       corr[qt] = fast_exp2(m[qt] - m_new);
       float pr[4][4];
@@ -1133,6 +1192,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
           acc[qt][db] = a;
         }
     }
+    __builtin_amdgcn_sched_barrier(0x6);
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int half = 0; half < 2; ++half)
 #pragma unroll
@@ -1143,6 +1204,16 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) acc[qt][db] = attn_mfma<T>(va, pb[qt][half], acc[qt][db]);
       }
+    {  // four value tiles requested ahead, then two reads per two matrix instructions
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
+#pragma unroll
+      for (int r = 0; r < 12; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 1);
+    }
+    __builtin_amdgcn_s_setprio(0);
   };
 
   for (int kb = 0; kb < n_blk; ++kb) {
@@ -1165,8 +1236,7 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
     float lt = l[qt];
-    lt += __shfl_xor(lt, 16);
-    lt += __shfl_xor(lt, 32);
+    lt = rows_sum(lt);
     const int pos = tpos + 16 * qt + i;
     if (pos >= p.tokens) continue;
     const float inv = lt > 0.f ? 1.f / lt : 0.f;
@@ -1733,9 +1803,10 @@ static int prefill_attention_impl(mui_stream_t stream, int dtype, const void* q_
   const bool grouped = (group == 1 || group == 2 || group == 4 || group == 8) &&
                        (g_prefill_group_tokens > 0 ? tokens >= g_prefill_group_tokens : g_prefill_group_tokens == 0 && tokens >= 512);
   if (grouped) {
+    if (ceil_div(tokens, 16) > 65535) return MUI_ERR_UNSUPPORTED;  // position tiles are the grid's y
 #define MUI_PG_LAUNCH(TT, GG)                                                                          \
     do {                                                                                                 \
-      const dim3 pg_grid(ceil_div(tokens, 128 / (GG == 8 ? 4 : GG)), n_kv_heads, batch);                  \
+      const dim3 pg_grid(n_kv_heads * batch, ceil_div(tokens, 128 / (GG == 8 ? 4 : GG)));                 \
       if (masked) hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, true>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p); \
       else hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, false>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p);       \
     } while (0)
@@ -1749,7 +1820,8 @@ static int prefill_attention_impl(mui_stream_t stream, int dtype, const void* q_
 #undef MUI_PG_LAUNCH
     return launch_status();
   }
-  dim3 grid(ceil_div(tokens, 16), n_q_heads, batch);
+  if (ceil_div(tokens, 16) > 65535) return MUI_ERR_UNSUPPORTED;
+  dim3 grid(n_q_heads * batch, ceil_div(tokens, 16));
   if (dtype == MUI_DTYPE_F16) {
     if (masked) hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4, true>), grid, dim3(4 * kWave), 0, s, p);
     else hipLaunchKernelGGL((attn_prefill_mfma_kernel<F16, 4, false>), grid, dim3(4 * kWave), 0, s, p);
