@@ -22,8 +22,8 @@
 //   waves (2 x 2), two workgroups per CU; 64 x 128 x 128 and 32 x 64 x 256 with a single LDS stage
 //   for small matrices. For grids of a round or two of workgroups (short prompts, matrices of a few
 //   thousand rows) shapes whose waves ALSO split K, each taking every fourth 32-value chunk of a
-//   k-step: 128 x 128 x 128, 128 x 64 x 128 and 64 x 128 x 128 on sixteen waves, 32 x 64 x 256 on
-//   eight -- the LDS traffic per matrix instruction of a larger tile and four waves per SIMD
+//   k-step: 128 x 128 x 128, 128 x 64 x 128 and 64 x 128 x 128 on sixteen waves, 64 x 64 x 256 and
+//   32 x 64 x 256 on eight -- the LDS traffic per matrix instruction of a larger tile and four waves per SIMD
 //   although there is one workgroup per CU; their partial tiles are exchanged through LDS in three
 //   rounds at the end. (int8 weights keep eight / four waves where more would leave threads
 //   without a chunk to stage.) With a caller-provided workspace a long K is shared between
@@ -423,7 +423,8 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
                                 // 5 = 64 x 128 on eight waves that split K four ways, 6 = 32 x 64 on four waves that split K,
                                 // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
-                                // 10 = 96 x 128 (linear only), 11 = 128 x 64 on sixteen waves that split K four ways
+                                // 10 = 96 x 128 (linear only), 11 = 128 x 64 on sixteen waves that split K four ways,
+                                // 12 = 64 x 64 on eight waves that split K four ways (linear only)
 
 template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
@@ -527,6 +528,9 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
     // round of workgroups (their 96-128 KB of LDS leave one per CU). 32 x 64 for up to 64 tokens
     // on 8192 rows (o_proj at 128 tokens 21.7 vs 28.3 us, down 60 vs 91 us).
     if (EPI == SK_LINEAR && tiles(32, 64) <= cus) which = 6;
+    // ... and 64 x 64 while that is still a single round: QKV at 128 tokens 33 -> 24.5 us, o_proj at
+    // 256 tokens 32 -> 23.5 us (k-steps of 128 instead of 256: 28.6 / 27.2 us)
+    else if (EPI == SK_LINEAR && tiles(64, 64) <= cus) which = 12;
     else if (tiles(256, 256) >= 5 * cus / 8 || 2 * tiles(64, 128) > cus) {
       // one workgroup per CU (eight waves): rounds x cost, a little more per round once the
       // rounds follow each other (their weights compete for the L2)
@@ -588,7 +592,12 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   if constexpr (EPI == SK_LINEAR && WF == WF_16BIT) {
     // 32 x 64 on eight waves (2 row halves x 4 shares of K): QKV at 64 tokens 21.7 -> 20.7 us, o_proj 20.2 -> 19.1 us
     if (which == 6) return launch_prefill_cfg<T, WF, EPI, 1, 4, 2, 1, 4, 256, 2>(s, p);
+    if (which == 12) return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 1, 4, 256, 2>(s, p);  // 64 x 64 likewise
   }
+  if constexpr (EPI == SK_LINEAR) {
+    if (which == 12) return launch_prefill_cfg<T, WF, EPI, 4, 4, 1, 1, 4, 256, 2>(s, p);  // int8: four waves that each hold the 64 x 64 tile
+  }
+  if (which == 12) which = 5;
   if (which == 6) return launch_prefill_cfg<T, WF, EPI, 2, 4, 1, 1, 4, 256, 2>(s, p);   // 32 x 64, four waves that each hold the tile split K
   if (which == 1) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 1, 64, 2>(s, p);
   if constexpr (EPI == SK_GATEUP) {
@@ -651,7 +660,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 }  // namespace mui
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
-  if (tile < 0 || tile > 11 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  if (tile < 0 || tile > 12 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;
