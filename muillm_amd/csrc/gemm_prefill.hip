@@ -18,7 +18,7 @@
 //   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
 //   Tile shapes, chosen per call by rounds of workgroups x cost per round (launch_prefill_t):
 //   256 rows x 256 tokens x 64 k and 128 x 256 x 64 on sixteen waves (4 x 4), 192 x 256 x 64 on
-//   eight (2 x 4) while the grid covers most of the chip; 128 x 128 x 64 and 96 x 128 x 64 on four
+//   twelve (3 x 4) while the grid covers most of the chip; 128 x 128 x 64 and 96 x 128 x 64 on four
 //   waves (2 x 2), two workgroups per CU; 64 x 128 x 128 and 32 x 64 x 256 with a single LDS stage
 //   for small matrices. For grids of a round or two of workgroups (short prompts, matrices of a few
 //   thousand rows) shapes whose waves ALSO split K, each taking every fourth 32-value chunk of a
@@ -85,12 +85,18 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
   constexpr int PITCH = KS;
   constexpr int CPR = KS / 8;            // 16-byte chunks of 8 elements per row and step
   constexpr int OUT_TILE = (EPI == SK_GATEUP) ? ROWS / 2 : ROWS;  // outputs per workgroup
-  constexpr int XCH = TOKS * CPR / kPfThreads;                     // token loads per thread and step
-  constexpr int WCH = (WF == WF_16BIT) ? ROWS * CPR / kPfThreads : ROWS * (KS / 16) / kPfThreads;
+  // chunks of a k-step per tile and per thread; where the threads do not divide them (twelve
+  // waves), the last round of chunks is staged by the first waves only: the others load a valid
+  // address all the same (rows and tokens are clamped) and skip the LDS write
+  constexpr int XCHUNKS = TOKS * CPR;
+  constexpr int WCHUNKS = ROWS * ((WF == WF_16BIT) ? CPR : KS / 16);
+  constexpr int XCH = (XCHUNKS + kPfThreads - 1) / kPfThreads;     // token loads per thread and step
+  constexpr int WCH = (WCHUNKS + kPfThreads - 1) / kPfThreads;
+  constexpr bool XEXACT = XCHUNKS % kPfThreads == 0, WEXACT = WCHUNKS % kPfThreads == 0;
   static_assert(EPI != SK_GATEUP || WR % 2 == 0, "gate/up needs an even number of row tiles per wave");
   static_assert(XCH >= 1 && WCH >= 1 && kPfThreads % CPR == 0, "tile shape");
-  static_assert(TOKS * CPR % kPfThreads == 0 && ROWS * ((WF == WF_16BIT) ? CPR : KS / 16) % kPfThreads == 0,
-                "every thread stages the same number of chunks");
+  static_assert(XCHUNKS >= kPfThreads && WCHUNKS >= kPfThreads, "every thread stages at least one chunk of each operand");
+  static_assert((XEXACT || XCHUNKS % 64 == 0) && (WEXACT || WCHUNKS % 64 == 0), "whole waves stage the last round of chunks");
   // NBUF == 2: step s + 1 is written to the other LDS stage while step s is multiplied, one
   // barrier per step instead of two
   typedef uint16_t WStage[ROWS * PITCH];
@@ -196,6 +202,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
     const bool xlive = k0 + xcol * 8 + 8 <= p.k;
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
+      if (!XEXACT && t + kPfThreads * i >= XCHUNKS) continue;  // uniform per wave
       float sq = 0.f;
       u32x4 b = make_b<T, NORM>(r.x[i], NORM ? r.g : r.x[i], sq);
       b = xlive ? b : zero;
@@ -206,6 +213,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
     if constexpr (WF == WF_16BIT) {
 #pragma unroll
       for (int i = 0; i < WCH; ++i) {
+        if (!WEXACT && t + kPfThreads * i >= WCHUNKS) continue;
         const int row = (t + kPfThreads * i) / CPR;
         *(u32x4*)&w_lds[buf][row * PITCH + ((xcol ^ swz(row)) * 8)] = xlive ? r.w[i] : zero;
       }
@@ -213,6 +221,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
       const bool wlive = k0 + wcol * 16 + 16 <= p.k;
 #pragma unroll
       for (int i = 0; i < WCH; ++i) {
+        if (!WEXACT && t + kPfThreads * i >= WCHUNKS) continue;
         const u32x4 lo = convert_a<T, WF>(r.w[i].x, r.w[i].y, nullptr, 0, 0);
         const u32x4 hi = convert_a<T, WF>(r.w[i].z, r.w[i].w, nullptr, 0, 0);
         const int row = (t + kPfThreads * i) / WCPR;
@@ -363,7 +372,8 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
   // ---- per-token rsqrt(mean(x^2) + eps): every thread adds the squares it staged to its tokens
   if constexpr (NORM) {
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) atomicAdd(&rs_lds[(t + kPfThreads * i) / CPR], ss[i]);
+    for (int i = 0; i < XCH; ++i)
+      if (XEXACT || t + kPfThreads * i < XCHUNKS) atomicAdd(&rs_lds[(t + kPfThreads * i) / CPR], ss[i]);
     __syncthreads();
     for (int i = t; i < TOKS; i += kPfThreads) rs_lds[i] = rsqrtf(rs_lds[i] / (float)p.k + p.eps);
     __syncthreads();
@@ -510,8 +520,8 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   // and a bit rounds of workgroups costs two rounds. Each shape has a cost per round of
   // workgroups (microseconds at K = 4096 on MI355X; only the ratios matter); the number of
   // rounds the grid needs decides between them. Measured on the Llama-3-8B shapes: QKV at 1536
-  // tokens is 144 tiles of 256 x 256 (109 us) but 192 of 192 x 256 (100 us; the built-in choice
-  // before took 134); o_proj and down at 2048 tokens are 128 tiles of 256 x 256 (112 / 363 us)
+  // tokens is 144 tiles of 256 x 256 (116 us) but 192 of 192 x 256 (92 us), at 2048 tokens 192
+  // (122 us) against 256 (99 us); o_proj and down at 2048 tokens are 128 tiles of 256 x 256 (112 / 363 us)
   // and 256 of 128 x 256 (78 / 270 us); QKV at 512 is 192 tiles of 128 x 128 (68 us), 256 of
   // 96 x 128 (62 us). Below three workgroups of 128 x 128 per four CUs: 64 x 128, then 32 x 64 (up
   // to 256 tokens on the 4096-row matrices).
@@ -549,8 +559,7 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
       auto offer = [&](int id, float cost) {
         if (cost < best * 0.97f) { best = cost; which = id; }  // bigger tiles win ties
       };
-      // (int8 rows are staged in 16-byte chunks of 16 codes: 192 and 96 rows do not divide evenly among the threads)
-      if (WF == WF_16BIT) offer(8, whole(tiles(192, 256), 100.f, 103.f));
+      offer(8, whole(tiles(192, 256), 85.f, 92.f));
       offer(7, whole(tiles(128, 256), WF == WF_16BIT ? 67.f : 73.f, WF == WF_16BIT ? 70.f : 76.f));
       offer(1, pairs(tiles(128, 128), 68.f, 92.f));
       if (EPI == SK_LINEAR && WF == WF_16BIT) offer(10, pairs(tiles(96, 128), 60.f, 76.f));
@@ -575,15 +584,17 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   // int8 rows hold a quarter of the 16-byte chunks per k-step: where sixteen waves would leave
   // threads without a chunk to stage, the int8 kernels keep eight.
   if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 4, 4, 4, 1, 64, 2>(s, p);      // 256 x 256, 4 x 4 waves of 64 x 64
+  // 192 x 256 on twelve waves (3 x 4 of 64 x 64, the wave tile of the 256 x 256 kernel; the token
+  // chunks of a k-step do not divide by 768 threads: the last round is staged by eight of the
+  // waves): QKV at 2048 tokens 119 -> 108 us, at 4096 232 -> 208 us against eight waves of 96 x 64
+  if (which == 8) return launch_prefill_cfg<T, WF, EPI, 4, 4, 3, 4, 1, 64, 2>(s, p);
   if constexpr (WF == WF_16BIT) {
-    if (which == 8) return launch_prefill_cfg<T, WF, EPI, 6, 4, 2, 4, 1, 64, 2>(s, p);    // 192 x 256, 2 x 4 waves of 96 x 64
     if (which == 7) return launch_prefill_cfg<T, WF, EPI, 2, 4, 4, 4, 1, 64, 2>(s, p);    // 128 x 256, 4 x 4 waves of 32 x 64
     if (which == 5) return launch_prefill_cfg<T, WF, EPI, 2, 4, 2, 2, 4, 128, 2>(s, p);   // 64 x 128, 2 x 2 waves x 4 shares of K
     if constexpr (EPI == SK_LINEAR) {
       if (which == 10) return launch_prefill_cfg<T, WF, EPI, 3, 4, 2, 2, 1, 64, 2>(s, p);  // 96 x 128, 2 x 2 waves of 48 x 64
     }
   }
-  if (which == 8) which = 7;   // int8 weights
   if (which == 10) which = 1;  // int8 weights, gate/up
   if (which == 7) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2>(s, p);      // 128 x 256, 2 x 4 waves of 64 x 64
   if (which == 9) return launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 2, 4, 128, 2>(s, p);     // 128 x 128, 2 x 2 waves x 4 shares of K
