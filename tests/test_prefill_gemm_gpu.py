@@ -26,8 +26,8 @@ def prompt_kernel_choice(request):
     """Every test runs with the built-in kernel choice and with each prompt kernel forced: the
     16-rows-per-workgroup kernel without LDS tiling (up to 128 tokens; longer prompts keep the
     built-in choice) and the shapes of the LDS-tiled kernel (the gate/up epilogue has no
-    32 x 64 and 96 x 128 shapes and takes 64 x 128 / 128 x 128 then; int8 weights have no 192- and
-    96-row shapes and take 128 x 256 / 128 x 128)."""
+    32 x 64, 64 x 64 and 96 x 128 shapes and takes 64 x 128 / 128 x 128 then; int8 weights have no
+    96-row shape and take 128 x 128)."""
     lib = _lib.load()
     knobs = {"auto": (0, 0), "wide": (0, 128), "tile-256x256": (4, -1), "ksplit-64x128": (5, -1), "ksplit-32x64": (6, -1), "tile-128x128": (1, -1), "tile-64x128": (2, -1), "tile-32x64": (3, -1),
              "tile-128x256": (7, -1), "tile-192x256": (8, -1), "tile-96x128": (10, -1), "ksplit-128x128": (9, -1), "ksplit-128x64": (11, -1), "ksplit-64x64": (12, -1)}
