@@ -69,7 +69,10 @@ __device__ __forceinline__ f32x4 xs_load(const float* src) {
 // Nobody waits for anybody.
 template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF,
           bool XS = false>
-__global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(const PrefillGemmParams p) {
+// (twelve waves: three per SIMD, so let the compiler use the registers of three)
+__global__ void __launch_bounds__(64 * NWR * NWT * NWK)
+    __attribute__((amdgpu_waves_per_eu(1, (NWR * NWT * NWK == 12) ? 3 : 8)))
+    prefill_gemm_kernel(const PrefillGemmParams p) {
   constexpr int kPfThreads = 64 * NWR * NWT * NWK;
   static_assert(!XS || (!NORM && EPI == SK_LINEAR && NBUF == 2), "workgroups that split K: plain linear, two stages");
   static_assert((KS / 32) % NWK == 0 && WT % NWK == 0, "k-split of the waves");
@@ -248,9 +251,9 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
       const int ks = kk * NWK + wk;
       u32x4 a[WR], b[WT];
 #pragma unroll
-      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[buf][a_base + i * 16 * PITCH + (((ks * 4 + lg) ^ lsw) * 8)];
-#pragma unroll
       for (int j = 0; j < WT; ++j) b[j] = *(const u32x4*)&x_lds[buf][b_base + j * 16 * PITCH + (((ks * 4 + lg) ^ lsw) * 8)];
+#pragma unroll
+      for (int i = 0; i < WR; ++i) a[i] = *(const u32x4*)&w_lds[buf][a_base + i * 16 * PITCH + (((ks * 4 + lg) ^ lsw) * 8)];
 #pragma unroll
       for (int i = 0; i < WR; ++i)
 #pragma unroll
@@ -277,6 +280,28 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK) prefill_gemm_kernel(cons
       if (s + 1 < se) store_step(s + 1, (s + 1 - sb) & 1, r0);  // uniform branch, no loads inside
       load_step(s + 2, r0);
       multiply((s - sb) & 1);
+      if constexpr (NWR * NWT * NWK == 12) {
+        // twelve waves have 168 registers each: the global loads stay in front of the multiply
+        // (left alone the compiler sinks them to its end, a barrier before they are needed) and
+        // the next operands are requested while the current ones are multiplied (QKV at 4096
+        // tokens 208 -> 204 us)
+        __builtin_amdgcn_sched_group_barrier(0x020, WCH + XCH + (NORM ? 1 : 0), 0);
+        static_assert(NWR * NWT * NWK != 12 || (WR == 4 && WT == 4 && KS / 32 / NWK == 2), "pinned order of the twelve-wave tile");
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);  // b0-3, a0, a1
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a2
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a3
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // second half of the k-step: b0, b1
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // b2, b3, a0, a1
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      }
       __syncthreads();
     }
   } else {
