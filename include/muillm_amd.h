@@ -320,7 +320,8 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
  * sits at key position q_start + t, keys are cache rows [0, seq_len), q_start + tokens <= seq_len.
  * The reference hands T > 1 to torch's scaled_dot_product_attention
  * (muillm/modules/attention/sdpaattention.py:221-245) after repeat_kv; here K/V are read per KV
- * head and no mask tensor is built. */
+ * head and no mask tensor is built. tokens may be at most 16 * 65535 (MUI_ERR_UNSUPPORTED beyond:
+ * the position tiles are one dimension of the grid). */
 int mui_prefill_attention(mui_stream_t stream, int dtype, const void* q_rotated, const void* k_cache,
                           const void* v_cache, long cache_batch_stride, long cache_head_stride,
                           long cache_token_stride, int seq_len, int q_start, void* out, int batch,
