@@ -365,6 +365,23 @@ int mui_greedy_advance(mui_stream_t stream, int dtype, const void* logits, long 
                        long tokens_stride, int max_steps, int64_t* unfinished,
                        const int64_t* eos_ids, int n_eos, long pad_token);
 
+/* mui_greedy_advance with the scan of a long row dealt out to several workgroups (one workgroup per
+ * 1024 chunks of 16 bytes, at most 32): a single workgroup pulls a 128k-entry row through one CU's
+ * load path. No counterpart in the reference (its argmax is torch's). `workspace` is
+ * mui_greedy_workspace_bytes(rows) bytes of 8-byte aligned device memory, zero-filled once by the
+ * caller before the first call; every call leaves it zero-filled again, so one buffer serves all the
+ * steps of a decode loop (and the replays of a captured one), but calls that share a buffer must not
+ * overlap. The result is the one mui_greedy_advance gives, bit for bit. With workspace == NULL (and
+ * workspace_bytes == 0), a buffer that is too small or misaligned, or rows that fit one workgroup,
+ * this is mui_greedy_advance. */
+size_t mui_greedy_workspace_bytes(int rows);
+int mui_greedy_advance_ws(mui_stream_t stream, int dtype, const void* logits, long row_stride,
+                          int rows, int vocab, int64_t* next_ids, int64_t* position_ids,
+                          int64_t* cache_position, int64_t* step, int64_t* tokens_out,
+                          long tokens_stride, int max_steps, int64_t* unfinished,
+                          const int64_t* eos_ids, int n_eos, long pad_token, void* workspace,
+                          size_t workspace_bytes);
+
 /* Sampling twin of mui_greedy_advance: tok = argmax_v(logits[b, v] / temperature - log q_v) with
  * q_v ~ Exp(1), which is the draw of the reference's sync-free multinomial
  * argmax(softmax(logits / temperature) / q) (muillm/sampling/multinomial.py:4-6) without

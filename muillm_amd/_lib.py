@@ -83,6 +83,9 @@ _SIGNATURES = {
     "mui_argmax": (c_int, [_P, c_int, _P, c_long, _P, c_int, c_int]),
     "mui_greedy_advance": (c_int, [_P, c_int, _P, c_long, c_int, c_int, _P, _P, _P, _P, _P, c_long, c_int, _P, _P,
                                    c_int, c_long]),
+    "mui_greedy_workspace_bytes": (ctypes.c_size_t, [c_int]),
+    "mui_greedy_advance_ws": (c_int, [_P, c_int, _P, c_long, c_int, c_int, _P, _P, _P, _P, _P, c_long, c_int, _P, _P,
+                                      c_int, c_long, _P, ctypes.c_size_t]),
     "mui_sample_advance": (c_int, [_P, c_int, _P, c_long, c_int, c_int, c_float, ctypes.c_uint64, _P, _P, _P, _P, _P,
                                    c_long, c_int, _P, _P, c_int, c_long]),
     "mui_embedding": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, c_int, c_int, c_int]),

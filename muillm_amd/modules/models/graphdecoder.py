@@ -54,6 +54,8 @@ class MuiGraphDecoder:
         self.eos = (torch.tensor(self.eos_token_ids, dtype=torch.int64, device=device)
                     if self.eos_token_ids else None)
         self.out_tokens = torch.zeros((batch, max_new_tokens), dtype=torch.int64, device=device)
+        # lets the token choice scan a long vocabulary on several workgroups; returns to zero every step
+        self._greedy_ws = muillm_ext.greedy_workspace(batch, device)
         self.logits = None
         self.mask4d = None  # static additive decode mask [B, 1, 1, capacity] when the prompts are padded
         self._stop_host = None  # pinned scalar for the sync-free stop check
@@ -80,7 +82,8 @@ class MuiGraphDecoder:
         else:
             muillm_ext.mui_greedy_advance(logits, self.ids, self.step, self.out_tokens, position_ids=self.pos,
                                           cache_position=self.cpos, unfinished=self.unfinished,
-                                          eos_token_ids=self.eos, pad_token_id=self.pad_token_id)
+                                          eos_token_ids=self.eos, pad_token_id=self.pad_token_id,
+                                          workspace=self._greedy_ws)
 
     def _filter_logits(self, logits):
         """HuggingFace's TopKLogitsWarper / TopPLogitsWarper on the temperature-scaled distribution:

@@ -989,7 +989,7 @@ def mui_argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torc
 def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch.Tensor, tokens_out: torch.Tensor,
                        position_ids: Optional[torch.Tensor] = None, cache_position: Optional[torch.Tensor] = None,
                        unfinished: Optional[torch.Tensor] = None, eos_token_ids: Optional[torch.Tensor] = None,
-                       pad_token_id: int = 0) -> None:
+                       pad_token_id: int = 0, workspace: Optional[torch.Tensor] = None) -> None:
     """Tail of a greedy decode step in one launch (everything in place, on the device):
     argmax of each logits row -> tokens_out[b, step[b]], next_ids[b]; position_ids[b], step[b]
     and cache_position[0] advance by one; unfinished[b] is cleared on an eos token or when
@@ -997,7 +997,10 @@ def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch
     muillm_add_tokens_check_finished does).
 
     logits [B, V] 16-bit; next_ids [B] or [B, 1]; step [B]; tokens_out [B, max_steps];
-    position_ids [B] or [B, 1]; cache_position [1]; unfinished [B]; all integers int64."""
+    position_ids [B] or [B, 1]; cache_position [1]; unfinished [B]; all integers int64.
+
+    workspace (see greedy_workspace): lets the scan of a long row run on several workgroups; the
+    same tokens either way."""
     _check_cuda(logits, "logits")
     if logits.stride(-1) != 1:
         logits = logits.contiguous()
@@ -1020,13 +1023,26 @@ def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch
         if eos_token_ids.dtype != torch.int64 or not eos_token_ids.is_contiguous():
             raise RuntimeError("eos_token_ids must be a contiguous int64 tensor")
         n_eos = eos_token_ids.numel()
+    ws_bytes = 0
+    if workspace is not None:
+        _check_cuda(workspace, "workspace")
+        if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+            raise RuntimeError("workspace must be a contiguous uint8 tensor (greedy_workspace makes one)")
+        ws_bytes = workspace.numel()
     check(
-        _lib.load().mui_greedy_advance(
+        _lib.load().mui_greedy_advance_ws(
             _stream(l2), _dtype_code(l2), l2.data_ptr(), l2.stride(0) if rows > 1 else v, rows, v,
             next_ids.data_ptr(), _ptr(position_ids), _ptr(cache_position), step.data_ptr(), tokens_out.data_ptr(),
-            tokens_out.stride(0), tokens_out.shape[1], _ptr(unfinished), _ptr(eos_token_ids), n_eos, int(pad_token_id)),
-        "mui_greedy_advance",
+            tokens_out.stride(0), tokens_out.shape[1], _ptr(unfinished), _ptr(eos_token_ids), n_eos, int(pad_token_id),
+            _ptr(workspace), ws_bytes),
+        "mui_greedy_advance_ws",
     )
+
+
+def greedy_workspace(rows: int, device) -> torch.Tensor:
+    """Zero-filled workspace for mui_greedy_advance on `rows` logits rows: one per decode loop (calls
+    that share it must not overlap); every call leaves it zero-filled again."""
+    return torch.zeros(_lib.load().mui_greedy_workspace_bytes(int(rows)), dtype=torch.uint8, device=device)
 
 
 def mui_sample_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch.Tensor, tokens_out: torch.Tensor,

@@ -463,6 +463,54 @@ def test_greedy_advance_kernel():
     assert torch.equal(out2[:, 0].cpu(), lg.float().argmax(-1).cpu())
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_greedy_advance_on_several_workgroups(dtype):
+    """The workspace form (a long row scanned by several workgroups, candidates folded under a 64-bit
+    atomic max) must choose the tokens of the plain form bit for bit -- ties to the lowest index also
+    across workgroups, -0 equal to +0, NaN and -inf never chosen, rows without any candidate give
+    token 0 -- step after step on one workspace, which every call leaves zero-filled."""
+    from muillm_amd import muillm_ext
+    g = torch.Generator().manual_seed(31)
+    B, V, steps = 6, 128256, 4     # 16032 chunks: 16 workgroups per row
+    ws = muillm_ext.greedy_workspace(B, DEV)
+    assert ws.numel() == 16 * B and int(ws.sum()) == 0
+    state = {}
+    for name in ("plain", "ws"):
+        state[name] = dict(ids=torch.zeros(B, 1, dtype=torch.int64, device=DEV), step=torch.zeros(B, dtype=torch.int64, device=DEV),
+                           toks=torch.full((B, steps), -1, dtype=torch.int64, device=DEV),
+                           pos=torch.full((B, 1), 7, dtype=torch.int64, device=DEV), cpos=torch.full((1,), 7, dtype=torch.int64, device=DEV),
+                           unf=torch.ones(B, dtype=torch.int64, device=DEV))
+    eos_t = torch.tensor([5], dtype=torch.int64, device=DEV)
+    for s_i in range(steps):
+        logits = torch.randn(B, V, generator=g).to(dtype)
+        top = float(logits.float().max()) + 1.0
+        logits[0, 100000] = top; logits[0, 2000] = top; logits[0, 70000] = top    # a tie across workgroups: 2000 wins
+        logits[1] = float("-inf"); logits[1, 3] = float("nan")                      # nothing to choose: token 0
+        logits[2] = float("nan"); logits[2, 127999] = -3.0                           # one candidate in the last workgroup
+        logits[3] = -1.0; logits[3, 90000] = 0.0; logits[3, 40000] = -0.0            # -0 == +0: the lower index wins
+        logits[4, 128255] = top                                                      # the very last element
+        if s_i == 2:
+            logits[5, 5] = top                                                       # row 5 stops on the eos token
+        lg = logits.to(DEV)
+        for name, w in (("plain", None), ("ws", ws)):
+            st = state[name]
+            muillm_ext.mui_greedy_advance(lg, st["ids"], st["step"], st["toks"], position_ids=st["pos"], cache_position=st["cpos"],
+                                          unfinished=st["unf"], eos_token_ids=eos_t, pad_token_id=9, workspace=w)
+        a, b = state["plain"], state["ws"]
+        for key in a:
+            assert torch.equal(a[key], b[key]), (key, s_i)
+        tok = b["toks"][:, s_i].cpu()
+        assert tok[0] == 2000 and tok[1] == 0 and tok[2] == 127999 and tok[3] == 40000 and tok[4] == 128255
+        assert int(ws.sum()) == 0, "the workspace must be zero-filled again after every call"
+    assert state["ws"]["unf"][5] == 0 and state["ws"]["toks"][5, 3] == 9
+    # a short vocabulary, unaligned rows and a missing workspace fall back to one workgroup
+    lg = torch.randn(2, 5000, generator=g).to(dtype).to(DEV)[:, :4999]
+    ids2 = torch.zeros(2, dtype=torch.int64, device=DEV); st2 = torch.zeros(2, dtype=torch.int64, device=DEV)
+    out2 = torch.zeros(2, 2, dtype=torch.int64, device=DEV)
+    muillm_ext.mui_greedy_advance(lg, ids2, st2, out2, workspace=muillm_ext.greedy_workspace(2, DEV))
+    assert torch.equal(out2[:, 0].cpu(), lg.float().argmax(-1).cpu())
+
+
 def test_generate_left_padded_batch_matches_single_runs():
     """Left-padded batch generation (static device-side mask + per-row rotary positions, graph
     replay) must give every row the tokens it gets when generated alone without padding."""
