@@ -1222,8 +1222,14 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     park();
     __syncthreads();
     load_block(base + kPgTok);  // in flight while this block is multiplied
+    // a block without hidden keys (all but the padded edge of a prompt) is handled like an unmasked one
+    bool block_clear = true;
+    if constexpr (MASKED) {
+      const u32x2 h4 = *(const u32x2*)&hidden_lds[4 * (lane & 15)];
+      block_clear = __builtin_amdgcn_ballot_w64(((h4.x | h4.y) & 0x7fff7fffu) != 0u) == 0;
+    }
     // a wave whose last query cannot see the half skips it (uniform per wave; LDS reads only)
-    if (!MASKED && base + 64 <= wave_all_see) {
+    if (block_clear && base + 64 <= wave_all_see) {
       attend_block();
     } else {
       if (base + 32 <= wave_all_see) attend(0, base, std::true_type{});
