@@ -20,6 +20,11 @@ from ..kvcache.cache_utils import MuiStaticCache, _next_pow2, create_static_cach
 
 
 class MuiGraphDecoder:
+    # decode steps per graph replay when nothing has to happen between steps on the host (no stop
+    # check due, no logits wanted): consecutive replays of a one-step graph start ~9 us apart from
+    # each other's end, kernels inside a graph abut
+    STEPS_PER_REPLAY = 4
+
     def __init__(self, lm, use_graph: bool = True, eos_token_ids=None, pad_token_id: int = 0,
                  do_sample: bool = False, temperature: float = 1.0, seed: int = 0,
                  top_k: Optional[int] = None, top_p: Optional[float] = None):
@@ -40,6 +45,7 @@ class MuiGraphDecoder:
         self.eos_token_ids = list(eos_token_ids) if eos_token_ids is not None else None
         self.pad_token_id = int(pad_token_id)
         self.graph = None
+        self.graph_multi = None  # STEPS_PER_REPLAY steps in one graph, captured on first use
         self._graph_key = None  # what the captured graph has baked in (see _capture_key)
         self.cache: Optional[MuiStaticCache] = None
         self._batch = None
@@ -127,9 +133,25 @@ class MuiGraphDecoder:
         self._restore(saved, seen)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            self.logits = self._step()
+            self._graph_logits = self._step()  # where every replay leaves its logits
+        self.logits = self._graph_logits
+        self.graph_multi = None
         self._graph_key = self._capture_key()
         # capture does not execute: the device state is as restored; the host counter moved once
+        self.cache._seen_tokens = seen
+        if self.cache.cpp_module is not None:
+            self.cache.cpp_module.seen_tokens = seen
+
+    def _capture_multi(self):
+        """STEPS_PER_REPLAY steps as one graph (the one-step graph has been captured and warmed up
+        before). Capture does not execute; only the host-side token counter moves and is put back."""
+        self.cache.device_length_mode = True  # (prefill switches it off) lengths are read on the device
+        seen = self.cache._seen_tokens
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(self.STEPS_PER_REPLAY):
+                self._multi_logits = self._step()  # the last step's
+        self.graph_multi = g
         self.cache._seen_tokens = seen
         if self.cache.cpp_module is not None:
             self.cache.cpp_module.seen_tokens = seen
@@ -225,16 +247,25 @@ class MuiGraphDecoder:
         check = stop_check_every > 0 and self.eos is not None
         pending = None  # (event, pinned host tensor) of the last stop-check copy
         done = 0
-        for i in range(n_steps):
+        if self.use_graph and not check and not collect_logits and n_steps >= 2 * self.STEPS_PER_REPLAY:
+            # nothing to do on the host between steps: several steps per replay
+            if self.graph_multi is None:
+                self._capture_multi()
+            for _ in range(n_steps // self.STEPS_PER_REPLAY):
+                self.graph_multi.replay()
+            self.logits = self._multi_logits
+            done = n_steps - n_steps % self.STEPS_PER_REPLAY
+        for i in range(done, n_steps):
             if check and pending is not None and pending[0].query():
                 if int(pending[1].item()) == 0:
                     break
                 pending = None
             if self.use_graph:
                 self.graph.replay()
-                lg = self.logits
+                lg = self._graph_logits
             else:
                 lg = self._step()
+            self.logits = lg  # logits of the last step taken
             done += 1
             if collect_logits:
                 logits_hist.append(lg.clone())

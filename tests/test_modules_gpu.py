@@ -246,6 +246,31 @@ def test_graph_decode_matches_eager(batch):
     assert dec.cache.get_seq_length() == 32 + n_new - 1
 
 
+def test_graph_decode_several_steps_per_replay():
+    """decode() without stop checks or logits collection replays STEPS_PER_REPLAY steps per graph
+    launch and finishes with single-step replays: tokens, the logits of the last step and the cache
+    length must be those of the eager loop, for step counts on both sides of a multiple."""
+    cfg = _small_config(layers=2)
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=6,
+                                         init_std=0.05)
+    g = torch.Generator().manual_seed(7)
+    ids = torch.randint(0, cfg.vocab_size, (2, 12), generator=g).to(DEV)
+    k = MuiGraphDecoder.STEPS_PER_REPLAY
+    for n_steps in (2 * k, 3 * k + 1, 2 * k - 1):
+        results = []
+        for use_graph in (False, True):
+            dec = MuiGraphDecoder(lm, use_graph=use_graph)
+            dec.prefill(ids, n_steps + 2)    # emits the first token
+            dec.decode(1)
+            dec.decode(n_steps)
+            torch.cuda.synchronize()
+            results.append((dec.out_tokens.clone(), dec.logits.clone(), dec.cache.get_seq_length(), dec))
+        assert torch.equal(results[0][0], results[1][0]), n_steps
+        assert torch.equal(results[0][1], results[1][1]), n_steps
+        assert results[0][2] == results[1][2] == 12 + 1 + n_steps
+        assert (results[1][3].graph_multi is not None) == (n_steps >= 2 * k)
+
+
 def test_graph_decoder_reuse_after_cache_growth_and_multi_turn():
     """One decoder object, one cache object, a second generation that needs a larger cache: the
     cache tensors are re-allocated, so the captured step must be recorded again (a stale graph
