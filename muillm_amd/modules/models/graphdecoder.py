@@ -25,12 +25,20 @@ class MuiGraphDecoder:
     # each other's end, kernels inside a graph abut
     STEPS_PER_REPLAY = 4
 
-    def __init__(self, lm, use_graph: bool = True, eos_token_ids=None, pad_token_id: int = 0,
+    def __init__(self, lm, use_graph: Optional[bool] = True, eos_token_ids=None, pad_token_id: int = 0,
                  do_sample: bool = False, temperature: float = 1.0, seed: int = 0,
                  top_k: Optional[int] = None, top_p: Optional[float] = None):
         """do_sample=True draws from softmax(logits / temperature) on the device (the reference's
         sync-free multinomial, muillm/sampling/multinomial.py:4-6) instead of taking the argmax;
-        the draws are a function of (seed, batch row, step), so a run is reproducible."""
+        the draws are a function of (seed, batch row, step), so a run is reproducible.
+
+        use_graph: True replays the captured decode step, False enqueues every step's kernels on the
+        stream, None chooses when the first step is due: stream launches where the whole layer stack
+        is one library call (the host then needs ~0.8 ms for a 2.6 ms step of the 8B shape, and the
+        rate is the same as or a little above graph replay -- 383-386 against 380-382 tokens/s at
+        batch 1 -- without graph replay's slower first ~70 launches in a fresh process: 2.69 against
+        2.62 ms per step), graph replay where the layers run as separate module calls and the host
+        would be the limit."""
         self.lm = lm
         self.use_graph = use_graph
         self.do_sample = do_sample
@@ -240,6 +248,10 @@ class MuiGraphDecoder:
         gets the same effect with its Synchronizer, csrc/sync.cu:16-118, muillm/sampling/generation.py);
         the few steps issued past the end only write pad tokens."""
         logits_hist = []
+        if self.use_graph is None:
+            model = getattr(self.lm, "model", None)
+            stack = model._decode_stack(self.cache, self._batch, self.ids) if hasattr(model, "_decode_stack") else None
+            self.use_graph = stack is None
         if self.use_graph and self.graph is None:
             self._capture()
         if not self.use_graph:

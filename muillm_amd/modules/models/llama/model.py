@@ -398,14 +398,16 @@ class MuiLlamaForCausalLM(MuiModule):
                                  hidden_states=outputs.hidden_states, attentions=outputs.attentions)
 
     @torch.no_grad()
-    def generate_greedy(self, input_ids: torch.LongTensor, max_new_tokens: int, use_graph: bool = True,
+    def generate_greedy(self, input_ids: torch.LongTensor, max_new_tokens: int, use_graph: Optional[bool] = None,
                         cache: Optional[MuiStaticCache] = None, return_logits: bool = False):
         """Prefill on the prompt, then max_new_tokens greedy decode steps at the prompt's batch
         size. Returns int64 [B, prompt + max_new_tokens] (and, optionally, the per-step fp16
         logits of the decode steps).
 
-        use_graph=True captures one decode step (model forward, argmax, position bookkeeping,
-        all on the device) into a HIP graph and replays it; False runs the same step eagerly."""
+        use_graph=True captures the decode step (model forward, argmax, position bookkeeping,
+        all on the device) into a HIP graph and replays it; False enqueues the same step on the
+        stream every time; None (default) lets the decoder choose (MuiGraphDecoder: stream launches
+        when the layer stack is one library call, graph replay otherwise)."""
         dec = self._decoder_for(use_graph=use_graph)
         cache = self._reusable_cache(dec, cache, input_ids)
         return dec.generate(input_ids, max_new_tokens, cache=cache, return_logits=return_logits)
@@ -434,7 +436,7 @@ class MuiLlamaForCausalLM(MuiModule):
     def generate(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
                  max_new_tokens: int = 20, do_sample: bool = False, temperature: float = 1.0,
                  top_k: Optional[int] = None, top_p: Optional[float] = None,
-                 eos_token_id=None, pad_token_id: Optional[int] = None, seed: int = 0, use_graph: bool = True,
+                 eos_token_id=None, pad_token_id: Optional[int] = None, seed: int = 0, use_graph: Optional[bool] = None,
                  cache: Optional[MuiStaticCache] = None, **unused):
         """HuggingFace-style entry point over the device-resident decode loop (the reference routes
         generate() through its MuiGenerationMixin._sample, muillm/sampling/generation.py:77-408).
