@@ -259,10 +259,10 @@ class MuiGraphDecoder:
         check = stop_check_every > 0 and self.eos is not None
         pending = None  # (event, pinned host tensor) of the last stop-check copy
         done = 0
+        if self.use_graph and not check and not collect_logits and self.graph_multi is None:
+            self._capture_multi()  # on the first such call, however short: a later long one finds it ready
         if self.use_graph and not check and not collect_logits and n_steps >= 2 * self.STEPS_PER_REPLAY:
             # nothing to do on the host between steps: several steps per replay
-            if self.graph_multi is None:
-                self._capture_multi()
             for _ in range(n_steps // self.STEPS_PER_REPLAY):
                 self.graph_multi.replay()
             self.logits = self._multi_logits

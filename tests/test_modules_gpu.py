@@ -268,7 +268,7 @@ def test_graph_decode_several_steps_per_replay():
         assert torch.equal(results[0][0], results[1][0]), n_steps
         assert torch.equal(results[0][1], results[1][1]), n_steps
         assert results[0][2] == results[1][2] == 12 + 1 + n_steps
-        assert (results[1][3].graph_multi is not None) == (n_steps >= 2 * k)
+        assert results[1][3].graph_multi is not None
 
 
 def test_graph_decoder_reuse_after_cache_growth_and_multi_turn():
