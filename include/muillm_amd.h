@@ -373,14 +373,20 @@ int mui_greedy_advance(mui_stream_t stream, int dtype, const void* logits, long 
  * steps of a decode loop (and the replays of a captured one), but calls that share a buffer must not
  * overlap. The result is the one mui_greedy_advance gives, bit for bit. With workspace == NULL (and
  * workspace_bytes == 0), a buffer that is too small or misaligned, or rows that fit one workgroup,
- * this is mui_greedy_advance. */
+ * this is mui_greedy_advance.
+ * embed_table / embed_out (both or neither): the workgroup that finishes row b also copies row
+ * `tok` of the 16-bit embedding table (rows embed_row_stride elements apart, embed_dim wide) to
+ * embed_out[b, :] (dense [rows, embed_dim]), so that the next decode step starts from the embedding
+ * without a gather launch of its own (whose two dependent loads -- token id, then the row -- cost
+ * 4.8 us at the head of every step); pad_token must then be a row of the table (< vocab). */
 size_t mui_greedy_workspace_bytes(int rows);
 int mui_greedy_advance_ws(mui_stream_t stream, int dtype, const void* logits, long row_stride,
                           int rows, int vocab, int64_t* next_ids, int64_t* position_ids,
                           int64_t* cache_position, int64_t* step, int64_t* tokens_out,
                           long tokens_stride, int max_steps, int64_t* unfinished,
                           const int64_t* eos_ids, int n_eos, long pad_token, void* workspace,
-                          size_t workspace_bytes);
+                          size_t workspace_bytes, const void* embed_table, long embed_row_stride,
+                          void* embed_out, int embed_dim);
 
 /* Sampling twin of mui_greedy_advance: tok = argmax_v(logits[b, v] / temperature - log q_v) with
  * q_v ~ Exp(1), which is the draw of the reference's sync-free multinomial

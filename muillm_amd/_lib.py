@@ -85,7 +85,7 @@ _SIGNATURES = {
                                    c_int, c_long]),
     "mui_greedy_workspace_bytes": (ctypes.c_size_t, [c_int]),
     "mui_greedy_advance_ws": (c_int, [_P, c_int, _P, c_long, c_int, c_int, _P, _P, _P, _P, _P, c_long, c_int, _P, _P,
-                                      c_int, c_long, _P, ctypes.c_size_t]),
+                                      c_int, c_long, _P, ctypes.c_size_t, _P, c_long, _P, c_int]),
     "mui_sample_advance": (c_int, [_P, c_int, _P, c_long, c_int, c_int, c_float, ctypes.c_uint64, _P, _P, _P, _P, _P,
                                    c_long, c_int, _P, _P, c_int, c_long]),
     "mui_embedding": (c_int, [_P, c_int, _P, c_long, _P, c_int, _P, c_int, c_int, c_int]),

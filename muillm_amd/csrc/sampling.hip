@@ -105,10 +105,12 @@ struct GreedyParams {
   int64_t* tokens_out; long tokens_stride; int max_steps;  // [B, >= max_steps]
   int64_t* unfinished;      // [B] or null
   const int64_t* eos_ids; int n_eos; long pad_token;
+  // optional: the chosen token's embedding row, for the next step's first layer
+  const uint16_t* embed_table; long embed_stride; uint16_t* embed_out; int embed_dim;  // out [B, embed_dim] dense
 };
 
 // what thread 0 does with row b's choice
-__device__ __forceinline__ void greedy_finish(const GreedyParams& p, int b, int best_i) {
+__device__ __forceinline__ int64_t greedy_finish(const GreedyParams& p, int b, int best_i) {
   int64_t tok = best_i;
   const bool was_unfinished = p.unfinished ? (p.unfinished[b] != 0) : true;
   if (p.unfinished && p.n_eos > 0 && !was_unfinished) tok = p.pad_token;
@@ -123,6 +125,28 @@ __device__ __forceinline__ void greedy_finish(const GreedyParams& p, int b, int 
     for (int i = 0; i < p.n_eos; ++i) unfinished = unfinished && (tok != p.eos_ids[i]);
     p.unfinished[b] = unfinished ? 1 : 0;
   }
+  return tok;
+}
+
+// The workgroup that finished row b hands the token to all its threads (thread 0 calls with the
+// token, the others with anything) and copies that row of the embedding table to embed_out[b]:
+// the embedding gather at the head of the next decode step, a launch of two dependent loads
+// (token id, then the row), becomes the tail of this one. `mine` is uniform per workgroup.
+__device__ __forceinline__ void gather_embedding(const GreedyParams& p, int b, int64_t tok, bool mine) {
+  __shared__ long long tok_s;
+  if (p.embed_table == nullptr) return;  // uniform
+  if (threadIdx.x == 0) tok_s = mine ? tok : -1;
+  __syncthreads();
+  const long long tk = tok_s;
+  if (tk < 0) return;
+  const uint16_t* src = p.embed_table + tk * p.embed_stride;
+  uint16_t* dst = p.embed_out + (long)b * p.embed_dim;
+  const bool vec = ((p.embed_dim | p.embed_stride) & 7) == 0 && (((uintptr_t)p.embed_table | (uintptr_t)p.embed_out) & 15u) == 0;
+  if (vec) {
+    for (int c = threadIdx.x; c < (p.embed_dim >> 3); c += kArgmaxThreads) *(u32x4*)(dst + (c << 3)) = ld16(src + (c << 3));
+  } else {
+    for (int i = threadIdx.x; i < p.embed_dim; i += kArgmaxThreads) dst[i] = src[i];
+  }
 }
 
 template <typename T>
@@ -130,8 +154,9 @@ __global__ void __launch_bounds__(kArgmaxThreads) greedy_advance_kernel(const Gr
   const int b = blockIdx.x;
   const bool vec = ((p.row_stride & 7) == 0) && ((((uintptr_t)p.logits) & 15u) == 0);
   const int best_i = row_argmax<T>(p.logits + (long)b * p.row_stride, vec, p.vocab);
-  if (threadIdx.x != 0) return;
-  greedy_finish(p, b, best_i);
+  int64_t tok = 0;
+  if (threadIdx.x == 0) tok = greedy_finish(p, b, best_i);
+  gather_embedding(p, b, tok, true);
 }
 
 // The same with the scan of a row dealt out to gridDim.x workgroups (one workgroup pulls a 128k-entry
@@ -148,20 +173,26 @@ __global__ void __launch_bounds__(kArgmaxThreads) greedy_advance_parts_kernel(co
   float best;
   int best_i;
   slice_argmax<T>(p.logits + (long)b * p.row_stride, true, p.vocab, part, n_parts, best, best_i);
-  if (threadIdx.x != 0) return;
-  if (best_i != 0x7fffffff) {
-    const uint32_t u = __float_as_uint(best + 0.f);  // -0 counts as +0, as it does under ==
-    const uint32_t image = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-    const unsigned long long key = ((unsigned long long)image << 32) | (0xffffffffu - (uint32_t)best_i);
-    __hip_atomic_fetch_max(best_word + b, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  int64_t tok = 0;
+  bool last = false;
+  if (threadIdx.x == 0) {
+    if (best_i != 0x7fffffff) {
+      const uint32_t u = __float_as_uint(best + 0.f);  // -0 counts as +0, as it does under ==
+      const uint32_t image = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+      const unsigned long long key = ((unsigned long long)image << 32) | (0xffffffffu - (uint32_t)best_i);
+      __hip_atomic_fetch_max(best_word + b, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the candidate has arrived before the count goes up
+    const unsigned before = __hip_atomic_fetch_add(arrived + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = before + 1 == (unsigned)n_parts;
+    if (last) {
+      const unsigned long long w = __hip_atomic_load(best_word + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(best_word + b, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(arrived + b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      tok = greedy_finish(p, b, w ? (int)(0xffffffffu - (uint32_t)(w & 0xffffffffu)) : 0);
+    }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the candidate has arrived before the count goes up
-  const unsigned before = __hip_atomic_fetch_add(arrived + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (before + 1 != (unsigned)n_parts) return;
-  const unsigned long long w = __hip_atomic_load(best_word + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(best_word + b, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(arrived + b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  greedy_finish(p, b, w ? (int)(0xffffffffu - (uint32_t)(w & 0xffffffffu)) : 0);
+  gather_embedding(p, b, tok, last);  // the last arriver's workgroup copies, the others leave
 }
 
 }  // namespace mui
@@ -190,8 +221,11 @@ extern "C" int mui_greedy_advance_ws(mui_stream_t stream, int dtype, const void*
                                      int64_t* cache_position, int64_t* step, int64_t* tokens_out,
                                      long tokens_stride, int max_steps, int64_t* unfinished,
                                      const int64_t* eos_ids, int n_eos, long pad_token, void* workspace,
-                                     size_t workspace_bytes) {
+                                     size_t workspace_bytes, const void* embed_table, long embed_row_stride,
+                                     void* embed_out, int embed_dim) {
   MUI_CHECK_ARG(logits && next_ids && step && tokens_out && rows > 0 && vocab > 0 && row_stride >= vocab);
+  MUI_CHECK_ARG((embed_table == nullptr) == (embed_out == nullptr));
+  MUI_CHECK_ARG(!embed_table || (embed_dim > 0 && embed_row_stride >= embed_dim && pad_token >= 0 && pad_token < vocab));
   MUI_CHECK_ARG(max_steps >= 0 && tokens_stride >= max_steps && n_eos >= 0 && (n_eos == 0 || eos_ids));
   MUI_CHECK_ARG(workspace || workspace_bytes == 0);
   if (dtype != MUI_DTYPE_F16 && dtype != MUI_DTYPE_BF16) return MUI_ERR_INVALID_ARG;
@@ -201,6 +235,8 @@ extern "C" int mui_greedy_advance_ws(mui_stream_t stream, int dtype, const void*
   p.next_ids = next_ids; p.position_ids = position_ids; p.cache_position = cache_position;
   p.step = step; p.tokens_out = tokens_out; p.tokens_stride = tokens_stride; p.max_steps = max_steps;
   p.unfinished = unfinished; p.eos_ids = eos_ids; p.n_eos = n_eos; p.pad_token = pad_token;
+  p.embed_table = (const uint16_t*)embed_table; p.embed_stride = embed_row_stride;
+  p.embed_out = (uint16_t*)embed_out; p.embed_dim = embed_dim;
   hipStream_t s = (hipStream_t)stream;
   // one workgroup per 1024 chunks of 16 bytes (one load per thread), 32 at most; rows that cannot be
   // read in 16-byte chunks, rows of a single part and calls without a workspace take one workgroup
@@ -230,5 +266,5 @@ extern "C" int mui_greedy_advance(mui_stream_t stream, int dtype, const void* lo
                                   const int64_t* eos_ids, int n_eos, long pad_token) {
   return mui_greedy_advance_ws(stream, dtype, logits, row_stride, rows, vocab, next_ids, position_ids, cache_position,
                                step, tokens_out, tokens_stride, max_steps, unfinished, eos_ids, n_eos, pad_token,
-                               nullptr, 0);
+                               nullptr, 0, nullptr, 0, nullptr, 0);
 }

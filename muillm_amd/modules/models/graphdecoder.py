@@ -70,6 +70,15 @@ class MuiGraphDecoder:
         self.out_tokens = torch.zeros((batch, max_new_tokens), dtype=torch.int64, device=device)
         # lets the token choice scan a long vocabulary on several workgroups; returns to zero every step
         self._greedy_ws = muillm_ext.greedy_workspace(batch, device)
+        # greedy decoding: the token choice leaves the chosen token's embedding row here, and the
+        # next step starts from it instead of launching a gather (token id -> row: two dependent
+        # loads at the head of every step)
+        table = getattr(getattr(getattr(self.lm, "model", None), "embed_tokens", None), "weight", None)
+        self._embed_table = None
+        if (not self.do_sample and table is not None and table.is_cuda and table.dim() == 2 and table.stride(1) == 1
+                and table.dtype in (torch.float16, torch.bfloat16)):
+            self._embed_table = table
+            self.hidden = torch.zeros((batch, 1, table.shape[1]), dtype=table.dtype, device=device)
         self.logits = None
         self.mask4d = None  # static additive decode mask [B, 1, 1, capacity] when the prompts are padded
         self._stop_host = None  # pinned scalar for the sync-free stop check
@@ -78,7 +87,9 @@ class MuiGraphDecoder:
 
     def _step(self):
         """One decode step on the static buffers (this is what gets captured)."""
-        out = self.lm(input_ids=self.ids, position_ids=self.pos, cache_position=self.cpos,
+        fold = self._embed_table is not None
+        out = self.lm(input_ids=None if fold else self.ids, inputs_embeds=self.hidden if fold else None,
+                      position_ids=self.pos, cache_position=self.cpos,
                       past_key_values=self.cache, use_cache=True, attention_mask=self.mask4d,
                       all_ones_mask=self.mask4d is None, float_logits=False)
         logits = out.logits[:, -1, :]
@@ -97,7 +108,8 @@ class MuiGraphDecoder:
             muillm_ext.mui_greedy_advance(logits, self.ids, self.step, self.out_tokens, position_ids=self.pos,
                                           cache_position=self.cpos, unfinished=self.unfinished,
                                           eos_token_ids=self.eos, pad_token_id=self.pad_token_id,
-                                          workspace=self._greedy_ws)
+                                          workspace=self._greedy_ws, embed_table=self._embed_table,
+                                          embed_out=self.hidden if self._embed_table is not None else None)
 
     def _filter_logits(self, logits):
         """HuggingFace's TopKLogitsWarper / TopPLogitsWarper on the temperature-scaled distribution:
@@ -131,7 +143,7 @@ class MuiGraphDecoder:
         self.cache.device_length_mode = True
         seen = self.cache._seen_tokens
         # warm up on a side stream (allocator, lazy module state), then restore the cache counters
-        saved = [t.clone() for t in (self.ids, self.pos, self.cpos, self.step, self.out_tokens, self.unfinished)]
+        saved = [t.clone() for t in self._step_state()]
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -164,8 +176,15 @@ class MuiGraphDecoder:
         if self.cache.cpp_module is not None:
             self.cache.cpp_module.seen_tokens = seen
 
+    def _step_state(self):
+        """The device tensors a decode step changes (besides the cache slot it writes)."""
+        state = [self.ids, self.pos, self.cpos, self.step, self.out_tokens, self.unfinished]
+        if self._embed_table is not None:
+            state.append(self.hidden)
+        return state
+
     def _restore(self, saved, seen):
-        for dst, src in zip((self.ids, self.pos, self.cpos, self.step, self.out_tokens, self.unfinished), saved):
+        for dst, src in zip(self._step_state(), saved):
             dst.copy_(src)
         self.cache._seen_tokens = seen
         if self.cache.cpp_module is not None:

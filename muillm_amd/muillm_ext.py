@@ -989,7 +989,8 @@ def mui_argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torc
 def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch.Tensor, tokens_out: torch.Tensor,
                        position_ids: Optional[torch.Tensor] = None, cache_position: Optional[torch.Tensor] = None,
                        unfinished: Optional[torch.Tensor] = None, eos_token_ids: Optional[torch.Tensor] = None,
-                       pad_token_id: int = 0, workspace: Optional[torch.Tensor] = None) -> None:
+                       pad_token_id: int = 0, workspace: Optional[torch.Tensor] = None,
+                       embed_table: Optional[torch.Tensor] = None, embed_out: Optional[torch.Tensor] = None) -> None:
     """Tail of a greedy decode step in one launch (everything in place, on the device):
     argmax of each logits row -> tokens_out[b, step[b]], next_ids[b]; position_ids[b], step[b]
     and cache_position[0] advance by one; unfinished[b] is cleared on an eos token or when
@@ -1000,7 +1001,9 @@ def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch
     position_ids [B] or [B, 1]; cache_position [1]; unfinished [B]; all integers int64.
 
     workspace (see greedy_workspace): lets the scan of a long row run on several workgroups; the
-    same tokens either way."""
+    same tokens either way. embed_table [V, H] / embed_out [B, H] or [B, 1, H] (16-bit, the logits'
+    dtype): the chosen token's embedding row is copied to embed_out[b] in the same launch, for a
+    next step that starts from inputs_embeds."""
     _check_cuda(logits, "logits")
     if logits.stride(-1) != 1:
         logits = logits.contiguous()
@@ -1029,12 +1032,23 @@ def mui_greedy_advance(logits: torch.Tensor, next_ids: torch.Tensor, step: torch
         if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
             raise RuntimeError("workspace must be a contiguous uint8 tensor (greedy_workspace makes one)")
         ws_bytes = workspace.numel()
+    e_stride = e_dim = 0
+    if (embed_table is None) != (embed_out is None):
+        raise RuntimeError("embed_table and embed_out go together")
+    if embed_table is not None:
+        _check_cuda(embed_table, "embed_table")
+        _check_cuda(embed_out, "embed_out")
+        e_dim = embed_table.shape[-1]
+        if (embed_table.dim() != 2 or embed_table.dtype != l2.dtype or embed_table.stride(1) != 1 or embed_table.shape[0] < v
+                or embed_out.dtype != l2.dtype or not embed_out.is_contiguous() or embed_out.numel() != rows * e_dim):
+            raise RuntimeError("embed_table must be [>= V, H] and embed_out a contiguous [B, H], both in the logits' dtype")
+        e_stride = embed_table.stride(0)
     check(
         _lib.load().mui_greedy_advance_ws(
             _stream(l2), _dtype_code(l2), l2.data_ptr(), l2.stride(0) if rows > 1 else v, rows, v,
             next_ids.data_ptr(), _ptr(position_ids), _ptr(cache_position), step.data_ptr(), tokens_out.data_ptr(),
             tokens_out.stride(0), tokens_out.shape[1], _ptr(unfinished), _ptr(eos_token_ids), n_eos, int(pad_token_id),
-            _ptr(workspace), ws_bytes),
+            _ptr(workspace), ws_bytes, _ptr(embed_table), e_stride, _ptr(embed_out), e_dim),
         "mui_greedy_advance_ws",
     )
 

@@ -536,6 +536,32 @@ def test_greedy_advance_on_several_workgroups(dtype):
     assert torch.equal(out2[:, 0].cpu(), lg.float().argmax(-1).cpu())
 
 
+def test_greedy_advance_leaves_the_embedding_row():
+    """With an embedding table the launch that chooses the token also copies that token's row to
+    embed_out (finished rows: the pad token's), in the single-workgroup form and in the workspace form."""
+    from muillm_amd import muillm_ext
+    g = torch.Generator().manual_seed(41)
+    for dtype, V, H in ((torch.float16, 128256, 4096), (torch.bfloat16, 1000, 72), (torch.float16, 333, 13)):
+        B = 3
+        table = torch.randn(V, H, generator=g).to(dtype).to(DEV)
+        logits = torch.randn(B, V, generator=g).to(dtype).to(DEV)
+        logits[1, 7] = 100.0                                # row 1 chooses the eos token 7 ...
+        for ws in (None, muillm_ext.greedy_workspace(B, DEV)):
+            ids = torch.zeros(B, 1, dtype=torch.int64, device=DEV); step = torch.zeros(B, dtype=torch.int64, device=DEV)
+            toks = torch.zeros(B, 2, dtype=torch.int64, device=DEV); unf = torch.ones(B, dtype=torch.int64, device=DEV)
+            eos_t = torch.tensor([7], dtype=torch.int64, device=DEV)
+            emb = torch.full((B, 1, H), 5.0, dtype=dtype, device=DEV)
+            for s_i in range(2):
+                muillm_ext.mui_greedy_advance(logits, ids, step, toks, unfinished=unf, eos_token_ids=eos_t, pad_token_id=2,
+                                              workspace=ws, embed_table=table, embed_out=emb)
+                assert torch.equal(emb[:, 0], table[ids.view(-1)]), (dtype, V, s_i)
+            assert toks[1].tolist() == [7, 2]                # ... and emits the pad token (and its row) afterwards
+            if ws is not None:
+                assert int(ws.sum()) == 0
+    with pytest.raises(RuntimeError):
+        muillm_ext.mui_greedy_advance(logits, ids, step, toks, embed_table=table)
+
+
 def test_generate_left_padded_batch_matches_single_runs():
     """Left-padded batch generation (static device-side mask + per-row rotary positions, graph
     replay) must give every row the tokens it gets when generated alone without padding."""
