@@ -5,9 +5,10 @@
 
 A "step" is one greedy decode step (one token for one user) of a randomly initialised
 Llama-3-8B-shaped fp16 decoder: 32 layers, hidden 4096, 32/8 heads x 128, MLP 14336, vocab
-128256, static KV cache, 32-token random prompt, batch 1. The step (embedding gather, 32 x
+128256, static KV cache, 32-token random prompt, batch 1. The step (32 x
 [fused norm+QKV GEMV, fused RoPE + cache write + flash decoding, o_proj GEMV + residual,
-fused norm + gate/up + SiLU GEMV, down GEMV + residual], final norm, lm_head GEMV, argmax)
+fused norm + gate/up + SiLU GEMV, down GEMV + residual], final norm + lm_head GEMV, token
+choice, which also fetches the chosen token's embedding row for the next step)
 runs the way the library's decoder chooses (`config.launch`: one library call per step that
 enqueues the whole layer stack on the stream, or replay of the captured step from a HIP graph; the
 `variants` force each); all inputs are resident in HBM before the timed region.
