@@ -37,6 +37,7 @@ HBM_PEAK_GBPS = 8000.0
 # (x2.0000 to KiB) and 114,783.2 for the GEMV; WRITE_SIZE reads 229,376.0 for the copy (x1.0) and 224.0 for
 # the GEMV. 235,038,826 B fetched + 229,417 B written.
 GATEUP_TRAFFIC_BYTES = 235038826 + 229417
+GATEUP_TRAFFIC_SOURCE = "profiles/gateup_gemv_llama3_8b_pmc_traffic.md (rocprofv3 --pmc counter runs; not re-measured by this run)"
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16 matrix-core peak
 BASELINE_TOKENS_PER_S = 210.0  # reference README: Llama-3-8B fp16 bs1 on 1x MI300X
 
@@ -57,7 +58,10 @@ def _event_time_us(fn, iters, warm):
     return s.elapsed_time(e) * 1e3 / iters
 
 
-def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=None, batch=1):
+def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=None, batch=1, windows=1):
+    """`windows` timed generations, each the whole workload again: prompt prefill into the emptied
+    cache, `warmup` untimed decode steps, then exactly `steps` timed ones between two device
+    synchronisations. Returns the list of window times (seconds) and the decoder."""
     import torch
 
     from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
@@ -66,14 +70,31 @@ def bench_decode(lm, steps, warmup, prompt_len=32, use_graph=None, batch=1):
     g = torch.Generator().manual_seed(0)
     ids = torch.randint(0, lm.config.vocab_size, (batch, prompt_len), generator=g).to(dev)
     dec = MuiGraphDecoder(lm, use_graph=use_graph)
-    dec.prefill(ids, steps + warmup + 1)
-    dec.decode(warmup)  # captures the graph on first use, then W untimed replays
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    dec.decode(steps)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    return dt, dec
+    times = []
+    for w in range(windows):
+        if w:
+            dec.cache.reset()
+        dec.prefill(ids, steps + warmup + 1, cache=dec.cache if w else None)
+        dec.decode(warmup)  # captures the graph on first use, then W untimed steps
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.decode(steps)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return (times if windows > 1 else times[0]), dec
+
+
+def _median(vals):
+    v = sorted(vals)
+    n = len(v)
+    return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
+
+
+def _rate_summary(times, steps, per_step=1):
+    """Median / min / max rate over timed windows, and which window was the fastest."""
+    rates = [per_step * steps / t for t in times]
+    return {"median": round(_median(rates), 2), "min": round(min(rates), 2), "max": round(max(rates), 2),
+            "windows": [round(r, 2) for r in rates], "fastest_window": rates.index(max(rates))}
 
 
 def bench_prefill(lm, tokens, iters=3):
@@ -118,9 +139,11 @@ def bench_int8_variant(config, steps, warmup, group_size=0):
                                            finalize=False)
     lm8 = init_engine(base, device="cuda", engine_config=MuiEngineConfig(qm))
     torch.cuda.synchronize()
-    dt, dec = bench_decode(lm8, steps, warmup)
+    t, dec = bench_decode(lm8, steps, warmup, windows=3)
+    dt = _median(t)
     del dec
-    dt_graph, dec = bench_decode(lm8, steps, warmup, use_graph=True)
+    t, dec = bench_decode(lm8, steps, warmup, use_graph=True, windows=3)
+    dt_graph = _median(t)
     hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
     hq, hkv, d = config.num_attention_heads, config.num_key_value_heads, hid // config.num_attention_heads
     codes = config.num_hidden_layers * ((hq + 2 * hkv) * d * hid + hid * hid + 3 * hid * inter)
@@ -133,6 +156,56 @@ def bench_int8_variant(config, steps, warmup, group_size=0):
             "weight_bytes_per_token": wbytes, "hbm_floor_ms": round(wbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4),
             "format": ("uint8 + fp16 (scale, min) per group of %d inputs (the reference's RTN format); lm_head fp16" % group_size)
             if group_size else "int8 per output channel + fp16 scale; lm_head fp16"}
+
+
+def bench_hf_dropin(config, steps, prompt_len=32, windows=3):
+    """The drop-in path the reference's own number is taken on (examples/llama3_8b.py:98-106,148-167
+    there): a HuggingFace LlamaForCausalLM -- here built at the 8B shape straight on the device with
+    random weights, no checkpoint --, init_engine() on it, a short warm-up generate(), then timed
+    model.generate(ids, max_new_tokens=steps) calls, prompt prefill included in the time."""
+    import torch
+
+    try:
+        from transformers import LlamaConfig, LlamaForCausalLM
+    except Exception as e:  # transformers is optional for this library
+        return {"skipped": "transformers not importable: %r" % (e,)}
+    from muillm_amd.engine import init_engine
+
+    hf_cfg = LlamaConfig(hidden_size=config.hidden_size, intermediate_size=config.intermediate_size,
+                         num_hidden_layers=config.num_hidden_layers, num_attention_heads=config.num_attention_heads,
+                         num_key_value_heads=config.num_key_value_heads, vocab_size=config.vocab_size,
+                         max_position_embeddings=config.max_position_embeddings, rms_norm_eps=config.rms_norm_eps,
+                         rope_theta=500000.0, tie_word_embeddings=False)
+    torch.manual_seed(0)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        with torch.device("cuda"):
+            hf = LlamaForCausalLM(hf_cfg)
+    finally:
+        torch.set_default_dtype(prev)
+    hf.eval()
+    model = init_engine(hf, device="cuda")
+    ids = torch.randint(0, config.vocab_size, (1, prompt_len), generator=torch.Generator().manual_seed(0)).to("cuda")
+    model.generate(ids, max_new_tokens=10)  # the reference's example warms up the same way
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(windows):
+        t0 = time.perf_counter()
+        out = model.generate(ids, max_new_tokens=steps)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    assert out.shape == (1, prompt_len + steps)
+    dt = _median(times)
+    res = {"new_tokens_per_s": round(steps / dt, 2), "new_tokens_per_s_windows": [round(steps / t, 2) for t in times],
+           "reference_formula_total_tokens_per_s": round((prompt_len + steps) / dt, 2),
+           "what": "transformers.LlamaForCausalLM (random init at the 8B shape) -> init_engine -> model.generate("
+                   "ids[1, %d], max_new_tokens=%d), greedy, timed over the whole call: prefill + %d decode steps; "
+                   "reference_formula counts prompt + new tokens over the same time, as examples/llama3_8b.py does"
+                   % (prompt_len, steps, steps)}
+    del model, hf
+    torch.cuda.empty_cache()
+    return res
 
 
 def measured_copy_ceiling():
@@ -184,14 +257,19 @@ def gateup_roofline(lm):
         gp, up, pitch, nw = ptrs[i % len(ptrs)]
         lib.mui_gateup_silu(stream, 0, gp, up, pitch, x.data_ptr(), nw, 1e-5, h.data_ptr(), inter, hid, 1)
 
-    us = _event_time_us(fn, iters=20 * len(ptrs), warm=len(ptrs))
+    samples = [_event_time_us(fn, iters=8 * len(ptrs), warm=len(ptrs)) for _ in range(5)]
+    us = _median(samples)
     alg_bytes = 2 * inter * hid * 2 + 2 * (hid + hid + inter)  # G and U once, x, gamma, h
     achieved = alg_bytes / us / 1e3
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": GATEUP_TRAFFIC_BYTES if (hid, inter) == (4096, 14336) else None,
+            "traffic_source": GATEUP_TRAFFIC_SOURCE if (hid, inter) == (4096, 14336) else None,
             "kernel": "gemv_kernel<F16,R=4,CH=2,NORM,GATEUP> (fused RMSNorm + gate/up + SiLU*mul)",
-            "avg_launch_us": round(us, 2), "algorithmic_bytes_per_launch": alg_bytes}
+            "avg_launch_us": round(us, 2), "avg_launch_us_min": round(min(samples), 2),
+            "avg_launch_us_max": round(max(samples), 2),
+            "samples": "median of 5 x (8 launches per layer's buffer, HIP events on the launch stream)",
+            "algorithmic_bytes_per_launch": alg_bytes}
 
 
 def pmc_probe(launches=6):
@@ -855,6 +933,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--windows", type=int, default=5,
+                    help="timed windows of --steps steps (each a fresh generation); value = their median")
     ap.add_argument("--layers", type=int, default=32, help="decoder depth (32 = the Llama-3-8B shape; fewer is NOT the benchmark)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
@@ -932,7 +1012,10 @@ def main():
     if args.only_kernel_table:
         print(json.dumps({"kernels": kernel_table(lm)}))
         return
-    dt, dec = bench_decode(lm, args.steps, args.warmup)
+    times, dec = bench_decode(lm, args.steps, args.warmup, windows=args.windows)
+    times = times if isinstance(times, list) else [times]
+    head = _rate_summary(times, args.steps)
+    dt = _median(times)
     tokens_per_s = args.steps / dt
     hid, inter, v = config.hidden_size, config.intermediate_size, config.vocab_size
     hq, hkv, d = config.num_attention_heads, config.num_key_value_heads, 128
@@ -941,6 +1024,9 @@ def main():
     result = {
         "metric": "tokens/s/user, Llama-3-8B-shaped fp16 decode, batch 1",
         "value": round(tokens_per_s, 2),
+        "value_min": head["min"], "value_max": head["max"], "value_windows": head["windows"],
+        "value_is": "median of %d timed windows, each a fresh generation (prefill, %d warm-up steps, %d timed steps); "
+                    "fastest window: #%d" % (args.windows, args.warmup, args.steps, head["fastest_window"]),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -971,10 +1057,13 @@ def main():
     del dec
     if not args.no_variants:
         # the two launch modes, each forced, on the headline's step counts
-        dt_g, dec_g = bench_decode(lm, args.steps, args.warmup, use_graph=True)
-        dt_e, dec_e = bench_decode(lm, args.steps, args.warmup, use_graph=False)
-        result["variants"] = {"fp16_graph_replay_tokens_per_s": round(args.steps / dt_g, 2),
-                              "fp16_stream_launches_tokens_per_s": round(args.steps / dt_e, 2)}
+        t_g, dec_g = bench_decode(lm, args.steps, args.warmup, use_graph=True, windows=args.windows)
+        t_e, dec_e = bench_decode(lm, args.steps, args.warmup, use_graph=False, windows=args.windows)
+        t_g, t_e = (t if isinstance(t, list) else [t] for t in (t_g, t_e))
+        sg, se = _rate_summary(t_g, args.steps), _rate_summary(t_e, args.steps)
+        result["variants"] = {"fp16_graph_replay_tokens_per_s": sg["median"], "fp16_graph_replay_windows": sg["windows"],
+                              "fp16_stream_launches_tokens_per_s": se["median"],
+                              "fp16_stream_launches_windows": se["windows"]}
         del dec_e, dec_g
         for ctx in (4096,):
             dt_c, dec_c = bench_decode(lm, 64, 8, prompt_len=ctx)
@@ -992,12 +1081,15 @@ def main():
         del lm
         torch.cuda.empty_cache()
         lm_bf = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.bfloat16, device="cuda", seed=0)
-        dt_bf, dec_bf = bench_decode(lm_bf, args.steps, args.warmup)
-        result["variants"]["bf16_tokens_per_s"] = round(args.steps / dt_bf, 2)
+        t_bf, dec_bf = bench_decode(lm_bf, args.steps, args.warmup, windows=3)
+        result["variants"]["bf16_tokens_per_s"] = _rate_summary(t_bf, args.steps)["median"]
         del dec_bf, lm_bf
         torch.cuda.empty_cache()
         result["variants"]["int8"] = bench_int8_variant(config, args.steps, args.warmup)
         result["variants"]["int8_group128"] = bench_int8_variant(config, args.steps, args.warmup, group_size=128)
+        result["variants"]["hf_dropin_generate"] = bench_hf_dropin(config, args.steps)
+        if "new_tokens_per_s" in result["variants"]["hf_dropin_generate"]:
+            result["variants"]["hf_dropin_generate_tokens_per_s"] = result["variants"]["hf_dropin_generate"]["new_tokens_per_s"]
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(config)
         result["cpu_baseline"]["gpu_over_cpu"] = round(tokens_per_s / result["cpu_baseline"]["value"], 1)

@@ -40,6 +40,7 @@ class MuiGraphDecoder:
         2.62 ms per step), graph replay where the layers run as separate module calls and the host
         would be the limit."""
         self.lm = lm
+        self._requested_mode = use_graph  # None: chosen again at every decode() call
         self.use_graph = use_graph
         self.do_sample = do_sample
         self.temperature = float(temperature)
@@ -49,13 +50,17 @@ class MuiGraphDecoder:
         self.top_k = int(top_k) if top_k else None
         self.top_p = float(top_p) if top_p is not None and top_p < 1.0 else None
         if self.top_k or self.top_p:
-            self.use_graph = False
+            self.use_graph = self._requested_mode = False
         self.eos_token_ids = list(eos_token_ids) if eos_token_ids is not None else None
         self.pad_token_id = int(pad_token_id)
         self.graph = None
         self.graph_multi = None  # STEPS_PER_REPLAY steps in one graph, captured on first use
         self._graph_key = None  # what the captured graph has baked in (see _capture_key)
         self.cache: Optional[MuiStaticCache] = None
+        self.owns_cache = False  # True when prefill() created self.cache itself
+        self._window = 0  # sliding window kept in mask4d by every step (0: none)
+        self._embed_table = None
+        self.mask4d = None
         self._batch = None
 
     # -- static device state shared by every replay --
@@ -88,6 +93,11 @@ class MuiGraphDecoder:
     def _step(self):
         """One decode step on the static buffers (this is what gets captured)."""
         fold = self._embed_table is not None
+        if self._window:
+            # sliding window (the reference's mistral/model.py:590-602): the token in slot c sees the
+            # keys after c - window; the window only moves forward, so the keys it leaves behind
+            # stay hidden in the static mask
+            self.mask4d.masked_fill_(self._key_index <= (self.cpos - self._window), torch.finfo(self.mask4d.dtype).min)
         out = self.lm(input_ids=None if fold else self.ids, inputs_embeds=self.hidden if fold else None,
                       position_ids=self.pos, cache_position=self.cpos,
                       past_key_values=self.cache, use_cache=True, attention_mask=self.mask4d,
@@ -135,9 +145,13 @@ class MuiGraphDecoder:
         when the cache grows, which also changes the head stride and the capacity the kernels
         clamp to), the batch size and whether a padding mask is part of the step."""
         c = self.cache
+        # the weights a captured step reads (the embedding table of the folded gather included): a
+        # model moved with .to() or quantised again after the first generate() must be captured anew
+        weights = hash(tuple(t.data_ptr() for t in self.lm.parameters()) + tuple(t.data_ptr() for t in self.lm.buffers()))
         return (id(c), self._batch, c.max_cache_len, tuple(t.data_ptr() for t in c.key_cache),
                 tuple(t.data_ptr() for t in c.value_cache),
-                None if self.mask4d is None else self.mask4d.data_ptr())
+                None if self.mask4d is None else self.mask4d.data_ptr(), self._window, weights,
+                None if self._embed_table is None else self._embed_table.data_ptr())
 
     def _capture(self):
         self.cache.device_length_mode = True
@@ -206,10 +220,13 @@ class MuiGraphDecoder:
         if past and padded:
             raise ValueError("a left-padded prompt needs an empty cache (call cache.reset() first)")
         total = past + prompt_len + max_new_tokens
+        window = getattr(lm.config, "sliding_window", None)
+        windowed = bool(window) and total > int(window)  # decided for the whole generation: a captured step keeps its mask
         max_pos = lm.model.rotary_emb.max_seq_len_cached
         if total > max_pos:
             raise ValueError(f"cached tokens + prompt + max_new_tokens = {total} exceeds the {max_pos} rotary "
                              "positions of this model (max_position_embeddings)")
+        self.owns_cache = cache is None or (cache is self.cache and self.owns_cache)
         if cache is None:
             cache = create_static_cache(lm.engine_config, lm.config, batch, total, device, lm.model.mdtype)
         else:
@@ -232,14 +249,17 @@ class MuiGraphDecoder:
         if self._batch != batch or getattr(self, "_max_new", 0) < max_new_tokens:
             self._alloc_state(batch, max_new_tokens, device)
             self.graph = None
-        if padded:
+        if padded or windowed:
             mdtype = lm.model.mdtype
-            if self.mask4d is None or self.mask4d.shape[-1] != cache.max_cache_len:
+            if self.mask4d is None or self.mask4d.shape[-1] != cache.max_cache_len or self.mask4d.shape[0] != batch:
                 self.mask4d = torch.zeros((batch, 1, 1, cache.max_cache_len), dtype=mdtype, device=device)
             self.mask4d.zero_()
-            self.mask4d[:, 0, 0, :prompt_len].masked_fill_(am == 0, torch.finfo(mdtype).min)
+            if padded:
+                self.mask4d[:, 0, 0, :prompt_len].masked_fill_(am == 0, torch.finfo(mdtype).min)
+            self._key_index = torch.arange(cache.max_cache_len, device=device)
         else:
             self.mask4d = None
+        self._window = int(window) if windowed else 0
         # a captured step is only good for the buffers it was recorded on
         if self.graph is not None and self._graph_key != self._capture_key():
             self.graph = None
@@ -267,7 +287,8 @@ class MuiGraphDecoder:
         gets the same effect with its Synchronizer, csrc/sync.cu:16-118, muillm/sampling/generation.py);
         the few steps issued past the end only write pad tokens."""
         logits_hist = []
-        if self.use_graph is None:
+        if self._requested_mode is None:
+            # chosen per call: another batch size or a caller's cache may change what the layer stack takes
             model = getattr(self.lm, "model", None)
             stack = model._decode_stack(self.cache, self._batch, self.ids) if hasattr(model, "_decode_stack") else None
             self.use_graph = stack is None

@@ -1,7 +1,7 @@
 """MuiLlamaModel / MuiLlamaForCausalLM -- the decoder harness around the fused layers
 (muillm/modules/models/llama/model.py:75-873 of the reference; its Mistral file differs in
 feeding config.sliding_window into the mask -- here the Mistral names alias the Llama classes,
-which serve sequences up to the window and refuse longer ones).
+whose forward() does the same whenever the config carries a sliding window).
 
 Semantics kept from the reference: embed -> N x MuiDecoderLayer -> final MuiRMSNorm ->
 lm_head (MuiLinear) -> fp32 logits; a MuiStaticCache with power-of-two capacity is created
@@ -158,12 +158,15 @@ class MuiLlamaModel(MuiModule):
         return self._stack
 
     def _update_causal_mask(self, attention_mask, inputs_shape, cache_position, past_key_values,
-                            output_attentions, all_ones_mask, past_seen_tokens: int):
+                            output_attentions, all_ones_mask, past_seen_tokens: int,
+                            sliding_window: Optional[int] = None):
         """Additive 4-D mask [B, 1, T, S_total] (0 keep / finfo.min drop), or None when SDPA's
-        is_causal / the mask-free decode kernel suffice (llama/model.py:437-613 of the reference)."""
+        is_causal / the mask-free decode kernel suffice (llama/model.py:437-613 of the reference).
+        sliding_window=W also drops the keys at or before position - W, so that every query sees
+        its last W keys (mistral/model.py:590-602 of the reference)."""
         if (not output_attentions) and _ignore_causal_mask_sdpa(
-                attention_mask, inputs_shape, past_seen_tokens, all_ones_mask=all_ones_mask,
-                is_training=self.training):
+                attention_mask, inputs_shape, past_seen_tokens, sliding_window=sliding_window,
+                all_ones_mask=all_ones_mask, is_training=self.training):
             return None
         bsz, q_len = inputs_shape[0], inputs_shape[1]
         target_length = past_seen_tokens + q_len
@@ -172,7 +175,11 @@ class MuiLlamaModel(MuiModule):
         if attention_mask is not None and attention_mask.dim() == 4:
             return attention_mask
         causal = torch.full((q_len, target_length), fill_value=min_dtype, dtype=dtype, device=device)
-        causal = causal * (torch.arange(target_length, device=device) > cache_position.reshape(-1, 1))
+        keys = torch.arange(target_length, device=device)
+        hidden = keys > cache_position.reshape(-1, 1)
+        if sliding_window is not None:
+            hidden = hidden | (keys <= cache_position.reshape(-1, 1) - int(sliding_window))
+        causal = causal * hidden
         causal = causal[None, None, :, :].expand(bsz, 1, -1, -1)
         if attention_mask is not None:
             causal = causal.clone()
@@ -211,12 +218,13 @@ class MuiLlamaModel(MuiModule):
                              "of this model (max_position_embeddings)")
         if isinstance(past_key_values, MuiStaticCache) and batch_size > past_key_values.max_batch_size:
             raise ValueError(f"batch {batch_size} exceeds the cache's max_batch_size {past_key_values.max_batch_size}")
-        # Mistral's sliding-window attention (the reference feeds config.sliding_window into its mask,
-        # muillm/modules/models/mistral/model.py:484,593-602) is not built: inside the window it is
-        # plain causal attention, beyond it this refuses instead of attending to keys it should not
+        # Mistral's sliding-window attention, as the reference does it: config.sliding_window goes into
+        # the mask (muillm/modules/models/mistral/model.py:484,593-602). Up to the window it is plain
+        # causal attention; beyond it the mask hides the keys at or before position - window, single
+        # tokens take the masked decode kernel and prompts the 4-D-mask route. (A 4-D mask from the
+        # caller is used as it is: the device-resident decode loop maintains the window in its own.)
         window = getattr(self.config, "sliding_window", None)
-        if window and tot_seq_len > int(window):
-            raise NotImplementedError(f"sliding-window attention: {tot_seq_len} tokens exceed sliding_window={window}")
+        windowed = bool(window) and tot_seq_len > int(window)
 
         if use_cache:
             if past_key_values is None:
@@ -233,19 +241,22 @@ class MuiLlamaModel(MuiModule):
         if all_ones_mask is None:
             all_ones_mask = attention_mask is None
         causal_mask = None
-        if not all_ones_mask or q_len > 1:
+        if not all_ones_mask or q_len > 1 or windowed:
             causal_mask = self._update_causal_mask(attention_mask, inputs_shape, cache_position, past_key_values,
-                                                   output_attentions, all_ones_mask, past_seen_tokens)
-        if all_ones_mask and q_len == 1:
+                                                   output_attentions, all_ones_mask, past_seen_tokens,
+                                                   sliding_window=int(window) if windowed else None)
+        if all_ones_mask and q_len == 1 and not windowed:
             causal_mask = None
         elif causal_mask is not None:
             causal_mask = causal_mask[:, :, :, :tot_seq_len]
+        if windowed:
+            all_ones_mask = False  # the layers must apply the mask even without padding
         # a padded prompt whose 4-D mask was built right here from a 2-D one: the attention layers
         # get the key padding as such and keep the library's prompt kernel (a 4-D mask from the
         # caller may hold anything and stays with SDPA)
         key_padding_mask = None
         if (causal_mask is not None and q_len > 1 and attention_mask is not None and attention_mask.dim() == 2
-                and torch.device(self.mdevice).type == "cuda" and self.mdtype in (torch.float16, torch.bfloat16)):
+                and not windowed and torch.device(self.mdevice).type == "cuda" and self.mdtype in (torch.float16, torch.bfloat16)):
             key_padding_mask = muillm_ext.key_padding_mask16(attention_mask, self.mdtype, tot_seq_len)
         position_ids = position_ids.contiguous()
 
@@ -425,8 +436,10 @@ class MuiLlamaForCausalLM(MuiModule):
     @staticmethod
     def _reusable_cache(dec, cache, input_ids):
         """Without a cache from the caller, a kept decoder starts again on its own (emptied) cache
-        when the batch size fits: same buffers, so its captured graph stays valid."""
-        if cache is None and dec.cache is not None and dec.cache.max_batch_size == input_ids.shape[0] \
+        when the batch size fits: same buffers, so its captured graph stays valid. A cache that a
+        caller handed to an earlier call is the caller's (multi-turn state) and is never touched."""
+        if cache is None and dec.cache is not None and dec.owns_cache \
+                and dec.cache.max_batch_size == input_ids.shape[0] \
                 and dec.cache.key_cache[0].device == input_ids.device:
             dec.cache.reset()
             return dec.cache
@@ -462,7 +475,7 @@ class MuiLlamaForCausalLM(MuiModule):
                             stop_check_every=8 if eos else 0)
 
 
-# Mistral shares the Llama implementation up to config.sliding_window tokens (forward() refuses
-# longer sequences: the reference's mistral/model.py:484,593-602 masks keys outside the window)
+# Mistral shares the Llama implementation; config.sliding_window, where set, goes into the attention
+# mask once a sequence outgrows it (forward() above; the reference's mistral/model.py:484,593-602)
 MuiMistralModel = MuiLlamaModel
 MuiMistralForCausalLM = MuiLlamaForCausalLM

@@ -365,11 +365,13 @@ def decoder_layer(
     n_heads: int,
     n_kv_heads: int,
     store_dtype: torch.dtype = torch.float16,
+    sliding_window: Optional[int] = None,
 ):
     """One decoder layer with the rounding points of the fused path: q/k/v, attention
     output, post-attention hidden state and MLP intermediate are stored in `store_dtype`
     between kernels; everything inside a kernel is float64 here.
-    Causal masking is applied for T > 1 (prefill)."""
+    Causal masking is applied for T > 1 (prefill). sliding_window=W hides, from the query in
+    cache slot c, the keys at or before c - W (muillm/modules/models/mistral/model.py:590-602)."""
     b, t, hid = h.shape
     d = hid // n_heads
     eps = p["eps"]
@@ -382,11 +384,14 @@ def decoder_layer(
     qr, kr = rnd(qr), rnd(kr)
     kk, vv, seen = static_cache_update(k_cache, v_cache, kr, v, cache_position, seen_tokens)
     mask = None
-    if t > 1:
+    if t > 1 or (sliding_window is not None and kk.shape[2] > sliding_window):
         s = kk.shape[2]
         qpos = cache_position.view(t, 1)
         kpos = torch.arange(s).view(1, s)
-        mask = torch.where(kpos <= qpos, 0.0, float("-inf")).to(_HI).view(1, 1, t, s)
+        visible = kpos <= qpos
+        if sliding_window is not None:
+            visible = visible & (kpos > qpos - sliding_window)
+        mask = torch.where(visible, 0.0, float("-inf")).to(_HI).view(1, 1, t, s)
     attn = rnd(decode_attention(qr, kk, vv, mask))
     h1 = rnd(linear(attn, p["wo"], residual=h))
     out = gateupdown_mlp(h1, p["wg"], p["wu"], p["wd"], p["ln2"], eps, residual=h1,
@@ -398,7 +403,8 @@ def decoder_layer(
 # Whole decoder -- muillm/modules/models/llama/model.py:298-322,360-406,778-785
 # --------------------------------------------------------------------------------------
 def decoder_model_step(ids, params, k_caches, v_caches, cos, sin, seen_tokens: int, n_heads: int,
-                       n_kv_heads: int, store_dtype: torch.dtype = torch.float16):
+                       n_kv_heads: int, store_dtype: torch.dtype = torch.float16,
+                       sliding_window: Optional[int] = None):
     """Embed -> layers -> final RMSNorm -> lm_head for `ids` [B, T] appended after
     `seen_tokens` cached tokens. params: {'embed', 'layers': [layer dicts], 'norm', 'lm_head',
     'eps'}. Returns (logits float64 [B, T, V], new seen_tokens). Hidden states between layers
@@ -410,7 +416,7 @@ def decoder_model_step(ids, params, k_caches, v_caches, cos, sin, seen_tokens: i
     seen = seen_tokens
     for li, lp in enumerate(params["layers"]):
         h, seen = decoder_layer(h, lp, k_caches[li], v_caches[li], cos, sin, pos, cpos, seen_tokens,
-                                n_heads, n_kv_heads, store_dtype)
+                                n_heads, n_kv_heads, store_dtype, sliding_window)
     hn = rmsnorm(h, params["norm"], params["eps"]).to(store_dtype)
     return linear(hn, params["lm_head"]), seen
 

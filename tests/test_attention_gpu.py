@@ -8,12 +8,14 @@ static-cache test (tests/test_static_kvcache.py:52-112 there)."""
 
 import functools
 import math
+import os
 
 import pytest
 import torch
 
 import oracle
 from muillm_amd import _lib, muillm_ext
+from tests.util import record_error
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -46,7 +48,10 @@ def _mk(shape, g, std=1.0, dtype=torch.float16):
 
 
 def _max_abs(got, ref):
-    return float((got.detach().cpu().double().reshape(-1) - ref.double().reshape(-1)).abs().max())
+    err = float((got.detach().cpu().double().reshape(-1) - ref.double().reshape(-1)).abs().max())
+    test = os.environ.get("PYTEST_CURRENT_TEST", "").split("::")[-1].split(" ")[0]
+    record_error("%s [%s]" % (test, str(got.dtype).replace("torch.", "")), err, ATOL, "max_abs")
+    return err
 
 
 # ------------------------------------------------------------------------------------

@@ -1,10 +1,13 @@
 """Parity at the sizes the benchmark is quoted on (Llama-3-8B shape: hidden 4096, intermediate
 14336, 32 query / 8 KV heads of 128, RMSNorm eps 1e-5, weights ~ N(0, 0.02)):
 
-* one full-shape decoder layer (+ embedding, final norm and a small lm_head) against the CPU
-  oracle, 32-token prompt then single-token decode steps: fp16, bf16 and per-channel int8;
-* the whole 32-layer model: tokens and logits of HIP-graph replay == eager decode, bit for bit,
-  for a 32-token prompt + 32 greedy steps (fp16, bf16, per-channel int8).
+* two full-shape decoder layers (+ embedding, final norm and a small lm_head) against the CPU
+  oracle, 32-token prompt then single-token decode steps: fp16, bf16 and per-channel int8 (two
+  layers, so that an error in the hand-off between layers at this width cannot hide);
+* the whole 32-layer model as the benchmark runs it -- 32-token prompt, 256 greedy steps, static
+  cache of 512 slots: tokens and per-step logits identical, bit for bit, between stream launches
+  through the one-call layer stack (the decoder's default), HIP-graph replay and the walk over the
+  layer modules (fp16, bf16, per-channel int8 and the reference's group-of-128 int8 format).
 
 The second test follows the recipe of the reference's static-cache test (prefill, then
 single-token steps over a growing static cache, tests/test_static_kvcache.py:52-112 there)."""
@@ -65,14 +68,14 @@ def _oracle_params(lm):
                 eps=cfg.rms_norm_eps)
 
 
-def _build(layers, vocab, dtype, int8, seed):
+def _build(layers, vocab, dtype, int8, seed, group_size=0):
     cfg = _cfg(layers, vocab)
     if not int8:
         return MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=dtype, device=DEV, seed=seed,
                                                init_std=0.02)
     base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=dtype, device=DEV, seed=seed,
                                            init_std=0.02, finalize=False)
-    qm = Int8WeightOnlyQuantizationMethod(group_size=0, modules=["qkv_proj", "o_proj", "mlp"])
+    qm = Int8WeightOnlyQuantizationMethod(group_size=group_size, modules=["qkv_proj", "o_proj", "mlp"])
     return init_engine(base, device=DEV, engine_config=MuiEngineConfig(qm))
 
 
@@ -85,7 +88,8 @@ def test_full_shape_decoder_layer_vs_oracle(kind):
     exact: a 2^-9 relative perturbation of every operand of five chained projections, which over
     65536 logits puts a handful beyond 3 % of the logits' rms."""
     dtype = torch.bfloat16 if kind == "bf16" else torch.float16
-    lm = _build(1, 2048, dtype, kind == "int8", seed=21)
+    n_layers = 2
+    lm = _build(n_layers, 2048, dtype, kind == "int8", seed=21)
     with torch.no_grad():
         # norm gammas away from 1 so that a dropped or misplaced gamma shows
         for layer in lm.model.layers:
@@ -94,8 +98,8 @@ def test_full_shape_decoder_layer_vs_oracle(kind):
     params = _oracle_params(lm)
     cos, sin = oracle.rope_tables(500000.0, D, 512)
     ids = torch.randint(0, 2048, (1, 32), generator=torch.Generator().manual_seed(3))
-    kcs = [torch.zeros(1, HKV, 64, D, dtype=dtype)]
-    vcs = [torch.zeros(1, HKV, 64, D, dtype=dtype)]
+    kcs = [torch.zeros(1, HKV, 64, D, dtype=dtype) for _ in range(n_layers)]
+    vcs = [torch.zeros(1, HKV, 64, D, dtype=dtype) for _ in range(n_layers)]
     tol = 3e-2 if kind == "bf16" else 1e-2
     elem = 5e-2 if kind == "bf16" else None
     ref, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, HQ, HKV, store_dtype=dtype)
@@ -111,26 +115,44 @@ def test_full_shape_decoder_layer_vs_oracle(kind):
             out = lm(input_ids=nxt.unsqueeze(1).to(DEV), past_key_values=cache)
         assert_parity(out.logits, ref, tol, f"{kind} full-shape decode step {step}", elementwise=elem)
         nxt = ref[:, -1].argmax(-1)
-    # the layer's cache rows equal the oracle's within one 16-bit ulp of rounding flips
+    # the first layer's cache rows equal the oracle's within one 16-bit ulp of rounding flips
     kd = cache.key_cache[0][:, :, :seen].float().cpu()
     assert float((kd - kcs[0][:, :, :seen].float()).abs().max()) <= (0.05 if kind == "bf16" else 0.01)
 
 
-@pytest.mark.parametrize("kind", ["fp16", "bf16", "int8"])
-def test_full_model_graph_replay_equals_eager(kind):
-    """The 32-layer, vocabulary-128256 model the headline number is quoted on: 32-token prompt,
-    32 greedy steps; tokens and per-step logits identical between HIP-graph replay and eager."""
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "int8", "int8_group128"])
+def test_full_model_256_steps_every_launch_mode(kind):
+    """The 32-layer, vocabulary-128256 model the headline number is quoted on, as the benchmark runs
+    it: 32-token prompt, 256 greedy steps, cache capacity 512. Tokens and the logits of every step
+    are identical between stream launches through the one-call layer stack (the decoder's default
+    mode), HIP-graph replay and the per-layer module calls (the recipe of the reference's
+    tests/test_static_kvcache.py:52-112: prefill, then single-token steps over the static cache)."""
     dtype = torch.bfloat16 if kind == "bf16" else torch.float16
-    lm = _build(32, 128256, dtype, kind == "int8", seed=0)
+    lm = _build(32, 128256, dtype, kind.startswith("int8"), seed=0, group_size=128 if kind == "int8_group128" else 0)
     ids = torch.randint(0, 128256, (1, 32), generator=torch.Generator().manual_seed(0)).to(DEV)
-    n_new = 32
-    eager, eager_logits = lm.generate_greedy(ids, n_new, use_graph=False, return_logits=True)
+    n_new = 256
+    dec_default = MuiGraphDecoder(lm, use_graph=None)
+    stream, stream_logits = dec_default.generate(ids, n_new, return_logits=True)
+    assert dec_default.use_graph is False, "the one-call layer stack did not take this model"
+    assert dec_default.cache.get_max_length() == 512
+    assert stream.shape == (1, 32 + n_new) and torch.isfinite(stream_logits).all()
+    assert len(set(stream[0, 32:].tolist())) > 1, "degenerate generation"
     dec = MuiGraphDecoder(lm, use_graph=True)
     graph, graph_logits = dec.generate(ids, n_new, return_logits=True)
-    assert eager.shape == (1, 32 + n_new)
-    assert torch.isfinite(eager_logits).all()
-    assert torch.equal(eager, graph), "graph replay and eager decode disagree"
-    assert torch.equal(eager_logits, graph_logits)
-    assert len(set(eager[0, 32:].tolist())) > 1, "degenerate generation"
-    del lm, dec
+    assert torch.equal(stream, graph), "graph replay and stream launches disagree"
+    assert torch.equal(stream_logits, graph_logits)
+    del graph_logits, dec
+    # without collecting logits the graph decoder replays several steps per launch
+    dec = MuiGraphDecoder(lm, use_graph=True)
+    assert torch.equal(dec.generate(ids, n_new), stream)
+    del dec
+    lm.model.use_decoder_stack = False  # the layer modules, one call per kernel
+    try:
+        dec = MuiGraphDecoder(lm, use_graph=False)
+        modules, module_logits = dec.generate(ids, n_new, return_logits=True)
+    finally:
+        lm.model.use_decoder_stack = True
+    assert torch.equal(stream, modules), "layer modules and the one-call stack disagree"
+    assert torch.equal(stream_logits, module_logits)
+    del lm, dec, dec_default
     torch.cuda.empty_cache()

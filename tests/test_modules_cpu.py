@@ -326,12 +326,72 @@ def test_forward_refuses_a_batch_larger_than_the_cache():
         lm(input_ids=torch.randint(0, 64, (2, 4)), past_key_values=cache)
 
 
-def test_sliding_window_is_refused_beyond_the_window():
-    lm = _tiny_lm(max_pos=64, sliding_window=8)
+@pytest.mark.skipif(not _hf.HAVE_TRANSFORMERS, reason="transformers not installed")
+def test_sliding_window_matches_hf_mistral_and_the_oracle():
+    """A Mistral config with sliding_window=8 on 20 tokens: the converted model's full forward (mask
+    route) and its prefill + single-token steps across the window's edge give HuggingFace's logits;
+    the oracle's sliding mask gives them too (which pins it for the GPU tests)."""
+    torch.manual_seed(0)
+    kw = dict(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+              num_key_value_heads=1, vocab_size=320, max_position_embeddings=128, rms_norm_eps=1e-5)
+    hf = _hf.MistralForCausalLM(_hf.MistralConfig(**kw, sliding_window=8)).eval()
+    hf_full = _hf.MistralForCausalLM(_hf.MistralConfig(**kw, sliding_window=None)).eval()
+    hf_full.load_state_dict(hf.state_dict())
+    ids = torch.randint(0, 320, (2, 20))
     with torch.no_grad():
-        out = lm(input_ids=torch.randint(0, 64, (1, 8)))                    # inside the window: plain causal
-        with pytest.raises(NotImplementedError, match="sliding"):
-            lm(input_ids=torch.randint(0, 64, (1, 1)), past_key_values=out.past_key_values)
+        ref = hf(input_ids=ids, use_cache=False).logits
+        ref_full = hf_full(input_ids=ids, use_cache=False).logits
+    assert float((ref - ref_full)[:, 8:].abs().max()) > 1e-3  # the window does change the result here
+    assert torch.allclose(ref[:, :8], ref_full[:, :8], atol=1e-5)
+    model = init_engine(copy.deepcopy(hf), device="cpu")
+    with torch.no_grad():
+        out = model(input_ids=ids)
+        assert torch.allclose(out.logits, ref, atol=3e-4, rtol=1e-4)
+        cache = model(input_ids=ids[:, :5]).past_key_values
+        for t in range(5, 20):
+            step = model(input_ids=ids[:, t : t + 1], past_key_values=cache)
+            assert torch.allclose(step.logits[:, 0], ref[:, t], atol=3e-4, rtol=1e-4), t
+    # the oracle with the same window
+    sd = {k: v.double() for k, v in hf.state_dict().items()}
+    layers = []
+    for i in range(2):
+        p = f"model.layers.{i}."
+        layers.append(dict(ln1=sd[p + "input_layernorm.weight"], wq=sd[p + "self_attn.q_proj.weight"],
+                           wk=sd[p + "self_attn.k_proj.weight"], wv=sd[p + "self_attn.v_proj.weight"],
+                           wo=sd[p + "self_attn.o_proj.weight"], ln2=sd[p + "post_attention_layernorm.weight"],
+                           wg=sd[p + "mlp.gate_proj.weight"], wu=sd[p + "mlp.up_proj.weight"],
+                           wd=sd[p + "mlp.down_proj.weight"], eps=1e-5))
+    params = dict(embed=sd["model.embed_tokens.weight"], layers=layers, norm=sd["model.norm.weight"],
+                  lm_head=sd["lm_head.weight"], eps=1e-5)
+    cos, sin = oracle.rope_tables(_hf.rope_theta_of(hf.config), 128, 32)
+    mk = lambda: [torch.zeros(2, 1, 32, 128, dtype=torch.float64) for _ in range(2)]
+    kc, vc = mk(), mk()
+    lg, seen = oracle.decoder_model_step(ids, params, kc, vc, cos, sin, 0, 2, 1, store_dtype=torch.float64, sliding_window=8)
+    assert torch.allclose(lg, ref.double(), atol=2e-4)
+    kc, vc = mk(), mk()
+    lg, seen = oracle.decoder_model_step(ids[:, :5], params, kc, vc, cos, sin, 0, 2, 1, store_dtype=torch.float64, sliding_window=8)
+    for t in range(5, 20):
+        lg, seen = oracle.decoder_model_step(ids[:, t : t + 1], params, kc, vc, cos, sin, seen, 2, 1,
+                                             store_dtype=torch.float64, sliding_window=8)
+        assert torch.allclose(lg[:, 0], ref[:, t].double(), atol=2e-4), t
+
+
+def test_reusable_cache_never_touches_a_callers_cache():
+    """generate(ids, cache=mine) followed by generate(other_ids) must not reset or reuse `mine`: only a
+    cache the decoder created itself is recycled."""
+    from muillm_amd.modules.models.graphdecoder import MuiGraphDecoder
+
+    lm = _tiny_lm(max_pos=64)
+    dec = MuiGraphDecoder(lm, use_graph=False)
+    mine = create_static_cache(MuiEngineConfig(), lm.config, max_batch_size=1, seq_len=16, device="cpu", dtype=torch.float32)
+    ids = torch.randint(0, 64, (1, 4))
+    dec.cache, dec.owns_cache = mine, False  # what prefill(ids, n, cache=mine) records
+    assert MuiLlamaForCausalLM._reusable_cache(dec, None, ids) is None
+    dec.owns_cache = True  # a cache prefill() created itself is recycled (emptied)
+    mine._seen_tokens = 5
+    assert MuiLlamaForCausalLM._reusable_cache(dec, None, ids) is mine and mine.get_seq_length() == 0
+    other = create_static_cache(MuiEngineConfig(), lm.config, max_batch_size=1, seq_len=16, device="cpu", dtype=torch.float32)
+    assert MuiLlamaForCausalLM._reusable_cache(dec, other, ids) is other
 
 
 def test_graph_decoder_prefill_guards_and_capture_key():

@@ -246,6 +246,46 @@ def test_graph_decode_matches_eager(batch):
     assert dec.cache.get_seq_length() == 32 + n_new - 1
 
 
+@pytest.mark.parametrize("prompt_len", [8, 24])
+def test_sliding_window_generation_both_launch_modes(prompt_len):
+    """A Mistral-style config with sliding_window=16: generations that start inside the window and
+    cross it (prompt 8) or start beyond it (prompt 24, whose prefill takes the masked route) give the
+    oracle's windowed logits step by step, the same tokens and bit-identical logits from stream
+    launches and from HIP-graph replay, and differ from the unwindowed model once the window is
+    left (the reference's mistral/model.py:590-602)."""
+    cfg = _small_config(layers=2)
+    cfg.sliding_window = 16
+    lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), cfg, dtype=torch.float16, device=DEV, seed=11,
+                                         init_std=0.05)
+    params = _oracle_params(lm)
+    d = 128
+    cos, sin = oracle.rope_tables(cfg.rope_theta, d, cfg.max_position_embeddings)
+    ids = torch.randint(0, cfg.vocab_size, (2, prompt_len), generator=torch.Generator().manual_seed(3))
+    n_new = 20
+    runs = []
+    for use_graph in (False, True, None):
+        dec = MuiGraphDecoder(lm, use_graph=use_graph)
+        toks, logits = dec.generate(ids.to(DEV), n_new, return_logits=True)
+        assert dec._window == 16 and dec.mask4d is not None
+        runs.append((toks.cpu(), logits.cpu()))
+    for toks, logits in runs[1:]:
+        assert torch.equal(toks, runs[0][0]) and torch.equal(logits, runs[0][1])
+    toks, logits = runs[0]
+    # teacher-forced oracle over the generated sequence, with and without the window
+    for window, must_match in ((16, True), (None, False)):
+        kcs = [torch.zeros(2, 2, 64, d, dtype=torch.float16) for _ in range(2)]
+        vcs = [torch.zeros(2, 2, 64, d, dtype=torch.float16) for _ in range(2)]
+        ref, seen = oracle.decoder_model_step(toks[:, :prompt_len], params, kcs, vcs, cos, sin, 0, 4, 2, sliding_window=window)
+        worst = oracle.rel_err(logits[:, 0], ref[:, -1])
+        for step in range(1, n_new):
+            ref, seen = oracle.decoder_model_step(toks[:, prompt_len + step - 1 : prompt_len + step], params, kcs, vcs,
+                                                  cos, sin, seen, 4, 2, sliding_window=window)
+            if must_match:
+                assert_parity(logits[:, step], ref[:, 0], 1e-2, f"windowed decode step {step} (prompt {prompt_len})")
+            worst = max(worst, oracle.rel_err(logits[:, step], ref[:, 0]))
+        assert (worst <= 1e-2) == must_match, (window, worst)
+
+
 def test_graph_decode_several_steps_per_replay():
     """decode() without stop checks or logits collection replays STEPS_PER_REPLAY steps per graph
     launch and finishes with single-step replays: tokens, the logits of the last step and the cache

@@ -189,6 +189,54 @@ def test_channel_rtn_closed_forms():
     assert float(s2[0]) == 1 / 64 and q2.tolist() == [[127, 2, 4, -2]]
 
 
+def test_int8_linear_compositions_brute_force():
+    """The two dequantise-then-linear oracle functions against numpy loops that index every code,
+    scale and minimum themselves: distinct per-row / per-group (scale, min) values, so that a
+    swapped column, a transposed scale or a wrong group index changes the result."""
+    rng = np.random.default_rng(7)
+    n, k, gs = 3, 8, 4
+    x = rng.standard_normal((2, k))
+    bias, res = rng.standard_normal(n), rng.standard_normal((2, n))
+    xt, bt, rt = torch.from_numpy(x), torch.from_numpy(bias), torch.from_numpy(res)
+    # per-channel: y[t, r] = sum_j x[t, j] * q[r, j] * s[r] + bias[r] + res[t, r]
+    q = rng.integers(-127, 128, size=(n, k)).astype(np.int8)
+    s = np.array([2.0 ** -6, 3 * 2.0 ** -9, 5 * 2.0 ** -8], dtype=np.float16)  # exact products in fp16
+    want = np.zeros((2, n))
+    for t in range(2):
+        for r in range(n):
+            acc = 0.0
+            for j in range(k):
+                acc += x[t, j] * (float(q[r, j]) * float(s[r]))
+            want[t, r] = acc + bias[r] + res[t, r]
+    got = oracle.int8_channel_linear(xt, torch.from_numpy(q), torch.from_numpy(s), None, 0.0, bt, rt)
+    # the per-channel oracle rounds q*s to fp16 (the dense dequantisation): exact for these scales
+    assert np.abs(got.numpy() - want).max() < 1e-12
+    same = oracle.linear(xt, torch.from_numpy(q).double() * torch.from_numpy(s).double()[:, None], None, 0.0, bt, rt)
+    assert torch.allclose(got, same, atol=1e-12, rtol=0)
+    # group format: row r, group g owns pair r * (k / gs) + g: w = code * scale + min, not rounded
+    qu = rng.integers(0, 256, size=(n, k)).astype(np.uint8)
+    smv = (rng.standard_normal((n * (k // gs), 2)) * 0.01).astype(np.float16)
+    want = np.zeros((2, n))
+    for t in range(2):
+        for r in range(n):
+            acc = 0.0
+            for j in range(k):
+                pair = smv[r * (k // gs) + j // gs]
+                acc += x[t, j] * (float(qu[r, j]) * float(pair[0]) + float(pair[1]))
+            want[t, r] = acc + bias[r] + res[t, r]
+    got = oracle.int8_group_linear(xt, torch.from_numpy(qu), torch.from_numpy(smv), gs, None, 0.0, bt, rt)
+    assert np.abs(got.numpy() - want).max() < 1e-12
+    # and against the pinned dense dequantisation (fp32 result of the fma, before the 16-bit store)
+    dq = oracle.rtn_dequantize_group(torch.from_numpy(qu), torch.from_numpy(smv), gs, torch.float32)
+    via_dq = oracle.linear(xt, dq, None, 0.0, bt, rt)
+    assert float((got - via_dq).abs().max()) < 1e-5
+    # a fused norm goes in front of both, as in linear()
+    gam = torch.from_numpy(rng.standard_normal(k))
+    a = oracle.int8_channel_linear(xt, torch.from_numpy(q), torch.from_numpy(s), gam, 1e-5)
+    b = oracle.linear(oracle.rmsnorm(xt, gam, 1e-5), torch.from_numpy(q).double() * torch.from_numpy(s).double()[:, None])
+    assert torch.allclose(a, b, atol=1e-12, rtol=0)
+
+
 def test_rope_properties_and_brute_force():
     d = 8
     cos, sin = oracle.rope_tables(10000.0, d, 64)

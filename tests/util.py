@@ -1,5 +1,19 @@
 """Shared checks for the parity tests."""
+import json
+import os
+
 import torch
+
+
+def record_error(what: str, measured: float, gate: float, kind: str = "max_rel"):
+    """Every parity assertion reports what it measured: printed (pytest -s / -rP show it) and, when
+    MUI_PARITY_LOG names a file, appended there as one JSON line per assertion."""
+    line = {"what": what, "kind": kind, "measured": float(measured), "gate": float(gate)}
+    print("parity %s: %s = %.3e (gate %.1e)" % (what, kind, measured, gate))
+    path = os.environ.get("MUI_PARITY_LOG")
+    if path:
+        with open(path, "a") as f:
+            f.write(json.dumps(line) + "\n")
 
 
 def assert_parity(got: torch.Tensor, ref: torch.Tensor, rel: float = 1e-2, what: str = "", tight: float = None,
@@ -17,8 +31,13 @@ def assert_parity(got: torch.Tensor, ref: torch.Tensor, rel: float = 1e-2, what:
     denom = r.abs().max().clamp_min(1e-30)
     rms = r.pow(2).mean().sqrt().clamp_min(1e-30)
     max_rel = float(err.max() / denom)
-    assert max_rel <= rel, f"{what}: max rel err {max_rel:.3e} > {rel}"
     e = rel if elementwise is None else elementwise
+    # smallest factor f for which |got-ref| <= f*|ref| + f*rms(ref) holds everywhere
+    elem_needed = float((err / (r.abs() + rms)).max())
+    tag = "%s [%s]" % (what, str(got.dtype).replace("torch.", ""))
+    record_error(tag, max_rel, rel, "max_err_over_max_ref")
+    record_error(tag, elem_needed, e, "elementwise_factor")
+    assert max_rel <= rel, f"{what}: max rel err {max_rel:.3e} > {rel}"
     bad = err > e * r.abs() + e * rms
     assert not bool(bad.any()), f"{what}: {int(bad.sum())} elements outside {e}*|ref|+{e}*rms"
     if tight is not None:
