@@ -42,6 +42,14 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16 matrix-core peak
 BASELINE_TOKENS_PER_S = 210.0  # reference README: Llama-3-8B fp16 bs1 on 1x MI300X
 
 
+def _progress(msg):
+    """Stage marker on stderr (stdout carries the one JSON line): a long run stays visibly alive."""
+    print("[bench %.0fs] %s" % (time.perf_counter() - _T0, msg), file=sys.stderr, flush=True)
+
+
+_T0 = time.perf_counter()
+
+
 def _event_time_us(fn, iters, warm):
     import torch
 
@@ -1012,6 +1020,7 @@ def main():
     if args.only_kernel_table:
         print(json.dumps({"kernels": kernel_table(lm)}))
         return
+    _progress("model built; headline decode windows")
     times, dec = bench_decode(lm, args.steps, args.warmup, windows=args.windows)
     times = times if isinstance(times, list) else [times]
     head = _rate_summary(times, args.steps)
@@ -1049,14 +1058,17 @@ def main():
             "end_to_end_frac_of_hbm_floor": round(weight_bytes / (HBM_PEAK_GBPS * 1e9) / (dt / args.steps), 4),
         },
     }
+    _progress("headline %.2f tokens/s; roofline" % tokens_per_s)
     result["roofline"] = gateup_roofline(lm)
     result["roofline"]["measured_copy_ceiling_GB/s"] = measured_copy_ceiling()
     result["roofline"]["measured_read_ceiling_GB/s"] = measured_read_ceiling()
     if not args.no_kernel_table:
+        _progress("kernel table")
         result["kernels"] = kernel_table(lm)
     del dec
     if not args.no_variants:
         # the two launch modes, each forced, on the headline's step counts
+        _progress("variants: launch modes")
         t_g, dec_g = bench_decode(lm, args.steps, args.warmup, use_graph=True, windows=args.windows)
         t_e, dec_e = bench_decode(lm, args.steps, args.warmup, use_graph=False, windows=args.windows)
         t_g, t_e = (t if isinstance(t, list) else [t] for t in (t_g, t_e))
@@ -1070,9 +1082,11 @@ def main():
             result["variants"]["fp16_context%d_tokens_per_s" % ctx] = round(64 / dt_c, 2)
             del dec_c
             torch.cuda.empty_cache()
+        _progress("variants: prefill")
         for ptoks in (512, 4096):
             result["variants"]["prefill_%d" % ptoks] = bench_prefill(lm, ptoks)
             torch.cuda.empty_cache()
+        _progress("variants: batches")
         for bsz in (4, 8, 16):
             dt_b, dec_b = bench_decode(lm, min(args.steps, 128), min(args.warmup, 8), batch=bsz)
             result["variants"]["fp16_batch%d_aggregate_tokens_per_s" % bsz] = round(bsz * min(args.steps, 128) / dt_b, 1)
@@ -1080,17 +1094,22 @@ def main():
             del dec_b
         del lm
         torch.cuda.empty_cache()
+        _progress("variants: bf16")
         lm_bf = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.bfloat16, device="cuda", seed=0)
         t_bf, dec_bf = bench_decode(lm_bf, args.steps, args.warmup, windows=3)
         result["variants"]["bf16_tokens_per_s"] = _rate_summary(t_bf, args.steps)["median"]
         del dec_bf, lm_bf
         torch.cuda.empty_cache()
+        _progress("variants: int8")
         result["variants"]["int8"] = bench_int8_variant(config, args.steps, args.warmup)
+        _progress("variants: int8 group 128")
         result["variants"]["int8_group128"] = bench_int8_variant(config, args.steps, args.warmup, group_size=128)
+        _progress("variants: HuggingFace drop-in generate()")
         result["variants"]["hf_dropin_generate"] = bench_hf_dropin(config, args.steps)
         if "new_tokens_per_s" in result["variants"]["hf_dropin_generate"]:
             result["variants"]["hf_dropin_generate_tokens_per_s"] = result["variants"]["hf_dropin_generate"]["new_tokens_per_s"]
     if not args.no_cpu_baseline:
+        _progress("cpu baseline")
         result["cpu_baseline"] = cpu_baseline(config)
         result["cpu_baseline"]["gpu_over_cpu"] = round(tokens_per_s / result["cpu_baseline"]["value"], 1)
     print(json.dumps(result))
