@@ -418,6 +418,62 @@ def _graph_chain_us(launch, n=400, replays=10):
     return round(a.elapsed_time(b) * 1e3 / (replays * n), 3)
 
 
+def probe_warm(lm, steps, warmup):
+    """Cache warming by the idle workgroups of the short-context attention launch
+    (mui_attn_decode_fused_warm): the pair [fused RoPE + cache write + attention at 64 cached tokens,
+    o_proj GEMV + residual] over the model's 32 o_proj matrices, HIP-event timed, and the decode
+    rate on stream launches, for a few settings of mui_tune_warm (workgroups, percent) in one process."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    f16 = dict(device="cuda", dtype=torch.float16)
+    hq, hkv, d, S = 32, 8, 128, 64
+    hid = lm.config.hidden_size
+    layers = lm.model.layers
+    op = [l.self_attn.o_proj.weight for l in layers]
+    qs = (hq + 2 * hkv) * d
+    qkvx = torch.randn(1, qs, **f16)
+    caches = [(torch.randn(1, hkv, 512, d, **f16), torch.randn(1, hkv, 512, d, **f16)) for _ in layers]
+    cos, sin = [t.cuda() for t in _rope_tables_f32(512, d)]
+    pos = torch.full((1, 1), S - 1, dtype=torch.int64, device="cuda")
+    cpos = torch.full((1,), S - 1, dtype=torch.int64, device="cuda")
+    o = torch.empty(1, hq * d, **f16)
+    res, y = torch.randn(hid, **f16), torch.empty(hid, **f16)
+    slab = lib.mui_linear_row_group_bytes(16, hq * d, op[0].stride(0) * 2)
+
+    def pair(i, attn_only=False, gemv_only=False):
+        kc, vc = caches[i % len(caches)]
+        w = op[i % len(op)]
+        if not gemv_only:
+            lib.mui_attn_decode_fused_warm(stream, 0, qkvx.data_ptr(), qs, qkvx.data_ptr() + 2 * hq * d, qs,
+                                           qkvx.data_ptr() + 2 * (hq + hkv) * d, qs, cos.data_ptr(), sin.data_ptr(), d // 2,
+                                           cos.shape[0], pos.data_ptr(), 1, cpos.data_ptr(), S, kc.data_ptr(), vc.data_ptr(),
+                                           hkv * 512 * d, 512 * d, d, None, 0, None, None, 1, o.data_ptr(), 1, hq, hkv, d, 512,
+                                           w.data_ptr(), w.numel() * 2, slab)
+        if not attn_only:
+            lib.mui_linear(stream, 0, w.data_ptr(), w.stride(0), o.data_ptr(), None, 0.0, None, None, res.data_ptr(),
+                           y.data_ptr(), hid, hq * d, 1)
+
+    out = {"slab_bytes": slab}
+    settings = [("off", -1, 0), ("wg256_pct100", 256, 100), ("wg256_pct75", 256, 75), ("wg256_pct50", 256, 50),
+                ("wg128_pct100", 128, 100), ("wg512_pct100", 512, 100), ("wg224_pct90", 224, 90), ("off_again", -1, 0)]
+    for name, wgs, pct in settings:
+        _lib.check(lib.mui_tune_warm(wgs, pct), "mui_tune_warm")
+        row = {"attention+o_proj_us": round(_median([_event_time_us(pair, 320, 64) for _ in range(3)]), 2),
+               "attention_us": round(_median([_event_time_us(lambda i: pair(i, attn_only=True), 320, 64) for _ in range(3)]), 2),
+               "o_proj_alone_us": round(_median([_event_time_us(lambda i: pair(i, gemv_only=True), 320, 64) for _ in range(3)]), 2)}
+        times, dec = bench_decode(lm, steps, warmup, use_graph=False, windows=3)
+        row["decode_tokens_per_s"] = _rate_summary(times, steps)
+        del dec
+        out[name] = row
+        _progress("probe-warm %s: %s" % (name, row))
+    _lib.check(lib.mui_tune_warm(0, 0), "mui_tune_warm")
+    print(json.dumps({"probe_warm": out}))
+
+
 def probe_kernel_boundary():
     """What one dependent kernel costs inside a replayed HIP graph when it has next to nothing to do:
     the read probe over 16 B and over 64 KiB, and a 256 x 256 GEMV (alone, and two of them feeding each
@@ -963,6 +1019,8 @@ def main():
                     help="launch flash decoding at 32k context a few times and exit (for rocprofv3 --pmc)")
     ap.add_argument("--probe-kernel-boundary", action="store_true",
                     help="time chains of near-empty dependent kernels in a replayed HIP graph and exit")
+    ap.add_argument("--probe-warm", action="store_true",
+                    help="time attention + o_proj and the decode rate over cache-warming settings and exit")
     ap.add_argument("--probe-flash-splits", action="store_true",
                     help="time fused flash decoding at batch 1 over the number of sequence splits and exit")
     ap.add_argument("--probe-prompt", action="store_true",
@@ -1019,6 +1077,9 @@ def main():
 
     if args.only_kernel_table:
         print(json.dumps({"kernels": kernel_table(lm)}))
+        return
+    if args.probe_warm:
+        probe_warm(lm, args.steps, args.warmup)
         return
     _progress("model built; headline decode windows")
     times, dec = bench_decode(lm, args.steps, args.warmup, windows=args.windows)

@@ -313,6 +313,34 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
                           void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
                           int max_cache_len);
 
+/* mui_attn_decode_fused that also announces what the NEXT kernel on the stream will stream:
+ * next_weights / next_weight_bytes (16-byte aligned; NULL / 0: nothing) -- in a decoder layer the
+ * o_proj matrix (csrc/modules/parallel_decoder_module.cpp:22-62 of the reference gives the order).
+ * At short context and small batch the attention launch occupies one workgroup per query head
+ * and is bound by latency: the rest of the chip and the whole memory system idle for its
+ * duration. With this call, extra workgroups of the same launch pull those bytes on chip (L2 of
+ * the XCD whose workgroups will read them, and the memory-side cache) and discard them; results
+ * are those of mui_attn_decode_fused bit for bit. next_slab_bytes (a multiple of 16) is the
+ * contiguous run one consumer workgroup reads at a time (for the GEMVs here: rows per group x
+ * row pitch, see mui_linear_row_group_bytes); slab i is fetched by a workgroup on XCD i mod 8.
+ * Launch shapes that fill the chip themselves (split sequences, larger batches) ignore the hint.
+ * No counterpart in the reference. */
+int mui_attn_decode_fused_warm(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                               const void* k_new, long k_batch_stride, const void* v_new,
+                               long v_batch_stride, const float* cos_table, const float* sin_table,
+                               int rope_row_stride, int rope_rows, const int64_t* position_ids,
+                               long position_batch_stride, const int64_t* cache_position, int seq_len,
+                               void* k_cache, void* v_cache, long cache_batch_stride,
+                               long cache_head_stride, long cache_token_stride, const void* mask,
+                               long mask_batch_stride, void* q_out, void* scratch, int n_splits,
+                               void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                               int max_cache_len, const void* next_weights, size_t next_weight_bytes,
+                               int next_slab_bytes);
+
+/* Bytes of weight matrix that one workgroup of the single-token linear kernels reads per step
+ * (rows per row group x pitch_bytes), for mui_attn_decode_fused_warm; weight_bits 16 or 8. */
+int mui_linear_row_group_bytes(int weight_bits, int k, long pitch_bytes);
+
 /* Causal attention of `tokens` > 1 new query tokens per batch row (prefill, or a chunk of it)
  * over a static cache that already holds their rotated keys and values:
  *   out[b, t, h*D:(h+1)*D] = softmax_{s <= q_start + t}(q[b,h,t,:] . K[b, h/(Hq/Hkv), s, :] / sqrt(D)) V[...]

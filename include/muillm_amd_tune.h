@@ -58,6 +58,12 @@ int mui_tune_prefill(int tile, int wide_max_tokens);
  * K/V block between all query heads of a KV head (0 = built-in choice, negative = never) */
 int mui_tune_prefill_attention(int group_kernel_min_tokens);
 
+/* Cache warming by the idle workgroups of the unsplit decode-attention launch
+ * (mui_attn_decode_fused_warm): workgroups = warm workgroups added to the launch (a multiple of 8;
+ * 0 = built-in choice, negative = off), percent = share of the announced bytes that is fetched
+ * (0 = built-in choice) */
+int mui_tune_warm(int workgroups, int percent);
+
 /* Measurement aid without a counterpart in the reference: reads `bytes` (a multiple of 16, from
  * a 16-byte aligned address) of device memory once with the access shape of the GEMV kernels and
  * discards them. One launch takes the least time any kernel that must read that many bytes can

@@ -76,6 +76,10 @@ _SIGNATURES = {
     "mui_attn_decode_fused": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, c_int, _P,
                                       c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
                                       _P, c_int, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mui_attn_decode_fused_warm": (c_int, [_P, c_int, _P, c_long, _P, c_long, _P, c_long, _P, _P, c_int, c_int, _P,
+                                           c_long, _P, c_int, _P, _P, c_long, c_long, c_long, _P, c_long, _P,
+                                           _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, _P, ctypes.c_size_t, c_int]),
+    "mui_linear_row_group_bytes": (c_int, [c_int, c_int, c_long]),
     "mui_prefill_attention": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, c_int, c_int, _P, c_int, c_int,
                                       c_int, c_int, c_int]),
     "mui_prefill_attention_masked": (c_int, [_P, c_int, _P, _P, _P, c_long, c_long, c_long, c_int, c_int, _P, c_long, _P,
@@ -98,6 +102,7 @@ _SIGNATURES = {
     "mui_tune_skinny": (c_int, [c_int, c_int, c_int]),
     "mui_tune_prefill": (c_int, [c_int, c_int]),
     "mui_tune_prefill_attention": (c_int, [c_int]),
+    "mui_tune_warm": (c_int, [c_int, c_int]),
 }
 
 

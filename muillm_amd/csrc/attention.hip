@@ -68,6 +68,11 @@ struct AttnParams {
   uint16_t* out;          // [B, Hq * D]
   int hq, hkv, n_splits, max_t;
   float scale_log2;       // log2(e) / sqrt(D)
+  // optional: bytes the next kernel will stream (its weights), pulled on chip by extra workgroups
+  // of the unsplit head-parallel launch, which leaves most CUs idle (see warm_cache)
+  const char* warm;
+  long warm_bytes;
+  int warm_slab, warm_wgs;
 };
 
 template <typename T>
@@ -191,6 +196,14 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   __shared__ float lds_l[NW][G];
   __shared__ __attribute__((aligned(16))) float tile[NW][G][kHeadDim];
 
+  if constexpr (DIRECT && G == 1) {
+    // workgroups past the query heads: cache warmers for the next kernel (batch row 0 only)
+    if ((int)blockIdx.y >= p.hq) {
+      if (blockIdx.z == 0)
+        warm_cache(p.warm, p.warm_bytes, p.warm_slab, (int)blockIdx.y - p.hq, p.warm_wgs, threadIdx.x, kAttnThreads);
+      return;
+    }
+  }
   const int split = blockIdx.x, b = blockIdx.z;
   const int head0 = blockIdx.y * G;          // first query head of this workgroup
   const int group = p.hq / p.hkv;            // query heads per KV head (a multiple of G)
@@ -1456,7 +1469,12 @@ template <typename T, int G, bool MFMA_ONLY = false>
 static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
   dim3 grid(p.n_splits, p.hq / G, batch);
   const int nw = attn_waves_for(G);
-  if (MFMA_ONLY || (G == p.hq / p.hkv && g_attn_mfma_tokens >= 0)) {
+  const bool mfma = MFMA_ONLY || (G == p.hq / p.hkv && g_attn_mfma_tokens >= 0);
+  // cache warmers ride along with the unsplit one-workgroup-per-query-head launch of the vector
+  // kernel only (the other shapes fill the chip themselves); they sit behind the head workgroups
+  // in y, and hq % 8 == 0 keeps their XCD the one warm_cache() counts on
+  if (G == 1 && !mfma && p.n_splits == 1 && p.warm && p.warm_wgs > 0 && p.hq % 8 == 0) grid.y += p.warm_wgs;
+  if (mfma) {
     if (p.n_splits == 1)
       hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, true>), grid, dim3(8 * kWave), 0, s, p);
     else
@@ -1658,16 +1676,27 @@ extern "C" int mui_flash_decode_static(mui_stream_t stream, int dtype, const voi
                           n_q_heads, n_kv_heads, head_dim, max_cache_len);
 }
 
-extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
-                                     const void* k_new, long k_batch_stride, const void* v_new,
-                                     long v_batch_stride, const float* cos_table, const float* sin_table,
-                                     int rope_row_stride, int rope_rows, const int64_t* position_ids,
-                                     long position_batch_stride, const int64_t* cache_position,
-                                     int seq_len, void* k_cache, void* v_cache, long cache_batch_stride,
-                                     long cache_head_stride, long cache_token_stride, const void* mask,
-                                     long mask_batch_stride, void* q_out, void* scratch, int n_splits,
-                                     void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
-                                     int max_cache_len) {
+static int g_warm_wgs = 0;      // 0: built-in choice (256); < 0: cache warming off
+static int g_warm_percent = 0;  // 0: built-in choice; share of the announced bytes that is warmed
+
+extern "C" int mui_tune_warm(int workgroups, int percent) {
+  if (percent < 0 || percent > 100 || (workgroups > 0 && workgroups % 8 != 0)) return MUI_ERR_INVALID_ARG;
+  g_warm_wgs = workgroups;
+  g_warm_percent = percent;
+  return MUI_OK;
+}
+
+extern "C" int mui_attn_decode_fused_warm(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                                          const void* k_new, long k_batch_stride, const void* v_new,
+                                          long v_batch_stride, const float* cos_table, const float* sin_table,
+                                          int rope_row_stride, int rope_rows, const int64_t* position_ids,
+                                          long position_batch_stride, const int64_t* cache_position,
+                                          int seq_len, void* k_cache, void* v_cache, long cache_batch_stride,
+                                          long cache_head_stride, long cache_token_stride, const void* mask,
+                                          long mask_batch_stride, void* q_out, void* scratch, int n_splits,
+                                          void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                                          int max_cache_len, const void* next_weights, size_t next_weight_bytes,
+                                          int next_slab_bytes) {
   int st = check_attn_shape(dtype, batch, n_q_heads, n_kv_heads, head_dim, n_splits, max_cache_len);
   if (st != MUI_OK) return st;
   MUI_CHECK_ARG(q && k_new && v_new && k_cache && v_cache && out && cache_position);
@@ -1711,7 +1740,38 @@ extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void*
   p.n_splits = n_splits;
   p.max_t = max_cache_len;
   p.scale_log2 = kLog2e / sqrtf((float)head_dim);
+  if (next_weights && next_weight_bytes >= 16 && g_warm_wgs >= 0) {
+    MUI_CHECK_ARG(aligned16(next_weights) && next_slab_bytes >= 16 && next_slab_bytes % 16 == 0);
+    // the eight L2s hold 32 MB together; the share beyond what fits would only push out its own head
+    const int percent = g_warm_percent > 0 ? g_warm_percent : 100;
+    size_t bytes = next_weight_bytes / 100 * percent;
+    bytes -= bytes % (size_t)next_slab_bytes;
+    if (bytes >= (size_t)next_slab_bytes) {
+      p.warm = (const char*)next_weights;
+      p.warm_bytes = (long)bytes;
+      p.warm_slab = next_slab_bytes;
+      p.warm_wgs = g_warm_wgs > 0 ? g_warm_wgs : 256;
+    }
+  }
   return launch_attn((hipStream_t)stream, dtype, p, batch);
+}
+
+extern "C" int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
+                                     const void* k_new, long k_batch_stride, const void* v_new,
+                                     long v_batch_stride, const float* cos_table, const float* sin_table,
+                                     int rope_row_stride, int rope_rows, const int64_t* position_ids,
+                                     long position_batch_stride, const int64_t* cache_position,
+                                     int seq_len, void* k_cache, void* v_cache, long cache_batch_stride,
+                                     long cache_head_stride, long cache_token_stride, const void* mask,
+                                     long mask_batch_stride, void* q_out, void* scratch, int n_splits,
+                                     void* out, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                                     int max_cache_len) {
+  return mui_attn_decode_fused_warm(stream, dtype, q, q_batch_stride, k_new, k_batch_stride, v_new, v_batch_stride,
+                                    cos_table, sin_table, rope_row_stride, rope_rows, position_ids,
+                                    position_batch_stride, cache_position, seq_len, k_cache, v_cache,
+                                    cache_batch_stride, cache_head_stride, cache_token_stride, mask,
+                                    mask_batch_stride, q_out, scratch, n_splits, out, batch, n_q_heads, n_kv_heads,
+                                    head_dim, max_cache_len, nullptr, 0, 0);
 }
 
 extern "C" int mui_rope_kv_write(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,

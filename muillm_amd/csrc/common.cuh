@@ -191,6 +191,37 @@ __device__ __forceinline__ void row16_reduce_scatter(float (&v)[N], int lane) {
   else v[0] += dpp_f32<kDppXor1>(v[0]);
 }
 
+// Pulls [base, base + bytes) into the cache hierarchy with ordinary (cacheable) 128-bit loads and
+// drops the data: work for workgroups that would otherwise idle while a latency-bound kernel runs,
+// so that the next, bandwidth-bound kernel finds (part of) its weights on chip. The range is cut
+// into slabs of slab_bytes; slab s goes to warm workgroup s % n_wg. Workgroups are handed to the
+// eight XCDs round-robin by linear workgroup id, and each XCD has its own L2: with n_wg a multiple
+// of 8 and the warm workgroups starting at a linear id that is one too, slab s lands in the L2 of
+// XCD s % 8 -- where the consumer's workgroup s % 8 (mod 8) will look for it. Loads are issued
+// eight at a time with clamped addresses (no load behind a branch).
+__device__ __forceinline__ void warm_cache(const char* base, long bytes, int slab_bytes, int wg, int n_wg, int tid,
+                                           int n_threads) {
+  const long n_slabs = (bytes + slab_bytes - 1) / slab_bytes;
+  const long my_slabs = wg < n_slabs ? (n_slabs - wg + n_wg - 1) / n_wg : 0;
+  const int per_slab = (slab_bytes / 16 + n_threads - 1) / n_threads;  // loads per thread and slab
+  const long n_loads = my_slabs * per_slab;
+  constexpr int kBatch = 8;
+  for (long i0 = 0; i0 < n_loads; i0 += kBatch) {
+    u32x4 v[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      long i = i0 + j;
+      i = i < n_loads ? i : 0;
+      const long slab = wg + (i / per_slab) * n_wg;
+      long off = slab * slab_bytes + ((i % per_slab) * (long)n_threads + tid) * 16;
+      off = off + 16 <= bytes ? off : 0;
+      v[j] = ld16(base + off);
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) asm volatile("" ::"v"(v[j]));
+  }
+}
+
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
 
 // host-side helpers ----------------------------------------------------------------------

@@ -82,12 +82,19 @@ extern "C" int mui_decoder_stack_step(mui_stream_t stream, const mui_decoder_sta
                                     m->norm_eps, nullptr, nullptr, w.qkv, qkv_n, m->hidden, batch);
     if (st != MUI_OK) return st;
     const char* q = w.qkv;
-    st = mui_attn_decode_fused(stream, m->dtype, q, qkv_n, q + (size_t)qd * 2, qkv_n,
-                               q + (size_t)(qd + kvd) * 2, qkv_n, m->cos_table, m->sin_table, (int)m->rope_row_stride, (int)m->rope_rows,
-                               position_ids, position_batch_stride, cache_position, seq_len, L.k_cache,
-                               L.v_cache, m->cache_batch_stride, m->cache_head_stride, m->cache_token_stride,
-                               mask, mask_batch_stride, nullptr, w.scratch, n_splits, w.attn, batch,
-                               m->n_q_heads, m->n_kv_heads, m->head_dim, m->max_cache_len);
+    // the attention launch is told what follows it: at short context its idle workgroups fetch the
+    // o_proj matrix on chip while the few busy ones wait on latency
+    const int o_bits = L.o_scales ? 8 : 16;
+    const long o_pitch_bytes = L.o_pitch * (o_bits / 8);
+    const int o_slab = batch == 1 ? mui_linear_row_group_bytes(o_bits, qd, o_pitch_bytes) : 0;
+    const size_t o_bytes = o_slab > 0 ? (size_t)m->hidden * (size_t)o_pitch_bytes : 0;
+    st = mui_attn_decode_fused_warm(stream, m->dtype, q, qkv_n, q + (size_t)qd * 2, qkv_n,
+                                    q + (size_t)(qd + kvd) * 2, qkv_n, m->cos_table, m->sin_table, (int)m->rope_row_stride, (int)m->rope_rows,
+                                    position_ids, position_batch_stride, cache_position, seq_len, L.k_cache,
+                                    L.v_cache, m->cache_batch_stride, m->cache_head_stride, m->cache_token_stride,
+                                    mask, mask_batch_stride, nullptr, w.scratch, n_splits, w.attn, batch,
+                                    m->n_q_heads, m->n_kv_heads, m->head_dim, m->max_cache_len,
+                                    o_bytes ? L.o_weight : nullptr, o_bytes, o_slab);
     if (st != MUI_OK) return st;
     st = !L.o_scales ? mui_linear(stream, m->dtype, L.o_weight, L.o_pitch, w.attn, nullptr, 0.f, nullptr, nullptr, h,
                                   w.h_a, m->hidden, qd, batch)

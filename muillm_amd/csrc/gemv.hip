@@ -303,6 +303,16 @@ extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
 
 extern "C" size_t mui_linear_workspace_bytes(void) { return prefill_workspace_bytes(); }
 
+// rows per row group of the single-token kernels (gemv_multi.hip launch_mt_t, int8_multi.hip
+// launch_i8m_t at one token) times the row pitch
+extern "C" int mui_linear_row_group_bytes(int weight_bits, int k, long pitch_bytes) {
+  if (k <= 0 || pitch_bytes <= 0 || !(weight_bits == 16 || weight_bits == 8)) return 0;
+  const int chunks = weight_bits == 16 ? ceil_div(k >> 3, 256) : ceil_div(k >> 4, 256);
+  const int rows = weight_bits == 16 ? (chunks <= 2 ? 4 : 2) : (chunks <= 1 ? 8 : 2);
+  const long bytes = rows * pitch_bytes;
+  return bytes > (1 << 30) ? 0 : (int)bytes;
+}
+
 extern "C" int mui_linear(mui_stream_t stream, int dtype, const void* weights, long w_pitch,
                           const void* x, const void* norm_weights, float epsilon,
                           const void* mul_bias, const void* add_bias, const void* residual,

@@ -91,7 +91,17 @@ class MuiBaseAttention(MuiModule):
             query_states[:, 0, :], key_states[:, 0, :], value_states[:, 0, :],
             self.rotary_emb.cos32, self.rotary_emb.sin32, position_ids, cache_position,
             cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx],
-            seq_len=seq_len, mask=mask, seq_len_hint=cache.max_cache_len)
+            seq_len=seq_len, mask=mask, seq_len_hint=cache.max_cache_len, next_weights=self._next_weights())
+
+    def _next_weights(self):
+        """The matrix o_proj will stream right after the attention kernel (16-bit weights or int8 codes)."""
+        o = self.o_proj
+        w = getattr(o, "weights_int8", None)
+        if w is None:
+            w = getattr(o, "weights_uint8", None)
+        if w is None:
+            w = getattr(o, "weight", None)
+        return w if isinstance(w, torch.Tensor) else None
 
     def _decode_or_none(self, q, k, v, attention_mask, all_ones_mask, q_len):
         """The two-step decode path (already rotated q, cache views) for T == 1."""

@@ -915,8 +915,14 @@ def muillm_causal_transformer_decoding_masked(q, k, v, m, n_splits=None) -> torc
 
 def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_position, k_cache, v_cache,
                                seq_len: Optional[int] = None, mask=None, n_splits: Optional[int] = None,
-                               seq_len_hint: Optional[int] = None, want_q_out: bool = False):
+                               seq_len_hint: Optional[int] = None, want_q_out: bool = False,
+                               next_weights: Optional[torch.Tensor] = None):
     """RoPE(q, k) + cache write + flash decoding in one call.
+
+    next_weights: the 2-D weight matrix (16-bit, or 8-bit codes) that the next single-token linear on
+    this stream will read (a decoder layer's o_proj): when the launch leaves most of the chip idle
+    -- one token at short context --, its spare workgroups fetch that matrix on chip meanwhile
+    (mui_attn_decode_fused_warm); results do not change.
 
     q [B, Hq*D], k/v [B, Hkv*D]: un-rotated rows of the new token (views into the fused QKV
     output are fine: unit inner stride, any batch stride). cos32/sin32: fp32 tables.
@@ -952,15 +958,23 @@ def mui_attention_decode_fused(q, k, v, cos32, sin32, position_ids, cache_positi
     out = torch.empty((b, 1, hq * d), dtype=q.dtype, device=q.device)
     q_out = torch.empty((b, hq, 1, d), dtype=q.dtype, device=q.device) if want_q_out else None
     bs = lambda tns: tns.stride(0) if b > 1 else tns.shape[1]
+    warm_ptr, warm_bytes, warm_slab = None, 0, 0
+    if (next_weights is not None and b == 1 and next_weights.is_cuda and next_weights.dim() == 2
+            and next_weights.stride(1) == 1 and next_weights.element_size() in (1, 2)
+            and next_weights.data_ptr() % 16 == 0):
+        pitch_bytes = next_weights.stride(0) * next_weights.element_size()
+        warm_slab = lib.mui_linear_row_group_bytes(8 * next_weights.element_size(), next_weights.shape[1], pitch_bytes)
+        if warm_slab > 0 and warm_slab % 16 == 0:
+            warm_ptr, warm_bytes = next_weights.data_ptr(), next_weights.shape[0] * pitch_bytes
     check(
-        lib.mui_attn_decode_fused(
+        lib.mui_attn_decode_fused_warm(
             _stream(q2), _dtype_code(q2), q2.data_ptr(), bs(q2), k2.data_ptr(), bs(k2), v2.data_ptr(), bs(v2),
             _ptr(cos32), _ptr(sin32), cos32.stride(0) if cos32 is not None else 0,
             cos32.shape[0] if cos32 is not None else 0,
             pos.data_ptr(), pos_bs, cache_position.data_ptr(), -1 if seq_len is None else int(seq_len),
             k_cache.data_ptr(), v_cache.data_ptr(), cb, chs, cts, mask_ptr, mask_bs, _ptr(q_out),
-            _ptr(scratch), n_splits, out.data_ptr(), b, hq, hkv, d, max_t),
-        "mui_attn_decode_fused",
+            _ptr(scratch), n_splits, out.data_ptr(), b, hq, hkv, d, max_t, warm_ptr, warm_bytes, warm_slab),
+        "mui_attn_decode_fused_warm",
     )
     return (out, q_out) if want_q_out else out
 

@@ -59,12 +59,18 @@ def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
 # --------------------------------------------------------------------------------------
 # RMSNorm -- muillm/modules/norm/rmsnorm.py:138-146 (HF LlamaRMSNorm form)
 # --------------------------------------------------------------------------------------
-def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, reference_path: bool = False):
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, reference_path: bool = False,
+            round_to: Optional[torch.dtype] = None):
     """y = weight * x * rsqrt(mean(x^2, -1) + eps).
 
     reference_path=True reproduces the fallback literally: fp32 upcast, the normalised
     activations rounded back to the input dtype BEFORE the multiply by weight
-    (rmsnorm.py:140-146)."""
+    (rmsnorm.py:140-146).
+    round_to=dtype: the exact result rounded once to that 16-bit type and returned in float64 --
+    what the reference's RMSNorm kernel stores (one rounding after the multiply by weight,
+    csrc/norm/rmsnorm_fp16_kernels.cu:111-115 and its bf16 twin), which is the operand its matrix
+    multiply then reads whenever the norm and the linear are separate launches (multi-token
+    inputs, csrc/modules/linear_module.cpp:57-79)."""
     if reference_path:
         input_dtype = x.dtype
         h = x.to(torch.float32)
@@ -73,7 +79,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, reference_path: b
         return weight * h.to(input_dtype)
     xh, wh = _hi(x), _hi(weight)
     variance = xh.pow(2).mean(-1, keepdim=True)
-    return wh * (xh * torch.rsqrt(variance + eps))
+    out = wh * (xh * torch.rsqrt(variance + eps))
+    return out.to(round_to).to(_HI) if round_to is not None else out
 
 
 # --------------------------------------------------------------------------------------
@@ -88,8 +95,12 @@ def linear(
     residual: Optional[torch.Tensor] = None,
     mul_bias: Optional[torch.Tensor] = None,
     reference_path: bool = False,
+    norm_round: Optional[torch.dtype] = None,
 ):
     """y = F.linear(rmsnorm(x) if norm_weights else x, weight, bias) (+ residual).
+
+    norm_round=dtype: the normalised activations pass through that 16-bit type on their way into
+    the product (rmsnorm(round_to=dtype)), accumulation still in float64.
 
     `mul_bias` follows the kernel-level form y = (W x) * mul_bias + bias + residual
     (csrc/linear/linear_fp16_kernels.cu:163-356); the Python layer always passes None."""
@@ -104,7 +115,7 @@ def linear(
         if residual is not None:
             out = out + residual
         return out
-    xh = rmsnorm(x, norm_weights, eps) if norm_weights is not None else _hi(x)
+    xh = rmsnorm(x, norm_weights, eps, round_to=norm_round) if norm_weights is not None else _hi(x)
     out = xh @ _hi(weight).T
     if mul_bias is not None:
         out = out * _hi(mul_bias)
@@ -121,12 +132,13 @@ def multilinear(
     norm_weights: Optional[torch.Tensor] = None,
     eps: float = 0.0,
     biases: Optional[Sequence[torch.Tensor]] = None,
+    norm_round: Optional[torch.dtype] = None,
 ) -> Tuple[torch.Tensor, ...]:
     """Fused QKV: one linear over the row-concatenated weights, returned as last-dim slices
     (muillm/modules/multilinear.py:56-66,186-237)."""
     w = torch.cat(list(weights), dim=0)
     b = torch.cat(list(biases), dim=0) if biases is not None else None
-    out = linear(x, w, norm_weights, eps, b)
+    out = linear(x, w, norm_weights, eps, b, norm_round=norm_round)
     outs, start = [], 0
     for wi in weights:
         outs.append(out[..., start : start + wi.shape[0]])
@@ -137,10 +149,10 @@ def multilinear(
 # --------------------------------------------------------------------------------------
 # Gate/Up/Down MLP -- muillm/modules/gateupdownmlp.py:343-359
 # --------------------------------------------------------------------------------------
-def gateup_silu(x, gate_w, up_w, norm_weights=None, eps: float = 0.0):
+def gateup_silu(x, gate_w, up_w, norm_weights=None, eps: float = 0.0, norm_round: Optional[torch.dtype] = None):
     """silu(G xn) * (U xn): the intermediate the fused kernel writes
-    (csrc/ffn/gateup_fp16_kernels.cu:596-601)."""
-    xh = rmsnorm(x, norm_weights, eps) if norm_weights is not None else _hi(x)
+    (csrc/ffn/gateup_fp16_kernels.cu:596-601). norm_round: as in linear()."""
+    xh = rmsnorm(x, norm_weights, eps, round_to=norm_round) if norm_weights is not None else _hi(x)
     g = xh @ _hi(gate_w).T
     u = xh @ _hi(up_w).T
     return F.silu(g) * u
@@ -149,6 +161,7 @@ def gateup_silu(x, gate_w, up_w, norm_weights=None, eps: float = 0.0):
 def gateupdown_mlp(
     x, gate_w, up_w, down_w, norm_weights=None, eps: float = 0.0, residual=None,
     reference_path: bool = False, round_intermediate: Optional[torch.dtype] = None,
+    norm_round: Optional[torch.dtype] = None,
 ):
     """out = down(silu(gate(xn)) * up(xn)) + residual  (_forward_unfused, :343-359).
 
@@ -163,7 +176,7 @@ def gateupdown_mlp(
         if residual is not None:
             out = out + residual
         return out
-    h = gateup_silu(x, gate_w, up_w, norm_weights, eps)
+    h = gateup_silu(x, gate_w, up_w, norm_weights, eps, norm_round=norm_round)
     if round_intermediate is not None:
         h = h.to(round_intermediate).to(_HI)
     out = h @ _hi(down_w).T
@@ -366,17 +379,19 @@ def decoder_layer(
     n_kv_heads: int,
     store_dtype: torch.dtype = torch.float16,
     sliding_window: Optional[int] = None,
+    norm_round: Optional[torch.dtype] = None,
 ):
     """One decoder layer with the rounding points of the fused path: q/k/v, attention
     output, post-attention hidden state and MLP intermediate are stored in `store_dtype`
-    between kernels; everything inside a kernel is float64 here.
+    between kernels; everything inside a kernel is float64 here (norm_round=dtype: except the
+    normalised activations, which pass through that type as in linear()).
     Causal masking is applied for T > 1 (prefill). sliding_window=W hides, from the query in
     cache slot c, the keys at or before c - W (muillm/modules/models/mistral/model.py:590-602)."""
     b, t, hid = h.shape
     d = hid // n_heads
     eps = p["eps"]
     rnd = lambda z: z.to(store_dtype)
-    q, k, v = multilinear(h, [p["wq"], p["wk"], p["wv"]], p["ln1"], eps)
+    q, k, v = multilinear(h, [p["wq"], p["wk"], p["wv"]], p["ln1"], eps, norm_round=norm_round)
     q = rnd(q).view(b, t, n_heads, d).transpose(1, 2)
     k = rnd(k).view(b, t, n_kv_heads, d).transpose(1, 2)
     v = rnd(v).view(b, t, n_kv_heads, d).transpose(1, 2)
@@ -395,7 +410,7 @@ def decoder_layer(
     attn = rnd(decode_attention(qr, kk, vv, mask))
     h1 = rnd(linear(attn, p["wo"], residual=h))
     out = gateupdown_mlp(h1, p["wg"], p["wu"], p["wd"], p["ln2"], eps, residual=h1,
-                         round_intermediate=store_dtype)
+                         round_intermediate=store_dtype, norm_round=norm_round)
     return rnd(out), seen
 
 
@@ -404,7 +419,7 @@ def decoder_layer(
 # --------------------------------------------------------------------------------------
 def decoder_model_step(ids, params, k_caches, v_caches, cos, sin, seen_tokens: int, n_heads: int,
                        n_kv_heads: int, store_dtype: torch.dtype = torch.float16,
-                       sliding_window: Optional[int] = None):
+                       sliding_window: Optional[int] = None, norm_round: Optional[torch.dtype] = None):
     """Embed -> layers -> final RMSNorm -> lm_head for `ids` [B, T] appended after
     `seen_tokens` cached tokens. params: {'embed', 'layers': [layer dicts], 'norm', 'lm_head',
     'eps'}. Returns (logits float64 [B, T, V], new seen_tokens). Hidden states between layers
@@ -416,7 +431,7 @@ def decoder_model_step(ids, params, k_caches, v_caches, cos, sin, seen_tokens: i
     seen = seen_tokens
     for li, lp in enumerate(params["layers"]):
         h, seen = decoder_layer(h, lp, k_caches[li], v_caches[li], cos, sin, pos, cpos, seen_tokens,
-                                n_heads, n_kv_heads, store_dtype, sliding_window)
+                                n_heads, n_kv_heads, store_dtype, sliding_window, norm_round)
     hn = rmsnorm(h, params["norm"], params["eps"]).to(store_dtype)
     return linear(hn, params["lm_head"]), seen
 

@@ -81,12 +81,14 @@ def _build(layers, vocab, dtype, int8, seed, group_size=0):
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16", "int8"])
 def test_full_shape_decoder_layer_vs_oracle(kind):
-    """Gate: logits within 1e-2 (fp16, int8 weights with fp16 activations) of the oracle, max error
-    over max |ref| and elementwise. bf16: 3e-2 on the max form and 5e-2 elementwise -- the bf16
-    kernels feed gamma * x, rounded once to bf16, to the packed dot / matrix-core instructions (the
-    HuggingFace layers round the normalised activations to bf16 as well), the oracle keeps them
-    exact: a 2^-9 relative perturbation of every operand of five chained projections, which over
-    65536 logits puts a handful beyond 3 % of the logits' rms."""
+    """Gate: logits within 1e-2 of the oracle, max error over max |ref| and elementwise, in all
+    three types. The oracle stores what the kernels store between launches in the 16-bit type; for
+    bf16 it also passes the normalised activations gamma * x through bf16 (norm_round), as the
+    reference's RMSNorm kernel does before its matrix product whenever the two are separate
+    launches (csrc/norm/rmsnorm_fp16_kernels.cu:111-115, csrc/modules/linear_module.cpp:57-79) and
+    as the bf16 kernels here do for the packed dot / matrix-core instructions. Against the oracle
+    with exact normalised activations bf16 measures 1.5e-2 of max |ref| (4.5e-2 elementwise): kept
+    as a second, labelled and wider assertion."""
     dtype = torch.bfloat16 if kind == "bf16" else torch.float16
     n_layers = 2
     lm = _build(n_layers, 2048, dtype, kind == "int8", seed=21)
@@ -100,20 +102,24 @@ def test_full_shape_decoder_layer_vs_oracle(kind):
     ids = torch.randint(0, 2048, (1, 32), generator=torch.Generator().manual_seed(3))
     kcs = [torch.zeros(1, HKV, 64, D, dtype=dtype) for _ in range(n_layers)]
     vcs = [torch.zeros(1, HKV, 64, D, dtype=dtype) for _ in range(n_layers)]
-    tol = 3e-2 if kind == "bf16" else 1e-2
-    elem = 5e-2 if kind == "bf16" else None
-    ref, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, HQ, HKV, store_dtype=dtype)
+    nr = dtype if kind == "bf16" else None
+    ref, seen = oracle.decoder_model_step(ids, params, kcs, vcs, cos, sin, 0, HQ, HKV, store_dtype=dtype, norm_round=nr)
     with torch.no_grad():
         out = lm(input_ids=ids.to(DEV))
-    assert_parity(out.logits, ref, tol, f"{kind} full-shape prefill logits", elementwise=elem)
+    assert_parity(out.logits, ref, 1e-2, f"{kind} full-shape prefill logits")
+    if kind == "bf16":  # second, labelled assertion: exact normalised activations in the oracle
+        kx = [torch.zeros_like(t) for t in kcs]
+        vx = [torch.zeros_like(t) for t in vcs]
+        ref_x, _ = oracle.decoder_model_step(ids, params, kx, vx, cos, sin, 0, HQ, HKV, store_dtype=dtype)
+        assert_parity(out.logits, ref_x, 3e-2, "bf16 full-shape prefill logits vs exact operands", elementwise=6e-2)
     cache = out.past_key_values
     nxt = ref[:, -1].argmax(-1)
     for step in range(3):
         ref, seen = oracle.decoder_model_step(nxt.unsqueeze(1), params, kcs, vcs, cos, sin, seen, HQ, HKV,
-                                              store_dtype=dtype)
+                                              store_dtype=dtype, norm_round=nr)
         with torch.no_grad():
             out = lm(input_ids=nxt.unsqueeze(1).to(DEV), past_key_values=cache)
-        assert_parity(out.logits, ref, tol, f"{kind} full-shape decode step {step}", elementwise=elem)
+        assert_parity(out.logits, ref, 1e-2, f"{kind} full-shape decode step {step}")
         nxt = ref[:, -1].argmax(-1)
     # the first layer's cache rows equal the oracle's within one 16-bit ulp of rounding flips
     kd = cache.key_cache[0][:, :, :seen].float().cpu()

@@ -61,9 +61,10 @@ def test_linear_single_token(n, k, norm, res, bias, dtype):
         None, x.to(DEV), w.to(DEV), None if gamma is None else gamma.to(DEV), eps,
         None, None if b is None else b.to(DEV), None if r is None else r.to(DEV))
     assert y.shape == (1, n) and y.dtype == dtype
-    rel = 1e-2
+    # one gate for both 16-bit types (measured on MI355X: bf16 worst 3.9e-3 of max |ref|, 4.8e-3 on
+    # the elementwise form); `tight` is a sanity bound in units of rms(ref), wider for bf16's 8 bits
     tight = 4e-3 if dtype == torch.float16 else 3e-2
-    assert_parity(y, ref, rel if dtype == torch.float16 else 2e-2, f"linear {n}x{k}", tight=tight)
+    assert_parity(y, ref, 1e-2, f"linear {n}x{k}", tight=tight)
 
 
 def test_linear_config1_reference_tolerance():
@@ -167,7 +168,7 @@ def test_linear_small_batch_edge_shapes(tokens, n, k, norm, dtype):
     y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), None if gamma is None else gamma.to(DEV),
                                          1e-5, mul_bias=mb.to(DEV), add_bias=ab.to(DEV), residual=r.to(DEV))
     assert y.shape == (tokens, n) and y.dtype == dtype
-    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 3e-2, f"edge {tokens} {n}x{k} norm={norm} {dtype}")
+    assert_parity(y, ref, 1e-2, f"edge {tokens} {n}x{k} norm={norm} {dtype}")
 
 
 @pytest.mark.parametrize("tokens", [5, 16])
@@ -213,7 +214,7 @@ def test_linear_rows_longer_than_one_pass(tokens, k, dtype):
     y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), mul_bias=mb.to(DEV), add_bias=ab.to(DEV),
                                          residual=r.to(DEV))
     assert y.shape == (tokens, n) and y.dtype == dtype
-    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 3e-2, f"long rows {tokens} x {k} {dtype}")
+    assert_parity(y, ref, 1e-2, f"long rows {tokens} x {k} {dtype}")
 
 
 def test_linear_reference_recipe_batch4():

@@ -237,6 +237,59 @@ def test_int8_linear_compositions_brute_force():
     assert torch.allclose(a, b, atol=1e-12, rtol=0)
 
 
+def test_rounded_normalised_activations_mode():
+    """rmsnorm(round_to=dtype) / norm_round: the exact gamma * x_hat rounded ONCE to the 16-bit type
+    (what the reference's RMSNorm kernel stores, csrc/norm/rmsnorm_fp16_kernels.cu:111-115) -- closed
+    forms that tell one rounding from none and from the fallback's two (rmsnorm.py:140-146)."""
+    bf = torch.bfloat16
+    x = torch.ones(1, 4)
+    # x_hat = 1 (eps = 0): the result is gamma itself, rounded to bf16 (8 significant bits, ties to even)
+    gam = torch.tensor([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8, 1 + 2.0 ** -7, 0.7])
+    y = oracle.rmsnorm(x, gam, 0.0, round_to=bf)
+    assert y.dtype == torch.float64
+    assert y[0].tolist() == [1.0, 1 + 2.0 ** -6, 1 + 2.0 ** -7, float(torch.tensor(0.7).to(bf))]
+    assert oracle.rmsnorm(x, gam, 0.0)[0, 0].item() == 1 + 2.0 ** -8        # un-rounded mode untouched
+    # one rounding, not the fallback's two
+    g = torch.Generator().manual_seed(3)
+    xr = torch.randn(64, 512, generator=g).to(bf)
+    gr = (1 + 0.1 * torch.randn(512, generator=g)).to(bf)
+    once = oracle.rmsnorm(xr, gr, 1e-5, round_to=bf)
+    exact = oracle.rmsnorm(xr, gr, 1e-5)
+    twice = oracle.rmsnorm(xr, gr, 1e-5, reference_path=True).double()
+    assert torch.equal(once, exact.to(bf).double())
+    assert float((once - exact).abs().max()) <= float(exact.abs().max()) * 2.0 ** -8
+    assert not torch.equal(once, twice)
+    assert float((twice - exact).abs().mean()) > float((once - exact).abs().mean())  # two roundings lose more
+    # linear / gateup_silu / gateupdown_mlp with norm_round == the same functions fed the rounded activations
+    w, wu, wd = torch.randn(24, 512, generator=g) * 0.05, torch.randn(24, 512, generator=g) * 0.05, torch.randn(512, 24, generator=g) * 0.05
+    assert torch.equal(oracle.linear(xr, w, gr, 1e-5, norm_round=bf), oracle.linear(once, w))
+    assert torch.equal(oracle.gateup_silu(xr, w, wu, gr, 1e-5, norm_round=bf), oracle.gateup_silu(once, w, wu))
+    assert torch.equal(oracle.gateupdown_mlp(xr, w, wu, wd, gr, 1e-5, norm_round=bf), oracle.gateupdown_mlp(once, w, wu, wd))
+    q, k, v = oracle.multilinear(xr, [w[:8], w[8:16], w[16:]], gr, 1e-5, norm_round=bf)
+    assert torch.equal(torch.cat([q, k, v], -1), oracle.linear(once, w))
+
+
+def test_bf16_gateup_elementwise_error_is_set_by_the_8_bit_operands():
+    """Why the bf16 gate/up tests carry a second, wider elementwise assertion against the oracle
+    with exact normalised activations: with gamma * x rounded to bf16 (once, as the RMSNorm kernel of
+    the reference does; or twice, as its Python fallback does, rmsnorm.py:140-146) and everything
+    else exact, single elements of silu(G x) * (U x) already sit more than 1e-2 * (|ref| + rms) away,
+    while the error over max |ref| stays far below 1e-2."""
+    g = torch.Generator().manual_seed(0)
+    bf = torch.bfloat16
+    x = torch.randn(16, 4096, generator=g).to(bf)
+    gam = (1 + 0.1 * torch.randn(4096, generator=g)).to(bf)
+    wg = (0.02 * torch.randn(2048, 4096, generator=g)).to(bf)
+    wu = (0.02 * torch.randn(2048, 4096, generator=g)).to(bf)
+    exact = oracle.gateup_silu(x, wg, wu, gam, 1e-5)
+    rms = exact.pow(2).mean().sqrt()
+    for rounded in (oracle.gateup_silu(x, wg, wu, gam, 1e-5, norm_round=bf),
+                    oracle.gateup_silu(oracle.rmsnorm(x, gam, 1e-5, reference_path=True), wg, wu)):
+        err = (rounded - exact).abs()
+        assert float(err.max() / exact.abs().max()) < 5e-3
+        assert 1e-2 < float((err / (exact.abs() + rms)).max()) < 4e-2
+
+
 def test_rope_properties_and_brute_force():
     d = 8
     cos, sin = oracle.rope_tables(10000.0, d, 64)

@@ -94,7 +94,7 @@ def test_linear_prompt_mul_bias_and_bf16(tokens, dtype):
     ref = (oracle.linear(x, w, gamma, 1e-5).double() * mb.double() + ab.double() + r.double())
     y = muillm_ext.muillm_linear_forward(None, x.to(DEV), w.to(DEV), gamma.to(DEV), 1e-5, mb.to(DEV), ab.to(DEV), r.to(DEV))
     assert y.shape == (2, tokens, n) and y.dtype == dtype
-    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 2e-2, f"prompt linear mul_bias {dtype}")
+    assert_parity(y, ref, 1e-2, f"prompt linear mul_bias {dtype}")
 
 
 @pytest.mark.parametrize("tokens", [33, 64, 128, 512])
@@ -109,10 +109,19 @@ def test_gateup_prompt(tokens, n, k, dtype):
     ref = oracle.gateup_silu(x, wg, wu, gamma, 1e-5)
     packed = torch.stack([wg, wu], dim=1).contiguous().to(DEV)   # the module's interleaved [N, 2, K] buffer
     h = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, packed[:, 0], packed[:, 1], x.to(DEV))
-    # bf16: gamma * x is rounded to 8 significant bits before the matrix cores see it, and SiLU * mul
-    # multiplies two such results: 2.5e-2 on the max form, 4e-2 on the elementwise form
-    assert_parity(h, ref, 1e-2 if dtype == torch.float16 else 2.5e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype}",
-                  elementwise=None if dtype == torch.float16 else 4e-2)
+    if dtype == torch.float16:
+        assert_parity(h, ref, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype}")
+    else:
+        # bf16. The gate, at 1e-2 in both forms: against the normalised activations as the reference's
+        # own route for several tokens hands them to its GEMM -- its RMSNorm kernel rounds gamma * x
+        # once to bf16 (csrc/norm/rmsnorm_fp16_kernels.cu:111-115 and the bf16 twin), the matrix
+        # product reads that (csrc/modules/linear_module.cpp:57-79) --, accumulated in float64.
+        ref_r = oracle.gateup_silu(x, wg, wu, gamma, 1e-5, norm_round=dtype)
+        assert_parity(h, ref_r, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype} vs rounded operand")
+        # Second, labelled assertion against the un-rounded oracle: 1e-2 of max |ref| holds there too;
+        # element by element, 8-bit operands under SiLU * mul leave single values up to 3.3e-2 of
+        # |ref| + rms(ref) away (the reference's fallback, which rounds twice, sits at the same level)
+        assert_parity(h, ref, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype} vs exact operand", elementwise=4e-2)
     h2 = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, wg.to(DEV), wu.to(DEV), x.to(DEV))  # two dense matrices
     assert torch.equal(h, h2)
 
@@ -150,7 +159,7 @@ def test_int8_channel_linear_prompt(tokens, n, k, dtype):
     wexact = q.double() * s.double()[:, None]
     ref = oracle.linear(x, wexact, gamma, 1e-5, None, r)
     y = muillm_ext.mui_int8_channel_linear_forward(x.to(DEV), q.to(DEV), s.to(DEV), gamma.to(DEV), 1e-5, None, r.to(DEV))
-    assert_parity(y, ref, 1e-2 if dtype == torch.float16 else 2e-2, f"int8 prompt linear {tokens}x{n}x{k} {dtype}")
+    assert_parity(y, ref, 1e-2, f"int8 prompt linear {tokens}x{n}x{k} {dtype}")
 
 
 @pytest.mark.parametrize("tokens", [65, 200])
