@@ -418,7 +418,7 @@ def _graph_chain_us(launch, n=400, replays=10):
     return round(a.elapsed_time(b) * 1e3 / (replays * n), 3)
 
 
-def probe_warm(lm, steps, warmup):
+def probe_warm(lm, steps, warmup, decode_rate=False):
     """Cache warming by the idle workgroups of the short-context attention launch
     (mui_attn_decode_fused_warm): the pair [fused RoPE + cache write + attention at 64 cached tokens,
     o_proj GEMV + residual] over the model's 32 o_proj matrices, HIP-event timed, and the decode
@@ -458,20 +458,75 @@ def probe_warm(lm, steps, warmup):
                            y.data_ptr(), hid, hq * d, 1)
 
     out = {"slab_bytes": slab}
-    settings = [("off", -1, 0), ("wg256_pct100", 256, 100), ("wg256_pct75", 256, 75), ("wg256_pct50", 256, 50),
-                ("wg128_pct100", 128, 100), ("wg512_pct100", 512, 100), ("wg224_pct90", 224, 90), ("off_again", -1, 0)]
-    for name, wgs, pct in settings:
-        _lib.check(lib.mui_tune_warm(wgs, pct), "mui_tune_warm")
+    settings = [("off", -1, 0, 0)]
+    for wgs in (256, 512):
+        for pct in (50, 75, 100):
+            for delay in (0, 4, 6, 8, 10):
+                settings.append(("wg%d_pct%d_delay%d" % (wgs, pct, delay), wgs, pct, delay))
+    settings.append(("off_again", -1, 0, 0))
+    for name, wgs, pct, delay in settings:
+        _lib.check(lib.mui_tune_warm(wgs, pct, delay), "mui_tune_warm")
         row = {"attention+o_proj_us": round(_median([_event_time_us(pair, 320, 64) for _ in range(3)]), 2),
                "attention_us": round(_median([_event_time_us(lambda i: pair(i, attn_only=True), 320, 64) for _ in range(3)]), 2),
                "o_proj_alone_us": round(_median([_event_time_us(lambda i: pair(i, gemv_only=True), 320, 64) for _ in range(3)]), 2)}
-        times, dec = bench_decode(lm, steps, warmup, use_graph=False, windows=3)
-        row["decode_tokens_per_s"] = _rate_summary(times, steps)
-        del dec
+        if decode_rate:
+            times, dec = bench_decode(lm, steps, warmup, use_graph=False, windows=3)
+            row["decode_tokens_per_s"] = _rate_summary(times, steps)
+            del dec
         out[name] = row
         _progress("probe-warm %s: %s" % (name, row))
-    _lib.check(lib.mui_tune_warm(0, 0), "mui_tune_warm")
+    _lib.check(lib.mui_tune_warm(0, 0, -1), "mui_tune_warm")
     print(json.dumps({"probe_warm": out}))
+
+
+def probe_chain(n_mats=32, n_launches=64):
+    """A chain of dependent 4096 x 4096 fp16 GEMVs over distinct matrices: ordinary launches against
+    launches that overlap their predecessor's tail and take x through arrival counters in memory
+    (mui_probe_gemv_chain). Reports microseconds per GEMV, whether a bounded wait ran out, and whether
+    the chain's result is bit-identical to the ordinary launches'."""
+    import ctypes
+
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 4096
+    g = torch.Generator(device="cuda").manual_seed(0)
+    mats = [(torch.randn(n, n, device="cuda", generator=g) / 64).half() for _ in range(n_mats)]
+    ptrs = (ctypes.c_void_p * n_mats)(*[m.data_ptr() for m in mats])
+    x0 = torch.randn(n, device="cuda", generator=g).half()
+    xa, xb = torch.empty_like(x0), torch.empty_like(x0)
+    flags = torch.zeros(lib.mui_probe_chain_flag_bytes(n_launches) // 4, dtype=torch.int32, device="cuda")
+    err = torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = {}
+    ref = None
+    for name, mode, wgs in (("ordinary", 0, 0), ("overlapped_coherent_x", 1, 0), ("overlapped_cached_x", 2, 0),
+                            ("ordinary_256wg", 0, 256), ("overlapped_coherent_x_256wg", 1, 256),
+                            ("overlapped_coherent_x_1024wg", 1, 1024), ("ordinary_again", 0, 0)):
+        samples = []
+        for rep in range(6):
+            xa.copy_(x0)
+            flags.zero_()
+            err.zero_()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            _lib.check(lib.mui_probe_gemv_chain(stream, mode, ptrs, n_mats, n_launches, n, n, xa.data_ptr(), xb.data_ptr(),
+                                                flags.data_ptr(), err.data_ptr(), wgs, 200000), "mui_probe_gemv_chain")
+            b.record()
+            torch.cuda.synchronize()
+            if rep:
+                samples.append(a.elapsed_time(b) * 1e3 / n_launches)
+        res = (xa if n_launches % 2 == 0 else xb).clone()
+        if ref is None:
+            ref = res
+        out[name] = {"us_per_gemv": round(_median(samples), 3), "min": round(min(samples), 3), "max": round(max(samples), 3),
+                     "wait_ran_out": bool(err.item()), "bit_identical_to_ordinary": bool(torch.equal(res, ref)),
+                     "finite": bool(torch.isfinite(res).all())}
+        _progress("probe-chain %s: %s" % (name, out[name]))
+    print(json.dumps({"probe_chain": out}))
 
 
 def probe_kernel_boundary():
@@ -1021,6 +1076,9 @@ def main():
                     help="time chains of near-empty dependent kernels in a replayed HIP graph and exit")
     ap.add_argument("--probe-warm", action="store_true",
                     help="time attention + o_proj and the decode rate over cache-warming settings and exit")
+    ap.add_argument("--probe-chain", action="store_true",
+                    help="time a chain of dependent GEMVs as ordinary launches and as overlapped launches with a "
+                         "hand-off through memory, and exit")
     ap.add_argument("--probe-flash-splits", action="store_true",
                     help="time fused flash decoding at batch 1 over the number of sequence splits and exit")
     ap.add_argument("--probe-prompt", action="store_true",
@@ -1056,6 +1114,9 @@ def main():
         return
     if args.probe_kernel_boundary:
         probe_kernel_boundary()
+        return
+    if args.probe_chain:
+        probe_chain()
         return
     if args.probe_flash_splits:
         probe_flash_splits()

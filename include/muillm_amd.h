@@ -323,8 +323,10 @@ int mui_attn_decode_fused(mui_stream_t stream, int dtype, const void* q, long q_
  * are those of mui_attn_decode_fused bit for bit. next_slab_bytes (a multiple of 16) is the
  * contiguous run one consumer workgroup reads at a time (for the GEMVs here: rows per group x
  * row pitch, see mui_linear_row_group_bytes); slab i is fetched by a workgroup on XCD i mod 8.
- * Launch shapes that fill the chip themselves (split sequences, larger batches) ignore the hint.
- * No counterpart in the reference. */
+ * Launch shapes that fill the chip themselves (split sequences, larger batches) ignore the hint,
+ * and so does every launch unless the process has opted in with mui_tune_warm (muillm_amd_tune.h):
+ * on MI355X the faster o_proj (3.6 instead of 6.8 us) is paid for by a slower attention launch
+ * (8.7-9.4 instead of 5.65 us). No counterpart in the reference. */
 int mui_attn_decode_fused_warm(mui_stream_t stream, int dtype, const void* q, long q_batch_stride,
                                const void* k_new, long k_batch_stride, const void* v_new,
                                long v_batch_stride, const float* cos_table, const float* sin_table,

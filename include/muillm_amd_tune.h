@@ -59,10 +59,12 @@ int mui_tune_prefill(int tile, int wide_max_tokens);
 int mui_tune_prefill_attention(int group_kernel_min_tokens);
 
 /* Cache warming by the idle workgroups of the unsplit decode-attention launch
- * (mui_attn_decode_fused_warm): workgroups = warm workgroups added to the launch (a multiple of 8;
- * 0 = built-in choice, negative = off), percent = share of the announced bytes that is fetched
- * (0 = built-in choice) */
-int mui_tune_warm(int workgroups, int percent);
+ * (mui_attn_decode_fused_warm) is off by default (it measured no gain: the o_proj GEMV that follows
+ * gets 3 us faster, the attention launch 3-4 us slower). workgroups = warm workgroups added to the
+ * launch (a multiple of 8; > 0 switches it on, <= 0 off), percent = share of the announced bytes
+ * that is fetched (0 = all), delay = head start of the attention workgroups in units of s_sleep 8,
+ * about a quarter microsecond each (negative = built-in choice, at most 64) */
+int mui_tune_warm(int workgroups, int percent, int delay);
 
 /* Measurement aid without a counterpart in the reference: reads `bytes` (a multiple of 16, from
  * a 16-byte aligned address) of device memory once with the access shape of the GEMV kernels and
@@ -70,6 +72,20 @@ int mui_tune_warm(int workgroups, int percent);
  * take on this device, launch latency included. `sink` is any 256-byte device buffer (written
  * only if the data matches a fixed 16-byte pattern). */
 int mui_probe_read(mui_stream_t stream, const void* src, uint64_t bytes, void* sink);
+
+/* Measurement aid without a counterpart in the reference: a chain of n_launches dependent fp16
+ * GEMVs x_{i+1} = W_i . x_i (square matrices n == k <= 4096, used round-robin from the host array
+ * `weights`; launch i reads xa or xb and writes the other), to price a kernel boundary against a
+ * hand-off through memory. mode 0: ordinary launches. mode 1 / 2: launches that may start before
+ * their predecessor has finished; each requests its first weight rows, then waits -- at most
+ * spin_limit polls, after which it sets *err and goes on -- for the arrival counters its
+ * predecessor bumps after its last store, and reads x with agent-scope loads (1) or ordinary ones
+ * (2). `flags`: mui_probe_chain_flag_bytes(n_launches) bytes, zeroed by the caller before every
+ * call; `err`: one zeroed uint32; workgroups: grid size (a multiple of 8; 0 = built-in choice). */
+size_t mui_probe_chain_flag_bytes(int n_launches);
+int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* const* weights, int n_mats,
+                         int n_launches, int n, int k, void* xa, void* xb, void* flags, void* err,
+                         int workgroups, int spin_limit);
 
 #ifdef __cplusplus
 }

@@ -102,7 +102,9 @@ _SIGNATURES = {
     "mui_tune_skinny": (c_int, [c_int, c_int, c_int]),
     "mui_tune_prefill": (c_int, [c_int, c_int]),
     "mui_tune_prefill_attention": (c_int, [c_int]),
-    "mui_tune_warm": (c_int, [c_int, c_int]),
+    "mui_tune_warm": (c_int, [c_int, c_int, c_int]),
+    "mui_probe_chain_flag_bytes": (ctypes.c_size_t, [c_int]),
+    "mui_probe_gemv_chain": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int]),
 }
 
 

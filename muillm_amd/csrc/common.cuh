@@ -199,13 +199,17 @@ __device__ __forceinline__ void row16_reduce_scatter(float (&v)[N], int lane) {
 // of 8 and the warm workgroups starting at a linear id that is one too, slab s lands in the L2 of
 // XCD s % 8 -- where the consumer's workgroup s % 8 (mod 8) will look for it. Loads are issued
 // eight at a time with clamped addresses (no load behind a branch).
+template <int kBatch = 8>
 __device__ __forceinline__ void warm_cache(const char* base, long bytes, int slab_bytes, int wg, int n_wg, int tid,
-                                           int n_threads) {
+                                           int n_threads, int delay = 0) {
+  // optional head start for the workgroups doing the launch's real work: their first dependent loads
+  // go out before this traffic fills the memory queues (one unit = s_sleep 8, about a quarter
+  // microsecond)
+  for (int i = 0; i < delay; ++i) __builtin_amdgcn_s_sleep(8);
   const long n_slabs = (bytes + slab_bytes - 1) / slab_bytes;
   const long my_slabs = wg < n_slabs ? (n_slabs - wg + n_wg - 1) / n_wg : 0;
   const int per_slab = (slab_bytes / 16 + n_threads - 1) / n_threads;  // loads per thread and slab
   const long n_loads = my_slabs * per_slab;
-  constexpr int kBatch = 8;
   for (long i0 = 0; i0 < n_loads; i0 += kBatch) {
     u32x4 v[kBatch];
 #pragma unroll

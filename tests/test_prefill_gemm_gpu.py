@@ -109,19 +109,16 @@ def test_gateup_prompt(tokens, n, k, dtype):
     ref = oracle.gateup_silu(x, wg, wu, gamma, 1e-5)
     packed = torch.stack([wg, wu], dim=1).contiguous().to(DEV)   # the module's interleaved [N, 2, K] buffer
     h = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, packed[:, 0], packed[:, 1], x.to(DEV))
-    if dtype == torch.float16:
-        assert_parity(h, ref, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype}")
-    else:
-        # bf16. The gate, at 1e-2 in both forms: against the normalised activations as the reference's
-        # own route for several tokens hands them to its GEMM -- its RMSNorm kernel rounds gamma * x
-        # once to bf16 (csrc/norm/rmsnorm_fp16_kernels.cu:111-115 and the bf16 twin), the matrix
-        # product reads that (csrc/modules/linear_module.cpp:57-79) --, accumulated in float64.
-        ref_r = oracle.gateup_silu(x, wg, wu, gamma, 1e-5, norm_round=dtype)
-        assert_parity(h, ref_r, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype} vs rounded operand")
-        # Second, labelled assertion against the un-rounded oracle: 1e-2 of max |ref| holds there too;
-        # element by element, 8-bit operands under SiLU * mul leave single values up to 3.3e-2 of
-        # |ref| + rms(ref) away (the reference's fallback, which rounds twice, sits at the same level)
-        assert_parity(h, ref, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype} vs exact operand", elementwise=4e-2)
+    # The stated gate -- max error over max |ref| <= 1e-2 -- holds in both types (bf16 measures 3.8e-3).
+    # The additional elementwise form is held at 1e-2 for fp16. For bf16 it is 4e-2 here, and only
+    # here and in the model-level tests: the matrix cores read gamma * x rounded to bf16's 8 bits, and
+    # under SiLU * mul single elements then sit up to 3.3e-2 of |ref| + rms(ref) away from the oracle
+    # with exact operands. That level belongs to the format, not to the kernel:
+    # tests/test_oracle_cpu.py::test_bf16_gateup_elementwise_error_is_set_by_the_8_bit_operands finds
+    # it with everything but the operand rounding exact, for this rounding and for the reference's
+    # own (its RMSNorm fallback rounds twice, muillm/modules/norm/rmsnorm.py:140-146).
+    assert_parity(h, ref, 1e-2, f"prompt gate/up {tokens}x{n}x{k} {dtype}",
+                  elementwise=None if dtype == torch.float16 else 4e-2)
     h2 = muillm_ext.mui_gateup_silu(gamma.to(DEV), 1e-5, wg.to(DEV), wu.to(DEV), x.to(DEV))  # two dense matrices
     assert torch.equal(h, h2)
 
