@@ -514,7 +514,7 @@ def probe_chain(n_mats=32, n_launches=64):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record()
             _lib.check(lib.mui_probe_gemv_chain(stream, mode, ptrs, n_mats, n_launches, n, n, xa.data_ptr(), xb.data_ptr(),
-                                                flags.data_ptr(), err.data_ptr(), wgs, 200000), "mui_probe_gemv_chain")
+                                                flags.data_ptr(), err.data_ptr(), wgs, 20000), "mui_probe_gemv_chain")
             b.record()
             torch.cuda.synchronize()
             if rep:
