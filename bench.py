@@ -504,7 +504,10 @@ def probe_chain(n_mats=32, n_launches=64):
     ref = None
     for name, mode, wgs in (("ordinary", 0, 0), ("overlapped_coherent_x", 1, 0), ("overlapped_cached_x", 2, 0),
                             ("ordinary_256wg", 0, 256), ("overlapped_coherent_x_256wg", 1, 256),
-                            ("overlapped_coherent_x_1024wg", 1, 1024), ("ordinary_again", 0, 0)):
+                            ("overlapped_coherent_x_1024wg", 1, 1024),
+                            ("overlapped_poll_wave", 3, 0), ("overlapped_poll_wave_all_weights_first", 4, 0),
+                            ("overlapped_poll_wave_256wg", 3, 256), ("overlapped_poll_wave_all_weights_first_256wg", 4, 256),
+                            ("ordinary_again", 0, 0)):
         samples = []
         for rep in range(6):
             xa.copy_(x0)

@@ -134,6 +134,120 @@ __global__ void __launch_bounds__(kChainThreads) chain_gemv_kernel(
   }
 }
 
+// Second form of the hand-off: a fifth wave does nothing but poll the counters and then fetch x into
+// LDS (its loads do not queue behind weight loads: loads return in order within a wave), and the four
+// weight waves request PF row groups -- for a 4096 x 4096 matrix on 512 workgroups: everything they
+// will ever read -- before they wait for it. n_groups must be a multiple of gridDim.x * PF... not
+// required: row groups past the end are clamped and dropped.
+template <int PF>
+__global__ void __launch_bounds__(kChainThreads + kWave) chain_gemv_pollwave_kernel(
+    const uint16_t* w, const uint16_t* x, uint16_t* y, int n, int k, const uint32_t* flag_in,
+    uint32_t expected, uint32_t* flag_out, uint32_t* err, int spin_limit) {
+  __shared__ float red[2][kChainThreads / kWave][kChainR];
+  __shared__ __attribute__((aligned(16))) uint16_t xs[kChainCH * kChainThreads * 8];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int kc = k >> 3;
+  const int n_groups = n / kChainR;
+  const bool poller = wave == kChainThreads / kWave;
+  int coff[kChainCH];
+#pragma unroll
+  for (int j = 0; j < kChainCH; ++j) {
+    const int c = (t & (kChainThreads - 1)) + kChainThreads * j;
+    coff[j] = c < kc ? (c << 3) : 0;
+  }
+  u32x4 wr[PF][kChainR][kChainCH];
+  auto issue = [&](int slot, int rg) {
+    const int g = rg < n_groups ? rg : n_groups - 1;
+#pragma unroll
+    for (int r = 0; r < kChainR; ++r) {
+      const uint16_t* rp = w + (long)(g * kChainR + r) * k;
+#pragma unroll
+      for (int j = 0; j < kChainCH; ++j) wr[slot][r][j] = ld16_stream(rp + coff[j]);
+    }
+  };
+  if (!poller) {
+#pragma unroll
+    for (int f = 0; f < PF; ++f) issue(f, blockIdx.x + f * gridDim.x);
+  } else {
+    if (flag_in != nullptr && lane < kChainCounters) {
+      int spins = 0;
+      while ((int)(__hip_atomic_load(flag_in + lane * kChainCounterStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
+                   expected) < 0) {
+        __builtin_amdgcn_s_sleep(1);
+        if (++spins > spin_limit) {
+          __hip_atomic_fetch_or(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+      }
+    }
+    // (the wave reconverges here: the loads below follow every lane's last poll)
+    for (int c = lane; c < kc; c += kWave) {
+      const uint64_t* xp = (const uint64_t*)(x + (c << 3));
+      const uint64_t lo = __hip_atomic_load(xp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint64_t hi = __hip_atomic_load(xp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *(uint64_t*)&xs[(c << 3)] = lo;
+      *(uint64_t*)&xs[(c << 3) + 4] = hi;
+    }
+  }
+  __syncthreads();
+  u32x4 xq[kChainCH];
+#pragma unroll
+  for (int j = 0; j < kChainCH; ++j) {
+    const int c = (t & (kChainThreads - 1)) + kChainThreads * j;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    xq[j] = c < kc ? *(const u32x4*)&xs[c << 3] : zero;
+  }
+
+  int buf = 0;
+  int rg = blockIdx.x;
+  for (int it = 0; rg < n_groups; rg += gridDim.x, ++it) {
+    float acc[kChainR];
+    if (!poller) {
+      const int slot = it % PF;
+#pragma unroll
+      for (int r = 0; r < kChainR; ++r) {
+        float a = 0.f;
+#pragma unroll
+        for (int f = 0; f < PF; ++f) {
+          if (f == slot) {
+#pragma unroll
+            for (int j = 0; j < kChainCH; ++j) {
+              a = chain_dot2(wr[f][r][j].x, xq[j].x, a);
+              a = chain_dot2(wr[f][r][j].y, xq[j].y, a);
+              a = chain_dot2(wr[f][r][j].z, xq[j].z, a);
+              a = chain_dot2(wr[f][r][j].w, xq[j].w, a);
+            }
+          }
+        }
+        acc[r] = a;
+      }
+      const int nxt = rg + PF * gridDim.x;
+      if (nxt < n_groups) {
+#pragma unroll
+        for (int f = 0; f < PF; ++f)
+          if (f == slot) issue(f, nxt);
+      }
+#pragma unroll
+      for (int r = 0; r < kChainR; ++r) acc[r] = wave_sum(acc[r]);
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < kChainR; ++r) red[buf][wave][r] = acc[r];
+      }
+    }
+    __syncthreads();
+    if (t < kChainR) {
+      const float v = (red[buf][0][t] + red[buf][1][t]) + (red[buf][2][t] + red[buf][3][t]);
+      __hip_atomic_store(y + rg * kChainR + t, F16::pack(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    buf ^= 1;
+  }
+  if (t < kChainR) __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (t == 0)
+    __hip_atomic_fetch_add(flag_out + (blockIdx.x % kChainCounters) * kChainCounterStride, 1u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+
 }  // namespace mui
 
 using namespace mui;
@@ -150,7 +264,7 @@ extern "C" int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* c
                                     int workgroups, int spin_limit) {
   MUI_CHECK_ARG(weights && n_mats > 0 && n_launches > 0 && xa && xb && err);
   MUI_CHECK_ARG(n == k && k > 0 && k <= kChainCH * kChainThreads * 8 && (k & 7) == 0 && (n % kChainR) == 0);
-  MUI_CHECK_ARG(mode == 0 || ((mode == 1 || mode == 2) && flags));
+  MUI_CHECK_ARG(mode == 0 || ((mode >= 1 && mode <= 4) && flags));
   MUI_CHECK_ARG(spin_limit > 0 && spin_limit <= (1 << 22));
   const int n_groups = n / kChainR;
   int grid = workgroups > 0 ? workgroups : balanced_grid(n_groups, 3);
@@ -170,7 +284,15 @@ extern "C" int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* c
       const uint32_t* fin = i == 0 ? nullptr : fl + (size_t)(i - 1) * kChainCounters * kChainCounterStride;
       uint32_t* fout = fl + (size_t)i * kChainCounters * kChainCounterStride;
       const uint32_t expected = (uint32_t)(grid / kChainCounters);
-      if (mode == 1)
+      if (mode == 3)
+        hipExtLaunchKernelGGL((chain_gemv_pollwave_kernel<1>), dim3(grid), dim3(kChainThreads + kWave), 0, s, nullptr,
+                              nullptr, hipExtAnyOrderLaunch, w, x, y, n, k, fin, expected, fout, (uint32_t*)err,
+                              spin_limit);
+      else if (mode == 4)
+        hipExtLaunchKernelGGL((chain_gemv_pollwave_kernel<2>), dim3(grid), dim3(kChainThreads + kWave), 0, s, nullptr,
+                              nullptr, hipExtAnyOrderLaunch, w, x, y, n, k, fin, expected, fout, (uint32_t*)err,
+                              spin_limit);
+      else if (mode == 1)
         hipExtLaunchKernelGGL((chain_gemv_kernel<true, true>), dim3(grid), dim3(kChainThreads), 0, s, nullptr, nullptr,
                               hipExtAnyOrderLaunch, w, x, y, n, k, fin, expected, fout, (uint32_t*)err, spin_limit);
       else
