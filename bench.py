@@ -507,6 +507,7 @@ def probe_chain(n_mats=32, n_launches=64):
                             ("overlapped_coherent_x_1024wg", 1, 1024),
                             ("overlapped_poll_wave", 3, 0), ("overlapped_poll_wave_all_weights_first", 4, 0),
                             ("overlapped_poll_wave_256wg", 3, 256), ("overlapped_poll_wave_all_weights_first_256wg", 4, 256),
+                            ("independent_ordinary", 6, 0), ("independent_free_to_overlap", 5, 0),
                             ("ordinary_again", 0, 0)):
         samples = []
         for rep in range(6):
@@ -523,6 +524,8 @@ def probe_chain(n_mats=32, n_launches=64):
             if rep:
                 samples.append(a.elapsed_time(b) * 1e3 / n_launches)
         res = (xa if n_launches % 2 == 0 else xb).clone()
+        if mode in (5, 6):
+            res = ref  # independent launches: timing only
         if ref is None:
             ref = res
         out[name] = {"us_per_gemv": round(_median(samples), 3), "min": round(min(samples), 3), "max": round(max(samples), 3),

@@ -181,12 +181,21 @@ __global__ void __launch_bounds__(kChainThreads + kWave) chain_gemv_pollwave_ker
       }
     }
     // (the wave reconverges here: the loads below follow every lane's last poll)
-    for (int c = lane; c < kc; c += kWave) {
-      const uint64_t* xp = (const uint64_t*)(x + (c << 3));
-      const uint64_t lo = __hip_atomic_load(xp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const uint64_t hi = __hip_atomic_load(xp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      *(uint64_t*)&xs[(c << 3)] = lo;
-      *(uint64_t*)&xs[(c << 3) + 4] = hi;
+    // all of x requested before the first value is used: one round trip, not one per chunk
+    constexpr int kIter = kChainCH * kChainThreads / kWave;
+    uint64_t lo[kIter], hi[kIter];
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+      const int c = lane + i * kWave;
+      const uint64_t* xp = (const uint64_t*)(x + ((c < kc ? c : 0) << 3));
+      lo[i] = __hip_atomic_load(xp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      hi[i] = __hip_atomic_load(xp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int i = 0; i < kIter; ++i) {
+      const int c = lane + i * kWave;
+      *(uint64_t*)&xs[(c << 3)] = lo[i];
+      *(uint64_t*)&xs[(c << 3) + 4] = hi[i];
     }
   }
   __syncthreads();
@@ -264,7 +273,7 @@ extern "C" int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* c
                                     int workgroups, int spin_limit) {
   MUI_CHECK_ARG(weights && n_mats > 0 && n_launches > 0 && xa && xb && err);
   MUI_CHECK_ARG(n == k && k > 0 && k <= kChainCH * kChainThreads * 8 && (k & 7) == 0 && (n % kChainR) == 0);
-  MUI_CHECK_ARG(mode == 0 || ((mode >= 1 && mode <= 4) && flags));
+  MUI_CHECK_ARG(mode == 0 || mode == 5 || mode == 6 || ((mode >= 1 && mode <= 4) && flags));
   MUI_CHECK_ARG(spin_limit > 0 && spin_limit <= (1 << 22));
   const int n_groups = n / kChainR;
   int grid = workgroups > 0 ? workgroups : balanced_grid(n_groups, 3);
@@ -277,7 +286,18 @@ extern "C" int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* c
     const uint16_t* w = (const uint16_t*)weights[i % n_mats];
     const uint16_t* x = (const uint16_t*)((i & 1) ? xb : xa);
     uint16_t* y = (uint16_t*)((i & 1) ? xa : xb);
-    if (mode == 0) {
+    if (mode == 5 || mode == 6) {
+      // independent GEMVs (every launch reads xa and writes its own half of xb's ... the same y: the
+      // results are not used), ordinary (6) or free to overlap (5): what overlap alone is worth
+      if (mode == 6)
+        hipLaunchKernelGGL((chain_gemv_kernel<false, false>), dim3(grid), dim3(kChainThreads), 0, s, w,
+                           (const uint16_t*)xa, (uint16_t*)xb, n, k, (const uint32_t*)nullptr, 0u, (uint32_t*)nullptr,
+                           (uint32_t*)err, spin_limit);
+      else
+        hipExtLaunchKernelGGL((chain_gemv_kernel<false, false>), dim3(grid), dim3(kChainThreads), 0, s, nullptr, nullptr,
+                              hipExtAnyOrderLaunch, w, (const uint16_t*)xa, (uint16_t*)xb, n, k, (const uint32_t*)nullptr,
+                              0u, (uint32_t*)nullptr, (uint32_t*)err, spin_limit);
+    } else if (mode == 0) {
       hipLaunchKernelGGL((chain_gemv_kernel<false, false>), dim3(grid), dim3(kChainThreads), 0, s, w, x, y, n, k,
                          (const uint32_t*)nullptr, 0u, (uint32_t*)nullptr, (uint32_t*)err, spin_limit);
     } else {
