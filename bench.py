@@ -532,6 +532,35 @@ def probe_chain(n_mats=32, n_launches=64):
                      "wait_ran_out": bool(err.item()), "bit_identical_to_ordinary": bool(torch.equal(res, ref)),
                      "finite": bool(torch.isfinite(res).all())}
         _progress("probe-chain %s: %s" % (name, out[name]))
+    # the chain dealt alternately to two streams (two hardware queues)
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    for name, mode, wgs in (("two_streams_independent", 0, 0), ("two_streams_handoff", 1, 0),
+                            ("two_streams_poll_wave", 2, 0), ("two_streams_poll_wave_all_weights_first", 3, 0),
+                            ("two_streams_handoff_256wg", 1, 256), ("two_streams_poll_wave_all_weights_first_256wg", 3, 256)):
+        samples = []
+        for rep in range(6):
+            xa.copy_(x0)
+            flags.zero_()
+            err.zero_()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(sa)
+            sb.wait_event(a)
+            _lib.check(lib.mui_probe_gemv_chain2(sa.cuda_stream, sb.cuda_stream, mode, ptrs, n_mats, n_launches, n, n,
+                                                 xa.data_ptr(), xb.data_ptr(), flags.data_ptr(), err.data_ptr(), wgs, 20000),
+                       "mui_probe_gemv_chain2")
+            done_b = torch.cuda.Event()
+            done_b.record(sb)
+            sa.wait_event(done_b)
+            b.record(sa)
+            torch.cuda.synchronize()
+            if rep:
+                samples.append(a.elapsed_time(b) * 1e3 / n_launches)
+        res = (xa if n_launches % 2 == 0 else xb).clone()
+        out[name] = {"us_per_gemv": round(_median(samples), 3), "min": round(min(samples), 3), "max": round(max(samples), 3),
+                     "wait_ran_out": bool(err.item()),
+                     "bit_identical_to_ordinary": None if mode == 0 else bool(torch.equal(res, ref))}
+        _progress("probe-chain %s: %s" % (name, out[name]))
     print(json.dumps({"probe_chain": out}))
 
 

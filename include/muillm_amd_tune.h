@@ -86,6 +86,13 @@ size_t mui_probe_chain_flag_bytes(int n_launches);
 int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* const* weights, int n_mats,
                          int n_launches, int n, int k, void* xa, void* xb, void* flags, void* err,
                          int workgroups, int spin_limit);
+/* The same chain dealt alternately to two streams (ordinary launches; a kernel meets its predecessor,
+ * which runs on the other stream, through the arrival counters): mode 0 independent GEMVs without
+ * hand-off, 1 the hand-off of mode 1 above, 2 / 3 a variant whose fifth wave polls and fetches x
+ * while the other four have one / two row groups of weights in flight. */
+int mui_probe_gemv_chain2(mui_stream_t stream_a, mui_stream_t stream_b, int mode,
+                          const void* const* weights, int n_mats, int n_launches, int n, int k, void* xa,
+                          void* xb, void* flags, void* err, int workgroups, int spin_limit);
 
 #ifdef __cplusplus
 }

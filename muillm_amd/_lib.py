@@ -105,6 +105,7 @@ _SIGNATURES = {
     "mui_tune_warm": (c_int, [c_int, c_int, c_int]),
     "mui_probe_chain_flag_bytes": (ctypes.c_size_t, [c_int]),
     "mui_probe_gemv_chain": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int]),
+    "mui_probe_gemv_chain2": (c_int, [_P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, c_int, c_int]),
 }
 
 

@@ -323,3 +323,45 @@ extern "C" int mui_probe_gemv_chain(mui_stream_t stream, int mode, const void* c
   }
   return MUI_OK;
 }
+
+// The same chain dealt alternately to TWO streams (launch i goes to stream i % 2; ordinary launches,
+// so a kernel waits for the launch two before it through its own queue and for its predecessor, on
+// the other queue, through the arrival counters): two kernels can then be resident at a time -- the
+// one that computes and its successor, whose weights are already on their way. mode 0: independent
+// GEMVs (no hand-off, results unused: what two queues overlap at best); 1: hand-off as in
+// mui_probe_gemv_chain mode 1; 2 / 3: the poll-wave kernel with one / two row groups requested first.
+extern "C" int mui_probe_gemv_chain2(mui_stream_t stream_a, mui_stream_t stream_b, int mode,
+                                     const void* const* weights, int n_mats, int n_launches, int n, int k, void* xa,
+                                     void* xb, void* flags, void* err, int workgroups, int spin_limit) {
+  MUI_CHECK_ARG(weights && n_mats > 0 && n_launches > 0 && xa && xb && err && flags);
+  MUI_CHECK_ARG(n == k && k > 0 && k <= kChainCH * kChainThreads * 8 && (k & 7) == 0 && (n % kChainR) == 0);
+  MUI_CHECK_ARG(mode >= 0 && mode <= 3 && spin_limit > 0 && spin_limit <= (1 << 22));
+  const int n_groups = n / kChainR;
+  int grid = workgroups > 0 ? workgroups : balanced_grid(n_groups, 3);
+  if (grid > n_groups) grid = n_groups;
+  if (grid % kChainCounters != 0) return MUI_ERR_INVALID_ARG;
+  uint32_t* fl = (uint32_t*)flags;
+  for (int i = 0; i < n_launches; ++i) {
+    hipStream_t s = (hipStream_t)((i & 1) ? stream_b : stream_a);
+    const uint16_t* w = (const uint16_t*)weights[i % n_mats];
+    const uint16_t* x = (const uint16_t*)((i & 1) ? xb : xa);
+    uint16_t* y = (uint16_t*)((i & 1) ? xa : xb);
+    const uint32_t* fin = i == 0 ? nullptr : fl + (size_t)(i - 1) * kChainCounters * kChainCounterStride;
+    uint32_t* fout = fl + (size_t)i * kChainCounters * kChainCounterStride;
+    const uint32_t expected = (uint32_t)(grid / kChainCounters);
+    if (mode == 0)
+      hipLaunchKernelGGL((chain_gemv_kernel<false, false>), dim3(grid), dim3(kChainThreads), 0, s, w, (const uint16_t*)xa,
+                         (uint16_t*)xb, n, k, (const uint32_t*)nullptr, 0u, (uint32_t*)nullptr, (uint32_t*)err, spin_limit);
+    else if (mode == 1)
+      hipLaunchKernelGGL((chain_gemv_kernel<true, true>), dim3(grid), dim3(kChainThreads), 0, s, w, x, y, n, k, fin,
+                         expected, fout, (uint32_t*)err, spin_limit);
+    else if (mode == 2)
+      hipLaunchKernelGGL((chain_gemv_pollwave_kernel<1>), dim3(grid), dim3(kChainThreads + kWave), 0, s, w, x, y, n, k,
+                         fin, expected, fout, (uint32_t*)err, spin_limit);
+    else
+      hipLaunchKernelGGL((chain_gemv_pollwave_kernel<2>), dim3(grid), dim3(kChainThreads + kWave), 0, s, w, x, y, n, k,
+                         fin, expected, fout, (uint32_t*)err, spin_limit);
+    if (hipGetLastError() != hipSuccess) return MUI_ERR_LAUNCH;
+  }
+  return MUI_OK;
+}
