@@ -14,6 +14,18 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
+@pytest.fixture(params=["wave-per-row", "chunks-per-thread"], autouse=True)
+def int8_kernel_choice(request):
+    """Every test runs twice: with the built-in choice (rows of at most 4096 codes at 1..4 tokens take
+    the kernel that gives each wave whole rows, int8_wave.hip) and with that kernel switched off (the
+    kernel that deals a row's chunks out to a workgroup's threads, int8_multi.hip, serves them)."""
+    lib = _lib.load()
+    if request.param == "chunks-per-thread":
+        _lib.check(lib.mui_tune_int8_wave(0, 0), "mui_tune_int8_wave")
+    yield request.param
+    _lib.check(lib.mui_tune_int8_wave(1, 0), "mui_tune_int8_wave")
+
+
 def _gen(seed=0):
     g = torch.Generator(device="cpu")
     g.manual_seed(seed)
@@ -159,6 +171,27 @@ def test_group_linear(n, k, gs, tokens):
                                               None, None, r.to(DEV))
     assert_parity(y, ref, 1e-2, f"int8 group {n}x{k} gs={gs}", tight=4e-3)
     assert oracle.rel_err(y.cpu(), oracle.linear(x, w, gamma, 1e-5, None, r)) < 3e-2
+
+
+@pytest.mark.parametrize("n,k,gs", [(14336, 4096, 128), (300, 1024, 64), (5, 64, 16)])
+@pytest.mark.parametrize("tokens", [2, 3, 4])
+def test_group_gateup_small_batches(n, k, gs, tokens):
+    g = _gen(16)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    qg, smg = oracle.rtn_quantize_group(wg, gs)
+    qu, smu = oracle.rtn_quantize_group(wu, gs)
+    shift = gs.bit_length() - 1
+    ng = k // gs
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    wgd = (qg.reshape(-1, gs).double() * smg[:, None, 0].double() + smg[:, None, 1].double()).reshape(n, k)
+    wud = (qu.reshape(-1, gs).double() * smu[:, None, 0].double() + smu[:, None, 1].double()).reshape(n, k)
+    ref = oracle.gateup_silu(x, wgd, wud, gamma, 1e-5)
+    packed_w = torch.stack([qg, qu], dim=1).to(DEV)
+    packed_s = torch.stack([smg.reshape(n, ng, 2), smu.reshape(n, ng, 2)], dim=1).to(DEV)
+    h = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, packed_w, packed_s, shift, x.to(DEV))
+    assert h.shape == (tokens, n)
+    assert_parity(h, ref, 1e-2, f"int8 group gateup {n}x{k} b={tokens}", tight=9e-3)
 
 
 @pytest.mark.parametrize("n,k,gs", [(14336, 4096, 128), (100, 512, 32)])
