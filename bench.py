@@ -1097,8 +1097,6 @@ def main():
                     help="experiment: mui_tune_attention(waves per workgroup, min tokens per split, "
                          "longest unsplit sequence (-1 disables the head-parallel unsplit mode), shortest sequence for "
                          "the matrix-core kernel (-1 disables it))")
-    ap.add_argument("--tune-int8-wave", default=None, metavar="ON,WORKGROUPS_PER_CU",
-                    help="experiment: mui_tune_int8_wave(on, workgroups per CU) before anything is timed")
     ap.add_argument("--only-kernel-table", action="store_true",
                     help="only time the per-kernel table (for rocprofv3 kernel traces of the C1-C4 shapes)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -1169,11 +1167,6 @@ def main():
 
         w, mt, dt, mf = (int(v) for v in args.tune_attention.split(","))
         _lib.check(_lib.load().mui_tune_attention(w, mt, dt, mf), "mui_tune_attention")
-    if args.tune_int8_wave:
-        from muillm_amd import _lib
-
-        on, per_cu = (int(v) for v in args.tune_int8_wave.split(","))
-        _lib.check(_lib.load().mui_tune_int8_wave(on, per_cu), "mui_tune_int8_wave")
     config = MuiDecoderConfig.llama3_8b(num_hidden_layers=args.layers, max_position_embeddings=8192)
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
     torch.cuda.synchronize()

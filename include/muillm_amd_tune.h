@@ -25,10 +25,6 @@ int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
  * points through the packed-dot int8 kernel (default on) */
 int mui_tune_packed_dot(int linear_on, int int8_on);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
-/* int8 weights on rows of at most 4096 codes, 1..4 fp16 tokens: on != 0 (default) takes the kernel
- * that gives every wave whole rows (no reduction across waves), 0 the one that deals a row's chunks
- * out to the workgroup's threads; workgroups_per_cu 0 = built-in choice */
-int mui_tune_int8_wave(int on, int workgroups_per_cu);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the
  * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1536;

@@ -378,8 +378,6 @@ void skinny_set_lt(int on) { g_skinny_lt = on; }
 
 static int g_int8_multi = 1;  // 2..4 tokens of int8 weights: vector-ALU kernel (int8_multi.hip) first
 void skinny_set_int8_multi(int on) { g_int8_multi = on; }
-static int g_int8_wave = 1;   // rows of at most 4096 int8 weights, 1..4 tokens: one wave per row (int8_wave.hip)
-void skinny_set_int8_wave(int on) { g_int8_wave = on; }
 
 // entry used by gemv.hip / int8.hip for tokens >= 2
 int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams& p) {
@@ -390,10 +388,6 @@ int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams&
   // the vector-ALU kernel wins there too (gate/up at 4 tokens 26.9 vs 36.9 us, down 17.6 vs 20.7 us)
   const bool lt_first = g_skinny_lt && wf == WF_I8_CHANNEL && p.tokens >= 3 &&
                         (p.k > 8192 || (epi == SK_GATEUP && p.n >= 8192));
-  if (wf != WF_16BIT && g_int8_wave && p.tokens <= 4) {
-    const int st = launch_int8_wave(s, dtype, wf, epi, p);
-    if (st != MUI_ERR_UNSUPPORTED) return st;
-  }
   if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4 && !lt_first) {
     const int st = launch_int8_multi(s, dtype, wf, epi, p);
     if (st != MUI_ERR_UNSUPPORTED) return st;

@@ -366,13 +366,6 @@ extern "C" int mui_tune_int8(int rows, int wgs_per_cu) {
   return MUI_OK;
 }
 
-extern "C" int mui_tune_int8_wave(int on, int wgs_per_cu) {
-  if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
-  skinny_set_int8_wave(on != 0);
-  int8_wave_set_per_cu(wgs_per_cu);
-  return MUI_OK;
-}
-
 extern "C" int mui_int8_linear(mui_stream_t stream, int dtype, const void* weights_i8, long w_pitch,
                                const void* scales, const void* x, const void* norm_weights,
                                float epsilon, const void* add_bias, const void* residual, void* y,

@@ -170,11 +170,6 @@ int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 =
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 void skinny_set_int8_multi(int on);
-// 1..4 tokens, int8 weights, fp16 activations, rows of at most 4096 weights: one wave per row
-// (int8_wave.hip); same contract
-int launch_int8_wave(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
-void skinny_set_int8_wave(int on);
-void int8_wave_set_per_cu(int per_cu);
 void int8_set_packed_dot(bool on);  // int8.hip: single fp16 token through int8_multi.hip
 
 }  // namespace mui

@@ -14,18 +14,6 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
-@pytest.fixture(params=["wave-per-row", "chunks-per-thread"], autouse=True)
-def int8_kernel_choice(request):
-    """Every test runs twice: with the built-in choice (rows of at most 4096 codes at 1..4 tokens take
-    the kernel that gives each wave whole rows, int8_wave.hip) and with that kernel switched off (the
-    kernel that deals a row's chunks out to a workgroup's threads, int8_multi.hip, serves them)."""
-    lib = _lib.load()
-    if request.param == "chunks-per-thread":
-        _lib.check(lib.mui_tune_int8_wave(0, 0), "mui_tune_int8_wave")
-    yield request.param
-    _lib.check(lib.mui_tune_int8_wave(1, 0), "mui_tune_int8_wave")
-
-
 def _gen(seed=0):
     g = torch.Generator(device="cpu")
     g.manual_seed(seed)
