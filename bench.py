@@ -1097,6 +1097,9 @@ def main():
                     help="experiment: mui_tune_attention(waves per workgroup, min tokens per split, "
                          "longest unsplit sequence (-1 disables the head-parallel unsplit mode), shortest sequence for "
                          "the matrix-core kernel (-1 disables it))")
+    ap.add_argument("--tune-skinny", default=None, metavar="MIN_TOKENS,STREAM_B,MULTI_MAX_TOKENS",
+                    help="experiment: mui_tune_skinny(...) before anything is timed (2,0,1 sends int8 weights at "
+                         "2..4 tokens to the matrix-core kernel)")
     ap.add_argument("--only-kernel-table", action="store_true",
                     help="only time the per-kernel table (for rocprofv3 kernel traces of the C1-C4 shapes)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -1167,6 +1170,11 @@ def main():
 
         w, mt, dt, mf = (int(v) for v in args.tune_attention.split(","))
         _lib.check(_lib.load().mui_tune_attention(w, mt, dt, mf), "mui_tune_attention")
+    if args.tune_skinny:
+        from muillm_amd import _lib
+
+        a, b, c = (int(v) for v in args.tune_skinny.split(","))
+        _lib.check(_lib.load().mui_tune_skinny(a, b, c), "mui_tune_skinny")
     config = MuiDecoderConfig.llama3_8b(num_hidden_layers=args.layers, max_position_embeddings=8192)
     lm = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0)
     torch.cuda.synchronize()

@@ -147,6 +147,19 @@ __device__ __forceinline__ u32x4 convert_a(uint32_t w0, uint32_t w1, const uint1
   }
 }
 
+// group format with the (scale, min) pair already in a register: u8 * scale + min, rounded once
+template <typename T>
+__device__ __forceinline__ u32x4 convert_a_pair(uint32_t w0, uint32_t w1, uint32_t pair) {
+  const uint32_t v[2] = {w0, w1};
+  const float sc = T::lo(pair), mn = T::hi(pair);
+  float f[8];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) f[4 * m + b] = fmaf((float)((v[m] >> (8 * b)) & 0xffu), sc, mn);
+  return pack8<T>(f);
+}
+
 // tiled matrix-core GEMM for prompts (gemm_prefill.hip): any token count, 16-bit or per-channel int8
 int launch_prefill_gemm(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 size_t prefill_workspace_bytes();  // what SkinnyParams::workspace must hold for the prompt GEMM to use it
