@@ -56,6 +56,16 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   p.s0 = s0; p.s1 = s1; p.s_pitch = s_pitch; p.group_shift = group_shift;
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
   constexpr int WB = (WF == WF_16BIT) ? 2 : 1;   // bytes per weight
+  // Group format with fp16 activations and groups of at least 128 codes: the codes reach the matrix
+  // cores as the integers 1024 + u8 (a byte dropped into the mantissa of 1024.0: two byte permutes
+  // per four codes instead of a convert, a multiply-add and a pack per code), the products of a
+  // group's k-steps are accumulated on their own and folded into the running sums once per group:
+  //   sum_k (u8_k * scale + min) x_k = scale * (sum_k (1024 + u8_k) x_k) + (min - 1024 scale) * sum_k x_k
+  // with sum_k x_k from one more matrix instruction against a tile of ones. For (scale, min) to be
+  // one pair per lane the product is taken transposed -- token rows as the first operand, weight
+  // rows as the second --, so that lane (g, i) holds tokens 4 g .. 4 g + 3 of weight row i, the row
+  // whose pairs it already loads for the conversion layout.
+  constexpr bool GACC = WF == WF_U8_GROUP && GP > 0 && T::kDtype == MUI_DTYPE_F16;
   // k-values per wave and pass: 256 (512 bytes of a 16-bit row). Per-channel int8 weights in
   // B-stationary mode can take 512 (BIGP), so that a pass again covers 512 contiguous bytes of
   // each row and a load instruction two rows of them: with 256-byte runs and half the bytes in
@@ -277,10 +287,14 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
 #pragma unroll
     for (int q = 0; q < NLD; ++q) *(u32x4*)(la + (q * RPI + ld_row) * PITCH + ld_chunk * 16) = ok ? a[q] : zero;
     if constexpr (!BSTAT) {
-      const bool count = NORM && i < passes && pass_k0(i) + xl_chunk * 8 < p.k;
+      const bool x_ok = pass_k0(i) + xl_chunk * 8 < p.k;
+      const bool count = NORM && i < passes && x_ok;
 #pragma unroll
       for (int q = 0; q < XL; ++q) {
         u32x4 v = b[q];
+        // group format: a code zeroed past the row end still stands for `min` (or 1024 + 0), so the
+        // token values of those k-values are zeroed as well
+        if constexpr (WF == WF_U8_GROUP) v = x_ok ? v : zero;
         if constexpr (NORM) {
           float sq = 0.f;
           v = make_b<T, true>(v, gm, sq);
@@ -305,6 +319,34 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     }
     const uint16_t* srow = scale_row(blockIdx.x + (i / passes) * gridDim.x);
     const int k0 = pass_k0(i);
+    if constexpr (GACC) {
+      constexpr int SEG = STEPS / GP;  // k-steps that share a (scale, min) pair
+      const u32x4 ones = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+#pragma unroll
+      for (int q = 0; q < GP; ++q) {
+        f32x4 part = {0.f, 0.f, 0.f, 0.f}, part1 = {0.f, 0.f, 0.f, 0.f}, xs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < SEG; ++s2) {
+          const int s = q * SEG + s2;
+          // (steps past the wave's range in a partial B-stationary pass multiply zeroed weights)
+          u32x4 av, bv;
+          av.x = __builtin_amdgcn_perm(0x64646464u, a8[s].x, 0x04010400u);
+          av.y = __builtin_amdgcn_perm(0x64646464u, a8[s].x, 0x04030402u);
+          av.z = __builtin_amdgcn_perm(0x64646464u, a8[s].y, 0x04010400u);
+          av.w = __builtin_amdgcn_perm(0x64646464u, a8[s].y, 0x04030402u);
+          if constexpr (BSTAT) bv = bq[half * STEPS + s];
+          else bv = bx[s];
+          if (s2 & 1) part1 = mfma16x16x32<T>(bv, av, part1);
+          else part = mfma16x16x32<T>(bv, av, part);
+          xs = mfma16x16x32<T>(bv, ones, xs);
+        }
+        const float sc = T::lo(sp[q]), cm = fmaf(-1024.f, sc, T::hi(sp[q]));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc, part[r] + part1[r], fmaf(cm, xs[r], acc[r]));
+      }
+      __builtin_amdgcn_wave_barrier();
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       if (BSTAT && !FULL && half * STEPS + s >= jmax) break;
@@ -328,7 +370,10 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   auto finish = [&](int i, const Extras& ex) {
     if ((i % passes) == passes - 1) {  // last pass of the tile: reduce over the waves
 #pragma unroll
-      for (int r = 0; r < 4; ++r) tile[buf][wave][4 * g + r][r16] = acc[r] + acc1[r];
+      for (int r = 0; r < 4; ++r) {
+        if constexpr (GACC) tile[buf][wave][r16][4 * g + r] = acc[r];  // transposed product: [weight row][token]
+        else tile[buf][wave][4 * g + r][r16] = acc[r] + acc1[r];
+      }
       acc = f32x4{0.f, 0.f, 0.f, 0.f};
       acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
       if constexpr (NORM && !BSTAT) {

@@ -161,8 +161,35 @@ def test_group_linear(n, k, gs, tokens):
     assert oracle.rel_err(y.cpu(), oracle.linear(x, w, gamma, 1e-5, None, r)) < 3e-2
 
 
+@pytest.mark.parametrize("matrix_cores", [False, True])
+@pytest.mark.parametrize("n,k,gs", [(4096, 14336, 128), (64, 4224, 128), (40, 8448, 256), (33, 4096, 128), (4096, 4096, 4096)])
+@pytest.mark.parametrize("tokens", [3, 4, 8, 16])
+def test_group_linear_long_rows_and_group_accumulation(n, k, gs, tokens, matrix_cores):
+    """Groups of 128 codes and more on the matrix-core kernel (its default from 5 tokens; forced here
+    from 3): rows streamed in passes (K = 14336), a last pass that ends inside the row (K = 4224,
+    8448), rows that do not fill a 16-row tile, one group per row -- the per-group accumulation
+    must give what the oracle's dequantise-then-multiply gives."""
+    lib = _lib.load()
+    if matrix_cores:
+        _lib.check(lib.mui_tune_skinny(2, 0, 1), "mui_tune_skinny")
+    try:
+        g = _gen(25)
+        w = _mk((n, k), g, 0.02)
+        q, smv = oracle.rtn_quantize_group(w, gs)
+        shift = gs.bit_length() - 1
+        x = _mk((tokens, k), g)
+        gamma = _mk((k,), g, 0.1, 1.0) if k <= 4224 else None
+        r = _mk((tokens, n), g)
+        ref = oracle.int8_group_linear(x, q, smv, gs, gamma, 1e-5, None, r)
+        y = muillm_ext.muillm_int8_linear_forward(x.to(DEV), q.to(DEV), smv.to(DEV), shift,
+                                                  None if gamma is None else gamma.to(DEV), 1e-5, None, None, r.to(DEV))
+        assert_parity(y, ref, 1e-2, f"int8 group {n}x{k} gs={gs} b={tokens} mfma={matrix_cores}", tight=4e-3)
+    finally:
+        _lib.check(lib.mui_tune_skinny(2, 0, 0), "mui_tune_skinny")
+
+
 @pytest.mark.parametrize("n,k,gs", [(14336, 4096, 128), (300, 1024, 64), (5, 64, 16)])
-@pytest.mark.parametrize("tokens", [2, 3, 4])
+@pytest.mark.parametrize("tokens", [2, 3, 4, 8])
 def test_group_gateup_small_batches(n, k, gs, tokens):
     g = _gen(16)
     wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
