@@ -384,9 +384,11 @@ int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams&
   // int8 at up to 4 tokens: the vector-ALU kernel, except at 3-4 tokens long rows (down 4096 x
   // 14336 at 4 tokens: 13.6 vs 16.4 us) and tall gate/up matrices (2 x 14336 x 4096: a steady
   // 27 us against 27-34 us), where the matrix-core kernel measured faster -- with per-channel
-  // scales; in the group format (a scale pair per 8 codes in the matrix-core kernel's inner loop)
-  // the vector-ALU kernel wins there too (gate/up at 4 tokens 26.9 vs 36.9 us, down 17.6 vs 20.7 us)
-  const bool lt_first = g_skinny_lt && wf == WF_I8_CHANNEL && p.tokens >= 3 &&
+  // scales and, for fp16 activations, with the reference's groups of 128 codes or more, which that
+  // kernel scales once per group (gate/up at 4 tokens 24.3 vs 29.4 us, down 16.7 vs 18.9 us); smaller
+  // groups and bf16 convert code by code there and stay on the vector-ALU kernel
+  const bool lt_format = wf == WF_I8_CHANNEL || (wf == WF_U8_GROUP && p.group_shift >= 7 && dtype == MUI_DTYPE_F16);
+  const bool lt_first = g_skinny_lt && lt_format && p.tokens >= 3 &&
                         (p.k > 8192 || (epi == SK_GATEUP && p.n >= 8192));
   if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4 && !lt_first) {
     const int st = launch_int8_multi(s, dtype, wf, epi, p);

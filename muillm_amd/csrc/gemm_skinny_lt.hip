@@ -66,6 +66,15 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   // rows as the second --, so that lane (g, i) holds tokens 4 g .. 4 g + 3 of weight row i, the row
   // whose pairs it already loads for the conversion layout.
   constexpr bool GACC = WF == WF_U8_GROUP && GP > 0 && T::kDtype == MUI_DTYPE_F16;
+  // Per-channel int8 with fp16 activations, same idea: the codes enter as 1024 + 128 + q (sign bit
+  // flipped, byte dropped into the mantissa of 1024.0) and 1152 * sum_k x_k is taken off the finished
+  // sums -- sum_k x_k over a wave's K range is a constant of the wave in B-stationary mode (sixteen
+  // matrix instructions against a tile of ones, once), and one more matrix instruction per step in
+  // streaming mode -- instead of a packed subtract per two codes on the way to the operand.
+  constexpr bool CACC = WF == WF_I8_CHANNEL && T::kDtype == MUI_DTYPE_F16;
+  const u32x4 ones16 = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+  f32x4 xs_wave = {0.f, 0.f, 0.f, 0.f};  // CACC, B-stationary: sum of this wave's token operands per token column
+  f32x4 xs_run = {0.f, 0.f, 0.f, 0.f};   // CACC, streaming: the same over the passes of the current tile
   // k-values per wave and pass: 256 (512 bytes of a 16-bit row). Per-channel int8 weights in
   // B-stationary mode can take 512 (BIGP), so that a pass again covers 512 contiguous bytes of
   // each row and a load instruction two rows of them: with 256-byte runs and half the bytes in
@@ -294,7 +303,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
         u32x4 v = b[q];
         // group format: a code zeroed past the row end still stands for `min` (or 1024 + 0), so the
         // token values of those k-values are zeroed as well
-        if constexpr (WF == WF_U8_GROUP) v = x_ok ? v : zero;
+        if constexpr (WF != WF_16BIT) v = x_ok ? v : zero;
         if constexpr (NORM) {
           float sq = 0.f;
           v = make_b<T, true>(v, gm, sq);
@@ -321,7 +330,6 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     const int k0 = pass_k0(i);
     if constexpr (GACC) {
       constexpr int SEG = STEPS / GP;  // k-steps that share a (scale, min) pair
-      const u32x4 ones = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
 #pragma unroll
       for (int q = 0; q < GP; ++q) {
         f32x4 part = {0.f, 0.f, 0.f, 0.f}, part1 = {0.f, 0.f, 0.f, 0.f}, xs = {0.f, 0.f, 0.f, 0.f};
@@ -338,7 +346,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
           else bv = bx[s];
           if (s2 & 1) part1 = mfma16x16x32<T>(bv, av, part1);
           else part = mfma16x16x32<T>(bv, av, part);
-          xs = mfma16x16x32<T>(bv, ones, xs);
+          xs = mfma16x16x32<T>(bv, ones16, xs);
         }
         const float sc = T::lo(sp[q]), cm = fmaf(-1024.f, sc, T::hi(sp[q]));
 #pragma unroll
@@ -353,7 +361,13 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
       u32x4 av, bv;
       if constexpr (WF == WF_16BIT) av = a16[s];
       else {
-        if constexpr (WF == WF_U8_GROUP && GP > 0) {
+        if constexpr (CACC) {
+          const uint32_t u0 = a8[s].x ^ 0x80808080u, u1 = a8[s].y ^ 0x80808080u;
+          av.x = __builtin_amdgcn_perm(0x64646464u, u0, 0x04010400u);
+          av.y = __builtin_amdgcn_perm(0x64646464u, u0, 0x04030402u);
+          av.z = __builtin_amdgcn_perm(0x64646464u, u1, 0x04010400u);
+          av.w = __builtin_amdgcn_perm(0x64646464u, u1, 0x04030402u);
+        } else if constexpr (WF == WF_U8_GROUP && GP > 0) {
           av = convert_a_pair<T>(a8[s].x, a8[s].y, sp[s / (STEPS / GP)]);
         } else {
           const int ke = k0 + 32 * s + 8 * g;  // (clamped: the scale pair of a k past the row end is never used)
@@ -364,6 +378,7 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
       else bv = bx[s];
       if (s & 1) acc1 = mfma16x16x32<T>(av, bv, acc1);
       else acc = mfma16x16x32<T>(av, bv, acc);
+      if constexpr (CACC && !BSTAT) xs_run = mfma16x16x32<T>(ones16, bv, xs_run);
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -372,8 +387,10 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         if constexpr (GACC) tile[buf][wave][r16][4 * g + r] = acc[r];  // transposed product: [weight row][token]
+        else if constexpr (CACC) tile[buf][wave][4 * g + r][r16] = fmaf(-1152.f, BSTAT ? xs_wave[r] : xs_run[r], acc[r] + acc1[r]);
         else tile[buf][wave][4 * g + r][r16] = acc[r] + acc1[r];
       }
+      xs_run = f32x4{0.f, 0.f, 0.f, 0.f};
       acc = f32x4{0.f, 0.f, 0.f, 0.f};
       acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
       if constexpr (NORM && !BSTAT) {
@@ -433,6 +450,10 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
 #pragma unroll
         for (int j = 0; j < kLtSteps; ++j) bq[h * kLtSteps + j] = *(const u32x4*)(la + r16 * kLtXPitch + (4 * j + g) * 16);
         __builtin_amdgcn_wave_barrier();
+      }
+      if constexpr (CACC) {
+#pragma unroll
+        for (int j = 0; j < 2 * kLtSteps; ++j) xs_wave = mfma16x16x32<T>(ones16, bq[j], xs_wave);
       }
     }
   };
