@@ -810,7 +810,7 @@ def pmc_probe_attention(launches=3):
     print(json.dumps({"pmc_probe_attention": info}))
 
 
-def kernel_table(lm):
+def kernel_table(lm, int8_tokens=(1, 4)):
     """GB/s of each fused kernel family at the benchmark shapes, HIP-event timed through the C ABI
     with pre-allocated outputs. Weights rotate over distinct buffers totalling >= 0.9 GB (the model's
     32 layers, or a ring) so neither L2 nor the 256 MB Infinity Cache can serve them ("cold").
@@ -828,7 +828,7 @@ def kernel_table(lm):
     f16 = dict(device="cuda", dtype=torch.float16)
     gamma = (1 + 0.1 * torch.randn(hid)).half().cuda()
     X, RES = torch.randn(16, hid, **f16), torch.randn(16, hid, **f16)
-    HMID = torch.randn(8, inter, **f16)
+    HMID = torch.randn(16, inter, **f16)
     Y = torch.empty(16 * max(v, inter), **f16)
     out = {}
 
@@ -900,7 +900,7 @@ def kernel_table(lm):
         return [(torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda"),
                  (torch.rand(n, **f16) * 1e-3 + 1e-4)) for _ in range(cnt)]
 
-    for b in (1, 4):
+    for b in int8_tokens:
         for name, n, k, norm, resid in (("qkv", n_qkv, hid, True, False), ("o_proj", hid, hid, False, True),
                                         ("down", hid, inter, False, True)):
             ring = i8_ring(n, k)
@@ -938,7 +938,7 @@ def kernel_table(lm):
         return [(torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda"),
                  torch.rand(n * (k // gsz), 2, **f16) * 1e-3 + 1e-4) for _ in range(cnt)]
 
-    for b in (1, 4):
+    for b in int8_tokens:
         for name, n, k, norm, resid in (("qkv", n_qkv, hid, True, False), ("o_proj", hid, hid, False, True),
                                         ("down", hid, inter, False, True)):
             ring = g_ring(n, k)
@@ -1100,6 +1100,8 @@ def main():
     ap.add_argument("--tune-skinny", default=None, metavar="MIN_TOKENS,STREAM_B,MULTI_MAX_TOKENS",
                     help="experiment: mui_tune_skinny(...) before anything is timed (2,0,1 sends int8 weights at "
                          "2..4 tokens to the matrix-core kernel)")
+    ap.add_argument("--table-int8-tokens", default="1,4", metavar="LIST",
+                    help="token counts of the int8 rows of the kernel table (the baseline's configuration: 1,4)")
     ap.add_argument("--only-kernel-table", action="store_true",
                     help="only time the per-kernel table (for rocprofv3 kernel traces of the C1-C4 shapes)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -1180,7 +1182,7 @@ def main():
     torch.cuda.synchronize()
 
     if args.only_kernel_table:
-        print(json.dumps({"kernels": kernel_table(lm)}))
+        print(json.dumps({"kernels": kernel_table(lm, tuple(int(v) for v in args.table_int8_tokens.split(",")))}))
         return
     if args.probe_warm:
         probe_warm(lm, args.steps, args.warmup)

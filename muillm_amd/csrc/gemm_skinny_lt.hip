@@ -44,7 +44,7 @@ constexpr int kLtXLoads = 8;                 // load instructions per 16-row til
 // used (any group size >= 16). A load inside the multiply phase is the youngest one outstanding and
 // waiting for it waits for the prefetched pass behind which it queued (loads return in order): down
 // 4096 x 14336 at 4 tokens ran 20.7 us that way against 13.5 us with per-channel scales.
-template <typename T, int WF, bool NORM, int EPI, bool BSTAT, bool FULL, bool HB, bool BIGP, int GP = 0>
+template <typename T, int WF, bool NORM, int EPI, bool BSTAT, bool FULL, bool HB, int GP = 0>
 __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
     // scalars, hottest first (the leading ones are preloaded into SGPRs at wave launch)
     const void* w0, const void* w1, long pitch, const uint16_t* x, int n, int k, int tokens, int n_tiles, int spw,
@@ -75,15 +75,12 @@ __global__ void __launch_bounds__(kLtThreads) gemm_skinny_lt_kernel(
   const u32x4 ones16 = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
   f32x4 xs_wave = {0.f, 0.f, 0.f, 0.f};  // CACC, B-stationary: sum of this wave's token operands per token column
   f32x4 xs_run = {0.f, 0.f, 0.f, 0.f};   // CACC, streaming: the same over the passes of the current tile
-  // k-values per wave and pass: 256 (512 bytes of a 16-bit row). Per-channel int8 weights in
-  // B-stationary mode can take 512 (BIGP), so that a pass again covers 512 contiguous bytes of
-  // each row and a load instruction two rows of them: with 256-byte runs and half the bytes in
-  // flight the int8 gate/up shape (7 tiles per workgroup) ran 33.7 us, with 512 it runs 27.9 us.
-  // With one or two tiles per workgroup the finer passes overlap better (QKV 8.9 vs 10.8 us), so
-  // the launcher picks by tiles per workgroup. (The group format stays at 256: its scale
-  // operands do not fit the register file beside the larger pass.)
-  constexpr int SUB = BIGP ? 2 * kLtSub : kLtSub;
-  static_assert(!BIGP || (BSTAT && WF == WF_I8_CHANNEL), "large passes: per-channel int8, B-stationary");
+  // k-values per wave and pass: 256 (512 bytes of a 16-bit row, 256 of an 8-bit one). (Passes of 512
+  // codes for per-channel int8 -- 512 contiguous bytes per row again -- were ahead while the codes
+  // were converted with a packed subtract per pair; with the offset taken off the finished sums
+  // instead the finer passes win on every shape: gate/up 2 x 14336 x 4096 at 4 / 8 / 16 tokens 22.7 /
+  // 23.4 / 25.4 us against 26.5 / 27.2 / 28.8 us.)
+  constexpr int SUB = kLtSub;
   constexpr int STEPS = SUB / 32;                // MFMAs per pass
   constexpr int PB = 2 * kLtSub / SUB;           // B-stationary: passes per tile (2 or 1)
   constexpr int ROWB = SUB * WB;                 // bytes of a row segment of one pass
@@ -527,35 +524,27 @@ static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
   constexpr int OUT = (EPI == SK_GATEUP) ? 8 : 16;
   const int n_tiles = ceil_div(p.n, OUT);
   const int grid = balanced_grid(n_tiles, 1);  // ~150 KB of LDS: one workgroup per CU
-#define MUI_LT_G(NORMV, BSTATV, FULLV, HBV, BIGV, GPV, SPW)                                                           \
-  hipLaunchKernelGGL((gemm_skinny_lt_kernel<T, WF, NORMV, EPI, BSTATV, FULLV, HBV, BIGV, GPV>), dim3(grid),           \
+#define MUI_LT_G(NORMV, BSTATV, FULLV, HBV, GPV, SPW)                                                                 \
+  hipLaunchKernelGGL((gemm_skinny_lt_kernel<T, WF, NORMV, EPI, BSTATV, FULLV, HBV, GPV>), dim3(grid),                 \
                      dim3(kLtThreads), 0, s, p.w0, p.w1, p.pitch, p.x, p.n, p.k, p.tokens, n_tiles, SPW, p.gamma, p.y, \
                      p.eps, p.residual, p.mul_bias, p.add_bias, p.s0, p.s1, p.s_pitch, p.group_shift)
   // group format: groups of 128 codes carry two (scale, min) pairs with every 256-value pass, larger
   // groups one; smaller groups load the pair of each MFMA step where it is used
-#define MUI_LT(NORMV, BSTATV, FULLV, HBV, BIGV, SPW)                                \
-  do {                                                                              \
-    if constexpr (WF == WF_U8_GROUP) {                                              \
-      if (p.group_shift == 7) MUI_LT_G(NORMV, BSTATV, FULLV, HBV, BIGV, 2, SPW);    \
-      else if (p.group_shift >= 8) MUI_LT_G(NORMV, BSTATV, FULLV, HBV, BIGV, 1, SPW); \
-      else MUI_LT_G(NORMV, BSTATV, FULLV, HBV, BIGV, 0, SPW);                       \
-    } else {                                                                        \
-      MUI_LT_G(NORMV, BSTATV, FULLV, HBV, BIGV, 0, SPW);                            \
-    }                                                                               \
+#define MUI_LT(NORMV, BSTATV, FULLV, HBV, SPW)                                \
+  do {                                                                        \
+    if constexpr (WF == WF_U8_GROUP) {                                        \
+      if (p.group_shift == 7) MUI_LT_G(NORMV, BSTATV, FULLV, HBV, 2, SPW);    \
+      else if (p.group_shift >= 8) MUI_LT_G(NORMV, BSTATV, FULLV, HBV, 1, SPW); \
+      else MUI_LT_G(NORMV, BSTATV, FULLV, HBV, 0, SPW);                       \
+    } else {                                                                  \
+      MUI_LT_G(NORMV, BSTATV, FULLV, HBV, 0, SPW);                            \
+    }                                                                         \
   } while (0)
   if (p.k <= kLtWaves * 2 * kLtSub && p.k % 256 == 0) {
     const bool full = p.k == kLtWaves * 2 * kLtSub;
     const bool hb = p.tokens <= 8;
-    const bool big = WF == WF_I8_CHANNEL && n_tiles >= 3 * grid;
-#define MUI_LT_HB(NORMV, FULLV)                                                                              \
-  {                                                                                                          \
-    if constexpr (WF == WF_I8_CHANNEL) {                                                                     \
-      if (big) { if (hb) MUI_LT(NORMV, true, FULLV, true, true, 1); else MUI_LT(NORMV, true, FULLV, false, true, 1); } \
-      else { if (hb) MUI_LT(NORMV, true, FULLV, true, false, 1); else MUI_LT(NORMV, true, FULLV, false, false, 1); }   \
-    } else {                                                                                                 \
-      if (hb) MUI_LT(NORMV, true, FULLV, true, false, 1); else MUI_LT(NORMV, true, FULLV, false, false, 1);  \
-    }                                                                                                        \
-  }
+#define MUI_LT_HB(NORMV, FULLV) \
+  { if (hb) MUI_LT(NORMV, true, FULLV, true, 1); else MUI_LT(NORMV, true, FULLV, false, 1); }
     if (p.gamma) { if (full) MUI_LT_HB(true, true) else MUI_LT_HB(true, false) }
     else { if (full) MUI_LT_HB(false, true) else MUI_LT_HB(false, false) }
 #undef MUI_LT_HB
@@ -565,8 +554,8 @@ static int launch_lt_t(hipStream_t s, const SkinnyParams& p) {
   if (p.k % (WF == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
   const int spw = ceil_div(ceil_div(p.k, kLtSub), kLtWaves);
   const bool hb = p.tokens <= 8;
-  if (p.gamma) { if (hb) MUI_LT(true, false, false, true, false, spw); else MUI_LT(true, false, false, false, false, spw); }
-  else { if (hb) MUI_LT(false, false, false, true, false, spw); else MUI_LT(false, false, false, false, false, spw); }
+  if (p.gamma) { if (hb) MUI_LT(true, false, false, true, spw); else MUI_LT(true, false, false, false, spw); }
+  else { if (hb) MUI_LT(false, false, false, true, spw); else MUI_LT(false, false, false, false, spw); }
 #undef MUI_LT
 #undef MUI_LT_G
   return launch_status();
