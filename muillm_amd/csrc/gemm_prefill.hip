@@ -369,7 +369,10 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's stores have arrived
     __syncthreads();                                    // ... and everybody's
     __shared__ unsigned xs_arrived;
-    if (t == 0) xs_arrived = __hip_atomic_fetch_add(&p.part_count[xs_tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // release (everybody's partial tile, ordered before this thread by the barrier, is visible
+    // device-wide before the count goes up) and acquire (the workgroup that sees the full count sees
+    // every tile): the ordering the memory model gives, not one chip's write acknowledgements
+    if (t == 0) xs_arrived = __hip_atomic_fetch_add(&p.part_count[xs_tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (xs_arrived + 1 != (unsigned)p.k_splits) return;  // uniform: somebody else finishes the tile
 #pragma unroll

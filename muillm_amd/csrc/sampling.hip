@@ -182,8 +182,10 @@ __global__ void __launch_bounds__(kArgmaxThreads) greedy_advance_parts_kernel(co
       const unsigned long long key = ((unsigned long long)image << 32) | (0xffffffffu - (uint32_t)best_i);
       __hip_atomic_fetch_max(best_word + b, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the candidate has arrived before the count goes up
-    const unsigned before = __hip_atomic_fetch_add(arrived + b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // release: the candidate is visible device-wide before the count goes up; acquire: whoever sees
+    // the full count sees every candidate (the memory model's own ordering, not a property of one
+    // chip generation's write acknowledgements)
+    const unsigned before = __hip_atomic_fetch_add(arrived + b, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     last = before + 1 == (unsigned)n_parts;
     if (last) {
       const unsigned long long w = __hip_atomic_load(best_word + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -553,9 +553,24 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
 
 
 # Row-interleaved twins of gate/up buffers that arrived in the reference's per-element packing,
-# keyed by the identity and version of the source tensors (bounded: one entry per quantised MLP).
+# keyed by the address and version of the source tensors (bounded: one entry per quantised MLP).
+# An entry also holds weak references to the two source tensors' storages: a hit counts only while
+# both are alive (an address handed out again by the allocator after the first model is freed must
+# not find the first model's twin), and an entry whose sources have died is dropped.
 _REPACKED_GATEUP: "OrderedDict" = None
 _REPACKED_GATEUP_MAX = 256
+
+
+def _storage_ref(t: torch.Tensor):
+    """A callable that gives the identity (`_cdata`) of t's storage while that storage is alive and
+    None once it has been freed; holds no reference that would keep the tensor alive."""
+    import weakref
+
+    st = t.untyped_storage()
+    cdata = st._cdata
+    alive = weakref.ref(st)  # dies with the Python storage object, which t keeps alive through its base
+    holder = weakref.ref(t)
+    return lambda: cdata if (holder() is not None or alive() is not None) else None
 
 
 def _is_reference_gateup_packing(gate_up_weights: torch.Tensor) -> bool:
@@ -592,13 +607,18 @@ def _row_interleaved_gateup(gate_up_weights: torch.Tensor, gate_up_scales_min_va
     key = (w.data_ptr(), smv.data_ptr(), w._version, smv._version, n, k, int(group_size_shift), smv.dtype)
     hit = _REPACKED_GATEUP.get(key)
     if hit is not None:
-        _REPACKED_GATEUP.move_to_end(key)
-        return hit
+        out_w, out_smv, w_ref, smv_ref = hit
+        if w_ref() == w.untyped_storage()._cdata and smv_ref() == smv.untyped_storage()._cdata:
+            _REPACKED_GATEUP.move_to_end(key)
+            return out_w, out_smv
+        del _REPACKED_GATEUP[key]  # same address, other (or dead) storage: a stale twin
+    for stale in [kk for kk, v in _REPACKED_GATEUP.items() if v[2]() is None or v[3]() is None]:
+        del _REPACKED_GATEUP[stale]
     out_w = torch.empty((n, 2, k), dtype=torch.uint8, device=w.device)
     out_smv = torch.empty((n, 2, g, 2), dtype=smv.dtype, device=smv.device)
     check(_lib.load().mui_int8_repack_gateup(_stream(w), w.data_ptr(), smv.data_ptr(), int(group_size_shift),
                                              out_w.data_ptr(), out_smv.data_ptr(), n, k), "mui_int8_repack_gateup")
-    _REPACKED_GATEUP[key] = (out_w, out_smv)
+    _REPACKED_GATEUP[key] = (out_w, out_smv, _storage_ref(w), _storage_ref(smv))
     while len(_REPACKED_GATEUP) > _REPACKED_GATEUP_MAX:
         _REPACKED_GATEUP.popitem(last=False)
     return out_w, out_smv

@@ -24,11 +24,9 @@ _INT8_LAYER_REPLACEMENTS = {
 
 
 def _recursive_setattr(model: nn.Module, module_name: str, new_module: nn.Module):
-    split_list = module_name.split(".")
-    current_module = model
-    for name in split_list[:-1]:
-        current_module = getattr(current_module, name)
-    current_module.__setattr__(split_list[-1], new_module)
+    """Put new_module where the dotted name points (the parent is found through get_submodule)."""
+    parent_name, _, leaf = module_name.rpartition(".")
+    setattr(model.get_submodule(parent_name) if parent_name else model, leaf, new_module)
 
 
 def _module_name_matches(module_name: str, modules: List[str]) -> bool:
