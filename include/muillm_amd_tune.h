@@ -1,6 +1,7 @@
 /*
  * muillm_amd_tune.h -- measurement aids of libmuillm_amd.so, kept apart from the product ABI
- * (muillm_amd.h), whose entry points are stateless.
+ * (muillm_amd.h), whose entry points are stateless once mui_tune_lock() has been called (or in a
+ * process that never calls anything declared here).
  *
  * The mui_tune_* calls set PROCESS-GLOBAL launch-shape overrides that the product entry points
  * read at launch time; they are for benchmark sweeps and for tests that pin one kernel variant,
@@ -17,6 +18,12 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+
+/* One-way switch: after this call every mui_tune_* call returns MUI_ERR_UNSUPPORTED and changes
+ * nothing, for the rest of the process. A deployment calls it once after start-up, so that the
+ * product entry points behave as the stateless functions muillm_amd.h describes whatever else is
+ * loaded into the process. */
+int mui_tune_lock(void);
 
 /* Launch-shape knobs (0 restores the built-in choice). */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);

@@ -96,6 +96,7 @@ _SIGNATURES = {
     "mui_decoder_stack_workspace_bytes": (ctypes.c_size_t, [_P, c_int, c_int]),
     "mui_decoder_stack_step": (c_int, [_P, _P, c_int, _P, _P, _P, c_long, _P, c_int, _P, c_long, c_int, _P]),
     "mui_probe_read": (c_int, [_P, _P, ctypes.c_uint64, _P]),
+    "mui_tune_lock": (c_int, []),
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_packed_dot": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),

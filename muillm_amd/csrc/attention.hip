@@ -1536,12 +1536,14 @@ static int g_attn_min_tokens = 0;  // 0: built-in choice; else fewest tokens wor
 static int g_prefill_group_tokens = 0;
 
 extern "C" int mui_tune_prefill_attention(int group_kernel_min_tokens) {
+  MUI_TUNE_GUARD();
   g_prefill_group_tokens = group_kernel_min_tokens;
   return MUI_OK;
 }
 
 extern "C" int mui_tune_attention(int waves_per_workgroup, int min_tokens_per_split, int direct_tokens,
                                   int mfma_tokens) {
+  MUI_TUNE_GUARD();
   if (!(waves_per_workgroup == 0 || waves_per_workgroup == 4 || waves_per_workgroup == 8 || waves_per_workgroup == 16))
     return MUI_ERR_INVALID_ARG;
   if (min_tokens_per_split < 0) return MUI_ERR_INVALID_ARG;
@@ -1688,6 +1690,7 @@ static int g_warm_percent = 0;  // 0: built-in choice; share of the announced by
 static int g_warm_delay = -1;   // < 0: built-in choice; head start of the attention workgroups (s_sleep 8 units)
 
 extern "C" int mui_tune_warm(int workgroups, int percent, int delay) {
+  MUI_TUNE_GUARD();
   if (percent < 0 || percent > 100 || (workgroups > 0 && workgroups % 8 != 0) || delay > 64) return MUI_ERR_INVALID_ARG;
   g_warm_wgs = workgroups;
   g_warm_percent = percent;

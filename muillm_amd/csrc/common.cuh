@@ -229,6 +229,13 @@ __device__ __forceinline__ void warm_cache(const char* base, long bytes, int sla
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
 
 // host-side helpers ----------------------------------------------------------------------
+// true once mui_tune_lock() has been called: every mui_tune_* call is refused from then on
+bool tune_locked();
+#define MUI_TUNE_GUARD()                              \
+  do {                                                \
+    if (mui::tune_locked()) return MUI_ERR_UNSUPPORTED; \
+  } while (0)
+
 static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 

@@ -5,6 +5,21 @@
 
 #include "common.cuh"
 
+#include <atomic>
+
+namespace mui {
+static std::atomic<int> g_tune_locked{0};
+bool tune_locked() { return g_tune_locked.load(std::memory_order_relaxed) != 0; }
+}  // namespace mui
+
+// One-way switch for deployments: the launch-shape choices in force at this moment (the built-in
+// ones, unless the process has tuned) stay for the rest of the process, and no caller -- a plugin,
+// a test helper left in by accident -- can change another caller's kernels any more.
+extern "C" int mui_tune_lock(void) {
+  mui::g_tune_locked.store(1, std::memory_order_relaxed);
+  return MUI_OK;
+}
+
 extern "C" int mui_abi_version(void) { return MUI_ABI_VERSION; }
 
 extern "C" const char* mui_status_string(int status) {

@@ -699,6 +699,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 }  // namespace mui
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
+  MUI_TUNE_GUARD();
   if (tile < 0 || tile > 12 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens

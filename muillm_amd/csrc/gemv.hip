@@ -277,6 +277,7 @@ static int g_gemv_dot2 = 1;
 static int g_multi_max_tokens = 2;
 
 extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens) {
+  MUI_TUNE_GUARD();
   if (min_tokens < 1 || min_tokens > MUI_MAX_TOKENS + 1) return MUI_ERR_INVALID_ARG;
   if (multi_max_tokens < 0 || multi_max_tokens > 8) return MUI_ERR_INVALID_ARG;
   g_skinny_min_tokens = min_tokens;
@@ -288,12 +289,14 @@ extern "C" int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_token
 }
 
 extern "C" int mui_tune_packed_dot(int linear_on, int int8_on) {
+  MUI_TUNE_GUARD();
   g_gemv_dot2 = linear_on != 0;
   int8_set_packed_dot(int8_on != 0);
   return MUI_OK;
 }
 
 extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
+  MUI_TUNE_GUARD();
   if (!(rows_linear == 0 || rows_linear == 2 || rows_linear == 4)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_tune.rows_linear = rows_linear;

@@ -359,6 +359,7 @@ int int8_tuned_rows() { return g_int8_rows; }
 }  // namespace mui
 
 extern "C" int mui_tune_int8(int rows, int wgs_per_cu) {
+  MUI_TUNE_GUARD();
   if (!(rows == 0 || rows == 2 || rows == 4 || rows == 8 || rows == 16)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_int8_rows = rows;

@@ -74,3 +74,26 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_tune_lock_freezes_the_knobs():
+    """mui_tune_lock() is a one-way switch, so it is tried in a process of its own: before it the
+    knobs answer, after it every one of them refuses and nothing changes (none of them touches a
+    GPU, the library loads without one)."""
+    import subprocess
+    import sys
+
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "from muillm_amd import _lib\n"
+        "lib = _lib.load()\n"
+        "assert lib.mui_tune_gemv(4, 2) == 0 and lib.mui_tune_gemv(0, 0) == 0\n"
+        "assert lib.mui_tune_lock() == 0\n"
+        "calls = [lib.mui_tune_gemv(4, 2), lib.mui_tune_int8(8, 2), lib.mui_tune_attention(8, 0, 0, 0),\n"
+        "         lib.mui_tune_skinny(2, 0, 0), lib.mui_tune_packed_dot(1, 1), lib.mui_tune_prefill(0, 0),\n"
+        "         lib.mui_tune_prefill_attention(0), lib.mui_tune_warm(256, 100, 0)]\n"
+        "assert calls == [-2] * len(calls), calls\n"
+        "print('locked')\n"
+    ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))),)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "locked" in out.stdout, out.stderr
