@@ -33,11 +33,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the gate/up GEMV at the Llama-3-8B shape, from two `rocprofv3 --pmc` runs of
 # `bench.py --pmc-probe` (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
-# counter reads for the probe's elementwise copy of 234,881,024 B: FETCH_SIZE reads 114,706.1 for the copy
-# (x2.0000 to KiB) and 114,783.2 for the GEMV; WRITE_SIZE reads 229,376.0 for the copy (x1.0) and 224.0 for
-# the GEMV. 235,038,826 B fetched + 229,417 B written.
-GATEUP_TRAFFIC_BYTES = 235038826 + 229417
-GATEUP_TRAFFIC_SOURCE = "profiles/gateup_gemv_llama3_8b_pmc_traffic.md (rocprofv3 --pmc counter runs; not re-measured by this run)"
+# counter reads for the probe's elementwise copy of 234,881,024 B: FETCH_SIZE reads 114,706.4 for the copy
+# (x1.99968 to KiB) and 114,783.9 for the GEMV; WRITE_SIZE reads 229,376.0 for the copy (x1.0) and 224.02
+# for the GEMV. 235,039,678 B fetched + 229,396 B written.
+GATEUP_TRAFFIC_BYTES = 235039678 + 229396
+GATEUP_TRAFFIC_SOURCE = ("profiles/gateup_gemv_llama3_8b_pmc_traffic.md: rocprofv3 --pmc counter runs of 2026-11-26 on "
+                         "commit 1a733c7 (counters need profiler runs of their own; not re-measured by this run)")
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16 matrix-core peak
 BASELINE_TOKENS_PER_S = 210.0  # reference README: Llama-3-8B fp16 bs1 on 1x MI300X
 
