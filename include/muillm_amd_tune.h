@@ -32,6 +32,13 @@ int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
  * points through the packed-dot int8 kernel (default on) */
 int mui_tune_packed_dot(int linear_on, int int8_on);
 int mui_tune_int8(int rows_per_group, int workgroups_per_cu);
+/* the 4 x 4 x 4 matrix-instruction int8 kernel (fp16 activations, up to 4 tokens): on = 0 sends its
+ * shapes to the older kernels; min_tokens = fewest tokens it takes (0 = default: 2 with per-channel
+ * scales, 3 with the group format); workgroups per
+ * CU (0 = built-in); register sets = row groups in flight per workgroup: 0 = built-in choice (two
+ * where a norm is fused or a workgroup has more than two groups), 1 = one, 2 = two wherever a
+ * workgroup has more than one group */
+int mui_tune_int8_quad(int on, int min_tokens, int workgroups_per_cu, int sets);
 /* waves per attention workgroup (4, 8 = default for <= 4 query heads per KV head, 16), the
  * fewest cached tokens that justify one more sequence split (default: two passes), and the
  * longest sequence that mui_flash_decode_splits leaves unsplit at small batch (default 1536;

@@ -100,6 +100,7 @@ _SIGNATURES = {
     "mui_tune_gemv": (c_int, [c_int, c_int]),
     "mui_tune_packed_dot": (c_int, [c_int, c_int]),
     "mui_tune_int8": (c_int, [c_int, c_int]),
+    "mui_tune_int8_quad": (c_int, [c_int, c_int, c_int, c_int]),
     "mui_tune_skinny": (c_int, [c_int, c_int, c_int]),
     "mui_tune_prefill": (c_int, [c_int, c_int]),
     "mui_tune_prefill_attention": (c_int, [c_int]),

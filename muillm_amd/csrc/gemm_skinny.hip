@@ -381,7 +381,11 @@ void skinny_set_int8_multi(int on) { g_int8_multi = on; }
 
 // entry used by gemv.hip / int8.hip for tokens >= 2
 int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams& p) {
-  // int8 at up to 4 tokens: the vector-ALU kernel, except at 3-4 tokens long rows (down 4096 x
+  // int8 at 2-4 tokens with fp16 activations: the 4 x 4 x 4 matrix-instruction kernel (int8_quad.hip:
+  // QKV 6144 x 4096 at 4 tokens 7.6 us against 9.0 us on the vector ALUs, gate/up 2 x 14336 x 4096
+  // 20.5 us against 22.9 us on the kernel below). What it declines (one token, bf16, the group format
+  // up to two tokens, rows longer than 14336):
+  // the vector-ALU kernel, except at 3-4 tokens long rows (down 4096 x
   // 14336 at 4 tokens: 13.6 vs 16.4 us) and tall gate/up matrices (2 x 14336 x 4096: a steady
   // 27 us against 27-34 us), where the matrix-core kernel measured faster -- with per-channel
   // scales and, for fp16 activations, with the reference's groups of 128 codes or more, which that
@@ -390,6 +394,10 @@ int launch_skinny(hipStream_t s, int dtype, int wf, int epi, const SkinnyParams&
   const bool lt_format = wf == WF_I8_CHANNEL || (wf == WF_U8_GROUP && p.group_shift >= 7 && dtype == MUI_DTYPE_F16);
   const bool lt_first = g_skinny_lt && lt_format && p.tokens >= 3 &&
                         (p.k > 8192 || (epi == SK_GATEUP && p.n >= 8192));
+  if (wf != WF_16BIT && p.tokens <= 4) {
+    const int st = launch_int8_quad(s, dtype, wf, epi, p);
+    if (st != MUI_ERR_UNSUPPORTED) return st;
+  }
   if (wf != WF_16BIT && g_int8_multi && p.tokens <= 4 && !lt_first) {
     const int st = launch_int8_multi(s, dtype, wf, epi, p);
     if (st != MUI_ERR_UNSUPPORTED) return st;

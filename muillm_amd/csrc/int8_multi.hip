@@ -55,13 +55,18 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
     coff[j] = cvalid[j] ? (c << 4) : 0;
   }
 
-  u32x4 w[R][CH];
-  uint32_t sm[R][CH];  // group format: packed (scale, min) of the chunk's group
-  // what the epilogue thread of a group needs from memory (residual, per-channel scales) rides
-  // along with the group's weights: loaded inside the epilogue it would add a memory round trip
-  // to the end of the kernel
-  uint32_t ep_res = 0, ep_s0 = 0, ep_s1 = 0;
-  auto issue = [&](int rg) {
+  // The weights of a row group, the (scale, min) pairs of the group format, and what the epilogue
+  // thread of the group needs from memory (residual, per-channel scales): loaded inside the
+  // epilogue that would add a memory round trip to the end of the kernel. Every thread requests
+  // the epilogue values, from clamped addresses (no load behind a branch).
+  struct Set {
+    u32x4 w[R][CH];
+    uint32_t sm[R][CH];
+    uint32_t res, s0, s1;
+  };
+  const int ep_o = (t / TOK) < OUT ? t / TOK : OUT - 1;
+  const int ep_tk = (t % TOK) < tokens ? t % TOK : tokens - 1;
+  auto issue = [&](Set& st, int rg) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       int row;
@@ -80,30 +85,27 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       const uint8_t* rp = base + (long)row * pitch;
 #pragma unroll
       for (int j = 0; j < CH; ++j) {
-        w[r][j] = ld16_stream(rp + coff[j]);
+        st.w[r][j] = ld16_stream(rp + coff[j]);
         if constexpr (WF == WF_U8_GROUP)
-          sm[r][j] = ld4(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
+          st.sm[r][j] = ld4(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
       }
     }
-    if (t < OUT * TOK) {
-      const int row = rg * OUT + t / TOK, tk = t % TOK;
-      if (row < n && tk < tokens) {
-        if constexpr (WF == WF_I8_CHANNEL) {
-          ep_s0 = ld2(a.s0 + (long)row * a.s_pitch);
-          if constexpr (EPI == SK_GATEUP) ep_s1 = ld2(a.s1 + (long)row * a.s_pitch);
-        }
-        if constexpr (EPI == SK_LINEAR) {
-          if (a.residual) ep_res = ld2(a.residual + (long)tk * n + row);
-        }
-      }
+    int row = rg * OUT + ep_o;
+    row = row < n ? row : n - 1;
+    if constexpr (WF == WF_I8_CHANNEL) {
+      st.s0 = ld2(a.s0 + (long)row * a.s_pitch);
+      if constexpr (EPI == SK_GATEUP) st.s1 = ld2(a.s1 + (long)row * a.s_pitch);
     }
+    if constexpr (EPI == SK_LINEAR) st.res = ld2(a.residual ? a.residual + ((long)ep_tk * n + row) : x);
   };
   // ---- token operands: gamma * x as packed fp16, the chunk's sum of them on the side. They are
   // requested before the first weights: loads return in order, so the operand preparation (and a
   // fused norm's reduction) then overlaps the flight of the first row group instead of following
   // it (QKV with fused norm 7.5 -> 6.4 us at one token). No load sits behind a branch (clamped
   // addresses, dead lanes zeroed by selects).
-  int rg = blockIdx.x;  // the grid never exceeds the number of row groups
+  // The grid never exceeds the number of row groups; group i of this workgroup is blockIdx.x + i * gridDim.x.
+  const int n_my = (n_groups - 1 - (int)blockIdx.x) / (int)gridDim.x + 1;
+  auto group_of = [&](int i) -> int { return blockIdx.x + i * gridDim.x; };
   u32x4 xq[TOK][CH][2];
   u32x4 gq[CH][2];
 #pragma unroll
@@ -122,7 +124,8 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       for (int hf = 0; hf < 2; ++hf) gq[j][hf] = ld16(gamma + coff[j] + 8 * hf);
     }
   }
-  issue(rg);
+  Set set;
+  issue(set, group_of(0));
 
   float xsum[TOK][CH];
   float ss[TOK];
@@ -141,9 +144,12 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
         b = live ? b : zero;
         ss[tk] += live ? sq : 0.f;
         xq[tk][j][hf] = b;
-        float bf[8];
-        unpack8<T>(b, bf);
-        xsum[tk][j] += ((bf[0] + bf[1]) + (bf[2] + bf[3])) + ((bf[4] + bf[5]) + (bf[6] + bf[7]));
+        // sum of the eight operands: packed dots against (1, 1)
+        const uint32_t bw[4] = {b.x, b.y, b.z, b.w};
+        const f16x2 one2 = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          xsum[tk][j] = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, bw[d]), one2, xsum[tk][j], false);
       }
     }
   }
@@ -155,9 +161,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
     for (int j = 0; j < CH; ++j) s += xsum[tk][j];
     acc_init[tk] = -kOffset * s;
   }
-  float rs[TOK];
-#pragma unroll
-  for (int tk = 0; tk < TOK; ++tk) rs[tk] = 1.f;
+  float rsv = 1.f;  // 1 / rms of the epilogue thread's token
   if constexpr (NORM) {
 #pragma unroll
     for (int tk = 0; tk < TOK; ++tk) {
@@ -165,15 +169,16 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       if (lane == 0) red_ss[wave][tk] = s;
     }
     __syncthreads();
-#pragma unroll
-    for (int tk = 0; tk < TOK; ++tk) {
+    if (t < OUT * TOK) {
+      const int tk = t % TOK;
       const float tot = (red_ss[0][tk] + red_ss[1][tk]) + (red_ss[2][tk] + red_ss[3][tk]);
-      rs[tk] = rsqrtf(tot / (float)k + eps);
+      rsv = rsqrtf(tot / (float)k + eps);
     }
   }
 
   int buf = 0;
-  for (; rg < n_groups; rg += gridDim.x) {
+  // group `rg` out of register set `st`; REFILL: the set is requested again for group `nxt`
+  auto pass = [&](Set& st, int rg, auto refill, int nxt) {
     float acc[NH][NVH];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -183,7 +188,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
 #pragma unroll
       for (int j = 0; j < CH; ++j) {
         // 16 bytes -> 8 packed pairs (1024 + b): pairs 0..3 meet xq[..][0], pairs 4..7 meet xq[..][1]
-        const uint32_t wv[4] = {w[r][j].x ^ kFlip, w[r][j].y ^ kFlip, w[r][j].z ^ kFlip, w[r][j].w ^ kFlip};
+        const uint32_t wv[4] = {st.w[r][j].x ^ kFlip, st.w[r][j].y ^ kFlip, st.w[r][j].z ^ kFlip, st.w[r][j].w ^ kFlip};
         uint32_t pr[8];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -204,7 +209,7 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
             ar[tk] = s;
           } else {
             // w = u8 * scale + min over this chunk's group: scale * (s - 1024 xsum) + min * xsum
-            const float sc = T::lo(sm[r][j]), mn = T::hi(sm[r][j]);
+            const float sc = T::lo(st.sm[r][j]), mn = T::hi(st.sm[r][j]);
             ar[tk] = fmaf(sc, fmaf(-kOffset, xsum[tk][j], s), fmaf(mn, xsum[tk][j], ar[tk]));
           }
         }
@@ -215,9 +220,8 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
         acc[v / NVH][v % NVH] = ar[tk];
       }
     }
-    const uint32_t cur_res = ep_res, cur_s0 = ep_s0, cur_s1 = ep_s1;
-    const int nxt = rg + gridDim.x;
-    if (nxt < n_groups) issue(nxt);
+    const uint32_t cur_res = st.res, cur_s0 = st.s0, cur_s1 = st.s1;
+    if constexpr (decltype(refill)::value) issue(st, nxt);
 
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
@@ -230,9 +234,6 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       const int o = t / TOK, tk = t % TOK;
       const int row = rg * OUT + o;
       if (row < n && tk < tokens) {
-        float rsv = rs[0];
-#pragma unroll
-        for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
         auto total = [&](int r) {
           float v = 0.f;
 #pragma unroll
@@ -257,7 +258,11 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       }
     }
     buf ^= 1;
-  }
+  };
+  constexpr std::true_type kRefill{};
+  constexpr std::false_type kLast{};
+  for (int i = 0; i + 1 < n_my; ++i) pass(set, group_of(i), kRefill, group_of(i + 1));
+  pass(set, group_of(n_my - 1), kLast, 0);
 }
 
 template <int R, int CH, int EPI, int WF, int TOK>

@@ -183,6 +183,8 @@ int gemv_tuned_wgs_per_cu();  // mui_tune_gemv's workgroups-per-CU override (0 =
 // 2..4 tokens, int8 weights, fp16 activations (int8_multi.hip); same contract
 int launch_int8_multi(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 void skinny_set_int8_multi(int on);
+// 1..4 tokens, int8 weights, fp16 activations on the 4 x 4 x 4 matrix instruction (int8_quad.hip); same contract
+int launch_int8_quad(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 void int8_set_packed_dot(bool on);  // int8.hip: single fp16 token through int8_multi.hip
 
 }  // namespace mui

@@ -91,7 +91,7 @@ def test_tune_lock_freezes_the_knobs():
         "assert lib.mui_tune_lock() == 0\n"
         "calls = [lib.mui_tune_gemv(4, 2), lib.mui_tune_int8(8, 2), lib.mui_tune_attention(8, 0, 0, 0),\n"
         "         lib.mui_tune_skinny(2, 0, 0), lib.mui_tune_packed_dot(1, 1), lib.mui_tune_prefill(0, 0),\n"
-        "         lib.mui_tune_prefill_attention(0), lib.mui_tune_warm(256, 100, 0)]\n"
+        "         lib.mui_tune_prefill_attention(0), lib.mui_tune_warm(256, 100, 0), lib.mui_tune_int8_quad(1, 0, 0, 0)]\n"
         "assert calls == [-2] * len(calls), calls\n"
         "print('locked')\n"
     ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))),)

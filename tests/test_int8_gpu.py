@@ -209,6 +209,109 @@ def test_group_gateup_small_batches(n, k, gs, tokens):
     assert_parity(h, ref, 1e-2, f"int8 group gateup {n}x{k} b={tokens}", tight=9e-3)
 
 
+QUAD_SHAPES = [
+    # (n, k): one case per (waves, segments-per-wave) instance of the 4 x 4 x 4 kernel and its tails
+    (6144, 4096),   # 4 waves x 4 segments, two row groups per workgroup
+    (4096, 14336),  # 8 x 7
+    (1030, 1024),   # 4 x 1, n not a multiple of 4
+    (515, 2032),    # 4 x 2, last segment ends inside the row
+    (64, 4112),     # 8 x 4, one block past 4096
+    (9, 8192),      # 8 x 4 full
+    (3, 16),        # a single block
+    (10000, 512),   # many groups per workgroup: the loop over pairs of register sets
+]
+
+
+@pytest.mark.parametrize("sets", [0, 1, 2])
+@pytest.mark.parametrize("n,k", QUAD_SHAPES)
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4])
+def test_quad_kernel_channel_linear(n, k, tokens, sets):
+    """Per-channel int8 at 1..4 tokens on the 4 x 4 x 4 matrix-instruction kernel (forced from one
+    token; its default starts at two), with the launcher's choice of register sets, with one and with two, with and without the
+    fused norm, bias and residual -- against the oracle, and against the older kernels' output."""
+    lib = _lib.load()
+    g = _gen(31)
+    w = _mk((n, k), g, 0.02)
+    q, s = oracle.rtn_quantize_channel(w)
+    x = _mk((tokens, k), g)
+    r = _mk((tokens, n), g)
+    bias = _mk((n,), g, 0.1)
+    for norm, use_bias, use_res in [(True, False, True), (False, True, False), (True, True, True)]:
+        gamma = _mk((k,), g, 0.1, 1.0) if norm else None
+        ref = oracle.int8_channel_linear(x, q, s, gamma, 1e-5, bias if use_bias else None, r if use_res else None)
+        args = (x.to(DEV), q.to(DEV), s.to(DEV), None if gamma is None else gamma.to(DEV), 1e-5,
+                bias.to(DEV) if use_bias else None, r.to(DEV) if use_res else None)
+        _lib.check(lib.mui_tune_int8_quad(1, 1, 0, sets), "mui_tune_int8_quad")
+        try:
+            y = muillm_ext.mui_int8_channel_linear_forward(*args)
+            _lib.check(lib.mui_tune_int8_quad(0, 0, 0, 0), "mui_tune_int8_quad")
+            y_old = muillm_ext.mui_int8_channel_linear_forward(*args)
+        finally:
+            _lib.check(lib.mui_tune_int8_quad(1, 0, 0, 0), "mui_tune_int8_quad")
+        what = f"int8 channel quad {n}x{k} b={tokens} sets={sets} norm={norm} bias={use_bias} res={use_res}"
+        assert_parity(y, ref, 1e-2, what, tight=4e-3)
+        assert_parity(y, y_old.float().cpu(), 1e-2, what + " vs older kernels", tight=4e-3)
+
+
+@pytest.mark.parametrize("n,k,gs", [(6144, 4096, 128), (4096, 14336, 128), (515, 2032, 16), (64, 4224, 64),
+                                    (33, 4096, 4096), (10000, 512, 32)])
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4])
+def test_quad_kernel_group_linear(n, k, gs, tokens):
+    """The reference's group format on the same kernel: (scale, min) folded in once per lane and
+    256-code segment on separately accumulated products."""
+    lib = _lib.load()
+    g = _gen(32)
+    w = _mk((n, k), g, 0.02)
+    q, smv = oracle.rtn_quantize_group(w, gs)
+    shift = gs.bit_length() - 1
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    r = _mk((tokens, n), g)
+    ref = oracle.int8_group_linear(x, q, smv, gs, gamma, 1e-5, None, r)
+    _lib.check(lib.mui_tune_int8_quad(1, 1, 0, 0), "mui_tune_int8_quad")
+    try:
+        y = muillm_ext.muillm_int8_linear_forward(x.to(DEV), q.to(DEV), smv.to(DEV), shift, gamma.to(DEV), 1e-5,
+                                                  None, None, r.to(DEV))
+    finally:
+        _lib.check(lib.mui_tune_int8_quad(1, 0, 0, 0), "mui_tune_int8_quad")
+    assert_parity(y, ref, 1e-2, f"int8 group quad {n}x{k} gs={gs} b={tokens}", tight=4e-3)
+
+
+@pytest.mark.parametrize("fmt", ["channel", "group"])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (301, 1024), (5, 272), (2000, 8192)])
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4])
+def test_quad_kernel_gateup(n, k, tokens, fmt):
+    lib = _lib.load()
+    g = _gen(33)
+    wg, wu = _mk((n, k), g, 0.02), _mk((n, k), g, 0.02)
+    x = _mk((tokens, k), g)
+    gamma = _mk((k,), g, 0.1, 1.0)
+    _lib.check(lib.mui_tune_int8_quad(1, 1, 0, 0), "mui_tune_int8_quad")
+    try:
+        if fmt == "channel":
+            qg, sg = oracle.rtn_quantize_channel(wg)
+            qu, su = oracle.rtn_quantize_channel(wu)
+            ref = oracle.gateup_silu(x, oracle.rtn_dequantize_channel(qg, sg), oracle.rtn_dequantize_channel(qu, su), gamma, 1e-5)
+            h = muillm_ext.mui_int8_channel_gateupsilu_forward(gamma.to(DEV), 1e-5, qg.to(DEV), qu.to(DEV), sg.to(DEV),
+                                                               su.to(DEV), x.to(DEV))
+        else:
+            gs = 16 if k % 128 else 128
+            qg, smg = oracle.rtn_quantize_group(wg, gs)
+            qu, smu = oracle.rtn_quantize_group(wu, gs)
+            ng = k // gs
+            wgd = (qg.reshape(-1, gs).double() * smg[:, None, 0].double() + smg[:, None, 1].double()).reshape(n, k)
+            wud = (qu.reshape(-1, gs).double() * smu[:, None, 0].double() + smu[:, None, 1].double()).reshape(n, k)
+            ref = oracle.gateup_silu(x, wgd, wud, gamma, 1e-5)
+            packed_w = torch.stack([qg, qu], dim=1).to(DEV)
+            packed_s = torch.stack([smg.reshape(n, ng, 2), smu.reshape(n, ng, 2)], dim=1).to(DEV)
+            h = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, packed_w, packed_s, gs.bit_length() - 1,
+                                                          x.to(DEV))
+    finally:
+        _lib.check(lib.mui_tune_int8_quad(1, 0, 0, 0), "mui_tune_int8_quad")
+    assert h.shape == (tokens, n)
+    assert_parity(h, ref, 1e-2, f"int8 {fmt} gateup quad {n}x{k} b={tokens}", tight=9e-3)
+
+
 @pytest.mark.parametrize("n,k,gs", [(14336, 4096, 128), (100, 512, 32)])
 def test_group_gateup(n, k, gs):
     g = _gen(6)
