@@ -16,7 +16,7 @@
 // same instruction against a tile of ones delivers it in exactly that layout.
 //
 // A workgroup of WV waves works on groups of 4 U weight rows (U times two gate/up pairs); wave w
-// takes the 256-code segments w, w + WV, ... of the rows (Q per wave), the sixteen blocks of a wave
+// takes Q consecutive 256-code segments of the rows, the sixteen blocks of a wave
 // are added up in registers (DPP inside a row of 16 lanes, row swaps across rows) and the waves
 // through LDS. One workgroup of eight waves per CU with eight rows per group measured best on the
 // Llama-3-8B shapes: every workgroup prepares the token operands of its whole K range, so many
@@ -81,12 +81,13 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
   const int b = lane >> 2;  // block: codes 16 b .. 16 b + 15 of each 256-code segment
   const int n_groups = (n + OUT - 1) / OUT;
 
-  // segment q of this wave covers codes (q * WV + wave) * 256 .. + 255 of a row
+  // segment q of this wave covers codes (wave * Q + q) * 256 .. + 255 of a row (a contiguous span per
+  // wave: QKV 6144 x 4096 at 4 tokens 7.3 us, against 7.5 us with the waves interleaved segment by segment)
   int koff[Q];
   bool kval[Q];
 #pragma unroll
   for (int q = 0; q < Q; ++q) {
-    const int kk = (q * WV + wave) * 256 + 16 * b;
+    const int kk = (wave * Q + q) * 256 + 16 * b;
     kval[q] = kk < k;
     koff[q] = kval[q] ? kk : 0;
   }
