@@ -58,7 +58,13 @@ __device__ __forceinline__ float quad_rows_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <int WV, int Q, int U, bool NORM, int EPI, int WF, bool TWO>
+// GW (group format, groups of at least 128 codes): a wave's span of Q segments holds at most 16
+// groups, so lane 4 b + j requests the span's pair number b of its row -- one load per lane and
+// four rows -- and the pair of segment q is fetched from the lane that holds it with a
+// ds_bpermute; one load per lane and segment otherwise. (The per-segment loads doubled the
+// kernel's load instructions: gate/up 2 x 14336 x 4096 at 4 tokens 23.3 us with them, 21.3 us with
+// the pairs taken out of the timing altogether, 20.5 us with per-channel scales.)
+template <int WV, int Q, int U, bool NORM, int EPI, int WF, bool TWO, bool GW = false>
 __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
     // scalars, hottest first (preloaded into SGPRs at wave launch)
     const uint8_t* w0, const uint8_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
@@ -99,9 +105,24 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
   // longer count the loads in flight and would wait for the other set's weights as well.
   struct Set {
     u32x4 w[U][Q];
-    uint32_t sp[U][Q];
+    uint32_t sp[U][GW ? 1 : Q];
     uint32_t res, s0, s1;
   };
+  // GW: first group of this wave's span, the pair this lane requests (clamped to the row's last
+  // group), and for every segment the byte address (lane * 4) of the lane holding its pair
+  int gw_load = 0;
+  int gw_src[GW ? Q : 1] = {};
+  if constexpr (GW) {
+    const int g0 = (wave * Q * 256) >> a.group_shift;
+    const int g_last = ((k + (1 << a.group_shift) - 1) >> a.group_shift) - 1;
+    gw_load = g0 + b < g_last ? g0 + b : g_last;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      int gi = ((((wave * Q + q) * 256) + 16 * b) >> a.group_shift) - g0;
+      gi = gi < 15 ? gi : 15;
+      gw_src[q] = (4 * gi + j) * 4;
+    }
+  }
   auto issue = [&](Set& st, int rg) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -122,8 +143,9 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
 #pragma unroll
       for (int q = 0; q < Q; ++q) {
         st.w[u][q] = ld16_stream(rp + koff[q]);
-        if constexpr (GROUP) st.sp[u][q] = ld4(sbase + (long)row * a.s_pitch + 2 * (koff[q] >> a.group_shift));
+        if constexpr (GROUP && !GW) st.sp[u][q] = ld4(sbase + (long)row * a.s_pitch + 2 * (koff[q] >> a.group_shift));
       }
+      if constexpr (GW) st.sp[u][0] = ld4(sbase + (long)row * a.s_pitch + 2 * gw_load);
     }
   };
   // the epilogue's mapping: thread o * 4 + tk finishes output o of the group for token tk
@@ -258,7 +280,10 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
         }
         if constexpr (GROUP) {
           // w = u8 * scale + min over the segment's group: scale * (sum - 1024 xs) + min * xs
-          const float sc = T::lo(st.sp[u][q]), cm = fmaf(-kOffset, sc, T::hi(st.sp[u][q]));
+          uint32_t pair;
+          if constexpr (GW) pair = (uint32_t)__builtin_amdgcn_ds_bpermute(gw_src[q], (int)st.sp[u][0]);
+          else pair = st.sp[u][q];
+          const float sc = T::lo(pair), cm = fmaf(-kOffset, sc, T::hi(pair));
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[u][i] = fmaf(sc, part[i] + part1[i], fmaf(cm, xs[q][i], acc[u][i]));
         }
@@ -338,8 +363,9 @@ static int g_i8q_on = 1;       // mui_tune_int8_quad: 0 sends 2..4 tokens to the
 static int g_i8q_min_tokens = 0;  // 0: two tokens with per-channel scales, three with the group format
 static int g_i8q_per_cu = 0;   // workgroups per CU, 0 = built-in
 static int g_i8q_sets = 0;     // 1: one register set everywhere
+static int g_i8q_wide_pairs = 1;  // group format: one (scale, min) load per lane and four rows where groups allow
 
-template <int WV, int Q, int U, int EPI, int WF>
+template <int WV, int Q, int U, int EPI, int WF, bool GW = false>
 static int launch_i8q_wq(hipStream_t s, const SkinnyParams& p) {
   constexpr int OUT = ((EPI == SK_GATEUP) ? 2 : 4) * U;
   Int8QuadArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual,
@@ -352,10 +378,10 @@ static int launch_i8q_wq(hipStream_t s, const SkinnyParams& p) {
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kernel, WV * kWave, 0) != hipSuccess || nb < 1) nb = 1;
     return nb;
   };
-  static const int res_two[2] = {resident(int8_quad_kernel<WV, Q, U, false, EPI, WF, true>),
-                                 resident(int8_quad_kernel<WV, Q, U, true, EPI, WF, true>)};
-  static const int res_one[2] = {resident(int8_quad_kernel<WV, Q, U, false, EPI, WF, false>),
-                                 resident(int8_quad_kernel<WV, Q, U, true, EPI, WF, false>)};
+  static const int res_two[2] = {resident(int8_quad_kernel<WV, Q, U, false, EPI, WF, true, GW>),
+                                 resident(int8_quad_kernel<WV, Q, U, true, EPI, WF, true, GW>)};
+  static const int res_one[2] = {resident(int8_quad_kernel<WV, Q, U, false, EPI, WF, false, GW>),
+                                 resident(int8_quad_kernel<WV, Q, U, true, EPI, WF, false, GW>)};
   const int want = g_i8q_per_cu > 0 ? g_i8q_per_cu : (WV == 4 ? 3 : 1);
   const int nm = p.gamma ? 1 : 0;
   // Two register sets where workgroups have more than one group (a ragged grid's last ones may have
@@ -374,7 +400,7 @@ static int launch_i8q_wq(hipStream_t s, const SkinnyParams& p) {
     grid = balanced_grid(n_groups, per_cu);
   }
 #define MUI_I8Q_LAUNCH(NORMV, TWOV)                                                                             \
-  hipLaunchKernelGGL((int8_quad_kernel<WV, Q, U, NORMV, EPI, WF, TWOV>), dim3(grid), dim3(WV* kWave), 0, s,         \
+  hipLaunchKernelGGL((int8_quad_kernel<WV, Q, U, NORMV, EPI, WF, TWOV, GW>), dim3(grid), dim3(WV* kWave), 0, s,         \
                      (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k, p.tokens, \
                      p.eps, a)
   if (two) { if (p.gamma) MUI_I8Q_LAUNCH(true, true); else MUI_I8Q_LAUNCH(false, true); }
@@ -386,6 +412,16 @@ static int launch_i8q_wq(hipStream_t s, const SkinnyParams& p) {
 template <int EPI, int WF>
 static int launch_i8q_t(hipStream_t s, const SkinnyParams& p) {
   const int segs = ceil_div(p.k, 256);
+  if constexpr (WF == WF_U8_GROUP) {
+    if (p.group_shift >= 7 && g_i8q_wide_pairs) {
+      if (segs <= 4) return launch_i8q_wq<4, 1, 2, EPI, WF, true>(s, p);
+      if (segs <= 8) return launch_i8q_wq<8, 1, 2, EPI, WF, true>(s, p);
+      if (segs <= 16) return launch_i8q_wq<8, 2, 2, EPI, WF, true>(s, p);
+      if (segs <= 32) return launch_i8q_wq<8, 4, 1, EPI, WF, true>(s, p);
+      if (segs <= 56) return launch_i8q_wq<8, 7, 1, EPI, WF, true>(s, p);
+      return MUI_ERR_UNSUPPORTED;
+    }
+  }
   if (segs <= 4) return launch_i8q_wq<4, 1, 2, EPI, WF>(s, p);
   if (segs <= 8) return launch_i8q_wq<8, 1, 2, EPI, WF>(s, p);
   if (segs <= 16) return launch_i8q_wq<8, 2, 2, EPI, WF>(s, p);
