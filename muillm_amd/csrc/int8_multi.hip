@@ -21,14 +21,18 @@ constexpr int kI8mWaves = kI8mThreads / kWave;
 
 struct Int8MultiArgs {
   const uint16_t* s0; const uint16_t* s1; long s_pitch; int group_shift;
-  const uint16_t* add_bias; const uint16_t* residual; long x_pitch;
+  const uint16_t* add_bias; const uint16_t* residual;
 };
 
 template <int R, int CH, bool NORM, int EPI, int WF, int TOK>
 __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
-    // scalars, hottest first (preloaded into SGPRs at wave launch)
-    const uint8_t* w0, const uint8_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
-    uint16_t* y, int n, int k, int tokens, float eps, const Int8MultiArgs a) {
+    // The first 14 dwords arrive in SGPRs at wave launch, the rest through scalar loads: everything
+    // the addresses of the token rows and of the first weights are made of is among the former, and
+    // nothing that needs the latter is allowed in front of those loads (sched_barrier below) --
+    // with `tokens`, the bias pointers or the grid size consumed early, the compiler put the wait
+    // for the scalar loads in front of the first vector load (QKV 6144 x 4096 and o_proj at one token).
+    const uint8_t* w0, const uint8_t* w1, const uint16_t* x, const uint16_t* gamma, int pitch, int n, int k,
+    int tokens, int x_pitch, uint16_t* y, float eps, const Int8MultiArgs a) {
   using T = F16;
   constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
   constexpr int NV = R * TOK;             // partial sums per row group
@@ -66,28 +70,42 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
   };
   const int ep_o = (t / TOK) < OUT ? t / TOK : OUT - 1;
   const int ep_tk = (t % TOK) < tokens ? t % TOK : tokens - 1;
-  auto issue = [&](Set& st, int rg) {
+  auto issue_w = [&](Set& st, int rg) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       int row;
       const uint8_t* base;
-      const uint16_t* sbase;
       if constexpr (EPI == SK_GATEUP) {
         row = rg * OUT + (r >> 1);
         base = (r & 1) ? w1 : w0;
-        sbase = (r & 1) ? a.s1 : a.s0;
       } else {
         row = rg * R + r;
         base = w0;
-        sbase = a.s0;
       }
       row = row < n ? row : n - 1;
       const uint8_t* rp = base + (long)row * pitch;
 #pragma unroll
-      for (int j = 0; j < CH; ++j) {
-        st.w[r][j] = ld16_stream(rp + coff[j]);
-        if constexpr (WF == WF_U8_GROUP)
-          st.sm[r][j] = ld4(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
+      for (int j = 0; j < CH; ++j) st.w[r][j] = ld16_stream(rp + coff[j]);
+    }
+  };
+  // the group format's (scale, min) pairs and the epilogue's values: their addresses need scalars
+  // that are not preloaded
+  auto issue_rest = [&](Set& st, int rg) {
+    if constexpr (WF == WF_U8_GROUP) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        int row;
+        const uint16_t* sbase;
+        if constexpr (EPI == SK_GATEUP) {
+          row = rg * OUT + (r >> 1);
+          sbase = (r & 1) ? a.s1 : a.s0;
+        } else {
+          row = rg * R + r;
+          sbase = a.s0;
+        }
+        row = row < n ? row : n - 1;
+#pragma unroll
+        for (int j = 0; j < CH; ++j) st.sm[r][j] = ld4(sbase + (long)row * a.s_pitch + 2 * (coff[j] >> a.group_shift));
       }
     }
     int row = rg * OUT + ep_o;
@@ -103,14 +121,11 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
   // fused norm's reduction) then overlaps the flight of the first row group instead of following
   // it (QKV with fused norm 7.5 -> 6.4 us at one token). No load sits behind a branch (clamped
   // addresses, dead lanes zeroed by selects).
-  // The grid never exceeds the number of row groups; group i of this workgroup is blockIdx.x + i * gridDim.x.
-  const int n_my = (n_groups - 1 - (int)blockIdx.x) / (int)gridDim.x + 1;
-  auto group_of = [&](int i) -> int { return blockIdx.x + i * gridDim.x; };
   u32x4 xq[TOK][CH][2];
   u32x4 gq[CH][2];
 #pragma unroll
   for (int tk = 0; tk < TOK; ++tk) {
-    const long xrow = tk == 0 ? 0 : (long)(tk < tokens ? tk : tokens - 1) * a.x_pitch;
+    const long xrow = tk == 0 ? 0 : (long)(tk < tokens ? tk : tokens - 1) * x_pitch;
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
 #pragma unroll
@@ -125,7 +140,12 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
     }
   }
   Set set;
-  issue(set, group_of(0));
+  issue_w(set, blockIdx.x);
+  __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a scalar load moves in front of the loads above
+  // The grid never exceeds the number of row groups; group i of this workgroup is blockIdx.x + i * gridDim.x.
+  const int n_my = (n_groups - 1 - (int)blockIdx.x) / (int)gridDim.x + 1;
+  auto group_of = [&](int i) -> int { return blockIdx.x + i * gridDim.x; };
+  issue_rest(set, blockIdx.x);
 
   float xsum[TOK][CH];
   float ss[TOK];
@@ -221,7 +241,10 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       }
     }
     const uint32_t cur_res = st.res, cur_s0 = st.s0, cur_s1 = st.s1;
-    if constexpr (decltype(refill)::value) issue(st, nxt);
+    if constexpr (decltype(refill)::value) {
+      issue_w(st, nxt);
+      issue_rest(st, nxt);
+    }
 
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
@@ -267,12 +290,13 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
 
 template <int R, int CH, int EPI, int WF, int TOK>
 static int launch_i8m_rc(hipStream_t s, const SkinnyParams& p, int grid) {
-  Int8MultiArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual,
-                     p.x_pitch > 0 ? p.x_pitch : (long)p.k};
+  Int8MultiArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual};
+  const long x_pitch = p.x_pitch > 0 ? p.x_pitch : (long)p.k;
+  if (p.pitch > 0x7fffffffL || x_pitch > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
 #define MUI_I8M_LAUNCH(NORMV)                                                                              \
   hipLaunchKernelGGL((int8_multi_kernel<R, CH, NORMV, EPI, WF, TOK>), dim3(grid), dim3(kI8mThreads), 0, s,  \
-                     (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k,      \
-                     p.tokens, p.eps, a)
+                     (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.x, p.gamma, (int)p.pitch, p.n, p.k,      \
+                     p.tokens, (int)x_pitch, p.y, p.eps, a)
   if (p.gamma) MUI_I8M_LAUNCH(true); else MUI_I8M_LAUNCH(false);
 #undef MUI_I8M_LAUNCH
   return launch_status();

@@ -39,7 +39,7 @@ constexpr int kDppRor8 = 0x128;
 
 struct Int8QuadArgs {
   const uint16_t* s0; const uint16_t* s1; long s_pitch; int group_shift;
-  const uint16_t* add_bias; const uint16_t* residual; long x_pitch;
+  const uint16_t* add_bias; const uint16_t* residual;
 };
 
 __device__ __forceinline__ f32x4 mfma4(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, f32x4 c) {
@@ -66,9 +66,11 @@ __device__ __forceinline__ float quad_rows_sum(float v) {
 // the pairs taken out of the timing altogether, 20.5 us with per-channel scales.)
 template <int WV, int Q, int U, bool NORM, int EPI, int WF, bool TWO, bool GW = false>
 __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
-    // scalars, hottest first (preloaded into SGPRs at wave launch)
-    const uint8_t* w0, const uint8_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
-    uint16_t* y, int n, int k, int tokens, float eps, const Int8QuadArgs a) {
+    // The first 14 dwords arrive in SGPRs at wave launch, the rest through scalar loads: everything
+    // the addresses of the token rows and of the first weights are made of is among the former, and
+    // nothing that needs the latter may move in front of those loads (sched_barrier below).
+    const uint8_t* w0, const uint8_t* w1, const uint16_t* x, const uint16_t* gamma, int pitch, int n, int k,
+    int tokens, int x_pitch, uint16_t* y, float eps, const Int8QuadArgs a) {
   using T = F16;
   constexpr int OUT4 = (EPI == SK_GATEUP) ? 2 : 4;  // outputs of four weight rows
   constexpr int OUT = OUT4 * U;                     // outputs per row group (U times four weight rows)
@@ -108,44 +110,22 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
     uint32_t sp[U][GW ? 1 : Q];
     uint32_t res, s0, s1;
   };
-  // GW: first group of this wave's span, the pair this lane requests (clamped to the row's last
-  // group), and for every segment the byte address (lane * 4) of the lane holding its pair
-  int gw_load = 0;
-  int gw_src[GW ? Q : 1] = {};
-  if constexpr (GW) {
-    const int g0 = (wave * Q * 256) >> a.group_shift;
-    const int g_last = ((k + (1 << a.group_shift) - 1) >> a.group_shift) - 1;
-    gw_load = g0 + b < g_last ? g0 + b : g_last;
-#pragma unroll
-    for (int q = 0; q < Q; ++q) {
-      int gi = ((((wave * Q + q) * 256) + 16 * b) >> a.group_shift) - g0;
-      gi = gi < 15 ? gi : 15;
-      gw_src[q] = (4 * gi + j) * 4;
-    }
-  }
-  auto issue = [&](Set& st, int rg) {
+  auto issue_w = [&](Set& st, int rg) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int row;
       const uint8_t* base;
-      const uint16_t* sbase;
       if constexpr (EPI == SK_GATEUP) {
         row = rg * OUT + u * OUT4 + (j >> 1);
         base = (j & 1) ? w1 : w0;
-        sbase = (j & 1) ? a.s1 : a.s0;
       } else {
         row = rg * OUT + u * OUT4 + j;
         base = w0;
-        sbase = a.s0;
       }
       row = row < n ? row : n - 1;
       const uint8_t* rp = base + (long)row * pitch;
 #pragma unroll
-      for (int q = 0; q < Q; ++q) {
-        st.w[u][q] = ld16_stream(rp + koff[q]);
-        if constexpr (GROUP && !GW) st.sp[u][q] = ld4(sbase + (long)row * a.s_pitch + 2 * (koff[q] >> a.group_shift));
-      }
-      if constexpr (GW) st.sp[u][0] = ld4(sbase + (long)row * a.s_pitch + 2 * gw_load);
+      for (int q = 0; q < Q; ++q) st.w[u][q] = ld16_stream(rp + koff[q]);
     }
   };
   // the epilogue's mapping: thread o * 4 + tk finishes output o of the group for token tk
@@ -165,12 +145,9 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
   // the first weights (loads return in order: the preparation then overlaps the flight of the first
   // row group instead of following it). No load sits behind a branch (clamped addresses, dead lanes
   // zeroed by selects).
-  // The grid never exceeds the number of row groups; group i of this workgroup is blockIdx.x + i * gridDim.x.
-  const int n_my = (n_groups - 1 - (int)blockIdx.x) / (int)gridDim.x + 1;
-  auto group_of = [&](int i) -> int { return blockIdx.x + i * gridDim.x; };
   u32x4 xa[Q][2];
   {
-    const long xrow = (long)(j < tokens ? j : tokens - 1) * a.x_pitch;
+    const long xrow = (long)(j < tokens ? j : tokens - 1) * x_pitch;
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
 #pragma unroll
@@ -186,7 +163,55 @@ __global__ void __launch_bounds__(WV* kWave) int8_quad_kernel(
     }
   }
   Set sets[NSET];
-  issue(sets[0], group_of(0));
+  issue_w(sets[0], blockIdx.x);
+  __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a scalar load moves in front of the loads above
+  // The grid never exceeds the number of row groups; group i of this workgroup is blockIdx.x + i * gridDim.x.
+  const int n_my = (n_groups - 1 - (int)blockIdx.x) / (int)gridDim.x + 1;
+  auto group_of = [&](int i) -> int { return blockIdx.x + i * gridDim.x; };
+  // GW: first group of this wave's span, the pair this lane requests (clamped to the row's last
+  // group), and for every segment the byte address (lane * 4) of the lane holding its pair
+  int gw_load = 0;
+  int gw_src[GW ? Q : 1] = {};
+  if constexpr (GW) {
+    const int g0 = (wave * Q * 256) >> a.group_shift;
+    const int g_last = ((k + (1 << a.group_shift) - 1) >> a.group_shift) - 1;
+    gw_load = g0 + b < g_last ? g0 + b : g_last;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      int gi = ((((wave * Q + q) * 256) + 16 * b) >> a.group_shift) - g0;
+      gi = gi < 15 ? gi : 15;
+      gw_src[q] = (4 * gi + j) * 4;
+    }
+  }
+  // the group format's (scale, min) pairs of a row group
+  auto issue_pairs = [&](Set& st, int rg) {
+    if constexpr (GROUP) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        int row;
+        const uint16_t* sbase;
+        if constexpr (EPI == SK_GATEUP) {
+          row = rg * OUT + u * OUT4 + (j >> 1);
+          sbase = (j & 1) ? a.s1 : a.s0;
+        } else {
+          row = rg * OUT + u * OUT4 + j;
+          sbase = a.s0;
+        }
+        row = row < n ? row : n - 1;
+        if constexpr (GW) {
+          st.sp[u][0] = ld4(sbase + (long)row * a.s_pitch + 2 * gw_load);
+        } else {
+#pragma unroll
+          for (int q = 0; q < Q; ++q) st.sp[u][q] = ld4(sbase + (long)row * a.s_pitch + 2 * (koff[q] >> a.group_shift));
+        }
+      }
+    }
+  };
+  auto issue = [&](Set& st, int rg) {
+    issue_w(st, rg);
+    issue_pairs(st, rg);
+  };
+  issue_pairs(sets[0], group_of(0));
   issue_extras(sets[0], group_of(0));
   if constexpr (TWO) {
     // (a workgroup of a ragged grid that has a single group requests it twice: one group of the launch)
@@ -368,8 +393,9 @@ static int g_i8q_wide_pairs = 1;  // group format: one (scale, min) load per lan
 template <int WV, int Q, int U, int EPI, int WF, bool GW = false>
 static int launch_i8q_wq(hipStream_t s, const SkinnyParams& p) {
   constexpr int OUT = ((EPI == SK_GATEUP) ? 2 : 4) * U;
-  Int8QuadArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual,
-                    p.x_pitch > 0 ? p.x_pitch : (long)p.k};
+  Int8QuadArgs a = {p.s0, p.s1, p.s_pitch, p.group_shift, p.add_bias, p.residual};
+  const long x_pitch = p.x_pitch > 0 ? p.x_pitch : (long)p.k;
+  if (p.pitch > 0x7fffffffL || x_pitch > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
   const int n_groups = ceil_div(p.n, OUT);
   // workgroups per CU: three of four waves, two of eight -- or what the registers of the instance
   // allow, asked once per instance (a grid larger than what is resident runs its tail as a second round)
@@ -401,8 +427,8 @@ static int launch_i8q_wq(hipStream_t s, const SkinnyParams& p) {
   }
 #define MUI_I8Q_LAUNCH(NORMV, TWOV)                                                                             \
   hipLaunchKernelGGL((int8_quad_kernel<WV, Q, U, NORMV, EPI, WF, TWOV, GW>), dim3(grid), dim3(WV* kWave), 0, s,         \
-                     (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k, p.tokens, \
-                     p.eps, a)
+                     (const uint8_t*)p.w0, (const uint8_t*)p.w1, p.x, p.gamma, (int)p.pitch, p.n, p.k, p.tokens, \
+                     (int)x_pitch, p.y, p.eps, a)
   if (two) { if (p.gamma) MUI_I8Q_LAUNCH(true, true); else MUI_I8Q_LAUNCH(false, true); }
   else { if (p.gamma) MUI_I8Q_LAUNCH(true, false); else MUI_I8Q_LAUNCH(false, false); }
 #undef MUI_I8Q_LAUNCH
