@@ -184,8 +184,22 @@ __device__ __forceinline__ void attend_block(const u32x4 (&kreg)[UU], const u32x
   }
 }
 
+// The arguments in front are copies of the struct's fields: leading scalar arguments arrive in
+// SGPRs at wave launch (14 dwords), a struct only through scalar loads, and the kernel's first act
+// is a dependent load through one of them (the cache slot), which then starts together with the
+// loads of the struct instead of after them.
 template <typename T, int G, int U, int NW, bool DIRECT>
-__global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(
+    const int64_t* cache_position, const int64_t* position_ids, long pos_bs, const uint16_t* q, uint16_t* k_cache,
+    uint16_t* v_cache, const float* cos_table, const AttnParams pr) {
+  AttnParams p = pr;
+  p.cache_position = cache_position; p.position_ids = position_ids; p.pos_bs = pos_bs; p.q = q; p.k_cache = k_cache;
+  p.v_cache = v_cache; p.cos = cos_table;
+  // the two device scalars everything else waits for, requested before anything waits for the
+  // struct (their addresses are in SGPRs already)
+  const long slot_dev = cache_position ? (long)cache_position[0] : -1;
+  const long pos_dev = position_ids ? (long)position_ids[(long)blockIdx.z * pos_bs] : -1;
+  __builtin_amdgcn_sched_barrier(0);
   constexpr int kAttnThreads = NW * kWave;
   constexpr int kWorkers = NW * 4;      // DPP rows per workgroup
   constexpr bool kPipe = (NW <= 8);     // <= 2 waves per SIMD: double-buffer K/V in registers
@@ -217,10 +231,10 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(const AttnParam
   const int wk = wave * 4 + ts;
 
   const bool has_new = p.k_new != nullptr;
-  const int slot = has_new ? (int)p.cache_position[0] : -1;
+  const int slot = has_new ? (int)slot_dev : -1;
   int S = p.seq_len >= 0 ? p.seq_len : slot + 1;
   S = S < p.max_t ? S : p.max_t;
-  long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+  long pos = p.position_ids ? pos_dev : (long)(slot >= 0 ? slot : S - 1);
   pos = pos < 0 ? 0 : (pos >= p.rope_rows ? p.rope_rows - 1 : pos);  // never index past the tables
 
   constexpr int kBlock = kWorkers * U;  // tokens per workgroup iteration
@@ -1461,9 +1475,11 @@ static inline int attn_waves_for(int g) {
 template <typename T, int G, int NW>
 static void launch_attn_nw(hipStream_t s, const AttnParams& p, dim3 grid) {
   if (p.n_splits == 1)
-    hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, true>), grid, dim3(NW * kWave), 0, s, p);
+    hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, true>), grid, dim3(NW * kWave), 0, s,
+                       p.cache_position, p.position_ids, p.pos_bs, p.q, p.k_cache, p.v_cache, p.cos, p);
   else
-    hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, false>), grid, dim3(NW * kWave), 0, s, p);
+    hipLaunchKernelGGL((attn_decode_kernel<T, G, unroll_for(NW), NW, false>), grid, dim3(NW * kWave), 0, s,
+                       p.cache_position, p.position_ids, p.pos_bs, p.q, p.k_cache, p.v_cache, p.cos, p);
 }
 
 template <typename T, int G, bool MFMA_ONLY = false>
