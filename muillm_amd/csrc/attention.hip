@@ -507,7 +507,16 @@ constexpr int kMfKStride = 136;   // 16-bit elements per K tile row (256 + 16 by
 constexpr int kMfVStride = 144;   // 16-bit elements per V tile row: 288 bytes keep the transposed reads spread over the banks
 
 template <typename T, int G, int NW, bool DIRECT>
-__global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(
+    // leading copies of the struct's fields, as in attn_decode_kernel
+    const int64_t* cache_position, const int64_t* position_ids, long pos_bs, const uint16_t* q, uint16_t* k_cache,
+    uint16_t* v_cache, const float* cos_table, const AttnParams pr) {
+  AttnParams p = pr;
+  p.cache_position = cache_position; p.position_ids = position_ids; p.pos_bs = pos_bs; p.q = q; p.k_cache = k_cache;
+  p.v_cache = v_cache; p.cos = cos_table;
+  const long slot_dev = cache_position ? (long)cache_position[0] : -1;
+  const long pos_dev = position_ids ? (long)position_ids[(long)blockIdx.z * pos_bs] : -1;
+  __builtin_amdgcn_sched_barrier(0);
   constexpr int kAttnThreads = NW * kWave;
   constexpr int kBlock = NW * kMfTok;  // tokens per workgroup pass
   __shared__ __attribute__((aligned(16))) uint16_t q_lds[16][kHeadDim];
@@ -535,10 +544,10 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_mfma_kernel(const Attn
   const int i = lane & 15;
 
   const bool has_new = p.k_new != nullptr;
-  const int slot = has_new ? (int)p.cache_position[0] : -1;
+  const int slot = has_new ? (int)slot_dev : -1;
   int S = p.seq_len >= 0 ? p.seq_len : slot + 1;
   S = S < p.max_t ? S : p.max_t;
-  long pos = p.position_ids ? (long)p.position_ids[(long)b * p.pos_bs] : (long)(slot >= 0 ? slot : S - 1);
+  long pos = p.position_ids ? pos_dev : (long)(slot >= 0 ? slot : S - 1);
   pos = pos < 0 ? 0 : (pos >= p.rope_rows ? p.rope_rows - 1 : pos);  // never index past the tables
 
   int chunk = (S + p.n_splits - 1) / p.n_splits;
@@ -1493,9 +1502,11 @@ static int launch_attn_g(hipStream_t s, const AttnParams& p, int batch) {
   if (G == 1 && !mfma && p.n_splits == 1 && p.warm && p.warm_wgs > 0 && p.hq % 8 == 0) grid.y += p.warm_wgs;
   if (mfma) {
     if (p.n_splits == 1)
-      hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, true>), grid, dim3(8 * kWave), 0, s, p);
+      hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, true>), grid, dim3(8 * kWave), 0, s, p.cache_position,
+                         p.position_ids, p.pos_bs, p.q, p.k_cache, p.v_cache, p.cos, p);
     else
-      hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, false>), grid, dim3(8 * kWave), 0, s, p);
+      hipLaunchKernelGGL((attn_decode_mfma_kernel<T, G, 8, false>), grid, dim3(8 * kWave), 0, s, p.cache_position,
+                         p.position_ids, p.pos_bs, p.q, p.k_cache, p.v_cache, p.cos, p);
   } else if constexpr (MFMA_ONLY) {
     return MUI_ERR_UNSUPPORTED;
   } else if constexpr (G <= 4) {
