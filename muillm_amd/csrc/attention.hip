@@ -295,28 +295,35 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(
   if (use_mask) fetch(0, ka, va, valid_a, std::true_type{});
   else fetch(0, ka, va, valid_a, std::false_type{});
 
-  // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once) ----
-  for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
-    const int g = e / kHeadDim, d = e % kHeadDim;
-    const int head = head0 + g;
-    const uint16_t* qp = p.q + (long)b * p.q_bs + (long)head * p.q_hs;
-    const uint16_t r = T::pack(rope_elem<T>(qp, d, cos_row, sin_row));
-    q_lds[g][d] = r;
-    if (p.q_out && split == 0) p.q_out[((long)b * p.hq + head) * kHeadDim + d] = r;
-  }
-  // ---- the owner of the new slot rotates k, writes k/v to the cache and keeps them in LDS ----
-  if (owner) {
-    const long coff = (long)b * p.c_bs + (long)kvh * p.c_hs + (long)slot * p.c_ts;
-    if (t < kHeadDim) {
-      const uint16_t* kp = p.k_new + (long)b * p.k_bs + (long)kvh * p.k_hs;
-      const uint16_t r = T::pack(rope_elem<T>(kp, t, cos_row, sin_row));
-      kn_lds[t] = r;
-      if (writer) p.k_cache[coff + t] = r;
-    } else if (t < 2 * kHeadDim) {
-      const int d = t - kHeadDim;
-      const uint16_t v = p.v_new[(long)b * p.v_bs + (long)kvh * p.v_hs + d];
-      vn_lds[d] = v;
-      if (writer) p.v_cache[coff + d] = v;
+  // ---- rotate the G query heads of this KV head into LDS (16-bit, rounded once); the owner of
+  //      the new slot also rotates k, writes k/v to the cache and keeps them in LDS. One index
+  //      space over the threads (q elements, then k, then v): with 128 + 128 + 128 elements on
+  //      512 threads every element has its own thread and the three groups' loads are in flight
+  //      together, instead of the first two waves doing q and then k, one round trip after the other ----
+  {
+    constexpr int NQ = G * kHeadDim;
+    const int total = NQ + (owner ? 2 * kHeadDim : 0);
+    const long coff = (long)b * p.c_bs + (long)kvh * p.c_hs + (long)(slot >= 0 ? slot : 0) * p.c_ts;
+    for (int e = t; e < total; e += kAttnThreads) {
+      if (e < NQ) {
+        const int g = e / kHeadDim, d = e % kHeadDim;
+        const int head = head0 + g;
+        const uint16_t* qp = p.q + (long)b * p.q_bs + (long)head * p.q_hs;
+        const uint16_t r = T::pack(rope_elem<T>(qp, d, cos_row, sin_row));
+        q_lds[g][d] = r;
+        if (p.q_out && split == 0) p.q_out[((long)b * p.hq + head) * kHeadDim + d] = r;
+      } else if (e < NQ + kHeadDim) {
+        const int d = e - NQ;
+        const uint16_t* kp = p.k_new + (long)b * p.k_bs + (long)kvh * p.k_hs;
+        const uint16_t r = T::pack(rope_elem<T>(kp, d, cos_row, sin_row));
+        kn_lds[d] = r;
+        if (writer) p.k_cache[coff + d] = r;
+      } else {
+        const int d = e - NQ - kHeadDim;
+        const uint16_t v = p.v_new[(long)b * p.v_bs + (long)kvh * p.v_hs + d];
+        vn_lds[d] = v;
+        if (writer) p.v_cache[coff + d] = v;
+      }
     }
   }
   __syncthreads();
