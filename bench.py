@@ -1101,6 +1101,8 @@ def main():
     ap.add_argument("--tune-skinny", default=None, metavar="MIN_TOKENS,STREAM_B,MULTI_MAX_TOKENS",
                     help="experiment: mui_tune_skinny(...) before anything is timed (2,0,1 sends int8 weights at "
                          "2..4 tokens to the matrix-core kernel)")
+    ap.add_argument("--tune-gemv", default=None, metavar="ROWS,WGS_PER_CU",
+                    help="experiment: mui_tune_gemv(...) before anything is timed")
     ap.add_argument("--tune-int8-quad", default=None, metavar="ON,MIN_TOKENS,WGS_PER_CU,SETS",
                     help="experiment: mui_tune_int8_quad(...) before anything is timed")
     ap.add_argument("--table-int8-tokens", default="1,4", metavar="LIST",
@@ -1175,6 +1177,9 @@ def main():
 
         w, mt, dt, mf = (int(v) for v in args.tune_attention.split(","))
         _lib.check(_lib.load().mui_tune_attention(w, mt, dt, mf), "mui_tune_attention")
+    if args.tune_gemv:
+        from muillm_amd import _lib
+        _lib.check(_lib.load().mui_tune_gemv(*(int(v) for v in args.tune_gemv.split(","))), "mui_tune_gemv")
     if args.tune_int8_quad:
         from muillm_amd import _lib
         _lib.check(_lib.load().mui_tune_int8_quad(*(int(v) for v in args.tune_int8_quad.split(","))), "mui_tune_int8_quad")

@@ -26,6 +26,8 @@ extern "C" {
 int mui_tune_lock(void);
 
 /* Launch-shape knobs (0 restores the built-in choice). */
+/* rows_per_group: 0, 2 or 4; or 100 + n: the fewest row groups per workgroup from which the
+ * one-token GEMV keeps two of them in flight (built-in: 4, i.e. the lm_head; 100: never) */
 int mui_tune_gemv(int rows_per_group, int workgroups_per_cu);
 /* single-token routing: linear_on -> mui_linear (and bf16 mui_gateup_silu) through the packed-dot
  * kernel of the multi-token GEMV (default on); int8_on -> a single fp16 token of the int8 entry

@@ -297,6 +297,10 @@ extern "C" int mui_tune_packed_dot(int linear_on, int int8_on) {
 
 extern "C" int mui_tune_gemv(int rows_linear, int wgs_per_cu) {
   MUI_TUNE_GUARD();
+  if (rows_linear >= 100) {  // experiments: 100 + n = fewest row groups per workgroup for two register sets (100: never)
+    gemv_multi_set_two(rows_linear - 100);
+    rows_linear = 0;
+  }
   if (!(rows_linear == 0 || rows_linear == 2 || rows_linear == 4)) return MUI_ERR_INVALID_ARG;
   if (wgs_per_cu < 0 || wgs_per_cu > 32) return MUI_ERR_INVALID_ARG;
   g_tune.rows_linear = rows_linear;

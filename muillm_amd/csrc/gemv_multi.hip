@@ -27,7 +27,10 @@ __device__ __forceinline__ float dot2_mt<BF16>(uint32_t a, uint32_t b, float c) 
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_mt, a), __builtin_bit_cast(bf16x2_mt, b), c, false);
 }
 
-template <typename T, int R, int CH, bool NORM, int EPI, int TOK>
+// TWO (one token, work lists of several row groups per workgroup -- the lm_head): two register
+// sets; the weights of group i + 2 are requested as soon as group i has been multiplied, so a
+// workgroup always has a whole group in flight while it reduces, synchronises and stores.
+template <typename T, int R, int CH, bool NORM, int EPI, int TOK, bool TWO = false>
 __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
     // scalars, hottest first (preloaded into SGPRs at wave launch)
     const uint16_t* w0, const uint16_t* w1, long pitch, const uint16_t* x, const uint16_t* gamma,
@@ -54,9 +57,15 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
     coff[j] = cvalid[j] ? (c << 3) : 0;
   }
 
-  u32x4 w[R][CH];
-  uint32_t res_w = 0;  // residual (16-bit pattern) that belongs to the weights in w
-  auto issue = [&](int rg) {
+  constexpr int NSET = TWO ? 2 : 1;
+  struct Set {
+    u32x4 w[R][CH];
+    uint32_t res;  // residual (16-bit pattern) that belongs to the weights in w
+  };
+  Set sets[NSET];
+#pragma unroll
+  for (int u = 0; u < NSET; ++u) sets[u].res = 0;
+  auto issue_w = [&](Set& st, int rg) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       int row;
@@ -71,14 +80,24 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
       row = row < n ? row : n - 1;
       const uint16_t* rp = base + (long)row * pitch;
 #pragma unroll
-      for (int j = 0; j < CH; ++j) w[r][j] = ld16_stream(rp + coff[j]);
+      for (int j = 0; j < CH; ++j) st.w[r][j] = ld16_stream(rp + coff[j]);
     }
-    // the residual value of this group's epilogue thread rides along with the weights: loaded
-    // inside the epilogue it would add a memory round trip to the end of the kernel
+  };
+  // the residual value of a group's epilogue thread rides along with the weights: loaded inside
+  // the epilogue it would add a memory round trip to the end of the kernel. With two sets every
+  // thread requests it, from a clamped address: behind a branch the compiler could no longer count
+  // the loads in flight and would wait for the other set's weights as well.
+  auto issue_res = [&](Set& st, int rg) {
     if constexpr (EPI == SK_LINEAR) {
-      if (residual && t < OUT * TOK) {
-        const int row = rg * OUT + t / TOK, tk = t % TOK;
-        if (row < n && tk < tokens) res_w = ld2(residual + (long)tk * n + row);
+      if constexpr (TWO) {
+        int row = rg * OUT + (t / TOK < OUT ? t / TOK : OUT - 1);
+        row = row < n ? row : n - 1;
+        st.res = ld2(residual ? residual + row : x);
+      } else {
+        if (residual && t < OUT * TOK) {
+          const int row = rg * OUT + t / TOK, tk = t % TOK;
+          if (row < n && tk < tokens) st.res = ld2(residual + (long)tk * n + row);
+        }
       }
     }
   };
@@ -103,7 +122,16 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
 #pragma unroll
     for (int j = 0; j < CH; ++j) gq[j] = ld16(gamma + coff[j]);
   }
-  issue(rg);
+  issue_w(sets[0], rg);
+  issue_res(sets[0], rg);
+  // group i of this workgroup is blockIdx.x + i * gridDim.x
+  const int n_my = (n_groups - 1 - (int)blockIdx.x) / (int)gridDim.x + 1;
+  auto group_of = [&](int i) -> int { return blockIdx.x + i * gridDim.x; };
+  if constexpr (TWO) {
+    // (a workgroup of a ragged grid that has a single group requests it twice)
+    issue_w(sets[1], group_of(n_my > 1 ? 1 : 0));
+    issue_res(sets[1], group_of(n_my > 1 ? 1 : 0));
+  }
 
   float ss[TOK];
 #pragma unroll
@@ -137,7 +165,9 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
   }
 
   int buf = 0;
-  for (; rg < n_groups; rg += gridDim.x) {
+  // group `g` out of register set `st`; refill: the set is requested again for group `nxt` (its
+  // weights once this group has been multiplied, the residual once the epilogue has used it)
+  auto pass = [&](Set& st, int g, auto refill, int nxt) {
     float acc[NV];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -146,17 +176,19 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
         float a = 0.f;
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-          a = dot2_mt<T>(w[r][j].x, xq[tk][j].x, a);
-          a = dot2_mt<T>(w[r][j].y, xq[tk][j].y, a);
-          a = dot2_mt<T>(w[r][j].z, xq[tk][j].z, a);
-          a = dot2_mt<T>(w[r][j].w, xq[tk][j].w, a);
+          a = dot2_mt<T>(st.w[r][j].x, xq[tk][j].x, a);
+          a = dot2_mt<T>(st.w[r][j].y, xq[tk][j].y, a);
+          a = dot2_mt<T>(st.w[r][j].z, xq[tk][j].z, a);
+          a = dot2_mt<T>(st.w[r][j].w, xq[tk][j].w, a);
         }
         acc[r * TOK + tk] = a;
       }
     }
-    const uint32_t res_cur = res_w;
-    const int nxt = rg + gridDim.x;
-    if (nxt < n_groups) issue(nxt);  // keep the memory pipe full during the reduction
+    const uint32_t res_cur = st.res;
+    if constexpr (decltype(refill)::value) {
+      issue_w(st, nxt);  // keep the memory pipe full during the reduction
+      if constexpr (!TWO) issue_res(st, nxt);
+    }
 
     // all NV sums of a 16-lane row in one multi-value DPP reduction; the 16 row partials
     // (4 waves x 4 rows) are added by the epilogue threads
@@ -166,7 +198,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
 
     if (t < OUT * TOK) {
       const int o = t / TOK, tk = t % TOK;
-      const int row = rg * OUT + o;
+      const int row = g * OUT + o;
       if (row < n && tk < tokens) {
         float rsv = rs[0];
 #pragma unroll
@@ -184,22 +216,57 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
           v = total(o);
           if (mul_bias) v *= T::one(mul_bias[row]);
           if (add_bias) v += T::one(add_bias[row]);
-          if (residual) v += T::one((uint16_t)res_cur);
+          if (residual) v += T::one((uint16_t)(TWO ? st.res : res_cur));
         }
         y[(long)tk * n + row] = T::pack(v);
       }
     }
+    if constexpr (TWO && decltype(refill)::value) issue_res(st, nxt);
     buf ^= 1;
+  };
+  constexpr std::true_type kRefill{};
+  constexpr std::false_type kLast{};
+  if constexpr (!TWO) {
+    for (int i = 0; i + 1 < n_my; ++i) pass(sets[0], group_of(i), kRefill, group_of(i + 1));
+    pass(sets[0], group_of(n_my - 1), kLast, 0);
+  } else {
+    // pairs of groups whose sets are both refilled, then the last one to three groups
+    int i = 0;
+    for (; i + 3 < n_my; i += 2) {
+      pass(sets[0], group_of(i), kRefill, group_of(i + 2));
+      pass(sets[1], group_of(i + 1), kRefill, group_of(i + 3));
+    }
+    const int rem = n_my - i;
+    if (rem == 3) {
+      pass(sets[0], group_of(i), kRefill, group_of(i + 2));
+      pass(sets[1], group_of(i + 1), kLast, 0);
+      pass(sets[0], group_of(i + 2), kLast, 0);
+    } else if (rem == 2) {
+      pass(sets[0], group_of(i), kLast, 0);
+      pass(sets[1], group_of(i + 1), kLast, 0);
+    } else {
+      pass(sets[0], group_of(i), kLast, 0);
+    }
   }
 }
 
+static int g_mt_two_min_passes = 4;  // fewest row groups per workgroup that take two register sets (0: never)
+void gemv_multi_set_two(int min_passes) { g_mt_two_min_passes = min_passes; }
+
 template <typename T, int R, int CH, int EPI, int TOK>
 static int launch_mt_rc(hipStream_t s, const SkinnyParams& p, int grid) {
-#define MUI_MT_LAUNCH(NORMV)                                                                                   \
-  hipLaunchKernelGGL((gemv_multi_kernel<T, R, CH, NORMV, EPI, TOK>), dim3(grid), dim3(kMtThreads), 0, s,        \
+#define MUI_MT_LAUNCH(NORMV, TWOV)                                                                              \
+  hipLaunchKernelGGL((gemv_multi_kernel<T, R, CH, NORMV, EPI, TOK, TWOV>), dim3(grid), dim3(kMtThreads), 0, s,  \
                      (const uint16_t*)p.w0, (const uint16_t*)p.w1, p.pitch, p.x, p.gamma, p.y, p.n, p.k,        \
                      p.tokens, (int)(p.x_pitch > 0 ? p.x_pitch : (long)p.k), p.eps, p.residual, p.mul_bias, p.add_bias)
-  if (p.gamma) MUI_MT_LAUNCH(true); else MUI_MT_LAUNCH(false);
+  if constexpr (TOK == 1 && CH <= 2 && EPI == SK_LINEAR) {
+    constexpr int OUT = R;
+    if (g_mt_two_min_passes > 0 && ceil_div(p.n, OUT) >= (long)g_mt_two_min_passes * grid) {
+      if (p.gamma) MUI_MT_LAUNCH(true, true); else MUI_MT_LAUNCH(false, true);
+      return launch_status();
+    }
+  }
+  if (p.gamma) MUI_MT_LAUNCH(true, false); else MUI_MT_LAUNCH(false, false);
 #undef MUI_MT_LAUNCH
   return launch_status();
 }

@@ -174,6 +174,7 @@ void skinny_set_lt(int on);  // 0: operands loaded straight from HBM in MFMA ord
 // 1..8 tokens, 16-bit weights: the single-token GEMV structure with the token operands packed
 // in registers (gemv_multi.hip); returns MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_gemv_multi(hipStream_t s, int dtype, int epilogue, const SkinnyParams& p);
+void gemv_multi_set_two(int min_passes);  // fewest row groups per workgroup for its two-set variant (0: never)
 // MFMA skinny GEMM whose weight rows are read as contiguous runs and turned into operands
 // through wave-private LDS (gemm_skinny_lt.hip); MUI_ERR_UNSUPPORTED for shapes it does not cover
 int launch_skinny_lt(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
