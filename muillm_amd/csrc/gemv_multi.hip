@@ -165,71 +165,126 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
   }
 
   int buf = 0;
-  // group `g` out of register set `st`; refill: the set is requested again for group `nxt` (its
-  // weights once this group has been multiplied, the residual once the epilogue has used it)
-  auto pass = [&](Set& st, int g, auto refill, int nxt) {
-    float acc[NV];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-#pragma unroll
-      for (int tk = 0; tk < TOK; ++tk) {
-        float a = 0.f;
-#pragma unroll
-        for (int j = 0; j < CH; ++j) {
-          a = dot2_mt<T>(st.w[r][j].x, xq[tk][j].x, a);
-          a = dot2_mt<T>(st.w[r][j].y, xq[tk][j].y, a);
-          a = dot2_mt<T>(st.w[r][j].z, xq[tk][j].z, a);
-          a = dot2_mt<T>(st.w[r][j].w, xq[tk][j].w, a);
-        }
-        acc[r * TOK + tk] = a;
-      }
-    }
-    const uint32_t res_cur = st.res;
-    if constexpr (decltype(refill)::value) {
-      issue_w(st, nxt);  // keep the memory pipe full during the reduction
-      if constexpr (!TWO) issue_res(st, nxt);
-    }
-
-    // all NV sums of a 16-lane row in one multi-value DPP reduction; the 16 row partials
-    // (4 waves x 4 rows) are added by the epilogue threads
-    row16_reduce_scatter<NV>(acc, lane);
-    if ((lane & (16 / NV - 1)) == 0 || NV == 16) red[buf][t >> 4][(lane & 15) / (16 / NV)] = acc[0];
-    __syncthreads();
-
-    if (t < OUT * TOK) {
-      const int o = t / TOK, tk = t % TOK;
-      const int row = g * OUT + o;
-      if (row < n && tk < tokens) {
-        float rsv = rs[0];
-#pragma unroll
-        for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
-        auto total = [&](int r) {
-          float v = 0.f;
-#pragma unroll
-          for (int q = 0; q < kMtWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
-          return v * rsv;
-        };
-        float v;
-        if constexpr (EPI == SK_GATEUP) {
-          v = silu_f32(total(2 * o)) * total(2 * o + 1);
-        } else {
-          v = total(o);
-          if (mul_bias) v *= T::one(mul_bias[row]);
-          if (add_bias) v += T::one(add_bias[row]);
-          if (residual) v += T::one((uint16_t)(TWO ? st.res : res_cur));
-        }
-        y[(long)tk * n + row] = T::pack(v);
-      }
-    }
-    if constexpr (TWO && decltype(refill)::value) issue_res(st, nxt);
-    buf ^= 1;
-  };
-  constexpr std::true_type kRefill{};
-  constexpr std::false_type kLast{};
   if constexpr (!TWO) {
-    for (int i = 0; i + 1 < n_my; ++i) pass(sets[0], group_of(i), kRefill, group_of(i + 1));
-    pass(sets[0], group_of(n_my - 1), kLast, 0);
+    // one register set: the next group is requested behind a (uniform) branch once the current one
+    // has been multiplied. (Requested unconditionally, with the last pass peeled, the compiler gave
+    // the refilled weights registers of their own and copied them back at the top of the loop: the
+    // MLP at 2 tokens went from 56.6 to 70 us.)
+    for (; rg < n_groups; rg += gridDim.x) {
+      float acc[NV];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int tk = 0; tk < TOK; ++tk) {
+          float a = 0.f;
+#pragma unroll
+          for (int j = 0; j < CH; ++j) {
+            a = dot2_mt<T>(sets[0].w[r][j].x, xq[tk][j].x, a);
+            a = dot2_mt<T>(sets[0].w[r][j].y, xq[tk][j].y, a);
+            a = dot2_mt<T>(sets[0].w[r][j].z, xq[tk][j].z, a);
+            a = dot2_mt<T>(sets[0].w[r][j].w, xq[tk][j].w, a);
+          }
+          acc[r * TOK + tk] = a;
+        }
+      }
+      const uint32_t res_cur = sets[0].res;
+      const int nxt = rg + gridDim.x;
+      if (nxt < n_groups) {  // keep the memory pipe full during the reduction
+        issue_w(sets[0], nxt);
+        issue_res(sets[0], nxt);
+      }
+
+      // all NV sums of a 16-lane row in one multi-value DPP reduction; the 16 row partials
+      // (4 waves x 4 rows) are added by the epilogue threads
+      row16_reduce_scatter<NV>(acc, lane);
+      if ((lane & (16 / NV - 1)) == 0 || NV == 16) red[buf][t >> 4][(lane & 15) / (16 / NV)] = acc[0];
+      __syncthreads();
+
+      if (t < OUT * TOK) {
+        const int o = t / TOK, tk = t % TOK;
+        const int row = rg * OUT + o;
+        if (row < n && tk < tokens) {
+          float rsv = rs[0];
+#pragma unroll
+          for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
+          auto total = [&](int r) {
+            float v = 0.f;
+#pragma unroll
+            for (int q = 0; q < kMtWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
+            return v * rsv;
+          };
+          float v;
+          if constexpr (EPI == SK_GATEUP) {
+            v = silu_f32(total(2 * o)) * total(2 * o + 1);
+          } else {
+            v = total(o);
+            if (mul_bias) v *= T::one(mul_bias[row]);
+            if (add_bias) v += T::one(add_bias[row]);
+            if (residual) v += T::one((uint16_t)res_cur);
+          }
+          y[(long)tk * n + row] = T::pack(v);
+        }
+      }
+      buf ^= 1;
+    }
   } else {
+    // group `g` out of register set `st`; refill: the set is requested again for group `nxt` (its
+    // weights once this group has been multiplied, the residual once the epilogue has used it)
+    auto pass = [&](Set& st, int g, auto refill, int nxt) {
+      float acc[NV];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int tk = 0; tk < TOK; ++tk) {
+          float a = 0.f;
+#pragma unroll
+          for (int j = 0; j < CH; ++j) {
+            a = dot2_mt<T>(st.w[r][j].x, xq[tk][j].x, a);
+            a = dot2_mt<T>(st.w[r][j].y, xq[tk][j].y, a);
+            a = dot2_mt<T>(st.w[r][j].z, xq[tk][j].z, a);
+            a = dot2_mt<T>(st.w[r][j].w, xq[tk][j].w, a);
+          }
+          acc[r * TOK + tk] = a;
+        }
+      }
+      if constexpr (decltype(refill)::value) issue_w(st, nxt);  // keep the memory pipe full during the reduction
+
+      // all NV sums of a 16-lane row in one multi-value DPP reduction; the 16 row partials
+      // (4 waves x 4 rows) are added by the epilogue threads
+      row16_reduce_scatter<NV>(acc, lane);
+      if ((lane & (16 / NV - 1)) == 0 || NV == 16) red[buf][t >> 4][(lane & 15) / (16 / NV)] = acc[0];
+      __syncthreads();
+
+      if (t < OUT * TOK) {
+        const int o = t / TOK, tk = t % TOK;
+        const int row = g * OUT + o;
+        if (row < n && tk < tokens) {
+          float rsv = rs[0];
+#pragma unroll
+          for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
+          auto total = [&](int r) {
+            float v = 0.f;
+#pragma unroll
+            for (int q = 0; q < kMtWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
+            return v * rsv;
+          };
+          float v;
+          if constexpr (EPI == SK_GATEUP) {
+            v = silu_f32(total(2 * o)) * total(2 * o + 1);
+          } else {
+            v = total(o);
+            if (mul_bias) v *= T::one(mul_bias[row]);
+            if (add_bias) v += T::one(add_bias[row]);
+            if (residual) v += T::one((uint16_t)st.res);
+          }
+          y[(long)tk * n + row] = T::pack(v);
+        }
+      }
+      if constexpr (decltype(refill)::value) issue_res(st, nxt);
+      buf ^= 1;
+    };
+    constexpr std::true_type kRefill{};
+    constexpr std::false_type kLast{};
     // pairs of groups whose sets are both refilled, then the last one to three groups
     int i = 0;
     for (; i + 3 < n_my; i += 2) {
