@@ -414,27 +414,18 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(
   };
   merge_rows(std::integral_constant<int, 16>{});
   merge_rows(std::integral_constant<int, 32>{});
-  // ---- stage 2: merge the NW waves through LDS ----
-  if (lane == 0) {
-#pragma unroll
-    for (int g = 0; g < G; ++g) lds_m[wave][g] = m[g];
-  }
-  __syncthreads();
-  float f[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float mx = lds_m[0][g];
-#pragma unroll
-    for (int w2 = 1; w2 < NW; ++w2) mx = fmaxf(mx, lds_m[w2][g]);
-    const float m_use = (mx == -INFINITY) ? 0.f : mx;
-    f[g] = fast_exp2(m[g] - m_use);
-  }
+  // ---- stage 2: merge the NW waves through LDS: every wave leaves its (m, l, acc) as they are,
+  //      one barrier, and the output threads scale by 2^(m_wave - max) as they add (the products
+  //      and their order are the ones of scaling before the store, without that store's barrier) ----
   if (ts == 0) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      if (dc == 0) lds_l[wave][g] = l[g] * f[g];
-      f32x4 a0 = {acc[g][0] * f[g], acc[g][1] * f[g], acc[g][2] * f[g], acc[g][3] * f[g]};
-      f32x4 a1 = {acc[g][4] * f[g], acc[g][5] * f[g], acc[g][6] * f[g], acc[g][7] * f[g]};
+      if (dc == 0) {
+        lds_m[wave][g] = m[g];
+        lds_l[wave][g] = l[g];
+      }
+      f32x4 a0 = {acc[g][0], acc[g][1], acc[g][2], acc[g][3]};
+      f32x4 a1 = {acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
       *(f32x4*)&tile[wave][g][dc * 8] = a0;
       *(f32x4*)&tile[wave][g][dc * 8 + 4] = a1;
     }
@@ -444,12 +435,16 @@ __global__ void __launch_bounds__(NW * kWave) attn_decode_kernel(
   for (int e = t; e < G * kHeadDim; e += kAttnThreads) {
     const int g = e / kHeadDim, d = e % kHeadDim;
     const int head = head0 + g;
-    float a = 0.f, lsum = 0.f, mx = lds_m[0][g];
+    float mx = lds_m[0][g];
+#pragma unroll
+    for (int w2 = 1; w2 < NW; ++w2) mx = fmaxf(mx, lds_m[w2][g]);
+    const float m_use = (mx == -INFINITY) ? 0.f : mx;
+    float a = 0.f, lsum = 0.f;
 #pragma unroll
     for (int w2 = 0; w2 < NW; ++w2) {
-      a += tile[w2][g][d];
-      lsum += lds_l[w2][g];
-      mx = fmaxf(mx, lds_m[w2][g]);
+      const float f = fast_exp2(lds_m[w2][g] - m_use);
+      a += tile[w2][g][d] * f;
+      lsum += lds_l[w2][g] * f;
     }
     if constexpr (DIRECT) {
       p.out[((long)b * p.hq + head) * kHeadDim + d] = T::pack(lsum > 0.f ? a / lsum : 0.f);
