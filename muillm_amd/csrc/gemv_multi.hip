@@ -38,6 +38,7 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
     const uint16_t* mul_bias, const uint16_t* add_bias) {
   constexpr int OUT = (EPI == SK_GATEUP) ? R / 2 : R;
   static_assert(EPI != SK_GATEUP || (R % 2 == 0), "gate/up needs row pairs");
+  static_assert(16 * OUT * TOK <= kMtThreads, "sixteen epilogue lanes per output");
   constexpr int NV = R * TOK;  // partial sums per row group: value r * TOK + token
   __shared__ float red[2][kMtWaves * 4][NV];  // [buffer][wave * 4 + 16-lane row][value]
   __shared__ float red_ss[kMtWaves][TOK];
@@ -89,13 +90,14 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
   // the loads in flight and would wait for the other set's weights as well.
   auto issue_res = [&](Set& st, int rg) {
     if constexpr (EPI == SK_LINEAR) {
+      // (the epilogue's finishing thread of output o, token tk is thread 16 * (o * TOK + tk))
       if constexpr (TWO) {
-        int row = rg * OUT + (t / TOK < OUT ? t / TOK : OUT - 1);
+        int row = rg * OUT + ((t >> 4) / TOK < OUT ? (t >> 4) / TOK : OUT - 1);
         row = row < n ? row : n - 1;
         st.res = ld2(residual ? residual + row : x);
       } else {
-        if (residual && t < OUT * TOK) {
-          const int row = rg * OUT + t / TOK, tk = t % TOK;
+        if (residual && (t & 15) == 0 && (t >> 4) < OUT * TOK) {
+          const int row = rg * OUT + (t >> 4) / TOK, tk = (t >> 4) % TOK;
           if (row < n && tk < tokens) st.res = ld2(residual + (long)tk * n + row);
         }
       }
@@ -200,24 +202,23 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
       if ((lane & (16 / NV - 1)) == 0 || NV == 16) red[buf][t >> 4][(lane & 15) / (16 / NV)] = acc[0];
       __syncthreads();
 
-      if (t < OUT * TOK) {
-        const int o = t / TOK, tk = t % TOK;
+      // sixteen lanes per output: each fetches one of the 16 row partials, a DPP butterfly adds them
+      // (one thread adding all sixteen was a chain of sixteen dependent LDS reads at the end of the kernel)
+      if (t < 16 * OUT * TOK) {
+        const int part = t & 15, o = (t >> 4) / TOK, tk = (t >> 4) % TOK;
         const int row = rg * OUT + o;
-        if (row < n && tk < tokens) {
+        float v0 = row16_sum(red[buf][part][((EPI == SK_GATEUP) ? 2 * o : o) * TOK + tk]);
+        float v1 = 0.f;
+        if constexpr (EPI == SK_GATEUP) v1 = row16_sum(red[buf][part][(2 * o + 1) * TOK + tk]);
+        if (part == 0 && row < n && tk < tokens) {
           float rsv = rs[0];
 #pragma unroll
           for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
-          auto total = [&](int r) {
-            float v = 0.f;
-#pragma unroll
-            for (int q = 0; q < kMtWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
-            return v * rsv;
-          };
           float v;
           if constexpr (EPI == SK_GATEUP) {
-            v = silu_f32(total(2 * o)) * total(2 * o + 1);
+            v = silu_f32(v0 * rsv) * (v1 * rsv);
           } else {
-            v = total(o);
+            v = v0 * rsv;
             if (mul_bias) v *= T::one(mul_bias[row]);
             if (add_bias) v += T::one(add_bias[row]);
             if (residual) v += T::one((uint16_t)res_cur);
@@ -255,24 +256,21 @@ __global__ void __launch_bounds__(kMtThreads) gemv_multi_kernel(
       if ((lane & (16 / NV - 1)) == 0 || NV == 16) red[buf][t >> 4][(lane & 15) / (16 / NV)] = acc[0];
       __syncthreads();
 
-      if (t < OUT * TOK) {
-        const int o = t / TOK, tk = t % TOK;
+      if (t < 16 * OUT * TOK) {  // sixteen lanes per output, as above
+        const int part = t & 15, o = (t >> 4) / TOK, tk = (t >> 4) % TOK;
         const int row = g * OUT + o;
-        if (row < n && tk < tokens) {
+        float v0 = row16_sum(red[buf][part][((EPI == SK_GATEUP) ? 2 * o : o) * TOK + tk]);
+        float v1 = 0.f;
+        if constexpr (EPI == SK_GATEUP) v1 = row16_sum(red[buf][part][(2 * o + 1) * TOK + tk]);
+        if (part == 0 && row < n && tk < tokens) {
           float rsv = rs[0];
 #pragma unroll
           for (int i = 1; i < TOK; ++i) rsv = (tk == i) ? rs[i] : rsv;
-          auto total = [&](int r) {
-            float v = 0.f;
-#pragma unroll
-            for (int q = 0; q < kMtWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
-            return v * rsv;
-          };
           float v;
           if constexpr (EPI == SK_GATEUP) {
-            v = silu_f32(total(2 * o)) * total(2 * o + 1);
+            v = silu_f32(v0 * rsv) * (v1 * rsv);
           } else {
-            v = total(o);
+            v = v0 * rsv;
             if (mul_bias) v *= T::one(mul_bias[row]);
             if (add_bias) v += T::one(add_bias[row]);
             if (residual) v += T::one((uint16_t)st.res);
