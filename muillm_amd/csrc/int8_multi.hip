@@ -68,8 +68,10 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
     uint32_t sm[R][CH];
     uint32_t res, s0, s1;
   };
-  const int ep_o = (t / TOK) < OUT ? t / TOK : OUT - 1;
-  const int ep_tk = (t % TOK) < tokens ? t % TOK : tokens - 1;
+  // the epilogue gives every output sixteen lanes; lane 0 of them, thread 16 * (o * TOK + tk), finishes it
+  static_assert(16 * OUT * TOK <= kI8mThreads, "sixteen epilogue lanes per output");
+  const int ep_o = ((t >> 4) / TOK) < OUT ? (t >> 4) / TOK : OUT - 1;
+  const int ep_tk = ((t >> 4) % TOK) < tokens ? (t >> 4) % TOK : tokens - 1;
   auto issue_w = [&](Set& st, int rg) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -189,8 +191,8 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
       if (lane == 0) red_ss[wave][tk] = s;
     }
     __syncthreads();
-    if (t < OUT * TOK) {
-      const int tk = t % TOK;
+    if (t < 16 * OUT * TOK) {
+      const int tk = (t >> 4) % TOK;
       const float tot = (red_ss[0][tk] + red_ss[1][tk]) + (red_ss[2][tk] + red_ss[3][tk]);
       rsv = rsqrtf(tot / (float)k + eps);
     }
@@ -253,26 +255,25 @@ __global__ void __launch_bounds__(kI8mThreads) int8_multi_kernel(
     }
     __syncthreads();
 
-    if (t < OUT * TOK) {
-      const int o = t / TOK, tk = t % TOK;
+    // sixteen lanes per output: each fetches one of the 16 row partials, a DPP butterfly adds them
+    // (one thread adding all sixteen was a chain of sixteen dependent LDS reads at the end of the kernel)
+    if (t < 16 * OUT * TOK) {
+      const int part = t & 15, o = (t >> 4) / TOK, tk = (t >> 4) % TOK;
       const int row = rg * OUT + o;
-      if (row < n && tk < tokens) {
-        auto total = [&](int r) {
-          float v = 0.f;
-#pragma unroll
-          for (int q = 0; q < kI8mWaves * 4; ++q) v += red[buf][q][r * TOK + tk];
-          return v * rsv;
-        };
+      const float v0 = row16_sum(red[buf][part][((EPI == SK_GATEUP) ? 2 * o : o) * TOK + tk]) * rsv;
+      float v1 = 0.f;
+      if constexpr (EPI == SK_GATEUP) v1 = row16_sum(red[buf][part][(2 * o + 1) * TOK + tk]) * rsv;
+      if (part == 0 && row < n && tk < tokens) {
         float v;
         if constexpr (EPI == SK_GATEUP) {
-          float g = total(2 * o), u = total(2 * o + 1);
+          float g = v0, u = v1;
           if constexpr (WF == WF_I8_CHANNEL) {
             g *= T::one((uint16_t)cur_s0);
             u *= T::one((uint16_t)cur_s1);
           }
           v = silu_f32(g) * u;
         } else {
-          v = total(o);
+          v = v0;
           if constexpr (WF == WF_I8_CHANNEL) v *= T::one((uint16_t)cur_s0);
           if (a.add_bias) v += T::one(a.add_bias[row]);
           if (a.residual) v += T::one((uint16_t)cur_res);
