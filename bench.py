@@ -1101,6 +1101,9 @@ def main():
     ap.add_argument("--tune-skinny", default=None, metavar="MIN_TOKENS,STREAM_B,MULTI_MAX_TOKENS",
                     help="experiment: mui_tune_skinny(...) before anything is timed (2,0,1 sends int8 weights at "
                          "2..4 tokens to the matrix-core kernel)")
+    ap.add_argument("--tune-prefill", default=None, metavar="TILE,WIDE_MAX_TOKENS",
+                    help="experiment: mui_tune_prefill(...) before anything is timed (100 + tile: operand tiles staged "
+                         "through registers instead of loaded straight into LDS)")
     ap.add_argument("--tune-gemv", default=None, metavar="ROWS,WGS_PER_CU",
                     help="experiment: mui_tune_gemv(...) before anything is timed")
     ap.add_argument("--tune-int8-quad", default=None, metavar="ON,MIN_TOKENS,WGS_PER_CU,SETS",
@@ -1166,6 +1169,9 @@ def main():
     if args.probe_flash_splits:
         probe_flash_splits()
         return
+    if args.tune_prefill:
+        from muillm_amd import _lib
+        _lib.check(_lib.load().mui_tune_prefill(*(int(v) for v in args.tune_prefill.split(","))), "mui_tune_prefill")
     if args.probe_prompt or args.pmc_probe_prompt:
         probe_prompt(counters_only=args.pmc_probe_prompt)
         return

@@ -66,6 +66,8 @@ int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
  * 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 and 11 = 128 x 64 with waves that split K like 5,
  * 10 = 96 x 128 (linear only), 12 = 64 x 64 with waves that split K like 6 (linear only); shapes that a weight format or epilogue lacks fall back to the next
  * one that it has. A forced tile also keeps mui_linear_ws from sharing K between workgroups.
+ * 100 + tile: the same, and the 256 x 256 tile stages its operands through registers instead of
+ * loading them straight into LDS.
  * wide_max_tokens = longest prompt served by the weight-streaming 16-rows-per-workgroup kernel
  * instead of the LDS-tiled one (0 restores the built-in choice; at most 128; negative: never) */
 int mui_tune_prefill(int tile, int wide_max_tokens);

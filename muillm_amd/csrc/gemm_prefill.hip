@@ -67,8 +67,18 @@ __device__ __forceinline__ f32x4 xs_load(const float* src) {
 // workgroup delivers its partial tile in fp32 and counts itself in; whoever arrives last adds the
 // partials up in index order (the same sum whichever workgroup that is) and runs the epilogue.
 // Nobody waits for anybody.
+// DMA: both operand tiles go from global memory straight into the LDS stages
+// (global_load_lds_dwordx4: lane i of a wave instruction delivers its 16 bytes to LDS slot i of a
+// 1 KB block, i.e. eight 128-byte rows of a tile), without staging registers. Staged through
+// registers, the tile's sixteen waves have none to spare (128 each), the compiler lets the loaded
+// values share registers with the matrix operands and therefore sinks the loads of step s + 2 to the
+// end of step s's multiplications -- a barrier and a few instructions before step s + 1 waits for
+// them: most of an L2 round trip per k-step with the matrix pipes idle. With the DMA the loads of
+// step s + 1 are issued before step s is multiplied and are waited for after it. The swizzle is
+// applied on the global side: slot (row r, chunk s) receives logical chunk s ^ swz(r). Needs 16-bit
+// weights, K a multiple of the k-step, no fused norm (a prompt's norm is a launch of its own).
 template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF,
-          bool XS = false>
+          bool XS = false, bool DMA = false>
 // (twelve waves: three per SIMD, so let the compiler use the registers of three)
 __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
     __attribute__((amdgpu_waves_per_eu(1, (NWR * NWT * NWK == 12) ? 3 : 8)))
@@ -174,6 +184,43 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   };
 
   const int n_steps = (p.k + KS - 1) / KS;
+  // DMA: per wave instruction q the source of this lane's slot (fixed but for the k-step's offset)
+  constexpr int kNWaves = kPfThreads / 64;
+  constexpr int WQ = DMA ? ROWS / (8 * kNWaves) : 1, XQ = DMA ? TOKS / (8 * kNWaves) : 1;
+  const uint8_t* dma_w[WQ];
+  const uint8_t* dma_x[XQ];
+  if constexpr (DMA) {
+    static_assert(!DMA || (WF == WF_16BIT && !NORM && NBUF == 2 && NWK == 1 && !XS && CPR == 8), "what the DMA path covers");
+    static_assert(!DMA || (WQ * 8 * kNWaves == ROWS && XQ * 8 * kNWaves == TOKS), "whole 8-row blocks per wave");
+    const int sr = lane >> 3, sc = lane & 7;
+#pragma unroll
+    for (int q = 0; q < WQ; ++q) {
+      const int r = (q * kNWaves + wave) * 8 + sr;
+      bool up;
+      const int o = weight_row(r, up);
+      dma_w[q] = ((EPI == SK_GATEUP && up) ? p.w1 : p.w0) + (long)o * p.pitch + ((sc ^ swz(r)) * 16);
+    }
+#pragma unroll
+    for (int q = 0; q < XQ; ++q) {
+      const int r = (q * kNWaves + wave) * 8 + sr;
+      int tk = t0 + r;
+      tk = tk < p.tokens ? tk : p.tokens - 1;
+      dma_x[q] = (const uint8_t*)(p.x + (long)tk * p.k) + ((sc ^ swz(r)) * 16);
+    }
+  }
+  auto dma_step = [&](int step, int buf) {
+    const long kb = (long)step * KS * 2;
+#pragma unroll
+    for (int q = 0; q < WQ; ++q)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(dma_w[q] + kb),
+                                       (__attribute__((address_space(3))) void*)&w_lds[buf][(q * kNWaves + wave) * 8 * PITCH],
+                                       16, 0, 0);
+#pragma unroll
+    for (int q = 0; q < XQ; ++q)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(dma_x[q] + kb),
+                                       (__attribute__((address_space(3))) void*)&x_lds[buf][(q * kNWaves + wave) * 8 * PITCH],
+                                       16, 0, 0);
+  };
   // one k-step of the tile in registers, on its way from global memory to LDS
   struct Stage { u32x4 w[WCH], x[XCH], g; };
   auto load_step = [&](int step, Stage& r) {
@@ -264,8 +311,18 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   const int sb = XS ? (int)((long)n_steps * xs_share / p.k_splits) : 0;
   const int se = XS ? (int)((long)n_steps * (xs_share + 1) / p.k_splits) : n_steps;
   Stage r0;
-  load_step(sb, r0);
-  if constexpr (NBUF == 2) {
+  if constexpr (DMA) {
+    dma_step(sb, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's blocks of the step are in LDS
+    __syncthreads();
+    for (int s = sb; s < se; ++s) {
+      if (s + 1 < se) dma_step(s + 1, (s + 1 - sb) & 1);  // the other stage: last read before the barrier just passed
+      multiply((s - sb) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+    }
+  } else if constexpr (NBUF == 2) {
+    load_step(sb, r0);
     // two LDS stages: step s + 1 moves from the registers to the other stage and step s + 2 is
     // requested from memory before step s is multiplied, so that the LDS writes and the loads
     // proceed under the matrix instructions; one barrier per step. (A second register stage
@@ -305,6 +362,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
       __syncthreads();
     }
   } else {
+    load_step(sb, r0);
     for (int s = 0; s < n_steps; ++s) {
       __syncthreads();  // the previous step's operands have been read
       store_step(s, 0, r0);
@@ -458,6 +516,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   }
 }
 
+static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
                                 // 5 = 64 x 128 on eight waves that split K four ways, 6 = 32 x 64 on four waves that split K,
                                 // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
@@ -489,6 +548,17 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
     return launch_status();
   };
   if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
+  constexpr int kWaves8 = 8 * NWR * NWT * NWK;
+  if constexpr (WF == WF_16BIT && NBUF == 2 && NWK == 1 && KS == 64 && ROWS % kWaves8 == 0 && TOKS % kWaves8 == 0 &&
+                ROWS * TOKS >= 256 * 256) {
+    // The DMA has one k-step of lead (two LDS stages), the register-staged path two. On the 256 x 256
+    // tile a step is 2048 matrix-pipe cycles per SIMD, enough for an L2 round trip, and the DMA wins
+    // (gate/up at 4096 tokens 834 -> 800 us, down 410 -> 390 us, o_proj 136 -> 123 us, gate/up at 512
+    // 129 -> 118 us); on 128 x 256, half of that, it loses (down at 2048 tokens 264 -> 293 us, o_proj
+    // 77 -> 88 us, gate/up at 256 88 -> 99 us).
+    if (g_prefill_dma && ROWS * TOKS >= 256 * 256 && p.k % KS == 0 && p.pitch % 16 == 0 && (p.k & 7) == 0)
+      return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, false, true>);
+  }
   return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
 }
 
@@ -700,6 +770,12 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   MUI_TUNE_GUARD();
+  if (tile >= 100) {  // experiments: 100 + tile keeps every operand tile on the register-staged path
+    mui::g_prefill_dma = 0;
+    tile -= 100;
+  } else {
+    mui::g_prefill_dma = 1;
+  }
   if (tile < 0 || tile > 12 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
