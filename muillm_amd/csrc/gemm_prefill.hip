@@ -17,7 +17,8 @@
 //   chunks are XOR-swizzled (conflict-free 128-bit reads and writes); the loads of step s + 2 are
 //   in flight and step s + 1 is on its way into the other LDS stage while step s is multiplied.
 //   Tile shapes, chosen per call by rounds of workgroups x cost per round (launch_prefill_t):
-//   256 rows x 256 tokens x 64 k and 128 x 256 x 64 on sixteen waves (4 x 4), 192 x 256 x 64 on
+//   256 rows x 256 tokens x 64 k on eight waves (4 x 2; sixteen where a norm is fused or the loads
+//   cannot go straight into LDS), 128 x 256 x 64 on sixteen (4 x 4), 192 x 256 x 64 on
 //   twelve (3 x 4) while the grid covers most of the chip; 128 x 128 x 64 and 96 x 128 x 64 on four
 //   waves (2 x 2), two workgroups per CU; 64 x 128 x 128 and 32 x 64 x 256 with a single LDS stage
 //   for small matrices. For grids of a round or two of workgroups (short prompts, matrices of a few
@@ -32,6 +33,8 @@
 //   rows of the same outputs, so SiLU * mul happens in registers.
 //   Token tiles of one row tile are placed on the same XCD (workgroup id modulo 8) so that the
 //   re-reads of its weights hit that XCD's L2.
+#include <type_traits>
+
 #include "skinny.cuh"
 
 namespace mui {
@@ -77,8 +80,17 @@ __device__ __forceinline__ f32x4 xs_load(const float* src) {
 // step s + 1 are issued before step s is multiplied and are waited for after it. The swizzle is
 // applied on the global side: slot (row r, chunk s) receives logical chunk s ^ swz(r). Needs 16-bit
 // weights, K a multiple of the k-step, no fused norm (a prompt's norm is a launch of its own).
+// PIPE (with DMA; the 256 x 256 tile on eight waves of 64 x 128): the software-pipelined loop. A wave
+// holds the operands of both halves of a k-step in registers; the LDS reads of one half and the
+// loads of the step after next are dealt out between the matrix instructions of the other half in
+// a pinned order, and the one barrier per step has thirty-two matrix instructions of every wave
+// behind it. Timed with the shader's own cycle counter the loop runs at 2283 cycles per k-step of
+// 2048 matrix-pipe cycles per SIMD (2150 with the loads taken out) -- and at a shader clock of 1.36 GHz,
+// which is what a microsecond figure on this part reflects: the board's power limit sets the clock
+// under this load, and operand bytes read from LDS per matrix instruction are what the eight waves
+// save over sixteen (192 instead of 256 KB per k-step).
 template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF,
-          bool XS = false, bool DMA = false>
+          bool XS = false, bool DMA = false, bool PIPE = false>
 // (twelve waves: three per SIMD, so let the compiler use the registers of three)
 __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
     __attribute__((amdgpu_waves_per_eu(1, (NWR * NWT * NWK == 12) ? 3 : 8)))
@@ -187,39 +199,58 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   // DMA: per wave instruction q the source of this lane's slot (fixed but for the k-step's offset)
   constexpr int kNWaves = kPfThreads / 64;
   constexpr int WQ = DMA ? ROWS / (8 * kNWaves) : 1, XQ = DMA ? TOKS / (8 * kNWaves) : 1;
-  const uint8_t* dma_w[WQ];
-  const uint8_t* dma_x[XQ];
+  // per wave instruction q: a base address that is the same for the wave's lanes (the matrix, or the
+  // up matrix for the instructions that cover up rows: eight consecutive tile rows never straddle
+  // the two) and this lane's 32-bit byte offset from it; only the base moves with the k-step
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  unsigned dma_wo[WQ], dma_xo[XQ];
   if constexpr (DMA) {
     static_assert(!DMA || (WF == WF_16BIT && !NORM && NBUF == 2 && NWK == 1 && !XS && CPR == 8), "what the DMA path covers");
     static_assert(!DMA || (WQ * 8 * kNWaves == ROWS && XQ * 8 * kNWaves == TOKS), "whole 8-row blocks per wave");
+    static_assert(!DMA || EPI != SK_GATEUP || (8 * WR) % 8 == 0, "gate and up rows change at multiples of eight tile rows");
     const int sr = lane >> 3, sc = lane & 7;
 #pragma unroll
     for (int q = 0; q < WQ; ++q) {
       const int r = (q * kNWaves + wave) * 8 + sr;
       bool up;
       const int o = weight_row(r, up);
-      dma_w[q] = ((EPI == SK_GATEUP && up) ? p.w1 : p.w0) + (long)o * p.pitch + ((sc ^ swz(r)) * 16);
+      dma_wo[q] = (unsigned)((long)o * p.pitch + ((sc ^ swz(r)) * 16));
     }
 #pragma unroll
     for (int q = 0; q < XQ; ++q) {
       const int r = (q * kNWaves + wave) * 8 + sr;
       int tk = t0 + r;
       tk = tk < p.tokens ? tk : p.tokens - 1;
-      dma_x[q] = (const uint8_t*)(p.x + (long)tk * p.k) + ((sc ^ swz(r)) * 16);
+      dma_xo[q] = (unsigned)((long)tk * p.k * 2 + ((sc ^ swz(r)) * 16));
     }
   }
-  auto dma_step = [&](int step, int buf) {
+  // load instruction i of a k-step: the weight blocks first, then the token blocks
+  auto dma_one = [&](int step, int buf, int i) {
     const long kb = (long)step * KS * 2;
-#pragma unroll
-    for (int q = 0; q < WQ; ++q)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(dma_w[q] + kb),
-                                       (__attribute__((address_space(3))) void*)&w_lds[buf][(q * kNWaves + wave) * 8 * PITCH],
+    // (the lane offset is made opaque to the optimiser: widened to 64 bits outside the loop it would
+    // cost a register pair and a 64-bit add per load instead of the scalar-base addressing mode)
+    if (i < WQ) {
+      const int q = i;
+      bool up;
+      weight_row((q * kNWaves + wave_u) * 8, up);
+      const uint8_t* base = ((EPI == SK_GATEUP && up) ? p.w1 : p.w0) + kb;
+      unsigned off = dma_wo[q];
+      asm volatile("" : "+v"(off));
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off),
+                                       (__attribute__((address_space(3))) void*)&w_lds[buf][(q * kNWaves + wave_u) * 8 * PITCH],
                                        16, 0, 0);
-#pragma unroll
-    for (int q = 0; q < XQ; ++q)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(dma_x[q] + kb),
-                                       (__attribute__((address_space(3))) void*)&x_lds[buf][(q * kNWaves + wave) * 8 * PITCH],
+    } else {
+      const int q = i - WQ;
+      unsigned off = dma_xo[q];
+      asm volatile("" : "+v"(off));
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)((const uint8_t*)p.x + kb + off),
+                                       (__attribute__((address_space(3))) void*)&x_lds[buf][(q * kNWaves + wave_u) * 8 * PITCH],
                                        16, 0, 0);
+    }
+  };
+  auto dma_step = [&](int step, int buf) {
+#pragma unroll
+    for (int i = 0; i < WQ + XQ; ++i) dma_one(step, buf, i);
   };
   // one k-step of the tile in registers, on its way from global memory to LDS
   struct Stage { u32x4 w[WCH], x[XCH], g; };
@@ -311,7 +342,98 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   const int sb = XS ? (int)((long)n_steps * xs_share / p.k_splits) : 0;
   const int se = XS ? (int)((long)n_steps * (xs_share + 1) / p.k_splits) : n_steps;
   Stage r0;
-  if constexpr (DMA) {
+  if constexpr (DMA && PIPE) {
+    // Two operand register sets per wave: the LDS reads of one half of a k-step are issued while the
+    // other half is multiplied, one read per two matrix instructions, so a wave always has sixteen
+    // or more matrix instructions to issue that wait for nothing; the barrier sits between the two
+    // halves of a step, with the second half's multiplications behind it.
+    static_assert(!PIPE || (KS == 64 && NWK == 1), "two halves per k-step");
+    u32x4 a[2][WR], b[2][WT];
+    // operand read i of a half step: the WT token operands first, then the WR weight operands
+    auto read_one = [&](int buf, int kk, int set, int i) {
+      if (i < WT) b[set][i] = *(const u32x4*)&x_lds[buf][b_base + i * 16 * PITCH + (((kk * 4 + lg) ^ lsw) * 8)];
+      else a[set][i - WT] = *(const u32x4*)&w_lds[buf][a_base + (i - WT) * 16 * PITCH + (((kk * 4 + lg) ^ lsw) * 8)];
+    };
+    auto read_ops = [&](int buf, int kk, int set) {
+#pragma unroll
+      for (int i = 0; i < WT + WR; ++i) read_one(buf, kk, set, i);
+    };
+    auto mm = [&](int set, int i0, int i1) {
+#pragma unroll
+      for (int i = i0; i < i1; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) acc[i][j] = mfma16x16x32<T>(a[set][i], b[set][j], acc[i][j]);
+    };
+    // pinned order of a region: `per` matrix instructions, then one instruction of the masked kind
+    // (0x100 LDS read, 0x010 memory load), `n` times; then the remaining matrix instructions
+    auto pin = [&](auto maskc, auto perc, auto nc, auto totalc) {
+      constexpr int MASK = decltype(maskc)::value, PER = decltype(perc)::value, N = decltype(nc)::value,
+                    TOTAL = decltype(totalc)::value;
+#pragma unroll
+      for (int r = 0; r < N; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+        __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+      }
+      if constexpr (TOTAL > PER * N) __builtin_amdgcn_sched_group_barrier(0x008, TOTAL - PER * N, 0);
+    };
+    static_assert(!PIPE || WR * WT >= 2 * (WR + WT), "two matrix instructions per read");
+    dma_step(sb, 0);
+    if (sb + 1 < se) dma_step(sb + 1, 1);
+    if (sb + 1 < se) __builtin_amdgcn_s_waitcnt(0x0F70 | (WQ + XQ));  // all but the second step's loads
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    read_ops(0, 0, 0);
+    static_assert(!PIPE || (WR >= 2 && WT >= (WR + WT + WR - 2) / (WR - 1) + (WQ + XQ + WR - 1) / WR), "schedule of the second half: a matrix instruction per read and load");
+    for (int s = sb; s < se; ++s) {
+      const int buf = (s - sb) & 1;
+      read_ops(buf, 1, 1);
+      mm(0, 0, WR);
+      pin(std::integral_constant<int, 0x100>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, WR + WT>{},
+          std::integral_constant<int, WR * WT>{});
+      __builtin_amdgcn_sched_barrier(0);
+      // this wave's reads of the stage have returned, its share of the next stage has landed
+      __builtin_amdgcn_s_waitcnt(0x0070);
+      __syncthreads();
+      // (the last two steps load the last step once more, into a stage that nobody reads any more,
+      // and read stale operands that nobody multiplies: no branch, one schedule)
+      // second half: one row of matrix instructions per region, each with its share of the next
+      // half's operand reads and of the loads of the step after next -- spread over the whole half,
+      // so that the eight waves, which all leave the barrier together, do not queue their loads
+      // faster than the CU's memory pipeline takes them (a wave that waits to issue a load does not
+      // issue the matrix instructions behind it either)
+      const int nxt = s + 2 < se ? s + 2 : se - 1;
+      // (the reads in all but the last region: the first matrix instruction of the next half waits
+      // for the last of them)
+      constexpr int RD = (WR + WT + WR - 2) / (WR - 1), LD = (WQ + XQ + WR - 1) / WR;  // reads / loads per region
+#pragma unroll
+      for (int i = 0; i < WR; ++i) {
+#pragma unroll
+        for (int l = 0; l < LD; ++l)
+          if (i * LD + l < WQ + XQ) dma_one(nxt, buf, i * LD + l);
+#pragma unroll
+        for (int r = 0; r < RD; ++r)
+          if (i < WR - 1 && i * RD + r < WR + WT) read_one(buf ^ 1, 0, 0, i * RD + r);
+        mm(1, i, i + 1);
+        // a matrix instruction, a load, ..., a matrix instruction, a read, ... (loads first: they have the longer way)
+#pragma unroll
+        for (int g = 0; g < LD; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        if (i < WR - 1) {
+#pragma unroll
+          for (int g = 0; g < RD; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, WT - (LD + RD), 0);
+        } else {
+          __builtin_amdgcn_sched_group_barrier(0x008, WT - LD, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  } else if constexpr (DMA) {
     dma_step(sb, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's blocks of the step are in LDS
     __syncthreads();
@@ -523,7 +645,7 @@ static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 1
                                 // 10 = 96 x 128 (linear only), 11 = 128 x 64 on sixteen waves that split K four ways,
                                 // 12 = 64 x 64 on eight waves that split K four ways (linear only)
 
-template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF>
+template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF, bool PIPE = false>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   p.n_tiles = ceil_div(p.n, EPI == SK_GATEUP ? ROWS / 2 : ROWS);
@@ -547,7 +669,9 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
     hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(64 * NWR * NWT * NWK), lds, s, p);
     return launch_status();
   };
-  if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
+  if constexpr (!PIPE) {
+    if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
+  }
   constexpr int kWaves8 = 8 * NWR * NWT * NWK;
   if constexpr (WF == WF_16BIT && NBUF == 2 && NWK == 1 && KS == 64 && ROWS % kWaves8 == 0 && TOKS % kWaves8 == 0 &&
                 ROWS * TOKS >= 256 * 256) {
@@ -556,10 +680,12 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
     // (gate/up at 4096 tokens 834 -> 800 us, down 410 -> 390 us, o_proj 136 -> 123 us, gate/up at 512
     // 129 -> 118 us); on 128 x 256, half of that, it loses (down at 2048 tokens 264 -> 293 us, o_proj
     // 77 -> 88 us, gate/up at 256 88 -> 99 us).
-    if (g_prefill_dma && ROWS * TOKS >= 256 * 256 && p.k % KS == 0 && p.pitch % 16 == 0 && (p.k & 7) == 0)
-      return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, false, true>);
+    if (g_prefill_dma && ROWS * TOKS >= 256 * 256 && p.k % KS == 0 && p.pitch % 16 == 0 && (p.k & 7) == 0 &&
+        (long)p.n * p.pitch < (1L << 32) && (long)p.tokens * p.k * 2 < (1L << 32))  // 32-bit offsets from the operands' bases
+      return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, false, true, PIPE>);
   }
-  return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
+  if constexpr (PIPE) return MUI_ERR_UNSUPPORTED;  // the caller falls back to the sixteen-wave tile
+  else return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
 }
 
 // Workspace of the K split over workgroups (mui_linear_ws): arrival counters, then partial tiles
@@ -681,6 +807,17 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   // 4096 881 -> 854 us; 128 x 256: 75 -> 68 us per round; 128 x 128 splitting K: 46 -> 42 us).
   // int8 rows hold a quarter of the 16-byte chunks per k-step: where sixteen waves would leave
   // threads without a chunk to stage, the int8 kernels keep eight.
+  if constexpr (WF == WF_16BIT) {
+    // 256 x 256 on 4 x 2 waves of 64 x 128 with two operand register sets (the software-pipelined
+    // loop): where its loads can go straight into LDS it is 5-8 % ahead of the sixteen waves below
+    // (gate/up at 4096 tokens 775 -> 736 us, down 386 -> 356 us, QKV 224 -> 209 us, down at 2048
+    // tokens 345 -> 315 us; bit-equal results: the same products in the same order)
+    if (which == 4 && !p.gamma) {
+      const int st = launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, p);
+      if (st != MUI_ERR_UNSUPPORTED) return st;
+    }
+  }
+  if (which == 13) which = 4;  // the sixteen-wave kernel on request
   if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 4, 4, 4, 1, 64, 2>(s, p);      // 256 x 256, 4 x 4 waves of 64 x 64
   // 192 x 256 on twelve waves (3 x 4 of 64 x 64, the wave tile of the 256 x 256 kernel; the token
   // chunks of a k-step do not divide by 768 threads: the last round is staged by eight of the
@@ -776,7 +913,7 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   } else {
     mui::g_prefill_dma = 1;
   }
-  if (tile < 0 || tile > 12 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;

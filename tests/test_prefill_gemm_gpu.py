@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
-@pytest.fixture(params=["auto", "wide", "tile-256x256", "tile-128x128", "tile-64x128", "tile-32x64", "ksplit-64x128", "ksplit-32x64", "tile-128x256", "tile-192x256", "tile-96x128", "ksplit-128x128", "ksplit-128x64", "ksplit-64x64"], autouse=True)
+@pytest.fixture(params=["auto", "wide", "tile-256x256", "tile-128x128", "tile-64x128", "tile-32x64", "ksplit-64x128", "ksplit-32x64", "tile-128x256", "tile-192x256", "tile-96x128", "ksplit-128x128", "ksplit-128x64", "ksplit-64x64", "tile-256x256-16-waves", "tile-256x256-register-staged"], autouse=True)
 def prompt_kernel_choice(request):
     """Every test runs with the built-in kernel choice and with each prompt kernel forced: the
     16-rows-per-workgroup kernel without LDS tiling (up to 128 tokens; longer prompts keep the
@@ -30,7 +30,8 @@ def prompt_kernel_choice(request):
     96-row shape and take 128 x 128)."""
     lib = _lib.load()
     knobs = {"auto": (0, 0), "wide": (0, 128), "tile-256x256": (4, -1), "ksplit-64x128": (5, -1), "ksplit-32x64": (6, -1), "tile-128x128": (1, -1), "tile-64x128": (2, -1), "tile-32x64": (3, -1),
-             "tile-128x256": (7, -1), "tile-192x256": (8, -1), "tile-96x128": (10, -1), "ksplit-128x128": (9, -1), "ksplit-128x64": (11, -1), "ksplit-64x64": (12, -1)}
+             "tile-128x256": (7, -1), "tile-192x256": (8, -1), "tile-96x128": (10, -1), "ksplit-128x128": (9, -1), "ksplit-128x64": (11, -1), "ksplit-64x64": (12, -1),
+             "tile-256x256-16-waves": (13, -1), "tile-256x256-register-staged": (104, -1)}
     _lib.check(lib.mui_tune_prefill(*knobs[request.param]), "mui_tune_prefill")
     # the built-in choice runs as shipped (prompts normalised by one rmsnorm launch in front of
     # the GEMM); the forced kernels keep the norm fused into the GEMM, which the C entry points
