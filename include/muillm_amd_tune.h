@@ -65,11 +65,13 @@ int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
  * four ways (2 x 2 wave tiles; int8: two token halves), 6 = 32 x 64 on four waves that split K,
  * 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 and 11 = 128 x 64 with waves that split K like 5,
  * 10 = 96 x 128 (linear only), 12 = 64 x 64 with waves that split K like 6 (linear only),
- * 13 = 256 x 256 on sixteen waves (4 itself runs on eight software-pipelined waves where it can: 16-bit
- * weights, no fused norm, K a multiple of 64); shapes that a weight format or epilogue lacks fall back
- * to the next one that it has. A forced tile also keeps mui_linear_ws from sharing K between workgroups.
- * 100 + tile: the same, and the 256 x 256 tile stages its operands through registers (on sixteen
- * waves) instead of loading them straight into LDS.
+ * 13 = 256 x 256 on sixteen waves (4, 7 and 8 themselves run on eight software-pipelined waves where
+ * they can: 16-bit weights, no fused norm, K a multiple of 64; 8 for linear only); shapes that a weight
+ * format or epilogue lacks fall back to the next one that it has. A forced tile also keeps
+ * mui_linear_ws from sharing K between workgroups.
+ * 100 + tile: the same, and no tile loads its operands straight into LDS (all are staged through
+ * registers, on sixteen or twelve waves). 200 + tile: the same as tile, but 128 x 256 and 192 x 256
+ * keep their sixteen / twelve waves.
  * wide_max_tokens = longest prompt served by the weight-streaming 16-rows-per-workgroup kernel
  * instead of the LDS-tiled one (0 restores the built-in choice; at most 128; negative: never) */
 int mui_tune_prefill(int tile, int wide_max_tokens);

@@ -383,7 +383,6 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
     else __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     read_ops(0, 0, 0);
-    static_assert(!PIPE || (WR >= 2 && WT >= (WR + WT + WR - 2) / (WR - 1) + (WQ + XQ + WR - 1) / WR), "schedule of the second half: a matrix instruction per read and load");
     for (int s = sb; s < se; ++s) {
       const int buf = (s - sb) & 1;
       read_ops(buf, 1, 1);
@@ -402,36 +401,42 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
       // faster than the CU's memory pipeline takes them (a wave that waits to issue a load does not
       // issue the matrix instructions behind it either)
       const int nxt = s + 2 < se ? s + 2 : se - 1;
-      // (the reads in all but the last region: the first matrix instruction of the next half waits
-      // for the last of them)
-      constexpr int RD = (WR + WT + WR - 2) / (WR - 1), LD = (WQ + XQ + WR - 1) / WR;  // reads / loads per region
+      // (the reads in all but the last region where they fit there: the first matrix instruction of
+      // the next half waits for the last of them)
+      constexpr int NL = WQ + XQ, NR = WR + WT;
+      constexpr int LD = (NL + WR - 1) / WR;                             // loads per region
+      constexpr int RD_EARLY = (NR + WR - 2) / (WR - 1);                 // reads per region, last region free
+      constexpr bool EARLY = RD_EARLY + LD <= WT;
+      constexpr int RD = EARLY ? RD_EARLY : (NR + WR - 1) / WR;
+      static_assert(!PIPE || RD + LD <= WT, "schedule of the second half: a matrix instruction per read and load");
+      auto region = [&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int nl = NL - i * LD < 0 ? 0 : (NL - i * LD < LD ? NL - i * LD : LD);
+        constexpr int nr = (EARLY && i == WR - 1) || NR - i * RD < 0 ? 0 : (NR - i * RD < RD ? NR - i * RD : RD);
 #pragma unroll
-      for (int i = 0; i < WR; ++i) {
+        for (int l = 0; l < nl; ++l) dma_one(nxt, buf, i * LD + l);
 #pragma unroll
-        for (int l = 0; l < LD; ++l)
-          if (i * LD + l < WQ + XQ) dma_one(nxt, buf, i * LD + l);
-#pragma unroll
-        for (int r = 0; r < RD; ++r)
-          if (i < WR - 1 && i * RD + r < WR + WT) read_one(buf ^ 1, 0, 0, i * RD + r);
+        for (int r = 0; r < nr; ++r) read_one(buf ^ 1, 0, 0, i * RD + r);
         mm(1, i, i + 1);
         // a matrix instruction, a load, ..., a matrix instruction, a read, ... (loads first: they have the longer way)
 #pragma unroll
-        for (int g = 0; g < LD; ++g) {
+        for (int g = 0; g < nl; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
-        if (i < WR - 1) {
 #pragma unroll
-          for (int g = 0; g < RD; ++g) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          }
-          __builtin_amdgcn_sched_group_barrier(0x008, WT - (LD + RD), 0);
-        } else {
-          __builtin_amdgcn_sched_group_barrier(0x008, WT - LD, 0);
+        for (int g = 0; g < nr; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        if constexpr (WT - nl - nr > 0) __builtin_amdgcn_sched_group_barrier(0x008, WT - nl - nr, 0);
         __builtin_amdgcn_sched_barrier(0);
-      }
+      };
+      static_assert(!PIPE || (WR >= 2 && WR <= 4), "regions of the second half");
+      region(std::integral_constant<int, 0>{});
+      region(std::integral_constant<int, 1>{});
+      if constexpr (WR > 2) region(std::integral_constant<int, 2>{});
+      if constexpr (WR > 3) region(std::integral_constant<int, 3>{});
     }
   } else if constexpr (DMA) {
     dma_step(sb, 0);
@@ -638,12 +643,22 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   }
 }
 
-static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
                                 // 5 = 64 x 128 on eight waves that split K four ways, 6 = 32 x 64 on four waves that split K,
                                 // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
                                 // 10 = 96 x 128 (linear only), 11 = 128 x 64 on sixteen waves that split K four ways,
                                 // 12 = 64 x 64 on eight waves that split K four ways (linear only)
+
+static int g_prefill_pipe_small = 1;  // experiments: the pipelined loop on the 128 x 256 and 192 x 256 tiles too
+static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
+
+// what the LDS-direct loads need: whole k-steps of 64, 16-byte aligned rows, 32-bit byte offsets from
+// the operands' bases
+static bool lds_direct_loads_serve(const PrefillGemmParams& p) {
+  return g_prefill_dma && p.k % 64 == 0 && p.pitch % 16 == 0 && (long)p.n * p.pitch < (1L << 32) &&
+         (long)p.tokens * p.k * 2 < (1L << 32);
+}
+static bool pipelined_loop_serves(const PrefillGemmParams& p) { return lds_direct_loads_serve(p); }
 
 template <typename T, int WF, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF, bool PIPE = false>
 static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
@@ -674,14 +689,13 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   }
   constexpr int kWaves8 = 8 * NWR * NWT * NWK;
   if constexpr (WF == WF_16BIT && NBUF == 2 && NWK == 1 && KS == 64 && ROWS % kWaves8 == 0 && TOKS % kWaves8 == 0 &&
-                ROWS * TOKS >= 256 * 256) {
+                (PIPE || ROWS * TOKS >= 256 * 256)) {
     // The DMA has one k-step of lead (two LDS stages), the register-staged path two. On the 256 x 256
     // tile a step is 2048 matrix-pipe cycles per SIMD, enough for an L2 round trip, and the DMA wins
     // (gate/up at 4096 tokens 834 -> 800 us, down 410 -> 390 us, o_proj 136 -> 123 us, gate/up at 512
     // 129 -> 118 us); on 128 x 256, half of that, it loses (down at 2048 tokens 264 -> 293 us, o_proj
     // 77 -> 88 us, gate/up at 256 88 -> 99 us).
-    if (g_prefill_dma && ROWS * TOKS >= 256 * 256 && p.k % KS == 0 && p.pitch % 16 == 0 && (p.k & 7) == 0 &&
-        (long)p.n * p.pitch < (1L << 32) && (long)p.tokens * p.k * 2 < (1L << 32))  // 32-bit offsets from the operands' bases
+    if (lds_direct_loads_serve(p))
       return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, false, true, PIPE>);
   }
   if constexpr (PIPE) return MUI_ERR_UNSUPPORTED;  // the caller falls back to the sixteen-wave tile
@@ -778,13 +792,17 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
         const float last = rest == 0 ? 0.f : rest <= cus ? single : single + (twin - single) * (float)(rest - cus) / (float)cus;
         return (float)full * twin + last;
       };
-      float best = whole(tiles(256, 256), 100.f, 111.f);
+      // (the three big tiles cost less per round where the software-pipelined loop serves them)
+      const bool pipe = WF == WF_16BIT && !p.gamma && pipelined_loop_serves(p);
+      float best = whole(tiles(256, 256), pipe ? 96.f : 100.f, pipe ? 106.f : 111.f);
       which = 4;
       auto offer = [&](int id, float cost) {
         if (cost < best * 0.97f) { best = cost; which = id; }  // bigger tiles win ties
       };
-      offer(8, whole(tiles(192, 256), 85.f, 92.f));
-      offer(7, whole(tiles(128, 256), WF == WF_16BIT ? 67.f : 73.f, WF == WF_16BIT ? 70.f : 76.f));
+      if (pipe && EPI == SK_LINEAR) offer(8, whole(tiles(192, 256), 74.f, 80.f));
+      else offer(8, whole(tiles(192, 256), 85.f, 92.f));
+      if (pipe) offer(7, whole(tiles(128, 256), 63.f, 66.f));
+      else offer(7, whole(tiles(128, 256), WF == WF_16BIT ? 67.f : 73.f, WF == WF_16BIT ? 70.f : 76.f));
       offer(1, pairs(tiles(128, 128), 68.f, 92.f));
       if (EPI == SK_LINEAR && WF == WF_16BIT) offer(10, pairs(tiles(96, 128), 60.f, 76.f));
       // 128 x 128 on waves that split K: the fastest single tile (QKV at 512 tokens 43 vs 62 us,
@@ -818,6 +836,16 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
     }
   }
   if (which == 13) which = 4;  // the sixteen-wave kernel on request
+  if constexpr (WF == WF_16BIT) {
+    if (g_prefill_pipe_small && !p.gamma) {
+      int st = MUI_ERR_UNSUPPORTED;
+      if (which == 7) st = launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, p);    // 128 x 256, 2 x 4 waves of 64 x 64
+      if constexpr (EPI == SK_LINEAR) {
+        if (which == 8) st = launch_prefill_cfg<T, WF, EPI, 3, 8, 4, 2, 1, 64, 2, true>(s, p);  // 192 x 256, 4 x 2 waves of 48 x 128
+      }
+      if (st != MUI_ERR_UNSUPPORTED) return st;
+    }
+  }
   if (which == 4) return launch_prefill_cfg<T, WF, EPI, 4, 4, 4, 4, 1, 64, 2>(s, p);      // 256 x 256, 4 x 4 waves of 64 x 64
   // 192 x 256 on twelve waves (3 x 4 of 64 x 64, the wave tile of the 256 x 256 kernel; the token
   // chunks of a k-step do not divide by 768 threads: the last round is staged by eight of the
@@ -907,13 +935,15 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
 
 extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   MUI_TUNE_GUARD();
-  if (tile >= 100) {  // experiments: 100 + tile keeps every operand tile on the register-staged path
-    mui::g_prefill_dma = 0;
-    tile -= 100;
-  } else {
-    mui::g_prefill_dma = 1;
-  }
+  // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
+  // 100 + tile keeps every operand tile on the register-staged path
+  const int pipe_small = tile >= 200 ? 0 : 1;
+  if (tile >= 200) tile -= 200;
+  const int dma = tile >= 100 ? 0 : 1;
+  if (tile >= 100) tile -= 100;
   if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_pipe_small = pipe_small;
+  mui::g_prefill_dma = dma;
   mui::g_prefill_tile = tile;
   mui::g_wide_max_tokens = wide_max_tokens;  // 0: built-in rule; negative: never; n: prompts up to n tokens
   return MUI_OK;

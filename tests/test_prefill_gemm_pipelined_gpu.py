@@ -1,8 +1,9 @@
-"""GPU parity of the software-pipelined 256 x 256 prompt tile (mui_linear / mui_gateup_silu beyond
-MUI_MAX_TOKENS tokens, 16-bit weights, no fused norm, K a multiple of 64): eight waves with two
-operand register sets each, operands loaded straight into LDS. Checked against the CPU oracle at
-the decode kernels' gate (max error over max |ref| <= 1e-2) and bit for bit against the two older
-kernels of the same tile, which multiply the same products in the same order.
+"""GPU parity of the software-pipelined prompt tiles (mui_linear / mui_gateup_silu beyond
+MUI_MAX_TOKENS tokens, 16-bit weights, no fused norm, K a multiple of 64): 256 x 256, 128 x 256 and
+192 x 256 (linear only) on eight waves with two operand register sets each, operands loaded
+straight into LDS. Checked against the CPU oracle at the decode kernels' gate (max error over
+max |ref| <= 1e-2) and bit for bit against the older kernels of the same tiles, which multiply the
+same products in the same order.
 
 The reference hands these calls to the framework's GEMM (csrc/modules/linear_module.cpp:57-79)."""
 
@@ -36,11 +37,11 @@ def _mk(shape, g, std=1.0, mean=0.0, dtype=torch.float16):
     (700, 512, 400, True),      # gate/up, ragged
     (14336, 4096, 512, True),   # gate/up at the benchmark shape
 ])
-def test_software_pipelined_256_tile(dtype, n, k, tokens, gateup):
-    """The 256 x 256 tile on eight waves with two operand register sets per wave (what the tile
-    choice 4 runs for 16-bit weights without a fused norm when K is a multiple of 64) against the
-    oracle, and bit for bit against the sixteen-wave kernel of the same tile (choice 13) and its
-    register-staged form (104): the three multiply the same products in the same order."""
+def test_software_pipelined_tiles(dtype, n, k, tokens, gateup):
+    """Tile choices 4 (256 x 256), 7 (128 x 256) and 8 (192 x 256; the gate/up epilogue has none and
+    takes its twelve-wave kernel) run the software-pipelined loop here; 13, 207, 208 and 104 are the
+    older kernels of the same tiles (sixteen / sixteen / twelve waves, LDS-direct or
+    register-staged operands)."""
     lib = _lib.load()
     s = torch.cuda.current_stream().cuda_stream
     g = _gen(11)
@@ -56,7 +57,7 @@ def test_software_pipelined_256_tile(dtype, n, k, tokens, gateup):
         wd, r, b = w.to(DEV), r.to(DEV), b.to(DEV)
     xd = x.to(DEV)
     outs = {}
-    for choice in (4, 13, 104):
+    for choice in (4, 13, 104, 7, 207, 8, 208):
         _lib.check(lib.mui_tune_prefill(choice, -1), "mui_tune_prefill")
         y = torch.zeros(tokens, n, dtype=dtype, device=DEV)
         if gateup:
@@ -68,5 +69,7 @@ def test_software_pipelined_256_tile(dtype, n, k, tokens, gateup):
         torch.cuda.synchronize()
         outs[choice] = y
     _lib.check(lib.mui_tune_prefill(0, 0), "mui_tune_prefill")
-    assert_parity(outs[4], ref, 1e-2, f"pipelined 256 x 256 tile {dtype} {tokens}x{n}x{k} gateup={gateup}")
+    for choice in (4, 7, 8):
+        assert_parity(outs[choice], ref, 1e-2, f"pipelined tile choice {choice} {dtype} {tokens}x{n}x{k} gateup={gateup}")
     assert torch.equal(outs[4], outs[13]) and torch.equal(outs[4], outs[104])
+    assert torch.equal(outs[7], outs[207]) and torch.equal(outs[8], outs[208]) and torch.equal(outs[4], outs[7])
