@@ -65,6 +65,18 @@ __device__ __forceinline__ f32x4 xs_load(const float* src) {
                __uint_as_float((uint32_t)(b >> 32))};
 }
 
+// SiLU(g) * u of the gate/up epilogues, the product rounded to fp32 before it is rounded to the 16-bit
+// type. Left alone the compiler merges the product and the conversion into one mixed-precision
+// instruction (v_fma_mixlo_f16) for some outputs and not for others, depending on the code around
+// them, and the instruction does not round like the pair it replaces: two kernels of the same tile
+// then differ in the last place of a few outputs in a hundred thousand. The empty asm keeps the
+// product a value of its own.
+__device__ __forceinline__ float gateup_f32(float g, float u) {
+  float r = silu_f32(g) * u;
+  asm volatile("" : "+v"(r));
+  return r;
+}
+
 // XS: K is also split over p.k_splits workgroups per tile (short prompts on matrices of few row
 // tiles, where one workgroup per tile would leave most CUs idle and a long K to each): every
 // workgroup delivers its partial tile in fp32 and counts itself in; whoever arrives last adds the
@@ -597,6 +609,97 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   const int tok_l = wt * 16 * WT + (lane & 15);
   const int sub = (lane >> 4) * 4;
   constexpr int OT = (EPI == SK_GATEUP) ? WR / 2 : WR;  // output row tiles per wave
+  // Whole tiles of the software-pipelined kernels leave through LDS: a lane's accumulators are four
+  // outputs of one token (8 bytes of a row of y, sixteen rows per store instruction), which reaches
+  // memory as 32-byte pieces -- and the residual the same way. Instead the wave's block of y goes
+  // through a wave-private LDS tile [token][output] (the operand stages are free by now) and is
+  // loaded / stored 16 bytes per lane in whole rows of the wave tile (128 bytes per token with 64
+  // outputs per wave): the residual rows come in that way, are picked up in accumulator layout,
+  // replaced in place by the rounded results and leave that way. 64 tokens per pass. Chunk c of
+  // row r sits in slot (c + r) % 8 of its 128-byte LDS row.
+  if constexpr (PIPE) {
+    constexpr int OW = 16 * OT;                  // outputs per wave
+    constexpr int CE = OW / 8;                   // 16-byte chunks per row of the wave's block
+    constexpr int LPR = CE > 4 ? 8 : 4;          // lanes per row in the row-wise phases
+    constexpr int RPI = kWave / LPR;             // rows per row-wise instruction
+    constexpr int JG = WT < 4 ? WT : 4;          // token tiles of 16 per pass
+    constexpr int NI = 16 * JG / RPI;            // row-wise instructions per pass
+    static_assert(!PIPE || (WT % JG == 0 && CE <= 8 && (size_t)kNWaves * 16 * JG * 128 <= (size_t)NBUF * (sizeof(WStage) + sizeof(XStage))),
+                  "the waves' epilogue tiles fit the operand stages");
+    const bool whole = t0 + TOKS <= p.tokens && o0 + OUT_TILE <= p.n && (p.n & 7) == 0 &&
+                       (((uintptr_t)p.y | (uintptr_t)p.residual) & 15) == 0;  // uniform
+    if (whole) {
+      __builtin_amdgcn_s_waitcnt(0x0070);  // this wave's last (unused) loads have landed, its reads returned
+      __syncthreads();                     // ... and everybody's: the stages are free
+      unsigned char* et = pf_smem + (size_t)wave_u * (16 * JG * 128);
+      const int ow0 = o0 + wr * OW;                    // first output of the wave
+      const int rrow = lane / LPR, rch = lane % LPR;   // row-wise phases: row inside an instruction, chunk
+      const int arow = lane & 15, ag = lane >> 4;      // accumulator layout: token row, group of four outputs
+#pragma unroll
+      for (int j0 = 0; j0 < WT; j0 += JG) {
+        const int tw0 = t0 + wt * 16 * WT + 16 * j0;   // first token of the pass
+        if constexpr (EPI != SK_GATEUP) {
+          if (p.residual) {
+            u32x4 rr[NI];
+#pragma unroll
+            for (int it = 0; it < NI; ++it) {
+              const int row = it * RPI + rrow;
+              rr[it] = ld16(p.residual + (long)(tw0 + row) * p.n + ow0 + (rch < CE ? rch : 0) * 8);
+            }
+#pragma unroll
+            for (int it = 0; it < NI; ++it) {
+              const int row = it * RPI + rrow;
+              if (rch < CE) *(u32x4*)(et + row * 128 + ((rch + row) & 7) * 16) = rr[it];
+            }
+          }
+        }
+#pragma unroll
+        for (int jj = 0; jj < JG; ++jj) {
+          const int j = j0 + jj;
+          const int row = 16 * jj + arow;
+#pragma unroll
+          for (int i = 0; i < OT; ++i) {
+            unsigned char* slot = et + row * 128 + (((2 * i + (ag >> 1)) + row) & 7) * 16 + (ag & 1) * 8;
+            float v[4];
+            float res4[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (EPI != SK_GATEUP) {
+              if (p.residual) {
+                const u32x2 rq = *(const u32x2*)slot;
+                res4[0] = T::one((uint16_t)(rq.x & 0xffffu)); res4[1] = T::one((uint16_t)(rq.x >> 16));
+                res4[2] = T::one((uint16_t)(rq.y & 0xffffu)); res4[3] = T::one((uint16_t)(rq.y >> 16));
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int oe = ow0 + 16 * i + 4 * ag + e;
+              if constexpr (EPI == SK_GATEUP) {
+                v[e] = gateup_f32(acc[i][j][e], acc[i + OT][j][e]);
+              } else {
+                float r = acc[i][j][e];
+                if (p.mul_bias) r *= T::one(p.mul_bias[oe]);
+                if (p.add_bias) r += T::one(p.add_bias[oe]);
+                if (p.residual) r += res4[e];
+                v[e] = r;
+              }
+            }
+            u32x2 pk;
+            pk.x = (uint32_t)T::pack(v[0]) | ((uint32_t)T::pack(v[1]) << 16);
+            pk.y = (uint32_t)T::pack(v[2]) | ((uint32_t)T::pack(v[3]) << 16);
+            *(u32x2*)slot = pk;
+          }
+        }
+#pragma unroll
+        for (int it = 0; it < NI; ++it) {
+          const int row = it * RPI + rrow;
+          if (rch < CE) {
+            const u32x4 out = *(const u32x4*)(et + row * 128 + ((rch + row) & 7) * 16);
+            *(u32x4*)(p.y + (long)(tw0 + row) * p.n + ow0 + rch * 8) = out;
+          }
+        }
+      }
+      return;
+    }
+  }
   // The four residual values of a lane and tile are adjacent: one 8-byte load where the row allows
   // it, and all of a wave's loads requested before the first store (y may be the residual itself:
   // every lane reads exactly what it writes later; behind a store the compiler has to keep a load
@@ -650,7 +753,7 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
             g *= T::one(p.s0[(long)oe * p.s_pitch]);
             u *= T::one(p.s1[(long)oe * p.s_pitch]);
           }
-          v[e] = silu_f32(g) * u;
+          v[e] = gateup_f32(g, u);
         } else {
           float r = acc[i][j][e] * rs;
           if constexpr (WF == WF_I8_CHANNEL) r *= T::one(p.s0[(long)oe * p.s_pitch]);
