@@ -210,27 +210,28 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   const int n_steps = (p.k + KS - 1) / KS;
   // DMA: per wave instruction q the source of this lane's slot (fixed but for the k-step's offset)
   constexpr int kNWaves = kPfThreads / 64;
-  constexpr int WQ = DMA ? ROWS / (8 * kNWaves) : 1, XQ = DMA ? TOKS / (8 * kNWaves) : 1;
+  constexpr int DRI = 64 / CPR;  // tile rows per load instruction (8 with k-steps of 64, 4 with 128, 2 with 256)
+  constexpr int WQ = DMA ? ROWS / (DRI * kNWaves) : 1, XQ = DMA ? TOKS / (DRI * kNWaves) : 1;
   // per wave instruction q: a base address that is the same for the wave's lanes (the matrix, or the
   // up matrix for the instructions that cover up rows: eight consecutive tile rows never straddle
   // the two) and this lane's 32-bit byte offset from it; only the base moves with the k-step
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   unsigned dma_wo[WQ], dma_xo[XQ];
   if constexpr (DMA) {
-    static_assert(!DMA || (WF == WF_16BIT && !NORM && NBUF == 2 && NWK == 1 && !XS && CPR == 8), "what the DMA path covers");
-    static_assert(!DMA || (WQ * 8 * kNWaves == ROWS && XQ * 8 * kNWaves == TOKS), "whole 8-row blocks per wave");
-    static_assert(!DMA || EPI != SK_GATEUP || (8 * WR) % 8 == 0, "gate and up rows change at multiples of eight tile rows");
-    const int sr = lane >> 3, sc = lane & 7;
+    static_assert(!DMA || (WF == WF_16BIT && !NORM && NBUF >= 2 && !XS && CPR >= 8 && CPR <= 64), "what the DMA path covers");
+    static_assert(!DMA || (WQ >= 1 && XQ >= 1 && WQ * DRI * kNWaves == ROWS && XQ * DRI * kNWaves == TOKS), "whole 1 KB blocks per wave");
+    static_assert(!DMA || EPI != SK_GATEUP || (8 * WR) % DRI == 0, "gate and up rows change at multiples of a block's rows");
+    const int sr = lane / CPR, sc = lane % CPR;
 #pragma unroll
     for (int q = 0; q < WQ; ++q) {
-      const int r = (q * kNWaves + wave) * 8 + sr;
+      const int r = (q * kNWaves + wave) * DRI + sr;
       bool up;
       const int o = weight_row(r, up);
       dma_wo[q] = (unsigned)((long)o * p.pitch + ((sc ^ swz(r)) * 16));
     }
 #pragma unroll
     for (int q = 0; q < XQ; ++q) {
-      const int r = (q * kNWaves + wave) * 8 + sr;
+      const int r = (q * kNWaves + wave) * DRI + sr;
       int tk = t0 + r;
       tk = tk < p.tokens ? tk : p.tokens - 1;
       dma_xo[q] = (unsigned)((long)tk * p.k * 2 + ((sc ^ swz(r)) * 16));
@@ -244,19 +245,19 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
     if (i < WQ) {
       const int q = i;
       bool up;
-      weight_row((q * kNWaves + wave_u) * 8, up);
+      weight_row((q * kNWaves + wave_u) * DRI, up);
       const uint8_t* base = ((EPI == SK_GATEUP && up) ? p.w1 : p.w0) + kb;
       unsigned off = dma_wo[q];
       asm volatile("" : "+v"(off));
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off),
-                                       (__attribute__((address_space(3))) void*)&w_lds[buf][(q * kNWaves + wave_u) * 8 * PITCH],
+                                       (__attribute__((address_space(3))) void*)&w_lds[buf][(q * kNWaves + wave_u) * DRI * PITCH],
                                        16, 0, 0);
     } else {
       const int q = i - WQ;
       unsigned off = dma_xo[q];
       asm volatile("" : "+v"(off));
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)((const uint8_t*)p.x + kb + off),
-                                       (__attribute__((address_space(3))) void*)&x_lds[buf][(q * kNWaves + wave_u) * 8 * PITCH],
+                                       (__attribute__((address_space(3))) void*)&x_lds[buf][(q * kNWaves + wave_u) * DRI * PITCH],
                                        16, 0, 0);
     }
   };
@@ -451,15 +452,26 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
       if constexpr (WR > 3) region(std::integral_constant<int, 3>{});
     }
   } else if constexpr (DMA) {
-    dma_step(sb, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's blocks of the step are in LDS
-    __syncthreads();
+    // NBUF stages, NBUF - 1 k-steps of loads in flight. Every pass issues a step's loads -- past the
+    // last step the last one once more, into a stage nobody reads any more --, so that "all but the
+    // newest (NBUF - 2) steps' loads" is a fixed count to wait for (loads return in order). (Used with
+    // two stages; three stages on the short prompts' tiles whose waves split K lost to their
+    // register-staged loops.)
+    constexpr int LEAD = NBUF - 1;
+    static_assert(!DMA || PIPE || (LEAD - 1) * (WQ + XQ) <= 15, "the wait's load count");
+#pragma unroll
+    for (int a = 0; a < LEAD; ++a) dma_step(sb + a < se ? sb + a : se - 1, a);
+    int buf = 0, fill = LEAD;  // stage of step s; stage that step s + LEAD goes to (= the one step s - 1 used)
     for (int s = sb; s < se; ++s) {
-      if (s + 1 < se) dma_step(s + 1, (s + 1 - sb) & 1);  // the other stage: last read before the barrier just passed
-      multiply((s - sb) & 1);
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((LEAD - 1) * (WQ + XQ)));  // this wave's blocks of step s have landed
+      __syncthreads();  // ... and everybody's; everybody is done reading step s - 1
+      dma_step(s + LEAD < se ? s + LEAD : se - 1, fill);
+      multiply(buf);
+      buf = buf + 1 == NBUF ? 0 : buf + 1;
+      fill = fill + 1 == NBUF ? 0 : fill + 1;
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();  // the stages are free (and no load is still on its way into them)
   } else if constexpr (NBUF == 2) {
     load_step(sb, r0);
     // two LDS stages: step s + 1 moves from the registers to the other stage and step s + 2 is
@@ -787,10 +799,10 @@ static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 1
 static int g_prefill_pipe_small = 1;  // experiments: the pipelined loop on the 128 x 256 and 192 x 256 tiles too
 static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
 
-// what the LDS-direct loads need: whole k-steps of 64, 16-byte aligned rows, 32-bit byte offsets from
+// what the LDS-direct loads need: whole k-steps, 16-byte aligned rows, 32-bit byte offsets from
 // the operands' bases
-static bool lds_direct_loads_serve(const PrefillGemmParams& p) {
-  return g_prefill_dma && p.k % 64 == 0 && p.pitch % 16 == 0 && (long)p.n * p.pitch < (1L << 32) &&
+static bool lds_direct_loads_serve(const PrefillGemmParams& p, int k_step = 64) {
+  return g_prefill_dma && p.k % k_step == 0 && p.pitch % 16 == 0 && (long)p.n * p.pitch < (1L << 32) &&
          (long)p.tokens * p.k * 2 < (1L << 32);
 }
 static bool pipelined_loop_serves(const PrefillGemmParams& p) { return lds_direct_loads_serve(p); }
