@@ -77,7 +77,9 @@ int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
 int mui_tune_prefill(int tile, int wide_max_tokens);
 
 /* Prompt attention (mui_prefill_attention): fewest query tokens that take the kernel sharing each
- * K/V block between all query heads of a KV head (0 = built-in choice, negative = never) */
+ * K/V block between all query heads of a KV head (0 = built-in choice, negative = never);
+ * 1000000 + n: the same as n, and that kernel stages its K/V rows through registers instead of
+ * loading them straight into LDS */
 int mui_tune_prefill_attention(int group_kernel_min_tokens);
 
 /* Cache warming by the idle workgroups of the unsplit decode-attention launch

@@ -979,16 +979,38 @@ __global__ void __launch_bounds__(NW * kWave) attn_prefill_mfma_kernel(const Pre
 // ---------------------------------------------------------------------------------------
 constexpr int kPgTok = 64;  // tokens per LDS block
 
-template <typename T, int G, bool MASKED>
+// DMA: the K and V rows of a block go from global memory straight into one of TWO LDS tile pairs
+// (global_load_lds_dwordx4: a wave instruction delivers four whole 256-byte rows), the block after
+// the current one while the current one is multiplied: no staging registers, no copy into LDS
+// between two barriers (a fifth of a block's time), one barrier per block. The rows are unpadded;
+// 16-byte chunk c of row r sits in chunk slot c ^ (r % 16), applied on the global side of the load
+// and in every LDS address (the sixteen rows of an operand read, and the rows of a transposing
+// read, then fall into different banks). Needs 16-byte aligned cache rows.
+extern __shared__ __align__(16) unsigned char pg_smem[];
+template <typename T, int G, bool MASKED, bool DMA = false>
 __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) attn_prefill_group_kernel(const PrefillParams p) {
   constexpr int NW = (G == 8) ? 8 : 4;
   constexpr int kThreads = NW * kWave;
   constexpr int PB = NW / G;           // blocks of 32 query positions per workgroup
   constexpr int POS = PB * 32;
   constexpr int LCH = kPgTok * 16 / kThreads;  // 16-byte chunks of K (and of V) per thread and block
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[kPgTok][kMfKStride];
-  __shared__ __attribute__((aligned(16))) uint16_t v_lds[kPgTok][kMfVStride];
-  __shared__ __attribute__((aligned(16))) uint16_t hidden_lds[MASKED ? kPgTok : 8];  // mask entries of the block
+  constexpr int KROW = DMA ? kHeadDim : kMfKStride, VROW = DMA ? kHeadDim : kMfVStride;  // elements per LDS row
+  constexpr int NST = DMA ? 2 : 1;                                                      // LDS stages
+  __shared__ __attribute__((aligned(16))) uint16_t k_static[DMA ? 8 : kPgTok * kMfKStride];
+  __shared__ __attribute__((aligned(16))) uint16_t v_static[DMA ? 8 : kPgTok * kMfVStride];
+  uint16_t* k_lds = DMA ? (uint16_t*)pg_smem : k_static;                                // [NST][kPgTok][KROW]
+  uint16_t* v_lds = DMA ? (uint16_t*)pg_smem + NST * kPgTok * KROW : v_static;          // [NST][kPgTok][VROW]
+  __shared__ __attribute__((aligned(16))) uint16_t hidden_lds[MASKED ? NST * kPgTok : 8];  // mask entries of the block
+  int cur = 0;  // stage the current block is in
+  // element offset of 16-bit element `col` of row `row` of the current K / V tile
+  auto k_at = [&](int row, int col) -> const uint16_t* {
+    if constexpr (DMA) return k_lds + (cur * kPgTok + row) * KROW + ((((col >> 3) ^ row) & 15) << 3) + (col & 7);
+    else return k_lds + row * KROW + col;
+  };
+  auto v_at = [&](int row, int col) -> const uint16_t* {
+    if constexpr (DMA) return v_lds + (cur * kPgTok + row) * VROW + ((((col >> 3) ^ row) & 15) << 3) + (col & 7);
+    else return v_lds + row * VROW + col;
+  };
 
   const int tile = gridDim.y - 1 - blockIdx.y;  // long key ranges first
   const int kvh = blockIdx.x % p.hkv, b = blockIdx.x / p.hkv;
@@ -1045,16 +1067,47 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
 #pragma unroll
     for (int u = 0; u < LCH; ++u) {
       const int c = t + kThreads * u;
-      *(u32x4*)&k_lds[c >> 4][(c & 15) * 8] = kreg[u];
-      *(u32x4*)&v_lds[c >> 4][(c & 15) * 8] = vreg[u];
+      *(u32x4*)&k_lds[(c >> 4) * KROW + (c & 15) * 8] = kreg[u];
+      *(u32x4*)&v_lds[(c >> 4) * VROW + (c & 15) * 8] = vreg[u];
     }
     if constexpr (MASKED) {
       if (t < 16) *(u32x2*)&hidden_lds[4 * t] = hreg;
     }
   };
+  // DMA: the block's 16 + 16 groups of four rows are dealt to the waves; lane l of an instruction
+  // fills chunk slot l % 16 of row l / 16 of its group
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto dma_block = [&](int base, int stage) {
+    constexpr int NI = 16 / NW;  // instructions per wave and tile
+#pragma unroll
+    for (int q = 0; q < NI; ++q) {
+      const int grp = q * NW + wave_u;
+      const int row = 4 * grp + (lane >> 4);
+      const int tok = base + row;
+      // rows past the key range read row 0 (their scores are masked)
+      const long off = (long)(tok < kv_end ? tok : 0) * p.c_ts + (((lane ^ row) & 15) << 3);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kc + off),
+                                       (__attribute__((address_space(3))) void*)(k_lds + (stage * kPgTok + 4 * grp) * KROW),
+                                       16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vc + off),
+                                       (__attribute__((address_space(3))) void*)(v_lds + (stage * kPgTok + 4 * grp) * VROW),
+                                       16, 0, 0);
+    }
+  };
+  auto load_hidden = [&](int base) {  // DMA path: the mask entries still travel through a register
+    if constexpr (MASKED) {
+      const int m0 = base + 4 * (t & 15);
+      hreg = ld8(mrow + (m0 < kv_end ? m0 : 0));
+    }
+  };
 
   const int n_blk = (kv_end + kPgTok - 1) / kPgTok;
-  load_block(0);
+  if constexpr (DMA) {
+    dma_block(0, 0);
+    load_hidden(0);
+  } else {
+    load_block(0);
+  }
 
   // B operands: rotated q of this wave's head, positions tpos + 16 qt + i, chunk g + 4 j
   u32x4 qreg[2][4];
@@ -1082,8 +1135,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     for (int qt = 0; qt < 2; ++qt) { s1[qt] = f32x4{0.f, 0.f, 0.f, 0.f}; s2[qt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const u32x4 ka1 = *(const u32x4*)&k_lds[r0 + i][(g + 4 * j) * 8];
-      const u32x4 ka2 = *(const u32x4*)&k_lds[r0 + 16 + i][(g + 4 * j) * 8];
+      const u32x4 ka1 = *(const u32x4*)k_at(r0 + i, (g + 4 * j) * 8);
+      const u32x4 ka2 = *(const u32x4*)k_at(r0 + 16 + i, (g + 4 * j) * 8);
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) {
         s1[qt] = attn_mfma<T>(ka1, qreg[qt][j], s1[qt]);
@@ -1094,8 +1147,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     float corr[2];
     u32x2 hid[2] = {u32x2{0u, 0u}, u32x2{0u, 0u}};
     if constexpr (MASKED) {
-      hid[0] = *(const u32x2*)&hidden_lds[r0 + 4 * g];
-      hid[1] = *(const u32x2*)&hidden_lds[r0 + 16 + 4 * g];
+      hid[0] = *(const u32x2*)&hidden_lds[cur * kPgTok + r0 + 4 * g];
+      hid[1] = *(const u32x2*)&hidden_lds[cur * kPgTok + r0 + 16 + 4 * g];
     }
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
@@ -1145,8 +1198,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     }
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
-      const u32x2 lo = lds_read_tr16(&v_lds[r0 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
-      const u32x2 hi = lds_read_tr16(&v_lds[r0 + 16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+      const u32x2 lo = lds_read_tr16(v_at(r0 + 4 * g + (i >> 2), 16 * db + 4 * (i & 3)));
+      const u32x2 hi = lds_read_tr16(v_at(r0 + 16 + 4 * g + (i >> 2), 16 * db + 4 * (i & 3)));
       const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) acc[qt][db] = attn_mfma<T>(va, pb[qt], acc[qt][db]);
@@ -1171,7 +1224,7 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
-        const u32x4 ka = *(const u32x4*)&k_lds[16 * h + i][(g + 4 * j) * 8];
+        const u32x4 ka = *(const u32x4*)k_at(16 * h + i, (g + 4 * j) * 8);
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) sc4[qt][h] = attn_mfma<T>(ka, qreg[qt][j], sc4[qt][h]);
       }
@@ -1237,8 +1290,8 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     for (int half = 0; half < 2; ++half)
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
-        const u32x2 lo = lds_read_tr16(&v_lds[32 * half + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
-        const u32x2 hi = lds_read_tr16(&v_lds[32 * half + 16 + 4 * g + (i >> 2)][16 * db + 4 * (i & 3)]);
+        const u32x2 lo = lds_read_tr16(v_at(32 * half + 4 * g + (i >> 2), 16 * db + 4 * (i & 3)));
+        const u32x2 hi = lds_read_tr16(v_at(32 * half + 16 + 4 * g + (i >> 2), 16 * db + 4 * (i & 3)));
         const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) acc[qt][db] = attn_mfma<T>(va, pb[qt][half], acc[qt][db]);
@@ -1257,14 +1310,25 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
 
   for (int kb = 0; kb < n_blk; ++kb) {
     const int base = kb * kPgTok;
-    __syncthreads();  // every wave is done with the previous block
-    park();
-    __syncthreads();
-    load_block(base + kPgTok);  // in flight while this block is multiplied
+    if constexpr (DMA) {
+      cur = kb & 1;
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's rows of the block have landed (and its mask entries)
+      if constexpr (MASKED) {
+        if (t < 16) *(u32x2*)&hidden_lds[cur * kPgTok + 4 * t] = hreg;
+      }
+      __syncthreads();  // ... and everybody's; every wave is done with the block before, whose stage is free
+      dma_block(base + kPgTok, cur ^ 1);  // in flight while this block is multiplied (past the range: row 0, never read)
+      load_hidden(base + kPgTok);
+    } else {
+      __syncthreads();  // every wave is done with the previous block
+      park();
+      __syncthreads();
+      load_block(base + kPgTok);  // in flight while this block is multiplied
+    }
     // a block without hidden keys (all but the padded edge of a prompt) is handled like an unmasked one
     bool block_clear = true;
     if constexpr (MASKED) {
-      const u32x2 h4 = *(const u32x2*)&hidden_lds[4 * (lane & 15)];
+      const u32x2 h4 = *(const u32x2*)&hidden_lds[cur * kPgTok + 4 * (lane & 15)];
       block_clear = __builtin_amdgcn_ballot_w64(((h4.x | h4.y) & 0x7fff7fffu) != 0u) == 0;
     }
     // a wave whose last query cannot see the half skips it (uniform per wave; LDS reads only)
@@ -1278,6 +1342,7 @@ __global__ void __launch_bounds__((G == 8 ? 8 : 4) * kWave, (G == 8 ? 1 : 2)) at
     }
   }
 
+  if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0F70);  // the last block's (unused) successor has landed
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
     float lt = l[qt];
@@ -1563,10 +1628,29 @@ static int g_attn_min_tokens = 0;  // 0: built-in choice; else fewest tokens wor
 // prompt attention: 0 = built-in choice (the KV-group kernel from 512 query tokens), n > 0 = from n
 // tokens, negative = never
 static int g_prefill_group_tokens = 0;
+static int g_prefill_attn_direct = 1;  // 0: K / V rows staged through registers
 
 extern "C" int mui_tune_prefill_attention(int group_kernel_min_tokens) {
   MUI_TUNE_GUARD();
+  // experiments: 1000000 + n keeps the K / V rows of the KV-group kernel on the register-staged path
+  g_prefill_attn_direct = group_kernel_min_tokens >= 1000000 ? 0 : 1;
+  if (group_kernel_min_tokens >= 1000000) group_kernel_min_tokens -= 1000000;
   g_prefill_group_tokens = group_kernel_min_tokens;
+  return MUI_OK;
+}
+
+// launch of a KV-group kernel variant that needs the dynamic LDS limit raised (once per kernel and device)
+template <typename K>
+static int launch_pg_direct(K kernel, dim3 grid, int threads, int lds, hipStream_t s, const PrefillParams& p) {
+  static int raised_for = -1;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return MUI_ERR_DEVICE;
+  if (raised_for != dev) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return MUI_ERR_LAUNCH;
+    raised_for = dev;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, s, p);
   return MUI_OK;
 }
 
@@ -1914,10 +1998,19 @@ static int prefill_attention_impl(mui_stream_t stream, int dtype, const void* q_
                        (g_prefill_group_tokens > 0 ? tokens >= g_prefill_group_tokens : g_prefill_group_tokens == 0 && tokens > 256);
   if (grouped) {
     if (ceil_div(tokens, 16) > 65535) return MUI_ERR_UNSUPPORTED;  // position tiles are the grid's y
+    // K / V rows straight into LDS where every cache row is 16-byte aligned
+    const bool direct = g_prefill_attn_direct && ((((uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0) &&
+                        ((cache_batch_stride | cache_head_stride | cache_token_stride) & 7) == 0;
 #define MUI_PG_LAUNCH(TT, GG)                                                                          \
     do {                                                                                                 \
       const dim3 pg_grid(n_kv_heads * batch, ceil_div(tokens, 128 / (GG == 8 ? 4 : GG)));                 \
-      if (masked) hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, true>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p); \
+      if (direct) {                                                                                      \
+        constexpr int kDirectLds = 2 * kPgTok * 2 * kHeadDim * 2; /* two stages of a K and a V tile */   \
+        int st;                                                                                          \
+        if (masked) st = launch_pg_direct(attn_prefill_group_kernel<TT, GG, true, true>, pg_grid, (GG == 8 ? 8 : 4) * kWave, kDirectLds, s, p); \
+        else st = launch_pg_direct(attn_prefill_group_kernel<TT, GG, false, true>, pg_grid, (GG == 8 ? 8 : 4) * kWave, kDirectLds, s, p);       \
+        if (st != MUI_OK) return st;                                                                     \
+      } else if (masked) hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, true>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p); \
       else hipLaunchKernelGGL((attn_prefill_group_kernel<TT, GG, false>), pg_grid, dim3((GG == 8 ? 8 : 4) * kWave), 0, s, p);       \
     } while (0)
     if (dtype == MUI_DTYPE_F16) {

@@ -414,7 +414,7 @@ def test_prefill_attention(b, hq, hkv, t, past, dtype):
     assert _attn_err(out, ref) <= (ATOL if dtype == torch.float16 else BF16_PROMPT_ATOL)
 
 
-@pytest.mark.parametrize("choice", ["auto", "kv-group", "per-head"])
+@pytest.mark.parametrize("choice", ["auto", "kv-group", "kv-group-register-staged", "per-head"])
 @pytest.mark.parametrize("b,hq,hkv,t,past", [
     (1, 32, 8, 2048, 0),     # the kernel shared by the four query heads of a KV head
     (1, 32, 8, 1000, 24),    # ragged: not a multiple of the 32-position blocks, continues a cache
@@ -430,7 +430,7 @@ def test_prefill_attention_long_prompts(b, hq, hkv, t, past, dtype, choice):
     if dtype == torch.bfloat16 and t > 1000:
         t = 520
     lib = _lib.load()
-    _lib.check(lib.mui_tune_prefill_attention({"auto": 0, "kv-group": 1, "per-head": -1}[choice]), "tune")
+    _lib.check(lib.mui_tune_prefill_attention({"auto": 0, "kv-group": 1, "kv-group-register-staged": 1000001, "per-head": -1}[choice]), "tune")
     try:
         g = _gen(23)
         s = past + t
@@ -452,7 +452,7 @@ def test_prefill_attention_long_prompts(b, hq, hkv, t, past, dtype, choice):
         _lib.check(lib.mui_tune_prefill_attention(0), "tune")
 
 
-@pytest.mark.parametrize("choice", ["kv-group", "per-head"])
+@pytest.mark.parametrize("choice", ["kv-group", "kv-group-register-staged", "per-head"])
 @pytest.mark.parametrize("b,hq,hkv,t,past,padding", [
     (3, 32, 8, 200, 0, "left"),      # the reference's padded batches (tokenizer padding on the left)
     (2, 32, 8, 610, 0, "left"),
@@ -466,7 +466,7 @@ def test_prefill_attention_key_padding_mask(b, hq, hkv, t, past, padding, dtype,
     (muillm/modules/models/llama/model.py:437-613): every row that sees a key; rows that see none
     (padding queries of a left-padded row) come out as zeros."""
     lib = _lib.load()
-    _lib.check(lib.mui_tune_prefill_attention({"kv-group": 1, "per-head": -1}[choice]), "tune")
+    _lib.check(lib.mui_tune_prefill_attention({"kv-group": 1, "kv-group-register-staged": 1000001, "per-head": -1}[choice]), "tune")
     try:
         g = _gen(29)
         s = past + t
@@ -526,13 +526,15 @@ def test_prefill_attention_8k_rows_vs_oracle_and_kernels_agree():
     q, kc, vc = _mk((1, 32, t, D), g), _mk((1, 8, t, D), g), _mk((1, 8, t, D), g)
     qd, kd, vd = q.to(DEV), kc.to(DEV), vc.to(DEV)
     outs = {}
-    for name, knob in (("kv-group", 1), ("per-head", -1)):
+    for name, knob in (("kv-group", 1), ("kv-group-register-staged", 1000001), ("per-head", -1)):
         _lib.check(lib.mui_tune_prefill_attention(knob), "tune")
         try:
             outs[name] = muillm_ext.mui_prefill_attention(qd, kd, vd)
         finally:
             _lib.check(lib.mui_tune_prefill_attention(0), "tune")
     assert float((outs["kv-group"].float() - outs["per-head"].float()).abs().max()) <= 2 * ATOL
+    # K / V rows loaded straight into LDS or staged through registers: the same arithmetic
+    assert torch.equal(outs["kv-group"], outs["kv-group-register-staged"])
     rows = torch.tensor(list(range(0, 24)) + list(range(4085, 4110)) + list(range(t - 24, t)))
     ref = oracle.decode_attention(q[:, :, rows], kc, vc, _causal_mask(t, t, 0)[:, :, rows])
     assert _max_abs(outs["kv-group"][:, rows], ref) <= ATOL
