@@ -837,11 +837,11 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   constexpr int kWaves8 = 8 * NWR * NWT * NWK;
   if constexpr (WF == WF_16BIT && NBUF == 2 && NWK == 1 && KS == 64 && ROWS % kWaves8 == 0 && TOKS % kWaves8 == 0 &&
                 (PIPE || ROWS * TOKS >= 256 * 256)) {
-    // The DMA has one k-step of lead (two LDS stages), the register-staged path two. On the 256 x 256
-    // tile a step is 2048 matrix-pipe cycles per SIMD, enough for an L2 round trip, and the DMA wins
-    // (gate/up at 4096 tokens 834 -> 800 us, down 410 -> 390 us, o_proj 136 -> 123 us, gate/up at 512
-    // 129 -> 118 us); on 128 x 256, half of that, it loses (down at 2048 tokens 264 -> 293 us, o_proj
-    // 77 -> 88 us, gate/up at 256 88 -> 99 us).
+    // LDS-direct operand loads: always with the software-pipelined loop; with the sixteen-wave loop
+    // on the 256 x 256 tile only, where a k-step (2048 matrix-pipe cycles per SIMD) covers an L2
+    // round trip (gate/up at 4096 tokens 834 -> 800 us, down 410 -> 390 us, o_proj 136 -> 123 us);
+    // with that loop on 128 x 256, half of that, they lose (down at 2048 tokens 264 -> 293 us,
+    // o_proj 77 -> 88 us, gate/up at 256 88 -> 99 us).
     if (lds_direct_loads_serve(p))
       return launch(prefill_gemm_kernel<T, WF, false, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, false, true, PIPE>);
   }
@@ -965,8 +965,10 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
       which = (tiles(64, 128) >= want || EPI == SK_GATEUP) ? 2 : 3;
     }
   }
-  // Sixteen waves per workgroup (four per SIMD, at most 128 registers each) on all but the smallest
-  // shapes: 3-16 % ahead of eight waves with twice the wave tile, although a wave then reads 8
+  // Where the software-pipelined eight-wave loop does not apply (fused norm, int8 weights, K not a
+  // multiple of 64): sixteen waves per workgroup (four per SIMD, at most 128 registers each) on all
+  // but the smallest shapes, with the compiler's own schedule 3-16 % ahead of eight waves with twice
+  // the wave tile, although a wave then reads 8
   // instead of 6 KB of operands per 16 matrix instructions -- more waves to fill the gaps between
   // a step's phases (256 x 256: o_proj at 2048 tokens 115 -> 104 us, down 375 -> 323 us, gate/up at
   // 4096 881 -> 854 us; 128 x 256: 75 -> 68 us per round; 128 x 128 splitting K: 46 -> 42 us).
