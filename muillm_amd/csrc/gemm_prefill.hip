@@ -103,10 +103,8 @@ __device__ __forceinline__ float gateup_f32(float g, float u) {
 // save over sixteen (192 instead of 256 KB per k-step).
 template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF,
           bool XS = false, bool DMA = false, bool PIPE = false>
-// (twelve waves: three per SIMD, so let the compiler use the registers of three)
-__global__ void __launch_bounds__(64 * NWR * NWT * NWK)
-    __attribute__((amdgpu_waves_per_eu(1, (NWR * NWT * NWK == 12) ? 3 : 8)))
-    prefill_gemm_kernel(const PrefillGemmParams p) {
+// one tile: the work of workgroup id `vb` of a grid of one workgroup per tile
+__device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, const unsigned vb) {
   constexpr int kPfThreads = 64 * NWR * NWT * NWK;
   static_assert(!XS || (!NORM && EPI == SK_LINEAR && NBUF == 2), "workgroups that split K: plain linear, two stages");
   static_assert((KS / 32) % NWK == 0 && WT % NWK == 0, "k-split of the waves");
@@ -155,11 +153,25 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   // 8 XCDs, so ids that share id % 8 share an L2; give each XCD whole row tiles
   // (XS: the share of K is the fastest index -- with 8 shares it is the XCD, whose L2 then holds
   // one k-range of x for all row tiles)
-  const int xs_share = XS ? (int)(blockIdx.x % (unsigned)p.k_splits) : 0;
-  const int xs_tile = XS ? (int)(blockIdx.x / (unsigned)p.k_splits) : 0;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int tile_n = XS ? xs_tile / p.t_tiles : (slot / p.t_tiles) * 8 + xcd;
-  const int tile_t = XS ? xs_tile % p.t_tiles : slot % p.t_tiles;
+  const int xs_share = XS ? (int)(vb % (unsigned)p.k_splits) : 0;
+  const int xs_tile = XS ? (int)(vb / (unsigned)p.k_splits) : 0;
+  const int xcd = vb & 7, slot = vb >> 3;
+  // An XCD's slots walk its row tiles in panels of p.row_group row tiles x all token tiles, rows
+  // fastest: the 32 workgroups that an XCD runs at a time then share few row tiles AND few token
+  // tiles (4 x 8 instead of 1 x 32 at 8192 tokens), and its L2 fetches a third of the bytes.
+  int tile_n, tile_t;
+  if constexpr (XS) {
+    tile_n = xs_tile / p.t_tiles;
+    tile_t = xs_tile % p.t_tiles;
+  } else {
+    const int rows8 = (p.n_tiles + 7) >> 3;                  // row tiles of this XCD (the last may lie past the matrix)
+    const int per_panel = p.row_group * p.t_tiles;
+    const int panel = slot / per_panel, w = slot - panel * per_panel;
+    int rows_here = rows8 - panel * p.row_group;
+    rows_here = rows_here < p.row_group ? rows_here : p.row_group;
+    tile_n = (panel * p.row_group + w % rows_here) * 8 + xcd;
+    tile_t = w / rows_here;
+  }
   if (tile_n >= p.n_tiles) return;  // uniform for the workgroup, before any barrier
   const int o0 = tile_n * OUT_TILE;  // first output of the tile
   const int t0 = tile_t * TOKS;      // first token of the tile
@@ -790,6 +802,27 @@ __global__ void __launch_bounds__(64 * NWR * NWT * NWK)
   }
 }
 
+// The kernel: one tile per workgroup, or -- the software-pipelined tiles, whose grids are rounds of
+// one workgroup per CU -- a grid of at most p.persist_blocks workgroups that each walk the tiles
+// vb, vb + gridDim.x, ... (the grid is a multiple of 8, so a workgroup stays with its XCD's row
+// tiles): no new workgroup has to be set up between two tiles of a CU, and a tile's stores drain
+// while the next tile's first loads are on their way.
+template <typename T, int WF, bool NORM, int EPI, int WR, int WT, int NWR, int NWT, int NWK, int KS, int NBUF,
+          bool XS = false, bool DMA = false, bool PIPE = false>
+// (twelve waves: three per SIMD, so let the compiler use the registers of three)
+__global__ void __launch_bounds__(64 * NWR * NWT * NWK)
+    __attribute__((amdgpu_waves_per_eu(1, (NWR * NWT * NWK == 12) ? 3 : 8)))
+    prefill_gemm_kernel(const PrefillGemmParams p) {
+  if constexpr (PIPE) {
+    for (unsigned vb = blockIdx.x; vb < (unsigned)p.total_blocks; vb += gridDim.x) {
+      if (vb != blockIdx.x) __syncthreads();  // every wave has left the tile before: its LDS is free
+      prefill_gemm_tile<T, WF, NORM, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, XS, DMA, PIPE>(p, vb);
+    }
+  } else {
+    prefill_gemm_tile<T, WF, NORM, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF, XS, DMA, PIPE>(p, blockIdx.x);
+  }
+}
+
 static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 128, 2 = 64 x 128, 3 = 32 x 64, 4 = 256 x 256,
                                 // 5 = 64 x 128 on eight waves that split K four ways, 6 = 32 x 64 on four waves that split K,
                                 // 7 = 128 x 256, 8 = 192 x 256, 9 = 128 x 128 on eight waves that split K four ways,
@@ -798,6 +831,8 @@ static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 1
 
 static int g_prefill_pipe_small = 1;  // experiments: the pipelined loop on the 128 x 256 and 192 x 256 tiles too
 static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
+static int g_prefill_row_group = 4;   // row tiles per panel of an XCD's tile walk (experiments: 1 = one row tile after another)
+static int g_prefill_persistent = 1;  // experiments: 0 launches one workgroup per tile on the pipelined tiles too
 
 // what the LDS-direct loads need: whole k-steps, 16-byte aligned rows, 32-bit byte offsets from
 // the operands' bases
@@ -828,9 +863,16 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
         raised_for = dev;
       }
     }
-    hipLaunchKernelGGL(kernel, dim3((int)grid), dim3(64 * NWR * NWT * NWK), lds, s, p);
+    long blocks = grid;
+    if constexpr (PIPE) {  // a round of workgroups that walk the tiles (a multiple of 8: a workgroup keeps its XCD)
+      const long round = device_cus() / 8 * 8;
+      if (g_prefill_persistent && round >= 8 && blocks > round) blocks = round;
+    }
+    hipLaunchKernelGGL(kernel, dim3((int)blocks), dim3(64 * NWR * NWT * NWK), lds, s, p);
     return launch_status();
   };
+  p.total_blocks = (int)grid;
+  p.row_group = g_prefill_row_group;
   if constexpr (!PIPE) {
     if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
   }
@@ -1086,11 +1128,17 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   MUI_TUNE_GUARD();
   // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
   // 100 + tile keeps every operand tile on the register-staged path
+  const int row_group = tile >= 800 ? 1 : 4;   // 800 + tile: an XCD walks one row tile after another
+  if (tile >= 800) tile -= 800;
+  const int persistent = tile >= 400 ? 0 : 1;  // 400 + tile: one workgroup per tile on the pipelined tiles too
+  if (tile >= 400) tile -= 400;
   const int pipe_small = tile >= 200 ? 0 : 1;
   if (tile >= 200) tile -= 200;
   const int dma = tile >= 100 ? 0 : 1;
   if (tile >= 100) tile -= 100;
   if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_row_group = row_group;
+  mui::g_prefill_persistent = persistent;
   mui::g_prefill_pipe_small = pipe_small;
   mui::g_prefill_dma = dma;
   mui::g_prefill_tile = tile;
