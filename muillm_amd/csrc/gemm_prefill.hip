@@ -1128,8 +1128,9 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   MUI_TUNE_GUARD();
   // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
   // 100 + tile keeps every operand tile on the register-staged path
-  const int row_group = tile >= 800 ? 1 : 4;   // 800 + tile: an XCD walks one row tile after another
-  if (tile >= 800) tile -= 800;
+  // 800 + tile: an XCD walks one row tile after another; 1600 + tile / 2400 + tile: panels of 8 / 2 row tiles
+  const int row_group = tile >= 2400 ? 2 : tile >= 1600 ? 8 : tile >= 800 ? 1 : 4;
+  if (tile >= 800) tile -= tile >= 2400 ? 2400 : tile >= 1600 ? 1600 : 800;
   const int persistent = tile >= 400 ? 0 : 1;  // 400 + tile: one workgroup per tile on the pipelined tiles too
   if (tile >= 400) tile -= 400;
   const int pipe_small = tile >= 200 ? 0 : 1;
