@@ -71,7 +71,10 @@ int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
  * mui_linear_ws from sharing K between workgroups.
  * 100 + tile: the same, and no tile loads its operands straight into LDS (all are staged through
  * registers, on sixteen or twelve waves). 200 + tile: the same as tile, but 128 x 256 and 192 x 256
- * keep their sixteen / twelve waves.
+ * keep their sixteen / twelve waves. 400 + tile: the software-pipelined tiles are launched as one
+ * workgroup per tile instead of a persistent round of workgroups. 800 + tile: an XCD's workgroups
+ * walk one row tile after another instead of panels of four row tiles (1600 + tile: panels of
+ * eight, 2400 + tile: of two). The offsets add up (e.g. 1204 = 800 + 400 + 4).
  * wide_max_tokens = longest prompt served by the weight-streaming 16-rows-per-workgroup kernel
  * instead of the LDS-tiled one (0 restores the built-in choice; at most 128; negative: never) */
 int mui_tune_prefill(int tile, int wide_max_tokens);
