@@ -650,7 +650,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     constexpr int NI = 16 * JG / RPI;            // row-wise instructions per pass
     static_assert(!PIPE || (WT % JG == 0 && CE <= 8 && (size_t)kNWaves * 16 * JG * 128 <= (size_t)NBUF * (sizeof(WStage) + sizeof(XStage))),
                   "the waves' epilogue tiles fit the operand stages");
-    const bool whole = t0 + TOKS <= p.tokens && o0 + OUT_TILE <= p.n && (p.n & 7) == 0 &&
+    const bool whole = t0 + TOKS <= p.tokens && o0 + OUT_TILE <= p.n && (p.y_pitch & 7) == 0 &&
                        (((uintptr_t)p.y | (uintptr_t)p.residual) & 15) == 0;  // uniform
     if (whole) {
       __builtin_amdgcn_s_waitcnt(0x0070);  // this wave's last (unused) loads have landed, its reads returned
@@ -668,7 +668,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
 #pragma unroll
             for (int it = 0; it < NI; ++it) {
               const int row = it * RPI + rrow;
-              rr[it] = ld16(p.residual + (long)(tw0 + row) * p.n + ow0 + (rch < CE ? rch : 0) * 8);
+              rr[it] = ld16(p.residual + (long)(tw0 + row) * p.y_pitch + ow0 + (rch < CE ? rch : 0) * 8);
             }
 #pragma unroll
             for (int it = 0; it < NI; ++it) {
@@ -717,7 +717,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
           const int row = it * RPI + rrow;
           if (rch < CE) {
             const u32x4 out = *(const u32x4*)(et + row * 128 + ((rch + row) & 7) * 16);
-            *(u32x4*)(p.y + (long)(tw0 + row) * p.n + ow0 + rch * 8) = out;
+            *(u32x4*)(p.y + (long)(tw0 + row) * p.y_pitch + ow0 + rch * 8) = out;
           }
         }
       }
@@ -729,7 +729,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
   // every lane reads exactly what it writes later; behind a store the compiler has to keep a load
   // where it is). Four 2-byte loads per output, each waited for, cost the 256 x 256 tile 39 us of
   // epilogue against 10 us without a residual.
-  const bool res_quads = EPI != SK_GATEUP && p.residual != nullptr && (p.n & 3) == 0;
+  const bool res_quads = EPI != SK_GATEUP && p.residual != nullptr && (p.y_pitch & 3) == 0;
   u32x2 resq[WT][OT];
   if constexpr (EPI != SK_GATEUP) {
     if (res_quads) {
@@ -742,7 +742,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
         for (int i = 0; i < OT; ++i) {
           int o = o0 + wr * 16 * OT + 16 * i + sub;
           o = o + 3 < p.n ? o : 0;  // (never used then)
-          resq[j][i] = *(const u32x2*)(p.residual + (long)tok * p.n + o);
+          resq[j][i] = *(const u32x2*)(p.residual + (long)tok * p.y_pitch + o);
         }
       }
     }
@@ -759,7 +759,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       const int o = o0 + wr * 16 * OT + 16 * i + sub;
       if (o >= p.n) continue;
       float v[4];
-      const bool quad = o + 3 < p.n && (p.n & 3) == 0;
+      const bool quad = o + 3 < p.n && (p.y_pitch & 3) == 0;
       float res4[4] = {0.f, 0.f, 0.f, 0.f};
       if constexpr (EPI != SK_GATEUP) {
         if (res_quads && quad) {
@@ -783,11 +783,11 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
           if constexpr (WF == WF_I8_CHANNEL) r *= T::one(p.s0[(long)oe * p.s_pitch]);
           if (p.mul_bias) r *= T::one(p.mul_bias[oe]);
           if (p.add_bias) r += T::one(p.add_bias[oe]);
-          if (p.residual) r += quad ? res4[e] : T::one(p.residual[(long)tok * p.n + oe]);
+          if (p.residual) r += quad ? res4[e] : T::one(p.residual[(long)tok * p.y_pitch + oe]);
           v[e] = r;
         }
       }
-      uint16_t* dst = p.y + (long)tok * p.n + o;
+      uint16_t* dst = p.y + (long)tok * p.y_pitch + o;
       if (quad) {
         u32x2 pk;
         pk.x = (uint32_t)T::pack(v[0]) | ((uint32_t)T::pack(v[1]) << 16);
@@ -832,6 +832,7 @@ static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 1
 static int g_prefill_pipe_small = 1;  // experiments: the pipelined loop on the 128 x 256 and 192 x 256 tiles too
 static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
 static int g_prefill_row_group = 4;   // row tiles per panel of an XCD's tile walk (experiments: 1 = one row tile after another)
+static int g_prefill_bands = 1;       // experiments: 0 keeps gate/up in one launch whatever its last round holds
 static int g_prefill_persistent = 1;  // experiments: 0 launches one workgroup per tile on the pipelined tiles too
 
 // what the LDS-direct loads need: whole k-steps, 16-byte aligned rows, 32-bit byte offsets from
@@ -1016,6 +1017,29 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   // 4096 881 -> 854 us; 128 x 256: 75 -> 68 us per round; 128 x 128 splitting K: 46 -> 42 us).
   // int8 rows hold a quarter of the 16-byte chunks per k-step: where sixteen waves would leave
   // threads without a chunk to stage, the int8 kernels keep eight.
+  if constexpr (WF == WF_16BIT && EPI == SK_GATEUP) {
+    // Gate/up whose 256 x 256 tiles end in a round that is at most half full (2048 tokens: 896 tiles
+    // = 3.5 rounds of 256 CUs): the outputs of the whole rounds in one launch, the rest as one round
+    // of 128 x 256 tiles in a second one (a half-empty round of the big tile costs as much as a full
+    // one, a round of the small tile two thirds of it).
+    if (g_prefill_tile == 0 && g_prefill_bands && which == 4 && !p.gamma && pipelined_loop_serves(p)) {
+      const long tt = ceil_div(p.tokens, 256), row_tiles = ceil_div(p.n, 128);
+      if (cus % tt == 0 && cus / tt >= 2) {
+        const long per_round = cus / tt, whole_rows = row_tiles / per_round * per_round, rest = row_tiles - whole_rows;
+        if (whole_rows > 0 && rest > 0 && 2 * rest <= per_round) {
+          PrefillGemmParams a = p, b = p;
+          a.n = (int)(whole_rows * 128);
+          b.n = p.n - a.n;
+          b.w0 += (long)a.n * p.pitch;
+          b.w1 += (long)a.n * p.pitch;
+          b.y += a.n;
+          int st = launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, a);
+          if (st == MUI_OK) st = launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, b);
+          if (st != MUI_ERR_UNSUPPORTED) return st;
+        }
+      }
+    }
+  }
   if constexpr (WF == WF_16BIT) {
     // 256 x 256 on 4 x 2 waves of 64 x 128 with two operand register sets (the software-pipelined
     // loop): where its loads can go straight into LDS it is 5-8 % ahead of the sixteen waves below
@@ -1089,7 +1113,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
   p.w0 = (const uint8_t*)q.w0; p.w1 = (const uint8_t*)q.w1; p.pitch = q.pitch * esz;
   p.s0 = q.s0; p.s1 = q.s1; p.s_pitch = q.s_pitch;
   p.x = q.x; p.gamma = q.gamma; p.mul_bias = q.mul_bias; p.add_bias = q.add_bias; p.residual = q.residual;
-  p.y = q.y; p.n = q.n; p.k = q.k; p.tokens = q.tokens; p.eps = q.eps;
+  p.y = q.y; p.y_pitch = q.n; p.n = q.n; p.k = q.k; p.tokens = q.tokens; p.eps = q.eps;
   // a caller-provided workspace lets a long K be shared between workgroups when the tiles are few
   // (in front of the 16-rows-per-workgroup kernel only for K beyond 8192: down at 33 tokens 31 vs 50 us)
   const bool wide_default = q.tokens <= 40 && epilogue == SK_LINEAR && ceil_div(q.n, 16) <= device_cus();
@@ -1128,6 +1152,9 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   MUI_TUNE_GUARD();
   // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
   // 100 + tile keeps every operand tile on the register-staged path
+  // 3200 + tile: gate/up stays one launch whatever its last round of tiles holds
+  const int bands = tile >= 3200 ? 0 : 1;
+  if (tile >= 3200) tile -= 3200;
   // 800 + tile: an XCD walks one row tile after another; 1600 + tile / 2400 + tile: panels of 8 / 2 row tiles
   const int row_group = tile >= 2400 ? 2 : tile >= 1600 ? 8 : tile >= 800 ? 1 : 4;
   if (tile >= 800) tile -= tile >= 2400 ? 2400 : tile >= 1600 ? 1600 : 800;
@@ -1138,6 +1165,7 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   const int dma = tile >= 100 ? 0 : 1;
   if (tile >= 100) tile -= 100;
   if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_bands = bands;
   mui::g_prefill_row_group = row_group;
   mui::g_prefill_persistent = persistent;
   mui::g_prefill_pipe_small = pipe_small;

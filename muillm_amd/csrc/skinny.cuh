@@ -44,7 +44,8 @@ struct PrefillGemmParams {
   const uint16_t* mul_bias;
   const uint16_t* add_bias;
   const uint16_t* residual;  // [tokens, n] dense
-  uint16_t* y;               // [tokens, n] dense
+  uint16_t* y;               // [tokens, n]: row pitch y_pitch elements (n unless the launch covers a band of the outputs)
+  long y_pitch;              // (the residual has the same pitch)
   int n;        // outputs (weight rows; gate/up pairs)
   int k;
   int tokens;

@@ -73,3 +73,34 @@ def test_software_pipelined_tiles(dtype, n, k, tokens, gateup):
         assert_parity(outs[choice], ref, 1e-2, f"pipelined tile choice {choice} {dtype} {tokens}x{n}x{k} gateup={gateup}")
     assert torch.equal(outs[4], outs[13]) and torch.equal(outs[4], outs[104])
     assert torch.equal(outs[7], outs[207]) and torch.equal(outs[8], outs[208]) and torch.equal(outs[4], outs[7])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k,tokens", [
+    (4608, 256, 2048),     # 36 row tiles of the 256 x 256 tile at 8 token tiles: one whole round of 32 and a tail of 4
+    (4700, 128, 2000),     # the same with ragged outputs and tokens
+    (14336, 4096, 2048),   # the benchmark shape: 3.5 rounds
+])
+def test_gateup_whole_rounds_and_tail_in_two_launches(dtype, n, k, tokens):
+    """Gate/up whose 256 x 256 tiles end in a round that is at most half full is launched as the whole
+    rounds on that tile and the remaining outputs on 128 x 256 tiles (the built-in choice; on a
+    256-CU device these shapes take it): bit for bit what one launch on the 256 x 256 tile gives
+    (tile choice 4, checked against the oracle above), and against the oracle on the small shapes."""
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    g = _gen(12)
+    code = 0 if dtype == torch.float16 else 1
+    x = _mk((tokens, k), g, dtype=dtype)
+    wg, wu = _mk((n, k), g, 0.02, dtype=dtype), _mk((n, k), g, 0.02, dtype=dtype)
+    xd, wgd, wud = x.to(DEV), wg.to(DEV), wu.to(DEV)
+    outs = {}
+    for choice in (0, 4, 3200):
+        _lib.check(lib.mui_tune_prefill(choice, 0 if choice != 4 else -1), "mui_tune_prefill")
+        y = torch.zeros(tokens, n, dtype=dtype, device=DEV)
+        assert lib.mui_gateup_silu(s, code, wgd.data_ptr(), wud.data_ptr(), k, xd.data_ptr(), None, 0.0, y.data_ptr(), n, k, tokens) == 0
+        torch.cuda.synchronize()
+        outs[choice] = y
+    _lib.check(lib.mui_tune_prefill(0, 0), "mui_tune_prefill")
+    assert torch.equal(outs[0], outs[4]) and torch.equal(outs[0], outs[3200])
+    if k <= 256:
+        assert_parity(outs[0], oracle.gateup_silu(x, wg, wu), 1e-2, f"gate/up in two launches {dtype} {tokens}x{n}x{k}")
