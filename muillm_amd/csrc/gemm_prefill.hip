@@ -156,23 +156,28 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
   const int xs_share = XS ? (int)(vb % (unsigned)p.k_splits) : 0;
   const int xs_tile = XS ? (int)(vb / (unsigned)p.k_splits) : 0;
   const int xcd = vb & 7, slot = vb >> 3;
-  // An XCD's slots walk its row tiles in panels of p.row_group row tiles x all token tiles, rows
-  // fastest: the 32 workgroups that an XCD runs at a time then share few row tiles AND few token
-  // tiles (4 x 8 instead of 1 x 32 at 8192 tokens), and its L2 fetches a third of the bytes.
+  // The eight XCDs (each with an L2 of its own) divide the tile grid p.row_split ways by rows and
+  // 8 / p.row_split ways by tokens, interleaved: what every XCD fetches is its share of the weights
+  // and its share of x, and the split that fetches least depends on which of the two is bigger (the
+  // launcher chooses). Inside its share an XCD's slots walk panels of p.row_group row tiles x all its
+  // token tiles, rows fastest: the 32 workgroups that it runs at a time then share few row tiles AND
+  // few token tiles (4 x 8 instead of 1 x 32 at 8192 tokens), a third of the fetches again.
   int tile_n, tile_t;
   if constexpr (XS) {
     tile_n = xs_tile / p.t_tiles;
     tile_t = xs_tile % p.t_tiles;
   } else {
-    const int rows8 = (p.n_tiles + 7) >> 3;                  // row tiles of this XCD (the last may lie past the matrix)
-    const int per_panel = p.row_group * p.t_tiles;
+    const int rs = p.row_split, ts = 8 / rs;
+    const int xr = xcd % rs, xt = xcd / rs;
+    const int rows_x = (p.n_tiles + rs - 1) / rs, toks_x = (p.t_tiles + ts - 1) / ts;  // this XCD's share (its edge may lie outside)
+    const int per_panel = p.row_group * toks_x;
     const int panel = slot / per_panel, w = slot - panel * per_panel;
-    int rows_here = rows8 - panel * p.row_group;
+    int rows_here = rows_x - panel * p.row_group;
     rows_here = rows_here < p.row_group ? rows_here : p.row_group;
-    tile_n = (panel * p.row_group + w % rows_here) * 8 + xcd;
-    tile_t = w / rows_here;
+    tile_n = (panel * p.row_group + w % rows_here) * rs + xr;
+    tile_t = (w / rows_here) * ts + xt;
   }
-  if (tile_n >= p.n_tiles) return;  // uniform for the workgroup, before any barrier
+  if (tile_n >= p.n_tiles || tile_t >= p.t_tiles) return;  // uniform for the workgroup, before any barrier
   const int o0 = tile_n * OUT_TILE;  // first output of the tile
   const int t0 = tile_t * TOKS;      // first token of the tile
 
@@ -832,6 +837,7 @@ static int g_prefill_tile = 0;  // experiments: 0 = built-in choice, 1 = 128 x 1
 static int g_prefill_pipe_small = 1;  // experiments: the pipelined loop on the 128 x 256 and 192 x 256 tiles too
 static int g_prefill_dma = 1;   // 0: operand tiles staged through registers everywhere
 static int g_prefill_row_group = 4;   // row tiles per panel of an XCD's tile walk (experiments: 1 = one row tile after another)
+static int g_prefill_row_split = 0;   // experiments: 8, 4 or 2 forces the XCDs' split of the grid (0: the launcher's choice)
 static int g_prefill_bands = 1;       // experiments: 0 keeps gate/up in one launch whatever its last round holds
 static int g_prefill_persistent = 1;  // experiments: 0 launches one workgroup per tile on the pipelined tiles too
 
@@ -848,8 +854,22 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   constexpr int ROWS = 16 * WR * NWR, TOKS = 16 * WT * NWT;
   p.n_tiles = ceil_div(p.n, EPI == SK_GATEUP ? ROWS / 2 : ROWS);
   p.t_tiles = ceil_div(p.tokens, TOKS);
-  // whole row tiles per XCD: the grid covers ceil(n_tiles / 8) * 8 row tiles, the surplus exits
-  const long grid = (long)ceil_div(p.n_tiles, 8) * 8 * p.t_tiles;
+  // The XCDs' split of the grid: rows alone (8 x 1), or 4 x 2 / 2 x 4 rows x tokens where that cuts
+  // the bytes the eight L2s fetch between them -- weights x token splits + x x row splits -- by a
+  // fifth or more (down 4096 x 14336 at 4096 tokens: 0.70 instead of 1.06 GB; gate/up keeps 8 x 1).
+  p.row_split = 8;
+  if (g_prefill_row_split) {
+    p.row_split = g_prefill_row_split;
+  } else {
+    const double wb = (double)(EPI == SK_GATEUP ? 2 : 1) * p.n * p.k * (WF == WF_16BIT ? 2 : 1), xb = (double)p.tokens * p.k * 2;
+    double best = wb + 8 * xb;
+    for (int rs = 4; rs >= 2; rs /= 2) {
+      const double c = wb * (8 / rs) + xb * rs;
+      if (c < 0.8 * best && p.t_tiles >= 8 / rs * 4 && p.n_tiles >= rs * 4) { best = c; p.row_split = rs; }
+    }
+  }
+  // every XCD gets the same number of slots: its share rounded up, the surplus exits
+  const long grid = (long)ceil_div(p.n_tiles, p.row_split) * ceil_div(p.t_tiles, 8 / p.row_split) * 8;
   if (grid > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
   constexpr size_t lds = prefill_lds_bytes<ROWS, TOKS, KS, NBUF>();
   auto launch = [&](auto kernel) {
@@ -1152,6 +1172,9 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   MUI_TUNE_GUARD();
   // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
   // 100 + tile keeps every operand tile on the register-staged path
+  // 6400 + tile / 12800 + tile / 19200 + tile: the XCDs split the tile grid 8 x 1 / 4 x 2 / 2 x 4 (rows x tokens)
+  const int row_split = tile >= 19200 ? 2 : tile >= 12800 ? 4 : tile >= 6400 ? 8 : 0;
+  if (tile >= 6400) tile -= tile >= 19200 ? 19200 : tile >= 12800 ? 12800 : 6400;
   // 3200 + tile: gate/up stays one launch whatever its last round of tiles holds
   const int bands = tile >= 3200 ? 0 : 1;
   if (tile >= 3200) tile -= 3200;
@@ -1165,6 +1188,7 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   const int dma = tile >= 100 ? 0 : 1;
   if (tile >= 100) tile -= 100;
   if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_row_split = row_split;
   mui::g_prefill_bands = bands;
   mui::g_prefill_row_group = row_group;
   mui::g_prefill_persistent = persistent;

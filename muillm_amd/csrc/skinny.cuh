@@ -54,6 +54,7 @@ struct PrefillGemmParams {
   int t_tiles;  // token tiles
   // K split over workgroups (prefill_gemm_kernel<..., XS = true>): partial tiles and arrival counters
   int k_splits;
+  int row_split;          // the XCDs divide the tile grid row_split ways by rows, 8 / row_split ways by tokens
   int row_group;          // row tiles per panel of an XCD's tile walk
   int total_blocks;       // software-pipelined tiles: tiles of the launch (row tiles rounded up to 8, times token tiles)
   float* part;            // [tiles * k_splits] partial tiles in fp32
