@@ -387,6 +387,11 @@ def _byte_pitch(w: torch.Tensor, name: str) -> int:
 # about 4 ms per 8B-shaped pass, two chunks of the decode kernels less).
 INT8_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
 INT8_GROUP_CHUNK_MAX_TOKENS = 32
+# Per-channel format from this many tokens: the matrix is dequantised once per call (12–32 µs per
+# Llama-3-8B matrix) and the GEMM runs its software-pipelined loop on 16-bit weights, which the
+# converting loop cannot use (at 4096 tokens QKV 227 -> 182 µs, o_proj 128 -> 118, down 389 -> 381,
+# gate/up 817 -> 762; at 1024 tokens the conversion on the way to LDS is still ahead).
+INT8_DEQUANT_MIN_TOKENS = 2048
 
 
 def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
@@ -435,6 +440,9 @@ def mui_int8_channel_linear_forward(x, weights_i8, scales, norm_weights=None, ep
     x = x.contiguous()
     x, norm_weights = _norm_first(x, norm_weights, epsilon, INT8_CHUNK_MAX_TOKENS)
     tokens = _num_tokens(x)
+    if tokens >= INT8_DEQUANT_MIN_TOKENS and k % 16 == 0:
+        w = mui_int8_channel_dequantize_forward(weights_i8, scales)
+        return muillm_linear_forward(None, x, w, norm_weights, epsilon, None, add_bias, residual)
     if residual is not None:
         residual = residual.contiguous()
     y = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
@@ -476,6 +484,9 @@ def mui_int8_channel_gateupsilu_forward(norm_weights, epsilon, gate_i8, up_i8, g
     x = x.contiguous()
     x, norm_weights = _norm_first(x, norm_weights, epsilon, INT8_CHUNK_MAX_TOKENS)
     tokens = _num_tokens(x)
+    if tokens >= INT8_DEQUANT_MIN_TOKENS:
+        return mui_gateup_silu(norm_weights, epsilon, mui_int8_channel_dequantize_forward(gate_i8, gate_scales),
+                               mui_int8_channel_dequantize_forward(up_i8, up_scales), x)
     h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
     esz = x.element_size()
     for off, cnt in _token_chunks(tokens):

@@ -174,6 +174,41 @@ def test_int8_channel_gateup_prompt(tokens, n, k):
     assert_parity(h, ref, 1e-2, f"int8 prompt gate/up {tokens}x{n}x{k}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_int8_channel_long_prompt_dequantises_once(dtype, monkeypatch):
+    """From INT8_DEQUANT_MIN_TOKENS tokens the per-channel matrix is dequantised once per call
+    (T(float(q) * float(s)), the rounding of the dequantisation kernel) and the GEMM runs on 16-bit
+    weights. Gate 1e-2 against the oracle on the exact q * s, as for the converting GEMM, which must
+    also agree with it to 1e-2 of the output's maximum on the same inputs."""
+    g = _gen(14)
+    tokens, n, k = muillm_ext.INT8_DEQUANT_MIN_TOKENS, 520, 1024
+    q, s = oracle.rtn_quantize_channel(_mk((n, k), g, 0.02))
+    s = s.to(dtype)
+    x, gamma, r = _mk((tokens, k), g, dtype=dtype), _mk((k,), g, 0.1, 1.0, dtype=dtype), _mk((tokens, n), g, dtype=dtype)
+    ref = oracle.linear(x, q.double() * s.double()[:, None], gamma, 1e-5, None, r)
+    args = (x.to(DEV), q.to(DEV), s.to(DEV), gamma.to(DEV), 1e-5, None, r.to(DEV))
+    y = muillm_ext.mui_int8_channel_linear_forward(*args)
+    assert_parity(y, ref, 1e-2, f"int8 long prompt linear (dequantised once) {dtype}")
+    qu, su = oracle.rtn_quantize_channel(_mk((n, k), g, 0.02))
+    su = su.to(dtype)
+    refh = oracle.gateup_silu(x, q.double() * s.double()[:, None], qu.double() * su.double()[:, None], gamma, 1e-5)
+    pw = torch.stack([q, qu], dim=1).contiguous().to(DEV)
+    ps = torch.stack([s, su], dim=1).contiguous().to(DEV)
+    gargs = (gamma.to(DEV), 1e-5, pw[:, 0], pw[:, 1], ps[:, 0], ps[:, 1], x.to(DEV))
+    h = muillm_ext.mui_int8_channel_gateupsilu_forward(*gargs)
+    # bf16 gate/up: two 8-bit-mantissa operands of SiLU * mul set the elementwise floor (4e-2), as for 16-bit weights
+    assert_parity(h, refh, 1e-2, f"int8 long prompt gate/up (dequantised once) {dtype}",
+                  elementwise=None if dtype == torch.float16 else 4e-2)
+    # the same calls on the GEMM that converts the codes on their way to LDS
+    monkeypatch.setattr(muillm_ext, "INT8_DEQUANT_MIN_TOKENS", 1 << 30)
+    y2 = muillm_ext.mui_int8_channel_linear_forward(*args)
+    h2 = muillm_ext.mui_int8_channel_gateupsilu_forward(*gargs)
+    for name, a_, b_ in (("linear", y, y2), ("gate/up", h, h2)):
+        d = float((a_.float() - b_.float()).abs().max() / b_.float().abs().max())
+        print(f"[parity] int8 long prompt {name} {dtype}: dequantise-once vs converting GEMM {d:.2e} of max (gate 1e-2)")
+        assert d <= 1e-2
+
+
 @pytest.mark.parametrize("tokens", [65, 150])
 def test_int8_group_format_prompt(tokens):
     """The reference's group format at prompt sizes: dequantised by the library's kernel (bit-exact
