@@ -764,7 +764,7 @@ def _probe_prompt_whole_model():
         return (time.perf_counter() - t0) / iters * 1e3
 
     res = {}
-    for tokens in (64, 128, 512, 2048, 4096, 8192):
+    for tokens in (64, 128, 512, 1024, 2048, 4096, 8192):
         ours = run(tokens)
         muillm_ext.kernel_dispatchable = lambda x: dispatchable(x) and muillm_ext._num_tokens(x) <= 32
         try:

@@ -407,21 +407,35 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       if constexpr (TOTAL > PER * N) __builtin_amdgcn_sched_group_barrier(0x008, TOTAL - PER * N, 0);
     };
     static_assert(!PIPE || WR * WT >= 2 * (WR + WT), "two matrix instructions per read");
-    dma_step(sb, 0);
-    if (sb + 1 < se) dma_step(sb + 1, 1);
-    if (sb + 1 < se) __builtin_amdgcn_s_waitcnt(0x0F70 | (WQ + XQ));  // all but the second step's loads
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    // NBUF stages: the loads of step s + NBUF are issued in the second half of step s, into the stage
+    // that step s has just finished reading, and must have landed by the middle of step s + NBUF - 1:
+    // one k-step of lead with two stages, two with three (the 128 x 256 tile, whose k-step is too short
+    // to cover a trip to L2 under load)
+    static_assert(!PIPE || NBUF == 2 || NBUF == 3, "stages of the pipelined loop");
+    static_assert(!PIPE || (NBUF - 1) * (WQ + XQ) <= 15, "the waits' load counts");
+    if constexpr (NBUF == 2) {
+      dma_step(sb, 0);
+      if (sb + 1 < se) dma_step(sb + 1, 1);
+      if (sb + 1 < se) __builtin_amdgcn_s_waitcnt(0x0F70 | (WQ + XQ));  // all but the second step's loads
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+    } else {
+#pragma unroll
+      for (int a = 0; a < NBUF; ++a) dma_step(sb + a < se ? sb + a : se - 1, a);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((NBUF - 1) * (WQ + XQ)));    // the first step's loads
+    }
     __syncthreads();
     read_ops(0, 0, 0);
+    int buf = 0;
     for (int s = sb; s < se; ++s) {
-      const int buf = (s - sb) & 1;
+      const int nbuf = buf + 1 == NBUF ? 0 : buf + 1;
       read_ops(buf, 1, 1);
       mm(0, 0, WR);
       pin(std::integral_constant<int, 0x100>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, WR + WT>{},
           std::integral_constant<int, WR * WT>{});
       __builtin_amdgcn_sched_barrier(0);
-      // this wave's reads of the stage have returned, its share of the next stage has landed
-      __builtin_amdgcn_s_waitcnt(0x0070);
+      // this wave's reads of the stage have returned, its share of the next stage has landed (loads
+      // return in order: all but those of the NBUF - 2 steps after it)
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((NBUF - 2) * (WQ + XQ)));
       __syncthreads();
       // (the last two steps load the last step once more, into a stage that nobody reads any more,
       // and read stale operands that nobody multiplies: no branch, one schedule)
@@ -430,7 +444,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       // so that the eight waves, which all leave the barrier together, do not queue their loads
       // faster than the CU's memory pipeline takes them (a wave that waits to issue a load does not
       // issue the matrix instructions behind it either)
-      const int nxt = s + 2 < se ? s + 2 : se - 1;
+      const int nxt = s + NBUF < se ? s + NBUF : se - 1;
       // (the reads in all but the last region where they fit there: the first matrix instruction of
       // the next half waits for the last of them)
       constexpr int NL = WQ + XQ, NR = WR + WT;
@@ -446,7 +460,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
 #pragma unroll
         for (int l = 0; l < nl; ++l) dma_one(nxt, buf, i * LD + l);
 #pragma unroll
-        for (int r = 0; r < nr; ++r) read_one(buf ^ 1, 0, 0, i * RD + r);
+        for (int r = 0; r < nr; ++r) read_one(nbuf, 0, 0, i * RD + r);
         mm(1, i, i + 1);
         // a matrix instruction, a load, ..., a matrix instruction, a read, ... (loads first: they have the longer way)
 #pragma unroll
@@ -467,6 +481,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       region(std::integral_constant<int, 1>{});
       if constexpr (WR > 2) region(std::integral_constant<int, 2>{});
       if constexpr (WR > 3) region(std::integral_constant<int, 3>{});
+      buf = nbuf;
     }
   } else if constexpr (DMA) {
     // NBUF stages, NBUF - 1 k-steps of loads in flight. Every pass issues a step's loads -- past the
@@ -840,6 +855,7 @@ static int g_prefill_row_group = 4;   // row tiles per panel of an XCD's tile wa
 static int g_prefill_row_split = 0;   // experiments: 8, 4 or 2 forces the XCDs' split of the grid (0: the launcher's choice)
 static int g_prefill_bands = 1;       // experiments: 0 keeps gate/up in one launch whatever its last round holds
 static int g_prefill_persistent = 1;  // experiments: 0 launches one workgroup per tile on the pipelined tiles too
+static int g_prefill_stages3 = 1;     // experiments: 0 keeps the pipelined 128 x 256 tile on two LDS stages
 
 // what the LDS-direct loads need: whole k-steps, 16-byte aligned rows, 32-bit byte offsets from
 // the operands' bases
@@ -898,8 +914,8 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
     if (p.gamma) return launch(prefill_gemm_kernel<T, WF, true, EPI, WR, WT, NWR, NWT, NWK, KS, NBUF>);
   }
   constexpr int kWaves8 = 8 * NWR * NWT * NWK;
-  if constexpr (WF == WF_16BIT && NBUF == 2 && NWK == 1 && KS == 64 && ROWS % kWaves8 == 0 && TOKS % kWaves8 == 0 &&
-                (PIPE || ROWS * TOKS >= 256 * 256)) {
+  if constexpr (WF == WF_16BIT && (NBUF == 2 || (PIPE && NBUF == 3)) && NWK == 1 && KS == 64 && ROWS % kWaves8 == 0 &&
+                TOKS % kWaves8 == 0 && (PIPE || ROWS * TOKS >= 256 * 256)) {
     // LDS-direct operand loads: always with the software-pipelined loop; with the sixteen-wave loop
     // on the 256 x 256 tile only, where a k-step (2048 matrix-pipe cycles per SIMD) covers an L2
     // round trip (gate/up at 4096 tokens 834 -> 800 us, down 410 -> 390 us, o_proj 136 -> 123 us);
@@ -961,6 +977,17 @@ static int launch_prefill_xs(hipStream_t s, PrefillGemmParams p, int shares, voi
   return launch_status();
 }
 
+// Gate/up whose 256 x 256 tiles (128 outputs each) end in a round that is at most half full: the
+// number of row tiles that make whole rounds of workgroups, for a launch of their own -- or 0
+static long gateup_bands(const PrefillGemmParams& p) {
+  if (!g_prefill_bands) return 0;
+  const long cus = device_cus();
+  const long tt = ceil_div(p.tokens, 256), row_tiles = ceil_div(p.n, 128);
+  if (cus % tt != 0 || cus / tt < 2) return 0;
+  const long per_round = cus / tt, whole_rows = row_tiles / per_round * per_round, rest = row_tiles - whole_rows;
+  return (whole_rows > 0 && rest > 0 && 2 * rest <= per_round) ? whole_rows : 0;
+}
+
 template <typename T, int WF, int EPI>
 static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   // Big tiles re-read x and the weights least and keep the LDS traffic per matrix instruction
@@ -1004,14 +1031,19 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
       };
       // (the three big tiles cost less per round where the software-pipelined loop serves them)
       const bool pipe = WF == WF_16BIT && !p.gamma && pipelined_loop_serves(p);
-      float best = whole(tiles(256, 256), pipe ? 96.f : 100.f, pipe ? 106.f : 111.f);
+      float best = whole(tiles(256, 256), pipe ? 96.f : 100.f, pipe ? 100.f : 111.f);
       which = 4;
+      // (gate/up in two launches, see below: whole rounds of 256 x 256 and one round of 128 x 256)
+      if constexpr (WF == WF_16BIT && EPI == SK_GATEUP) {
+        if (pipe && gateup_bands(p) > 0) best = (float)((tiles(256, 256) + cus - 1) / cus - 1) * 100.f + 53.f;
+      }
       auto offer = [&](int id, float cost) {
         if (cost < best * 0.97f) { best = cost; which = id; }  // bigger tiles win ties
       };
       if (pipe && EPI == SK_LINEAR) offer(8, whole(tiles(192, 256), 74.f, 80.f));
+      else if (pipe) offer(8, whole(tiles(192, 256), 92.f, 98.f));  // gate/up: twelve waves beside pipelined 256 x 256 and 128 x 256
       else offer(8, whole(tiles(192, 256), 85.f, 92.f));
-      if (pipe) offer(7, whole(tiles(128, 256), 63.f, 66.f));
+      if (pipe) offer(7, whole(tiles(128, 256), 53.f, 58.f));  // (three LDS stages; 63 / 66 with two)
       else offer(7, whole(tiles(128, 256), WF == WF_16BIT ? 67.f : 73.f, WF == WF_16BIT ? 70.f : 76.f));
       offer(1, pairs(tiles(128, 128), 68.f, 92.f));
       if (EPI == SK_LINEAR && WF == WF_16BIT) offer(10, pairs(tiles(96, 128), 60.f, 76.f));
@@ -1042,11 +1074,10 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
     // = 3.5 rounds of 256 CUs): the outputs of the whole rounds in one launch, the rest as one round
     // of 128 x 256 tiles in a second one (a half-empty round of the big tile costs as much as a full
     // one, a round of the small tile two thirds of it).
-    if (g_prefill_tile == 0 && g_prefill_bands && which == 4 && !p.gamma && pipelined_loop_serves(p)) {
-      const long tt = ceil_div(p.tokens, 256), row_tiles = ceil_div(p.n, 128);
-      if (cus % tt == 0 && cus / tt >= 2) {
-        const long per_round = cus / tt, whole_rows = row_tiles / per_round * per_round, rest = row_tiles - whole_rows;
-        if (whole_rows > 0 && rest > 0 && 2 * rest <= per_round) {
+    if (g_prefill_tile == 0 && which == 4 && !p.gamma && pipelined_loop_serves(p)) {
+      {
+        const long whole_rows = gateup_bands(p);
+        if (whole_rows > 0) {
           PrefillGemmParams a = p, b = p;
           a.n = (int)(whole_rows * 128);
           b.n = p.n - a.n;
@@ -1054,7 +1085,8 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
           b.w1 += (long)a.n * p.pitch;
           b.y += a.n;
           int st = launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, a);
-          if (st == MUI_OK) st = launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, b);
+          if (st == MUI_OK) st = g_prefill_stages3 ? launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 3, true>(s, b)
+                                                  : launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, b);
           if (st != MUI_ERR_UNSUPPORTED) return st;
         }
       }
@@ -1074,7 +1106,9 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
   if constexpr (WF == WF_16BIT) {
     if (g_prefill_pipe_small && !p.gamma) {
       int st = MUI_ERR_UNSUPPORTED;
-      if (which == 7) st = launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, p);    // 128 x 256, 2 x 4 waves of 64 x 64
+      // 128 x 256, 2 x 4 waves of 64 x 64, three LDS stages
+      if (which == 7) st = g_prefill_stages3 ? launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 3, true>(s, p)
+                                             : launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, p);
       if constexpr (EPI == SK_LINEAR) {
         if (which == 8) st = launch_prefill_cfg<T, WF, EPI, 3, 8, 4, 2, 1, 64, 2, true>(s, p);  // 192 x 256, 4 x 2 waves of 48 x 128
       }
@@ -1173,6 +1207,8 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
   // 100 + tile keeps every operand tile on the register-staged path
   // 6400 + tile / 12800 + tile / 19200 + tile: the XCDs split the tile grid 8 x 1 / 4 x 2 / 2 x 4 (rows x tokens)
+  const int stages3 = tile >= 25600 ? 0 : 1;  // 25600 + tile: the pipelined 128 x 256 tile on two LDS stages
+  if (tile >= 25600) tile -= 25600;
   const int row_split = tile >= 19200 ? 2 : tile >= 12800 ? 4 : tile >= 6400 ? 8 : 0;
   if (tile >= 6400) tile -= tile >= 19200 ? 19200 : tile >= 12800 ? 12800 : 6400;
   // 3200 + tile: gate/up stays one launch whatever its last round of tiles holds
@@ -1188,6 +1224,7 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   const int dma = tile >= 100 ? 0 : 1;
   if (tile >= 100) tile -= 100;
   if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_stages3 = stages3;
   mui::g_prefill_row_split = row_split;
   mui::g_prefill_bands = bands;
   mui::g_prefill_row_group = row_group;
