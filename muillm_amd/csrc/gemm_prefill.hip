@@ -412,7 +412,9 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     // one k-step of lead with two stages, two with three (the 128 x 256 tile, whose k-step is too short
     // to cover a trip to L2 under load)
     static_assert(!PIPE || NBUF == 2 || NBUF == 3, "stages of the pipelined loop");
-    static_assert(!PIPE || (NBUF - 1) * (WQ + XQ) <= 15, "the waits' load counts");
+    static_assert(!PIPE || (NBUF - 1) * (WQ + XQ) <= 63, "the waits' load counts");
+    // s_waitcnt immediate for "at most n loads outstanding" (six bits: [3:0] and [15:14])
+    constexpr auto vm = [](int n) { return (n & 15) | ((n >> 4) << 14); };
     if constexpr (NBUF == 2) {
       dma_step(sb, 0);
       if (sb + 1 < se) dma_step(sb + 1, 1);
@@ -421,7 +423,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     } else {
 #pragma unroll
       for (int a = 0; a < NBUF; ++a) dma_step(sb + a < se ? sb + a : se - 1, a);
-      __builtin_amdgcn_s_waitcnt(0x0F70 | ((NBUF - 1) * (WQ + XQ)));    // the first step's loads
+      __builtin_amdgcn_s_waitcnt(0x0F70 | vm((NBUF - 1) * (WQ + XQ)));  // the first step's loads
     }
     __syncthreads();
     read_ops(0, 0, 0);
@@ -435,7 +437,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       __builtin_amdgcn_sched_barrier(0);
       // this wave's reads of the stage have returned, its share of the next stage has landed (loads
       // return in order: all but those of the NBUF - 2 steps after it)
-      __builtin_amdgcn_s_waitcnt(0x0070 | ((NBUF - 2) * (WQ + XQ)));
+      __builtin_amdgcn_s_waitcnt(0x0070 | vm((NBUF - 2) * (WQ + XQ)));
       __syncthreads();
       // (the last two steps load the last step once more, into a stage that nobody reads any more,
       // and read stale operands that nobody multiplies: no branch, one schedule)
