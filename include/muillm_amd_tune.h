@@ -77,7 +77,8 @@ int mui_tune_skinny(int min_tokens, int stream_b, int multi_max_tokens);
  * eight, 2400 + tile: of two). 3200 + tile: gate/up stays one launch whatever its last round of
  * tiles holds. 6400 / 12800 / 19200 + tile: the XCDs divide the tile grid 8 x 1 / 4 x 2 / 2 x 4 ways
  * (rows x tokens) instead of the launcher's choice. 25600 + tile: the software-pipelined 128 x 256 tile
- * keeps two LDS stages instead of three. The offsets add up (e.g. 1204 = 800 + 400 + 4).
+ * keeps two LDS stages instead of three. 51200 + tile: the software-pipelined 192 x 256 and 256 x 256 tiles
+ * keep two stages of the weight tile instead of three. The offsets add up (e.g. 1204 = 800 + 400 + 4).
  * wide_max_tokens = longest prompt served by the weight-streaming 16-rows-per-workgroup kernel
  * instead of the LDS-tiled one (0 restores the built-in choice; at most 128; negative: never) */
 int mui_tune_prefill(int tile, int wide_max_tokens);

@@ -49,6 +49,18 @@ template <int ROWS, int TOKS, int KS, int NBUF>
 constexpr size_t prefill_lds_bytes() {
   return (size_t)NBUF * (ROWS + TOKS) * KS * 2 + TOKS * 4;
 }
+// The software-pipelined loop on three stages: three of the weight tile, and of the token tile three
+// where 160 KB hold them, else two (the weights come from HBM, the token rows mostly from L2: the
+// weights get the extra k-step of lead)
+constexpr size_t kLdsPerWorkgroup = 160 * 1024;
+template <int ROWS, int TOKS, int KS, int NBUF>
+constexpr int pipe_x_stages() {
+  return (NBUF == 3 && prefill_lds_bytes<ROWS, TOKS, KS, 3>() > kLdsPerWorkgroup) ? 2 : NBUF;
+}
+template <int ROWS, int TOKS, int KS, int NBUF>
+constexpr size_t pipe_lds_bytes() {  // (no fused norm in this loop: no per-token sums behind the stages)
+  return (size_t)(NBUF * ROWS + pipe_x_stages<ROWS, TOKS, KS, NBUF>() * TOKS) * KS * 2;
+}
 
 // partial tiles between workgroups: agent-scope relaxed atomics (write-through stores, loads that
 // bypass the non-coherent caches; the XCDs do not share an L2)
@@ -137,8 +149,9 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
   typedef uint16_t WStage[ROWS * PITCH];
   typedef uint16_t XStage[TOKS * PITCH];
   WStage* w_lds = (WStage*)pf_smem;
+  constexpr int XB = PIPE ? pipe_x_stages<ROWS, TOKS, KS, NBUF>() : NBUF;  // stages of the token tile
   XStage* x_lds = (XStage*)(pf_smem + (size_t)NBUF * sizeof(WStage));
-  float* rs_lds = (float*)(pf_smem + (size_t)NBUF * (sizeof(WStage) + sizeof(XStage)));
+  float* rs_lds = (float*)(pf_smem + (size_t)NBUF * sizeof(WStage) + (size_t)XB * sizeof(XStage));  // (NORM only)
 
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
@@ -348,7 +361,9 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
   for (int i = 0; i < WR; ++i)
 #pragma unroll
     for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int i = t; i < TOKS; i += kPfThreads) rs_lds[i] = 0.f;
+  if constexpr (NORM) {
+    for (int i = t; i < TOKS; i += kPfThreads) rs_lds[i] = 0.f;
+  }
 
   const int a_base = (wr * 16 * WR + (lane & 15)) * PITCH;  // rows 16 i + lane % 16: the swizzle depends on the lane only
   const int b_base = (wt * 16 * WT + (lane & 15)) * PITCH;
@@ -380,13 +395,14 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     static_assert(!PIPE || (KS == 64 && NWK == 1), "two halves per k-step");
     u32x4 a[2][WR], b[2][WT];
     // operand read i of a half step: the WT token operands first, then the WR weight operands
-    auto read_one = [&](int buf, int kk, int set, int i) {
-      if (i < WT) b[set][i] = *(const u32x4*)&x_lds[buf][b_base + i * 16 * PITCH + (((kk * 4 + lg) ^ lsw) * 8)];
-      else a[set][i - WT] = *(const u32x4*)&w_lds[buf][a_base + (i - WT) * 16 * PITCH + (((kk * 4 + lg) ^ lsw) * 8)];
+    // (bw / bx: the stage of the weight tile / of the token tile)
+    auto read_one = [&](int bw, int bx, int kk, int set, int i) {
+      if (i < WT) b[set][i] = *(const u32x4*)&x_lds[bx][b_base + i * 16 * PITCH + (((kk * 4 + lg) ^ lsw) * 8)];
+      else a[set][i - WT] = *(const u32x4*)&w_lds[bw][a_base + (i - WT) * 16 * PITCH + (((kk * 4 + lg) ^ lsw) * 8)];
     };
-    auto read_ops = [&](int buf, int kk, int set) {
+    auto read_ops = [&](int bw, int bx, int kk, int set) {
 #pragma unroll
-      for (int i = 0; i < WT + WR; ++i) read_one(buf, kk, set, i);
+      for (int i = 0; i < WT + WR; ++i) read_one(bw, bx, kk, set, i);
     };
     auto mm = [&](int set, int i0, int i1) {
 #pragma unroll
@@ -410,7 +426,10 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     // NBUF stages: the loads of step s + NBUF are issued in the second half of step s, into the stage
     // that step s has just finished reading, and must have landed by the middle of step s + NBUF - 1:
     // one k-step of lead with two stages, two with three (the 128 x 256 tile, whose k-step is too short
-    // to cover a trip to L2 under load)
+    // to cover a trip to L2 under load). Where 160 KB do not hold three stages of both tiles the token
+    // tile keeps two (XB): a step then issues the token loads of step s + 2 FIRST and the weight loads
+    // of step s + 3 after them, so that "all but the newest WQ loads" is what the middle of the next
+    // step waits for.
     static_assert(!PIPE || NBUF == 2 || NBUF == 3, "stages of the pipelined loop");
     static_assert(!PIPE || (NBUF - 1) * (WQ + XQ) <= 63, "the waits' load counts");
     // s_waitcnt immediate for "at most n loads outstanding" (six bits: [3:0] and [15:14])
@@ -420,24 +439,38 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       if (sb + 1 < se) dma_step(sb + 1, 1);
       if (sb + 1 < se) __builtin_amdgcn_s_waitcnt(0x0F70 | (WQ + XQ));  // all but the second step's loads
       else __builtin_amdgcn_s_waitcnt(0x0F70);
-    } else {
+    } else if constexpr (XB == NBUF) {
 #pragma unroll
       for (int a = 0; a < NBUF; ++a) dma_step(sb + a < se ? sb + a : se - 1, a);
       __builtin_amdgcn_s_waitcnt(0x0F70 | vm((NBUF - 1) * (WQ + XQ)));  // the first step's loads
+    } else {
+      static_assert(!PIPE || XB == NBUF || (NBUF == 3 && XB == 2), "stages of the token tile");
+#pragma unroll
+      for (int a = 0; a < NBUF; ++a) {  // W(0) X(0) W(1) X(1) W(2)
+        const int st = sb + a < se ? sb + a : se - 1;
+#pragma unroll
+        for (int i = 0; i < WQ; ++i) dma_one(st, a, i);
+        if (a < XB) {
+#pragma unroll
+          for (int i = 0; i < XQ; ++i) dma_one(st, a, WQ + i);
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70 | vm(2 * WQ + XQ));  // the first step's loads
     }
     __syncthreads();
-    read_ops(0, 0, 0);
-    int buf = 0;
+    read_ops(0, 0, 0, 0);
+    int buf = 0, bx = 0;
     for (int s = sb; s < se; ++s) {
       const int nbuf = buf + 1 == NBUF ? 0 : buf + 1;
-      read_ops(buf, 1, 1);
+      const int nbx = bx + 1 == XB ? 0 : bx + 1;
+      read_ops(buf, bx, 1, 1);
       mm(0, 0, WR);
       pin(std::integral_constant<int, 0x100>{}, std::integral_constant<int, 2>{}, std::integral_constant<int, WR + WT>{},
           std::integral_constant<int, WR * WT>{});
       __builtin_amdgcn_sched_barrier(0);
       // this wave's reads of the stage have returned, its share of the next stage has landed (loads
       // return in order: all but those of the NBUF - 2 steps after it)
-      __builtin_amdgcn_s_waitcnt(0x0070 | vm((NBUF - 2) * (WQ + XQ)));
+      __builtin_amdgcn_s_waitcnt(0x0070 | vm(XB == NBUF ? (NBUF - 2) * (WQ + XQ) : WQ));
       __syncthreads();
       // (the last two steps load the last step once more, into a stage that nobody reads any more,
       // and read stale operands that nobody multiplies: no branch, one schedule)
@@ -447,6 +480,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       // faster than the CU's memory pipeline takes them (a wave that waits to issue a load does not
       // issue the matrix instructions behind it either)
       const int nxt = s + NBUF < se ? s + NBUF : se - 1;
+      const int nxt_x = s + XB < se ? s + XB : se - 1;
       // (the reads in all but the last region where they fit there: the first matrix instruction of
       // the next half waits for the last of them)
       constexpr int NL = WQ + XQ, NR = WR + WT;
@@ -460,9 +494,17 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
         constexpr int nl = NL - i * LD < 0 ? 0 : (NL - i * LD < LD ? NL - i * LD : LD);
         constexpr int nr = (EARLY && i == WR - 1) || NR - i * RD < 0 ? 0 : (NR - i * RD < RD ? NR - i * RD : RD);
 #pragma unroll
-        for (int l = 0; l < nl; ++l) dma_one(nxt, buf, i * LD + l);
+        for (int l = 0; l < nl; ++l) {
+          constexpr int j = i * LD;
+          if constexpr (XB == NBUF) {
+            dma_one(nxt, buf, j + l);
+          } else {  // token blocks first
+            if (j + l < XQ) dma_one(nxt_x, bx, WQ + j + l);
+            else dma_one(nxt, buf, j + l - XQ);
+          }
+        }
 #pragma unroll
-        for (int r = 0; r < nr; ++r) read_one(nbuf, 0, 0, i * RD + r);
+        for (int r = 0; r < nr; ++r) read_one(nbuf, nbx, 0, 0, i * RD + r);
         mm(1, i, i + 1);
         // a matrix instruction, a load, ..., a matrix instruction, a read, ... (loads first: they have the longer way)
 #pragma unroll
@@ -484,6 +526,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       if constexpr (WR > 2) region(std::integral_constant<int, 2>{});
       if constexpr (WR > 3) region(std::integral_constant<int, 3>{});
       buf = nbuf;
+      bx = nbx;
     }
   } else if constexpr (DMA) {
     // NBUF stages, NBUF - 1 k-steps of loads in flight. Every pass issues a step's loads -- past the
@@ -670,7 +713,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     constexpr int RPI = kWave / LPR;             // rows per row-wise instruction
     constexpr int JG = WT < 4 ? WT : 4;          // token tiles of 16 per pass
     constexpr int NI = 16 * JG / RPI;            // row-wise instructions per pass
-    static_assert(!PIPE || (WT % JG == 0 && CE <= 8 && (size_t)kNWaves * 16 * JG * 128 <= (size_t)NBUF * (sizeof(WStage) + sizeof(XStage))),
+    static_assert(!PIPE || (WT % JG == 0 && CE <= 8 && (size_t)kNWaves * 16 * JG * 128 <= (size_t)NBUF * sizeof(WStage) + (size_t)XB * sizeof(XStage)),
                   "the waves' epilogue tiles fit the operand stages");
     const bool whole = t0 + TOKS <= p.tokens && o0 + OUT_TILE <= p.n && (p.y_pitch & 7) == 0 &&
                        (((uintptr_t)p.y | (uintptr_t)p.residual) & 15) == 0;  // uniform
@@ -857,6 +900,7 @@ static int g_prefill_row_group = 4;   // row tiles per panel of an XCD's tile wa
 static int g_prefill_row_split = 0;   // experiments: 8, 4 or 2 forces the XCDs' split of the grid (0: the launcher's choice)
 static int g_prefill_bands = 1;       // experiments: 0 keeps gate/up in one launch whatever its last round holds
 static int g_prefill_persistent = 1;  // experiments: 0 launches one workgroup per tile on the pipelined tiles too
+static int g_prefill_stages3_big = 1;  // experiments: 0 keeps the pipelined 192 x 256 and 256 x 256 tiles on two stages of both tiles
 static int g_prefill_stages3 = 1;     // experiments: 0 keeps the pipelined 128 x 256 tile on two LDS stages
 
 // what the LDS-direct loads need: whole k-steps, 16-byte aligned rows, 32-bit byte offsets from
@@ -889,7 +933,8 @@ static int launch_prefill_cfg(hipStream_t s, PrefillGemmParams p) {
   // every XCD gets the same number of slots: its share rounded up, the surplus exits
   const long grid = (long)ceil_div(p.n_tiles, p.row_split) * ceil_div(p.t_tiles, 8 / p.row_split) * 8;
   if (grid > 0x7fffffffL) return MUI_ERR_UNSUPPORTED;
-  constexpr size_t lds = prefill_lds_bytes<ROWS, TOKS, KS, NBUF>();
+  constexpr size_t lds = PIPE ? pipe_lds_bytes<ROWS, TOKS, KS, NBUF>() : prefill_lds_bytes<ROWS, TOKS, KS, NBUF>();
+  static_assert(lds <= kLdsPerWorkgroup, "LDS of a workgroup");
   auto launch = [&](auto kernel) {
     if constexpr (lds > 65536) {
       // more dynamic LDS than the default limit: raised once per kernel (and device)
@@ -1086,7 +1131,8 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
           b.w0 += (long)a.n * p.pitch;
           b.w1 += (long)a.n * p.pitch;
           b.y += a.n;
-          int st = launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, a);
+          int st = g_prefill_stages3_big ? launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 3, true>(s, a)
+                                         : launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, a);
           if (st == MUI_OK) st = g_prefill_stages3 ? launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 3, true>(s, b)
                                                   : launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, b);
           if (st != MUI_ERR_UNSUPPORTED) return st;
@@ -1100,7 +1146,8 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
     // (gate/up at 4096 tokens 775 -> 736 us, down 386 -> 356 us, QKV 224 -> 209 us, down at 2048
     // tokens 345 -> 315 us; bit-equal results: the same products in the same order)
     if (which == 4 && !p.gamma) {
-      const int st = launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, p);
+      const int st = g_prefill_stages3_big ? launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 3, true>(s, p)
+                                           : launch_prefill_cfg<T, WF, EPI, 4, 8, 4, 2, 1, 64, 2, true>(s, p);
       if (st != MUI_ERR_UNSUPPORTED) return st;
     }
   }
@@ -1112,7 +1159,9 @@ static int launch_prefill_t(hipStream_t s, const PrefillGemmParams& p) {
       if (which == 7) st = g_prefill_stages3 ? launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 3, true>(s, p)
                                              : launch_prefill_cfg<T, WF, EPI, 4, 4, 2, 4, 1, 64, 2, true>(s, p);
       if constexpr (EPI == SK_LINEAR) {
-        if (which == 8) st = launch_prefill_cfg<T, WF, EPI, 3, 8, 4, 2, 1, 64, 2, true>(s, p);  // 192 x 256, 4 x 2 waves of 48 x 128
+        // 192 x 256, 4 x 2 waves of 48 x 128
+        if (which == 8) st = g_prefill_stages3_big ? launch_prefill_cfg<T, WF, EPI, 3, 8, 4, 2, 1, 64, 3, true>(s, p)
+                                                   : launch_prefill_cfg<T, WF, EPI, 3, 8, 4, 2, 1, 64, 2, true>(s, p);
       }
       if (st != MUI_ERR_UNSUPPORTED) return st;
     }
@@ -1209,6 +1258,8 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   // experiments: 200 + tile keeps the 128 x 256 and 192 x 256 tiles off the software-pipelined loop,
   // 100 + tile keeps every operand tile on the register-staged path
   // 6400 + tile / 12800 + tile / 19200 + tile: the XCDs split the tile grid 8 x 1 / 4 x 2 / 2 x 4 (rows x tokens)
+  const int stages3_big = tile >= 51200 ? 0 : 1;  // 51200 + tile: the pipelined 192 x 256 and 256 x 256 tiles on two LDS stages
+  if (tile >= 51200) tile -= 51200;
   const int stages3 = tile >= 25600 ? 0 : 1;  // 25600 + tile: the pipelined 128 x 256 tile on two LDS stages
   if (tile >= 25600) tile -= 25600;
   const int row_split = tile >= 19200 ? 2 : tile >= 12800 ? 4 : tile >= 6400 ? 8 : 0;
@@ -1226,6 +1277,7 @@ extern "C" int mui_tune_prefill(int tile, int wide_max_tokens) {
   const int dma = tile >= 100 ? 0 : 1;
   if (tile >= 100) tile -= 100;
   if (tile < 0 || tile > 13 || wide_max_tokens > 128) return MUI_ERR_INVALID_ARG;
+  mui::g_prefill_stages3_big = stages3_big;
   mui::g_prefill_stages3 = stages3;
   mui::g_prefill_row_split = row_split;
   mui::g_prefill_bands = bands;

@@ -40,7 +40,8 @@ def _mk(shape, g, std=1.0, mean=0.0, dtype=torch.float16):
 def test_software_pipelined_tiles(dtype, n, k, tokens, gateup):
     """Tile choices 4 (256 x 256), 7 (128 x 256) and 8 (192 x 256; the gate/up epilogue has none and
     takes its twelve-wave kernel) run the software-pipelined loop here, 7 on three LDS stages and
-    25607 the same tile on two; 13, 207, 208 and 104 are the older kernels of the same tiles (sixteen /
+    25607 the same tile on two, 4 and 8 on three stages of the weight tile and two of the token tile
+    and 51204 / 51208 on two of both; 13, 207, 208 and 104 are the older kernels of the same tiles (sixteen /
     sixteen / twelve waves, LDS-direct or register-staged operands). The shapes with one and two
     k-steps run the three-stage loop with fewer steps than stages."""
     lib = _lib.load()
@@ -58,7 +59,7 @@ def test_software_pipelined_tiles(dtype, n, k, tokens, gateup):
         wd, r, b = w.to(DEV), r.to(DEV), b.to(DEV)
     xd = x.to(DEV)
     outs = {}
-    for choice in (4, 13, 104, 7, 25607, 207, 8, 208):
+    for choice in (4, 51204, 13, 104, 7, 25607, 207, 8, 51208, 208):
         _lib.check(lib.mui_tune_prefill(choice, -1), "mui_tune_prefill")
         y = torch.zeros(tokens, n, dtype=dtype, device=DEV)
         if gateup:
@@ -74,7 +75,7 @@ def test_software_pipelined_tiles(dtype, n, k, tokens, gateup):
         assert_parity(outs[choice], ref, 1e-2, f"pipelined tile choice {choice} {dtype} {tokens}x{n}x{k} gateup={gateup}")
     assert torch.equal(outs[4], outs[13]) and torch.equal(outs[4], outs[104])
     assert torch.equal(outs[7], outs[207]) and torch.equal(outs[8], outs[208]) and torch.equal(outs[4], outs[7])
-    assert torch.equal(outs[7], outs[25607])
+    assert torch.equal(outs[7], outs[25607]) and torch.equal(outs[4], outs[51204]) and torch.equal(outs[8], outs[51208])
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
