@@ -713,6 +713,39 @@ def probe_prompt(counters_only=False):
     print(json.dumps({"probe_prompt": out}))
 
 
+_PROMPT_SHAPES_OTHER = (("70b_qkv", 10240, 8192, False), ("70b_o_proj", 8192, 8192, False), ("70b_gateup", 28672, 8192, True),
+                        ("70b_down", 8192, 28672, False), ("13b_qkv", 15360, 5120, False), ("13b_o_proj", 5120, 5120, False),
+                        ("13b_gateup", 13824, 5120, True), ("13b_down", 5120, 13824, False))
+
+
+def probe_prompt_other_shapes():
+    """The prompt GEMM at the projections of a Llama-3-70B- and a Llama-2-13B-shaped layer, 512 to 4096
+    tokens, beside torch.matmul on the same operands (for gate/up the matmul alone): the tile choice
+    was calibrated on the 8B shapes and has to carry over."""
+    import torch
+
+    from muillm_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    f16 = dict(device="cuda", dtype=torch.float16)
+    ws = torch.zeros(lib.mui_linear_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    out = {}
+    for name, n, k, gateup in _PROMPT_SHAPES_OTHER:
+        rows = 2 * n if gateup else n
+        ring = [torch.randn(rows, k, **f16) * 0.02 for _ in range(max(2, int(1e9 // (2 * rows * k)) + 1))]
+        for tokens in (512, 1024, 2048, 4096):
+            x, y = torch.randn(tokens, k, **f16), torch.empty(tokens, n, **f16)
+            yt = torch.empty(tokens, rows, **f16)
+            us = _event_time_us(lambda i: _prompt_gemm_call(lib, stream, ring[i % len(ring)], x, y, n, k, tokens, gateup, ws), 10, 2)
+            us_t = _event_time_us(lambda i: torch.matmul(x, ring[i % len(ring)].t(), out=yt), 10, 2)
+            out["%s_tokens%d" % (name, tokens)] = {"us": round(us, 1), "TFLOP/s": round(2.0 * tokens * rows * k / us / 1e6, 1),
+                                                   "torch_matmul_us": round(us_t, 1)}
+        del ring
+        torch.cuda.empty_cache()
+    print(json.dumps({"probe_prompt_other_shapes": out}))
+
+
 def trace_prefill(tokens, passes=3):
     """Prefill passes of the 8B-shaped fp16 model (embedding to last-token logits) for a kernel trace:
     two warm-up passes, then `passes` passes with a device synchronisation after each."""
@@ -1133,6 +1166,8 @@ def main():
                     help="time the prompt GEMMs and prompt attention at the Llama-3-8B shapes beside torch and exit")
     ap.add_argument("--trace-prefill", type=int, default=0, metavar="TOKENS",
                     help="a few prefill passes of the 8B-shaped model at this prompt length (for rocprofv3 --kernel-trace)")
+    ap.add_argument("--probe-prompt-other-shapes", action="store_true",
+                    help="time the prompt GEMM at the 70B- and 13B-shaped projections beside torch.matmul and exit")
     ap.add_argument("--pmc-probe-prompt", action="store_true",
                     help="launch the gate/up prompt GEMM (2048 tokens) and prompt attention (4096) three times and exit "
                          "(for rocprofv3 --pmc)")
@@ -1172,6 +1207,9 @@ def main():
     if args.tune_prefill:
         from muillm_amd import _lib
         _lib.check(_lib.load().mui_tune_prefill(*(int(v) for v in args.tune_prefill.split(","))), "mui_tune_prefill")
+    if args.probe_prompt_other_shapes:
+        probe_prompt_other_shapes()
+        return
     if args.probe_prompt or args.pmc_probe_prompt:
         probe_prompt(counters_only=args.pmc_probe_prompt)
         return
