@@ -107,3 +107,40 @@ def test_gateup_whole_rounds_and_tail_in_two_launches(dtype, n, k, tokens):
     assert torch.equal(outs[0], outs[4]) and torch.equal(outs[0], outs[3200])
     if k <= 256:
         assert_parity(outs[0], oracle.gateup_silu(x, wg, wu), 1e-2, f"gate/up in two launches {dtype} {tokens}x{n}x{k}")
+
+
+@pytest.mark.parametrize("n,k,tokens", [
+    (4096, 14336, 4096),   # down: one round of 256 x 256 tiles, the XCDs split rows x tokens 4 x 2, 224 k-steps
+    (6144, 4096, 4096),    # QKV: two rounds of 192 x 256 tiles walked by a persistent round of workgroups
+    (4096, 4096, 8192),    # o_proj: two rounds of 256 x 256 tiles in panels of four row tiles
+    (4096, 4096, 2048),    # o_proj: one round of 128 x 256 tiles on three LDS stages
+])
+def test_full_size_prompt_linears_against_the_older_kernels(n, k, tokens):
+    """The Llama-3-8B projections at whole-prompt sizes, where the built-in choice walks several rounds
+    of tiles, splits the grid over the XCDs by rows and tokens and keeps three LDS stages: bit for bit
+    what the sixteen- / twelve-wave kernels of the same tiles give with every such choice switched
+    off (100 + tile: register-staged operands; 800: one row tile after another; 6400: rows-only split;
+    51200 / 25600: two LDS stages), and within 1e-2 of the maximum of an fp32 product of the same
+    operands on the device (the CPU oracle takes minutes at these sizes; it gates the same kernels
+    on smaller shapes above)."""
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    g = _gen(13)
+    x = _mk((tokens, k), g).to(DEV)
+    w = _mk((n, k), g, 0.02).to(DEV)
+    r = _mk((tokens, n), g).to(DEV)
+    ref = x.float() @ w.float().t() + r.float()
+    which = 8 if n == 6144 else 7 if tokens == 2048 else 4
+    outs = {}
+    for choice in (0, 100 + which + 800 + 6400, 51200 + 25600 + which):
+        _lib.check(lib.mui_tune_prefill(choice, 0 if choice == 0 else -1), "mui_tune_prefill")
+        y = torch.zeros(tokens, n, dtype=torch.float16, device=DEV)
+        assert lib.mui_linear(s, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, r.data_ptr(), y.data_ptr(), n, k, tokens) == 0
+        torch.cuda.synchronize()
+        outs[choice] = y
+    _lib.check(lib.mui_tune_prefill(0, 0), "mui_tune_prefill")
+    err = float((outs[0].float() - ref).abs().max() / ref.abs().max())
+    print(f"[parity] full-size prompt linear {tokens}x{n}x{k}: max err over max |ref| {err:.2e} (gate 1e-2)")
+    assert err <= 1e-2
+    for choice, y in outs.items():
+        assert torch.equal(outs[0], y), f"choice {choice} differs from the built-in one"
