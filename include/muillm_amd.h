@@ -172,7 +172,9 @@ int mui_int8_gateup_silu(mui_stream_t stream, int dtype, const void* gate_i8, co
 /* muillm_int8_linear_forward on the reference's own RTN format
  * (muillm/quantization/rtnquantizer.py:49-88): weights_u8 uint8 [n_out, k_in],
  * scales_min_vals 16-bit [n_out * G, 2] = (scale, min) per group of 2^group_size_shift
- * inputs, w = u8 * scale + min. Requirements as above plus group size >= 16. */
+ * inputs, w = u8 * scale + min. Requirements as above plus group size >= 16. Any tokens >= 1:
+ * beyond MUI_MAX_TOKENS the tiled GEMM turns every chunk of codes into u8 * scale + min, rounded
+ * once to the 16-bit type -- the values mui_int8_group_dequantize writes -- on its way to LDS. */
 int mui_int8_group_linear(mui_stream_t stream, int dtype, const void* weights_u8, long w_pitch,
                           const void* scales_min_vals, int group_size_shift, const void* x,
                           const void* norm_weights, float epsilon, const void* add_bias,
@@ -180,7 +182,8 @@ int mui_int8_group_linear(mui_stream_t stream, int dtype, const void* weights_u8
 
 /* muillm_int8_gateupsilu_forward on the reference's RTN format. gate/up rows share gu_pitch
  * (bytes); the (scale, min) pairs of row n start at gate_smv + n * smv_pitch and
- * up_smv + n * smv_pitch (16-bit elements; 2 * G when dense, 4 * G when row-interleaved). */
+ * up_smv + n * smv_pitch (16-bit elements; 2 * G when dense, 4 * G when row-interleaved).
+ * Any tokens >= 1, as mui_int8_group_linear. */
 int mui_int8_group_gateup_silu(mui_stream_t stream, int dtype, const void* gate_u8,
                                const void* up_u8, long gu_pitch, const void* gate_smv,
                                const void* up_smv, long smv_pitch, int group_size_shift,

@@ -296,7 +296,7 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
     for (int i = 0; i < WQ + XQ; ++i) dma_one(step, buf, i);
   };
   // one k-step of the tile in registers, on its way from global memory to LDS
-  struct Stage { u32x4 w[WCH], x[XCH], g; };
+  struct Stage { u32x4 w[WCH], x[XCH], g; uint32_t pr[WF == WF_U8_GROUP ? WCH : 1]; };  // pr: the (scale, min) pair of a chunk of codes
   auto load_step = [&](int step, Stage& r) {
     // steps past the last one re-read step 0 (never stored): that keeps the loads out of branches;
     // chunks past the end of the row read the row's first chunk and are zeroed on the way to LDS
@@ -314,6 +314,13 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
       const int woff = wk + 16 <= p.k ? wk : 0;
 #pragma unroll
       for (int i = 0; i < WCH; ++i) r.w[i] = ld16_sel<kStreamW>(wptr(i) + woff);
+      if constexpr (WF == WF_U8_GROUP) {  // a chunk of 16 codes lies in one group (groups of 16 or more)
+#pragma unroll
+        for (int i = 0; i < WCH; ++i) {
+          const uint16_t* pairs = ((EPI == SK_GATEUP && (wrow[i] >> 30)) ? p.s1 : p.s0) + (long)(wrow[i] & ((1 << 30) - 1)) * p.s_pitch;
+          r.pr[i] = ld4(pairs + 2 * (woff >> p.group_shift));
+        }
+      }
     }
   };
 
@@ -346,8 +353,14 @@ __device__ __forceinline__ void prefill_gemm_tile(const PrefillGemmParams& p, co
 #pragma unroll
       for (int i = 0; i < WCH; ++i) {
         if (!WEXACT && t + kPfThreads * i >= WCHUNKS) continue;
-        const u32x4 lo = convert_a<T, WF>(r.w[i].x, r.w[i].y, nullptr, 0, 0);
-        const u32x4 hi = convert_a<T, WF>(r.w[i].z, r.w[i].w, nullptr, 0, 0);
+        u32x4 lo, hi;
+        if constexpr (WF == WF_U8_GROUP) {  // u8 * scale + min rounded once: what the dequantisation kernel writes
+          lo = convert_a_pair<T>(r.w[i].x, r.w[i].y, r.pr[i]);
+          hi = convert_a_pair<T>(r.w[i].z, r.w[i].w, r.pr[i]);
+        } else {
+          lo = convert_a<T, WF>(r.w[i].x, r.w[i].y, nullptr, 0, 0);
+          hi = convert_a<T, WF>(r.w[i].z, r.w[i].w, nullptr, 0, 0);
+        }
         const int row = (t + kPfThreads * i) / WCPR;
         uint16_t* dst = &w_lds[buf][row * PITCH];
         *(u32x4*)(dst + (((2 * wcol) ^ swz(row)) * 8)) = wlive ? lo : zero;
@@ -1216,7 +1229,7 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
   PrefillGemmParams p = {};
   const long esz = (wf == WF_16BIT) ? 2 : 1;
   p.w0 = (const uint8_t*)q.w0; p.w1 = (const uint8_t*)q.w1; p.pitch = q.pitch * esz;
-  p.s0 = q.s0; p.s1 = q.s1; p.s_pitch = q.s_pitch;
+  p.s0 = q.s0; p.s1 = q.s1; p.s_pitch = q.s_pitch; p.group_shift = q.group_shift;
   p.x = q.x; p.gamma = q.gamma; p.mul_bias = q.mul_bias; p.add_bias = q.add_bias; p.residual = q.residual;
   p.y = q.y; p.y_pitch = q.n; p.n = q.n; p.k = q.k; p.tokens = q.tokens; p.eps = q.eps;
   // a caller-provided workspace lets a long K be shared between workgroups when the tiles are few
@@ -1233,8 +1246,9 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
       if (dtype == MUI_DTYPE_BF16) return launch_prefill_xs<BF16>(s, p, shares, q.workspace);
     }
   }
-  if (wide) return launch_gemm_wide(s, dtype, wf, epilogue, q);
-  if (!(wf == WF_16BIT || wf == WF_I8_CHANNEL)) return MUI_ERR_UNSUPPORTED;
+  if (wide && wf != WF_U8_GROUP) return launch_gemm_wide(s, dtype, wf, epilogue, q);  // (that kernel has no group format)
+  if (!(wf == WF_16BIT || wf == WF_I8_CHANNEL || wf == WF_U8_GROUP)) return MUI_ERR_UNSUPPORTED;
+  if (wf == WF_U8_GROUP && (q.group_shift < 4 || (q.k & ((1 << q.group_shift) - 1)))) return MUI_ERR_UNSUPPORTED;
   if (q.k % (wf == WF_16BIT ? 8 : 16)) return MUI_ERR_UNSUPPORTED;
   if (q.x_pitch != 0 && q.x_pitch != q.k) return MUI_ERR_UNSUPPORTED;
 #define MUI_PF_CASE(TT, WFV, EPIV) \
@@ -1243,10 +1257,14 @@ int launch_prefill_gemm(hipStream_t s, int dtype, int wf, int epilogue, const Sk
   MUI_PF_CASE(F16, WF_16BIT, SK_GATEUP)
   MUI_PF_CASE(F16, WF_I8_CHANNEL, SK_LINEAR)
   MUI_PF_CASE(F16, WF_I8_CHANNEL, SK_GATEUP)
+  MUI_PF_CASE(F16, WF_U8_GROUP, SK_LINEAR)
+  MUI_PF_CASE(F16, WF_U8_GROUP, SK_GATEUP)
   MUI_PF_CASE(BF16, WF_16BIT, SK_LINEAR)
   MUI_PF_CASE(BF16, WF_16BIT, SK_GATEUP)
   MUI_PF_CASE(BF16, WF_I8_CHANNEL, SK_LINEAR)
   MUI_PF_CASE(BF16, WF_I8_CHANNEL, SK_GATEUP)
+  MUI_PF_CASE(BF16, WF_U8_GROUP, SK_LINEAR)
+  MUI_PF_CASE(BF16, WF_U8_GROUP, SK_GATEUP)
 #undef MUI_PF_CASE
   return MUI_ERR_INVALID_ARG;
 }

@@ -462,12 +462,21 @@ extern "C" int mui_int8_group_linear(mui_stream_t stream, int dtype, const void*
                                      const void* x, const void* norm_weights, float epsilon,
                                      const void* add_bias, const void* residual, void* y, int n_out,
                                      int k_in, int tokens) {
-  int st = check_int8_common(dtype, weights_u8, w_pitch, x, norm_weights, n_out, k_in, tokens);
+  int st = check_int8_common(dtype, weights_u8, w_pitch, x, norm_weights, n_out, k_in, tokens, true);
   if (st != MUI_OK) return st;
   MUI_CHECK_ARG(scales_min_vals && y);
   if (group_size_shift < 4 || group_size_shift > 30) return MUI_ERR_UNSUPPORTED;
   if (k_in & ((1 << group_size_shift) - 1)) return MUI_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
+  if (tokens > MUI_MAX_TOKENS) {  // a prompt: the tiled matrix-core GEMM, codes dequantised on the way to LDS
+    SkinnyParams sp = {};
+    sp.w0 = weights_u8; sp.pitch = w_pitch; sp.s0 = (const uint16_t*)scales_min_vals;
+    sp.s_pitch = 2L * (k_in >> group_size_shift); sp.group_shift = group_size_shift;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.add_bias = (const uint16_t*)add_bias; sp.residual = (const uint16_t*)residual;
+    sp.y = (uint16_t*)y; sp.n = n_out; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_prefill_gemm(s, dtype, WF_U8_GROUP, SK_LINEAR, sp);
+  }
   if (tokens >= 2 || (g_int8_dot2 && dtype == MUI_DTYPE_F16)) {
     SkinnyParams sp = {};
     sp.w0 = weights_u8; sp.pitch = w_pitch; sp.s0 = (const uint16_t*)scales_min_vals;
@@ -503,7 +512,7 @@ extern "C" int mui_int8_group_gateup_silu(mui_stream_t stream, int dtype, const 
                                           const void* up_smv, long smv_pitch, int group_size_shift,
                                           const void* x, const void* norm_weights, float epsilon,
                                           void* h, int n_inter, int k_in, int tokens) {
-  int st = check_int8_common(dtype, gate_u8, gu_pitch, x, norm_weights, n_inter, k_in, tokens);
+  int st = check_int8_common(dtype, gate_u8, gu_pitch, x, norm_weights, n_inter, k_in, tokens, true);
   if (st != MUI_OK) return st;
   MUI_CHECK_ARG(up_u8 && gate_smv && up_smv && h);
   if (!aligned16(up_u8)) return MUI_ERR_ALIGNMENT;
@@ -511,6 +520,15 @@ extern "C" int mui_int8_group_gateup_silu(mui_stream_t stream, int dtype, const 
   if (k_in & ((1 << group_size_shift) - 1)) return MUI_ERR_UNSUPPORTED;
   if (smv_pitch < 2L * (k_in >> group_size_shift) || (smv_pitch & 1)) return MUI_ERR_INVALID_ARG;
   hipStream_t s = (hipStream_t)stream;
+  if (tokens > MUI_MAX_TOKENS) {
+    SkinnyParams sp = {};
+    sp.w0 = gate_u8; sp.w1 = up_u8; sp.pitch = gu_pitch;
+    sp.s0 = (const uint16_t*)gate_smv; sp.s1 = (const uint16_t*)up_smv; sp.s_pitch = smv_pitch;
+    sp.group_shift = group_size_shift;
+    sp.x = (const uint16_t*)x; sp.gamma = (const uint16_t*)norm_weights;
+    sp.y = (uint16_t*)h; sp.n = n_inter; sp.k = k_in; sp.tokens = tokens; sp.eps = epsilon;
+    return launch_prefill_gemm(s, dtype, WF_U8_GROUP, SK_GATEUP, sp);
+  }
   if (tokens >= 2 || (g_int8_dot2 && dtype == MUI_DTYPE_F16)) {
     SkinnyParams sp = {};
     sp.w0 = gate_u8; sp.w1 = up_u8; sp.pitch = gu_pitch;

@@ -36,9 +36,10 @@ struct PrefillGemmParams {
   const uint8_t* w0;      // linear: matrix; gate/up: gate rows
   const uint8_t* w1;      // gate/up: up rows
   long pitch;             // weight row pitch in bytes
-  const uint16_t* s0;     // per-channel int8: scale of row n at s0[n * s_pitch]
+  const uint16_t* s0;     // per-channel int8: scale of row n at s0[n * s_pitch]; group format: (scale, min) pairs of row n at s0 + n * s_pitch + 2 g
   const uint16_t* s1;
   long s_pitch;
+  int group_shift;        // group format: log2 of the codes per (scale, min) pair
   const uint16_t* x;      // [tokens, k] dense
   const uint16_t* gamma;
   const uint16_t* mul_bias;
@@ -164,7 +165,7 @@ __device__ __forceinline__ u32x4 convert_a_pair(uint32_t w0, uint32_t w1, uint32
   return pack8<T>(f);
 }
 
-// tiled matrix-core GEMM for prompts (gemm_prefill.hip): any token count, 16-bit or per-channel int8
+// tiled matrix-core GEMM for prompts (gemm_prefill.hip): any token count, 16-bit weights or int8 codes of either format
 int launch_prefill_gemm(hipStream_t s, int dtype, int weight_format, int epilogue, const SkinnyParams& p);
 size_t prefill_workspace_bytes();  // what SkinnyParams::workspace must hold for the prompt GEMM to use it
 // 17..128 tokens: 16 weight rows per workgroup, K split over its waves, token columns in up to 8 MFMA tiles (gemm_wide.hip)

@@ -382,9 +382,9 @@ def _byte_pitch(w: torch.Tensor, name: str) -> int:
 
 # int8 weights: the decode kernels take chunks of MUI_MAX_TOKENS up to this many tokens; beyond, the
 # tiled matrix-core GEMM converts the codes on their way to LDS (per-channel format: no chunking,
-# 64 tokens of an 8B-shaped prefill take 5.6 ms on the GEMM against 8.9 ms in four chunks) or runs
-# on the matrix dequantised by the library's kernel (group format: dequantising every matrix costs
-# about 4 ms per 8B-shaped pass, two chunks of the decode kernels less).
+# 64 tokens of an 8B-shaped prefill take 5.6 ms on the GEMM against 8.9 ms in four chunks; group
+# format: two chunks of the decode kernels are still ahead of it at 17..32 tokens); long prompts run
+# on the matrix dequantised by the library's kernel (about 4 ms per 8B-shaped pass).
 INT8_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
 INT8_GROUP_CHUNK_MAX_TOKENS = 32
 # Per-channel format from this many tokens: the matrix is dequantised once per call (12–32 µs per
@@ -392,6 +392,10 @@ INT8_GROUP_CHUNK_MAX_TOKENS = 32
 # converting loop cannot use (at 4096 tokens QKV 227 -> 182 µs, o_proj 128 -> 118, down 389 -> 381,
 # gate/up 817 -> 762; at 1024 tokens the conversion on the way to LDS is still ahead).
 INT8_DEQUANT_MIN_TOKENS = 2048
+# The group format likewise, from 1024 tokens; 33 .. 1023 tokens go to the GEMM that applies (scale, min)
+# on the way to LDS (an 8B-shaped prefill of 64 tokens 9.4 -> 6.1 ms, 512 tokens 14.3 -> 12.1 ms, level at
+# 1024, 35.0 against 29.9 ms at 2048).
+INT8_GROUP_DEQUANT_MIN_TOKENS = 1024
 
 
 def int8_kernel_dispatchable(x: torch.Tensor) -> bool:
@@ -533,9 +537,10 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
     _check_contiguous(scales_min_vals, "scales_min_vals")
     _check_activations(x, k, "muillm_int8_linear_forward", _MAX_CALL_TOKENS, weights,
                        scales_min_vals, norm_weights, add_bias, residual)
-    if _num_tokens(x) > INT8_GROUP_CHUNK_MAX_TOKENS:
-        # a prompt: the reference's route (dequantise the matrix, then a GEMM,
-        # muillm/modules/quantized/int8linear.py:279-293) on this library's kernels
+    if _num_tokens(x) >= INT8_GROUP_DEQUANT_MIN_TOKENS:
+        # a long prompt: the reference's route (dequantise the matrix, then a GEMM,
+        # muillm/modules/quantized/int8linear.py:279-293) on this library's kernels; shorter ones go
+        # to the GEMM that dequantises the codes on their way to LDS (one call below)
         w = muillm_int8_dequantize_forward(weights, scales_min_vals, group_size_shift)
         return muillm_linear_forward(None, x, w, norm_weights, epsilon, None, add_bias, residual)
     if scales_min_vals.dtype != x.dtype or scales_min_vals.numel() != 2 * n * (k >> group_size_shift):
@@ -543,6 +548,7 @@ def muillm_int8_linear_forward(x, weights, scales_min_vals, group_size_shift, no
     if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
         raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
     x = x.contiguous()
+    x, norm_weights = _norm_first(x, norm_weights, epsilon, INT8_GROUP_CHUNK_MAX_TOKENS)
     tokens = _num_tokens(x)
     if add_bias is not None and add_bias.numel() == tokens * n and residual is None and tokens > 1:
         residual, add_bias = add_bias, None
@@ -657,12 +663,13 @@ def muillm_int8_gateupsilu_forward(norm_weights, epsilon, gate_up_weights, gate_
         raise RuntimeError("gate_up_scales_min_vals must hold N * 2 * K / group (scale, min) pairs in the activation dtype")
     if norm_weights is not None and (norm_weights.dtype != x.dtype or norm_weights.numel() != k):
         raise RuntimeError("norm weights must be one value per input feature in the activation dtype")
-    if _num_tokens(x) > INT8_GROUP_CHUNK_MAX_TOKENS:
-        # a prompt: dequantise gate and up once, then the tiled GEMM with the SiLU * mul epilogue
+    if _num_tokens(x) >= INT8_GROUP_DEQUANT_MIN_TOKENS:
+        # a long prompt: dequantise gate and up once, then the tiled GEMM with the SiLU * mul epilogue
         gd, ud = muillm_int8_gateupsilu_dequantize_forward(gate_up_weights, gate_up_scales_min_vals, group_size_shift)
         return mui_gateup_silu(norm_weights, epsilon, gd, ud, x)
     smv = gate_up_scales_min_vals.reshape(n, 2, g, 2)
     x = x.contiguous()
+    x, norm_weights = _norm_first(x, norm_weights, epsilon, INT8_GROUP_CHUNK_MAX_TOKENS)
     tokens = _num_tokens(x)
     h = torch.empty(list(x.shape[:-1]) + [n], dtype=x.dtype, device=x.device)
     gw, uw = gate_up_weights[:, 0, :], gate_up_weights[:, 1, :]
