@@ -383,10 +383,10 @@ def _byte_pitch(w: torch.Tensor, name: str) -> int:
 # int8 weights: the decode kernels take chunks of MUI_MAX_TOKENS up to this many tokens; beyond, the
 # tiled matrix-core GEMM converts the codes on their way to LDS (per-channel format: no chunking,
 # 64 tokens of an 8B-shaped prefill take 5.6 ms on the GEMM against 8.9 ms in four chunks; group
-# format: two chunks of the decode kernels are still ahead of it at 17..32 tokens); long prompts run
-# on the matrix dequantised by the library's kernel (about 4 ms per 8B-shaped pass).
+# format: 17..32 tokens 6.4 ms on the GEMM against 7.1 ms in two chunks); long prompts run on the
+# matrix dequantised by the library's kernel (about 4 ms per 8B-shaped pass).
 INT8_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
-INT8_GROUP_CHUNK_MAX_TOKENS = 32
+INT8_GROUP_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
 # Per-channel format from this many tokens: the matrix is dequantised once per call (12–32 µs per
 # Llama-3-8B matrix) and the GEMM runs its software-pipelined loop on 16-bit weights, which the
 # converting loop cannot use (at 4096 tokens QKV 227 -> 182 µs, o_proj 128 -> 118, down 389 -> 381,

@@ -385,7 +385,7 @@ def test_channel_linear_and_gateup_short_prompts(tokens, chunk_max, monkeypatch)
     """17..64 tokens: the tiled GEMM converting the codes on the way (the default), or the 16-token
     int8 kernels in chunks when the chunk limit is raised -- never a dequantised matrix for a
     library GEMM."""
-    assert muillm_ext.INT8_CHUNK_MAX_TOKENS == 16 and muillm_ext.INT8_GROUP_CHUNK_MAX_TOKENS == 32
+    assert muillm_ext.INT8_CHUNK_MAX_TOKENS == 16 and muillm_ext.INT8_GROUP_CHUNK_MAX_TOKENS == 16
     monkeypatch.setattr(muillm_ext, "INT8_CHUNK_MAX_TOKENS", chunk_max)
     g = _gen(31)
     n, k = 264, 1024
@@ -408,7 +408,7 @@ def test_channel_linear_and_gateup_short_prompts(tokens, chunk_max, monkeypatch)
     # longer prompts stay on the library's kernels too (the tiled GEMM of the same entry points)
     assert muillm_ext.int8_kernel_dispatchable(torch.zeros(65, k, dtype=torch.float16, device=DEV))
     assert muillm_ext._token_calls(64, 64) == [(0, 16), (16, 16), (32, 16), (48, 16)] and muillm_ext._token_calls(65, 64) == [(0, 65)]
-    assert muillm_ext._token_chunks(32, group_format=True) == [(0, 16), (16, 16)] and muillm_ext._token_chunks(33, group_format=True) == [(0, 33)]
+    assert muillm_ext._token_chunks(16, group_format=True) == [(0, 16)] and muillm_ext._token_chunks(17, group_format=True) == [(0, 17)]
 
 
 def test_wrappers_refuse_mismatched_operands():

@@ -210,14 +210,14 @@ def test_int8_channel_long_prompt_dequantises_once(dtype, monkeypatch):
 
 
 @pytest.mark.parametrize("route", ["scale-and-min-on-the-way-to-LDS", "dequantise-once"])
-@pytest.mark.parametrize("tokens", [65, 150])
+@pytest.mark.parametrize("tokens", [17, 40, 65, 150])
 def test_int8_group_format_prompt(tokens, route, monkeypatch):
     """The reference's group format at prompt sizes, on both routes the host layer has: the tiled GEMM
     that turns a chunk of codes into u8 * scale + min, rounded once, on its way to LDS (prompts of
     33 .. INT8_GROUP_DEQUANT_MIN_TOKENS - 1 tokens), and the matrix dequantised by the library's
     kernel (the same values, bit-exact definition) followed by the 16-bit GEMM -- the reference's
     own route (int8linear.py:279-293), taken for longer prompts."""
-    monkeypatch.setattr(muillm_ext, "INT8_GROUP_DEQUANT_MIN_TOKENS", 33 if route == "dequantise-once" else 1 << 30)
+    monkeypatch.setattr(muillm_ext, "INT8_GROUP_DEQUANT_MIN_TOKENS", 17 if route == "dequantise-once" else 1 << 30)
     g = _gen(6)
     n, k, gs = 1040, 1024, 128
     qw, smv = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
