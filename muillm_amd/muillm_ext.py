@@ -390,8 +390,9 @@ INT8_GROUP_CHUNK_MAX_TOKENS = MUI_MAX_TOKENS
 # Per-channel format from this many tokens: the matrix is dequantised once per call (12–32 µs per
 # Llama-3-8B matrix) and the GEMM runs its software-pipelined loop on 16-bit weights, which the
 # converting loop cannot use (at 4096 tokens QKV 227 -> 182 µs, o_proj 128 -> 118, down 389 -> 381,
-# gate/up 817 -> 762; at 1024 tokens the conversion on the way to LDS is still ahead).
-INT8_DEQUANT_MIN_TOKENS = 2048
+# gate/up 817 -> 762; an 8B-shaped prefill 27.5 -> 25.8 ms at 1536 tokens, while at 1024 tokens the
+# conversion on the way to LDS is still ahead, 17.7 against 19.5 ms).
+INT8_DEQUANT_MIN_TOKENS = 1280
 # The group format likewise, from 1024 tokens; 33 .. 1023 tokens go to the GEMM that applies (scale, min)
 # on the way to LDS (an 8B-shaped prefill of 64 tokens 9.4 -> 6.1 ms, 512 tokens 14.3 -> 12.1 ms, level at
 # 1024, 35.0 against 29.9 ms at 2048).
