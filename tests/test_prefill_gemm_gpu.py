@@ -209,30 +209,34 @@ def test_int8_channel_long_prompt_dequantises_once(dtype, monkeypatch):
         assert d <= 1e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("route", ["scale-and-min-on-the-way-to-LDS", "dequantise-once"])
 @pytest.mark.parametrize("tokens", [17, 40, 65, 150])
-def test_int8_group_format_prompt(tokens, route, monkeypatch):
+def test_int8_group_format_prompt(tokens, route, dtype, monkeypatch):
     """The reference's group format at prompt sizes, on both routes the host layer has: the tiled GEMM
     that turns a chunk of codes into u8 * scale + min, rounded once, on its way to LDS (prompts of
-    33 .. INT8_GROUP_DEQUANT_MIN_TOKENS - 1 tokens), and the matrix dequantised by the library's
+    17 .. INT8_GROUP_DEQUANT_MIN_TOKENS - 1 tokens), and the matrix dequantised by the library's
     kernel (the same values, bit-exact definition) followed by the 16-bit GEMM -- the reference's
     own route (int8linear.py:279-293), taken for longer prompts."""
     monkeypatch.setattr(muillm_ext, "INT8_GROUP_DEQUANT_MIN_TOKENS", 17 if route == "dequantise-once" else 1 << 30)
     g = _gen(6)
     n, k, gs = 1040, 1024, 128
     qw, smv = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
-    x, gamma, r = _mk((tokens, k), g), _mk((k,), g, 0.1, 1.0), _mk((tokens, n), g)
-    wd = oracle.rtn_dequantize_group(qw, smv, gs)               # what the dequantisation kernel produces
+    smv = smv.to(dtype)                                                # (scale, min) pairs in the activation dtype
+    x, gamma, r = _mk((tokens, k), g, dtype=dtype), _mk((k,), g, 0.1, 1.0, dtype=dtype), _mk((tokens, n), g, dtype=dtype)
+    wd = oracle.rtn_dequantize_group(qw, smv, gs, dtype=dtype)         # what the dequantisation kernel produces
     ref = oracle.linear(x, wd, gamma, 1e-5, None, r)
     y = muillm_ext.muillm_int8_linear_forward(x.to(DEV), qw.to(DEV), smv.to(DEV), 7, gamma.to(DEV), 1e-5,
                                               residual=r.to(DEV))
-    assert_parity(y, ref, 1e-2, "group-format prompt linear")
+    assert_parity(y, ref, 1e-2, f"group-format prompt linear {dtype}")
     qu, smu = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
+    smu = smu.to(dtype)
     pw = torch.stack([qw, qu], dim=1).contiguous().to(DEV)
     ps = torch.stack([smv.reshape(n, -1, 2), smu.reshape(n, -1, 2)], dim=1).contiguous().to(DEV)
     h = muillm_ext.muillm_int8_gateupsilu_forward(gamma.to(DEV), 1e-5, pw, ps, 7, x.to(DEV))
-    refh = oracle.gateup_silu(x, wd, oracle.rtn_dequantize_group(qu, smu, gs), gamma, 1e-5)
-    assert_parity(h, refh, 1e-2, "group-format prompt gate/up")
+    refh = oracle.gateup_silu(x, wd, oracle.rtn_dequantize_group(qu, smu, gs, dtype=dtype), gamma, 1e-5)
+    # bf16 gate/up: two 8-bit-mantissa operands of SiLU * mul set the elementwise floor (4e-2), as for 16-bit weights
+    assert_parity(h, refh, 1e-2, f"group-format prompt gate/up {dtype}", elementwise=None if dtype == torch.float16 else 4e-2)
 
 
 def test_prompt_abi_direct_and_errors():
