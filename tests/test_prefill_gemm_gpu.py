@@ -253,3 +253,42 @@ def test_prompt_abi_direct_and_errors():
     assert lib.mui_linear(s, 0, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), n, 12, tokens) == -2
     assert lib.mui_linear(s, 0, w.data_ptr() + 2, k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), n, k, tokens) == -4
     assert lib.mui_linear(s, 7, w.data_ptr(), k, x.data_ptr(), None, 0.0, None, None, None, y.data_ptr(), n, k, tokens) == -1
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_group_format_prompt_abi_with_fused_norm(dtype):
+    """mui_int8_group_linear / mui_int8_group_gateup_silu straight through the C ABI with 48 tokens
+    AND norm weights: the tiled GEMM normalises the token rows while staging them (the host layer
+    would normalise first) and applies (scale, min) to the codes on their way to LDS. Refused: groups
+    smaller than 16 codes and a K that is not a whole number of groups."""
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    g = _gen(15)
+    n, k, gs, tokens = 272, 1024, 128, 48
+    code = 0 if dtype == torch.float16 else 1
+    qw, smv = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
+    qu, smu = oracle.rtn_quantize_group(_mk((n, k), g, 0.02), gs)
+    smv, smu = smv.to(dtype), smu.to(dtype)
+    x, gamma, r = _mk((tokens, k), g, dtype=dtype), _mk((k,), g, 0.1, 1.0, dtype=dtype), _mk((tokens, n), g, dtype=dtype)
+    wd, ud = oracle.rtn_dequantize_group(qw, smv, gs, dtype=dtype), oracle.rtn_dequantize_group(qu, smu, gs, dtype=dtype)
+    qd, sd, xd, gd, rd = qw.to(DEV), smv.to(DEV), x.to(DEV), gamma.to(DEV), r.to(DEV)
+    y = torch.zeros(tokens, n, dtype=dtype, device=DEV)
+    st = lib.mui_int8_group_linear(s, code, qd.data_ptr(), k, sd.data_ptr(), 7, xd.data_ptr(), gd.data_ptr(), 1e-5, None,
+                                   rd.data_ptr(), y.data_ptr(), n, k, tokens)
+    assert st == 0
+    tol = 1e-2
+    assert_parity(y, oracle.linear(x, wd, gamma, 1e-5, None, r), tol, f"ABI group-format prompt linear, fused norm {dtype}")
+    pw = torch.stack([qw, qu], dim=1).contiguous().to(DEV)
+    ps = torch.stack([smv.reshape(n, -1, 2), smu.reshape(n, -1, 2)], dim=1).contiguous().to(DEV)
+    h = torch.zeros(tokens, n, dtype=dtype, device=DEV)
+    gcount = k // gs
+    st = lib.mui_int8_group_gateup_silu(s, code, pw.data_ptr(), pw.data_ptr() + k, 2 * k, ps.data_ptr(),
+                                        ps.data_ptr() + 2 * gcount * ps.element_size(), 4 * gcount, 7, xd.data_ptr(),
+                                        gd.data_ptr(), 1e-5, h.data_ptr(), n, k, tokens)
+    assert st == 0
+    assert_parity(h, oracle.gateup_silu(x, wd, ud, gamma, 1e-5), tol, f"ABI group-format prompt gate/up, fused norm {dtype}",
+                  elementwise=None if dtype == torch.float16 else 4e-2)
+    assert lib.mui_int8_group_linear(s, code, qd.data_ptr(), k, sd.data_ptr(), 3, xd.data_ptr(), None, 0.0, None, None,
+                                     y.data_ptr(), n, k, tokens) == -2
+    assert lib.mui_int8_group_linear(s, code, qd.data_ptr(), k, sd.data_ptr(), 9, xd.data_ptr(), None, 0.0, None, None,
+                                     y.data_ptr(), n, 1024 - 256, tokens) == -2
