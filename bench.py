@@ -746,6 +746,44 @@ def probe_prompt_other_shapes():
     print(json.dumps({"probe_prompt_other_shapes": out}))
 
 
+def probe_prompt_int8():
+    """Prefill of the 8B-shaped model with int8 decoder layers, per format and prompt length, on both
+    routes the host layer has: the tiled GEMM that converts the codes on their way to LDS, and every
+    matrix dequantised once per call followed by the GEMM on 16-bit weights (the reference's route).
+    The host layer's thresholds choose between them; here each is forced in turn."""
+    import torch
+
+    from muillm_amd import muillm_ext
+    from muillm_amd.engine import init_engine
+    from muillm_amd.engineconfig import MuiEngineConfig
+    from muillm_amd.modules.models.llama.model import MuiDecoderConfig, MuiLlamaForCausalLM
+    from muillm_amd.quantization.quantizationmethod import Int8WeightOnlyQuantizationMethod
+
+    config = MuiDecoderConfig.llama3_8b(max_position_embeddings=8192)
+    out = {}
+    for group_size, knob in ((0, "INT8_DEQUANT_MIN_TOKENS"), (128, "INT8_GROUP_DEQUANT_MIN_TOKENS")):
+        qm = Int8WeightOnlyQuantizationMethod(group_size=group_size, modules=["qkv_proj", "o_proj", "mlp"])
+        base = MuiLlamaForCausalLM.from_config(MuiEngineConfig(), config, dtype=torch.float16, device="cuda", seed=0,
+                                               finalize=False)
+        lm8 = init_engine(base, device="cuda", engine_config=MuiEngineConfig(qm))
+        torch.cuda.synchronize()
+        default = getattr(muillm_ext, knob)
+        name = "group128" if group_size else "per_channel"
+        out[name] = {"dequantise_once_from_tokens": default}
+        try:
+            for tokens in (32, 64, 512, 1024, 1536, 2048, 4096):
+                row = {}
+                for route, thr in (("codes_converted_on_the_way_to_lds", 1 << 30), ("dequantise_once_then_16bit_gemm", 17)):
+                    setattr(muillm_ext, knob, thr)
+                    row[route + "_ms"] = bench_prefill(lm8, tokens)["ms"]
+                out[name]["tokens%d" % tokens] = row
+        finally:
+            setattr(muillm_ext, knob, default)
+        del lm8, base
+        torch.cuda.empty_cache()
+    print(json.dumps({"probe_prompt_int8": out}))
+
+
 def trace_prefill(tokens, passes=3):
     """Prefill passes of the 8B-shaped fp16 model (embedding to last-token logits) for a kernel trace:
     two warm-up passes, then `passes` passes with a device synchronisation after each."""
@@ -1166,6 +1204,9 @@ def main():
                     help="time the prompt GEMMs and prompt attention at the Llama-3-8B shapes beside torch and exit")
     ap.add_argument("--trace-prefill", type=int, default=0, metavar="TOKENS",
                     help="a few prefill passes of the 8B-shaped model at this prompt length (for rocprofv3 --kernel-trace)")
+    ap.add_argument("--probe-prompt-int8", action="store_true",
+                    help="time the int8 model's prefill on both routes (codes converted in the GEMM / matrices "
+                         "dequantised first) in both formats and exit")
     ap.add_argument("--probe-prompt-other-shapes", action="store_true",
                     help="time the prompt GEMM at the 70B- and 13B-shaped projections beside torch.matmul and exit")
     ap.add_argument("--pmc-probe-prompt", action="store_true",
@@ -1207,6 +1248,9 @@ def main():
     if args.tune_prefill:
         from muillm_amd import _lib
         _lib.check(_lib.load().mui_tune_prefill(*(int(v) for v in args.tune_prefill.split(","))), "mui_tune_prefill")
+    if args.probe_prompt_int8:
+        probe_prompt_int8()
+        return
     if args.probe_prompt_other_shapes:
         probe_prompt_other_shapes()
         return
